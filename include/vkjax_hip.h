@@ -1,0 +1,123 @@
+/*
+ * vkjax_hip.h - C ABI of the MI355X device runtime behind vkJAX's jaxpr interpreter.
+ *
+ * This library takes the place of the Vulkan-Kompute objects the reference drives from
+ * Python (kp.Manager / kp.Tensor / kp.Sequence / kp.OpAlgoDispatch / kp.OpTensorSync*,
+ * package kp==0.7.0): a device context, HBM buffers, gfx950 code objects and a recorded
+ * sequence of uploads, kernel launches and downloads that is replayed with ONE call per
+ * run. All work of a context is issued on one in-order HIP stream; nothing synchronises
+ * with the host except the tail of vkj_seq_eval / vkj_seq_replay, the blocking buffer
+ * transfers and vkj_sync.
+ *
+ * Conventions: every function returns 0 on success, a positive hipError_t or a negative
+ * VKJ_E* code otherwise; vkj_last_error() returns the message of the calling thread's last
+ * failure. Handles are opaque 64-bit values owned by the library. Host memory passed in is
+ * owned by the caller and only has to stay valid for the duration of the call. A context
+ * and its objects must be used from one thread at a time.
+ */
+#ifndef VKJAX_HIP_H
+#define VKJAX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint64_t vkj_handle;
+
+enum {
+    VKJ_EINVAL   = -1,   /* bad argument (null pointer, out-of-range size, unknown handle) */
+    VKJ_ENOMEM   = -2,
+    VKJ_ESTATE   = -3,   /* call not valid in the object's current state */
+    VKJ_ENODEV   = -4    /* no usable GPU */
+};
+
+/* vkj_seq_eval flags */
+enum {
+    VKJ_EVAL_DEFAULT        = 0,
+    VKJ_EVAL_SKIP_UPLOADS   = 1,   /* inputs are already resident in HBM */
+    VKJ_EVAL_SKIP_DOWNLOADS = 2
+};
+
+typedef struct vkj_props {
+    char     name[256];
+    char     arch[64];                 /* e.g. "gfx950:sramecc+:xnack-" */
+    int32_t  compute_units;
+    int32_t  wavefront_size;
+    int32_t  max_threads_per_block;    /* replaces max_work_group_invocations */
+    int32_t  max_block_dim_x;          /* replaces max_work_group_size[0] */
+    int32_t  lds_bytes_per_block;
+    int32_t  clock_khz;
+    int32_t  memory_clock_khz;
+    int32_t  memory_bus_bits;
+    uint64_t hbm_bytes;
+} vkj_props;
+
+const char* vkj_last_error(void);
+int vkj_device_count(int* count);
+
+/* kp.Manager(device_index)            reference: vkjax/kompute_jaxpr_interpreter.py:19-20 */
+int vkj_ctx_create(int device, vkj_handle* ctx);
+int vkj_ctx_destroy(vkj_handle ctx);
+/* mgr.get_device_properties()         reference: vkjax/kompute_jaxpr_interpreter.py:100-102 */
+int vkj_device_props(vkj_handle ctx, vkj_props* out);
+/* blocks until everything issued on the context's stream has finished */
+int vkj_sync(vkj_handle ctx);
+
+/* Code objects built ahead of time for gfx950 replace the per-op SPIR-V produced by
+ * pyshaderc.compile_into_spirv          reference: vkjax/shaders.py:16-29 */
+int vkj_module_load(vkj_handle ctx, const void* image, size_t nbytes, vkj_handle* module);
+int vkj_module_unload(vkj_handle ctx, vkj_handle module);
+int vkj_module_get_function(vkj_handle ctx, vkj_handle module, const char* name, vkj_handle* function);
+
+/* mgr.tensor(array) + OpTensorSyncDevice  reference: vkjax/buffers.py:189-204 */
+int vkj_buf_alloc(vkj_handle ctx, size_t nbytes, vkj_handle* buf);
+int vkj_buf_free(vkj_handle ctx, vkj_handle buf);
+int vkj_buf_size(vkj_handle ctx, vkj_handle buf, size_t* nbytes);
+int vkj_buf_device_ptr(vkj_handle ctx, vkj_handle buf, uint64_t* device_address);
+int vkj_buf_memset(vkj_handle ctx, vkj_handle buf, size_t offset, int byte_value, size_t nbytes);
+/* blocking host->device / device->host copies (build-time constants, debugging reads:
+ * tensor.data(), OpTensorSyncLocal on all tensors  reference: vkjax/kompute_jaxpr_interpreter.py:85-89) */
+int vkj_buf_upload(vkj_handle ctx, vkj_handle buf, size_t offset, const void* host, size_t nbytes);
+int vkj_buf_download(vkj_handle ctx, vkj_handle buf, size_t offset, void* host, size_t nbytes);
+
+/* mgr.sequence(total_timestamps=n)    reference: vkjax/kompute_jaxpr_interpreter.py:48-49
+ * profiling != 0 records one timestamp before the first step and one after every step. */
+int vkj_seq_create(vkj_handle ctx, int profiling, vkj_handle* seq);
+int vkj_seq_destroy(vkj_handle seq);
+/* seq.record(kp.OpTensorSyncDevice([...]))  reference: vkjax/kompute_jaxpr_interpreter.py:51-53
+ * `slot` indexes the host_ptrs array given to vkj_seq_eval. */
+int vkj_seq_record_upload(vkj_handle seq, vkj_handle buf, size_t offset, int slot, size_t nbytes);
+/* mgr.algorithm(tensors, spirv, workgroup) + seq.record(kp.OpAlgoDispatch(algo))
+ *                                     reference: vkjax/kompute_jaxpr_interpreter.py:55-60
+ * `kernarg` is the kernel's argument block laid out by the caller. For each i < nbufs the
+ * 8 bytes at kernarg[buf_arg_offsets[i]] are overwritten with the device address of
+ * bufs[i] plus buf_byte_offsets[i] (may be NULL for all-zero). Addresses are resolved
+ * once, here. */
+int vkj_seq_record_launch(vkj_handle seq, vkj_handle function,
+                          const uint32_t grid[3], const uint32_t block[3], uint32_t lds_bytes,
+                          const void* kernarg, size_t kernarg_bytes,
+                          const vkj_handle* bufs, const uint32_t* buf_arg_offsets,
+                          const uint64_t* buf_byte_offsets, int nbufs);
+/* seq.record(kp.OpTensorSyncLocal([...]))   reference: vkjax/kompute_jaxpr_interpreter.py:62-63 */
+int vkj_seq_record_download(vkj_handle seq, vkj_handle buf, size_t offset, int slot, size_t nbytes);
+int vkj_seq_num_steps(vkj_handle seq, int* uploads, int* launches, int* downloads);
+/* sequence.eval()                     reference: vkjax/kompute_jaxpr_interpreter.py:77
+ * All uploads, then all launches, then all downloads, then one stream synchronisation.
+ * host_ptrs[slot] supplies the host address of every recorded upload and download. */
+int vkj_seq_eval(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t flags);
+/* Launches only, `iters` times back to back, bracketed by two events on the context's
+ * stream; *ms_total receives the elapsed device time of all iterations. Used for
+ * measurement with inputs resident in HBM. No counterpart in the reference. */
+int vkj_seq_replay(vkj_handle seq, int iters, float* ms_total);
+/* sequence.get_timestamps()           reference: vkjax/kompute_jaxpr_interpreter.py:91-95
+ * Milliseconds since the first timestamp of the last vkj_seq_eval; *count receives the
+ * number of timestamps available (steps + 1). */
+int vkj_seq_timestamps(vkj_handle seq, float* ms_out, int capacity, int* count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VKJAX_HIP_H */

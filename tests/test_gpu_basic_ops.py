@@ -1,0 +1,268 @@
+'''Per-primitive parity of the HIP path against the CPU oracle, on the case list of the
+reference's own test matrix (reference: tests/test_basic_ops.py:162-333; same functions, same
+shapes, same tolerances), with seeded inputs. Runs on the GPU box only.'''
+import numpy as np
+import pytest
+
+from vkjax_amd import minijax as mj
+from tests.common import check_against_oracle
+
+jnp, lax = mj.numpy, mj.lax
+pytestmark = pytest.mark.gpu
+rng = np.random.RandomState(1234)
+random, randint, uniform = rng.random_sample, rng.randint, rng.uniform
+
+
+def add0(x): return x + x
+def add1(x): return x + 1.0
+def add2(x, y): return x + y
+def add3(x, y): return mj.jit(add0)(x) + mj.jit(add2)(y, x)
+def add4(x, y): return mj.jit(add0)(x) + mj.jit(add2)(y, 1.0)
+def add00(): return lax.add(5, 100)
+def div0(x, y): return x / y
+def sub0(x, y): return x - y
+def mul0(x, y): return x * y
+def reshape1(x): return (x + 1).reshape(4, -1)
+def broadcast0(x): return lax.broadcast_in_dim(x, shape=(4,), broadcast_dimensions=())
+def broadcast1(x): return lax.broadcast_in_dim(x + 1, shape=(4, 1, 1), broadcast_dimensions=(0,))
+def broadcast2(x): return lax.broadcast_in_dim(x, shape=x.shape + (32,), broadcast_dimensions=tuple(np.arange(len(x.shape))))
+def broadcast3(x): return lax.broadcast_in_dim(x, shape=(32,) + x.shape, broadcast_dimensions=(1,))
+def dot0(x, y): return jnp.dot(x, y)
+dot1_const = random([100, 32]).astype(np.float64)
+def dot1(x): return jnp.dot(x, dot1_const)
+def dot_general0(x, y): return lax.dot_general(x, y, (((0,), (0,)), ((), ())))
+def dot_general1(x, y): return lax.dot_general(x, y, (((1,), (1,)), ((), ())))
+def dot_general2(x, y): return lax.dot_general(x, y, (((0,), (1,)), ((), ())))
+def reshape_dot(x, y): return x.reshape(-1, 4) @ y
+def relu0(x): return mj.nn.relu(x)
+def reduce_max0(x): return jnp.max(x, axis=0)
+def reduce_min0(x): return jnp.min(x, axis=0)
+def reduce_max1(x): return jnp.max(x, axis=1)
+def reduce_max2(x): return jnp.max(x, axis=[1, 2, 5])
+def reduce_sum0(x): return jnp.sum(x, axis=0)
+def reduce_sum1(x): return jnp.sum(x, axis=1)
+def reduce_sum2(x): return jnp.sum(x, axis=[0, 1, 2])
+def no_reduce1(x): return jnp.sum(x + 1, axis=())
+def reduce_prod0(x): return jnp.prod(x, axis=0)
+def argmax0(x): return jnp.argmax(x, axis=0)
+def argmin0(x): return jnp.argmin(x, axis=0)
+def gt0(x, y): return x > y
+def ge0(x, y): return x >= y
+def lt0(x, y): return x < y
+def le0(x, y): return x <= y
+def eq0(x, y): return x == y
+def eq1(x): return x == x.max(axis=-1)
+def ne0(x, y): return x != y
+def or0(x, y): return x | y
+def and0(x, y): return x & y
+def exp0(x): return jnp.exp(x)
+def log0(x): return jnp.log(x)
+def abs0(x): return jnp.abs(x)
+def rsqrt0(x): return lax.rsqrt(x)
+def iota0(): return jnp.arange(32)
+def select0(x, y, z): return jnp.where(x, y, z)
+def concatenate0(x, y): return jnp.concatenate([x, y], axis=-1)
+def gather0(x): return x[:, :, 4:7, :]
+def gather1a(x): return x[5, :]
+def gather1b(x): return x[:, 5]
+def gather_fn0(x, i):
+    return lax.gather(x, i, mj.core.GatherDimensionNumbers(offset_dims=(), collapsed_slice_dims=(0, 1), start_index_map=(0, 1)),
+                      slice_sizes=(1, 1))
+def take_along_axis0(x, i): return jnp.take_along_axis(x, i, axis=-1)
+def gather_fn1(x, i):
+    return lax.gather(x, i, mj.core.GatherDimensionNumbers(offset_dims=(0,), collapsed_slice_dims=(1,), start_index_map=(1,)),
+                      slice_sizes=(len(x), 1))
+def scatter_fn0(x, i, u):
+    return lax.scatter_add(x, i, u, mj.core.ScatterDimensionNumbers(update_window_dims=(), inserted_window_dims=(0, 1),
+                                                                    scatter_dims_to_operand_dims=(0, 1)))
+def scatter_add_fn1(x, i, u):
+    return lax.scatter_add(x, i, u, mj.core.ScatterDimensionNumbers(update_window_dims=(0,), inserted_window_dims=(1,),
+                                                                    scatter_dims_to_operand_dims=(1,)))
+def add_any0(x, y): return lax.add_any(x, y), np.float32(1)
+def transpose0(x): return x.T
+def rev0(x): return lax.rev(x, dimensions=[1, 2])
+def integer_pow0(x): return x ** 2
+def integer_pow1(x): return x ** 5
+def pow0(x, y): return lax.pow(x, y)
+def slice0(x): return lax.slice(x, [2], [33])
+def slice1(x): return lax.slice(x, [55, 5], [101, 10])
+def slice2(x): return lax.slice(x, [55, 5], [101, 10], [2, 3])
+def squeeze0(x): return jnp.squeeze(x)
+def threefry0a(): return lax.threefry2x32(*np.ones(4, 'uint32'))
+def threefry0b(): return lax.threefry2x32(*np.ones([4, 10], 'uint32'))
+def threefry1(x): return lax.threefry2x32(*x)
+def convert_element_type0(x): return x.astype(np.int32)
+def convert_element_type1(x): return x.astype(np.float32)
+def bitcast_convert_type0(x): return lax.bitcast_convert_type(x, 'float32')
+def shift_right_logical_1_32(): return lax.shift_right_logical(1, 32)
+
+
+param_matrix = [
+    (add0, 'add x+x scalar',            [5.0]),
+    (add0, 'add x+x array1d',           [random(32)]),
+    (add0, 'add x+x array3d',           [random((32, 32, 32))]),
+    (add00, '5+100',                    []),
+    (add1, 'add x+1 scalar',            [5.0]),
+    (add1, 'add x+1 array3d',           [random((32, 32, 32))]),
+    (add2, 'add x+y scalar-scalar',     [5.0, 7.0]),
+    (add2, 'add x+y scalar-array3d',    [5.0, random((32, 32, 32))]),
+    (add2, 'add x+y array3d-array3d',   [random((32, 32, 32)), random((32, 32, 32))]),
+    (add2, 'broadcast_add [2,32]+[32]', [random((2, 32)), random((32))]),
+    (add2, 'add x+y int',               [randint(65, size=(32, 32, 32)), randint(77, size=(32, 32, 32))]),
+    (add3, 'add nested (x+x)+(y+x)',    [5.0, 7.1]),
+    (add4, 'nested const (x+x)+(y+1)',  [5.0, 7.1]),
+    (div0, 'div0 x/y',                  [random([2, 32, 32, 3]), 255.0]),
+    (sub0, 'sub0 x-y',                  [random([2, 32, 32, 3]), 255.0]),
+    (sub0, 'sub0 (2,10)-(2,1)',         [random([2, 10]), random([2, 1])]),
+    (mul0, 'mul0 x*y',                  [random([2, 32, 32, 3]), 255.0]),
+    (reshape1, 'reshape1',              [random([2, 32, 32])]),
+    (broadcast0, 'broadcast scalar',    [random()]),
+    (broadcast1, 'broadcast 1D->3D',    [random(4)]),
+    (broadcast2, 'broadcast append',    [random(4)]),
+    (broadcast3, '(128)->(32,128)',     [random(128)]),
+    (dot0, 'dot0 x@y',                  [random([2, 100]), random([100, 32])]),
+    (dot1, 'dot1 x@const',              [random([2, 100])]),
+    (dot_general0, 'dot axes=(0,0)',    [random([100, 2]), random([100, 32])]),
+    (dot_general1, 'dot axes=(1,1)',    [random([2, 100]), random([32, 100])]),
+    (dot_general2, 'dot axes=(0,1)',    [random([100, 2]), random([32, 100])]),
+    (reshape_dot, 'reshape_dot',        [random([2, 77, 102]), random([4, 4])]),
+    (relu0, 'relu0',                    [random([32, 32, 32]) - 0.5]),
+    (lax.max, 'max_float32',            [random([77, 99, 200]), random([77, 99, 200])]),
+    (lax.min, 'min_float32',            [random([77, 99, 200]), random([77, 99, 200])]),
+    (lax.max, 'max_int32',              [randint(-1000, 1000, [77, 99, 200]), randint(-1000, 1000, [77, 99, 200])]),
+    (lax.min, 'min_int32',              [randint(-1000, 1000, [77, 99, 200]), randint(-1000, 1000, [77, 99, 200])]),
+    (reduce_max0, 'max(axis=0)',        [random([32, 32])]),
+    (reduce_min0, 'min(axis=0)',        [random([77, 99])]),
+    (reduce_max1, 'max(axis=1)',        [random([32, 32]) - 1.0]),
+    (reduce_max2, 'max(axis=125)',      [random([3, 33, 67, 99, 4, 7])]),
+    (reduce_sum0, 'sum(axis=0) 2D',     [random([32, 32])]),
+    (reduce_sum0, 'sum(axis=0) 1D',     [random([32])]),
+    (reduce_sum1, 'sum(axis=1)',        [random([32, 32])]),
+    (reduce_sum2, 'sum(axis=012)',      [random([65, 77, 22, 7])]),
+    (no_reduce1, 'no_reduce1(axis=())', [random([32])]),
+    (argmax0, 'argmax(axis=0)',         [random([99, 77])]),
+    (argmin0, 'argmin(axis=0)',         [random([99, 77])]),
+    (reduce_prod0, 'prod(axis=0)',      [random([32, 32]) + 0.5]),
+    (gt0, 'gt0',                        [random([32, 32]), random([32, 32])]),
+    (ge0, 'ge0',                        [random([32, 32]), random([32, 32])]),
+    (ge0, 'ge0 float>=bool',            [random([32, 32]) + 0.5, random([32, 32]) > 0.5]),
+    (ge0, 'ge0 bool>=float',            [random([32, 32]) > 0.5, random([32, 32]) + 0.5]),
+    (lt0, 'lt0',                        [random([32, 32]), random([32, 32])]),
+    (lt0, 'lt0 int[]<scalar',           [randint(999, size=[999]), 555]),
+    (le0, 'le0',                        [random([77, 99]), random([77, 99])]),
+    (eq0, 'eq0',                        [randint(0, 3, size=[32, 32]).astype(np.float32), randint(0, 3, size=[32, 32]).astype(np.float32)]),
+    (eq1, 'eq1 x==x.max(-1)',           [random([32, 32])]),
+    (ne0, 'x!=y',                       [random([77, 99]), random([77, 99])]),
+    (or0, 'or0 x|y',                    [random([77, 32]).astype('float32').view('uint32'), random([77, 32]).astype('float32').view('uint32')]),
+    (and0, 'and0 x&y',                  [random([77, 32]).astype('float32').view('uint32'), random([77, 32]).astype('float32').view('uint32')]),
+    (exp0, 'exp(x)',                    [uniform(0, 5, size=[32, 32])]),
+    (log0, 'log(x+100)',                [uniform(0, 5, size=[32, 32]) + 100]),
+    (abs0, 'abs(x)',                    [random([32, 32, 32]) - 0.5]),
+    (rsqrt0, 'rsqrt(x)',                [random([77, 40, 32]) * 10]),
+    (iota0, 'iota0',                    []),
+    (select0, 'select0',                [random([32, 32]) > 0.5, np.ones([32, 32]), np.zeros([32, 32])]),
+    (concatenate0, 'concatenate0',      [random([32, 32, 32]), random([32, 32, 16])]),
+    (gather0, 'gather0',                [random([40, 40, 40, 40])]),
+    (gather1a, 'gather1a x[5,:]',       [random([8, 8])]),
+    (gather1b, 'gather1b x[:,5]',       [random([8, 8])]),
+    (gather_fn0, 'gather_fn0',          [random([32, 10]), np.c_[randint(0, 32, size=[32]), randint(0, 10, size=[32])].reshape(32, 1, 2)]),
+    (scatter_fn0, 'scatter_fn0',        [random([32, 10]), np.c_[randint(0, 32, size=[32]), randint(0, 10, size=[32])].reshape(32, 1, 2),
+                                         random([32]).reshape(32, 1)]),
+    (take_along_axis0, 'take_along0',   [random([32, 10]), randint(0, 10, size=32)[:, np.newaxis]]),
+    (gather_fn1, 'gather_fn1',          [random([32, 10]), randint(0, 10, size=[1])]),
+    (scatter_add_fn1, 'scatter_add1',   [random([32, 10]), randint(0, 10, size=[1]), random(32)]),
+    (add_any0, 'add_any0',              [random([32, 32]), random([32, 32])]),
+    (transpose0, 'random([N,N]).T',     [random([32, 32])]),
+    (transpose0, 'random([N,M]).T',     [random([32, 65])]),
+    (rev0, 'rev0 dims=1,2',             [random([33, 77, 88, 11])]),
+    (integer_pow0, 'x**2',              [random([77, 9, 35])]),
+    (integer_pow1, 'x**5',              [random([77, 9, 35]) * 2 - 1]),
+    (integer_pow1, 'int**5',            [randint(-1000, 1000, size=[77, 9, 35])]),
+    (pow0, 'x**scalar',                 [random([77, 9, 35]), random()]),
+    (slice0, '1-D slice(x, [2],[33])',  [random([99])]),
+    (slice1, '2-D slice no strides',    [random([199, 99])]),
+    (slice2, '2-D slice + strides',     [random([199, 99])]),
+    (squeeze0, '5-D squeeze',           [random([199, 99, 1, 1, 5])]),
+    (threefry0a, 'all const size=1',    []),
+    (threefry0b, 'all const size=n',    []),
+    (threefry1, 'all zero size=1',      [np.zeros(4).astype('uint32')]),
+    (threefry1, 'all ones size=1',      [np.ones(4).astype('uint32')]),
+    (threefry1, 'all random size=1',    [randint(0, 10000000, size=4).astype('uint32')]),
+    (threefry1, 'all random size=65',   [randint(0, 10000000, size=(4, 65)).astype('uint32')]),
+    (threefry1, 'scalar_key_size=100',  [list(randint(0, 10000000, size=(2,)).astype('uint32'))
+                                         + list(randint(0, 10000000, size=(2, 100)).astype('uint32'))]),
+    (convert_element_type0, 'float2int', [random([77, 101]) * 65]),
+    (convert_element_type1, 'int2float', [randint(77, 101, size=(99, 99))]),
+    (convert_element_type1, 'bool2float', [random([77, 101]) > 0.5]),
+    (bitcast_convert_type0, 'uint2float', [random([77, 101]).astype('float32').view('uint32')]),
+    (lax.shift_left, 'x<<1',            [np.arange(-777, +777), 1]),
+    (lax.shift_left, 'x<<y',            [np.arange(-777, +777), randint(0, 20, size=777 * 2)]),
+    (lax.shift_right_logical, 'x>>1',   [np.arange(-777, +777), 1]),
+    (shift_right_logical_1_32, '1>>32', []),
+    (lax.shift_right_logical, 'uint>>9', [np.arange(-777, +777).astype('int32').view('uint32'), np.uint32(9)]),
+    (lax.shift_right_arithmetic, 'x>>1', [np.arange(-777, +777), 1]),
+    (lax.shift_right_arithmetic, 'uint32', [np.arange(-777, +777).astype('int32').view(np.uint32), np.uint32(1)]),
+    (lax.erf, 'erf(x)',                 [random([111, 283]) * 10 - 5]),
+    (lax.erf_inv, 'erf_inv(x)',         [random([111, 283]) * 2 - 1]),
+    (lax.rem, 'rem(x,y)',               [randint(1000, 10000, size=[77, 99]), int(randint(1, 1000))]),
+    (lax.nextafter, 'nextafter(X,inf)', [random([77, 101]) * 2 - 1, np.inf]),
+    (lax.nextafter, 'nextafter(X,-inf)', [random([77, 101]) * 2 - 1, -np.inf]),
+    (lax.nextafter, 'nextafter(X,0)',   [random([77, 101]) * 2 - 1, 0.0]),
+    (lax.nextafter, 'nextafter(X,Y)',   [random([77, 101]) * 2 - 1, random([77, 101])]),
+]
+
+for fname in ['cos', 'sin', 'tan', 'cosh', 'sinh', 'tanh', 'acos', 'asin', 'atan', 'acosh', 'asinh', 'atanh',
+              'ceil', 'floor', 'sign']:
+    param_matrix += [(getattr(lax, fname), fname, [random([77, 101]) * 2 - 1])]
+
+#(rtol, atol); everything else uses numpy.allclose defaults 1e-5 / 1e-8 (reference: tests/test_basic_ops.py:326-333)
+TOLERANCES = {
+    'erf(x)':        (1e-5, 1e-6),
+    'erf_inv(x)':    (1e-5, 1e-5),
+    'sum(axis=012)': (1e-4, 1e-8),
+    'sin':           (1e-5, 1e-6),
+    'sinh':          (1e-5, 1e-6),
+    'tan':           (1e-5, 1e-6),
+    #dot: north-star tolerance for contractions
+    'dot0 x@y': (1e-4, 1e-8), 'dot1 x@const': (1e-4, 1e-8), 'dot axes=(0,0)': (1e-4, 1e-8),
+    'dot axes=(1,1)': (1e-4, 1e-8), 'dot axes=(0,1)': (1e-4, 1e-8), 'reshape_dot': (1e-4, 1e-8),
+}
+
+
+@pytest.mark.parametrize('f,desc,args', param_matrix, ids=[p[1] for p in param_matrix])
+def test_matrix_hip_interpreter(f, desc, args):
+    print(f'case: {getattr(f, "__name__", f)} | {desc}', flush=True)
+    rtol, atol = TOLERANCES.get(desc, (1e-5, 1e-8))
+    check_against_oracle(f, args, rtol=rtol, atol=atol)
+
+
+def test_nextafter_direction():
+    '''reference: tests/test_basic_ops.py:367-382'''
+    import vkjax_amd
+    x = random([77, 101, 5]).astype(np.float32)
+    vkfunc = vkjax_amd.wrap(lax.nextafter, frontend='minijax')
+    assert np.all(vkfunc(x, np.inf) > x)
+    assert np.all(x > vkfunc(x, -np.inf))
+    assert np.all(np.sign(vkfunc(x, 0.0) - x) == np.sign(0 - x))
+    x2 = random(x.shape).astype(np.float32)
+    assert np.all(np.sign(vkfunc(x, x2) - x) == np.sign(x2 - x))
+
+
+def test_max_pool_negative_border_and_select_with_inf():
+    '''XLA semantics where the reference's shaders differ: padding of a max window is -inf, and
+    select picks without touching the other branch.'''
+    x = -1.0 - random([2, 5, 5, 3])
+    def pool(x): return lax.reduce_window(x, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), 'SAME')
+    y, ytrue, _ = check_against_oracle(pool, [x], exact=True)
+    assert np.all(y < 0)
+    p = random([8, 8]) > 0.5
+    a = np.where(random([8, 8]) > 0.5, np.inf, 1.0)
+    b = np.where(random([8, 8]) > 0.5, np.nan, -2.0)
+    check_against_oracle(select0, [p, a, b], exact=True)
+
+
+def test_argmax_ties_and_nan():
+    x = np.array([[1, 3, 3, 2], [np.nan, 5, np.nan, 1], [2, 2, 2, 2], [0, -1, 7, 7]], np.float32)
+    def f(x): return jnp.argmax(x, axis=1), jnp.argmin(x, axis=1)
+    (amax, amin), _, _ = check_against_oracle(f, [x], exact=True)
+    assert amax.tolist() == [1, 0, 0, 2] and amin.tolist() == [0, 0, 0, 1]

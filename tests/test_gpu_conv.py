@@ -1,0 +1,123 @@
+'''conv_general_dilated parity against the CPU oracle on the reference's case list
+(reference: tests/test_conv.py:66-85: NHWC/HWIO and NCHW/OIHW dimension numbers, 1x1/3x3/7x7,
+VALID/SAME/uneven explicit padding, stride 2, rhs and lhs dilation), plus reduce_window
+(reference: tests/test_reduce_window.py:18-21). Tolerance: rtol 1e-4 for contractions.'''
+import numpy as np
+import pytest
+
+from vkjax_amd import minijax as mj
+from tests.common import check_against_oracle
+
+jnp, lax = mj.numpy, mj.lax
+pytestmark = pytest.mark.gpu
+rng = np.random.RandomState(4321)
+random = rng.random_sample
+
+NHWC = mj.core.ConvDimensionNumbers((0, 3, 1, 2), (3, 2, 0, 1), (0, 3, 1, 2))
+NCHW = mj.core.ConvDimensionNumbers((0, 1, 2, 3), (0, 1, 2, 3), (0, 1, 2, 3))
+
+kernel_1x1 = random([1, 1, 5, 33])
+
+def conv0(x):     return lax.conv_general_dilated(x, kernel_1x1, (1, 1), 'VALID', dimension_numbers=NHWC)
+def conv1(x, k):  return lax.conv_general_dilated(x, k, (1, 1), 'VALID', dimension_numbers=NHWC)
+def conv1a(x, k): return lax.conv_general_dilated(x, k, (1, 1), 'VALID', dimension_numbers=NCHW)
+def conv2(x, k):  return lax.conv_general_dilated(x, k, (1, 1), 'SAME', dimension_numbers=NHWC)
+def conv3(x, k):  return lax.conv_general_dilated(x, k, (1, 1), [(2, 0), (0, 3)], dimension_numbers=NHWC)
+def conv4(x, k):  return lax.conv_general_dilated(x, k, (2, 2), 'SAME', dimension_numbers=NHWC)
+def conv5(x, k):  return lax.conv_general_dilated(x, k, (2, 2), 'VALID', rhs_dilation=(2, 2), dimension_numbers=NHWC)
+def conv6a(x, k): return lax.conv_general_dilated(x, k, (1, 1), [(2, 2), (3, 3)], lhs_dilation=(2, 2), dimension_numbers=NHWC)
+def conv6b(x, k): return lax.conv_general_dilated(x, k, (2, 2), [(0, 0), (0, 0)], lhs_dilation=(2, 2), dimension_numbers=NHWC)
+
+param_matrix = [
+    (conv0,  'conv0 1x1 const kernel no pad',               [random([11, 100, 100, 5])]),
+    (conv1,  'conv1 1x1 var kernel no pad',                 [random([11, 100, 100, 33]), random([1, 1, 33, 11])]),
+    (conv1,  'conv1 3x3 var kernel no pad',                 [random([40, 65, 33, 5]), random([3, 3, 5, 7])]),
+    (conv1a, 'conv1a 3x3 convdims 0123',                    [random([40, 8, 65, 35]), random([39, 8, 3, 3])]),
+    (conv2,  'conv2 1x1 var kernel +pad',                   [random([77, 17, 9, 12]), random([1, 1, 12, 11])]),
+    (conv2,  'conv2 3x3 var kernel +pad',                   [random([23, 44, 19, 7]), random([3, 3, 7, 38])]),
+    (conv2,  'conv2 7x7 var kernel +pad',                   [random([8, 12, 19, 3]), random([7, 7, 3, 4])]),
+    (conv3,  'conv3 3x3 uneven pad',                        [random([15, 67, 42, 11]), random([3, 3, 11, 38])]),
+    (conv4,  'conv4 1x1 window strides=2',                  [random([2, 67, 42, 3]), random([1, 1, 3, 2])]),
+    (conv4,  'conv4 3x3 window strides=2',                  [random([15, 67, 42, 11]), random([3, 3, 11, 7])]),
+    (conv5,  'conv5 3x3 window strides=2 + rhs_dilate=2',   [random([15, 67, 42, 11]), random([3, 3, 11, 7])]),
+    (conv6a, 'conv6a 3x3 window strides=1 + lhs_dilate=2',  [random([15, 67, 42, 11]), random([3, 3, 11, 7])]),
+    (conv6b, 'conv6b 3x3 window strides=2 + lhs_dilate=2',  [random([15, 67, 42, 11]), random([3, 3, 11, 7])]),
+    #shapes that take the 16-byte-load paths and every tile size
+    (conv2,  'fast 3x3 C64->64 (128x64 tile)',              [random([8, 56, 56, 64]), random([3, 3, 64, 64])]),
+    (conv1,  'fast 1x1 C64->256 (128x128 tile)',            [random([16, 56, 56, 64]), random([1, 1, 64, 256])]),
+    (conv4,  'fast 3x3 s2 C32->64',                         [random([4, 28, 28, 32]), random([3, 3, 32, 64])]),
+    (conv4,  'fast 1x1 s2 C128->96 (N not tile multiple)',  [random([3, 14, 14, 128]), random([1, 1, 128, 96])]),
+    (conv2,  'generic lhs, fast rhs 7x7 C3->64',            [random([2, 64, 64, 3]), random([7, 7, 3, 64])]),
+]
+
+
+@pytest.mark.parametrize('f,desc,args', param_matrix, ids=[p[1] for p in param_matrix])
+def test_convmatrix(f, desc, args):
+    print(f'case: {desc}', flush=True)
+    check_against_oracle(f, args, rtol=1e-4, atol=1e-6)
+
+
+def test_conv_integer_valued_is_exact():
+    '''Small-integer inputs make every product and partial sum exact in fp32, so any accumulation
+    order must give bit-identical results: catches indexing mistakes independently of rounding.'''
+    x = rng.randint(-4, 5, size=[3, 20, 17, 16]).astype(np.float32)
+    k = rng.randint(-3, 4, size=[3, 3, 16, 24]).astype(np.float32)
+    check_against_oracle(conv2, [x, k], exact=True)
+    check_against_oracle(conv4, [x, k], exact=True)
+
+
+def test_dot_integer_valued_is_exact_all_layouts():
+    a = rng.randint(-8, 9, size=[70, 132]).astype(np.float32)
+    b = rng.randint(-8, 9, size=[132, 52]).astype(np.float32)
+    check_against_oracle(lambda x, y: lax.dot_general(x, y, (((1,), (0,)), ((), ()))), [a, b], exact=True)
+    check_against_oracle(lambda x, y: lax.dot_general(x, y, (((0,), (0,)), ((), ()))), [a.T.copy(), b], exact=True)
+    check_against_oracle(lambda x, y: lax.dot_general(x, y, (((1,), (1,)), ((), ()))), [a, b.T.copy()], exact=True)
+    check_against_oracle(lambda x, y: lax.dot_general(x, y, (((0,), (1,)), ((), ()))), [a.T.copy(), b.T.copy()], exact=True)
+
+
+def test_dot_sizes():
+    for m, k, n in [(256, 784, 512), (256, 512, 10), (64, 2048, 1000), (1, 1, 1), (129, 33, 65), (300, 64, 64)]:
+        print(f'dot {m}x{k}x{n}', flush=True)
+        a, b = random([m, k]) - 0.5, random([k, n]) - 0.5
+        check_against_oracle(lambda x, y: jnp.dot(x, y), [a, b], rtol=1e-4, atol=1e-5)
+
+
+def reduce_window_max0(x): return lax.reduce_window(x, -jnp.inf, lax.max, (1, 2, 2, 1), (1, 1, 1, 1), 'VALID')
+def reduce_window_max1(x): return lax.reduce_window(x, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), 'SAME')
+def reduce_window_sum0(x): return lax.reduce_window(x, 0.0, lax.add, (1, 2, 2, 1), (1, 2, 2, 1), 'VALID')
+def reduce_window_sum1(x): return lax.reduce_window(x, 0.0, lax.add, (1, 3, 3, 1), (1, 2, 2, 1), 'SAME')
+def reduce_window_odd(x):  return lax.reduce_window(x, -jnp.inf, lax.max, (1, 3, 2, 3), (1, 2, 1, 2), ((0, 0), (1, 1), (0, 1), (1, 0)))
+
+pool_matrix = [
+    (reduce_window_max0, '2x2 no-pad',        [random([11, 100, 111, 5])], True),
+    (reduce_window_max1, '3x3 +pad',          [random([77, 10, 99, 17])], True),
+    (reduce_window_max1, '3x3 +pad C64',      [random([4, 56, 56, 64]) - 0.5], True),
+    (reduce_window_sum0, 'sum 2x2 s2',        [random([4, 28, 28, 32])], False),
+    (reduce_window_sum1, 'sum 3x3 s2 SAME',   [random([3, 15, 17, 6])], False),
+    (reduce_window_odd,  'window over C too', [random([3, 15, 17, 6]) - 0.5], True),
+]
+
+
+@pytest.mark.parametrize('f,desc,args,exact', pool_matrix, ids=[p[1] for p in pool_matrix])
+def test_reduce_window_matrix(f, desc, args, exact):
+    print(f'case: {desc}', flush=True)
+    check_against_oracle(f, args, exact=exact, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize('tile', ['128x128', '128x64', '64x64', '32x32'])
+def test_every_tile_and_loader_variant(tile):
+    '''All 16 kernel instantiations: each tile shape with 16-byte (f) or strided (g) loads on either operand.'''
+    from vkjax_amd import kernels as K
+    cases = {'ff': ([3, 20, 17, 16], [3, 3, 16, 24]), 'gg': ([2, 13, 11, 5], [3, 3, 5, 7]),
+             'gf': ([2, 13, 11, 3], [3, 3, 3, 64]), 'fg': ([2, 13, 11, 8], [3, 3, 8, 10])}
+    K.FORCE_CONV_TILE = tile
+    try:
+        for variant, (xs, ks) in cases.items():
+            print(f'tile {tile} loaders {variant}', flush=True)
+            x = rng.randint(-4, 5, size=xs).astype(np.float32)
+            k = rng.randint(-3, 4, size=ks).astype(np.float32)
+            _, _, fn = check_against_oracle(conv2, [x, k], exact=True)
+            kernel = list(fn._jaxpr_interpreters.values())[0].launches[0].kernel
+            assert kernel == f'conv_gemm_{tile}_{variant}', kernel
+    finally:
+        K.FORCE_CONV_TILE = None

@@ -1,0 +1,60 @@
+'''The benchmark workloads end to end through vkjax_amd.wrap against the CPU oracle, at sizes
+the oracle finishes in seconds; tolerances are the north-star ones (bit-exact RNG / gather /
+argmax, 1e-5 element-wise and reductions, 1e-4 dot and conv, 1e-3 ResNet logits).'''
+import numpy as np
+import pytest
+
+import vkjax_amd
+from vkjax_amd import minijax as mj, workloads as W
+from tests.common import check_against_oracle, assert_tree_close
+
+pytestmark = pytest.mark.gpu
+
+
+def test_affine():
+    check_against_oracle(W.affine, W.affine_inputs(), rtol=1e-4, atol=1e-6)
+
+
+def test_mlp():
+    (probs, labels), (probs_true, labels_true), _ = check_against_oracle(W.mlp, W.mlp_inputs(), rtol=1e-4, atol=1e-6)
+    assert np.allclose(probs.sum(axis=1), 1.0, atol=1e-5)
+
+
+def test_conv_block_small_and_full():
+    check_against_oracle(W.conv_block, W.conv_block_inputs(batch=2, size=14, channels=16), rtol=1e-4, atol=1e-5)
+    check_against_oracle(W.conv_block, W.conv_block_inputs(), rtol=1e-4, atol=1e-5)
+
+
+def test_resnet50_reduced_width():
+    '''The full layer graph (53 convolutions) at a quarter of the channel widths, batch 2, 64x64 images.'''
+    args = W.resnet50_inputs(batch=2, size=64, num_classes=40, width_scale=0.25)
+    (logits, labels), (logits_true, labels_true), _ = check_against_oracle(W.resnet50, args, rtol=1e-3, atol=1e-4)
+    assert labels.dtype == np.int32
+
+
+def test_resnet50_full_width_batch2():
+    args = W.resnet50_inputs(batch=2, size=224)
+    check_against_oracle(W.resnet50, args, rtol=1e-3, atol=1e-4)
+
+
+def test_rng_small_and_full_bit_exact():
+    check_against_oracle(lambda key: W.rng_uniform(key, (5, 7)), W.rng_inputs(), exact=True)
+    y, ytrue, _ = check_against_oracle(W.rng_uniform, W.rng_inputs(), exact=True)
+    assert y.shape == (4096, 4096) and y.dtype == np.float32
+    assert 0.0 <= y.min() and y.max() < 1.0 and abs(y.mean() - 0.5) < 1e-3
+
+
+def test_gather_scatter_small_exact_and_full():
+    #integer-valued updates make the atomic sums exact whatever their order
+    rng = np.random.default_rng(0)
+    table   = rng.random((97, 12), dtype=np.float32)
+    idx     = rng.integers(-97, 97, size=(33, 5)).astype(np.int32)
+    updates = rng.integers(-5, 6, size=(33, 5, 12)).astype(np.float32)
+    check_against_oracle(W.gather_scatter, [table, idx, updates], exact=True)
+    table, idx, updates = W.gather_scatter_inputs()
+    f = vkjax_amd.wrap(W.gather_scatter, frontend='minijax')
+    rows, acc = f(table, idx, updates)
+    assert np.array_equal(rows, table[idx])
+    expected = np.zeros(table.shape, np.float64)
+    np.add.at(expected, idx.reshape(-1), updates.reshape(-1, table.shape[1]).astype(np.float64))
+    assert np.allclose(acc, expected, rtol=1e-5, atol=1e-6)

@@ -1,0 +1,309 @@
+// fp32 implicit-GEMM convolution / matrix product on the MFMA units (v_mfma_f32_32x32x2_f32).
+//
+//   C[m, n] = sum_k A(m, k) * B(k, n)       m = (batch, out_y, out_x), n = out feature,
+//                                           k = (kernel_y, kernel_x, in feature), in feature fastest
+//   A(m, k) = lhs[b, y*SH + ky*DH - PH, x*SW + kx*DW - PW, c]   (zero outside; lhs dilation = only
+//                                                               multiples of LH/LW exist)
+//   B(k, n) = rhs[ky, kx, c, n]
+//
+// Both operands and the result are addressed through element strides, so any
+// ConvDimensionNumbers permutation, and dot_general with either contracting dimension, run
+// through the same kernel; the *_FAST template flags enable 16-byte loads when the feature
+// axis is contiguous. It supersedes the reference's scalar kernels conv2d.comp and
+// dot_general.comp (reference: vkjax/ops.py:277-297, 463-487; vkjax/shaders/conv2d.comp:44-95;
+// vkjax/shaders/dot_general.comp:10-34).
+//
+// Block = WGM x WGN waves, each wave owns TM x TN tiles of 32x32; block tile BM x BN with
+// BM = 32*WGM*TM, BN = 32*WGN*TN, K step 32. A and B tiles are staged through LDS
+// (A: [BM][36] so a lane reads 4 consecutive k with one 16-byte LDS load without bank
+// conflicts; B: [32][BN+4]); the next tiles are prefetched into registers while the MFMAs of
+// the current one run. The sum over k is order-free, so lanes 0-31 take k = 0..15 of a step and
+// lanes 32-63 take k = 16..31, which is what makes the 16-byte A reads possible.
+// After the k loop an optional chain of element-wise steps (per-feature vectors, full-size
+// tensors or scalars as operands) is applied to the accumulators before the single store.
+#include "common.h"
+
+#define CONV_BK 32
+#define CONV_MAX_EPI 6
+
+enum EwOpConv : uint32_t {
+#define EW_OP(name, num) CEW_##name = num,
+#include "ew_opcodes.h"
+#undef EW_OP
+};
+
+struct ConvParams {
+    int32_t M, N, K;
+    int32_t Ho, Wo;                 // M = batch * Ho * Wo
+    int32_t H, W, Cin;              // lhs spatial size (undilated) and features
+    int32_t KH, KW;
+    int32_t SH, SW, PH, PW, DH, DW, LH, LW;
+    int32_t xs_b, xs_h, xs_w, xs_c; // lhs strides in elements
+    int32_t ws_r, ws_s, ws_c, ws_n; // rhs strides
+    int32_t os_b, os_h, os_w, os_n; // out strides
+    int32_t c_contig;               // out is row-major [M, N]
+    int32_t tiles_m, tiles_n;
+    uint32_t nepi;                  // number of epilogue steps
+    uint32_t epi_op[CONV_MAX_EPI];
+    uint32_t epi_flags[CONV_MAX_EPI];   // bit1: operand is the left argument
+    uint32_t epi_kind[CONV_MAX_EPI];    // 0 none, 1 scalar, 2 per-feature vector [N], 3 full tensor laid out like out
+};
+
+struct ConvEpiPtrs { const float* p[CONV_MAX_EPI]; };
+
+__device__ __forceinline__ float epi_apply(uint32_t op, float a, float b) {
+    switch (op) {
+        case CEW_ADD_F: return a + b;
+        case CEW_SUB_F: return a - b;
+        case CEW_MUL_F: return a * b;
+        case CEW_DIV_F: return a / b;
+        case CEW_MAX_F: return (a > b || a != a) ? a : b;
+        case CEW_MIN_F: return (a < b || a != a) ? a : b;
+        default:        return a;
+    }
+}
+
+template <int WGM, int WGN, int TM, int TN, bool A_FAST, bool B_FAST>
+__device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
+                                               const float* __restrict__ w, const ConvEpiPtrs& epi,
+                                               const ConvParams& P) {
+    constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, BK = CONV_BK, NT = 64 * WGM * WGN;
+    constexpr int LDA = BK + 4, LDB = BN + 4;
+    __shared__ __attribute__((aligned(16))) float As[BM * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int l32 = lane & 31, half = lane >> 5;
+
+    // Consecutive block ids go to different XCDs (8 of them, each with its own L2). Hand every
+    // XCD a contiguous range of tiles so that the N-tiles of one M-tile share an L2.
+    int tile = blockIdx.x;
+    {
+        const int total = P.tiles_m * P.tiles_n, per = total / 8;
+        if (per > 0 && tile < per * 8) tile = (tile & 7) * per + (tile >> 3);
+    }
+    const int tile_m = tile / P.tiles_n, tile_n = tile - tile_m * P.tiles_n;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int HoWo = P.Ho * P.Wo;
+
+    // ---------------- per-thread load assignment ----------------
+    // A fast: 16-byte vectors along k. A generic: one row, a run of consecutive k.
+    constexpr int A_VPR   = BK / 4;                 // vectors per row
+    constexpr int A_RSTEP = NT / A_VPR;             // rows between a thread's vectors
+    constexpr int A_NV    = BM / A_RSTEP;           // vectors per thread
+    constexpr int A_KG    = NT / BM;                // generic: k groups
+    constexpr int A_KPT   = BK / A_KG;              // generic: k per thread
+    constexpr int A_ROWS  = A_FAST ? A_NV : 1;
+    int a_base[A_ROWS], a_hi0[A_ROWS], a_wi0[A_ROWS];
+#pragma unroll
+    for (int p = 0; p < A_ROWS; ++p) {
+        const int row = A_FAST ? (tid / A_VPR + p * A_RSTEP) : (tid % BM);
+        const int m = m0 + row;
+        if (m < P.M) {
+            const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
+            a_base[p] = b * P.xs_b;
+            a_hi0[p]  = ho * P.SH - P.PH;
+            a_wi0[p]  = wo * P.SW - P.PW;
+        } else {
+            a_base[p] = 0; a_hi0[p] = -(1 << 28); a_wi0[p] = -(1 << 28);
+        }
+    }
+    // position of this thread's first k inside the (ky, kx, c) space, advanced by BK per tile
+    int ak = A_FAST ? (tid % A_VPR) * 4 : (tid / BM) * A_KPT;
+    int ac, as_, ar;
+    {
+        const int rs = ak / P.Cin;
+        ac = ak - rs * P.Cin; ar = rs / P.KW; as_ = rs - ar * P.KW;
+    }
+
+    constexpr int B_VPR   = BN / 4;
+    constexpr int B_RSTEP = NT / B_VPR;
+    constexpr int B_NV    = BK / B_RSTEP;
+    constexpr int B_KG    = NT / BN;                // generic: k groups
+    constexpr int B_KPT   = BK / B_KG;
+
+    f32x4 a_reg[A_FAST ? A_NV : 1];
+    float a_sreg[A_FAST ? 1 : A_KPT];
+    f32x4 b_reg[B_FAST ? B_NV : 1];
+    float b_sreg[B_FAST ? 1 : B_KPT];
+
+    auto a_element_offset = [&](int p, int r, int s, int c, bool& ok) -> int {
+        int hi = a_hi0[p] + r * P.DH, wi = a_wi0[p] + s * P.DW;
+        ok = hi >= 0 && wi >= 0;
+        if (P.LH > 1) { ok = ok && (hi % P.LH == 0); hi /= P.LH; }
+        if (P.LW > 1) { ok = ok && (wi % P.LW == 0); wi /= P.LW; }
+        ok = ok && hi < P.H && wi < P.W;
+        return a_base[p] + hi * P.xs_h + wi * P.xs_w + c * P.xs_c;
+    };
+
+    auto load_tiles = [&](int k0) {
+        // ---- A ----
+        if constexpr (A_FAST) {
+            const bool kok = ak < P.K;
+#pragma unroll
+            for (int p = 0; p < A_NV; ++p) {
+                bool ok;
+                const int off = a_element_offset(p, ar, as_, ac, ok);
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (ok && kok) v = *reinterpret_cast<const f32x4*>(x + off);
+                a_reg[p] = v;
+            }
+        } else {
+            int c = ac, s = as_, r = ar, k = ak;
+#pragma unroll
+            for (int j = 0; j < A_KPT; ++j) {
+                bool ok;
+                const int off = a_element_offset(0, r, s, c, ok);
+                a_sreg[j] = (ok && k < P.K) ? x[off] : 0.f;
+                ++k; ++c;
+                if (c == P.Cin) { c = 0; ++s; if (s == P.KW) { s = 0; ++r; } }
+            }
+        }
+        // ---- B ----
+        if constexpr (B_FAST) {
+            const int n = n0 + (tid % B_VPR) * 4;
+#pragma unroll
+            for (int p = 0; p < B_NV; ++p) {
+                const int k = k0 + tid / B_VPR + p * B_RSTEP;
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (k < P.K && n < P.N) v = *reinterpret_cast<const f32x4*>(w + (int64_t)k * P.N + n);
+                b_reg[p] = v;
+            }
+        } else {
+            const int n = n0 + tid % BN;
+            int k = k0 + (tid / BN) * B_KPT;
+            const int rs = k / P.Cin;
+            int c = k - rs * P.Cin, r = rs / P.KW, s = rs - r * P.KW;
+#pragma unroll
+            for (int j = 0; j < B_KPT; ++j) {
+                b_sreg[j] = (k < P.K && n < P.N) ? w[r * P.ws_r + s * P.ws_s + c * P.ws_c + n * P.ws_n] : 0.f;
+                ++k; ++c;
+                if (c == P.Cin) { c = 0; ++s; if (s == P.KW) { s = 0; ++r; } }
+            }
+        }
+        // advance this thread's A position by one k tile
+        ak += BK; ac += BK;
+        while (ac >= P.Cin) { ac -= P.Cin; ++as_; if (as_ == P.KW) { as_ = 0; ++ar; } }
+    };
+
+    auto store_tiles = [&]() {
+        if constexpr (A_FAST) {
+#pragma unroll
+            for (int p = 0; p < A_NV; ++p) {
+                const int row = tid / A_VPR + p * A_RSTEP, kv = tid % A_VPR;
+                *reinterpret_cast<f32x4*>(&As[row * LDA + kv * 4]) = a_reg[p];
+            }
+        } else {
+            const int row = tid % BM, kb = (tid / BM) * A_KPT;
+#pragma unroll
+            for (int j = 0; j < A_KPT; ++j) As[row * LDA + kb + j] = a_sreg[j];
+        }
+        if constexpr (B_FAST) {
+#pragma unroll
+            for (int p = 0; p < B_NV; ++p) {
+                const int kr = tid / B_VPR + p * B_RSTEP, nv = tid % B_VPR;
+                *reinterpret_cast<f32x4*>(&Bs[kr * LDB + nv * 4]) = b_reg[p];
+            }
+        } else {
+            const int n = tid % BN, kb = (tid / BN) * B_KPT;
+#pragma unroll
+            for (int j = 0; j < B_KPT; ++j) Bs[(kb + j) * LDB + n] = b_sreg[j];
+        }
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    const int ktiles = (P.K + BK - 1) / BK;
+    load_tiles(0);
+    for (int kt = 0; kt < ktiles; ++kt) {
+        store_tiles();
+        __syncthreads();
+        if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
+        // lanes 0-31 consume k = 0..15 of the tile, lanes 32-63 k = 16..31
+#pragma unroll
+        for (int g = 0; g < BK / 8; ++g) {
+            const int kk = half * (BK / 2) + g * 4;
+            f32x4 af[TM];
+            float bf[TN][4];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                af[i] = *reinterpret_cast<const f32x4*>(&As[((wm * TM + i) * 32 + l32) * LDA + kk]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) bf[j][q] = Bs[(kk + q) * LDB + (wn * TN + j) * 32 + l32];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][q], bf[j][q], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // ---------------- epilogue + store ----------------
+    // accumulator element v of a lane: row = 8*(v/4) + 4*half + v%4, column = l32
+    auto out_offset = [&](int m, int n) -> int64_t {
+        if (P.c_contig) return (int64_t)m * P.N + n;
+        const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
+        return (int64_t)b * P.os_b + (int64_t)ho * P.os_h + (int64_t)wo * P.os_w + (int64_t)n * P.os_n;
+    };
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n0 + (wn * TN + j) * 32 + l32;
+        if (n >= P.N) continue;
+        for (uint32_t e = 0; e < P.nepi; ++e) {          // uniform, not unrolled
+            const uint32_t op = P.epi_op[e], kind = P.epi_kind[e];
+            const bool left = (P.epi_flags[e] & 2u) != 0;
+            const float* __restrict__ src = epi.p[e];
+            const float o1 = kind == 1 ? src[0] : kind == 2 ? src[n] : 0.f;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int m = m0 + (wm * TM + i) * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                    float o = o1;
+                    if (kind == 3) o = m < P.M ? src[out_offset(m, n)] : 0.f;
+                    const float y = acc[i][j][v];
+                    acc[i][j][v] = epi_apply(op, left ? o : y, left ? y : o);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + (wm * TM + i) * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                if (m < P.M) out[out_offset(m, n)] = acc[i][j][v];
+            }
+        }
+    }
+}
+
+#define CONV_KERNEL(name, WGM, WGN, TM, TN, AF, BF)                                                         \
+    extern "C" __global__ __launch_bounds__(64 * WGM * WGN) void name(                                       \
+        float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
+        ConvEpiPtrs epi, ConvParams P) {                                                                     \
+        conv_gemm_body<WGM, WGN, TM, TN, AF, BF>(out, x, w, epi, P);                                         \
+    }
+
+// name = conv_gemm_<BM>x<BN>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads)
+#define CONV_TILE(tag, WGM, WGN, TM, TN)                               \
+    CONV_KERNEL(conv_gemm_##tag##_ff, WGM, WGN, TM, TN, true, true)    \
+    CONV_KERNEL(conv_gemm_##tag##_fg, WGM, WGN, TM, TN, true, false)   \
+    CONV_KERNEL(conv_gemm_##tag##_gf, WGM, WGN, TM, TN, false, true)   \
+    CONV_KERNEL(conv_gemm_##tag##_gg, WGM, WGN, TM, TN, false, false)
+
+CONV_TILE(128x128, 2, 2, 2, 2)
+CONV_TILE(128x64, 2, 2, 2, 1)
+CONV_TILE(64x64, 2, 2, 1, 1)
+CONV_TILE(32x32, 1, 1, 1, 1)

@@ -1,0 +1,489 @@
+// Device runtime behind the vkJAX jaxpr interpreter on MI355X: contexts, HBM buffers,
+// gfx950 code objects and recorded sequences, exported through the C ABI declared in
+// include/vkjax_hip.h. Host-only translation unit; kernels live in separate code objects
+// that the caller loads with vkj_module_load.
+#include "vkjax_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    g_last_error = std::string(what) + ": " + hipGetErrorString(e);
+    return (int)e > 0 ? (int)e : VKJ_EINVAL;
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t _e = (expr);                         \
+        if (_e != hipSuccess) return hip_fail(_e, #expr); \
+    } while (0)
+
+constexpr uint32_t MAGIC_CTX = 0x766b4a43, MAGIC_BUF = 0x766b4a42, MAGIC_MOD = 0x766b4a4d,
+                   MAGIC_FN = 0x766b4a46, MAGIC_SEQ = 0x766b4a53;
+
+struct Ctx {
+    uint32_t    magic = MAGIC_CTX;
+    int         device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t  ev_begin = nullptr, ev_end = nullptr;
+};
+
+struct Buf {
+    uint32_t magic = MAGIC_BUF;
+    Ctx*     ctx = nullptr;
+    void*    dptr = nullptr;
+    size_t   nbytes = 0;
+};
+
+struct Mod {
+    uint32_t    magic = MAGIC_MOD;
+    Ctx*        ctx = nullptr;
+    hipModule_t module = nullptr;
+};
+
+struct Fn {
+    uint32_t      magic = MAGIC_FN;
+    Mod*          mod = nullptr;
+    hipFunction_t fn = nullptr;
+    std::string   name;
+};
+
+struct Transfer {
+    Buf*   buf;
+    size_t offset, nbytes;
+    int    slot;
+    void*  staging;    // pinned host memory owned by the sequence
+};
+
+struct Launch {
+    Fn*                  fn;
+    uint32_t             grid[3], block[3], lds;
+    std::vector<uint8_t> kernarg;
+};
+
+struct Seq {
+    uint32_t              magic = MAGIC_SEQ;
+    Ctx*                  ctx = nullptr;
+    bool                  profiling = false;
+    std::vector<Transfer> uploads, downloads;
+    std::vector<Launch>   launches;
+    std::vector<hipEvent_t> stamps;   // profiling: 1 + number of steps
+    int                   stamps_valid = 0;
+};
+
+template <class T>
+T* from_handle(vkj_handle h, uint32_t magic) {
+    T* p = reinterpret_cast<T*>(static_cast<uintptr_t>(h));
+    return (p && p->magic == magic) ? p : nullptr;
+}
+template <class T>
+vkj_handle to_handle(T* p) { return static_cast<vkj_handle>(reinterpret_cast<uintptr_t>(p)); }
+
+int use(Ctx* c) {
+    HIP_TRY(hipSetDevice(c->device));
+    return 0;
+}
+
+int issue_launch(Ctx* c, Launch& l) {
+    size_t size = l.kernarg.size();
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, l.kernarg.data(),
+                     HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+    hipError_t e = hipModuleLaunchKernel(l.fn->fn, l.grid[0], l.grid[1], l.grid[2],
+                                         l.block[0], l.block[1], l.block[2], l.lds, c->stream, nullptr, extra);
+    if (e != hipSuccess) {
+        g_last_error = "launch of " + l.fn->name + ": " + hipGetErrorString(e);
+        return (int)e;
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* vkj_last_error(void) { return g_last_error.c_str(); }
+
+int vkj_device_count(int* count) {
+    if (!count) return fail(VKJ_EINVAL, "vkj_device_count: null output");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) { *count = 0; return hip_fail(e, "hipGetDeviceCount"); }
+    *count = n;
+    return 0;
+}
+
+int vkj_ctx_create(int device, vkj_handle* out) {
+    if (!out) return fail(VKJ_EINVAL, "vkj_ctx_create: null output");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) return fail(VKJ_ENODEV, "vkj_ctx_create: no HIP device available (%s)",
+                                               e != hipSuccess ? hipGetErrorString(e) : "count is 0");
+    if (device < 0 || device >= n) return fail(VKJ_EINVAL, "vkj_ctx_create: device %d out of range [0,%d)", device, n);
+    Ctx* c = new (std::nothrow) Ctx();
+    if (!c) return fail(VKJ_ENOMEM, "vkj_ctx_create: out of host memory");
+    c->device = device;
+    HIP_TRY(hipSetDevice(device));
+    HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    HIP_TRY(hipEventCreate(&c->ev_begin));
+    HIP_TRY(hipEventCreate(&c->ev_end));
+    *out = to_handle(c);
+    return 0;
+}
+
+int vkj_ctx_destroy(vkj_handle h) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    if (!c) return fail(VKJ_EINVAL, "vkj_ctx_destroy: bad context handle");
+    if (int r = use(c)) return r;
+    hipStreamSynchronize(c->stream);
+    hipEventDestroy(c->ev_begin);
+    hipEventDestroy(c->ev_end);
+    hipStreamDestroy(c->stream);
+    c->magic = 0;
+    delete c;
+    return 0;
+}
+
+int vkj_device_props(vkj_handle h, vkj_props* out) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    if (!c || !out) return fail(VKJ_EINVAL, "vkj_device_props: bad argument");
+    hipDeviceProp_t p;
+    HIP_TRY(hipGetDeviceProperties(&p, c->device));
+    memset(out, 0, sizeof(*out));
+    snprintf(out->name, sizeof(out->name), "%s", p.name);
+    snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
+    out->compute_units         = p.multiProcessorCount;
+    out->wavefront_size        = p.warpSize;
+    out->max_threads_per_block = p.maxThreadsPerBlock;
+    out->max_block_dim_x       = p.maxThreadsDim[0];
+    out->lds_bytes_per_block   = (int32_t)p.sharedMemPerBlock;
+    out->clock_khz             = p.clockRate;
+    out->memory_clock_khz      = p.memoryClockRate;
+    out->memory_bus_bits       = p.memoryBusWidth;
+    out->hbm_bytes             = p.totalGlobalMem;
+    return 0;
+}
+
+int vkj_sync(vkj_handle h) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    if (!c) return fail(VKJ_EINVAL, "vkj_sync: bad context handle");
+    if (int r = use(c)) return r;
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return 0;
+}
+
+int vkj_module_load(vkj_handle h, const void* image, size_t nbytes, vkj_handle* out) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    if (!c || !image || !nbytes || !out) return fail(VKJ_EINVAL, "vkj_module_load: bad argument");
+    if (int r = use(c)) return r;
+    Mod* m = new (std::nothrow) Mod();
+    if (!m) return fail(VKJ_ENOMEM, "vkj_module_load: out of host memory");
+    m->ctx = c;
+    hipError_t e = hipModuleLoadData(&m->module, image);
+    if (e != hipSuccess) { delete m; return hip_fail(e, "hipModuleLoadData (is the code object built for this GPU's architecture?)"); }
+    *out = to_handle(m);
+    return 0;
+}
+
+int vkj_module_unload(vkj_handle h, vkj_handle mh) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Mod* m = from_handle<Mod>(mh, MAGIC_MOD);
+    if (!c || !m || m->ctx != c) return fail(VKJ_EINVAL, "vkj_module_unload: bad handle");
+    if (int r = use(c)) return r;
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(hipModuleUnload(m->module));
+    m->magic = 0;
+    delete m;
+    return 0;
+}
+
+int vkj_module_get_function(vkj_handle h, vkj_handle mh, const char* name, vkj_handle* out) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Mod* m = from_handle<Mod>(mh, MAGIC_MOD);
+    if (!c || !m || m->ctx != c || !name || !out) return fail(VKJ_EINVAL, "vkj_module_get_function: bad argument");
+    if (int r = use(c)) return r;
+    Fn* f = new (std::nothrow) Fn();
+    if (!f) return fail(VKJ_ENOMEM, "vkj_module_get_function: out of host memory");
+    f->mod = m;
+    f->name = name;
+    hipError_t e = hipModuleGetFunction(&f->fn, m->module, name);
+    if (e != hipSuccess) {
+        delete f;
+        g_last_error = std::string("kernel '") + name + "' not found in module: " + hipGetErrorString(e);
+        return (int)e;
+    }
+    *out = to_handle(f);   // lives as long as the process; functions are few and tiny
+    return 0;
+}
+
+int vkj_buf_alloc(vkj_handle h, size_t nbytes, vkj_handle* out) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    if (!c || !out) return fail(VKJ_EINVAL, "vkj_buf_alloc: bad argument");
+    if (int r = use(c)) return r;
+    Buf* b = new (std::nothrow) Buf();
+    if (!b) return fail(VKJ_ENOMEM, "vkj_buf_alloc: out of host memory");
+    b->ctx = c;
+    b->nbytes = nbytes;
+    hipError_t e = hipMalloc(&b->dptr, nbytes ? nbytes : 4);
+    if (e != hipSuccess) { delete b; return hip_fail(e, "hipMalloc"); }
+    *out = to_handle(b);
+    return 0;
+}
+
+int vkj_buf_free(vkj_handle h, vkj_handle bh) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
+    if (!c || !b || b->ctx != c) return fail(VKJ_EINVAL, "vkj_buf_free: bad handle");
+    if (int r = use(c)) return r;
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(hipFree(b->dptr));
+    b->magic = 0;
+    delete b;
+    return 0;
+}
+
+int vkj_buf_size(vkj_handle h, vkj_handle bh, size_t* nbytes) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
+    if (!c || !b || b->ctx != c || !nbytes) return fail(VKJ_EINVAL, "vkj_buf_size: bad argument");
+    *nbytes = b->nbytes;
+    return 0;
+}
+
+int vkj_buf_device_ptr(vkj_handle h, vkj_handle bh, uint64_t* addr) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
+    if (!c || !b || b->ctx != c || !addr) return fail(VKJ_EINVAL, "vkj_buf_device_ptr: bad argument");
+    *addr = (uint64_t)(uintptr_t)b->dptr;
+    return 0;
+}
+
+static int check_range(const char* who, Buf* b, size_t offset, size_t nbytes) {
+    if (offset > b->nbytes || nbytes > b->nbytes - offset)
+        return fail(VKJ_EINVAL, "%s: range [%zu, %zu) exceeds the buffer's %zu bytes", who, offset, offset + nbytes, b->nbytes);
+    return 0;
+}
+
+int vkj_buf_memset(vkj_handle h, vkj_handle bh, size_t offset, int value, size_t nbytes) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
+    if (!c || !b || b->ctx != c) return fail(VKJ_EINVAL, "vkj_buf_memset: bad handle");
+    if (int r = check_range("vkj_buf_memset", b, offset, nbytes)) return r;
+    if (int r = use(c)) return r;
+    if (nbytes) HIP_TRY(hipMemsetAsync((char*)b->dptr + offset, value, nbytes, c->stream));
+    return 0;
+}
+
+int vkj_buf_upload(vkj_handle h, vkj_handle bh, size_t offset, const void* host, size_t nbytes) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
+    if (!c || !b || b->ctx != c || (!host && nbytes)) return fail(VKJ_EINVAL, "vkj_buf_upload: bad argument");
+    if (int r = check_range("vkj_buf_upload", b, offset, nbytes)) return r;
+    if (int r = use(c)) return r;
+    if (nbytes) {
+        HIP_TRY(hipMemcpyAsync((char*)b->dptr + offset, host, nbytes, hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(hipStreamSynchronize(c->stream));
+    }
+    return 0;
+}
+
+int vkj_buf_download(vkj_handle h, vkj_handle bh, size_t offset, void* host, size_t nbytes) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
+    if (!c || !b || b->ctx != c || (!host && nbytes)) return fail(VKJ_EINVAL, "vkj_buf_download: bad argument");
+    if (int r = check_range("vkj_buf_download", b, offset, nbytes)) return r;
+    if (int r = use(c)) return r;
+    if (nbytes) {
+        HIP_TRY(hipMemcpyAsync(host, (char*)b->dptr + offset, nbytes, hipMemcpyDeviceToHost, c->stream));
+        HIP_TRY(hipStreamSynchronize(c->stream));
+    }
+    return 0;
+}
+
+int vkj_seq_create(vkj_handle h, int profiling, vkj_handle* out) {
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    if (!c || !out) return fail(VKJ_EINVAL, "vkj_seq_create: bad argument");
+    Seq* s = new (std::nothrow) Seq();
+    if (!s) return fail(VKJ_ENOMEM, "vkj_seq_create: out of host memory");
+    s->ctx = c;
+    s->profiling = profiling != 0;
+    *out = to_handle(s);
+    return 0;
+}
+
+int vkj_seq_destroy(vkj_handle sh) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_destroy: bad handle");
+    if (int r = use(s->ctx)) return r;
+    hipStreamSynchronize(s->ctx->stream);
+    for (auto& t : s->uploads)   if (t.staging) hipHostFree(t.staging);
+    for (auto& t : s->downloads) if (t.staging) hipHostFree(t.staging);
+    for (auto e : s->stamps) hipEventDestroy(e);
+    s->magic = 0;
+    delete s;
+    return 0;
+}
+
+static int record_transfer(const char* who, std::vector<Transfer>& list, Seq* s, vkj_handle bh,
+                           size_t offset, int slot, size_t nbytes) {
+    Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
+    if (!s || !b || b->ctx != s->ctx || slot < 0) return fail(VKJ_EINVAL, "%s: bad argument", who);
+    if (int r = check_range(who, b, offset, nbytes)) return r;
+    if (int r = use(s->ctx)) return r;
+    Transfer t{b, offset, nbytes, slot, nullptr};
+    if (nbytes) HIP_TRY(hipHostMalloc(&t.staging, nbytes, hipHostMallocDefault));
+    list.push_back(t);
+    return 0;
+}
+
+int vkj_seq_record_upload(vkj_handle sh, vkj_handle bh, size_t offset, int slot, size_t nbytes) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_record_upload: bad sequence handle");
+    return record_transfer("vkj_seq_record_upload", s->uploads, s, bh, offset, slot, nbytes);
+}
+
+int vkj_seq_record_download(vkj_handle sh, vkj_handle bh, size_t offset, int slot, size_t nbytes) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_record_download: bad sequence handle");
+    return record_transfer("vkj_seq_record_download", s->downloads, s, bh, offset, slot, nbytes);
+}
+
+int vkj_seq_record_launch(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], const uint32_t block[3],
+                          uint32_t lds_bytes, const void* kernarg, size_t kernarg_bytes,
+                          const vkj_handle* bufs, const uint32_t* buf_arg_offsets,
+                          const uint64_t* buf_byte_offsets, int nbufs) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    Fn*  f = from_handle<Fn>(fh, MAGIC_FN);
+    if (!s || !f || f->mod->ctx != s->ctx || !grid || !block || (!kernarg && kernarg_bytes) || nbufs < 0 ||
+        (nbufs && (!bufs || !buf_arg_offsets)))
+        return fail(VKJ_EINVAL, "vkj_seq_record_launch: bad argument");
+    for (int i = 0; i < 3; i++)
+        if (grid[i] == 0 || block[i] == 0)
+            return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): zero-sized grid or block", f->name.c_str());
+    if ((uint64_t)block[0] * block[1] * block[2] > 1024)
+        return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): more than 1024 threads per block", f->name.c_str());
+    if ((uint64_t)grid[0] * block[0] > 0xFFFFFFFFull || grid[1] > 65535 || grid[2] > 65535)
+        return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): grid too large", f->name.c_str());
+    Launch l;
+    l.fn = f;
+    for (int i = 0; i < 3; i++) { l.grid[i] = grid[i]; l.block[i] = block[i]; }
+    l.lds = lds_bytes;
+    l.kernarg.assign((const uint8_t*)kernarg, (const uint8_t*)kernarg + kernarg_bytes);
+    for (int i = 0; i < nbufs; i++) {
+        Buf* b = from_handle<Buf>(bufs[i], MAGIC_BUF);
+        if (!b || b->ctx != s->ctx) return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): bad buffer handle #%d", f->name.c_str(), i);
+        uint64_t off = buf_byte_offsets ? buf_byte_offsets[i] : 0;
+        if (off > b->nbytes) return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): offset of buffer #%d beyond its end", f->name.c_str(), i);
+        if ((size_t)buf_arg_offsets[i] + 8 > kernarg_bytes || (buf_arg_offsets[i] & 7))
+            return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): pointer slot #%d outside the argument block or misaligned", f->name.c_str(), i);
+        uint64_t addr = (uint64_t)(uintptr_t)b->dptr + off;
+        memcpy(l.kernarg.data() + buf_arg_offsets[i], &addr, 8);
+    }
+    s->launches.push_back(std::move(l));
+    return 0;
+}
+
+int vkj_seq_num_steps(vkj_handle sh, int* uploads, int* launches, int* downloads) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_num_steps: bad handle");
+    if (uploads)   *uploads   = (int)s->uploads.size();
+    if (launches)  *launches  = (int)s->launches.size();
+    if (downloads) *downloads = (int)s->downloads.size();
+    return 0;
+}
+
+int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t flags) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_eval: bad handle");
+    Ctx* c = s->ctx;
+    if (int r = use(c)) return r;
+    const bool up = !(flags & VKJ_EVAL_SKIP_UPLOADS), down = !(flags & VKJ_EVAL_SKIP_DOWNLOADS);
+    auto slot_ok = [&](const Transfer& t) { return t.nbytes == 0 || (host_ptrs && t.slot < nslots && host_ptrs[t.slot]); };
+    if (up)   for (auto& t : s->uploads)   if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for upload slot %d", t.slot);
+    if (down) for (auto& t : s->downloads) if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for download slot %d", t.slot);
+
+    size_t nstamps = 0;
+    if (s->profiling) {
+        nstamps = 3 + s->launches.size();       // begin, after uploads, after each launch, after downloads
+        while (s->stamps.size() < nstamps) {
+            hipEvent_t e;
+            HIP_TRY(hipEventCreate(&e));
+            s->stamps.push_back(e);
+        }
+        s->stamps_valid = 0;
+        HIP_TRY(hipEventRecord(s->stamps[0], c->stream));
+    }
+    if (up) for (auto& t : s->uploads) {
+        if (!t.nbytes) continue;
+        memcpy(t.staging, host_ptrs[t.slot], t.nbytes);
+        HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
+    }
+    if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[1], c->stream));
+    for (size_t i = 0; i < s->launches.size(); i++) {
+        if (int r = issue_launch(c, s->launches[i])) return r;
+        if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[2 + i], c->stream));
+    }
+    if (down) for (auto& t : s->downloads) {
+        if (!t.nbytes) continue;
+        HIP_TRY(hipMemcpyAsync(t.staging, (char*)t.buf->dptr + t.offset, t.nbytes, hipMemcpyDeviceToHost, c->stream));
+    }
+    if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[nstamps - 1], c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    if (down) for (auto& t : s->downloads)
+        if (t.nbytes) memcpy(host_ptrs[t.slot], t.staging, t.nbytes);
+    if (s->profiling) s->stamps_valid = (int)nstamps;
+    return 0;
+}
+
+int vkj_seq_replay(vkj_handle sh, int iters, float* ms_total) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s || iters < 1) return fail(VKJ_EINVAL, "vkj_seq_replay: bad argument");
+    Ctx* c = s->ctx;
+    if (int r = use(c)) return r;
+    HIP_TRY(hipEventRecord(c->ev_begin, c->stream));
+    for (int it = 0; it < iters; it++)
+        for (auto& l : s->launches)
+            if (int r = issue_launch(c, l)) return r;
+    HIP_TRY(hipEventRecord(c->ev_end, c->stream));
+    HIP_TRY(hipEventSynchronize(c->ev_end));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, c->ev_begin, c->ev_end));
+    if (ms_total) *ms_total = ms;
+    return 0;
+}
+
+int vkj_seq_timestamps(vkj_handle sh, float* ms_out, int capacity, int* count) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s || !count) return fail(VKJ_EINVAL, "vkj_seq_timestamps: bad argument");
+    if (!s->profiling) return fail(VKJ_ESTATE, "vkj_seq_timestamps: sequence was created without profiling");
+    *count = s->stamps_valid;
+    if (!ms_out) return 0;
+    if (int r = use(s->ctx)) return r;
+    for (int i = 0; i < s->stamps_valid && i < capacity; i++) {
+        float ms = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms, s->stamps[0], s->stamps[i]));
+        ms_out[i] = ms;
+    }
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,144 @@
+'''The jaxpr interpreter: analyses a closed jaxpr once into device ops and buffers, records
+them into one replayable sequence, and runs it with one native call per invocation.
+
+Same structure and public surface as the reference's JaxprInterpreter
+(vkjax/kompute_jaxpr_interpreter.py:14-102): constructor arguments `(jaxpr, static_argnums,
+profiling, reuse_buffers)`, `.run(*X, return_all=False)`, `.get_profiling_info()`, attributes
+`.jaxpr .static_argnums .bufferpool .all_ops .sequence`. The Kompute manager / tensors /
+sequence are replaced by the HIP runtime behind include/vkjax_hip.h.
+'''
+import os
+import typing as tp
+
+import numpy as np
+
+from . import fusion
+from . import hip
+from . import ops
+from .buffers import BufferPool, PlanOnlyDevice, to_device_words, view_or_convert_from_32bit
+from .minijax import core, tree_util
+
+
+class JaxprInterpreter:
+    def __init__(self, jaxpr, static_argnums: tp.Tuple[int, ...] = (), profiling: bool = False,
+                 reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False):
+        self.jaxpr          = jaxpr
+        self.static_argnums = tuple(static_argnums)
+        self.profiling      = profiling
+        self.fuse           = fuse
+        #plan_only builds ops, buffers and launch parameters without touching a GPU; such an
+        #interpreter cannot run
+        self.mgr            = PlanOnlyDevice() if plan_only else hip.Device.get()
+        self.workgroup_size = get_maximum_workgroup_size(self.mgr)
+        self.bufferpool     = BufferPool(self.mgr, self.workgroup_size, reuse_buffers)
+        self.sequence       = None
+        self.analyze_closed_jaxpr(jaxpr)
+
+    def analyze_closed_jaxpr(self, jaxpr):
+        '''Starts the analysis of the top level jaxpr.
+           Records operations into a sequence and creates required buffers.'''
+        assert len(jaxpr.consts) == len(jaxpr.jaxpr.constvars)
+        for constvar, constval in zip(jaxpr.jaxpr.constvars, jaxpr.consts):
+            b = self.bufferpool.get_buffer(constvar)
+            self.bufferpool.mark_buffer_as_constant(b, constvar, value=np.asarray(constval))
+
+        for v in list(jaxpr.jaxpr.invars) + list(jaxpr.jaxpr.outvars):
+            b = self.bufferpool.get_buffer(v)
+            if b is None:
+                continue
+            #inputs and outputs own their storage: it is never handed to another variable
+            self.bufferpool.mark_buffer_as_constant(b, v, None)
+
+        self.input_buffers  = [self.bufferpool.get_buffer(v) for v in jaxpr.jaxpr.invars]
+        self.all_ops        = ops.analyze_jaxpr(self.bufferpool, jaxpr.jaxpr)
+        if self.fuse:
+            self.all_ops    = fusion.fuse_ops(self.all_ops, self.bufferpool, jaxpr.jaxpr.outvars)
+        self.output_buffers = [self.bufferpool.get_buffer(v) for v in jaxpr.jaxpr.outvars]
+        self.bufferpool.create_tensors()
+        #lower every op now so that unsupported layouts fail at build time, not at run time
+        self.launches = [op.launch for op in self.all_ops]
+
+        if isinstance(self.mgr, PlanOnlyDevice):
+            return
+        self.sequence = self.mgr.sequence(profiling=self.profiling)
+        self._input_slots = []
+        for b in self.input_buffers:
+            self._input_slots.append(self.sequence.record_upload(b.tensor, b.nbytes()) if b is not None else None)
+        for op, launch in zip(self.all_ops, self.launches):
+            bufs = [((b.tensor if b is not None else None), off) for b, off in launch.buffers]
+            for (b, _), (t, _) in zip(launch.buffers, bufs):
+                assert b is None or t is not None, f'{op}: buffer without storage'
+            self.sequence.record_launch(launch.kernel, launch.grid, launch.block, bufs, launch.params, launch.lds)
+        self._output_slots = []
+        self._output_arrays = []
+        for b in self.output_buffers:
+            if b is None:
+                self._output_slots.append(None)
+                self._output_arrays.append(None)
+                continue
+            self._output_slots.append(self.sequence.record_download(b.tensor, b.nbytes()))
+            self._output_arrays.append(np.zeros(b.size, dtype=np.uint32))
+
+    def _flatten_args(self, X):
+        X = tree_util.tree_leaves([x for i, x in enumerate(X) if i not in self.static_argnums])
+        if len(self.input_buffers) != len(X):
+            raise TypeError(f'Expected {len(self.input_buffers)} input arguments, received {len(X)}')
+        return X
+
+    def run(self, *X, return_all=False):
+        '''Executes a previously recorded sequence with actual data'''
+        X = self._flatten_args(X)
+        if self.sequence is None:
+            raise RuntimeError('this interpreter was built with plan_only=True and has no device to run on')
+        host = [None] * self.sequence.n_slots
+        keep = []
+        for slot, x, var in zip(self._input_slots, X, self.jaxpr.jaxpr.invars):
+            if slot is None:
+                continue
+            words = to_device_words(np.asarray(x), core.canonicalize_dtype(var.aval.dtype))
+            if words.size != int(np.prod(var.aval.shape, dtype=np.int64)):
+                raise TypeError(f'argument of shape {np.shape(x)} does not match the traced shape {var.aval.shape}')
+            host[slot] = words
+            keep.append(words)
+        for slot, arr in zip(self._output_slots, self._output_arrays):
+            if slot is not None:
+                host[slot] = arr
+        self.sequence.eval(host)
+
+        output_values = []
+        for b, arr in zip(self.output_buffers, self._output_arrays):
+            if b is None:
+                output_values.append(None)
+                continue
+            output_values.append(view_or_convert_from_32bit(arr.copy(), b.dtype).reshape(b.shape))
+        output_values = tuple(output_values)
+        if not return_all:
+            return output_values
+        all_arrays = [(var, buf.numpy() if buf is not None else None) for var, buf in self.bufferpool.buffers.items()]
+        return output_values, dict(all_arrays)
+
+    def upload_inputs(self, *X):
+        '''Copy arguments into their HBM buffers without running (for measurements with resident inputs).'''
+        X = self._flatten_args(X)
+        for b, x, var in zip(self.input_buffers, X, self.jaxpr.jaxpr.invars):
+            if b is not None and b.size:
+                b.tensor.upload(to_device_words(np.asarray(x), core.canonicalize_dtype(var.aval.dtype)))
+
+    def replay(self, iters: int = 1) -> float:
+        '''Run only the kernels of the recorded sequence `iters` times on whatever the input
+        buffers hold; returns the elapsed device time in milliseconds.'''
+        return self.sequence.replay(iters)
+
+    def read_outputs(self):
+        return tuple(b.numpy() if b is not None else None for b in self.output_buffers)
+
+    def get_profiling_info(self):
+        timestamps = self.sequence.get_timestamps()
+        deltas     = np.diff(timestamps)
+        labels     = ['data2device'] + [op.equation for op in self.all_ops] + ['data2host']
+        return list(zip(labels, deltas))
+
+
+def get_maximum_workgroup_size(mgr) -> int:
+    devprops = mgr.get_device_properties()
+    return min(devprops['max_work_group_invocations'], devprops['max_work_group_size'][0])

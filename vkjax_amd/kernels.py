@@ -1,0 +1,385 @@
+'''Launch descriptors for the gfx950 kernels.
+
+Where the reference turned an op into SPIR-V by pasting shapes into GLSL text and compiling it
+at run time (vkjax/shaders.py:16-42, vkjax/ops.py:36-41), the kernels here are built ahead of
+time and take shapes and strides as kernel arguments. Each function below lays out the argument
+block of one kernel (a struct of 32-bit fields that follows the pointer arguments, mirroring the
+`struct ...Params` in vkjax_amd/csrc/kernels/*.hip) and picks grid, block and kernel variant.
+'''
+import os
+import re
+import typing as tp
+
+import numpy as np
+
+from .buffers import Buffer
+
+_KDIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc', 'kernels')
+
+
+def _read_opcodes() -> tp.Dict[str, int]:
+    text = open(os.path.join(_KDIR, 'ew_opcodes.h')).read()
+    return {m.group(1): int(m.group(2)) for m in re.finditer(r'^EW_OP\((\w+),\s*(\d+)\)', text, re.M)}
+
+
+EW = _read_opcodes()
+EW_MAX_STEPS = 8
+CONV_MAX_EPI = 6
+BLOCK = 256
+
+
+class Launch(tp.NamedTuple):
+    kernel:  str
+    grid:    tp.Tuple[int, int, int]
+    block:   tp.Tuple[int, int, int]
+    buffers: tp.List[tp.Tuple[tp.Optional[Buffer], int]]     #(buffer, byte offset) in argument order
+    params:  bytes
+    lds:     int = 0
+    #algorithmic work of this launch, for roofline accounting
+    bytes_moved: int = 0
+    flops:       int = 0
+
+
+def _u32(*values) -> bytes:
+    return np.asarray([int(v) & 0xFFFFFFFF for v in values], dtype=np.uint32).tobytes()
+
+
+def _i32(*values) -> bytes:
+    return np.asarray([int(v) for v in values], dtype=np.int32).tobytes()
+
+
+def _pad(seq, n, fill=0):
+    seq = list(seq)
+    assert len(seq) <= n, (seq, n)
+    return seq + [fill] * (n - len(seq))
+
+
+def _cdiv(a, b):
+    return -(-int(a) // int(b))
+
+
+def row_major_strides(shape) -> tp.Tuple[int, ...]:
+    strides, acc = [], 1
+    for s in reversed(shape):
+        strides.append(acc)
+        acc *= int(s)
+    return tuple(reversed(strides))
+
+
+# --------------------------------------------------------------------------- element-wise chains
+
+class EwOperand(tp.NamedTuple):
+    '''An array read by an element-wise chain: element `coords` of the output reads
+    buffer[offset + sum(coords * strides)] (strides in elements, one per output dim).'''
+    buffer:  Buffer
+    offset:  int
+    strides: tp.Tuple[int, ...]
+
+
+class EwStep(tp.NamedTuple):
+    op:           int
+    operand:      tp.Optional[EwOperand] = None
+    operand_left: bool = False
+    imm:          int = 0
+
+
+class EwChain:
+    '''out = step_n(... step_1(first) ...) over `shape`.'''
+    def __init__(self, out: Buffer, shape, first: EwOperand, steps: tp.Sequence[EwStep]):
+        self.out, self.shape, self.first, self.steps = out, tuple(int(s) for s in shape), first, list(steps)
+
+    def operands(self) -> tp.List[tp.Optional[EwOperand]]:
+        return [self.first] + [s.operand for s in self.steps]
+
+
+def broadcast_operand(buf: Buffer, out_shape) -> EwOperand:
+    '''Trailing-aligned numpy-style broadcast of `buf` to `out_shape` (reference: vkjax/ops.py:160-184).'''
+    out_shape = tuple(out_shape)
+    in_shape  = tuple(buf.shape)
+    if len(in_shape) > len(out_shape):
+        raise ValueError(f'Cannot broadcast from {in_shape} to {out_shape}')
+    in_strides = row_major_strides(in_shape)
+    strides    = [0] * len(out_shape)
+    for i in range(1, len(in_shape) + 1):
+        old, new = in_shape[-i], out_shape[-i]
+        if old != new and old != 1:
+            raise ValueError(f'Cannot broadcast from {in_shape} to {out_shape}')
+        strides[-i] = in_strides[-i] if old == new and old != 1 else 0
+    return EwOperand(buf, 0, tuple(strides))
+
+
+def _collapse(shape, stride_sets):
+    '''Drop size-1 dims and merge neighbours that every operand walks contiguously.'''
+    dims    = [(s, [st[i] for st in stride_sets]) for i, s in enumerate(shape) if s != 1]
+    if not dims:
+        return [1], [[0] for _ in stride_sets]
+    merged = [dims[0]]
+    for size, strides in dims[1:]:
+        psize, pstrides = merged[-1]
+        if all(ps == s * size for ps, s in zip(pstrides, strides)):
+            merged[-1] = (psize * size, strides)
+        else:
+            merged.append((size, strides))
+    out_dims    = [m[0] for m in merged]
+    out_strides = [[m[1][k] for m in merged] for k in range(len(stride_sets))]
+    return out_dims, out_strides
+
+
+def lower_ew_chain(chain: EwChain) -> Launch:
+    operands = chain.operands()
+    nsteps   = len(operands)
+    if nsteps > EW_MAX_STEPS:
+        raise ValueError(f'element-wise chain of {nsteps} steps exceeds the kernel limit of {EW_MAX_STEPS}')
+    n = int(np.prod(chain.shape, dtype=np.int64))
+    present = [o for o in operands if o is not None]
+    #the output is walked contiguously; include its strides so that merging respects it
+    out_strides = row_major_strides(chain.shape)
+    dims, strides = _collapse(chain.shape, [out_strides] + [o.strides for o in present])
+    if len(dims) > 4:
+        raise NotImplementedError(f'element-wise access pattern with {len(dims)} irreducible dimensions: {chain.shape}')
+    ndim    = len(dims)
+    strides = strides[1:]
+    vec = 4
+    if n % 4 or dims[-1] % 4:
+        vec = 1
+    for o, st in zip(present, strides):
+        if st[-1] not in (0, 1):
+            vec = 1
+        elif st[-1] == 1 and (o.offset % 4 or any(s % 4 for s in st[:-1])):
+            vec = 1
+    ops, flags, imms, stride_rows, buffers = [0], [1], [0], [], []
+    it = iter(strides)
+    for k, o in enumerate(operands):
+        if k > 0:
+            step = chain.steps[k - 1]
+            ops.append(step.op)
+            flags.append((1 if o is not None else 0) | (2 if step.operand_left else 0))
+            imms.append(step.imm)
+        if o is None:
+            stride_rows.append([0, 0, 0, 0])
+            buffers.append((None, 0))
+        else:
+            stride_rows.append(_pad(next(it), 4))
+            buffers.append((o.buffer, o.offset * 4))
+    while len(stride_rows) < EW_MAX_STEPS:
+        stride_rows.append([0, 0, 0, 0])
+        buffers.append((None, 0))
+    params = (_u32(n, ndim, *_pad(dims, 4, 1), nsteps, *_pad(ops, EW_MAX_STEPS), *_pad(flags, EW_MAX_STEPS),
+                   *_pad(imms, EW_MAX_STEPS))
+              + _i32(*[s for row in stride_rows for s in row]))
+    nbytes = 4 * n + sum(4 * min(n, o.buffer.size) for o in present)
+    return Launch(f'ew_chain_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                  [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
+
+
+def iota(out: Buffer, dimension: int) -> Launch:
+    n     = out.size
+    inner = int(np.prod(out.shape[dimension + 1:], dtype=np.int64))
+    size  = out.shape[dimension]
+    return Launch('iota_nd', (_cdiv(n, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0)],
+                  _u32(n, inner, size, int(out.dtype == np.float32)), bytes_moved=4 * n)
+
+
+def fill(out: Buffer, word: int) -> Launch:
+    n = out.size
+    return Launch('fill_u32', (_cdiv(n, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0)], _u32(n, word), bytes_moved=4 * n)
+
+
+def concat_part(out: Buffer, part: Buffer, dimension: int, offset_along_dim: int) -> Launch:
+    inner      = int(np.prod(out.shape[dimension + 1:], dtype=np.int64))
+    part_inner = part.shape[dimension] * inner
+    out_inner  = out.shape[dimension] * inner
+    n = part.size
+    return Launch('concat_part', (_cdiv(n, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (part, 0)],
+                  _u32(n, part_inner, out_inner, offset_along_dim * inner), bytes_moved=8 * n)
+
+
+# --------------------------------------------------------------------------- conv / dot
+
+class ConvGeometry(tp.NamedTuple):
+    '''Implicit-GEMM view of a convolution or matrix product (see csrc/kernels/conv_gemm.hip).'''
+    batch: int; Ho: int; Wo: int; N: int
+    H: int; W: int; Cin: int; KH: int; KW: int
+    SH: int = 1; SW: int = 1; PH: int = 0; PW: int = 0; DH: int = 1; DW: int = 1; LH: int = 1; LW: int = 1
+    xs: tp.Tuple[int, int, int, int] = (0, 0, 0, 1)      #lhs strides: batch, y, x, feature
+    ws: tp.Tuple[int, int, int, int] = (0, 0, 0, 1)      #rhs strides: ky, kx, in feature, out feature
+    os: tp.Tuple[int, int, int, int] = (0, 0, 0, 1)      #out strides: batch, y, x, feature
+
+    @property
+    def M(self): return self.batch * self.Ho * self.Wo
+    @property
+    def K(self): return self.KH * self.KW * self.Cin
+
+
+class ConvEpilogueStep(tp.NamedTuple):
+    op:           int
+    kind:         int                    #1 scalar, 2 per-feature vector [N], 3 full tensor laid out like the output
+    operand:      Buffer
+    operand_left: bool = False
+
+
+#(tag, BM, BN, threads, resident blocks per CU, relative MFMA efficiency of the tile shape)
+CONV_TILES = (('128x128', 128, 128, 256, 1, 1.00), ('128x64', 128, 64, 256, 1, 0.85),
+              ('64x64', 64, 64, 256, 3, 0.60), ('32x32', 32, 32, 64, 12, 0.30))
+
+#tests set this to a tile tag to exercise every kernel variant irrespective of the heuristic
+FORCE_CONV_TILE: tp.Optional[str] = None
+
+
+def choose_conv_tile(M: int, N: int, compute_units: int = 256):
+    '''Smallest estimated time: tiles are dealt out over the CUs, a tile costs BM*BN / efficiency,
+    and a block of one wave can drive only one of a CU's four MFMA units.'''
+    if FORCE_CONV_TILE is not None:
+        return next(t[:4] for t in CONV_TILES if t[0] == FORCE_CONV_TILE)
+    best, best_time = None, None
+    for tag, bm, bn, nt, occupancy, eff in CONV_TILES:
+        tiles   = _cdiv(M, bm) * _cdiv(N, bn)
+        per_cu  = _cdiv(tiles, compute_units)
+        simd    = min(1.0, (nt / 256) * min(occupancy, per_cu))
+        time    = per_cu * bm * bn / (eff * simd)
+        if best_time is None or time < best_time:
+            best, best_time = (tag, bm, bn, nt), time
+    return best
+
+
+def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: tp.Sequence[ConvEpilogueStep] = (),
+              compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0) -> Launch:
+    if len(epilogue) > CONV_MAX_EPI:
+        raise ValueError('too many epilogue steps')
+    M, N, K = g.M, g.N, g.K
+    for name, extent in (('lhs', lhs.size), ('rhs', rhs.size), ('out', out.size)):
+        if extent >= 2**31:
+            raise NotImplementedError(f'conv/dot {name} operand with {extent} elements exceeds 32-bit indexing')
+    tag, bm, bn, nt = choose_conv_tile(M, N, compute_units)
+    a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0
+              and all(s % 4 == 0 for s in g.xs[:3]))
+    b_fast = (g.ws[3] == 1 and N % 4 == 0 and rhs_offset % 4 == 0
+              and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
+    c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
+    tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
+    kinds = [e.kind for e in epilogue]
+    params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW, g.LH, g.LW,
+                   *g.xs, *g.ws, *g.os, int(c_contig), tiles_m, tiles_n)
+              + _u32(len(epilogue), *_pad([e.op for e in epilogue], CONV_MAX_EPI),
+                     *_pad([2 if e.operand_left else 0 for e in epilogue], CONV_MAX_EPI), *_pad(kinds, CONV_MAX_EPI)))
+    buffers = [(out, 0), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
+    buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
+    kernel  = f'conv_gemm_{tag}_{"f" if a_fast else "g"}{"f" if b_fast else "g"}'
+    nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue)
+    return Launch(kernel, (tiles_m * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
+                  bytes_moved=nbytes, flops=2 * M * N * K)
+
+
+# --------------------------------------------------------------------------- reductions
+
+RED = dict(reduce_sum=0, reduce_prod=1, reduce_max=2, reduce_min=3, argmax=4, argmin=5)
+_RTYPE = {np.dtype('float32'): 0, np.dtype('int32'): 1, np.dtype('uint32'): 2, np.dtype('bool'): 2}
+
+
+def _pow2_at_least(x: int) -> int:
+    p = 1
+    while p < x:
+        p *= 2
+    return p
+
+
+def reduce_3d(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str) -> Launch:
+    TI = min(64, _pow2_at_least(inner))
+    TR = BLOCK // TI
+    if outer > 65535:
+        raise NotImplementedError(f'reduction with {outer} outer rows and inner size {inner}')
+    params = _u32(outer, R, inner, RED[op], _RTYPE[inp.dtype], TI, TR)
+    return Launch('reduce_3d', (_cdiv(inner, TI), outer, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
+                  bytes_moved=4 * (inp.size + out.size))
+
+
+def reduce_general(out: Buffer, inp: Buffer, kept, reduced, op: str) -> Launch:
+    '''kept / reduced: lists of (size, stride) in row-major order of the output / of the reduce index.'''
+    if len(kept) > 4 or len(reduced) > 4:
+        raise NotImplementedError('reduction over more than 4 separate dimension groups')
+    n_out = int(np.prod([k[0] for k in kept], dtype=np.int64))
+    n_red = int(np.prod([r[0] for r in reduced], dtype=np.int64))
+    params = _u32(n_out, n_red, RED[op], _RTYPE[inp.dtype], len(kept), len(reduced),
+                  *_pad([k[0] for k in kept], 4, 1), *_pad([k[1] for k in kept], 4),
+                  *_pad([r[0] for r in reduced], 4, 1), *_pad([r[1] for r in reduced], 4))
+    return Launch('reduce_general', (_cdiv(n_out, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
+                  bytes_moved=4 * (inp.size + out.size))
+
+
+def pool(out: Buffer, inp: Buffer, op: str, window, strides, pad_low, dilation) -> Launch:
+    rank = len(inp.shape)
+    if rank > 4:
+        raise NotImplementedError('window reductions over more than 4 dimensions')
+    lead     = 4 - rank
+    in_dims  = [1] * lead + list(inp.shape)
+    out_dims = [1] * lead + list(out.shape)
+    window   = [1] * lead + list(window)
+    strides  = [1] * lead + list(strides)
+    dilation = [1] * lead + list(dilation)
+    pad_low  = [0] * lead + list(pad_low)
+    n   = out.size
+    vec = 4 if (window[3] == 1 and strides[3] == 1 and pad_low[3] == 0 and in_dims[3] % 4 == 0
+                and in_dims[3] == out_dims[3]) else 1
+    params = _u32(n, RED[op], _RTYPE[inp.dtype], *in_dims, *out_dims, *window, *strides, *dilation) + _i32(*pad_low)
+    return Launch(f'pool_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
+                  bytes_moved=4 * (inp.size + out.size))
+
+
+# --------------------------------------------------------------------------- gather / scatter / rng
+
+IDX_MAX_RANK = 6
+
+
+def gather_rows(out: Buffer, table: Buffer, idx: Buffer, n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1) -> Launch:
+    vec = 4 if row_len % 4 == 0 else 1
+    total = n_idx * (row_len // vec)
+    return Launch(f'gather_rows_v{vec}', (_cdiv(total, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (table, 0), (idx, 0)],
+                  _u32(n_idx, row_len, n_rows, idx_stride), bytes_moved=4 * (2 * n_idx * row_len + n_idx))
+
+
+def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, collapsed, start_index_map, slice_sizes) -> Launch:
+    out_rank, op_rank = len(out.shape), len(operand.shape)
+    if max(out_rank, op_rank, len(indices.shape)) > IDX_MAX_RANK:
+        raise NotImplementedError('gather with rank > 6')
+    batch_dims = list(indices.shape[:-1])
+    params = _u32(out.size, out_rank, op_rank, indices.shape[-1],
+                  *_pad(out.shape, IDX_MAX_RANK, 1), *_pad([int(d in offset_dims) for d in range(out_rank)], IDX_MAX_RANK),
+                  *_pad(operand.shape, IDX_MAX_RANK, 1), *_pad(row_major_strides(operand.shape), IDX_MAX_RANK),
+                  *_pad(slice_sizes, IDX_MAX_RANK, 1), *_pad([int(d in collapsed) for d in range(op_rank)], IDX_MAX_RANK),
+                  *_pad(start_index_map, IDX_MAX_RANK), *_pad(batch_dims, IDX_MAX_RANK, 1), len(batch_dims))
+    return Launch('gather_general', (_cdiv(out.size, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (operand, 0), (indices, 0)],
+                  params, bytes_moved=4 * (2 * out.size + indices.size))
+
+
+def scatter_add_rows(out: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1) -> Launch:
+    total = n_idx * row_len
+    return Launch('scatter_add_rows', (_cdiv(total, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (idx, 0), (updates, 0)],
+                  _u32(n_idx, row_len, n_rows, idx_stride, int(out.dtype == np.float32)),
+                  bytes_moved=4 * (total + n_idx + out.size))
+
+
+def scatter_add_general(out: Buffer, indices: Buffer, updates: Buffer, update_window_dims, inserted_window_dims,
+                        scatter_dims_to_operand_dims) -> Launch:
+    upd_rank, op_rank = len(updates.shape), len(out.shape)
+    if max(upd_rank, op_rank, len(indices.shape)) > IDX_MAX_RANK:
+        raise NotImplementedError('scatter-add with rank > 6')
+    window_dims = [updates.shape[d] for d in update_window_dims]
+    it = iter(window_dims)
+    window_sizes = [1 if d in inserted_window_dims else next(it) for d in range(op_rank)]
+    batch_dims = list(indices.shape[:-1])
+    params = _u32(updates.size, upd_rank, op_rank, indices.shape[-1], int(out.dtype == np.float32),
+                  *_pad(updates.shape, IDX_MAX_RANK, 1), *_pad([int(d in update_window_dims) for d in range(upd_rank)], IDX_MAX_RANK),
+                  *_pad(out.shape, IDX_MAX_RANK, 1), *_pad(row_major_strides(out.shape), IDX_MAX_RANK),
+                  *_pad([int(d in inserted_window_dims) for d in range(op_rank)], IDX_MAX_RANK),
+                  *_pad(window_sizes, IDX_MAX_RANK, 1), *_pad(scatter_dims_to_operand_dims, IDX_MAX_RANK),
+                  *_pad(batch_dims, IDX_MAX_RANK, 1))
+    return Launch('scatter_add_general', (_cdiv(max(updates.size, 1), BLOCK), 1, 1), (BLOCK, 1, 1),
+                  [(out, 0), (indices, 0), (updates, 0)], params, bytes_moved=4 * (updates.size + indices.size + out.size))
+
+
+def threefry2x32(out0: Buffer, out1: Buffer, key0: Buffer, key1: Buffer, x0: Buffer, x1: Buffer, key_is_scalar: bool) -> Launch:
+    n   = x0.size
+    vec = 4 if n % 4 == 0 else 1
+    return Launch(f'threefry2x32_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                  [(out0, 0), (out1, 0), (key0, 0), (key1, 0), (x0, 0), (x1, 0)], _u32(n, int(key_is_scalar)),
+                  bytes_moved=16 * n)

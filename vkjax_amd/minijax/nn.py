@@ -1,0 +1,25 @@
+'''Neural-network helpers as they appear in traced programs (relu under a custom-jvp
+call, softmax as max / sub / exp / sum / div), so that the device path sees the same
+primitive sequences as with `jax.nn`.'''
+import numpy as np
+
+from . import lax, numpy as mnp
+from .tracer import custom_jvp
+
+
+@custom_jvp
+def relu(x):
+    return mnp.maximum(x, 0)
+
+
+def softmax(x, axis=-1):
+    unnormalized = mnp.exp(x - lax.stop_gradient(mnp.max(x, axis, keepdims=True)))
+    return unnormalized / mnp.sum(unnormalized, axis, keepdims=True)
+
+
+def batch_norm_inference(x, scale, shift, mean, var, eps=1e-5):
+    '''Inference-mode batch norm over the trailing (channel) axis, written the way
+    flax/haiku modules of the period lower it: the per-channel factor first, then three
+    full-size broadcasting passes.'''
+    inv = scale * lax.rsqrt(var + np.float32(eps))
+    return (x - mean) * inv + shift

@@ -1,0 +1,62 @@
+'''Threefry-based random numbers with the counter layout of JAX's original
+(non-partitionable) implementation: counters are `iota(n)`, the first half feeds
+word 0 and the second half word 1 of the block function; odd sizes are padded with one
+zero counter and trimmed. `split(key, n)` is `threefry(key, iota(2n)).reshape(n, 2)`.
+(Primitive: reference vkjax/ops.py:550-560, vkjax/shaders/threefry2x32.comp.)'''
+import numpy as np
+
+from . import lax, numpy as mnp
+from .tracer import Tracer
+
+
+def PRNGKey(seed: int) -> np.ndarray:
+    seed = int(seed)
+    return np.array([(seed >> 32) & 0xFFFFFFFF, seed & 0xFFFFFFFF], dtype=np.uint32)
+
+
+def _key_halves(key):
+    if not isinstance(key, Tracer):
+        key = np.asarray(key, np.uint32)
+        return key[0], key[1]
+    k0 = lax.reshape(lax.slice(key, (0,), (1,)), ())
+    k1 = lax.reshape(lax.slice(key, (1,), (2,)), ())
+    return k0, k1
+
+
+def threefry_2x32(key, count):
+    '''Apply the block function to a flat uint32 counter array of any length.'''
+    k0, k1 = _key_halves(key)
+    n      = int(np.prod(count.shape))
+    flat   = mnp.reshape(count, (-1,))
+    odd    = n % 2
+    if odd:
+        flat = mnp.concatenate([flat, np.zeros((1,), np.uint32)])
+    x0, x1 = mnp.split(flat, 2)
+    y0, y1 = lax.threefry2x32(k0, k1, x0, x1)
+    out    = mnp.concatenate([y0, y1])
+    if odd:
+        out = lax.slice(out, (0,), (n,))
+    return mnp.reshape(out, count.shape)
+
+
+def split(key, num: int = 2):
+    counts = lax.iota(np.uint32, num * 2)
+    return mnp.reshape(threefry_2x32(key, counts), (num, 2))
+
+
+def random_bits(key, shape):
+    size = int(np.prod(shape, dtype=np.int64))
+    bits = threefry_2x32(key, lax.iota(np.uint32, size))
+    return mnp.reshape(bits, tuple(shape))
+
+
+def uniform(key, shape=(), dtype=np.float32, minval=0.0, maxval=1.0):
+    if np.dtype(dtype) != np.float32:
+        raise NotImplementedError('uniform: float32 only')
+    shape  = tuple(shape)
+    bits   = random_bits(key, shape)
+    #23 random mantissa bits under the exponent of 1.0 give a float in [1, 2)
+    fbits  = lax.bitwise_or(lax.shift_right_logical(bits, np.uint32(32 - 23)), np.uint32(0x3F800000))
+    floats = lax.sub(lax.bitcast_convert_type(fbits, np.float32), np.float32(1.0))
+    scaled = lax.add(lax.mul(floats, np.float32(maxval - minval)), np.float32(minval))
+    return lax.max(np.float32(minval), mnp.reshape(scaled, shape))

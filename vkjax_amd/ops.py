@@ -1,0 +1,614 @@
+'''Primitive dispatch: jaxpr equation -> list of device ops.
+
+Same contract as the reference's vkjax/ops.py: `analyze_jaxpr(bufferpool, jaxpr)` looks up one
+module-level function per primitive name (`-` replaced by `_`), each taking
+`(bufferpool, equation)` and returning a list of `Op`; unknown primitives raise
+NotImplementedError(equation); equations whose outputs are all dropped are skipped
+(reference: vkjax/ops.py:52-65). The accepted parameters follow the reference's functions and
+are widened where the kernels allow it (any-rank transpose, iota along any dimension,
+n-operand concatenate on any axis, general scatter-add, reduce_window_sum).
+
+Instead of SPIR-V bytes an Op carries a launch descriptor for an ahead-of-time built gfx950
+kernel. Element-wise work is expressed as an `EwChain` so that neighbouring element-wise ops
+can later be merged into one launch; broadcasts, slices, transposes and reversals are read
+through strides inside that kernel and never materialised on their own unless they are the
+whole op.
+'''
+import typing as tp
+
+import numpy as np
+
+from . import kernels as K
+from .buffers import Buffer, BufferPool
+from .kernels import EW, EwChain, EwOperand, EwStep, Launch
+from .minijax import core
+
+
+class Op:
+    '''One device launch. `buffers` lists the device arrays it touches in kernel-argument
+    order (entries can be None), `shader` names the kernel, `equation` is the jaxpr equation it
+    came from (or a label string for helper launches), as in the reference's Op tuple
+    (vkjax/ops.py:28-41).'''
+    __slots__ = ('equation', 'chain', '_launch', 'conv')
+
+    def __init__(self, equation, launch: tp.Optional[Launch] = None, chain: tp.Optional[EwChain] = None, conv=None):
+        self.equation = equation
+        self.chain    = chain
+        self._launch  = launch
+        self.conv     = conv          #(out, lhs, rhs, geometry, epilogue list) for conv/dot ops, so a fusion pass can extend it
+
+    @property
+    def launch(self) -> Launch:
+        if self._launch is None:
+            if self.chain is not None:
+                self._launch = K.lower_ew_chain(self.chain)
+            else:
+                out, lhs, rhs, geom, epilogue = self.conv
+                self._launch = K.conv_gemm(out, lhs, rhs, geom, epilogue)
+        return self._launch
+
+    def invalidate(self):
+        self._launch = None
+
+    @property
+    def buffers(self) -> tp.List[tp.Optional[Buffer]]:
+        return [b for b, _ in self.launch.buffers]
+
+    @property
+    def shader(self) -> str:
+        return self.launch.kernel
+
+    @property
+    def workgroup(self):
+        return self.launch.grid
+
+    def __repr__(self):
+        return f'Op({self.shader}, {self.equation})'
+
+
+def analyze_jaxpr(bufferpool: BufferPool, jaxpr) -> tp.List[Op]:
+    '''Analyzes (possibly inner) jaxprs'''
+    all_ops = []
+    for eq in jaxpr.eqns:
+        if all(core.is_dropped(v) for v in eq.outvars):
+            continue
+        opname = eq.primitive.name.replace('-', '_')
+        method = globals().get(opname, None)
+        if method is None or not callable(method) or opname.startswith('_'):
+            raise NotImplementedError(eq)
+        all_ops += method(bufferpool, eq)
+    return all_ops
+
+
+# ------------------------------------------------------------------ dtype helpers
+
+_F, _I, _U, _B = 'f', 'i', 'u', 'b'
+
+
+def _kind(dtype) -> str:
+    dtype = np.dtype(dtype)
+    if dtype == np.float32: return _F
+    if dtype == np.int32:   return _I
+    if dtype == np.uint32:  return _U
+    if dtype == np.bool_:   return _B
+    raise NotImplementedError(f'{dtype} data types currently not supported')
+
+
+#primitive name -> {operand kind -> opcode name}
+_BINARY = {
+    'add': {_F: 'ADD_F', _I: 'ADD_I', _U: 'ADD_I'},
+    'sub': {_F: 'SUB_F', _I: 'SUB_I', _U: 'SUB_I'},
+    'mul': {_F: 'MUL_F', _I: 'MUL_I', _U: 'MUL_I', _B: 'AND_X'},
+    'div': {_F: 'DIV_F', _I: 'DIV_I', _U: 'DIV_U'},
+    'rem': {_F: 'REM_F', _I: 'REM_I', _U: 'REM_U'},
+    'max': {_F: 'MAX_F', _I: 'MAX_I', _U: 'MAX_U', _B: 'OR_X'},
+    'min': {_F: 'MIN_F', _I: 'MIN_I', _U: 'MIN_U', _B: 'AND_X'},
+    'pow': {_F: 'POW_F'},
+    'nextafter': {_F: 'NEXTAFTER_F'},
+    'gt': {_F: 'GT_F', _I: 'GT_I', _U: 'GT_U', _B: 'GT_U'},
+    'ge': {_F: 'GE_F', _I: 'GE_I', _U: 'GE_U', _B: 'GE_U'},
+    'lt': {_F: 'LT_F', _I: 'LT_I', _U: 'LT_U', _B: 'LT_U'},
+    'le': {_F: 'LE_F', _I: 'LE_I', _U: 'LE_U', _B: 'LE_U'},
+    'eq': {_F: 'EQ_F', _I: 'EQ_X', _U: 'EQ_X', _B: 'EQ_X'},
+    'ne': {_F: 'NE_F', _I: 'NE_X', _U: 'NE_X', _B: 'NE_X'},
+    'and': {_I: 'AND_X', _U: 'AND_X', _B: 'AND_X'},
+    'or':  {_I: 'OR_X', _U: 'OR_X', _B: 'OR_X'},
+    'xor': {_I: 'XOR_X', _U: 'XOR_X', _B: 'XOR_X'},
+    'shift_left':             {_I: 'SHL_X', _U: 'SHL_X'},
+    'shift_right_logical':    {_I: 'SHR_L', _U: 'SHR_L'},
+    'shift_right_arithmetic': {_I: 'SHR_A', _U: 'SHR_A'},
+}
+_BINARY['add_any'] = _BINARY['add']
+
+_UNARY = {
+    'exp': {_F: 'EXP_F'}, 'log': {_F: 'LOG_F'}, 'rsqrt': {_F: 'RSQRT_F'}, 'sqrt': {_F: 'SQRT_F'},
+    'erf': {_F: 'ERF_F'}, 'erf_inv': {_F: 'ERFINV_F'},
+    'neg': {_F: 'NEG_F', _I: 'NEG_I', _U: 'NEG_I'},
+    'abs': {_F: 'ABS_F', _I: 'ABS_I', _U: 'NOP'},
+    'sign': {_F: 'SIGN_F', _I: 'SIGN_I'},
+    'cos': {_F: 'COS_F'}, 'sin': {_F: 'SIN_F'}, 'tan': {_F: 'TAN_F'},
+    'cosh': {_F: 'COSH_F'}, 'sinh': {_F: 'SINH_F'}, 'tanh': {_F: 'TANH_F'},
+    'acos': {_F: 'ACOS_F'}, 'asin': {_F: 'ASIN_F'}, 'atan': {_F: 'ATAN_F'},
+    'acosh': {_F: 'ACOSH_F'}, 'asinh': {_F: 'ASINH_F'}, 'atanh': {_F: 'ATANH_F'},
+    'ceil': {_F: 'CEIL_F'}, 'floor': {_F: 'FLOOR_F'},
+}
+
+
+def _opcode(table, name, dtype, equation):
+    try:
+        return EW[table[name][_kind(dtype)]]
+    except KeyError:
+        raise NotImplementedError(f'{name} on {np.dtype(dtype)}: {equation}')
+
+
+def _params_without_jax_bookkeeping(params: dict) -> dict:
+    #newer jax versions attach bookkeeping entries that do not change the computation
+    return {k: v for k, v in params.items() if k not in ('accumulation_type', 'sharding')}
+
+
+# ------------------------------------------------------------------ element-wise
+
+def element_wise_binary_op(bufferpool: BufferPool, equation):
+    assert _params_without_jax_bookkeeping(equation.params) == {}
+    assert len(equation.invars) == 2
+    assert len(equation.outvars) == 1
+    outvar = equation.outvars[0]
+    name   = equation.primitive.name
+    inbufs = [bufferpool.get_buffer(v) for v in equation.invars]
+    opcode = _opcode(_BINARY, name, inbufs[0].dtype, equation)
+    #implicit trailing-aligned broadcast is read in place through zero strides
+    #(the reference materialises it with an extra dispatch, vkjax/ops.py:84-86)
+    operands = [K.broadcast_operand(b, outvar.aval.shape) for b in inbufs]
+    outbuf   = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    chain    = EwChain(outbuf, outvar.aval.shape, operands[0], [EwStep(opcode, operands[1])])
+    return [Op(equation, chain=chain)]
+
+
+add = sub = mul = div = max = min = element_wise_binary_op
+gt = ge = lt = le = eq = ne = element_wise_binary_op
+add_any = pow = rem = nextafter = element_wise_binary_op
+shift_left = shift_right_logical = shift_right_arithmetic = element_wise_binary_op
+xor = element_wise_binary_op
+globals()['or']  = element_wise_binary_op
+globals()['and'] = element_wise_binary_op
+
+
+def element_wise_unary_op(bufferpool: BufferPool, equation):
+    assert _params_without_jax_bookkeeping(equation.params) == {}
+    assert len(equation.invars) == 1
+    assert len(equation.outvars) == 1
+    outvar, invar = equation.outvars[0], equation.invars[0]
+    assert tuple(outvar.aval.shape) == tuple(invar.aval.shape)
+    inbuf  = bufferpool.get_buffer(invar)
+    opcode = _opcode(_UNARY, equation.primitive.name, inbuf.dtype, equation)
+    outbuf = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    chain  = EwChain(outbuf, outvar.aval.shape, K.broadcast_operand(inbuf, outvar.aval.shape), [EwStep(opcode)])
+    return [Op(equation, chain=chain)]
+
+
+exp = log = neg = abs = rsqrt = sqrt = erf = erf_inv = sign = element_wise_unary_op
+cos = sin = tan = cosh = sinh = tanh = element_wise_unary_op
+acos = asin = atan = acosh = asinh = atanh = ceil = floor = element_wise_unary_op
+
+
+def integer_pow(bufferpool, equation):
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    y      = int(equation.params['y'])
+    if _kind(inbuf.dtype) == _F:
+        op = EW['IPOW_F']
+    else:
+        if y < 0:
+            raise NotImplementedError(f'negative integer power of integers: {equation}')
+        op = EW['IPOW_I']
+    chain = EwChain(outbuf, outbuf.shape, K.broadcast_operand(inbuf, outbuf.shape), [EwStep(op, imm=y)])
+    return [Op(equation, chain=chain)]
+
+
+def select(bufferpool, equation):
+    '''3-operand select (pred, on_true, on_false), equal shapes (reference: vkjax/ops.py:338-347).'''
+    shapes = [tuple(v.aval.shape) for v in equation.invars] + [tuple(equation.outvars[0].aval.shape)]
+    assert all(s == shapes[0] for s in shapes)
+    pred, on_true, on_false = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    return [Op(equation, chain=_select_chain(outbuf, pred, on_true, on_false))]
+
+
+def _select_chain(outbuf, pred, on_true, on_false):
+    shape = outbuf.shape
+    return EwChain(outbuf, shape, K.broadcast_operand(pred, shape),
+                   [EwStep(EW['SEL_P'], K.broadcast_operand(on_true, shape)),
+                    EwStep(EW['NOP'], K.broadcast_operand(on_false, shape))])
+
+
+def select_n(bufferpool, equation):
+    '''select_n(which, case0, case1) of newer jax: case1 where `which` is true.'''
+    if len(equation.invars) != 3 or _kind(equation.invars[0].aval.dtype) != _B:
+        raise NotImplementedError(equation)
+    pred, on_false, on_true = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    return [Op(equation, chain=_select_chain(outbuf, pred, on_true, on_false))]
+
+
+_CONVERT = {
+    (_F, _I): 'CVT_F2I', (_F, _U): 'CVT_F2U', (_I, _F): 'CVT_I2F', (_U, _F): 'CVT_U2F', (_B, _F): 'CVT_U2F',
+    (_F, _B): 'CVT_F2B', (_I, _B): 'CVT_X2B', (_U, _B): 'CVT_X2B',
+}
+
+
+def convert_element_type(bufferpool, equation):
+    invar, outvar = equation.invars[0], equation.outvars[0]
+    src, dst = _kind(core.canonicalize_dtype(invar.aval.dtype)), _kind(core.canonicalize_dtype(outvar.aval.dtype))
+    if (src, dst) not in _CONVERT:
+        #same bits on the device (int <-> uint, bool -> int, same type): a view is enough
+        return noop(bufferpool, equation)
+    inbuf  = bufferpool.get_buffer(invar)
+    outbuf = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    chain  = EwChain(outbuf, outbuf.shape, K.broadcast_operand(inbuf, outbuf.shape), [EwStep(EW[_CONVERT[(src, dst)]])])
+    return [Op(equation, chain=chain)]
+
+
+# ------------------------------------------------------------------ views and data movement
+
+def noop(bufferpool, equation):
+    '''No launch: the output is the input's storage seen with another dtype/shape.'''
+    assert len(equation.invars) == len(equation.outvars) == 1
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    outvar = equation.outvars[0]
+    outbuf = inbuf.view(core.canonicalize_dtype(outvar.aval.dtype), outvar.aval.shape)
+    bufferpool.set_buffer(outvar, outbuf)
+    return []
+
+
+stop_gradient = squeeze = bitcast_convert_type = noop
+copy = copy_p = optimization_barrier = noop
+
+
+def reshape(bufferpool, equation):
+    assert equation.params['dimensions'] is None
+    assert len(equation.outvars) == 1
+    assert len(equation.invars) >= 1
+    invar, outvar = equation.invars[0], equation.outvars[0]
+    assert core.canonicalize_dtype(invar.aval.dtype) == core.canonicalize_dtype(outvar.aval.dtype)
+    buffer = bufferpool.get_buffer(invar)
+    outbuf = buffer.view(buffer.dtype, outvar.aval.shape)
+    bufferpool.set_buffer(outvar, outbuf)
+    return []
+
+
+def _copy_op(equation, outbuf: Buffer, operand: EwOperand):
+    return Op(equation, chain=EwChain(outbuf, outbuf.shape, operand, []))
+
+
+def broadcast_in_dim(bufferpool, equation):
+    bdims = tuple(equation.params['broadcast_dimensions'])
+    assert np.all(np.diff(bdims) > 0)
+    invar, outvar = equation.invars[0], equation.outvars[0]
+    inbuf = bufferpool.get_buffer(invar)
+    if inbuf.size == int(np.prod(outvar.aval.shape, dtype=np.int64)):
+        #same size, just the same storage with a new shape
+        outbuf = inbuf.view(inbuf.dtype, outvar.aval.shape)
+        bufferpool.set_buffer(outvar, outbuf)
+        return []
+    outbuf     = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    in_strides = K.row_major_strides(inbuf.shape)
+    strides    = [0] * len(outbuf.shape)
+    for i, d in enumerate(bdims):
+        if inbuf.shape[i] != 1:
+            if inbuf.shape[i] != outbuf.shape[d]:
+                raise ValueError(f'Cannot broadcast from {inbuf.shape} to {outbuf.shape}')
+            strides[d] = in_strides[i]
+    return [_copy_op(equation, outbuf, EwOperand(inbuf, 0, tuple(strides)))]
+
+
+def slice(bufferpool, equation):
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    n       = len(inbuf.shape)
+    start   = equation.params['start_indices']
+    strides = equation.params['strides'] or (1,) * n
+    in_strides = K.row_major_strides(inbuf.shape)
+    offset  = sum(int(s) * st for s, st in zip(start, in_strides))
+    return [_copy_op(equation, outbuf, EwOperand(inbuf, offset, tuple(int(k) * st for k, st in zip(strides, in_strides))))]
+
+
+def transpose(bufferpool, equation):
+    perm   = tuple(equation.params['permutation'])
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    in_strides = K.row_major_strides(inbuf.shape)
+    return [_copy_op(equation, outbuf, EwOperand(inbuf, 0, tuple(in_strides[p] for p in perm)))]
+
+
+def rev(bufferpool, equation):
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    dims   = set(int(d) for d in equation.params['dimensions'])
+    in_strides = K.row_major_strides(inbuf.shape)
+    offset  = sum((inbuf.shape[d] - 1) * in_strides[d] for d in dims)
+    strides = tuple(-st if d in dims else st for d, st in enumerate(in_strides))
+    return [_copy_op(equation, outbuf, EwOperand(inbuf, offset, strides))]
+
+
+def iota(bufferpool, equation):
+    outvar = equation.outvars[0]
+    dimension = int(equation.params['dimension'])
+    assert 0 <= dimension < builtins_max(len(outvar.aval.shape), 1)
+    outbuf = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    if _kind(outbuf.dtype) == _B:
+        raise NotImplementedError(equation)
+    return [Op(equation, launch=K.iota(outbuf, dimension))]
+
+
+def concatenate(bufferpool, equation):
+    outvar = equation.outvars[0]
+    dim    = int(equation.params['dimension'])
+    inbufs = [bufferpool.get_buffer(v) for v in equation.invars]
+    for b in inbufs:
+        assert b.shape[:dim] == tuple(outvar.aval.shape[:dim]) and b.shape[dim + 1:] == tuple(outvar.aval.shape[dim + 1:])
+    outbuf = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    ops, offset = [], 0
+    for b in inbufs:
+        if b.size:
+            ops.append(Op(equation, launch=K.concat_part(outbuf, b, dim, offset)))
+        offset += b.shape[dim]
+    return ops
+
+
+# ------------------------------------------------------------------ nested calls (inlined)
+
+def _inline_call(bufferpool, equation, jaxpr, consts=()):
+    jaxpr = getattr(jaxpr, 'jaxpr', jaxpr)
+    assert len(equation.invars) == len(jaxpr.invars)
+    assert len(equation.outvars) == len(jaxpr.outvars)
+    for constvar, value in zip(getattr(jaxpr, 'constvars', []), consts):
+        b = bufferpool.get_buffer(constvar)
+        bufferpool.mark_buffer_as_constant(b, constvar, value=value)
+    for eq_var, jaxpr_var in zip(equation.invars, jaxpr.invars):
+        if str(eq_var) == '*':
+            continue
+        #connect call parameters to the function-local variables
+        bufferpool.set_buffer(jaxpr_var, bufferpool.get_buffer(eq_var))
+    all_ops = analyze_jaxpr(bufferpool, jaxpr)
+    for eq_var, jaxpr_var in zip(equation.outvars, jaxpr.outvars):
+        if core.is_dropped(eq_var):
+            continue
+        if str(jaxpr_var) == '*':
+            bufferpool.set_buffer(eq_var, None)
+            continue
+        #connect the function-local variables to the output variables
+        bufferpool.set_buffer(eq_var, bufferpool.get_buffer(jaxpr_var))
+    return all_ops
+
+
+def xla_call(bufferpool, equation):
+    assert equation.params.get('device') is None
+    assert equation.params.get('backend') is None
+    return _inline_call(bufferpool, equation, equation.params['call_jaxpr'])
+
+
+core_call = closed_call = remat = xla_call
+
+
+def pjit(bufferpool, equation):
+    closed = equation.params['jaxpr']
+    return _inline_call(bufferpool, equation, closed, getattr(closed, 'consts', ()))
+
+
+def custom_jvp_call_jaxpr(bufferpool, equation):
+    closed = equation.params['fun_jaxpr']
+    return _inline_call(bufferpool, equation, closed, getattr(closed, 'consts', ()))
+
+
+def custom_jvp_call(bufferpool, equation):
+    closed = equation.params['call_jaxpr']
+    return _inline_call(bufferpool, equation, closed, getattr(closed, 'consts', ()))
+
+
+custom_vjp_call = custom_vjp_call_jaxpr = custom_jvp_call
+
+
+# ------------------------------------------------------------------ contractions
+
+def dot_general(bufferpool, equation):
+    '''2-D x 2-D, one contracting dimension per side, no batch dimensions, float32
+    (reference: vkjax/ops.py:277-297). Lowered onto the implicit-GEMM kernel with a 1x1 window.'''
+    assert equation.params.get('precision') is None
+    (lc, rc), (lb, rb) = equation.params['dimension_numbers']
+    assert (tuple(lb), tuple(rb)) == ((), ())
+    assert tuple(lc) in [(0,), (1,)]
+    assert tuple(rc) in [(0,), (1,)]
+    assert len(equation.invars) == 2
+    assert len(equation.outvars) == 1
+    assert all(core.canonicalize_dtype(v.aval.dtype) == np.float32 for v in list(equation.invars) + list(equation.outvars))
+    lhs, rhs = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf   = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    assert len(lhs.shape) == 2 and len(rhs.shape) == 2
+    M, N = outbuf.shape
+    Kc   = lhs.shape[lc[0]]
+    lst, rst = K.row_major_strides(lhs.shape), K.row_major_strides(rhs.shape)
+    geom = K.ConvGeometry(batch=1, Ho=M, Wo=1, N=N, H=M, W=1, Cin=Kc, KH=1, KW=1,
+                          xs=(0, lst[1 - lc[0]], 0, lst[lc[0]]),
+                          ws=(rst[rc[0]] * Kc, rst[rc[0]] * Kc, rst[rc[0]], rst[1 - rc[0]]),
+                          os=(M * N, N, N, 1))
+    return [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+
+
+def conv_general_dilated(bufferpool, equation):
+    '''2-D convolution, any ConvDimensionNumbers permutation, strides, low/high padding, lhs and
+    rhs dilation, one feature group (reference: vkjax/ops.py:463-487).'''
+    params = equation.params
+    assert params.get('precision') is None
+    assert params['batch_group_count'] == 1
+    assert params['feature_group_count'] == 1
+    outvar = equation.outvars[0]
+    assert len(outvar.aval.shape) == 4      #2D conv
+    assert all(core.canonicalize_dtype(v.aval.dtype) == np.float32 for v in list(equation.invars) + [outvar])
+    lhs_spec, rhs_spec, out_spec = params['dimension_numbers']
+    lhs, rhs = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf   = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    lst, rst, ost = (K.row_major_strides(b.shape) for b in (lhs, rhs, outbuf))
+    pick = lambda seq, spec: tuple(seq[d] for d in spec)
+    batch, Cin, H, W = pick(lhs.shape, lhs_spec)
+    N, Cin_r, KH, KW = pick(rhs.shape, rhs_spec)
+    _, _, Ho, Wo     = pick(outbuf.shape, out_spec)
+    assert Cin == Cin_r
+    xs = pick(lst, lhs_spec); ws = pick(rst, rhs_spec); os_ = pick(ost, out_spec)
+    geom = K.ConvGeometry(batch=batch, Ho=Ho, Wo=Wo, N=N, H=H, W=W, Cin=Cin, KH=KH, KW=KW,
+                          SH=params['window_strides'][0], SW=params['window_strides'][1],
+                          PH=params['padding'][0][0], PW=params['padding'][1][0],
+                          DH=params['rhs_dilation'][0], DW=params['rhs_dilation'][1],
+                          LH=params['lhs_dilation'][0], LW=params['lhs_dilation'][1],
+                          xs=(xs[0], xs[2], xs[3], xs[1]),
+                          ws=(ws[2], ws[3], ws[1], ws[0]),
+                          os=(os_[0], os_[2], os_[3], os_[1]))
+    if outbuf.size == 0:
+        return []
+    return [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+
+
+# ------------------------------------------------------------------ reductions
+
+def reduce_op(bufferpool, equation):
+    axes = tuple(int(a) for a in equation.params['axes'])
+    if axes == ():
+        return noop(bufferpool, equation)
+    outvar, invar = equation.outvars[0], equation.invars[0]
+    name   = equation.primitive.name
+    inbuf  = bufferpool.get_buffer(invar)
+    outbuf = bufferpool.get_buffer(outvar, increment_op_counter=True)
+    if _kind(inbuf.dtype) == _B and name not in ('reduce_max', 'reduce_min'):
+        raise NotImplementedError(equation)
+    if outbuf.size == 0:
+        return []
+    shape   = inbuf.shape
+    strides = K.row_major_strides(shape)
+    #merge neighbouring dims with the same role, drop size-1 dims
+    groups = []
+    for d, (s, st) in enumerate(zip(shape, strides)):
+        if s == 1:
+            continue
+        red = d in axes
+        if groups and groups[-1][0] == red:
+            groups[-1] = (red, groups[-1][1] * s, st)
+        else:
+            groups.append((red, s, st))
+    roles = [g[0] for g in groups]
+    if not any(roles):
+        #only size-1 dims are reduced: copy (argmax of a single element is index 0)
+        if name in ('argmax', 'argmin'):
+            return [Op(equation, launch=K.fill(outbuf, 0))]
+        return [_copy_op(equation, outbuf, EwOperand(inbuf, 0, K.row_major_strides(outbuf.shape)))]
+    if roles in ([True], [False, True], [True, False], [False, True, False]):
+        outer = groups[0][1] if not roles[0] else 1
+        inner = groups[-1][1] if not roles[-1] else 1
+        R     = [g[1] for g in groups if g[0]][0]
+        if outer <= 65535:
+            return [Op(equation, launch=K.reduce_3d(outbuf, inbuf, outer, R, inner, name))]
+    kept    = [(g[1], g[2]) for g in groups if not g[0]]
+    reduced = [(g[1], g[2]) for g in groups if g[0]]
+    return [Op(equation, launch=K.reduce_general(outbuf, inbuf, kept, reduced, name))]
+
+
+reduce_max = reduce_min = reduce_sum = reduce_prod = argmin = argmax = reduce_op
+
+
+def _reduce_window(bufferpool, equation, op_name):
+    params = equation.params
+    n = len(equation.outvars[0].aval.shape)
+    assert n <= 4, NotImplemented
+    assert tuple(params.get('base_dilation') or (1,) * n) == (1,) * n, NotImplemented
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    if _kind(inbuf.dtype) == _B:
+        raise NotImplementedError(equation)
+    if outbuf.size == 0:
+        return []
+    launch = K.pool(outbuf, inbuf, op_name, params['window_dimensions'], params['window_strides'],
+                    [p[0] for p in params['padding']], tuple(params.get('window_dilation') or (1,) * n))
+    return [Op(equation, launch=launch)]
+
+
+def reduce_window_max(bufferpool, equation):
+    '''Window maximum; positions outside the array count as -inf (reference: vkjax/ops.py:505-524,
+    whose kernel used 0 there).'''
+    return _reduce_window(bufferpool, equation, 'reduce_max')
+
+
+def reduce_window_sum(bufferpool, equation):
+    return _reduce_window(bufferpool, equation, 'reduce_sum')
+
+
+# ------------------------------------------------------------------ indexing
+
+def gather(bufferpool, equation):
+    params = equation.params
+    dn     = params['dimension_numbers']
+    offset_dims, collapsed, start_index_map = (tuple(dn.offset_dims), tuple(dn.collapsed_slice_dims), tuple(dn.start_index_map))
+    slice_sizes = tuple(int(s) for s in params['slice_sizes'])
+    operand, indices = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    if outbuf.size == 0:
+        return []
+    if _kind(indices.dtype) not in (_I, _U):
+        raise NotImplementedError(equation)
+    op_rank, out_rank = len(operand.shape), len(outbuf.shape)
+    n_batch = len(indices.shape) - 1
+    #whole trailing slices addressed by one index on the leading axis: a row gather
+    is_rows = (collapsed == (0,) and start_index_map == (0,) and indices.shape[-1] == 1 and slice_sizes[0] == 1
+               and slice_sizes[1:] == tuple(operand.shape[1:])
+               and offset_dims == tuple(range(n_batch, out_rank)))
+    if is_rows:
+        row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
+        n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
+        return [Op(equation, launch=K.gather_rows(outbuf, operand, indices, n_idx, row_len, operand.shape[0]))]
+    return [Op(equation, launch=K.gather_general(outbuf, operand, indices, offset_dims, collapsed, start_index_map, slice_sizes))]
+
+
+def scatter_add(bufferpool, equation):
+    '''General XLA scatter-add (the reference implements two fixed patterns, vkjax/ops.py:404-433).
+    The operand is copied to the output first, then updates are added with HBM atomics.'''
+    dn = equation.params['dimension_numbers']
+    uwd, iwd, sd2od = tuple(dn.update_window_dims), tuple(dn.inserted_window_dims), tuple(dn.scatter_dims_to_operand_dims)
+    operand, indices, updates = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    if _kind(operand.dtype) == _B or _kind(indices.dtype) not in (_I, _U):
+        raise NotImplementedError(equation)
+    if outbuf.size == 0:
+        return []
+    ops = [_copy_op(equation, outbuf, EwOperand(operand, 0, K.row_major_strides(outbuf.shape)))]
+    if updates.size == 0:
+        return ops
+    n_batch = len(indices.shape) - 1
+    is_rows = (iwd == (0,) and sd2od == (0,) and indices.shape[-1] == 1
+               and uwd == tuple(range(n_batch, len(updates.shape)))
+               and tuple(updates.shape[n_batch:]) == tuple(operand.shape[1:]))
+    if is_rows:
+        row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
+        n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
+        ops.append(Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, operand.shape[0])))
+    else:
+        ops.append(Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od)))
+    return ops
+
+
+# ------------------------------------------------------------------ rng
+
+def threefry2x32(bufferpool, equation):
+    inbufs  = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbufs = [bufferpool.get_buffer(v) for v in equation.outvars]
+    bufferpool.op_counter += 1
+    assert inbufs[0].shape  == inbufs[1].shape
+    assert inbufs[2].shape  == inbufs[3].shape
+    assert outbufs[0].shape == outbufs[1].shape
+    assert all(_kind(b.dtype) == _U for b in inbufs + outbufs)
+    key_is_scalar = inbufs[0].shape in [(), (1,)]
+    if not key_is_scalar:
+        assert inbufs[0].shape == inbufs[2].shape
+    if outbufs[0].size == 0:
+        return []
+    return [Op(equation, launch=K.threefry2x32(*outbufs, *inbufs, key_is_scalar=key_is_scalar))]
+
+
+import builtins as _builtins
+builtins_max = _builtins.max

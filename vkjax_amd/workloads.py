@@ -1,0 +1,184 @@
+'''The five benchmark / parity workloads: the functions that get traced and their synthetic,
+seeded inputs. Written against the stand-in tracer (`vkjax_amd.minijax`), they produce the
+primitive sequences a jax front-end of the reference's era emits for the same models
+(`jnp.dot + b`, relu under a custom-jvp call, softmax, NHWC convolutions with inference-mode
+batch norm, `reduce_window` max pooling, threefry-based `random.uniform`, indexing gather and
+`.at[].add` scatter).
+
+Input recipe: numpy `default_rng(seed)`; "uniform" is `rng.random(shape, float32)`; He-normal is
+`standard_normal * sqrt(2 / fan_in)`; all weights are generated on the host.
+'''
+import typing as tp
+
+import numpy as np
+
+from . import minijax as mj
+
+jnp, lax, nn = mj.numpy, mj.lax, mj.nn
+
+NHWC = mj.core.ConvDimensionNumbers((0, 3, 1, 2), (3, 2, 0, 1), (0, 3, 1, 2))
+
+
+def he_normal(rng, shape, fan_in) -> np.ndarray:
+    return (rng.standard_normal(shape, dtype=np.float32) * np.sqrt(2.0 / fan_in)).astype(np.float32)
+
+
+# ------------------------------------------------------------------ 1: affine layer
+
+def affine(x, W, b):
+    return jnp.dot(x, W) + b
+
+
+def affine_inputs(seed=1):
+    rng = np.random.default_rng(seed)
+    return [rng.random((8, 128), dtype=np.float32), rng.random((128, 16), dtype=np.float32), rng.random((16,), dtype=np.float32)]
+
+
+# ------------------------------------------------------------------ 2: MLP
+
+def mlp(params, x):
+    h = nn.relu(jnp.dot(x, params['w1']) + params['b1'])
+    h = nn.relu(jnp.dot(h, params['w2']) + params['b2'])
+    logits = jnp.dot(h, params['w3']) + params['b3']
+    probs  = nn.softmax(logits, axis=-1)
+    return probs, jnp.argmax(probs, axis=1)
+
+
+def mlp_inputs(seed=2, batch=256, sizes=(784, 512, 512, 10)):
+    rng = np.random.default_rng(seed)
+    x = rng.random((batch, sizes[0]), dtype=np.float32)
+    params = {}
+    for i in range(3):
+        params[f'w{i + 1}'] = he_normal(rng, (sizes[i], sizes[i + 1]), sizes[i])
+        params[f'b{i + 1}'] = np.zeros((sizes[i + 1],), np.float32)
+    return [params, x]
+
+
+# ------------------------------------------------------------------ 3: conv block
+
+def conv_block(params, x):
+    y = lax.conv_general_dilated(x, params['w'], window_strides=(1, 1), padding=((1, 1), (1, 1)), dimension_numbers=NHWC)
+    y = nn.batch_norm_inference(y, params['scale'], params['shift'], params['mean'], params['var'])
+    y = nn.relu(y)
+    return lax.reduce_window(y, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (0, 1), (0, 1), (0, 0)))
+
+
+def conv_block_inputs(seed=3, batch=32, size=56, channels=64):
+    rng = np.random.default_rng(seed)
+    x = rng.random((batch, size, size, channels), dtype=np.float32)
+    params = dict(w=he_normal(rng, (3, 3, channels, channels), 9 * channels),
+                  scale=rng.standard_normal(channels, dtype=np.float32), shift=rng.standard_normal(channels, dtype=np.float32),
+                  mean=rng.standard_normal(channels, dtype=np.float32),
+                  var=(0.5 + rng.random(channels, dtype=np.float32)).astype(np.float32))
+    return [params, x]
+
+
+# ------------------------------------------------------------------ 4: ResNet-50
+
+RESNET50_STAGES = ((3, 64, 1), (4, 128, 2), (6, 256, 2), (3, 512, 2))      #(blocks, bottleneck width, stride of the first block)
+
+
+def _same_pads(size, window, stride):
+    out   = -(-size // stride)
+    total = max((out - 1) * stride + window - size, 0)
+    return (total // 2, total - total // 2)
+
+
+def _conv_bn(p, x, stride=1, pads=None, relu=True):
+    kh, kw = p['w'].shape[0], p['w'].shape[1]
+    if pads is None:
+        pads = (_same_pads(x.shape[1], kh, stride), _same_pads(x.shape[2], kw, stride))
+    y = lax.conv_general_dilated(x, p['w'], window_strides=(stride, stride), padding=pads, dimension_numbers=NHWC)
+    y = nn.batch_norm_inference(y, p['scale'], p['shift'], p['mean'], p['var'])
+    return nn.relu(y) if relu else y
+
+
+def resnet50(params, x):
+    '''ResNet-50 forward, inference mode. Layer table: 7x7/2 stem (padding 3) + BN + ReLU,
+    3x3/2 SAME max-pool, bottleneck stages (3, 4, 6, 3) with the stride on the 3x3 convolution
+    and a strided 1x1 projection on the first block of each stage, global average pool, 1000-way
+    dense layer. Returns (logits, argmax(logits)).'''
+    y = _conv_bn(params['stem'], x, stride=2, pads=((3, 3), (3, 3)))
+    y = lax.reduce_window(y, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1),
+                          ((0, 0), _same_pads(y.shape[1], 3, 2), _same_pads(y.shape[2], 3, 2), (0, 0)))
+    for s, (blocks, width, stride) in enumerate(RESNET50_STAGES):
+        for b in range(blocks):
+            p = params[f'stage{s}'][f'block{b}']
+            st = stride if b == 0 else 1
+            shortcut = _conv_bn(p['proj'], y, stride=st, relu=False) if 'proj' in p else y
+            z = _conv_bn(p['conv1'], y)
+            z = _conv_bn(p['conv2'], z, stride=st)
+            z = _conv_bn(p['conv3'], z, relu=False)
+            y = nn.relu(z + shortcut)
+    y = jnp.mean(y, axis=(1, 2))
+    logits = jnp.dot(y, params['fc']['w']) + params['fc']['b']
+    return logits, jnp.argmax(logits, axis=1)
+
+
+def _conv_bn_params(rng, kh, kw, cin, cout):
+    return dict(w=he_normal(rng, (kh, kw, cin, cout), kh * kw * cin),
+                scale=(0.5 + rng.random(cout, dtype=np.float32)).astype(np.float32),
+                shift=(0.1 * rng.standard_normal(cout, dtype=np.float32)).astype(np.float32),
+                mean=(0.1 * rng.standard_normal(cout, dtype=np.float32)).astype(np.float32),
+                var=(0.5 + rng.random(cout, dtype=np.float32)).astype(np.float32))
+
+
+def resnet50_params(seed=4, num_classes=1000, width_scale=1.0) -> dict:
+    '''`width_scale` < 1 shrinks every channel count (test-sized variants of the same graph).'''
+    rng = np.random.default_rng(seed)
+    c = lambda n: max(4, int(n * width_scale) // 4 * 4)
+    params = dict(stem=_conv_bn_params(rng, 7, 7, 3, c(64)))
+    cin = c(64)
+    for s, (blocks, width, stride) in enumerate(RESNET50_STAGES):
+        stage = {}
+        for b in range(blocks):
+            w, cout = c(width), c(width * 4)
+            block = dict(conv1=_conv_bn_params(rng, 1, 1, cin, w), conv2=_conv_bn_params(rng, 3, 3, w, w),
+                         conv3=_conv_bn_params(rng, 1, 1, w, cout))
+            if b == 0:
+                block['proj'] = _conv_bn_params(rng, 1, 1, cin, cout)
+            stage[f'block{b}'] = block
+            cin = cout
+        params[f'stage{s}'] = stage
+    params['fc'] = dict(w=he_normal(rng, (cin, num_classes), cin), b=np.zeros((num_classes,), np.float32))
+    return params
+
+
+def resnet50_inputs(seed=4, batch=64, size=224, num_classes=1000, width_scale=1.0):
+    params = resnet50_params(seed, num_classes, width_scale)
+    rng = np.random.default_rng(seed + 1000)
+    return [params, rng.random((batch, size, size, 3), dtype=np.float32)]
+
+
+# ------------------------------------------------------------------ 5: RNG + gather / scatter-add
+
+def rng_uniform(key, shape=(4096, 4096)):
+    k1, k2 = mj.random.split(key)
+    return mj.random.uniform(k2, shape)
+
+
+def rng_inputs(seed=5):
+    return [mj.random.PRNGKey(seed)]
+
+
+def gather_scatter(table, idx, updates):
+    rows = table[idx]
+    return rows, jnp.index_add(jnp.zeros(table.shape, np.float32), idx, updates)
+
+
+def gather_scatter_inputs(seed=5, rows=65536, cols=256, n0=8192, n1=32):
+    rng = np.random.default_rng(seed)
+    table   = rng.random((rows, cols), dtype=np.float32)
+    idx     = rng.integers(0, rows, size=(n0, n1)).astype(np.int32)
+    updates = rng.random((n0, n1, cols), dtype=np.float32)
+    return [table, idx, updates]
+
+
+WORKLOADS: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable]] = {
+    'affine':         (affine, affine_inputs),
+    'mlp':            (mlp, mlp_inputs),
+    'conv_block':     (conv_block, conv_block_inputs),
+    'resnet50':       (resnet50, resnet50_inputs),
+    'rng_uniform':    (rng_uniform, rng_inputs),
+    'gather_scatter': (gather_scatter, gather_scatter_inputs),
+}
