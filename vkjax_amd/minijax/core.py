@@ -115,8 +115,9 @@ class Literal:
     def __init__(self, val, aval: ShapedArray):
         self.val  = val
         self.aval = aval
-        #jax literals are unhashable but carry a .hash the pool keys on (reference: vkjax/buffers.py:80-87)
-        self.hash = id(self)
+        #jax literals are unhashable but carry a .hash derived from the value, which the pool keys on,
+        #so equal literals share one buffer (reference: vkjax/buffers.py:80-87)
+        self.hash = hash((aval.dtype.str, np.asarray(val).tobytes()))
 
     def __repr__(self):
         return str(self.val)
