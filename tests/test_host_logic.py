@@ -1,0 +1,244 @@
+'''Host-side behaviour that needs no GPU: the C ABI (library loads, exports every declared
+symbol, fails cleanly without a device), the trace cache of Function, the buffer pool's
+liveness reuse, the dispatch's error behaviour, and the kernel argument layouts.
+The literal expectations come from the reference's own tests (tests/test_function.py:13-60,
+tests/test_bufferpool.py:32-40,62-63).'''
+import ctypes
+import json
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import vkjax_amd
+from vkjax_amd import hip, kernels as K, minijax as mj, ops
+from vkjax_amd.buffers import Buffer, BufferPool, PlanOnlyDevice, to_device_words, view_or_convert_from_32bit
+from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
+from vkjax_amd.minijax import core
+
+ROOT   = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = json.load(open(os.path.join(ROOT, 'tests', 'golden', 'known_answers.json')))['reference_test_literals']
+jnp, lax = mj.numpy, mj.lax
+
+
+# ------------------------------------------------------------------ C ABI
+
+def test_library_exports_every_declared_symbol():
+    header   = open(os.path.join(ROOT, 'include', 'vkjax_hip.h')).read()
+    declared = set(re.findall(r'\b(vkj_\w+)\s*\(', header))
+    assert len(declared) >= 25
+    lib = hip.load_library()
+    for name in declared:
+        assert hasattr(lib, name), f'{name} declared in the header but not exported'
+    assert declared == set(hip.exported_symbols())
+
+
+def test_abi_fails_cleanly_on_bad_arguments():
+    lib = hip.load_library()
+    assert lib.vkj_ctx_destroy(0) == -1 and b'bad context handle' in lib.vkj_last_error()
+    assert lib.vkj_sync(12345) != 0
+    n = ctypes.c_int(-1)
+    lib.vkj_device_count(ctypes.byref(n))
+    assert n.value >= 0
+    if n.value == 0:
+        h = ctypes.c_uint64(0)
+        assert lib.vkj_ctx_create(0, ctypes.byref(h)) == -4          #VKJ_ENODEV
+        assert b'no HIP device' in lib.vkj_last_error()
+        with pytest.raises(hip.HipError):
+            hip.Device(0)
+
+
+def test_code_objects_are_built_for_gfx950():
+    for name in hip.KERNEL_MODULES:
+        path = os.path.join(hip.LIBDIR, f'{name}.hsaco')
+        assert os.path.exists(path), f'{path} missing: run python -m vkjax_amd.csrc.build'
+        assert b'gfx950' in open(path, 'rb').read()
+
+
+def test_kernel_argument_layouts_match_the_structs():
+    '''sizeof of every kernel parameter struct, taken from the compiler, equals the length of
+    the block the host packs.'''
+    src = r'''
+#include <cstdio>
+#include "elementwise.hip"
+#define EW_OP(a,b)
+#include "conv_gemm.hip"
+#include "reduce.hip"
+#include "index.hip"
+#include "threefry.hip"
+#define P(T) printf(#T " %zu\n", sizeof(T));
+int main(){ P(EwParams) P(IotaParams) P(FillParams) P(ConcatParams) P(ConvParams) P(ConvEpiPtrs) P(Reduce3dParams)
+ P(ReduceGeneralParams) P(PoolParams) P(GatherRowsParams) P(GatherGeneralParams) P(ScatterRowsParams) P(ScatterGeneralParams) P(ThreefryParams) }
+'''
+    import tempfile
+    kdir = os.path.join(ROOT, 'vkjax_amd', 'csrc', 'kernels')
+    with tempfile.TemporaryDirectory() as tmp:
+        open(os.path.join(tmp, 'sz.cpp'), 'w').write(src)
+        exe = os.path.join(tmp, 'sz')
+        subprocess.run(['/opt/rocm/bin/hipcc', '-x', 'hip', '--offload-arch=gfx950', '-O0', '-w', f'-I{kdir}',
+                        os.path.join(tmp, 'sz.cpp'), '-o', exe], check=True, capture_output=True)
+        sizes = dict(line.split() for line in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.splitlines())
+    sizes = {k: int(v) for k, v in sizes.items()}
+    f32 = np.dtype('float32')
+    b = lambda *shape: Buffer(None, f32, shape)
+    i = lambda *shape: Buffer(None, np.dtype('int32'), shape)
+    chain = K.EwChain(b(4, 8), (4, 8), K.broadcast_operand(b(4, 8), (4, 8)), [K.EwStep(K.EW['ADD_F'], K.broadcast_operand(b(8), (4, 8)))])
+    geom  = K.ConvGeometry(batch=1, Ho=4, Wo=4, N=8, H=4, W=4, Cin=4, KH=1, KW=1, xs=(64, 16, 4, 1), ws=(32, 32, 8, 1), os=(128, 32, 8, 1))
+    G, S = core.GatherDimensionNumbers, core.ScatterDimensionNumbers
+    launches = {
+        'EwParams': K.lower_ew_chain(chain), 'IotaParams': K.iota(i(8), 0), 'FillParams': K.fill(b(8), 0),
+        'ConcatParams': K.concat_part(b(4, 8), b(4, 3), 1, 0), 'ConvParams': K.conv_gemm(b(1, 4, 4, 8), b(1, 4, 4, 4), b(1, 1, 4, 8), geom),
+        'Reduce3dParams': K.reduce_3d(b(4), b(4, 8), 4, 8, 1, 'reduce_sum'),
+        'ReduceGeneralParams': K.reduce_general(b(4), b(4, 8), [(4, 8)], [(8, 1)], 'reduce_sum'),
+        'PoolParams': K.pool(b(1, 2, 2, 4), b(1, 4, 4, 4), 'reduce_max', (1, 2, 2, 1), (1, 2, 2, 1), (0, 0, 0, 0), (1, 1, 1, 1)),
+        'GatherRowsParams': K.gather_rows(b(3, 8), b(4, 8), i(3, 1), 3, 8, 4),
+        'GatherGeneralParams': K.gather_general(b(3, 8), b(4, 8), i(3, 1), (1,), (0,), (0,), (1, 8)),
+        'ScatterRowsParams': K.scatter_add_rows(b(4, 8), i(3, 1), b(3, 8), 3, 8, 4),
+        'ScatterGeneralParams': K.scatter_add_general(b(4, 8), i(3, 1), b(3, 8), (1,), (0,), (0,)),
+        'ThreefryParams': K.threefry2x32(*[Buffer(None, np.dtype('uint32'), (8,)) for _ in range(6)], key_is_scalar=False),
+    }
+    for struct, launch in launches.items():
+        assert len(launch.params) == sizes[struct], (struct, len(launch.params), sizes[struct])
+    assert sizes['ConvEpiPtrs'] == 8 * K.CONV_MAX_EPI
+    assert len(launches['ConvParams'].buffers) == 3 + K.CONV_MAX_EPI and len(launches['EwParams'].buffers) == 1 + K.EW_MAX_STEPS
+
+
+# ------------------------------------------------------------------ Function: trace cache
+
+TRACED = []
+
+def func0(x):
+    TRACED.append(x)
+    return x + 1
+
+
+def test_function_retraces_only_on_new_shape_or_dtype():
+    vk_func = vkjax_amd.Function(func0, frontend='minijax', plan_only=True)
+    get = lambda *a: vk_func._get_or_create_jaxpr_interpreter(a)
+    assert len(vk_func._jaxpr_interpreters) == 0
+    TRACED.clear(); get(65)
+    assert len(vk_func._jaxpr_interpreters) == 1 and isinstance(TRACED[-1], mj.Tracer)
+    TRACED.clear(); get(77)
+    assert len(vk_func._jaxpr_interpreters) == 1 and TRACED == []
+    get(np.zeros([4, 4])); get(np.zeros([4, 4]))
+    assert len(vk_func._jaxpr_interpreters) == 2
+    get(np.zeros([4, 5]))
+    assert len(vk_func._jaxpr_interpreters) == 3
+    #dtype is part of the key, and is preserved in the traced output type
+    x = np.arange(128).astype('uint32')
+    (_, s0), (_, s1) = get(x), get(x.astype('float32'))
+    assert len(vk_func._jaxpr_interpreters) == 5
+    assert s0.dtype == np.uint32 and s1.dtype == np.float32
+
+
+def test_static_argnums_are_not_device_arguments():
+    def f(x, flag):
+        return x * 2 if flag else x * 3
+    vk = vkjax_amd.wrap(f, static_argnums=(1,), frontend='minijax', plan_only=True)
+    interp, _ = vk._get_or_create_jaxpr_interpreter((np.ones(3), True))
+    assert len(interp.input_buffers) == 1
+    assert len(vk._jaxpr_interpreters) == 1
+    vk._get_or_create_jaxpr_interpreter((np.ones(3), False))
+    assert len(vk._jaxpr_interpreters) == 2
+
+
+def test_wrong_argument_count_raises_typeerror():
+    closed = mj.make_jaxpr(lambda x, y: x + y)(1.0, 2.0)
+    interp = JaxprInterpreter(closed, plan_only=True)
+    with pytest.raises(TypeError, match='Expected 2 input arguments, received 1'):
+        interp.run(1.0)
+    with pytest.raises(RuntimeError, match='plan_only'):
+        interp.run(1.0, 2.0)
+
+
+# ------------------------------------------------------------------ buffer pool
+
+def test_bufferpool_lowlevel_reuse():
+    pool = BufferPool(PlanOnlyDevice(), 1)
+    aval = core.ShapedArray((10, 10), 'float32')
+    v0, v1, v3 = core.Var(0, '', aval), core.Var(1, '', aval), core.Var(3, '', aval)
+    pool.get_buffer(v0, increment_op_counter=True); assert pool.op_counter == 1
+    pool.get_buffer(v1, increment_op_counter=True); assert pool.op_counter == 2
+    pool.get_buffer(v0, increment_op_counter=True); assert pool.op_counter == 3
+    pool.get_buffer(v3, increment_op_counter=True)
+    assert [pool.buffers[v].accesses for v in (v0, v1, v3)] == GOLDEN['bufferpool_lowlevel_accesses']
+    pool.create_tensors()
+    assert len(pool.unique_tensors()) == GOLDEN['bufferpool_lowlevel_unique_tensors']
+
+
+def test_bufferpool_highlevel_reuse():
+    def func(a, b):
+        c = a + 5
+        d = c * b
+        e = d - 2
+        f = e ** 3
+        g = f - 1
+        h = g * 5
+        return h
+    closed = mj.make_jaxpr(func)(65, 5)
+    pool = JaxprInterpreter(closed, reuse_buffers=True, fuse=False, plan_only=True).bufferpool
+    assert len(pool.buffers) == 11
+    assert len(pool.unique_tensors()) == GOLDEN['bufferpool_highlevel_unique_tensors']   #11 buffers overall, -3 re-used
+    pool = JaxprInterpreter(closed, reuse_buffers=False, fuse=False, plan_only=True).bufferpool
+    assert len(pool.unique_tensors()) == 11
+
+
+def test_views_share_storage_and_32bit_canonicalisation():
+    closed = mj.make_jaxpr(lambda x: lax.bitcast_convert_type((x + 1).reshape(2, 8), np.uint32))(np.zeros(16, np.float32))
+    interp = JaxprInterpreter(closed, fuse=False, plan_only=True)
+    assert [l.kernel for l in interp.launches] == ['ew_chain_v4']      #reshape and bitcast are free
+    words = to_device_words(np.array([True, False, True]))
+    assert words.dtype == np.uint32 and words.tolist() == [1, 0, 1]
+    assert view_or_convert_from_32bit(words, np.bool_).tolist() == [True, False, True]
+    assert to_device_words(np.array([1.5], np.float64)).view(np.float32)[0] == 1.5
+    assert to_device_words(np.array([-2], np.int64)).view(np.int32)[0] == -2
+    with pytest.raises(NotImplementedError):
+        to_device_words(np.array([1 + 2j]))
+
+
+# ------------------------------------------------------------------ dispatch errors
+
+def _eqn(name, invals, out_aval, **params):
+    invars = [core.Var(None, '', core.ShapedArray(np.shape(v), np.asarray(v).dtype)) for v in invals]
+    return core.JaxprEqn(invars, [core.Var(None, '', out_aval)], core.Primitive(name), params), invars
+
+
+def test_unknown_primitive_and_bad_params():
+    pool = BufferPool(PlanOnlyDevice())
+    eq, invars = _eqn('cholesky', [np.zeros((2, 2), np.float32)], core.ShapedArray((2, 2), 'float32'))
+    with pytest.raises(NotImplementedError):
+        ops.analyze_jaxpr(pool, core.Jaxpr([], invars, eq.outvars, [eq]))
+    eq, invars = _eqn('add', [np.zeros((2, 3), np.float32), np.zeros((4,), np.float32)], core.ShapedArray((2, 3), 'float32'))
+    with pytest.raises(ValueError, match='Cannot broadcast'):
+        ops.analyze_jaxpr(pool, core.Jaxpr([], invars, eq.outvars, [eq]))
+    eq, invars = _eqn('exp', [np.zeros((2,), np.int32)], core.ShapedArray((2,), 'int32'))
+    with pytest.raises(NotImplementedError):
+        ops.analyze_jaxpr(pool, core.Jaxpr([], invars, eq.outvars, [eq]))
+    eq, invars = _eqn('dot_general', [np.zeros((2, 3), np.float32), np.zeros((3, 2), np.float32)], core.ShapedArray((2, 2), 'float32'),
+                      dimension_numbers=(((1,), (0,)), ((), ())), precision='HIGHEST')
+    with pytest.raises(AssertionError):
+        ops.analyze_jaxpr(pool, core.Jaxpr([], invars, eq.outvars, [eq]))
+    with pytest.raises(NotImplementedError):
+        core.canonicalize_dtype(np.complex64)
+
+
+def test_dropped_outputs_are_skipped_and_calls_are_inlined():
+    aval = core.ShapedArray((4,), 'float32')
+    x = core.Var(None, '', aval)
+    dropped = core.JaxprEqn([x], [core.DropVar(aval)], core.Primitive('exp'), {})
+    kept    = core.JaxprEqn([x], [core.Var(None, '', aval)], core.Primitive('neg'), {})
+    pool = BufferPool(PlanOnlyDevice())
+    out = ops.analyze_jaxpr(pool, core.Jaxpr([], [x], kept.outvars, [dropped, kept]))
+    assert len(out) == 1 and out[0].equation is kept
+    closed = mj.make_jaxpr(lambda a, b: mj.jit(lambda u: u + u)(a) + mj.jit(lambda u, v: u + v)(b, 1.0))(5.0, 7.1)
+    interp = JaxprInterpreter(closed, fuse=False, plan_only=True)
+    assert [l.kernel for l in interp.launches] == ['ew_chain_v1'] * 3
+
+
+def test_opcode_table_and_tile_choice():
+    assert K.EW['ADD_F'] == 1 and K.EW['SEL_P'] == 50 and len(set(K.EW.values())) == len(K.EW)
+    assert K.choose_conv_tile(200704, 256)[0] == '128x128'
+    assert K.choose_conv_tile(200704, 64)[0] == '128x64'
+    assert K.choose_conv_tile(8, 16)[1] <= 64

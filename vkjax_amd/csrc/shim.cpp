@@ -9,7 +9,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
+#include <unordered_map>
 #include <string>
 #include <vector>
 
@@ -42,6 +44,7 @@ constexpr uint32_t MAGIC_CTX = 0x766b4a43, MAGIC_BUF = 0x766b4a42, MAGIC_MOD = 0
                    MAGIC_FN = 0x766b4a46, MAGIC_SEQ = 0x766b4a53;
 
 struct Ctx {
+    uint64_t    handle = 0;
     uint32_t    magic = MAGIC_CTX;
     int         device = 0;
     hipStream_t stream = nullptr;
@@ -49,6 +52,7 @@ struct Ctx {
 };
 
 struct Buf {
+    uint64_t    handle = 0;
     uint32_t magic = MAGIC_BUF;
     Ctx*     ctx = nullptr;
     void*    dptr = nullptr;
@@ -56,12 +60,14 @@ struct Buf {
 };
 
 struct Mod {
+    uint64_t    handle = 0;
     uint32_t    magic = MAGIC_MOD;
     Ctx*        ctx = nullptr;
     hipModule_t module = nullptr;
 };
 
 struct Fn {
+    uint64_t    handle = 0;
     uint32_t      magic = MAGIC_FN;
     Mod*          mod = nullptr;
     hipFunction_t fn = nullptr;
@@ -82,6 +88,7 @@ struct Launch {
 };
 
 struct Seq {
+    uint64_t    handle = 0;
     uint32_t              magic = MAGIC_SEQ;
     Ctx*                  ctx = nullptr;
     bool                  profiling = false;
@@ -91,13 +98,34 @@ struct Seq {
     int                   stamps_valid = 0;
 };
 
+// Handles are keys into a process-wide table, never raw addresses, so that a stale or made-up
+// handle is rejected instead of being dereferenced.
+struct Registry {
+    std::mutex mu;
+    std::unordered_map<uint64_t, std::pair<uint32_t, void*>> live;
+    uint64_t next = 0x1000;
+} g_registry;
+
 template <class T>
 T* from_handle(vkj_handle h, uint32_t magic) {
-    T* p = reinterpret_cast<T*>(static_cast<uintptr_t>(h));
-    return (p && p->magic == magic) ? p : nullptr;
+    std::lock_guard<std::mutex> lock(g_registry.mu);
+    auto it = g_registry.live.find(h);
+    if (it == g_registry.live.end() || it->second.first != magic) return nullptr;
+    return static_cast<T*>(it->second.second);
 }
 template <class T>
-vkj_handle to_handle(T* p) { return static_cast<vkj_handle>(reinterpret_cast<uintptr_t>(p)); }
+vkj_handle to_handle(T* p) {
+    std::lock_guard<std::mutex> lock(g_registry.mu);
+    const uint64_t h = g_registry.next++;
+    g_registry.live[h] = {p->magic, p};
+    p->handle = h;
+    return h;
+}
+template <class T>
+void retire(T* p) {
+    std::lock_guard<std::mutex> lock(g_registry.mu);
+    g_registry.live.erase(p->handle);
+}
 
 int use(Ctx* c) {
     HIP_TRY(hipSetDevice(c->device));
@@ -158,7 +186,7 @@ int vkj_ctx_destroy(vkj_handle h) {
     hipEventDestroy(c->ev_begin);
     hipEventDestroy(c->ev_end);
     hipStreamDestroy(c->stream);
-    c->magic = 0;
+    retire(c);
     delete c;
     return 0;
 }
@@ -211,7 +239,7 @@ int vkj_module_unload(vkj_handle h, vkj_handle mh) {
     if (int r = use(c)) return r;
     HIP_TRY(hipStreamSynchronize(c->stream));
     HIP_TRY(hipModuleUnload(m->module));
-    m->magic = 0;
+    retire(m);
     delete m;
     return 0;
 }
@@ -256,7 +284,7 @@ int vkj_buf_free(vkj_handle h, vkj_handle bh) {
     if (int r = use(c)) return r;
     HIP_TRY(hipStreamSynchronize(c->stream));
     HIP_TRY(hipFree(b->dptr));
-    b->magic = 0;
+    retire(b);
     delete b;
     return 0;
 }
@@ -338,7 +366,7 @@ int vkj_seq_destroy(vkj_handle sh) {
     for (auto& t : s->uploads)   if (t.staging) hipHostFree(t.staging);
     for (auto& t : s->downloads) if (t.staging) hipHostFree(t.staging);
     for (auto e : s->stamps) hipEventDestroy(e);
-    s->magic = 0;
+    retire(s);
     delete s;
     return 0;
 }
