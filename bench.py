@@ -48,6 +48,9 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-fuse', action='store_true')
     ap.add_argument('--profile-iters', type=int, default=3)
+    ap.add_argument('--calibration-copy', action='store_true',
+                    help='also launch one plain 256 MiB -> 256 MiB copy (kernel ew_chain_v4, the only dispatch with a 16777216-block '
+                         'grid), so that a hardware-counter run of this command holds a dispatch of known HBM traffic')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: the hot path runs on a single MI355X and nothing here shards '
@@ -71,6 +74,13 @@ def main():
     interp, _ = wrapped._get_or_create_jaxpr_interpreter(tuple(inputs))
     build_s = time.perf_counter() - t0
     interp.upload_inputs(*inputs)
+
+    if args.calibration_copy:
+        n = 64 * 1024 * 1024
+        copy = vkjax_amd.wrap(lambda x: x + 0.0, frontend='minijax')
+        ci, _ = copy._get_or_create_jaxpr_interpreter((np.zeros(n, np.float32),))
+        ci.replay(1)
+        dev.sync()
 
     for _ in range(args.warmup):
         interp.replay(1)

@@ -58,3 +58,55 @@ def test_gather_scatter_small_exact_and_full():
     expected = np.zeros(table.shape, np.float64)
     np.add.at(expected, idx.reshape(-1), updates.reshape(-1, table.shape[1]).astype(np.float64))
     assert np.allclose(acc, expected, rtol=1e-5, atol=1e-6)
+
+
+def test_fusion_does_not_change_a_single_bit():
+    '''The fused program (chains merged, batch-norm / ReLU / residual in the convolution epilogue)
+    performs the same fp32 operations in the same order as one launch per equation.'''
+    from vkjax_amd.minijax import tree_util
+    cases = [(W.mlp, W.mlp_inputs()), (W.conv_block, W.conv_block_inputs(batch=3, size=20, channels=24)),
+             (W.resnet50, W.resnet50_inputs(batch=2, size=64, num_classes=40, width_scale=0.25)),
+             (lambda key: W.rng_uniform(key, (33, 20)), W.rng_inputs())]
+    for f, args in cases:
+        fused   = vkjax_amd.wrap(f, frontend='minijax', fuse=True)
+        unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)
+        a, b = fused(*args), unfused(*args)
+        n_fused   = len(list(fused._jaxpr_interpreters.values())[0].launches)
+        n_unfused = len(list(unfused._jaxpr_interpreters.values())[0].launches)
+        assert n_fused < n_unfused
+        assert_tree_close(a, b, exact=True, what=getattr(f, '__name__', 'f'))
+
+
+def test_return_all_and_profiling():
+    '''The debugging surface of the reference: run(..., return_all=True) returns every variable
+    (reference: vkjax/kompute_jaxpr_interpreter.py:85-89) and profiling=True returns per-op timings
+    labelled data2device / equations / data2host (reference: :91-95).'''
+    from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
+    from oracle.eval_jaxpr import eval_closed_jaxpr
+    args   = W.affine_inputs()
+    closed = mj.make_jaxpr(W.affine)(*args)
+    interp = JaxprInterpreter(closed, reuse_buffers=False, fuse=False)
+    outs, env = interp.run(*args, return_all=True)
+    _, env_true = eval_closed_jaxpr(closed, *args, return_env=True)
+    for var, val in env_true.items():
+        assert np.allclose(env[var], val, rtol=1e-4, atol=1e-6), var
+    f = vkjax_amd.wrap(W.affine, profiling=True, frontend='minijax', fuse=False)
+    y, info = f(*args)
+    assert [label for label, _ in info][0] == 'data2device' and info[-1][0] == 'data2host'
+    assert len(info) == 2 + 2 and all(dt >= 0 for _, dt in info)
+
+
+def test_function_semantics_on_device():
+    '''reference: tests/test_function.py:13-16,48-60'''
+    def func0(x):
+        return x + 1
+    vk_func = vkjax_amd.Function(func0, frontend='minijax')
+    assert vk_func(65) == 66
+    assert vk_func(-5) == -4
+    x  = np.arange(128).astype('uint32')
+    y0 = vk_func(x)
+    y1 = vk_func(x.astype('float32'))
+    assert np.allclose(y0, y1) and y0.dtype == np.uint32 and y1.dtype == np.float32
+    assert len(vk_func._jaxpr_interpreters) == 3
+    with pytest.raises(TypeError):
+        list(vk_func._jaxpr_interpreters.values())[0].run(1, 2)

@@ -239,6 +239,8 @@ def test_dropped_outputs_are_skipped_and_calls_are_inlined():
 
 def test_opcode_table_and_tile_choice():
     assert K.EW['ADD_F'] == 1 and K.EW['SEL_P'] == 50 and len(set(K.EW.values())) == len(K.EW)
-    assert K.choose_conv_tile(200704, 256)[0] == '128x128'
-    assert K.choose_conv_tile(200704, 64)[0] == '128x64'
+    tags = [t[0] for t in K.CONV_TILES]
+    for m, n in [(200704, 256), (200704, 64), (3136, 512), (8, 16), (1, 1)]:
+        tag, bm, bn, nt = K.choose_conv_tile(m, n)
+        assert tag in tags and nt in (64, 256)
     assert K.choose_conv_tile(8, 16)[1] <= 64

@@ -21,6 +21,8 @@ from .minijax import core
 class TensorPlaceholder:
     def __init__(self, t=None):
         self.t = t
+        #set when fusion keeps the value in registers: the variable never gets storage
+        self.elided = False
 
 
 class PlannedTensor:
@@ -98,6 +100,8 @@ class Buffer:
     def numpy(self) -> np.ndarray:
         '''Blocking read of the device contents as an array of this buffer's dtype and shape.'''
         t = self.tensor
+        if self._placeholder.elided:
+            return None
         if t is None or getattr(t, 'handle', None) is None:
             raise RuntimeError('buffer has no device storage')
         raw = t.download(self.nbytes()) if self.size else np.zeros(0, np.uint32)
@@ -190,10 +194,8 @@ class BufferPool:
         #largest first: they are the easiest to reuse
         for i in reversed(order):
             b, v = buffers[i], keys[i]
-            if b.tensor is not None:
-                #constants, I/O, or a view whose sibling already got storage
-                if b.tensor in tensor_access_map:
-                    pass
+            if b.tensor is not None or b._placeholder.elided:
+                #constants, I/O, a view whose sibling already got storage, or a fused-away intermediate
                 continue
             t = self._search_for_free_tensor(b, tensor_access_map) if self.reuse_tensors else None
             if t is None:

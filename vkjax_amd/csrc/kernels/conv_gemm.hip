@@ -47,21 +47,10 @@ struct ConvParams {
     uint32_t epi_op[CONV_MAX_EPI];
     uint32_t epi_flags[CONV_MAX_EPI];   // bit1: operand is the left argument
     uint32_t epi_kind[CONV_MAX_EPI];    // 0 none, 1 scalar, 2 per-feature vector [N], 3 full tensor laid out like out
+    int32_t  epi_first_full;            // index of the first kind-3 step, or -1
 };
 
 struct ConvEpiPtrs { const float* p[CONV_MAX_EPI]; };
-
-__device__ __forceinline__ float epi_apply(uint32_t op, float a, float b) {
-    switch (op) {
-        case CEW_ADD_F: return a + b;
-        case CEW_SUB_F: return a - b;
-        case CEW_MUL_F: return a * b;
-        case CEW_DIV_F: return a / b;
-        case CEW_MAX_F: return (a > b || a != a) ? a : b;
-        case CEW_MIN_F: return (a < b || a != a) ? a : b;
-        default:        return a;
-    }
-}
 
 template <int WGM, int WGN, int TM, int TN, bool A_FAST, bool B_FAST>
 __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
@@ -71,6 +60,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     constexpr int LDA = BK + 4, LDB = BN + 4;
     __shared__ __attribute__((aligned(16))) float As[BM * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
+    __shared__ float Es[CONV_MAX_EPI * BN];         // per-column operands of the epilogue steps
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -86,6 +76,23 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     const int tile_m = tile / P.tiles_n, tile_n = tile - tile_m * P.tiles_n;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int HoWo = P.Ho * P.Wo;
+
+    // Scalar and per-feature epilogue operands are fetched once per block, at its very start, and
+    // parked in LDS behind the first k tile's loads, so that the epilogue never waits on global
+    // memory for them.
+    constexpr int E_PER_THREAD = (CONV_MAX_EPI * BN + NT - 1) / NT;
+    float e_reg[E_PER_THREAD];
+#pragma unroll
+    for (int q = 0; q < E_PER_THREAD; ++q) {
+        const int idx = tid + q * NT;
+        e_reg[q] = 0.f;
+        if (idx < (int)P.nepi * BN) {
+            const int e = idx / BN, n = n0 + idx - e * BN;
+            const uint32_t kind = P.epi_kind[e];
+            if (kind == 1) e_reg[q] = epi.p[e][0];
+            else if (kind == 2 && n < P.N) e_reg[q] = epi.p[e][n];
+        }
+    }
 
     // ---------------- per-thread load assignment ----------------
     // A fast: 16-byte vectors along k. A generic: one row, a run of consecutive k.
@@ -131,8 +138,10 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     auto a_element_offset = [&](int p, int r, int s, int c, bool& ok) -> int {
         int hi = a_hi0[p] + r * P.DH, wi = a_wi0[p] + s * P.DW;
         ok = hi >= 0 && wi >= 0;
-        if (P.LH > 1) { ok = ok && (hi % P.LH == 0); hi /= P.LH; }
-        if (P.LW > 1) { ok = ok && (wi % P.LW == 0); wi /= P.LW; }
+        if constexpr (!A_FAST) {                      // the 16-byte path is only chosen without lhs dilation
+            if (P.LH > 1) { ok = ok && (hi % P.LH == 0); hi /= P.LH; }
+            if (P.LW > 1) { ok = ok && (wi % P.LW == 0); wi /= P.LW; }
+        }
         ok = ok && hi < P.H && wi < P.W;
         return a_base[p] + hi * P.xs_h + wi * P.xs_w + c * P.xs_c;
     };
@@ -222,6 +231,10 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 
     const int ktiles = (P.K + BK - 1) / BK;
     load_tiles(0);
+#pragma unroll
+    for (int q = 0; q < E_PER_THREAD; ++q)
+        if (tid + q * NT < (int)P.nepi * BN) Es[tid + q * NT] = e_reg[q];
+    if (ktiles == 0) __syncthreads();            // otherwise the barriers of the k loop publish Es
     for (int kt = 0; kt < ktiles; ++kt) {
         store_tiles();
         __syncthreads();
@@ -251,46 +264,89 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     }
 
     // ---------------- epilogue + store ----------------
-    // accumulator element v of a lane: row = 8*(v/4) + 4*half + v%4, column = l32
-    auto out_offset = [&](int m, int n) -> int64_t {
-        if (P.c_contig) return (int64_t)m * P.N + n;
+    // accumulator element v of a lane: row = 8*(v/4) + 4*half + v%4, column = l32.
+    // Offsets fit 32 bits: the host refuses tensors of 2^31 elements or more.
+    auto out_offset = [&](int m, int n) -> int {
+        if (P.c_contig) return m * P.N + n;
         const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
-        return (int64_t)b * P.os_b + (int64_t)ho * P.os_h + (int64_t)wo * P.os_w + (int64_t)n * P.os_n;
+        return b * P.os_b + ho * P.os_h + wo * P.os_w + n * P.os_n;
     };
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
+    // offset of accumulator element v of sub-tile (i, j), or -1 outside the problem
+    auto elem_offset = [&](int i, int j, int v) -> int {
         const int n = n0 + (wn * TN + j) * 32 + l32;
-        if (n >= P.N) continue;
-        for (uint32_t e = 0; e < P.nepi; ++e) {          // uniform, not unrolled
-            const uint32_t op = P.epi_op[e], kind = P.epi_kind[e];
-            const bool left = (P.epi_flags[e] & 2u) != 0;
-            const float* __restrict__ src = epi.p[e];
-            const float o1 = kind == 1 ? src[0] : kind == 2 ? src[n] : 0.f;
+        const int m = m0 + (wm * TM + i) * 32 + 4 * half + 8 * (v / 4) + (v % 4);
+        return (m < P.M && n < P.N) ? out_offset(m, n) : -1;
+    };
+    // the first full-size operand (a residual input) is fetched for the whole tile at once
+    // (for the largest tile that would not fit the register file: it loads sub-tile by sub-tile)
+    constexpr bool PREFETCH_FULL = TM * TN <= 2;
+    float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
+    const int first_full = PREFETCH_FULL ? P.epi_first_full : -1;
+    if (PREFETCH_FULL && first_full >= 0) {
+        const float* __restrict__ src = epi.p[first_full];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int m = m0 + (wm * TM + i) * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-                    float o = o1;
-                    if (kind == 3) o = m < P.M ? src[out_offset(m, n)] : 0.f;
-                    const float y = acc[i][j][v];
-                    acc[i][j][v] = epi_apply(op, left ? o : y, left ? y : o);
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) { const int o = elem_offset(i, j, v); full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = o >= 0 ? src[o] : 0.f; }
+    }
+    for (int e = 0; e < (int)P.nepi; ++e) {              // uniform, not unrolled
+        const uint32_t kind = P.epi_kind[e];
+        const uint32_t code = P.epi_op[e] * 2u + ((P.epi_flags[e] >> 1) & 1u);   // bit0: operand on the left
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                float ov[16];
+                if (kind == 3) {
+                    if (PREFETCH_FULL && e == first_full) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) ov[v] = full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v];
+                    } else {
+                        const float* __restrict__ src = epi.p[e];
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) { const int o = elem_offset(i, j, v); ov[v] = o >= 0 ? src[o] : 0.f; }
+                    }
+                } else {
+                    const float o1 = Es[e * BN + (wn * TN + j) * 32 + l32];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) ov[v] = o1;
                 }
+#define EPI_LOOP(expr)                                              \
+                _Pragma("unroll") for (int v = 0; v < 16; ++v) {    \
+                    const float y = acc[i][j][v], o = ov[v];        \
+                    acc[i][j][v] = (expr);                          \
+                }
+                switch (code) {                              // one uniform branch per step, not per element
+                    case CEW_ADD_F * 2: case CEW_ADD_F * 2 + 1: EPI_LOOP(y + o) break;
+                    case CEW_MUL_F * 2: case CEW_MUL_F * 2 + 1: EPI_LOOP(y * o) break;
+                    case CEW_SUB_F * 2:     EPI_LOOP(y - o) break;
+                    case CEW_SUB_F * 2 + 1: EPI_LOOP(o - y) break;
+                    case CEW_DIV_F * 2:     EPI_LOOP(y / o) break;
+                    case CEW_DIV_F * 2 + 1: EPI_LOOP(o / y) break;
+                    case CEW_MAX_F * 2:     EPI_LOOP((y > o || y != y) ? y : o) break;
+                    case CEW_MAX_F * 2 + 1: EPI_LOOP((o > y || o != o) ? o : y) break;
+                    case CEW_MIN_F * 2:     EPI_LOOP((y < o || y != y) ? y : o) break;
+                    case CEW_MIN_F * 2 + 1: EPI_LOOP((o < y || o != o) ? o : y) break;
+                    default: break;
+                }
+#undef EPI_LOOP
             }
-        }
+    }
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int m = m0 + (wm * TM + i) * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-                if (m < P.M) out[out_offset(m, n)] = acc[i][j][v];
+                const int o = elem_offset(i, j, v);
+                if (o >= 0) out[o] = acc[i][j][v];
             }
-        }
-    }
 }
 
 #define CONV_KERNEL(name, WGM, WGN, TM, TN, AF, BF)                                                         \
-    extern "C" __global__ __launch_bounds__(64 * WGM * WGN) void name(                                       \
+    extern "C" __global__ __launch_bounds__(64 * WGM * WGN) __attribute__((amdgpu_waves_per_eu(2))) void name(                                     \
         float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
         ConvEpiPtrs epi, ConvParams P) {                                                                     \
         conv_gemm_body<WGM, WGN, TM, TN, AF, BF>(out, x, w, epi, P);                                         \

@@ -29,13 +29,14 @@ class Op:
     order (entries can be None), `shader` names the kernel, `equation` is the jaxpr equation it
     came from (or a label string for helper launches), as in the reference's Op tuple
     (vkjax/ops.py:28-41).'''
-    __slots__ = ('equation', 'chain', '_launch', 'conv')
+    __slots__ = ('equation', 'chain', '_launch', 'conv', 'index')
 
     def __init__(self, equation, launch: tp.Optional[Launch] = None, chain: tp.Optional[EwChain] = None, conv=None):
         self.equation = equation
         self.chain    = chain
         self._launch  = launch
         self.conv     = conv          #(out, lhs, rhs, geometry, epilogue list) for conv/dot ops, so a fusion pass can extend it
+        self.index    = None          #position in the program (the pool's op counter when the op was created)
 
     @property
     def launch(self) -> Launch:
@@ -76,7 +77,12 @@ def analyze_jaxpr(bufferpool: BufferPool, jaxpr) -> tp.List[Op]:
         method = globals().get(opname, None)
         if method is None or not callable(method) or opname.startswith('_'):
             raise NotImplementedError(eq)
-        all_ops += method(bufferpool, eq)
+        position   = bufferpool.op_counter
+        method_ops = method(bufferpool, eq)
+        for op in method_ops:
+            if op.index is None:
+                op.index = position
+        all_ops += method_ops
     return all_ops
 
 
