@@ -104,20 +104,23 @@ def test_reduce_window_matrix(f, desc, args, exact):
     check_against_oracle(f, args, exact=exact, rtol=1e-5, atol=1e-6)
 
 
-@pytest.mark.parametrize('tile', ['128x128', '128x64', '64x64', '32x32'])
-def test_every_tile_and_loader_variant(tile):
-    '''All 16 kernel instantiations: each tile shape with 16-byte (f) or strided (g) loads on either operand.'''
+@pytest.mark.parametrize('tile,bk', [('128x128', 32), ('128x64', 32), ('64x64', 32), ('64x64', 64), ('32x32', 32), ('32x32', 64)])
+def test_every_tile_and_loader_variant(tile, bk):
+    '''All 24 kernel instantiations: each tile shape and k step with 16-byte (f) or strided (g) loads on
+    either operand; the ff2 / ff3 cases have Cin % 64 == 0 (tap position kept in scalar registers) and a
+    1x1 unpadded kernel (rows addressed as a flat matrix).'''
     from vkjax_amd import kernels as K
     cases = {'ff': ([3, 20, 17, 16], [3, 3, 16, 24]), 'gg': ([2, 13, 11, 5], [3, 3, 5, 7]),
-             'gf': ([2, 13, 11, 3], [3, 3, 3, 64]), 'fg': ([2, 13, 11, 8], [3, 3, 8, 10])}
-    K.FORCE_CONV_TILE = tile
+             'gf': ([2, 13, 11, 3], [3, 3, 3, 64]), 'fg': ([2, 13, 11, 8], [3, 3, 8, 10]),
+             'ff2': ([2, 9, 11, 64], [3, 3, 64, 40]), 'ff3': ([2, 9, 11, 128], [1, 1, 128, 72])}
+    K.FORCE_CONV_TILE, K.FORCE_CONV_BK = tile, bk
     try:
         for variant, (xs, ks) in cases.items():
-            print(f'tile {tile} loaders {variant}', flush=True)
+            print(f'tile {tile} bk {bk} loaders {variant}', flush=True)
             x = rng.randint(-4, 5, size=xs).astype(np.float32)
             k = rng.randint(-3, 4, size=ks).astype(np.float32)
             _, _, fn = check_against_oracle(conv2, [x, k], exact=True)
             kernel = list(fn._jaxpr_interpreters.values())[0].launches[0].kernel
-            assert kernel == f'conv_gemm_{tile}_{variant}', kernel
+            assert kernel == f'conv_gemm_{tile}x{bk}_{variant[:2]}', kernel
     finally:
-        K.FORCE_CONV_TILE = None
+        K.FORCE_CONV_TILE = K.FORCE_CONV_BK = None

@@ -14,17 +14,19 @@
 // vkjax/shaders/dot_general.comp:10-34).
 //
 // Block = WGM x WGN waves, each wave owns TM x TN tiles of 32x32; block tile BM x BN with
-// BM = 32*WGM*TM, BN = 32*WGN*TN, K step 32. A and B tiles are staged through LDS
-// (A: [BM][36] so a lane reads 4 consecutive k with one 16-byte LDS load without bank
-// conflicts; B: [32][BN+4]); the next tiles are prefetched into registers while the MFMAs of
-// the current one run. The sum over k is order-free, so lanes 0-31 take k = 0..15 of a step and
-// lanes 32-63 take k = 16..31, which is what makes the 16-byte A reads possible.
+// BM = 32*WGM*TM, BN = 32*WGN*TN, K step BK (32 or 64). A and B tiles are staged through LDS
+// (A: [BM][BK+4] so a lane reads 4 consecutive k with one 16-byte LDS load without bank
+// conflicts; B: [BK][BN+4]); the next tiles are prefetched into registers while the MFMAs of
+// the current one run. The sum over k is order-free, so lanes 0-31 take the first half of a k
+// tile and lanes 32-63 the second half, which is what makes the 16-byte A reads possible.
+// The 16-byte paths read through buffer descriptors: a masked-out load is an out-of-range
+// offset that returns zeros, so padding, tile tails and partial tiles need no branches.
 // After the k loop an optional chain of element-wise steps (per-feature vectors, full-size
 // tensors or scalars as operands) is applied to the accumulators before the single store.
 #include "common.h"
 
-#define CONV_BK 32
 #define CONV_MAX_EPI 6
+#define CONV_OOB 0x80000000u     // byte offset beyond any descriptor: loads give 0, stores are dropped
 
 enum EwOpConv : uint32_t {
 #define EW_OP(name, num) CEW_##name = num,
@@ -48,15 +50,30 @@ struct ConvParams {
     uint32_t epi_flags[CONV_MAX_EPI];   // bit1: operand is the left argument
     uint32_t epi_kind[CONV_MAX_EPI];    // 0 none, 1 scalar, 2 per-feature vector [N], 3 full tensor laid out like out
     int32_t  epi_first_full;            // index of the first kind-3 step, or -1
+    int32_t  flat_rows;                 // m is the row index itself (batch = Wo = 1): no row decode
+    uint32_t x_bytes, w_bytes, out_bytes;   // sizes for the buffer descriptors (each below 2^31)
 };
 
 struct ConvEpiPtrs { const float* p[CONV_MAX_EPI]; };
 
-template <int WGM, int WGN, int TM, int TN, bool A_FAST, bool B_FAST>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ f32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0));
+}
+__device__ __forceinline__ float buffer_load_x1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+}
+__device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, byte_off, 0, 0);
+}
+
+template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST>
 __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
                                                const float* __restrict__ w, const ConvEpiPtrs& epi,
                                                const ConvParams& P) {
-    constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, BK = CONV_BK, NT = 64 * WGM * WGN;
+    constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, NT = 64 * WGM * WGN;
     constexpr int LDA = BK + 4, LDB = BN + 4;
     __shared__ __attribute__((aligned(16))) float As[BM * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
@@ -76,6 +93,9 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     const int tile_m = tile / P.tiles_n, tile_n = tile - tile_m * P.tiles_n;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int HoWo = P.Ho * P.Wo;
+
+    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, P.x_bytes), w_rsrc = make_rsrc(w, P.w_bytes),
+                                 o_rsrc = make_rsrc(out, P.out_bytes);
 
     // Scalar and per-feature epilogue operands are fetched once per block, at its very start, and
     // parked in LDS behind the first k tile's loads, so that the epilogue never waits on global
@@ -102,21 +122,27 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     constexpr int A_KG    = NT / BM;                // generic: k groups
     constexpr int A_KPT   = BK / A_KG;              // generic: k per thread
     constexpr int A_ROWS  = A_FAST ? A_NV : 1;
-    int a_base[A_ROWS], a_hi0[A_ROWS], a_wi0[A_ROWS];
+    // row state: element offset of (row, ky = kx = c = 0) and the input coordinates of that corner
+    int a_off[A_ROWS], a_hi0[A_ROWS], a_wi0[A_ROWS];
 #pragma unroll
     for (int p = 0; p < A_ROWS; ++p) {
         const int row = A_FAST ? (tid / A_VPR + p * A_RSTEP) : (tid % BM);
         const int m = m0 + row;
         if (m < P.M) {
-            const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
-            a_base[p] = b * P.xs_b;
-            a_hi0[p]  = ho * P.SH - P.PH;
-            a_wi0[p]  = wo * P.SW - P.PW;
+            int b = 0, ho = m, wo = 0;
+            if (!P.flat_rows) { b = m / HoWo; const int r2 = m - b * HoWo; ho = r2 / P.Wo; wo = r2 - ho * P.Wo; }
+            a_hi0[p] = ho * P.SH - P.PH;
+            a_wi0[p] = wo * P.SW - P.PW;
+            a_off[p] = b * P.xs_b + (A_FAST ? a_hi0[p] * P.xs_h + a_wi0[p] * P.xs_w + (tid % A_VPR) * 4 : 0);
         } else {
-            a_base[p] = 0; a_hi0[p] = -(1 << 28); a_wi0[p] = -(1 << 28);
+            a_off[p] = 0; a_hi0[p] = -(1 << 28); a_wi0[p] = -(1 << 28);
         }
     }
-    // position of this thread's first k inside the (ky, kx, c) space, advanced by BK per tile
+    // When a k tile never straddles two kernel taps (Cin % BK == 0) the tap (ky, kx) and first
+    // feature of a tile are the same for the whole block and live in scalar registers.
+    const bool uniform_taps = A_FAST && (P.Cin % BK == 0);
+    int t_r = 0, t_s = 0, t_c = 0;                  // uniform tile position
+    // otherwise every thread tracks the position of its own first k
     int ak = A_FAST ? (tid % A_VPR) * 4 : (tid / BM) * A_KPT;
     int ac, as_, ar;
     {
@@ -129,56 +155,55 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     constexpr int B_NV    = BK / B_RSTEP;
     constexpr int B_KG    = NT / BN;                // generic: k groups
     constexpr int B_KPT   = BK / B_KG;
+    // B fast: byte offset of this thread's first vector in tile 0, or out of range for columns >= N
+    const int      b_n    = n0 + (tid % B_VPR) * 4;
+    const uint32_t b_off0 = b_n < P.N ? (uint32_t)(((tid / B_VPR) * P.N + b_n) * 4) : CONV_OOB;
 
     f32x4 a_reg[A_FAST ? A_NV : 1];
     float a_sreg[A_FAST ? 1 : A_KPT];
     f32x4 b_reg[B_FAST ? B_NV : 1];
     float b_sreg[B_FAST ? 1 : B_KPT];
 
-    auto a_element_offset = [&](int p, int r, int s, int c, bool& ok) -> int {
-        int hi = a_hi0[p] + r * P.DH, wi = a_wi0[p] + s * P.DW;
-        ok = hi >= 0 && wi >= 0;
-        if constexpr (!A_FAST) {                      // the 16-byte path is only chosen without lhs dilation
-            if (P.LH > 1) { ok = ok && (hi % P.LH == 0); hi /= P.LH; }
-            if (P.LW > 1) { ok = ok && (wi % P.LW == 0); wi /= P.LW; }
-        }
-        ok = ok && hi < P.H && wi < P.W;
-        return a_base[p] + hi * P.xs_h + wi * P.xs_w + c * P.xs_c;
-    };
-
     auto load_tiles = [&](int k0) {
         // ---- A ----
         if constexpr (A_FAST) {
-            const bool kok = ak < P.K;
+            int r, s, koff;                          // tap of this thread's vector and its element offset
+            bool kok = true;
+            if (uniform_taps) {
+                r = t_r; s = t_s;
+                koff = t_r * P.DH * P.xs_h + t_s * P.DW * P.xs_w + t_c;
+            } else {
+                r = ar; s = as_;
+                koff = ar * P.DH * P.xs_h + as_ * P.DW * P.xs_w + ac - (tid % A_VPR) * 4;
+                kok = ak < P.K;
+            }
+            const int dh = r * P.DH, dw = s * P.DW;
 #pragma unroll
             for (int p = 0; p < A_NV; ++p) {
-                bool ok;
-                const int off = a_element_offset(p, ar, as_, ac, ok);
-                f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (ok && kok) v = *reinterpret_cast<const f32x4*>(x + off);
-                a_reg[p] = v;
+                const bool ok = kok && (uint32_t)(a_hi0[p] + dh) < (uint32_t)P.H && (uint32_t)(a_wi0[p] + dw) < (uint32_t)P.W;
+                a_reg[p] = buffer_load_x4(x_rsrc, ok ? (uint32_t)(a_off[p] + koff) * 4u : CONV_OOB);
             }
         } else {
             int c = ac, s = as_, r = ar, k = ak;
 #pragma unroll
             for (int j = 0; j < A_KPT; ++j) {
-                bool ok;
-                const int off = a_element_offset(0, r, s, c, ok);
-                a_sreg[j] = (ok && k < P.K) ? x[off] : 0.f;
+                int hi = a_hi0[0] + r * P.DH, wi = a_wi0[0] + s * P.DW;
+                bool ok = hi >= 0 && wi >= 0 && k < P.K;
+                if (P.LH > 1) { ok = ok && (hi % P.LH == 0); hi /= P.LH; }
+                if (P.LW > 1) { ok = ok && (wi % P.LW == 0); wi /= P.LW; }
+                ok = ok && hi < P.H && wi < P.W;
+                a_sreg[j] = ok ? x[a_off[0] + hi * P.xs_h + wi * P.xs_w + c * P.xs_c] : 0.f;
                 ++k; ++c;
                 if (c == P.Cin) { c = 0; ++s; if (s == P.KW) { s = 0; ++r; } }
             }
         }
         // ---- B ----
         if constexpr (B_FAST) {
-            const int n = n0 + (tid % B_VPR) * 4;
+            // rows k >= K fall beyond the descriptor and read as zeros
+            const uint32_t base = b_off0 == CONV_OOB ? CONV_OOB : b_off0 + (uint32_t)k0 * (uint32_t)P.N * 4u;
 #pragma unroll
-            for (int p = 0; p < B_NV; ++p) {
-                const int k = k0 + tid / B_VPR + p * B_RSTEP;
-                f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (k < P.K && n < P.N) v = *reinterpret_cast<const f32x4*>(w + (int64_t)k * P.N + n);
-                b_reg[p] = v;
-            }
+            for (int p = 0; p < B_NV; ++p)
+                b_reg[p] = buffer_load_x4(w_rsrc, base == CONV_OOB ? CONV_OOB : base + (uint32_t)(p * B_RSTEP) * (uint32_t)P.N * 4u);
         } else {
             const int n = n0 + tid % BN;
             int k = k0 + (tid / BN) * B_KPT;
@@ -191,9 +216,14 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
                 if (c == P.Cin) { c = 0; ++s; if (s == P.KW) { s = 0; ++r; } }
             }
         }
-        // advance this thread's A position by one k tile
-        ak += BK; ac += BK;
-        while (ac >= P.Cin) { ac -= P.Cin; ++as_; if (as_ == P.KW) { as_ = 0; ++ar; } }
+        // advance to the next k tile
+        if (uniform_taps) {
+            t_c += BK;
+            if (t_c == P.Cin) { t_c = 0; ++t_s; if (t_s == P.KW) { t_s = 0; ++t_r; } }
+        } else {
+            ak += BK; ac += BK;
+            while (ac >= P.Cin) { ac -= P.Cin; ++as_; if (as_ == P.KW) { as_ = 0; ++ar; } }
+        }
     };
 
     auto store_tiles = [&]() {
@@ -239,43 +269,52 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         store_tiles();
         __syncthreads();
         if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
-        // lanes 0-31 consume k = 0..15 of the tile, lanes 32-63 k = 16..31
-#pragma unroll
-        for (int g = 0; g < BK / 8; ++g) {
+        // lanes 0-31 consume the first half of the tile's k range, lanes 32-63 the second half.
+        // Fragments are double-buffered in registers: the LDS reads of group g+1 are in flight
+        // while the MFMAs of group g execute.
+        constexpr int G = BK / 8;
+        f32x4 af[2][TM];
+        float bf[2][TN][4];
+        auto load_frags = [&](int g, int buf) {
             const int kk = half * (BK / 2) + g * 4;
-            f32x4 af[TM];
-            float bf[TN][4];
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                af[i] = *reinterpret_cast<const f32x4*>(&As[((wm * TM + i) * 32 + l32) * LDA + kk]);
+                af[buf][i] = *reinterpret_cast<const f32x4*>(&As[((wm * TM + i) * 32 + l32) * LDA + kk]);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) bf[j][q] = Bs[(kk + q) * LDB + (wn * TN + j) * 32 + l32];
+                for (int q = 0; q < 4; ++q) bf[buf][j][q] = Bs[(kk + q) * LDB + (wn * TN + j) * 32 + l32];
+        };
+        load_frags(0, 0);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (g + 1 < G) load_frags(g + 1, (g + 1) & 1);
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][q], bf[j][q], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[g & 1][i][q], bf[g & 1][j][q], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     }
 
     // ---------------- epilogue + store ----------------
     // accumulator element v of a lane: row = 8*(v/4) + 4*half + v%4, column = l32.
-    // Offsets fit 32 bits: the host refuses tensors of 2^31 elements or more.
-    auto out_offset = [&](int m, int n) -> int {
-        if (P.c_contig) return m * P.N + n;
-        const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
-        return b * P.os_b + ho * P.os_h + wo * P.os_w + n * P.os_n;
-    };
-    // offset of accumulator element v of sub-tile (i, j), or -1 outside the problem
-    auto elem_offset = [&](int i, int j, int v) -> int {
+    // Byte offsets fit 31 bits: the host refuses larger tensors.
+    const bool whole_tile = m0 + BM <= P.M && n0 + BN <= P.N;
+    auto elem_offset = [&](int i, int j, int v) -> uint32_t {
         const int n = n0 + (wn * TN + j) * 32 + l32;
         const int m = m0 + (wm * TM + i) * 32 + 4 * half + 8 * (v / 4) + (v % 4);
-        return (m < P.M && n < P.N) ? out_offset(m, n) : -1;
+        int off;
+        if (P.c_contig) {
+            off = m * P.N + n;
+        } else {
+            const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
+            off = b * P.os_b + ho * P.os_h + wo * P.os_w + n * P.os_n;
+        }
+        return (whole_tile || (m < P.M && n < P.N)) ? (uint32_t)off * 4u : CONV_OOB;
     };
     // the first full-size operand (a residual input) is fetched for the whole tile at once
     // (for the largest tile that would not fit the register file: it loads sub-tile by sub-tile)
@@ -283,13 +322,14 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
     const int first_full = PREFETCH_FULL ? P.epi_first_full : -1;
     if (PREFETCH_FULL && first_full >= 0) {
-        const float* __restrict__ src = epi.p[first_full];
+        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(epi.p[first_full], P.out_bytes);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) { const int o = elem_offset(i, j, v); full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = o >= 0 ? src[o] : 0.f; }
+                for (int v = 0; v < 16; ++v)
+                    full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, elem_offset(i, j, v));
     }
     for (int e = 0; e < (int)P.nepi; ++e) {              // uniform, not unrolled
         const uint32_t kind = P.epi_kind[e];
@@ -304,9 +344,9 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 #pragma unroll
                         for (int v = 0; v < 16; ++v) ov[v] = full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v];
                     } else {
-                        const float* __restrict__ src = epi.p[e];
+                        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(epi.p[e], P.out_bytes);
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) { const int o = elem_offset(i, j, v); ov[v] = o >= 0 ? src[o] : 0.f; }
+                        for (int v = 0; v < 16; ++v) ov[v] = buffer_load_x1(f_rsrc, elem_offset(i, j, v));
                     }
                 } else {
                     const float o1 = Es[e * BN + (wn * TN + j) * 32 + l32];
@@ -339,27 +379,26 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int o = elem_offset(i, j, v);
-                if (o >= 0) out[o] = acc[i][j][v];
-            }
+            for (int v = 0; v < 16; ++v) buffer_store_x1(acc[i][j][v], o_rsrc, elem_offset(i, j, v));
 }
 
-#define CONV_KERNEL(name, WGM, WGN, TM, TN, AF, BF)                                                         \
-    extern "C" __global__ __launch_bounds__(64 * WGM * WGN) __attribute__((amdgpu_waves_per_eu(2))) void name(                                     \
+#define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF)                                                     \
+    extern "C" __global__ __launch_bounds__(64 * WGM * WGN) __attribute__((amdgpu_waves_per_eu(2))) void name( \
         float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
         ConvEpiPtrs epi, ConvParams P) {                                                                     \
-        conv_gemm_body<WGM, WGN, TM, TN, AF, BF>(out, x, w, epi, P);                                         \
+        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF>(out, x, w, epi, P);                                     \
     }
 
-// name = conv_gemm_<BM>x<BN>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads)
-#define CONV_TILE(tag, WGM, WGN, TM, TN)                               \
-    CONV_KERNEL(conv_gemm_##tag##_ff, WGM, WGN, TM, TN, true, true)    \
-    CONV_KERNEL(conv_gemm_##tag##_fg, WGM, WGN, TM, TN, true, false)   \
-    CONV_KERNEL(conv_gemm_##tag##_gf, WGM, WGN, TM, TN, false, true)   \
-    CONV_KERNEL(conv_gemm_##tag##_gg, WGM, WGN, TM, TN, false, false)
+// name = conv_gemm_<BM>x<BN>x<BK>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads)
+#define CONV_TILE(tag, WGM, WGN, TM, TN, BK)                               \
+    CONV_KERNEL(conv_gemm_##tag##_ff, WGM, WGN, TM, TN, BK, true, true)    \
+    CONV_KERNEL(conv_gemm_##tag##_fg, WGM, WGN, TM, TN, BK, true, false)   \
+    CONV_KERNEL(conv_gemm_##tag##_gf, WGM, WGN, TM, TN, BK, false, true)   \
+    CONV_KERNEL(conv_gemm_##tag##_gg, WGM, WGN, TM, TN, BK, false, false)
 
-CONV_TILE(128x128, 2, 2, 2, 2)
-CONV_TILE(128x64, 2, 2, 2, 1)
-CONV_TILE(64x64, 2, 2, 1, 1)
-CONV_TILE(32x32, 1, 1, 1, 1)
+CONV_TILE(128x128x32, 2, 2, 2, 2, 32)
+CONV_TILE(128x64x32, 2, 2, 2, 1, 32)
+CONV_TILE(64x64x32, 2, 2, 1, 1, 32)
+CONV_TILE(64x64x64, 2, 2, 1, 1, 64)
+CONV_TILE(32x32x32, 1, 1, 1, 1, 32)
+CONV_TILE(32x32x64, 1, 1, 1, 1, 64)

@@ -221,10 +221,13 @@ class ConvEpilogueStep(tp.NamedTuple):
 #(tag, BM, BN, threads, resident blocks per CU, relative MFMA efficiency of the tile shape)
 #(efficiencies are measured: TFLOP/s of each tile on large ResNet-50 layers relative to the best)
 CONV_TILES = (('128x128', 128, 128, 256, 2, 0.92), ('128x64', 128, 64, 256, 2, 0.88),
-              ('64x64', 64, 64, 256, 4, 1.00), ('32x32', 32, 32, 64, 16, 0.88))
+              ('64x64', 64, 64, 256, 4, 1.00), ('32x32', 32, 32, 64, 16, 0.80))
+#k steps each tile shape is built with
+CONV_TILE_BK = {'128x128': (32,), '128x64': (32,), '64x64': (32, 64), '32x32': (32, 64)}
 
-#tests set this to a tile tag to exercise every kernel variant irrespective of the heuristic
+#tests set these to exercise every kernel variant irrespective of the heuristics
 FORCE_CONV_TILE: tp.Optional[str] = None
+FORCE_CONV_BK:   tp.Optional[int] = None
 
 
 def choose_conv_tile(M: int, N: int, compute_units: int = 256):
@@ -244,30 +247,62 @@ def choose_conv_tile(M: int, N: int, compute_units: int = 256):
     return best
 
 
+def choose_conv_bk(tag: str, g: 'ConvGeometry') -> int:
+    '''The longer k step halves the barriers per MFMA. Measured on ResNet-50 layers it only pays
+    for the 64x64 tile on long contractions, and only when whole k tiles stay inside one kernel
+    tap (Cin % 64 == 0), which keeps the tap position in scalar registers.'''
+    options = CONV_TILE_BK[tag]
+    if FORCE_CONV_BK is not None and FORCE_CONV_BK in options:
+        return FORCE_CONV_BK
+    if tag == '64x64' and g.Cin % 64 == 0 and g.K >= 2048:
+        return 64
+    return 32
+
+
+def _flatten_pointwise(g: ConvGeometry) -> ConvGeometry:
+    '''A 1x1, stride-1, unpadded convolution over a dense feature-last array is a plain matrix
+    product of the [M, Cin] pixel matrix: present it as one batch of M rows so the kernel skips
+    the (batch, y, x) decode of every row.'''
+    dense_in  = g.xs[3] == 1 and g.xs[1] == g.W * g.xs[2] and g.xs[0] == g.H * g.W * g.xs[2]
+    dense_out = g.os == (g.Ho * g.Wo * g.N, g.Wo * g.N, g.N, 1)
+    pointwise = (g.KH == g.KW == 1 and g.SH == g.SW == 1 and g.PH == g.PW == 0 and g.LH == g.LW == 1
+                 and g.Ho == g.H and g.Wo == g.W)
+    if not (pointwise and dense_in and dense_out) or (g.batch == 1 and g.Wo == 1):
+        return g
+    M = g.M
+    return g._replace(batch=1, Ho=M, Wo=1, H=M, W=1, xs=(0, g.xs[2], 0, 1), os=(M * g.N, g.N, g.N, 1))
+
+
 def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: tp.Sequence[ConvEpilogueStep] = (),
               compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0) -> Launch:
     if len(epilogue) > CONV_MAX_EPI:
         raise ValueError('too many epilogue steps')
+    g = _flatten_pointwise(g)
     M, N, K = g.M, g.N, g.K
     for name, extent in (('lhs', lhs.size), ('rhs', rhs.size), ('out', out.size)):
-        if extent >= 2**31:
-            raise NotImplementedError(f'conv/dot {name} operand with {extent} elements exceeds 32-bit indexing')
+        if extent * 4 >= 2**31:
+            raise NotImplementedError(f'conv/dot {name} operand of {extent * 4} bytes exceeds the 2 GiB the kernel addresses')
     tag, bm, bn, nt = choose_conv_tile(M, N, compute_units)
+    bk = choose_conv_bk(tag, g)
     a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0
               and all(s % 4 == 0 for s in g.xs[:3]))
     b_fast = (g.ws[3] == 1 and N % 4 == 0 and rhs_offset % 4 == 0
               and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
     c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
+    flat_rows = g.batch == 1 and g.Wo == 1
     tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
     kinds = [e.kind for e in epilogue]
+    x_bytes = (lhs.size - lhs_offset) * 4
+    w_bytes = K * N * 4 if b_fast else (rhs.size - rhs_offset) * 4
     params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW, g.LH, g.LW,
                    *g.xs, *g.ws, *g.os, int(c_contig), tiles_m, tiles_n)
               + _u32(len(epilogue), *_pad([e.op for e in epilogue], CONV_MAX_EPI),
                      *_pad([2 if e.operand_left else 0 for e in epilogue], CONV_MAX_EPI), *_pad(kinds, CONV_MAX_EPI))
-              + _i32(kinds.index(3) if 3 in kinds else -1))
+              + _i32(kinds.index(3) if 3 in kinds else -1, int(flat_rows))
+              + _u32(x_bytes, w_bytes, out.size * 4))
     buffers = [(out, 0), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
     buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
-    kernel  = f'conv_gemm_{tag}_{"f" if a_fast else "g"}{"f" if b_fast else "g"}'
+    kernel  = f'conv_gemm_{tag}x{bk}_{"f" if a_fast else "g"}{"f" if b_fast else "g"}'
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue)
     return Launch(kernel, (tiles_m * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
                   bytes_moved=nbytes, flops=2 * M * N * K)
