@@ -48,8 +48,9 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-fuse', action='store_true')
     ap.add_argument('--profile-iters', type=int, default=3)
+    ap.add_argument('--dump-launches', default=None, help='write one line per launch (kernel, grid, FLOP, bytes, ms) to this file')
     ap.add_argument('--calibration-copy', action='store_true',
-                    help='also launch one plain 256 MiB -> 256 MiB copy (kernel ew_chain_v4, the only dispatch with a 16777216-block '
+                    help='also launch one plain 256 MiB -> 256 MiB copy (kernel ew_chain_v4_s2, the only dispatch with a 16777216-block '
                          'grid), so that a hardware-counter run of this command holds a dispatch of known HBM traffic')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -109,15 +110,23 @@ def main():
     prof = JaxprInterpreter(interp.jaxpr, interp.static_argnums, profiling=True, fuse=interp.fuse)
     prof.upload_inputs(*inputs)
     fam = {}
+    per_launch = np.zeros(len(prof.launches))
     for it in range(args.profile_iters + 1):
         prof.sequence.eval([None] * prof.sequence.n_slots, flags=hip.EVAL_SKIP_UPLOADS | hip.EVAL_SKIP_DOWNLOADS)
         if it == 0:
             continue                                            #warm-up
         stamps = prof.sequence.get_timestamps()
         durs   = np.diff(stamps)[1:1 + len(prof.launches)]      #[uploads | launches ... | downloads]
+        per_launch += durs
         for launch, ms in zip(prof.launches, durs):
             f = fam.setdefault(kernel_family(launch.kernel), dict(launches=0, ms=0.0, flops=0, bytes=0))
             f['launches'] += 1; f['ms'] += float(ms); f['flops'] += launch.flops; f['bytes'] += launch.bytes_moved
+    if args.dump_launches:
+        with open(args.dump_launches, 'w') as fh:
+            for op, launch, ms in zip(prof.all_ops, prof.launches, per_launch / max(args.profile_iters, 1)):
+                rate = f'{launch.flops / ms / 1e9:7.1f} TFLOP/s' if launch.flops else f'{launch.bytes_moved / ms / 1e6:7.0f} GB/s'
+                fh.write(f'{launch.kernel:28s} grid {launch.grid[0]:6d} {launch.flops / 1e9:8.3f} GFLOP {launch.bytes_moved / 1e6:8.1f} MB '
+                         f'{ms * 1e3:8.1f} us {rate}  {op.equation!r:.60s}\n')
     kernels = {}
     for name, f in fam.items():
         n = args.profile_iters

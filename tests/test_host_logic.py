@@ -60,25 +60,20 @@ def test_code_objects_are_built_for_gfx950():
 def test_kernel_argument_layouts_match_the_structs():
     '''sizeof of every kernel parameter struct, taken from the compiler, equals the length of
     the block the host packs.'''
-    src = r'''
-#include <cstdio>
-#include "elementwise.hip"
-#define EW_OP(a,b)
-#include "conv_gemm.hip"
-#include "reduce.hip"
-#include "index.hip"
-#include "threefry.hip"
-#define P(T) printf(#T " %zu\n", sizeof(T));
-int main(){ P(EwParams) P(IotaParams) P(FillParams) P(ConcatParams) P(ConvParams) P(ConvEpiPtrs) P(Reduce3dParams)
- P(ReduceGeneralParams) P(PoolParams) P(GatherRowsParams) P(GatherGeneralParams) P(ScatterRowsParams) P(ScatterGeneralParams) P(ThreefryParams) }
-'''
+    #the parameter structs and the #defines they use are lifted out of the kernel sources and
+    #compiled on their own with the host compiler
+    kdir  = os.path.join(ROOT, 'vkjax_amd', 'csrc', 'kernels')
+    text  = ''.join(open(os.path.join(kdir, f)).read() for f in sorted(os.listdir(kdir)) if f.endswith('.hip'))
+    defs  = re.findall(r'^#define\s+(?:EW_MAX_STEPS|CONV_MAX_EPI|IDX_MAX_RANK)\s+\d+\s*$', text, re.M)
+    decls = re.findall(r'^struct\s+\w+\s*\{[^}]*\};', text, re.M)
+    names = [re.match(r'struct\s+(\w+)', d).group(1) for d in decls]
+    src   = '#include <cstdio>\n#include <cstdint>\n' + '\n'.join(defs) + '\n' + '\n'.join(decls) + '\nint main(){\n' \
+          + ''.join(f'  printf("{n} %zu\\n", sizeof({n}));\n' for n in names) + '}\n'
     import tempfile
-    kdir = os.path.join(ROOT, 'vkjax_amd', 'csrc', 'kernels')
     with tempfile.TemporaryDirectory() as tmp:
         open(os.path.join(tmp, 'sz.cpp'), 'w').write(src)
         exe = os.path.join(tmp, 'sz')
-        subprocess.run(['/opt/rocm/bin/hipcc', '-x', 'hip', '--offload-arch=gfx950', '-O0', '-w', f'-I{kdir}',
-                        os.path.join(tmp, 'sz.cpp'), '-o', exe], check=True, capture_output=True)
+        subprocess.run(['g++', '-O0', '-w', os.path.join(tmp, 'sz.cpp'), '-o', exe], check=True, capture_output=True)
         sizes = dict(line.split() for line in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.splitlines())
     sizes = {k: int(v) for k, v in sizes.items()}
     f32 = np.dtype('float32')
@@ -188,7 +183,7 @@ def test_bufferpool_highlevel_reuse():
 def test_views_share_storage_and_32bit_canonicalisation():
     closed = mj.make_jaxpr(lambda x: lax.bitcast_convert_type((x + 1).reshape(2, 8), np.uint32))(np.zeros(16, np.float32))
     interp = JaxprInterpreter(closed, fuse=False, plan_only=True)
-    assert [l.kernel for l in interp.launches] == ['ew_chain_v4']      #reshape and bitcast are free
+    assert [l.kernel for l in interp.launches] == ['ew_chain_v4_s2']      #reshape and bitcast are free
     words = to_device_words(np.array([True, False, True]))
     assert words.dtype == np.uint32 and words.tolist() == [1, 0, 1]
     assert view_or_convert_from_32bit(words, np.bool_).tolist() == [True, False, True]
@@ -234,7 +229,7 @@ def test_dropped_outputs_are_skipped_and_calls_are_inlined():
     assert len(out) == 1 and out[0].equation is kept
     closed = mj.make_jaxpr(lambda a, b: mj.jit(lambda u: u + u)(a) + mj.jit(lambda u, v: u + v)(b, 1.0))(5.0, 7.1)
     interp = JaxprInterpreter(closed, fuse=False, plan_only=True)
-    assert [l.kernel for l in interp.launches] == ['ew_chain_v1'] * 3
+    assert [l.kernel for l in interp.launches] == ['ew_chain_v1_s2'] * 3
 
 
 def test_opcode_table_and_tile_choice():

@@ -25,9 +25,12 @@ struct EwParams {
     uint32_t dims[4];                  // row-major, dims[ndim-1] fastest; unused = 1
     uint32_t nsteps;                   // 1..8; step 0 is the initial load
     uint32_t op[EW_MAX_STEPS];         // opcode of step k (op[0] ignored)
-    uint32_t flags[EW_MAX_STEPS];      // bit0: step has an operand; bit1: operand is the LEFT argument
+    uint32_t flags[EW_MAX_STEPS];      // bit0: step has an operand; bit1: operand is the LEFT argument;
+                                       // bit2: the operand's fastest stride is 1 (else 0: one value per vector)
     uint32_t imm[EW_MAX_STEPS];        // immediate (integer_pow exponent)
     int32_t  stride[EW_MAX_STEPS][4];  // operand strides per collapsed dim, in elements
+    uint32_t nbytes[EW_MAX_STEPS];     // bytes readable from each operand pointer (0 = no operand)
+    uint32_t base[EW_MAX_STEPS];       // element offset of output element 0 in each operand
 };
 
 __device__ __forceinline__ uint32_t ipow_f(uint32_t xb, int32_t y) {
@@ -81,145 +84,180 @@ __device__ __noinline__ uint32_t ew_apply_rare(uint32_t op, uint32_t a, uint32_t
     }
 }
 
-// a = left argument, b = right argument.
-__device__ __forceinline__ uint32_t ew_apply(uint32_t op, uint32_t a, uint32_t b, uint32_t imm) {
-    const float x = u2f(a), y = u2f(b);
-    const int32_t p = (int32_t)a, q = (int32_t)b;
+// acc[j] = op(acc[j], v[j]) (or op(v[j], acc[j]) when `left`). The opcode is uniform: one branch
+// per step, with the loop over the lanes' VEC elements inside each case.
+template <int VEC>
+__device__ __forceinline__ void ew_apply_vec(uint32_t op, uint32_t (&acc)[VEC], const uint32_t (&v)[VEC], bool left, uint32_t imm) {
+#define EW_CASE(code, expr)                                                        \
+    case code:                                                                     \
+        _Pragma("unroll") for (int j = 0; j < VEC; ++j) {                          \
+            const uint32_t a = left ? v[j] : acc[j], b = left ? acc[j] : v[j];     \
+            const float x = u2f(a), y = u2f(b);                                    \
+            const int32_t p = (int32_t)a, q = (int32_t)b;                          \
+            (void)x; (void)y; (void)p; (void)q;                                    \
+            acc[j] = (expr);                                                       \
+        }                                                                          \
+        break;
     switch (op) {
-        case EW_NOP:     return a;
-        case EW_ADD_F:   return f2u(x + y);
-        case EW_SUB_F:   return f2u(x - y);
-        case EW_MUL_F:   return f2u(x * y);
-        case EW_DIV_F:   return f2u(x / y);
-        case EW_MAX_F:   return (x > y || x != x) ? a : b;      // NaN wins, as in XLA
-        case EW_MIN_F:   return (x < y || x != x) ? a : b;
-        case EW_ADD_I:   return a + b;
-        case EW_SUB_I:   return a - b;
-        case EW_MUL_I:   return a * b;
-        case EW_MAX_I:   return p > q ? a : b;
-        case EW_MIN_I:   return p < q ? a : b;
-        case EW_MAX_U:   return a > b ? a : b;
-        case EW_MIN_U:   return a < b ? a : b;
-        case EW_AND_X:   return a & b;
-        case EW_OR_X:    return a | b;
-        case EW_XOR_X:   return a ^ b;
-        case EW_SHL_X:   return b >= 32 ? 0u : a << b;
-        case EW_SHR_L:   return b >= 32 ? 0u : a >> b;
-        case EW_SHR_A:   return (uint32_t)(p >> (b >= 32 ? 31u : b));
-        case EW_GT_F:    return x >  y;
-        case EW_GE_F:    return x >= y;
-        case EW_LT_F:    return x <  y;
-        case EW_LE_F:    return x <= y;
-        case EW_EQ_F:    return x == y;
-        case EW_NE_F:    return x != y;
-        case EW_GT_I:    return p >  q;
-        case EW_GE_I:    return p >= q;
-        case EW_LT_I:    return p <  q;
-        case EW_LE_I:    return p <= q;
-        case EW_EQ_X:    return a == b;
-        case EW_NE_X:    return a != b;
-        case EW_GT_U:    return a >  b;
-        case EW_GE_U:    return a >= b;
-        case EW_LT_U:    return a <  b;
-        case EW_LE_U:    return a <= b;
-        case EW_NEG_F:   return a ^ 0x80000000u;
-        case EW_ABS_F:   return a & 0x7FFFFFFFu;
-        case EW_SIGN_F:  return x > 0.f ? f2u(1.0f) : x < 0.f ? f2u(-1.0f) : a;
-        case EW_NEG_I:   return 0u - a;
-        case EW_ABS_I:   return p < 0 ? 0u - a : a;
-        case EW_SIGN_I:  return (uint32_t)((p > 0) - (p < 0));
-        case EW_EXP_F:   return f2u(expf(x));
-        case EW_RSQRT_F: return f2u(1.0f / sqrtf(x));
-        case EW_CVT_F2I: return (uint32_t)(int32_t)x;           // truncates, saturates, NaN -> 0
-        case EW_CVT_F2U: return (uint32_t)x;
-        case EW_CVT_I2F: return f2u((float)p);
-        case EW_CVT_U2F: return f2u((float)a);
-        case EW_CVT_F2B: return x != 0.f;
-        case EW_CVT_X2B: return a != 0u;
-        default:         return ew_apply_rare(op, a, b, imm);
+        EW_CASE(EW_NOP,     a)
+        EW_CASE(EW_ADD_F,   f2u(x + y))
+        EW_CASE(EW_SUB_F,   f2u(x - y))
+        EW_CASE(EW_MUL_F,   f2u(x * y))
+        EW_CASE(EW_DIV_F,   f2u(x / y))
+        EW_CASE(EW_MAX_F,   (x > y || x != x) ? a : b)      // NaN wins, as in XLA
+        EW_CASE(EW_MIN_F,   (x < y || x != x) ? a : b)
+        EW_CASE(EW_ADD_I,   a + b)
+        EW_CASE(EW_SUB_I,   a - b)
+        EW_CASE(EW_MUL_I,   a * b)
+        EW_CASE(EW_MAX_I,   p > q ? a : b)
+        EW_CASE(EW_MIN_I,   p < q ? a : b)
+        EW_CASE(EW_MAX_U,   a > b ? a : b)
+        EW_CASE(EW_MIN_U,   a < b ? a : b)
+        EW_CASE(EW_AND_X,   a & b)
+        EW_CASE(EW_OR_X,    a | b)
+        EW_CASE(EW_XOR_X,   a ^ b)
+        EW_CASE(EW_SHL_X,   b >= 32 ? 0u : a << b)
+        EW_CASE(EW_SHR_L,   b >= 32 ? 0u : a >> b)
+        EW_CASE(EW_SHR_A,   (uint32_t)(p >> (b >= 32 ? 31u : b)))
+        EW_CASE(EW_GT_F,    x >  y)
+        EW_CASE(EW_GE_F,    x >= y)
+        EW_CASE(EW_LT_F,    x <  y)
+        EW_CASE(EW_LE_F,    x <= y)
+        EW_CASE(EW_EQ_F,    x == y)
+        EW_CASE(EW_NE_F,    x != y)
+        EW_CASE(EW_GT_I,    p >  q)
+        EW_CASE(EW_GE_I,    p >= q)
+        EW_CASE(EW_LT_I,    p <  q)
+        EW_CASE(EW_LE_I,    p <= q)
+        EW_CASE(EW_EQ_X,    a == b)
+        EW_CASE(EW_NE_X,    a != b)
+        EW_CASE(EW_GT_U,    a >  b)
+        EW_CASE(EW_GE_U,    a >= b)
+        EW_CASE(EW_LT_U,    a <  b)
+        EW_CASE(EW_LE_U,    a <= b)
+        EW_CASE(EW_NEG_F,   a ^ 0x80000000u)
+        EW_CASE(EW_ABS_F,   a & 0x7FFFFFFFu)
+        EW_CASE(EW_SIGN_F,  x > 0.f ? f2u(1.0f) : x < 0.f ? f2u(-1.0f) : a)
+        EW_CASE(EW_NEG_I,   0u - a)
+        EW_CASE(EW_ABS_I,   p < 0 ? 0u - a : a)
+        EW_CASE(EW_SIGN_I,  (uint32_t)((p > 0) - (p < 0)))
+        EW_CASE(EW_EXP_F,   f2u(expf(x)))
+        EW_CASE(EW_RSQRT_F, f2u(1.0f / sqrtf(x)))
+        EW_CASE(EW_CVT_F2I, (uint32_t)(int32_t)x)           // truncates, saturates, NaN -> 0
+        EW_CASE(EW_CVT_F2U, (uint32_t)x)
+        EW_CASE(EW_CVT_I2F, f2u((float)p))
+        EW_CASE(EW_CVT_U2F, f2u((float)a))
+        EW_CASE(EW_CVT_F2B, x != 0.f)
+        EW_CASE(EW_CVT_X2B, a != 0u)
+        default:
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                acc[j] = ew_apply_rare(op, left ? v[j] : acc[j], left ? acc[j] : v[j], imm);
+            break;
     }
+#undef EW_CASE
 }
 
-template <int VEC> struct EwVec;
-template <> struct EwVec<1> { uint32_t v[1]; };
-template <> struct EwVec<4> { uint32_t v[4]; };
+// Keeps a kernel argument in a scalar register from this point on. Used on every argument at
+// the top of the kernel so that the scalar loads of the argument block are issued together and
+// waited for once, instead of one round trip per operand slot further down. The 8-slot
+// instantiation would run out of scalar registers and leaves its arguments to be fetched on demand.
+#define EW_PIN(x) do { if constexpr (NS <= 6) asm volatile("" : "+s"(x)); } while (0)
 
-template <int VEC>
-__device__ __forceinline__ void ew_load(uint32_t (&dst)[VEC], const uint32_t* __restrict__ p, int64_t idx, int32_t last_stride) {
-    if constexpr (VEC == 4) {
-        if (last_stride == 1) {
-            const u32x4 t = *reinterpret_cast<const u32x4*>(p + idx);
-            dst[0] = t.x; dst[1] = t.y; dst[2] = t.z; dst[3] = t.w;
-        } else {                                   // stride 0 along the vector: one value, splat
-            const uint32_t t = p[idx];
-            dst[0] = dst[1] = dst[2] = dst[3] = t;
-        }
-    } else {
-        dst[0] = p[idx];
-    }
-}
-
-template <int VEC>
+// NS = number of step slots this instantiation looks at (the chain has at most NS steps).
+template <int VEC, int NS>
 __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const uint32_t* const (&in)[EW_MAX_STEPS],
                                               const EwParams& P) {
-    const uint32_t v = blockIdx.x * 256u + threadIdx.x;
-    const uint64_t i0 = (uint64_t)v * VEC;
-    if (i0 >= P.n) return;
+    uint32_t n = P.n, ndim = P.ndim, nsteps = P.nsteps;
+    uint32_t dims[4], op[NS], flags[NS], imm[NS], nbytes[NS], base[NS];
+    int32_t  stride[NS][4];
+    EW_PIN(n); EW_PIN(ndim); EW_PIN(nsteps);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) { dims[d] = P.dims[d]; EW_PIN(dims[d]); }
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+        flags[k] = P.flags[k]; nbytes[k] = P.nbytes[k]; base[k] = P.base[k];
+        EW_PIN(flags[k]); EW_PIN(nbytes[k]); EW_PIN(base[k]);
+        if constexpr (NS <= 6) asm volatile("" :: "s"(in[k]));
+#pragma unroll
+        for (int d = 0; d < 4; ++d) { stride[k][d] = P.stride[k][d]; EW_PIN(stride[k][d]); }
+    }
+
+    const uint32_t v  = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t i0 = v * VEC;                   // the host keeps n below 2^31
+    if (i0 >= n) return;
 
     // coordinates of the first element of this vector in the collapsed output space
     uint32_t c[4] = {0, 0, 0, 0};
     {
-        uint32_t r = (uint32_t)i0;
-        if (P.ndim > 1) {
+        uint32_t r = i0;
+        if (ndim > 1) {
 #pragma unroll
             for (int d = 3; d >= 1; --d) {
-                if (d < (int)P.ndim) { const uint32_t q = r / P.dims[d]; c[d] = r - q * P.dims[d]; r = q; }
+                if (d < (int)ndim) { const uint32_t q = r / dims[d]; c[d] = r - q * dims[d]; r = q; }
             }
         }
         c[0] = r;
     }
-    const int last = (int)P.ndim - 1;
-
-    uint32_t vals[EW_MAX_STEPS][VEC];
+    // Every operand is read through a buffer descriptor with one branch-free load per slot: 16 bytes
+    // (of which only the first dword is used where the operand is constant along the vector), or
+    // nothing at all for an empty slot, whose descriptor has size 0. All loads are in flight
+    // together; they are consumed after a single wait.
+    uint32_t vals[NS][VEC];
+    if constexpr (VEC == 4) {
+        u32x4 vec[NS];
 #pragma unroll
-    for (int k = 0; k < EW_MAX_STEPS; ++k) {
-        if (k < (int)P.nsteps && (P.flags[k] & 1u)) {
-            int64_t idx = 0;
+        for (int k = 0; k < NS; ++k) {
+            uint32_t idx = base[k] + c[0] * (uint32_t)stride[k][0];   // wraps correctly for negative strides
+            if (ndim > 1) {
 #pragma unroll
-            for (int d = 0; d < 4; ++d) idx += (int64_t)c[d] * P.stride[k][d];
-            ew_load<VEC>(vals[k], in[k], idx, P.stride[k][last]);
-        } else {
+                for (int d = 1; d < 4; ++d) idx += c[d] * (uint32_t)stride[k][d];
+            }
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, (int)nbytes[k], 0x00020000);
+            vec[k] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 4u, 0, 0);
+        }
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) vals[k][j] = 0;
+        for (int k = 0; k < NS; ++k) {
+            const bool is_vec = (flags[k] & 4u) != 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) vals[k][j] = is_vec ? vec[k][j] : vec[k][0];
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < NS; ++k) {
+            uint32_t idx = base[k] + c[0] * (uint32_t)stride[k][0];
+            if (ndim > 1) {
+#pragma unroll
+                for (int d = 1; d < 4; ++d) idx += c[d] * (uint32_t)stride[k][d];
+            }
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, (int)nbytes[k], 0x00020000);
+            vals[k][0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, idx * 4u, 0, 0);
         }
     }
+
+    // opcodes and immediates are fetched while the operand loads are in flight
+#pragma unroll
+    for (int k = 0; k < NS; ++k) { op[k] = P.op[k]; imm[k] = P.imm[k]; EW_PIN(op[k]); EW_PIN(imm[k]); }
 
     uint32_t acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = vals[0][j];
 
 #pragma unroll
-    for (int k = 1; k < EW_MAX_STEPS; ++k) {
-        if (k < (int)P.nsteps) {
-            const uint32_t op = P.op[k], imm = P.imm[k];
-            if (op >= EW_SEL_P && op <= EW_SEL_F) {
+    for (int k = 1; k < NS; ++k) {
+        if (k < (int)nsteps) {
+            if (op[k] >= EW_SEL_P && op[k] <= EW_SEL_F) {
                 // three-input select: this step's operand and the next step's operand (a NOP carrier)
-                const int k2 = (k + 1 < EW_MAX_STEPS) ? k + 1 : k;
+                const int k2 = (k + 1 < NS) ? k + 1 : k;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
                     const uint32_t s = vals[k][j], t = vals[k2][j];
-                    acc[j] = op == EW_SEL_P ? (acc[j] ? s : t)       // acc is the predicate
-                           : op == EW_SEL_T ? (s ? acc[j] : t)       // acc is on_true, s the predicate
-                                            : (s ? t : acc[j]);      // acc is on_false, s the predicate
+                    acc[j] = op[k] == EW_SEL_P ? (acc[j] ? s : t)       // acc is the predicate
+                           : op[k] == EW_SEL_T ? (s ? acc[j] : t)       // acc is on_true, s the predicate
+                                               : (s ? t : acc[j]);      // acc is on_false, s the predicate
                 }
             } else {
-                const bool operand_left = (P.flags[k] & 2u) != 0;
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    const uint32_t a = operand_left ? vals[k][j] : acc[j];
-                    const uint32_t b = operand_left ? acc[j] : vals[k][j];
-                    acc[j] = ew_apply(op, a, b, imm);
-                }
+                ew_apply_vec<VEC>(op[k], acc, vals[k], (flags[k] & 2u) != 0, imm[k]);
             }
         }
     }
@@ -232,19 +270,26 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     }
 }
 
-#define EW_KERNEL(name, VEC)                                                                          \
+#define EW_KERNEL(name, VEC, NS)                                                                      \
     extern "C" __global__ __launch_bounds__(256) void name(                                            \
         uint32_t* __restrict__ out, const uint32_t* in0, const uint32_t* in1, const uint32_t* in2,      \
         const uint32_t* in3, const uint32_t* in4, const uint32_t* in5, const uint32_t* in6,             \
         const uint32_t* in7, EwParams P) {                                                              \
         const uint32_t* const in[EW_MAX_STEPS] = {in0, in1, in2, in3, in4, in5, in6, in7};              \
-        ew_chain_body<VEC>(out, in, P);                                                                 \
+        ew_chain_body<VEC, NS>(out, in, P);                                                             \
     }
 
-// ew_chain_v4 requires: n % 4 == 0, dims[ndim-1] % 4 == 0, every operand's fastest stride in {0, 1},
+// ew_chain_v4* requires: n % 4 == 0, dims[ndim-1] % 4 == 0, every operand's fastest stride in {0, 1},
 // stride-1 operands 16-byte aligned with all slower strides % 4 == 0. The host checks this.
-EW_KERNEL(ew_chain_v1, 1)
-EW_KERNEL(ew_chain_v4, 4)
+// The _sN suffix is the number of step slots the kernel handles (chains of up to N steps).
+EW_KERNEL(ew_chain_v1_s2, 1, 2)
+EW_KERNEL(ew_chain_v1_s4, 1, 4)
+EW_KERNEL(ew_chain_v1_s6, 1, 6)
+EW_KERNEL(ew_chain_v1_s8, 1, 8)
+EW_KERNEL(ew_chain_v4_s2, 4, 2)
+EW_KERNEL(ew_chain_v4_s4, 4, 4)
+EW_KERNEL(ew_chain_v4_s6, 4, 6)
+EW_KERNEL(ew_chain_v4_s8, 4, 8)
 
 struct IotaParams { uint32_t n, inner, size, to_float; };
 

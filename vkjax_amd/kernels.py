@@ -147,28 +147,39 @@ def lower_ew_chain(chain: EwChain) -> Launch:
             vec = 1
         elif st[-1] == 1 and (o.offset % 4 or any(s % 4 for s in st[:-1])):
             vec = 1
-    ops, flags, imms, stride_rows, buffers = [0], [1], [0], [], []
+    ops, flags, imms, stride_rows, buffers, extents, bases = [], [], [], [], [], [], []
     it = iter(strides)
     for k, o in enumerate(operands):
-        if k > 0:
-            step = chain.steps[k - 1]
-            ops.append(step.op)
-            flags.append((1 if o is not None else 0) | (2 if step.operand_left else 0))
-            imms.append(step.imm)
+        step = chain.steps[k - 1] if k > 0 else None
+        ops.append(step.op if step else 0)
+        imms.append(step.imm if step else 0)
+        flag = 2 if (step and step.operand_left) else 0
         if o is None:
             stride_rows.append([0, 0, 0, 0])
             buffers.append((None, 0))
+            extents.append(0)
+            bases.append(0)
         else:
-            stride_rows.append(_pad(next(it), 4))
-            buffers.append((o.buffer, o.offset * 4))
+            st = next(it)
+            if o.buffer.size * 4 >= 2**32:
+                raise NotImplementedError('element-wise operand of 4 GiB or more')
+            extents.append(o.buffer.size * 4)
+            bases.append(o.offset)
+            flag |= 1 | (4 if st[-1] == 1 else 0)
+            stride_rows.append(_pad(st, 4))
+            buffers.append((o.buffer, 0))
+        flags.append(flag)
     while len(stride_rows) < EW_MAX_STEPS:
         stride_rows.append([0, 0, 0, 0])
         buffers.append((None, 0))
     params = (_u32(n, ndim, *_pad(dims, 4, 1), nsteps, *_pad(ops, EW_MAX_STEPS), *_pad(flags, EW_MAX_STEPS),
                    *_pad(imms, EW_MAX_STEPS))
-              + _i32(*[s for row in stride_rows for s in row]))
+              + _i32(*[s for row in stride_rows for s in row]) + _u32(*_pad(extents, EW_MAX_STEPS), *_pad(bases, EW_MAX_STEPS)))
     nbytes = 4 * n + sum(4 * min(n, o.buffer.size) for o in present)
-    return Launch(f'ew_chain_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+    if n >= 2**31:
+        raise NotImplementedError(f'element-wise op over {n} elements exceeds 32-bit indexing')
+    slots = 2 if nsteps <= 2 else 4 if nsteps <= 4 else 6 if nsteps <= 6 else 8
+    return Launch(f'ew_chain_v{vec}_s{slots}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                   [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
 
 
