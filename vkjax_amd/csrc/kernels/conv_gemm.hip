@@ -72,13 +72,29 @@ __device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t 
 template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST>
 __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
                                                const float* __restrict__ w, const ConvEpiPtrs& epi,
-                                               const ConvParams& P) {
+                                               const ConvParams& Pk) {
     constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, NT = 64 * WGM * WGN;
     constexpr int LDA = BK + 4, LDB = BN + 4;
     __shared__ __attribute__((aligned(16))) float As[BM * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
     __shared__ float Es[CONV_MAX_EPI * BN];         // per-column operands of the epilogue steps
 
+    // Copy the argument block into scalar registers once, at the very start. Left to itself the
+    // compiler fetches each field right before its first use; under load every such fetch costs
+    // about a microsecond, and the prologue and the epilogue would each chain several of them.
+    ConvParams P;
+#define CONV_PIN(f) P.f = Pk.f; asm volatile("" : "+s"(P.f));
+    CONV_PIN(M) CONV_PIN(N) CONV_PIN(K) CONV_PIN(Ho) CONV_PIN(Wo) CONV_PIN(H) CONV_PIN(W) CONV_PIN(Cin)
+    CONV_PIN(KH) CONV_PIN(KW) CONV_PIN(SH) CONV_PIN(SW) CONV_PIN(PH) CONV_PIN(PW) CONV_PIN(DH) CONV_PIN(DW)
+    CONV_PIN(LH) CONV_PIN(LW) CONV_PIN(xs_b) CONV_PIN(xs_h) CONV_PIN(xs_w) CONV_PIN(xs_c) CONV_PIN(ws_r) CONV_PIN(ws_s)
+    CONV_PIN(ws_c) CONV_PIN(ws_n) CONV_PIN(os_b) CONV_PIN(os_h) CONV_PIN(os_w) CONV_PIN(os_n) CONV_PIN(c_contig) CONV_PIN(tiles_m)
+    CONV_PIN(tiles_n) CONV_PIN(nepi) CONV_PIN(epi_first_full) CONV_PIN(flat_rows) CONV_PIN(x_bytes) CONV_PIN(w_bytes) CONV_PIN(out_bytes)
+#pragma unroll
+    for (int q = 0; q < CONV_MAX_EPI; ++q) {
+        CONV_PIN(epi_op[q]) CONV_PIN(epi_flags[q]) CONV_PIN(epi_kind[q])
+        asm volatile("" :: "s"(epi.p[q]));
+    }
+#undef CONV_PIN
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
     const int l32 = lane & 31, half = lane >> 5;
@@ -331,7 +347,9 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
                 for (int v = 0; v < 16; ++v)
                     full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, elem_offset(i, j, v));
     }
-    for (int e = 0; e < (int)P.nepi; ++e) {              // uniform, not unrolled
+#pragma unroll
+    for (int e = 0; e < CONV_MAX_EPI; ++e) {             // unrolled: the step descriptors stay in scalar registers
+        if (e >= (int)P.nepi) break;
         const uint32_t kind = P.epi_kind[e];
         const uint32_t code = P.epi_op[e] * 2u + ((P.epi_flags[e] >> 1) & 1u);   // bit0: operand on the left
 #pragma unroll
