@@ -124,9 +124,17 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         e_reg[q] = 0.f;
         if (idx < (int)P.nepi * BN) {
             const int e = idx / BN, n = n0 + idx - e * BN;
-            const uint32_t kind = P.epi_kind[e];
-            if (kind == 1) e_reg[q] = epi.p[e][0];
-            else if (kind == 2 && n < P.N) e_reg[q] = epi.p[e][n];
+            // pick step e's descriptor with selects: indexing the argument block with a run-time
+            // value would move the whole block from scalar registers to scratch memory
+            uint32_t kind = P.epi_kind[0];
+            const float* src = epi.p[0];
+#pragma unroll
+            for (int t = 1; t < CONV_MAX_EPI; ++t) {
+                kind = e == t ? P.epi_kind[t] : kind;
+                src  = e == t ? epi.p[t] : src;
+            }
+            if (kind == 1) e_reg[q] = src[0];
+            else if (kind == 2 && n < P.N) e_reg[q] = src[n];
         }
     }
 
@@ -320,17 +328,26 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     // accumulator element v of a lane: row = 8*(v/4) + 4*half + v%4, column = l32.
     // Byte offsets fit 31 bits: the host refuses larger tensors.
     const bool whole_tile = m0 + BM <= P.M && n0 + BN <= P.N;
+    // Outputs that are not a row-major [M, N] matrix need (batch, y, x) of every row: decoded once
+    // per row into the LDS space of the A tile (free after the k loop), -1 for rows beyond M.
+    int* const row_off = reinterpret_cast<int*>(As);
+    if (!P.c_contig) {
+        for (int r = tid; r < BM; r += NT) {
+            const int m = m0 + r;
+            const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
+            row_off[r] = m < P.M ? b * P.os_b + ho * P.os_h + wo * P.os_w : -1;
+        }
+        __syncthreads();
+    }
     auto elem_offset = [&](int i, int j, int v) -> uint32_t {
         const int n = n0 + (wn * TN + j) * 32 + l32;
-        const int m = m0 + (wm * TM + i) * 32 + 4 * half + 8 * (v / 4) + (v % 4);
-        int off;
+        const int r = (wm * TM + i) * 32 + 4 * half + 8 * (v / 4) + (v % 4);
         if (P.c_contig) {
-            off = m * P.N + n;
-        } else {
-            const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
-            off = b * P.os_b + ho * P.os_h + wo * P.os_w + n * P.os_n;
+            const int m = m0 + r;
+            return (whole_tile || (m < P.M && n < P.N)) ? (uint32_t)(m * P.N + n) * 4u : CONV_OOB;
         }
-        return (whole_tile || (m < P.M && n < P.N)) ? (uint32_t)off * 4u : CONV_OOB;
+        const int ro = row_off[r];
+        return (ro >= 0 && n < P.N) ? (uint32_t)(ro + n * P.os_n) * 4u : CONV_OOB;
     };
     // the first full-size operand (a residual input) is fetched for the whole tile at once
     // (for the largest tile that would not fit the register file: it loads sub-tile by sub-tile)
@@ -338,7 +355,10 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
     const int first_full = PREFETCH_FULL ? P.epi_first_full : -1;
     if (PREFETCH_FULL && first_full >= 0) {
-        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(epi.p[first_full], P.out_bytes);
+        const float* fp = epi.p[0];
+#pragma unroll
+        for (int t = 1; t < CONV_MAX_EPI; ++t) fp = first_full == t ? epi.p[t] : fp;
+        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(fp, P.out_bytes);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
