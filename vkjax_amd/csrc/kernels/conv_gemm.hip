@@ -19,10 +19,18 @@
 // conflicts; B: [BK][BN+4]); the next tiles are prefetched into registers while the MFMAs of
 // the current one run. The sum over k is order-free, so lanes 0-31 take the first half of a k
 // tile and lanes 32-63 the second half, which is what makes the 16-byte A reads possible.
-// The 16-byte paths read through buffer descriptors: a masked-out load is an out-of-range
-// offset that returns zeros, so padding, tile tails and partial tiles need no branches.
 // After the k loop an optional chain of element-wise steps (per-feature vectors, full-size
 // tensors or scalars as operands) is applied to the accumulators before the single store.
+//
+// The fp32 MFMA executes on the same lanes as ordinary vector instructions: measured, a wave's
+// vector instruction issues only once per 64-cycle MFMA of another wave on the same SIMD. Every
+// vector instruction therefore costs MFMA throughput, and the 16-byte paths are written to need
+// almost none: addresses are split into a per-thread part that is computed once per block and a
+// per-k-tile part that is wave-uniform and travels in the scalar offset operand of the buffer
+// instruction; taps that fall into the padding are looked up in a per-row bit mask built once;
+// rows and columns outside the matrices are caught by the range check of the buffer descriptor
+// (an out-of-range load returns zeros, an out-of-range store is dropped); row decoding uses
+// multiply-high division by constants prepared on the host.
 #include "common.h"
 
 #define CONV_MAX_EPI 6
@@ -34,24 +42,33 @@ enum EwOpConv : uint32_t {
 #undef EW_OP
 };
 
+// Argument block. The fields up to wo_shift are used by every variant and are fetched into
+// scalar registers in one batch when a block starts; the rest is only read by the generic
+// (strided) paths, where it is needed.
 struct ConvParams {
     int32_t M, N, K;
     int32_t Ho, Wo;                 // M = batch * Ho * Wo
     int32_t H, W, Cin;              // lhs spatial size (undilated) and features
     int32_t KH, KW;
-    int32_t SH, SW, PH, PW, DH, DW, LH, LW;
-    int32_t xs_b, xs_h, xs_w, xs_c; // lhs strides in elements
+    int32_t SH, SW, PH, PW, DH, DW;
+    int32_t xs_b, xs_h, xs_w;       // lhs strides in elements
+    int32_t tiles_m, tiles_n;
+    uint32_t flags;                 // bit0: out is row-major [M, N]; bit1: m is the row index itself
+                                    // (batch = Wo = 1: no row decode); bit2: some kernel taps of some
+                                    // rows fall outside the input; bits 8-11: number of epilogue
+                                    // steps; bits 16-19: 1 + index of the first kind-3 step, or 0;
+                                    // bits 20-24: the steps are, in this order, a subset of
+                                    // (acc - vector, * vector, + vector, + full tensor, max(acc, scalar)):
+                                    // bit 20+k set = template step k is present
+    uint32_t epi_desc[2];           // 10 bits per step, steps 0-2 in [0], 3-5 in [1]: bits 0-7 opcode * 2 +
+                                    // (operand is the left argument), bits 8-9 kind: 1 scalar,
+                                    // 2 per-feature vector [N], 3 full tensor laid out like out
+    uint32_t x_bytes, w_bytes, out_bytes;   // sizes for the buffer descriptors (each below 2^31)
+    uint32_t howo_magic, howo_shift;        // n / (Ho*Wo) = mulhi(n, magic) >> shift for 0 <= n < 2^31
+    uint32_t wo_magic, wo_shift;            // same for Wo; magic 0 stands for a divisor of 1
+    int32_t LH, LW, xs_c;           // lhs dilation and feature stride
     int32_t ws_r, ws_s, ws_c, ws_n; // rhs strides
     int32_t os_b, os_h, os_w, os_n; // out strides
-    int32_t c_contig;               // out is row-major [M, N]
-    int32_t tiles_m, tiles_n;
-    uint32_t nepi;                  // number of epilogue steps
-    uint32_t epi_op[CONV_MAX_EPI];
-    uint32_t epi_flags[CONV_MAX_EPI];   // bit1: operand is the left argument
-    uint32_t epi_kind[CONV_MAX_EPI];    // 0 none, 1 scalar, 2 per-feature vector [N], 3 full tensor laid out like out
-    int32_t  epi_first_full;            // index of the first kind-3 step, or -1
-    int32_t  flat_rows;                 // m is the row index itself (batch = Wo = 1): no row decode
-    uint32_t x_bytes, w_bytes, out_bytes;   // sizes for the buffer descriptors (each below 2^31)
 };
 
 struct ConvEpiPtrs { const float* p[CONV_MAX_EPI]; };
@@ -59,15 +76,27 @@ struct ConvEpiPtrs { const float* p[CONV_MAX_EPI]; };
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
-__device__ __forceinline__ f32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
-    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0));
+// voff: per-lane byte offset, soff: wave-uniform byte offset; the range check covers their sum
+__device__ __forceinline__ f32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
-__device__ __forceinline__ float buffer_load_x1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+__device__ __forceinline__ float buffer_load_x1(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
 }
-__device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, byte_off, 0, 0);
+__device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, voff, soff, 0);
 }
+__device__ __forceinline__ int magic_div(int n, uint32_t magic, uint32_t shift) {
+    return magic ? (int)(__umulhi((uint32_t)n, magic) >> shift) : n;
+}
+
+// Optional per-block phase time stamps (profiling builds only): slot s of block b lands in
+// ((uint64*)epi.p[CONV_MAX_EPI - 1])[16 * b + s].
+#ifdef CONV_PHASE_STAMPS
+#define CONV_STAMP(slot) stamps[slot] = wall_clock64();
+#else
+#define CONV_STAMP(slot)
+#endif
 
 template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST>
 __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
@@ -78,23 +107,32 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     __shared__ __attribute__((aligned(16))) float As[BM * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
     __shared__ float Es[CONV_MAX_EPI * BN];         // per-column operands of the epilogue steps
+#ifdef CONV_PHASE_STAMPS
+    unsigned long long stamps[16] = {};
+#endif
+    CONV_STAMP(0)
 
-    // Copy the argument block into scalar registers once, at the very start. Left to itself the
-    // compiler fetches each field right before its first use; under load every such fetch costs
-    // about a microsecond, and the prologue and the epilogue would each chain several of them.
-    ConvParams P;
+    // Copy the hot part of the argument block into scalar registers once, at the very start. Left
+    // to itself the compiler fetches each field right before its first use; under load every such
+    // fetch costs about a microsecond, and the prologue and the epilogue would each chain several.
+    struct {
+        int32_t M, N, K, Ho, Wo, H, W, Cin, KH, KW, SH, SW, PH, PW, DH, DW, xs_b, xs_h, xs_w, tiles_m, tiles_n;
+        uint32_t flags, epi_desc[2], x_bytes, w_bytes, out_bytes, howo_magic, howo_shift, wo_magic, wo_shift;
+    } P;
 #define CONV_PIN(f) P.f = Pk.f; asm volatile("" : "+s"(P.f));
+    asm volatile("" : "+s"(out), "+s"(x), "+s"(w));
+#pragma unroll
+    for (int q = 0; q < CONV_MAX_EPI; ++q) asm volatile("" :: "s"(epi.p[q]));
     CONV_PIN(M) CONV_PIN(N) CONV_PIN(K) CONV_PIN(Ho) CONV_PIN(Wo) CONV_PIN(H) CONV_PIN(W) CONV_PIN(Cin)
     CONV_PIN(KH) CONV_PIN(KW) CONV_PIN(SH) CONV_PIN(SW) CONV_PIN(PH) CONV_PIN(PW) CONV_PIN(DH) CONV_PIN(DW)
-    CONV_PIN(LH) CONV_PIN(LW) CONV_PIN(xs_b) CONV_PIN(xs_h) CONV_PIN(xs_w) CONV_PIN(xs_c) CONV_PIN(ws_r) CONV_PIN(ws_s)
-    CONV_PIN(ws_c) CONV_PIN(ws_n) CONV_PIN(os_b) CONV_PIN(os_h) CONV_PIN(os_w) CONV_PIN(os_n) CONV_PIN(c_contig) CONV_PIN(tiles_m)
-    CONV_PIN(tiles_n) CONV_PIN(nepi) CONV_PIN(epi_first_full) CONV_PIN(flat_rows) CONV_PIN(x_bytes) CONV_PIN(w_bytes) CONV_PIN(out_bytes)
-#pragma unroll
-    for (int q = 0; q < CONV_MAX_EPI; ++q) {
-        CONV_PIN(epi_op[q]) CONV_PIN(epi_flags[q]) CONV_PIN(epi_kind[q])
-        asm volatile("" :: "s"(epi.p[q]));
-    }
+    CONV_PIN(xs_b) CONV_PIN(xs_h) CONV_PIN(xs_w) CONV_PIN(tiles_m) CONV_PIN(tiles_n) CONV_PIN(flags)
+    CONV_PIN(epi_desc[0]) CONV_PIN(epi_desc[1]) CONV_PIN(x_bytes) CONV_PIN(w_bytes) CONV_PIN(out_bytes)
+    CONV_PIN(howo_magic) CONV_PIN(howo_shift) CONV_PIN(wo_magic) CONV_PIN(wo_shift)
 #undef CONV_PIN
+    static_assert(CONV_MAX_EPI == 6, "descriptor packing");
+    auto step_desc = [&](int e) -> uint32_t { return ((e < 3 ? P.epi_desc[0] : P.epi_desc[1]) >> (10 * (e < 3 ? e : e - 3))) & 1023u; };
+    const bool c_contig = P.flags & 1u, flat_rows = P.flags & 2u, masked = P.flags & 4u;
+    const int nepi = (P.flags >> 8) & 15u, epi_first_full = (int)((P.flags >> 16) & 15u) - 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
     const int l32 = lane & 31, half = lane >> 5;
@@ -110,31 +148,24 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int HoWo = P.Ho * P.Wo;
 
-    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, P.x_bytes), w_rsrc = make_rsrc(w, P.w_bytes),
-                                 o_rsrc = make_rsrc(out, P.out_bytes);
+    // The 16-byte A path addresses the input from (PH, PW) positions before its start, so that
+    // the offset of a row's top-left tap is never negative (a negative offset is out of range
+    // for the descriptor even when a later addition brings it back).
+    const uint32_t x_bias = A_FAST ? (uint32_t)(P.PH * P.xs_h + P.PW * P.xs_w) * 4u : 0u;
+    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(reinterpret_cast<const char*>(x) - x_bias, P.x_bytes + x_bias),
+                                 w_rsrc = make_rsrc(w, P.w_bytes), o_rsrc = make_rsrc(out, P.out_bytes);
 
     // Scalar and per-feature epilogue operands are fetched once per block, at its very start, and
     // parked in LDS behind the first k tile's loads, so that the epilogue never waits on global
-    // memory for them.
-    constexpr int E_PER_THREAD = (CONV_MAX_EPI * BN + NT - 1) / NT;
-    float e_reg[E_PER_THREAD];
+    // memory for them. Thread t fetches column t of every step.
+    float e_reg[CONV_MAX_EPI];
+    if (tid < BN) {
 #pragma unroll
-    for (int q = 0; q < E_PER_THREAD; ++q) {
-        const int idx = tid + q * NT;
-        e_reg[q] = 0.f;
-        if (idx < (int)P.nepi * BN) {
-            const int e = idx / BN, n = n0 + idx - e * BN;
-            // pick step e's descriptor with selects: indexing the argument block with a run-time
-            // value would move the whole block from scalar registers to scratch memory
-            uint32_t kind = P.epi_kind[0];
-            const float* src = epi.p[0];
-#pragma unroll
-            for (int t = 1; t < CONV_MAX_EPI; ++t) {
-                kind = e == t ? P.epi_kind[t] : kind;
-                src  = e == t ? epi.p[t] : src;
-            }
-            if (kind == 1) e_reg[q] = src[0];
-            else if (kind == 2 && n < P.N) e_reg[q] = src[n];
+        for (int e = 0; e < CONV_MAX_EPI; ++e) {
+            const uint32_t kind = step_desc(e) >> 8;             // 0 beyond the last step
+            e_reg[e] = 0.f;
+            if (kind == 1) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], 4u), 0u);
+            else if (kind == 2) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], (uint32_t)P.N * 4u), (uint32_t)(n0 + tid) * 4u);
         }
     }
 
@@ -146,25 +177,44 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     constexpr int A_KG    = NT / BM;                // generic: k groups
     constexpr int A_KPT   = BK / A_KG;              // generic: k per thread
     constexpr int A_ROWS  = A_FAST ? A_NV : 1;
-    // row state: element offset of (row, ky = kx = c = 0) and the input coordinates of that corner
-    int a_off[A_ROWS], a_hi0[A_ROWS], a_wi0[A_ROWS];
+    // fast: byte offset of (row, tap 0, this thread's k vector) from the biased base, out of range for rows beyond M;
+    //       bit t of a_inv set = tap t = ky*KW + kx of that row lies outside the input
+    // generic: element offset of the row's batch and the input coordinates of its tap 0
+    uint32_t a_voff[A_ROWS], a_inv[A_ROWS];
+    int a_off0 = 0, a_hi0 = 0, a_wi0 = 0;
 #pragma unroll
     for (int p = 0; p < A_ROWS; ++p) {
         const int row = A_FAST ? (tid / A_VPR + p * A_RSTEP) : (tid % BM);
         const int m = m0 + row;
-        if (m < P.M) {
-            int b = 0, ho = m, wo = 0;
-            if (!P.flat_rows) { b = m / HoWo; const int r2 = m - b * HoWo; ho = r2 / P.Wo; wo = r2 - ho * P.Wo; }
-            a_hi0[p] = ho * P.SH - P.PH;
-            a_wi0[p] = wo * P.SW - P.PW;
-            a_off[p] = b * P.xs_b + (A_FAST ? a_hi0[p] * P.xs_h + a_wi0[p] * P.xs_w + (tid % A_VPR) * 4 : 0);
+        int b = 0, ho = m, wo = 0;
+        if (!flat_rows) {
+            b = magic_div(m, P.howo_magic, P.howo_shift);
+            const int r2 = m - b * HoWo;
+            ho = magic_div(r2, P.wo_magic, P.wo_shift);
+            wo = r2 - ho * P.Wo;
+        }
+        const int hi0 = ho * P.SH - P.PH, wi0 = wo * P.SW - P.PW;
+        if constexpr (A_FAST) {
+            a_voff[p] = m < P.M ? (uint32_t)(b * P.xs_b + ho * P.SH * P.xs_h + wo * P.SW * P.xs_w + (tid % A_VPR) * 4) * 4u : CONV_OOB;
+            a_inv[p]  = 0u;
+            if (masked) {
+                uint32_t wbad = 0u;
+                for (int s = 0; s < P.KW; ++s) wbad |= ((uint32_t)(wi0 + s * P.DW) >= (uint32_t)P.W ? 1u : 0u) << s;
+                const uint32_t wall = (2u << (P.KW - 1)) - 1u;
+                for (int r = 0; r < P.KH; ++r)
+                    a_inv[p] |= ((uint32_t)(hi0 + r * P.DH) >= (uint32_t)P.H ? wall : wbad) << (r * P.KW);
+            }
         } else {
-            a_off[p] = 0; a_hi0[p] = -(1 << 28); a_wi0[p] = -(1 << 28);
+            a_voff[p] = 0u; a_inv[p] = 0u;
+            a_off0 = b * P.xs_b;
+            a_hi0 = m < P.M ? hi0 : -(1 << 28);
+            a_wi0 = m < P.M ? wi0 : -(1 << 28);
         }
     }
-    // When a k tile never straddles two kernel taps (Cin % BK == 0) the tap (ky, kx) and first
-    // feature of a tile are the same for the whole block and live in scalar registers.
-    const bool uniform_taps = A_FAST && (P.Cin % BK == 0);
+    // When a k tile never straddles two kernel taps (Cin % BK == 0, or there is only one tap) the
+    // tap (ky, kx) and first feature of a tile are the same for the whole block and live in
+    // scalar registers.
+    const bool uniform_taps = A_FAST && (P.Cin % BK == 0 || P.KH * P.KW == 1);
     int t_r = 0, t_s = 0, t_c = 0;                  // uniform tile position
     // otherwise every thread tracks the position of its own first k
     int ak = A_FAST ? (tid % A_VPR) * 4 : (tid / BM) * A_KPT;
@@ -181,7 +231,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     constexpr int B_KPT   = BK / B_KG;
     // B fast: byte offset of this thread's first vector in tile 0, or out of range for columns >= N
     const int      b_n    = n0 + (tid % B_VPR) * 4;
-    const uint32_t b_off0 = b_n < P.N ? (uint32_t)(((tid / B_VPR) * P.N + b_n) * 4) : CONV_OOB;
+    const uint32_t b_voff = b_n < P.N ? (uint32_t)((tid / B_VPR) * P.N + b_n) * 4u : CONV_OOB;
 
     f32x4 a_reg[A_FAST ? A_NV : 1];
     float a_sreg[A_FAST ? 1 : A_KPT];
@@ -191,32 +241,44 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     auto load_tiles = [&](int k0) {
         // ---- A ----
         if constexpr (A_FAST) {
-            int r, s, koff;                          // tap of this thread's vector and its element offset
-            bool kok = true;
             if (uniform_taps) {
-                r = t_r; s = t_s;
-                koff = t_r * P.DH * P.xs_h + t_s * P.DW * P.xs_w + t_c;
-            } else {
-                r = ar; s = as_;
-                koff = ar * P.DH * P.xs_h + as_ * P.DW * P.xs_w + ac - (tid % A_VPR) * 4;
-                kok = ak < P.K;
-            }
-            const int dh = r * P.DH, dw = s * P.DW;
+                // everything that changes from tile to tile is wave-uniform
+                const uint32_t soff = (uint32_t)(t_r * P.DH * P.xs_h + t_s * P.DW * P.xs_w + t_c) * 4u;
+                const bool     tail = k0 + BK > P.K;                 // only with a single tap
+                if (!masked && !tail) {
+                    // the common case issues the loads with no vector arithmetic at all
 #pragma unroll
-            for (int p = 0; p < A_NV; ++p) {
-                const bool ok = kok && (uint32_t)(a_hi0[p] + dh) < (uint32_t)P.H && (uint32_t)(a_wi0[p] + dw) < (uint32_t)P.W;
-                a_reg[p] = buffer_load_x4(x_rsrc, ok ? (uint32_t)(a_off[p] + koff) * 4u : CONV_OOB);
+                    for (int p = 0; p < A_NV; ++p) a_reg[p] = buffer_load_x4(x_rsrc, a_voff[p], soff);
+                } else {
+                    const uint32_t sh   = 31u - (uint32_t)(t_r * P.KW + t_s);
+                    const bool     kbad = tail && k0 + (tid % A_VPR) * 4 >= P.K;
+#pragma unroll
+                    for (int p = 0; p < A_NV; ++p) {
+                        const uint32_t v = a_voff[p] | ((a_inv[p] << sh) & CONV_OOB);
+                        a_reg[p] = buffer_load_x4(x_rsrc, kbad ? CONV_OOB : v, soff);
+                    }
+                }
+            } else {
+                const uint32_t koff = (uint32_t)(ar * P.DH * P.xs_h + as_ * P.DW * P.xs_w + ac - (tid % A_VPR) * 4) * 4u;
+                const uint32_t sh   = 31u - (uint32_t)(ar * P.KW + as_);
+                const bool     kok  = ak < P.K;
+#pragma unroll
+                for (int p = 0; p < A_NV; ++p) {
+                    uint32_t v = (a_voff[p] + koff) | (a_voff[p] & CONV_OOB);
+                    if (masked) v |= (a_inv[p] << sh) & CONV_OOB;
+                    a_reg[p] = buffer_load_x4(x_rsrc, kok ? v : CONV_OOB);
+                }
             }
         } else {
             int c = ac, s = as_, r = ar, k = ak;
 #pragma unroll
             for (int j = 0; j < A_KPT; ++j) {
-                int hi = a_hi0[0] + r * P.DH, wi = a_wi0[0] + s * P.DW;
+                int hi = a_hi0 + r * P.DH, wi = a_wi0 + s * P.DW;
                 bool ok = hi >= 0 && wi >= 0 && k < P.K;
-                if (P.LH > 1) { ok = ok && (hi % P.LH == 0); hi /= P.LH; }
-                if (P.LW > 1) { ok = ok && (wi % P.LW == 0); wi /= P.LW; }
+                if (Pk.LH > 1) { ok = ok && (hi % Pk.LH == 0); hi /= Pk.LH; }
+                if (Pk.LW > 1) { ok = ok && (wi % Pk.LW == 0); wi /= Pk.LW; }
                 ok = ok && hi < P.H && wi < P.W;
-                a_sreg[j] = ok ? x[a_off[0] + hi * P.xs_h + wi * P.xs_w + c * P.xs_c] : 0.f;
+                a_sreg[j] = ok ? x[a_off0 + hi * P.xs_h + wi * P.xs_w + c * Pk.xs_c] : 0.f;
                 ++k; ++c;
                 if (c == P.Cin) { c = 0; ++s; if (s == P.KW) { s = 0; ++r; } }
             }
@@ -224,10 +286,9 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         // ---- B ----
         if constexpr (B_FAST) {
             // rows k >= K fall beyond the descriptor and read as zeros
-            const uint32_t base = b_off0 == CONV_OOB ? CONV_OOB : b_off0 + (uint32_t)k0 * (uint32_t)P.N * 4u;
 #pragma unroll
             for (int p = 0; p < B_NV; ++p)
-                b_reg[p] = buffer_load_x4(w_rsrc, base == CONV_OOB ? CONV_OOB : base + (uint32_t)(p * B_RSTEP) * (uint32_t)P.N * 4u);
+                b_reg[p] = buffer_load_x4(w_rsrc, b_voff, (uint32_t)(k0 + p * B_RSTEP) * (uint32_t)P.N * 4u);
         } else {
             const int n = n0 + tid % BN;
             int k = k0 + (tid / BN) * B_KPT;
@@ -235,7 +296,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
             int c = k - rs * P.Cin, r = rs / P.KW, s = rs - r * P.KW;
 #pragma unroll
             for (int j = 0; j < B_KPT; ++j) {
-                b_sreg[j] = (k < P.K && n < P.N) ? w[r * P.ws_r + s * P.ws_s + c * P.ws_c + n * P.ws_n] : 0.f;
+                b_sreg[j] = (k < P.K && n < P.N) ? w[r * Pk.ws_r + s * Pk.ws_s + c * Pk.ws_c + n * Pk.ws_n] : 0.f;
                 ++k; ++c;
                 if (c == P.Cin) { c = 0; ++s; if (s == P.KW) { s = 0; ++r; } }
             }
@@ -243,7 +304,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         // advance to the next k tile
         if (uniform_taps) {
             t_c += BK;
-            if (t_c == P.Cin) { t_c = 0; ++t_s; if (t_s == P.KW) { t_s = 0; ++t_r; } }
+            if (t_c >= P.Cin) { t_c = 0; ++t_s; if (t_s == P.KW) { t_s = 0; ++t_r; } }
         } else {
             ak += BK; ac += BK;
             while (ac >= P.Cin) { ac -= P.Cin; ++as_; if (as_ == P.KW) { as_ = 0; ++ar; } }
@@ -284,15 +345,21 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     const int ktiles = (P.K + BK - 1) / BK;
+    CONV_STAMP(1)
     load_tiles(0);
+    if (tid < BN) {
 #pragma unroll
-    for (int q = 0; q < E_PER_THREAD; ++q)
-        if (tid + q * NT < (int)P.nepi * BN) Es[tid + q * NT] = e_reg[q];
+        for (int e = 0; e < CONV_MAX_EPI; ++e)
+            if (e < nepi) Es[e * BN + tid] = e_reg[e];
+    }
     if (ktiles == 0) __syncthreads();            // otherwise the barriers of the k loop publish Es
     for (int kt = 0; kt < ktiles; ++kt) {
         store_tiles();
         __syncthreads();
         if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
+#ifdef CONV_PHASE_STAMPS
+        if (kt == 0) { CONV_STAMP(2) }
+#endif
         // lanes 0-31 consume the first half of the tile's k range, lanes 32-63 the second half.
         // Fragments are double-buffered in registers: the LDS reads of group g+1 are in flight
         // while the MFMAs of group g execute.
@@ -323,37 +390,53 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         }
         __syncthreads();
     }
+    CONV_STAMP(3)
 
     // ---------------- epilogue + store ----------------
     // accumulator element v of a lane: row = 8*(v/4) + 4*half + v%4, column = l32.
     // Byte offsets fit 31 bits: the host refuses larger tensors.
-    const bool whole_tile = m0 + BM <= P.M && n0 + BN <= P.N;
     // Outputs that are not a row-major [M, N] matrix need (batch, y, x) of every row: decoded once
     // per row into the LDS space of the A tile (free after the k loop), -1 for rows beyond M.
     int* const row_off = reinterpret_cast<int*>(As);
-    if (!P.c_contig) {
+    if (!c_contig) {
         for (int r = tid; r < BM; r += NT) {
             const int m = m0 + r;
             const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
-            row_off[r] = m < P.M ? b * P.os_b + ho * P.os_h + wo * P.os_w : -1;
+            row_off[r] = m < P.M ? b * Pk.os_b + ho * Pk.os_h + wo * Pk.os_w : -1;
         }
         __syncthreads();
     }
-    auto elem_offset = [&](int i, int j, int v) -> uint32_t {
-        const int n = n0 + (wn * TN + j) * 32 + l32;
-        const int r = (wm * TM + i) * 32 + 4 * half + 8 * (v / 4) + (v % 4);
-        if (P.c_contig) {
-            const int m = m0 + r;
-            return (whole_tile || (m < P.M && n < P.N)) ? (uint32_t)(m * P.N + n) * 4u : CONV_OOB;
+    // Calls fn(v, per-lane byte offset, uniform byte offset) for the 16 accumulator elements a
+    // lane holds of sub-tile (i, j); the offsets are out of range outside the matrix. For a
+    // row-major result one per-lane offset serves all 16 (the row goes into the uniform part,
+    // and rows beyond M lie beyond the descriptor's size). The lane id goes through an opaque
+    // copy so that this arithmetic is redone at each use instead of occupying registers for
+    // the whole epilogue.
+    auto sub_tile = [&](int i, int j, auto&& fn) {
+        int l = l32;
+        asm volatile("" : "+v"(l));
+        const int n  = n0 + (wn * TN + j) * 32 + l;
+        const int r0 = (wm * TM + i) * 32 + 4 * half;
+        if (c_contig) {
+            const uint32_t base = n < P.N ? (uint32_t)((m0 + r0) * P.N + n) * 4u : CONV_OOB;
+            const uint32_t rowb = (uint32_t)P.N * 4u;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) fn(v, base, (uint32_t)(8 * (v / 4) + (v % 4)) * rowb);
+        } else {
+            const int* ro = row_off + r0 + (l - l32);
+            const int  cn = n < P.N ? n * Pk.os_n : -(1 << 30);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = ro[8 * (v / 4) + (v % 4)];
+                fn(v, (r >= 0 && cn >= 0) ? (uint32_t)(r + cn) * 4u : CONV_OOB, 0u);
+            }
         }
-        const int ro = row_off[r];
-        return (ro >= 0 && n < P.N) ? (uint32_t)(ro + n * P.os_n) * 4u : CONV_OOB;
     };
     // the first full-size operand (a residual input) is fetched for the whole tile at once
     // (for the largest tile that would not fit the register file: it loads sub-tile by sub-tile)
     constexpr bool PREFETCH_FULL = TM * TN <= 2;
     float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
-    const int first_full = PREFETCH_FULL ? P.epi_first_full : -1;
+    const int first_full = PREFETCH_FULL ? epi_first_full : -1;
     if (PREFETCH_FULL && first_full >= 0) {
         const float* fp = epi.p[0];
 #pragma unroll
@@ -363,61 +446,147 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, elem_offset(i, j, v));
+                sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) {
+                    full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, vo, so);
+                });
     }
-#pragma unroll
-    for (int e = 0; e < CONV_MAX_EPI; ++e) {             // unrolled: the step descriptors stay in scalar registers
-        if (e >= (int)P.nepi) break;
-        const uint32_t kind = P.epi_kind[e];
-        const uint32_t code = P.epi_op[e] * 2u + ((P.epi_flags[e] >> 1) & 1u);   // bit0: operand on the left
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                float ov[16];
-                if (kind == 3) {
-                    if (PREFETCH_FULL && e == first_full) {
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) ov[v] = full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v];
-                    } else {
-                        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(epi.p[e], P.out_bytes);
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) ov[v] = buffer_load_x1(f_rsrc, elem_offset(i, j, v));
-                    }
-                } else {
-                    const float o1 = Es[e * BN + (wn * TN + j) * 32 + l32];
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) ov[v] = o1;
-                }
-#define EPI_LOOP(expr)                                              \
-                _Pragma("unroll") for (int v = 0; v < 16; ++v) {    \
-                    const float y = acc[i][j][v], o = ov[v];        \
-                    acc[i][j][v] = (expr);                          \
-                }
-                switch (code) {                              // one uniform branch per step, not per element
-                    case CEW_ADD_F * 2: case CEW_ADD_F * 2 + 1: EPI_LOOP(y + o) break;
-                    case CEW_MUL_F * 2: case CEW_MUL_F * 2 + 1: EPI_LOOP(y * o) break;
-                    case CEW_SUB_F * 2:     EPI_LOOP(y - o) break;
-                    case CEW_SUB_F * 2 + 1: EPI_LOOP(o - y) break;
-                    case CEW_DIV_F * 2:     EPI_LOOP(y / o) break;
-                    case CEW_DIV_F * 2 + 1: EPI_LOOP(o / y) break;
-                    case CEW_MAX_F * 2:     EPI_LOOP((y > o || y != y) ? y : o) break;
-                    case CEW_MAX_F * 2 + 1: EPI_LOOP((o > y || o != o) ? o : y) break;
-                    case CEW_MIN_F * 2:     EPI_LOOP((y < o || y != y) ? y : o) break;
-                    case CEW_MIN_F * 2 + 1: EPI_LOOP((o < y || o != o) ? o : y) break;
-                    default: break;
-                }
-#undef EPI_LOOP
-            }
-    }
+#ifdef CONV_PHASE_STAMPS
+    if (first_full >= 0) { float sink = full[0][0][0]; asm volatile("" :: "v"(sink)); }
+    CONV_STAMP(4)
+#endif
+    // From here on the accumulators are handled as separate scalars: element-wise updates of a
+    // 16-register MFMA tuple make the compiler copy the whole tuple at every step.
+    float c[TM][TN][16];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) buffer_store_x1(acc[i][j][v], o_rsrc, elem_offset(i, j, v));
+            for (int v = 0; v < 16; ++v) c[i][j][v] = acc[i][j][v];
+    // one uniform branch per step and sub-tile, not per element
+    auto apply = [&](uint32_t code, float (&y)[16], auto&& operand) {
+#define EPI_LOOP(expr) _Pragma("unroll") for (int v = 0; v < 16; ++v) { const float a = y[v], o = operand(v); y[v] = (expr); }
+        switch (code) {                                          // bit0: operand on the left
+            case CEW_ADD_F * 2: case CEW_ADD_F * 2 + 1: EPI_LOOP(a + o) break;
+            case CEW_MUL_F * 2: case CEW_MUL_F * 2 + 1: EPI_LOOP(a * o) break;
+            case CEW_SUB_F * 2:     EPI_LOOP(a - o) break;
+            case CEW_SUB_F * 2 + 1: EPI_LOOP(o - a) break;
+            case CEW_DIV_F * 2:     EPI_LOOP(a / o) break;
+            case CEW_DIV_F * 2 + 1: EPI_LOOP(o / a) break;
+            case CEW_MAX_F * 2:     EPI_LOOP((a > o || a != a) ? a : o) break;
+            case CEW_MAX_F * 2 + 1: EPI_LOOP((o > a || o != o) ? o : a) break;
+            case CEW_MIN_F * 2:     EPI_LOOP((a < o || a != a) ? a : o) break;
+            case CEW_MIN_F * 2 + 1: EPI_LOOP((o < a || o != o) ? o : a) break;
+            default: __builtin_unreachable();                    // the host fuses no other operation
+        }
+#undef EPI_LOOP
+    };
+    const uint32_t slots = (P.flags >> 20) & 31u;
+    if (slots) {
+        // The usual chains (bias, batch norm, residual add, ReLU in that order, each optional) run as
+        // straight-line code: every step is one pass over a sub-tile's 16 values, in place.
+        const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u),
+                  e_res = __builtin_popcount(slots & 7u), e_max = __builtin_popcount(slots & 15u);
+        const float* rp = epi.p[0];
+#pragma unroll
+        for (int t = 1; t < CONV_MAX_EPI; ++t) rp = e_res == t ? epi.p[t] : rp;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                float (&y)[16] = c[i][j];
+                const int col = (wn * TN + j) * 32 + l32;
+                if (slots & 1u) {
+                    const float o = Es[col];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) y[v] = y[v] - o;
+                }
+                if (slots & 2u) {
+                    const float o = Es[e_mul * BN + col];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) y[v] = y[v] * o;
+                }
+                if (slots & 4u) {
+                    const float o = Es[e_add * BN + col];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) y[v] = y[v] + o;
+                }
+                if (slots & 8u) {
+                    if constexpr (PREFETCH_FULL) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) y[v] = y[v] + full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v];
+                    } else {
+                        float ov[16];
+                        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(rp, P.out_bytes);
+                        sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(f_rsrc, vo, so); });
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) y[v] = y[v] + ov[v];
+                    }
+                }
+                if (slots & 16u) {
+                    const float o = Es[e_max * BN + col];          // the same value in every lane
+                    if (__builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, o != o ? 1.f : 0.f)) == 0) {
+                        // max(y, o) that returns a NaN y, for o known not to be NaN: one compare
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) y[v] = !(y[v] <= o) ? y[v] : o;
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) y[v] = (y[v] > o || y[v] != y[v]) ? y[v] : o;
+                    }
+                }
+            }
+    } else {
+    // The step loop stays rolled (one copy of the step code keeps the kernel small enough for the
+    // instruction cache); descriptors and operand pointers are picked with scalar selects.
+#pragma nounroll
+    for (int e = 0; e < nepi; ++e) {
+        const uint32_t kind = step_desc(e) >> 8;
+        const uint32_t code = step_desc(e) & 255u;
+        const float* ep = epi.p[0];
+#pragma unroll
+        for (int t = 1; t < CONV_MAX_EPI; ++t) ep = e == t ? epi.p[t] : ep;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if (kind == 3) {
+                    if (PREFETCH_FULL && e == first_full) {
+                        apply(code, c[i][j], [&](int v) { return full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v]; });
+                    } else {
+                        float ov[16];
+                        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(ep, P.out_bytes);
+                        sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(f_rsrc, vo, so); });
+                        apply(code, c[i][j], [&](int v) { return ov[v]; });
+                    }
+                } else {
+                    // one value per column: used straight from its register
+                    const float o1 = Es[e * BN + (wn * TN + j) * 32 + l32];
+                    apply(code, c[i][j], [&](int) { return o1; });
+                }
+            }
+#ifdef CONV_PHASE_STAMPS
+        { float sink = c[0][0][0]; asm volatile("" :: "v"(sink)); const unsigned long long t = wall_clock64();
+          if (e == 0) stamps[8] = t; else if (e == 1) stamps[9] = t; else if (e == 2) stamps[10] = t;
+          else if (e == 3) stamps[11] = t; else if (e == 4) stamps[12] = t; else stamps[13] = t; }
+#endif
+    }
+    }
+#ifdef CONV_PHASE_STAMPS
+    { float sink = 0; for (int v = 0; v < 16; ++v) sink += c[0][0][v]; asm volatile("" :: "v"(sink)); }
+    CONV_STAMP(5)
+#endif
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) { buffer_store_x1(c[i][j][v], o_rsrc, vo, so); });
+#ifdef CONV_PHASE_STAMPS
+    CONV_STAMP(6)
+    if (epi.p[CONV_MAX_EPI - 1] != nullptr && tid == 0) {
+        unsigned long long* d = (unsigned long long*)epi.p[CONV_MAX_EPI - 1] + (size_t)blockIdx.x * 16;
+        for (int q = 0; q < 16; ++q) d[q] = stamps[q];
+    }
+#endif
 }
 
 #define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF)                                                     \

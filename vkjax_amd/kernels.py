@@ -284,6 +284,34 @@ def _flatten_pointwise(g: ConvGeometry) -> ConvGeometry:
     return g._replace(batch=1, Ho=M, Wo=1, H=M, W=1, xs=(0, g.xs[2], 0, 1), os=(M * g.N, g.N, g.N, 1))
 
 
+def _epilogue_template_slots(epilogue: tp.Sequence[ConvEpilogueStep]) -> int:
+    '''Bit k set = step k of the kernel's straight-line epilogue (acc - vector, acc * vector,
+    acc + vector, acc + full tensor, max(acc, scalar)) is present; 0 if the chain is not an
+    ordered subset of those and has to go through the kernel's general step loop.'''
+    template = ((EW['SUB_F'], 2, False), (EW['MUL_F'], 2, None), (EW['ADD_F'], 2, None),
+                (EW['ADD_F'], 3, None), (EW['MAX_F'], 1, False))
+    slots, k = 0, 0
+    for e in epilogue:
+        while k < len(template):
+            op, kind, left = template[k]
+            k += 1
+            if e.op == op and e.kind == kind and (left is None or bool(e.operand_left) == left):
+                slots |= 1 << (k - 1)
+                break
+        else:
+            return 0
+    return slots
+
+
+def _magic_division(d: int) -> tp.Tuple[int, int]:
+    '''(magic, shift) with n // d == (n * magic >> 32) >> shift for every 0 <= n < 2**31; magic 0 stands for d == 1.'''
+    if d <= 1:
+        return 0, 0
+    l = (d - 1).bit_length()                  #ceil(log2(d))
+    magic = -(-(1 << (31 + l)) // d)          #ceil(2**(31+l) / d) < 2**32
+    return magic, l - 1
+
+
 def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: tp.Sequence[ConvEpilogueStep] = (),
               compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0) -> Launch:
     if len(epilogue) > CONV_MAX_EPI:
@@ -295,8 +323,15 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
             raise NotImplementedError(f'conv/dot {name} operand of {extent * 4} bytes exceeds the 2 GiB the kernel addresses')
     tag, bm, bn, nt = choose_conv_tile(M, N, compute_units)
     bk = choose_conv_bk(tag, g)
+    #some kernel tap of some output position falls outside the input (padding, or a window that overhangs)
+    needs_masks = (g.PH > 0 or g.PW > 0 or (g.Ho - 1) * g.SH - g.PH + (g.KH - 1) * g.DH >= g.H
+                   or (g.Wo - 1) * g.SW - g.PW + (g.KW - 1) * g.DW >= g.W)
+    #the 16-byte A path keeps the validity of a row's taps in one 32-bit mask and addresses the
+    #input from (PH, PW) positions before its start
+    x_bias = (g.PH * g.xs[1] + g.PW * g.xs[2]) * 4
     a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0
-              and all(s % 4 == 0 for s in g.xs[:3]))
+              and all(s % 4 == 0 and s >= 0 for s in g.xs[:3]) and (not needs_masks or g.KH * g.KW <= 32)
+              and (lhs.size - lhs_offset) * 4 + x_bias <= 2**31)
     b_fast = (g.ws[3] == 1 and N % 4 == 0 and rhs_offset % 4 == 0
               and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
     c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
@@ -305,12 +340,17 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     kinds = [e.kind for e in epilogue]
     x_bytes = (lhs.size - lhs_offset) * 4
     w_bytes = K * N * 4 if b_fast else (rhs.size - rhs_offset) * 4
-    params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW, g.LH, g.LW,
-                   *g.xs, *g.ws, *g.os, int(c_contig), tiles_m, tiles_n)
-              + _u32(len(epilogue), *_pad([e.op for e in epilogue], CONV_MAX_EPI),
-                     *_pad([2 if e.operand_left else 0 for e in epilogue], CONV_MAX_EPI), *_pad(kinds, CONV_MAX_EPI))
-              + _i32(kinds.index(3) if 3 in kinds else -1, int(flat_rows))
-              + _u32(x_bytes, w_bytes, out.size * 4))
+    first_full = kinds.index(3) + 1 if 3 in kinds else 0
+    flags = (int(c_contig) | int(flat_rows) << 1 | int(needs_masks) << 2 | len(epilogue) << 8 | first_full << 16
+             | _epilogue_template_slots(epilogue) << 20)
+    descs = [0, 0]
+    for i, e in enumerate(epilogue):
+        assert e.op < 128 and 1 <= e.kind <= 3
+        descs[i // 3] |= ((e.op * 2 + int(e.operand_left)) | e.kind << 8) << (10 * (i % 3))
+    params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW,
+                   *g.xs[:3], tiles_m, tiles_n)
+              + _u32(flags, *descs, x_bytes, w_bytes, out.size * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
+              + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os))
     buffers = [(out, 0), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
     buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
     kernel  = f'conv_gemm_{tag}x{bk}_{"f" if a_fast else "g"}{"f" if b_fast else "g"}'
