@@ -104,11 +104,15 @@ def test_reduce_window_matrix(f, desc, args, exact):
     check_against_oracle(f, args, exact=exact, rtol=1e-5, atol=1e-6)
 
 
-@pytest.mark.parametrize('tile,bk', [('128x128', 32), ('128x64', 32), ('64x64', 32), ('64x64', 64), ('32x32', 32), ('32x32', 64)])
+TILES = [('128x128', 32), ('128x64', 32), ('64x64', 32), ('64x64', 64), ('32x32', 32), ('32x32', 64)]
+
+
+@pytest.mark.parametrize('tile,bk', TILES)
 def test_every_tile_and_loader_variant(tile, bk):
-    '''All 24 kernel instantiations: each tile shape and k step with 16-byte (f) or strided (g) loads on
-    either operand; the ff2 / ff3 cases have Cin % 64 == 0 (tap position kept in scalar registers) and a
-    1x1 unpadded kernel (rows addressed as a flat matrix).'''
+    '''All 30 kernel instantiations: each tile shape and k step with 16-byte (f) or strided (g) loads on
+    either operand, and the lean variant. The ff2 / ff3 cases have Cin % 64 == 0 (tap position kept in
+    scalar registers) and a 1x1 unpadded kernel (rows addressed as a flat matrix): they qualify for the
+    lean variant and run through both it and the general ff kernel.'''
     from vkjax_amd import kernels as K
     cases = {'ff': ([3, 20, 17, 16], [3, 3, 16, 24]), 'gg': ([2, 13, 11, 5], [3, 3, 5, 7]),
              'gf': ([2, 13, 11, 3], [3, 3, 3, 64]), 'fg': ([2, 13, 11, 8], [3, 3, 8, 10]),
@@ -116,11 +120,51 @@ def test_every_tile_and_loader_variant(tile, bk):
     K.FORCE_CONV_TILE, K.FORCE_CONV_BK = tile, bk
     try:
         for variant, (xs, ks) in cases.items():
-            print(f'tile {tile} bk {bk} loaders {variant}', flush=True)
-            x = rng.randint(-4, 5, size=xs).astype(np.float32)
-            k = rng.randint(-3, 4, size=ks).astype(np.float32)
-            _, _, fn = check_against_oracle(conv2, [x, k], exact=True)
-            kernel = list(fn._jaxpr_interpreters.values())[0].launches[0].kernel
-            assert kernel == f'conv_gemm_{tile}x{bk}_{variant[:2]}', kernel
+            for general in (True, False):
+                K.FORCE_CONV_GENERAL = general
+                expected = variant[:2] if general or variant not in ('ff2', 'ff3') else 'lean'
+                print(f'tile {tile} bk {bk} loaders {variant} -> {expected}', flush=True)
+                x = rng.randint(-4, 5, size=xs).astype(np.float32)
+                k = rng.randint(-3, 4, size=ks).astype(np.float32)
+                _, _, fn = check_against_oracle(conv2, [x, k], exact=True)
+                kernel = list(fn._jaxpr_interpreters.values())[0].launches[0].kernel
+                assert kernel == f'conv_gemm_{tile}x{bk}_{expected}', kernel
     finally:
         K.FORCE_CONV_TILE = K.FORCE_CONV_BK = None
+        K.FORCE_CONV_GENERAL = False
+
+
+@pytest.mark.parametrize('tile,bk', TILES)
+def test_lean_kernel_tile_chunks_with_epilogue(tile, bk):
+    '''The lean variant walking 1, 2, 3 or 5 consecutive M tiles per block (the last block of a launch gets
+    a shorter run), with and without padding taps, with a batch-norm + residual + ReLU epilogue, a
+    bias + ReLU epilogue and none; integer-valued data, so every result is exact.'''
+    from vkjax_amd import kernels as K
+    from vkjax_amd import minijax as mj
+    lax, nn = mj.lax, mj.nn
+    dn = ('NHWC', 'HWIO', 'NHWC')
+
+    def bn_res_relu(x, k, mean, scale, beta, res):
+        y = lax.conv_general_dilated(x, k, (1, 1), 'SAME', dimension_numbers=dn)
+        return nn.relu((y - mean) * scale + beta + res)
+
+    def bias_relu(x, k, bias):
+        return nn.relu(lax.conv_general_dilated(x, k, (2, 2), 'VALID', dimension_numbers=dn) + bias)
+
+    K.FORCE_CONV_TILE, K.FORCE_CONV_BK = tile, bk
+    try:
+        for chunk in (1, 2, 3, 5):
+            K.FORCE_CONV_CHUNK = chunk
+            for ksize, cin, cout in ((3, 64, 40), (1, 128, 72)):
+                print(f'tile {tile} bk {bk} chunk {chunk} kernel {ksize}x{ksize} {cin}->{cout}', flush=True)
+                x = rng.randint(-4, 5, size=[3, 13, 11, cin]).astype(np.float32)
+                k = rng.randint(-3, 4, size=[ksize, ksize, cin, cout]).astype(np.float32)
+                vec = lambda lo, hi: rng.randint(lo, hi, size=[cout]).astype(np.float32)
+                res = rng.randint(-50, 50, size=[3, 13, 11, cout]).astype(np.float32)
+                for f, args in ((bn_res_relu, [x, k, vec(-5, 5), vec(1, 4), vec(-9, 9), res]), (bias_relu, [x, k, vec(-9, 9)]),
+                                (conv2, [x, k])):
+                    _, _, fn = check_against_oracle(f, args, exact=True)
+                    launches = list(fn._jaxpr_interpreters.values())[0].launches
+                    assert [l.kernel for l in launches] == [f'conv_gemm_{tile}x{bk}_lean'], [l.kernel for l in launches]
+    finally:
+        K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = None

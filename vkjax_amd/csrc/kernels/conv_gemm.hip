@@ -59,7 +59,8 @@ struct ConvParams {
                                     // steps; bits 16-19: 1 + index of the first kind-3 step, or 0;
                                     // bits 20-24: the steps are, in this order, a subset of
                                     // (acc - vector, * vector, + vector, + full tensor, max(acc, scalar)):
-                                    // bit 20+k set = template step k is present
+                                    // bit 20+k set = template step k is present;
+                                    // bits 25-28: M tiles per block (at least 1)
     uint32_t epi_desc[2];           // 10 bits per step, steps 0-2 in [0], 3-5 in [1]: bits 0-7 opcode * 2 +
                                     // (operand is the left argument), bits 8-9 kind: 1 scalar,
                                     // 2 per-feature vector [N], 3 full tensor laid out like out
@@ -98,7 +99,11 @@ __device__ __forceinline__ int magic_div(int n, uint32_t magic, uint32_t shift) 
 #define CONV_STAMP(slot)
 #endif
 
-template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST>
+// LEAN: the variant for the common case, with the rarely needed paths compiled out (they cost
+// registers, and with them resident waves, even when not taken): both operands on the 16-byte
+// path, k tiles that never straddle kernel taps, a row-major result, an epilogue that fits the
+// straight-line template.
+template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST, bool LEAN>
 __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
                                                const float* __restrict__ w, const ConvEpiPtrs& epi,
                                                const ConvParams& Pk) {
@@ -107,6 +112,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     __shared__ __attribute__((aligned(16))) float As[BM * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
     __shared__ float Es[CONV_MAX_EPI * BN];         // per-column operands of the epilogue steps
+    __shared__ int   Rs[BM];                        // row offsets of outputs that are not row-major
 #ifdef CONV_PHASE_STAMPS
     unsigned long long stamps[16] = {};
 #endif
@@ -131,21 +137,28 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 #undef CONV_PIN
     static_assert(CONV_MAX_EPI == 6, "descriptor packing");
     auto step_desc = [&](int e) -> uint32_t { return ((e < 3 ? P.epi_desc[0] : P.epi_desc[1]) >> (10 * (e < 3 ? e : e - 3))) & 1023u; };
-    const bool c_contig = P.flags & 1u, flat_rows = P.flags & 2u, masked = P.flags & 4u;
+    const bool c_contig = LEAN || (P.flags & 1u), flat_rows = P.flags & 2u, masked = P.flags & 4u;
     const int nepi = (P.flags >> 8) & 15u, epi_first_full = (int)((P.flags >> 16) & 15u) - 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
     const int l32 = lane & 31, half = lane >> 5;
 
+    // A block works through up to `chunk` consecutive M tiles of one N tile, one after the other,
+    // as one flat sequence of k steps: while a step is computed the loads of the next one are in
+    // flight, also across the boundary between two M tiles. Only the first tile of a block pays
+    // the latency of the argument fetch, the address set-up and the first loads in full.
     // Consecutive block ids go to different XCDs (8 of them, each with its own L2). Hand every
-    // XCD a contiguous range of tiles so that the N-tiles of one M-tile share an L2.
-    int tile = blockIdx.x;
+    // XCD a contiguous range of work so that the N-tiles of one M-tile share an L2.
+    const int chunk = LEAN ? (P.flags >> 25) & 15u : 1;         // the general variants take one tile per block
+    const int chunks_m = (P.tiles_m + chunk - 1) / chunk;
+    int work = blockIdx.x;
     {
-        const int total = P.tiles_m * P.tiles_n, per = total / 8;
-        if (per > 0 && tile < per * 8) tile = (tile & 7) * per + (tile >> 3);
+        const int total = chunks_m * P.tiles_n, per = total / 8;
+        if (per > 0 && work < per * 8) work = (work & 7) * per + (work >> 3);
     }
-    const int tile_m = tile / P.tiles_n, tile_n = tile - tile_m * P.tiles_n;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int chunk_m = work / P.tiles_n, tile_n = work - chunk_m * P.tiles_n;
+    const int tile_m0 = chunk_m * chunk, nsub = LEAN ? min(chunk, P.tiles_m - tile_m0) : 1;
+    const int n0 = tile_n * BN;
     const int HoWo = P.Ho * P.Wo;
 
     // The 16-byte A path addresses the input from (PH, PW) positions before its start, so that
@@ -168,6 +181,15 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
             else if (kind == 2) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], (uint32_t)P.N * 4u), (uint32_t)(n0 + tid) * 4u);
         }
     }
+    // the first full-size operand (a residual input) is fetched for a whole tile at once, while
+    // the tile's last k step is computed (for the largest tile that would not fit the register
+    // file: it loads sub-tile by sub-tile in the epilogue)
+    constexpr bool PREFETCH_FULL = !LEAN && TM * TN <= 2;
+    const int first_full = (PREFETCH_FULL && c_contig) ? epi_first_full : -1;
+    const float* full_ptr = epi.p[0];
+#pragma unroll
+    for (int t = 1; t < CONV_MAX_EPI; ++t) full_ptr = epi_first_full == t ? epi.p[t] : full_ptr;
+    const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(full_ptr, P.out_bytes);
 
     // ---------------- per-thread load assignment ----------------
     // A fast: 16-byte vectors along k. A generic: one row, a run of consecutive k.
@@ -182,47 +204,54 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     // generic: element offset of the row's batch and the input coordinates of its tap 0
     uint32_t a_voff[A_ROWS], a_inv[A_ROWS];
     int a_off0 = 0, a_hi0 = 0, a_wi0 = 0;
-#pragma unroll
-    for (int p = 0; p < A_ROWS; ++p) {
-        const int row = A_FAST ? (tid / A_VPR + p * A_RSTEP) : (tid % BM);
-        const int m = m0 + row;
-        int b = 0, ho = m, wo = 0;
-        if (!flat_rows) {
-            b = magic_div(m, P.howo_magic, P.howo_shift);
-            const int r2 = m - b * HoWo;
-            ho = magic_div(r2, P.wo_magic, P.wo_shift);
-            wo = r2 - ho * P.Wo;
-        }
-        const int hi0 = ho * P.SH - P.PH, wi0 = wo * P.SW - P.PW;
-        if constexpr (A_FAST) {
-            a_voff[p] = m < P.M ? (uint32_t)(b * P.xs_b + ho * P.SH * P.xs_h + wo * P.SW * P.xs_w + (tid % A_VPR) * 4) * 4u : CONV_OOB;
-            a_inv[p]  = 0u;
-            if (masked) {
-                uint32_t wbad = 0u;
-                for (int s = 0; s < P.KW; ++s) wbad |= ((uint32_t)(wi0 + s * P.DW) >= (uint32_t)P.W ? 1u : 0u) << s;
-                const uint32_t wall = (2u << (P.KW - 1)) - 1u;
-                for (int r = 0; r < P.KH; ++r)
-                    a_inv[p] |= ((uint32_t)(hi0 + r * P.DH) >= (uint32_t)P.H ? wall : wbad) << (r * P.KW);
-            }
-        } else {
-            a_voff[p] = 0u; a_inv[p] = 0u;
-            a_off0 = b * P.xs_b;
-            a_hi0 = m < P.M ? hi0 : -(1 << 28);
-            a_wi0 = m < P.M ? wi0 : -(1 << 28);
-        }
-    }
     // When a k tile never straddles two kernel taps (Cin % BK == 0, or there is only one tap) the
     // tap (ky, kx) and first feature of a tile are the same for the whole block and live in
     // scalar registers.
-    const bool uniform_taps = A_FAST && (P.Cin % BK == 0 || P.KH * P.KW == 1);
+    const bool uniform_taps = LEAN || (A_FAST && (P.Cin % BK == 0 || P.KH * P.KW == 1));
     int t_r = 0, t_s = 0, t_c = 0;                  // uniform tile position
     // otherwise every thread tracks the position of its own first k
-    int ak = A_FAST ? (tid % A_VPR) * 4 : (tid / BM) * A_KPT;
-    int ac, as_, ar;
-    {
+    int ak = 0, ac = 0, as_ = 0, ar = 0;
+    // per-thread state for the M tile that starts at row m0, positioned at its first k tile
+    auto setup_rows = [&](int m0) {
+#pragma unroll
+        for (int p = 0; p < A_ROWS; ++p) {
+            const int row = A_FAST ? (tid / A_VPR + p * A_RSTEP) : (tid % BM);
+            const int m = m0 + row;
+            if (A_FAST && flat_rows) {
+                a_voff[p] = m < P.M ? (uint32_t)(m * P.xs_h + (tid % A_VPR) * 4) * 4u : CONV_OOB;
+                a_inv[p]  = 0u;
+                continue;
+            }
+            int b = 0, ho = m, wo = 0;
+            if (!flat_rows) {
+                b = magic_div(m, P.howo_magic, P.howo_shift);
+                const int r2 = m - b * HoWo;
+                ho = magic_div(r2, P.wo_magic, P.wo_shift);
+                wo = r2 - ho * P.Wo;
+            }
+            const int hi0 = ho * P.SH - P.PH, wi0 = wo * P.SW - P.PW;
+            if constexpr (A_FAST) {
+                a_voff[p] = m < P.M ? (uint32_t)(b * P.xs_b + ho * P.SH * P.xs_h + wo * P.SW * P.xs_w + (tid % A_VPR) * 4) * 4u : CONV_OOB;
+                a_inv[p]  = 0u;
+                if (masked) {
+                    uint32_t wbad = 0u;
+                    for (int s = 0; s < P.KW; ++s) wbad |= ((uint32_t)(wi0 + s * P.DW) >= (uint32_t)P.W ? 1u : 0u) << s;
+                    const uint32_t wall = (2u << (P.KW - 1)) - 1u;
+                    for (int r = 0; r < P.KH; ++r)
+                        a_inv[p] |= ((uint32_t)(hi0 + r * P.DH) >= (uint32_t)P.H ? wall : wbad) << (r * P.KW);
+                }
+            } else {
+                a_voff[p] = 0u; a_inv[p] = 0u;
+                a_off0 = b * P.xs_b;
+                a_hi0 = m < P.M ? hi0 : -(1 << 28);
+                a_wi0 = m < P.M ? wi0 : -(1 << 28);
+            }
+        }
+        t_r = 0; t_s = 0; t_c = 0;
+        ak = A_FAST ? (tid % A_VPR) * 4 : (tid / BM) * A_KPT;
         const int rs = ak / P.Cin;
         ac = ak - rs * P.Cin; ar = rs / P.KW; as_ = rs - ar * P.KW;
-    }
+    };
 
     constexpr int B_VPR   = BN / 4;
     constexpr int B_RSTEP = NT / B_VPR;
@@ -336,33 +365,52 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         }
     };
 
-    f32x16 acc[TM][TN];
+    // Calls fn(v, per-lane byte offset, uniform byte offset) for the 16 accumulator elements a
+    // lane holds of sub-tile (i, j) of the M tile at row m0: element v is row 8*(v/4) + 4*half +
+    // v%4, column l32. The offsets are out of range outside the matrix. For a row-major result
+    // one per-lane offset serves all 16 (the row goes into the uniform part, and rows beyond M lie
+    // beyond the descriptor's size). The lane id and the row pitch go through opaque copies so
+    // that this arithmetic is redone at each use instead of occupying registers for the whole
+    // loop. Byte offsets fit 31 bits: the host refuses larger tensors.
+    auto sub_tile = [&](int m0, int i, int j, auto&& fn) {
+        int l = l32;
+        asm volatile("" : "+v"(l));
+        const int n  = n0 + (wn * TN + j) * 32 + l;
+        const int r0 = (wm * TM + i) * 32 + 4 * half;
+        if (c_contig) {
+            const uint32_t base = n < P.N ? (uint32_t)((m0 + r0) * P.N + n) * 4u : CONV_OOB;
+            uint32_t rowb = (uint32_t)P.N * 4u;
+            asm volatile("" : "+s"(rowb));
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+            for (int v = 0; v < 16; ++v) fn(v, base, (uint32_t)(8 * (v / 4) + (v % 4)) * rowb);
+        } else {
+            const int* ro = Rs + r0 + (l - l32);
+            const int  cn = n < P.N ? n * Pk.os_n : -(1 << 30);
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+            for (int v = 0; v < 16; ++v) {
+                const int r = ro[8 * (v / 4) + (v % 4)];
+                fn(v, (r >= 0 && cn >= 0) ? (uint32_t)(r + cn) * 4u : CONV_OOB, 0u);
+            }
+        }
+    };
 
-    const int ktiles = (P.K + BK - 1) / BK;
+    float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
+    // K = 0 runs as one k step whose loads are all out of range
+    const int ktiles = max(1, (P.K + BK - 1) / BK);
+    setup_rows(tile_m0 * BM);
     CONV_STAMP(1)
     load_tiles(0);
     if (tid < BN) {
 #pragma unroll
         for (int e = 0; e < CONV_MAX_EPI; ++e)
-            if (e < nepi) Es[e * BN + tid] = e_reg[e];
+            if (e < nepi) Es[e * BN + tid] = e_reg[e];           // published by the barriers of the first k step
     }
-    if (ktiles == 0) __syncthreads();            // otherwise the barriers of the k loop publish Es
-    for (int kt = 0; kt < ktiles; ++kt) {
-        store_tiles();
-        __syncthreads();
-        if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
-#ifdef CONV_PHASE_STAMPS
-        if (kt == 0) { CONV_STAMP(2) }
-#endif
-        // lanes 0-31 consume the first half of the tile's k range, lanes 32-63 the second half.
-        // Fragments are double-buffered in registers: the LDS reads of group g+1 are in flight
-        // while the MFMAs of group g execute.
+
+    f32x16 acc[TM][TN];
+    // one k step on the tiles in LDS. Lanes 0-31 consume the first half of the tile's k range,
+    // lanes 32-63 the second half. Fragments are double-buffered in registers: the LDS reads of
+    // group g+1 are in flight while the MFMAs of group g execute.
+    auto compute = [&]() {
         constexpr int G = BK / 8;
         f32x4 af[2][TM];
         float bf[2][TN][4];
@@ -388,200 +436,194 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
                     for (int j = 0; j < TN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[g & 1][i][q], bf[g & 1][j][q], acc[i][j], 0, 0, 0);
         }
-        __syncthreads();
-    }
-    CONV_STAMP(3)
-
-    // ---------------- epilogue + store ----------------
-    // accumulator element v of a lane: row = 8*(v/4) + 4*half + v%4, column = l32.
-    // Byte offsets fit 31 bits: the host refuses larger tensors.
-    // Outputs that are not a row-major [M, N] matrix need (batch, y, x) of every row: decoded once
-    // per row into the LDS space of the A tile (free after the k loop), -1 for rows beyond M.
-    int* const row_off = reinterpret_cast<int*>(As);
-    if (!c_contig) {
-        for (int r = tid; r < BM; r += NT) {
-            const int m = m0 + r;
-            const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
-            row_off[r] = m < P.M ? b * Pk.os_b + ho * Pk.os_h + wo * Pk.os_w : -1;
-        }
-        __syncthreads();
-    }
-    // Calls fn(v, per-lane byte offset, uniform byte offset) for the 16 accumulator elements a
-    // lane holds of sub-tile (i, j); the offsets are out of range outside the matrix. For a
-    // row-major result one per-lane offset serves all 16 (the row goes into the uniform part,
-    // and rows beyond M lie beyond the descriptor's size). The lane id goes through an opaque
-    // copy so that this arithmetic is redone at each use instead of occupying registers for
-    // the whole epilogue.
-    auto sub_tile = [&](int i, int j, auto&& fn) {
-        int l = l32;
-        asm volatile("" : "+v"(l));
-        const int n  = n0 + (wn * TN + j) * 32 + l;
-        const int r0 = (wm * TM + i) * 32 + 4 * half;
-        if (c_contig) {
-            const uint32_t base = n < P.N ? (uint32_t)((m0 + r0) * P.N + n) * 4u : CONV_OOB;
-            const uint32_t rowb = (uint32_t)P.N * 4u;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) fn(v, base, (uint32_t)(8 * (v / 4) + (v % 4)) * rowb);
-        } else {
-            const int* ro = row_off + r0 + (l - l32);
-            const int  cn = n < P.N ? n * Pk.os_n : -(1 << 30);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = ro[8 * (v / 4) + (v % 4)];
-                fn(v, (r >= 0 && cn >= 0) ? (uint32_t)(r + cn) * 4u : CONV_OOB, 0u);
-            }
-        }
     };
-    // the first full-size operand (a residual input) is fetched for the whole tile at once
-    // (for the largest tile that would not fit the register file: it loads sub-tile by sub-tile)
-    constexpr bool PREFETCH_FULL = TM * TN <= 2;
-    float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
-    const int first_full = PREFETCH_FULL ? epi_first_full : -1;
-    if (PREFETCH_FULL && first_full >= 0) {
-        const float* fp = epi.p[0];
+
+    for (int sub = 0; sub < nsub; ++sub) {
+        const int m0 = (tile_m0 + sub) * BM;
 #pragma unroll
-        for (int t = 1; t < CONV_MAX_EPI; ++t) fp = first_full == t ? epi.p[t] : fp;
-        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(fp, P.out_bytes);
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = f32x16{};
+        // all k steps but the last: the next step's loads are in flight during the MFMAs
+        for (int kt = 1; kt < ktiles; ++kt) {
+            store_tiles();
+            __syncthreads();
+            load_tiles(kt * BK);
+#ifdef CONV_PHASE_STAMPS
+            if (kt == 1 && sub == 0) { CONV_STAMP(2) }
+#endif
+            compute();
+            __syncthreads();
+        }
+        // last k step: the loads in flight are those of the next M tile's first step and of
+        // the residual operand
+        store_tiles();
+        __syncthreads();
+        if (sub + 1 < nsub) {
+            setup_rows(m0 + BM);
+            load_tiles(0);
+        }
+        if (first_full >= 0) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) {
+                        full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, vo, so);
+                    });
+        }
+        compute();
+        __syncthreads();
+#ifdef CONV_PHASE_STAMPS
+        if (sub == 0) { CONV_STAMP(3) }
+#endif
+
+        // ---------------- epilogue + store of the finished M tile ----------------
+        // Outputs that are not a row-major [M, N] matrix need (batch, y, x) of every row: decoded
+        // once per row into LDS, -1 for rows beyond M.
+        if (!c_contig) {
+            for (int r = tid; r < BM; r += NT) {
+                const int m = m0 + r;
+                const int b = m / HoWo, r2 = m - b * HoWo, ho = r2 / P.Wo, wo = r2 - ho * P.Wo;
+                Rs[r] = m < P.M ? b * Pk.os_b + ho * Pk.os_h + wo * Pk.os_w : -1;
+            }
+            __syncthreads();
+        }
+        // From here on the accumulators are handled as separate scalars: element-wise updates of a
+        // 16-register MFMA tuple make the compiler copy the whole tuple at every step.
+        float c[TM][TN][16];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) {
-                    full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, vo, so);
-                });
-    }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) c[i][j][v] = acc[i][j][v];
 #ifdef CONV_PHASE_STAMPS
-    if (first_full >= 0) { float sink = full[0][0][0]; asm volatile("" :: "v"(sink)); }
-    CONV_STAMP(4)
-#endif
-    // From here on the accumulators are handled as separate scalars: element-wise updates of a
-    // 16-register MFMA tuple make the compiler copy the whole tuple at every step.
-    float c[TM][TN][16];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) c[i][j][v] = acc[i][j][v];
-    // one uniform branch per step and sub-tile, not per element
-    auto apply = [&](uint32_t code, float (&y)[16], auto&& operand) {
-#define EPI_LOOP(expr) _Pragma("unroll") for (int v = 0; v < 16; ++v) { const float a = y[v], o = operand(v); y[v] = (expr); }
-        switch (code) {                                          // bit0: operand on the left
-            case CEW_ADD_F * 2: case CEW_ADD_F * 2 + 1: EPI_LOOP(a + o) break;
-            case CEW_MUL_F * 2: case CEW_MUL_F * 2 + 1: EPI_LOOP(a * o) break;
-            case CEW_SUB_F * 2:     EPI_LOOP(a - o) break;
-            case CEW_SUB_F * 2 + 1: EPI_LOOP(o - a) break;
-            case CEW_DIV_F * 2:     EPI_LOOP(a / o) break;
-            case CEW_DIV_F * 2 + 1: EPI_LOOP(o / a) break;
-            case CEW_MAX_F * 2:     EPI_LOOP((a > o || a != a) ? a : o) break;
-            case CEW_MAX_F * 2 + 1: EPI_LOOP((o > a || o != o) ? o : a) break;
-            case CEW_MIN_F * 2:     EPI_LOOP((a < o || a != a) ? a : o) break;
-            case CEW_MIN_F * 2 + 1: EPI_LOOP((o < a || o != o) ? o : a) break;
-            default: __builtin_unreachable();                    // the host fuses no other operation
+        if (sub == 0) {
+            if (first_full >= 0) { float sink = full[0][0][0]; asm volatile("" :: "v"(sink)); }
+            CONV_STAMP(4)
         }
+#endif
+        const uint32_t slots = (P.flags >> 20) & 31u;
+        if (LEAN || slots) {
+            // The usual chains (bias, batch norm, residual add, ReLU in that order, each optional) run
+            // as straight-line code: every step is one pass over a sub-tile's 16 values, in place.
+            const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u),
+                      e_max = __builtin_popcount(slots & 15u);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    float (&y)[16] = c[i][j];
+                    const int col = (wn * TN + j) * 32 + l32;
+                    // without a prefetched copy the residual operand is requested first and used
+                    // after the per-feature steps
+                    float ov[16];
+                    if ((slots & 8u) && !(PREFETCH_FULL && first_full >= 0))
+                        sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(f_rsrc, vo, so); });
+                    if (slots & 1u) {
+                        const float o = Es[col];
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) y[v] = y[v] - o;
+                    }
+                    if (slots & 2u) {
+                        const float o = Es[e_mul * BN + col];
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) y[v] = y[v] * o;
+                    }
+                    if (slots & 4u) {
+                        const float o = Es[e_add * BN + col];
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) y[v] = y[v] + o;
+                    }
+                    if (slots & 8u) {
+                        if (PREFETCH_FULL && first_full >= 0) {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) y[v] = y[v] + full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v];
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) y[v] = y[v] + ov[v];
+                        }
+                    }
+                    if (slots & 16u) {
+                        const float o = Es[e_max * BN + col];          // the same value in every lane
+                        if (__builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, o != o ? 1.f : 0.f)) == 0) {
+                            // max(y, o) that returns a NaN y, for o known not to be NaN: one compare
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) y[v] = !(y[v] <= o) ? y[v] : o;
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) y[v] = (y[v] > o || y[v] != y[v]) ? y[v] : o;
+                        }
+                    }
+                }
+        } else if constexpr (!LEAN) {
+            // any other chain: one uniform branch per step and sub-tile, not per element
+            auto apply = [&](uint32_t code, float (&y)[16], auto&& operand) {
+#define EPI_LOOP(expr) _Pragma("unroll") for (int v = 0; v < 16; ++v) { const float a = y[v], o = operand(v); y[v] = (expr); }
+                switch (code) {                                          // bit0: operand on the left
+                    case CEW_ADD_F * 2: case CEW_ADD_F * 2 + 1: EPI_LOOP(a + o) break;
+                    case CEW_MUL_F * 2: case CEW_MUL_F * 2 + 1: EPI_LOOP(a * o) break;
+                    case CEW_SUB_F * 2:     EPI_LOOP(a - o) break;
+                    case CEW_SUB_F * 2 + 1: EPI_LOOP(o - a) break;
+                    case CEW_DIV_F * 2:     EPI_LOOP(a / o) break;
+                    case CEW_DIV_F * 2 + 1: EPI_LOOP(o / a) break;
+                    case CEW_MAX_F * 2:     EPI_LOOP((a > o || a != a) ? a : o) break;
+                    case CEW_MAX_F * 2 + 1: EPI_LOOP((o > a || o != o) ? o : a) break;
+                    case CEW_MIN_F * 2:     EPI_LOOP((a < o || a != a) ? a : o) break;
+                    case CEW_MIN_F * 2 + 1: EPI_LOOP((o < a || o != o) ? o : a) break;
+                    default: __builtin_unreachable();                    // the host fuses no other operation
+                }
 #undef EPI_LOOP
-    };
-    const uint32_t slots = (P.flags >> 20) & 31u;
-    if (slots) {
-        // The usual chains (bias, batch norm, residual add, ReLU in that order, each optional) run as
-        // straight-line code: every step is one pass over a sub-tile's 16 values, in place.
-        const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u),
-                  e_res = __builtin_popcount(slots & 7u), e_max = __builtin_popcount(slots & 15u);
-        const float* rp = epi.p[0];
-#pragma unroll
-        for (int t = 1; t < CONV_MAX_EPI; ++t) rp = e_res == t ? epi.p[t] : rp;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                float (&y)[16] = c[i][j];
-                const int col = (wn * TN + j) * 32 + l32;
-                if (slots & 1u) {
-                    const float o = Es[col];
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) y[v] = y[v] - o;
-                }
-                if (slots & 2u) {
-                    const float o = Es[e_mul * BN + col];
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) y[v] = y[v] * o;
-                }
-                if (slots & 4u) {
-                    const float o = Es[e_add * BN + col];
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) y[v] = y[v] + o;
-                }
-                if (slots & 8u) {
-                    if constexpr (PREFETCH_FULL) {
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) y[v] = y[v] + full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v];
-                    } else {
-                        float ov[16];
-                        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(rp, P.out_bytes);
-                        sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(f_rsrc, vo, so); });
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) y[v] = y[v] + ov[v];
-                    }
-                }
-                if (slots & 16u) {
-                    const float o = Es[e_max * BN + col];          // the same value in every lane
-                    if (__builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, o != o ? 1.f : 0.f)) == 0) {
-                        // max(y, o) that returns a NaN y, for o known not to be NaN: one compare
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) y[v] = !(y[v] <= o) ? y[v] : o;
-                    } else {
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) y[v] = (y[v] > o || y[v] != y[v]) ? y[v] : o;
-                    }
-                }
-            }
-    } else {
-    // The step loop stays rolled (one copy of the step code keeps the kernel small enough for the
-    // instruction cache); descriptors and operand pointers are picked with scalar selects.
+            };
+            // The step loop stays rolled: one copy of the step code keeps the kernel small.
 #pragma nounroll
-    for (int e = 0; e < nepi; ++e) {
-        const uint32_t kind = step_desc(e) >> 8;
-        const uint32_t code = step_desc(e) & 255u;
-        const float* ep = epi.p[0];
+            for (int e = 0; e < nepi; ++e) {
+                const uint32_t kind = step_desc(e) >> 8;
+                const uint32_t code = step_desc(e) & 255u;
 #pragma unroll
-        for (int t = 1; t < CONV_MAX_EPI; ++t) ep = e == t ? epi.p[t] : ep;
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        if (kind == 3) {
+                            if (PREFETCH_FULL && e == first_full) {
+                                apply(code, c[i][j], [&](int v) { return full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v]; });
+                            } else {
+                                float ov[16];
+                                // (the pointer table is re-read from the argument block: indexing the by-value
+                                // argument with a run-time value would make the compiler copy it to scratch memory)
+                                const float* const* table = reinterpret_cast<const float* const*>(
+                                    reinterpret_cast<const char*>(__builtin_amdgcn_kernarg_segment_ptr()) + 24);
+                                const __amdgpu_buffer_rsrc_t g_rsrc = make_rsrc(table[e], P.out_bytes);
+                                sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(g_rsrc, vo, so); });
+                                apply(code, c[i][j], [&](int v) { return ov[v]; });
+                            }
+                        } else {
+                            // one value per column: used straight from its register
+                            const float o1 = Es[e * BN + (wn * TN + j) * 32 + l32];
+                            apply(code, c[i][j], [&](int) { return o1; });
+                        }
+                    }
+            }
+        }
+#ifdef CONV_PHASE_STAMPS
+        if (sub == 0) {
+            { float sink = 0; for (int v = 0; v < 16; ++v) sink += c[0][0][v]; asm volatile("" :: "v"(sink)); }
+            CONV_STAMP(5)
+        }
+#endif
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                if (kind == 3) {
-                    if (PREFETCH_FULL && e == first_full) {
-                        apply(code, c[i][j], [&](int v) { return full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v]; });
-                    } else {
-                        float ov[16];
-                        const __amdgpu_buffer_rsrc_t f_rsrc = make_rsrc(ep, P.out_bytes);
-                        sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(f_rsrc, vo, so); });
-                        apply(code, c[i][j], [&](int v) { return ov[v]; });
-                    }
-                } else {
-                    // one value per column: used straight from its register
-                    const float o1 = Es[e * BN + (wn * TN + j) * 32 + l32];
-                    apply(code, c[i][j], [&](int) { return o1; });
-                }
-            }
+            for (int j = 0; j < TN; ++j)
+                sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) { buffer_store_x1(c[i][j][v], o_rsrc, vo, so); });
+        if (!c_contig) __syncthreads();          // Rs is rewritten for the next M tile
 #ifdef CONV_PHASE_STAMPS
-        { float sink = c[0][0][0]; asm volatile("" :: "v"(sink)); const unsigned long long t = wall_clock64();
-          if (e == 0) stamps[8] = t; else if (e == 1) stamps[9] = t; else if (e == 2) stamps[10] = t;
-          else if (e == 3) stamps[11] = t; else if (e == 4) stamps[12] = t; else stamps[13] = t; }
+        if (sub == 0) { CONV_STAMP(6) }
 #endif
     }
-    }
 #ifdef CONV_PHASE_STAMPS
-    { float sink = 0; for (int v = 0; v < 16; ++v) sink += c[0][0][v]; asm volatile("" :: "v"(sink)); }
-    CONV_STAMP(5)
-#endif
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-            sub_tile(i, j, [&](int v, uint32_t vo, uint32_t so) { buffer_store_x1(c[i][j][v], o_rsrc, vo, so); });
-#ifdef CONV_PHASE_STAMPS
-    CONV_STAMP(6)
+    CONV_STAMP(7)
     if (epi.p[CONV_MAX_EPI - 1] != nullptr && tid == 0) {
         unsigned long long* d = (unsigned long long*)epi.p[CONV_MAX_EPI - 1] + (size_t)blockIdx.x * 16;
         for (int q = 0; q < 16; ++q) d[q] = stamps[q];
@@ -589,19 +631,21 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 #endif
 }
 
-#define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF)                                                     \
+#define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF, LEAN)                                               \
     extern "C" __global__ __launch_bounds__(64 * WGM * WGN) __attribute__((amdgpu_waves_per_eu(2))) void name( \
         float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
         ConvEpiPtrs epi, ConvParams P) {                                                                     \
-        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF>(out, x, w, epi, P);                                     \
+        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF, LEAN>(out, x, w, epi, P);                               \
     }
 
-// name = conv_gemm_<BM>x<BN>x<BK>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads)
-#define CONV_TILE(tag, WGM, WGN, TM, TN, BK)                               \
-    CONV_KERNEL(conv_gemm_##tag##_ff, WGM, WGN, TM, TN, BK, true, true)    \
-    CONV_KERNEL(conv_gemm_##tag##_fg, WGM, WGN, TM, TN, BK, true, false)   \
-    CONV_KERNEL(conv_gemm_##tag##_gf, WGM, WGN, TM, TN, BK, false, true)   \
-    CONV_KERNEL(conv_gemm_##tag##_gg, WGM, WGN, TM, TN, BK, false, false)
+// name = conv_gemm_<BM>x<BN>x<BK>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads),
+//        conv_gemm_<BM>x<BN>x<BK>_lean for the common-case variant
+#define CONV_TILE(tag, WGM, WGN, TM, TN, BK)                                      \
+    CONV_KERNEL(conv_gemm_##tag##_lean, WGM, WGN, TM, TN, BK, true, true, true)   \
+    CONV_KERNEL(conv_gemm_##tag##_ff, WGM, WGN, TM, TN, BK, true, true, false)    \
+    CONV_KERNEL(conv_gemm_##tag##_fg, WGM, WGN, TM, TN, BK, true, false, false)   \
+    CONV_KERNEL(conv_gemm_##tag##_gf, WGM, WGN, TM, TN, BK, false, true, false)   \
+    CONV_KERNEL(conv_gemm_##tag##_gg, WGM, WGN, TM, TN, BK, false, false, false)
 
 CONV_TILE(128x128x32, 2, 2, 2, 2, 32)
 CONV_TILE(128x64x32, 2, 2, 2, 1, 32)

@@ -239,6 +239,8 @@ CONV_TILE_BK = {'128x128': (32,), '128x64': (32,), '64x64': (32, 64), '32x32': (
 #tests set these to exercise every kernel variant irrespective of the heuristics
 FORCE_CONV_TILE: tp.Optional[str] = None
 FORCE_CONV_BK:   tp.Optional[int] = None
+FORCE_CONV_CHUNK: tp.Optional[int] = None
+FORCE_CONV_GENERAL = False          #never pick the lean kernel variant
 
 
 def choose_conv_tile(M: int, N: int, compute_units: int = 256):
@@ -256,6 +258,16 @@ def choose_conv_tile(M: int, N: int, compute_units: int = 256):
         if best_time is None or time < best_time:
             best, best_time = (tag, bm, bn, nt), time
     return best
+
+
+def choose_conv_chunk(tiles_m: int, tiles_n: int, compute_units: int = 256) -> int:
+    '''M tiles one block works through. Longer chunks hide more start-up latency (only a block's
+    first tile pays for the argument fetch and the first loads); enough blocks must remain to
+    keep the CUs evenly loaded.'''
+    chunk = 1
+    while chunk < 8 and _cdiv(tiles_m, chunk * 2) * tiles_n >= 12 * compute_units:
+        chunk *= 2
+    return chunk
 
 
 def choose_conv_bk(tag: str, g: 'ConvGeometry') -> int:
@@ -335,14 +347,19 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     b_fast = (g.ws[3] == 1 and N % 4 == 0 and rhs_offset % 4 == 0
               and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
     c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
+    slots = _epilogue_template_slots(epilogue)
+    #the lean kernel variant covers the common case only (see the kernel source)
+    lean = (a_fast and b_fast and c_contig and (g.Cin % bk == 0 or g.KH * g.KW == 1)
+            and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL)
     flat_rows = g.batch == 1 and g.Wo == 1
     tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
+    chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean else 1
     kinds = [e.kind for e in epilogue]
     x_bytes = (lhs.size - lhs_offset) * 4
     w_bytes = K * N * 4 if b_fast else (rhs.size - rhs_offset) * 4
     first_full = kinds.index(3) + 1 if 3 in kinds else 0
     flags = (int(c_contig) | int(flat_rows) << 1 | int(needs_masks) << 2 | len(epilogue) << 8 | first_full << 16
-             | _epilogue_template_slots(epilogue) << 20)
+             | slots << 20 | chunk << 25)
     descs = [0, 0]
     for i, e in enumerate(epilogue):
         assert e.op < 128 and 1 <= e.kind <= 3
@@ -353,9 +370,9 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
               + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os))
     buffers = [(out, 0), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
     buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
-    kernel  = f'conv_gemm_{tag}x{bk}_{"f" if a_fast else "g"}{"f" if b_fast else "g"}'
+    kernel  = f'conv_gemm_{tag}x{bk}_' + ('lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue)
-    return Launch(kernel, (tiles_m * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
+    return Launch(kernel, (_cdiv(tiles_m, chunk) * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
                   bytes_moved=nbytes, flops=2 * M * N * K)
 
 
