@@ -152,6 +152,8 @@ def main():
                         launches_per_step=d['launches'] // args.profile_iters,
                         avg_launch_ms=round(d['ms'] / d['launches'], 5))
 
+    roofline['traffic'] = measured_hbm_traffic(args.workload, dominant)
+
     cpu_baseline = None
     if not args.no_cpu_baseline:
         cpu_baseline = time_cpu_baseline(args.workload, fn, make_inputs, kwargs)
@@ -168,6 +170,20 @@ def main():
         'roofline': roofline, 'kernels': kernels, 'cpu_baseline': cpu_baseline,
     }
     print(json.dumps(out))
+
+
+def measured_hbm_traffic(workload, family):
+    '''HBM bytes per launch of the dominant kernel family from the hardware-counter passes
+    (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each scaled by what the counter reads for a plain
+    copy of known size), as recorded in the committed summary of that profile; None if there is none.
+    Counters cannot be collected from inside this process.'''
+    import glob, re
+    here = os.path.dirname(os.path.abspath(__file__))
+    for path in sorted(glob.glob(os.path.join(here, 'profiles', f'*{workload}*.txt'))):
+        m = re.search(rf'^hbm_traffic_bytes_per_launch {re.escape(family)} (\d+)', open(path).read(), re.M)
+        if m:
+            return int(m.group(1))
+    return None
 
 
 def time_cpu_baseline(workload, fn, make_inputs, kwargs):
