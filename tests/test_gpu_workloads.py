@@ -51,6 +51,35 @@ def test_rng_small_and_full_bit_exact():
     assert 0.0 <= y.min() and y.max() < 1.0 and abs(y.mean() - 0.5) < 1e-3
 
 
+def test_random_stream_fusion_variants_bit_exact():
+    '''The fused counter + block function + concatenate + chain launch against the oracle's
+    one-primitive-at-a-time evaluation: lengths that are and are not multiples of 8 (16-byte and
+    4-byte stores), odd lengths (the legacy layout pads the counters and trims the result, which
+    keeps the chain a launch of its own), a range given at run time (scalar operands read from
+    device memory), raw bits, and a split feeding two draws.'''
+    from vkjax_amd.minijax import random as mrandom
+    key = W.rng_inputs()
+
+    def ranged(key, lo, hi):
+        u = mrandom.uniform(key, (64, 48))
+        return u * (hi - lo) + lo
+
+    def two_draws(key):
+        k1, k2 = mrandom.split(key)
+        return mrandom.uniform(k1, (24,)), mrandom.random_bits(k2, (6, 4))
+
+    cases = [(lambda key: mrandom.uniform(key, (40,)), key), (lambda key: mrandom.uniform(key, (6,)), key),
+             (lambda key: mrandom.uniform(key, (7, 3)), key), (lambda key: mrandom.uniform(key, (1,)), key),
+             (lambda key: mrandom.random_bits(key, (128,)), key), (lambda key: mrandom.uniform(key, (16, 8), minval=-3.0, maxval=5.0), key),
+             (ranged, list(key) + [np.float32(-2.0), np.float32(7.5)]), (two_draws, key)]
+    for i, (f, args) in enumerate(cases):
+        _, _, fn = check_against_oracle(f, args, exact=True)
+        kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+        if i not in (2, 3):                       #odd lengths keep the unfused launches
+            assert any(k.startswith('threefry2x32_stream') for k in kernels), kernels
+            assert not any(k.startswith(('iota', 'concat')) for k in kernels), kernels
+
+
 def test_gather_scatter_small_exact_and_full():
     #integer-valued updates make the atomic sums exact whatever their order
     rng = np.random.default_rng(0)

@@ -59,7 +59,7 @@ def build_shim(force=True):
 
 def build_kernel(name, force=True):
     src  = os.path.join(CSRC, 'kernels', f'{name}.hip')
-    deps = [src] + [os.path.join(CSRC, 'kernels', h) for h in ('common.h', 'ew_opcodes.h')]
+    deps = [src] + [os.path.join(CSRC, 'kernels', h) for h in ('common.h', 'ew_opcodes.h', 'ew_apply.h')]
     out  = hsaco_path(name)
     if not force and _newer(out, deps):
         return out

@@ -3,7 +3,7 @@
 // elements. 16 bytes per lane on each side when the length allows; pure integer ALU work,
 // bandwidth-bound. Supersedes vkjax/shaders/threefry2x32.comp (reference: vkjax/ops.py:550-560,
 // vkjax/shaders/threefry2x32.comp:38-91).
-#include "common.h"
+#include "ew_apply.h"
 
 struct ThreefryParams { uint32_t n, key_is_scalar; };
 
@@ -71,4 +71,76 @@ extern "C" __global__ __launch_bounds__(256) void threefry2x32_v1(uint32_t* out0
 extern "C" __global__ __launch_bounds__(256) void threefry2x32_v4(uint32_t* out0, uint32_t* out1, const uint32_t* key0, const uint32_t* key1,
                                                                   const uint32_t* in0, const uint32_t* in1, ThreefryParams P) {
     threefry_body<4>(out0, out1, key0, key1, in0, in1, P);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The whole random-bits pipeline in one pass. JAX (legacy counter layout) draws 2h words as
+//     c = iota(2h);  a, b = threefry2x32(key, c[:h], c[h:]);  bits = concatenate(a, b)
+// and then maps the bits through a chain of element-wise steps with scalar operands
+// (uniform: bits >> 9 | 0x3F800000, bitcast, - 1, * (max - min), + min, max(min, .)).
+// Here every thread generates its counters in registers (x0 = c0 + j, x1 = c1 + j), runs the block
+// function, applies the chain to both results and writes element j and element h + j of the final
+// array: 4 bytes written per element and nothing read, instead of twelve full-size passes.
+#define TF_MAX_STEPS 8
+
+struct ThreefryStreamParams {
+    uint32_t h;                        // elements per half: the output has 2h
+    uint32_t c0, c1;                   // first counter of each half
+    uint32_t nsteps;                   // element-wise steps applied to the bits (0..8)
+    uint32_t op[TF_MAX_STEPS];         // opcode of step k
+    uint32_t flags[TF_MAX_STEPS];      // bit0: the step has an operand (a single value); bit1: it is the LEFT argument
+    uint32_t imm[TF_MAX_STEPS];        // immediate of step k (integer_pow exponent)
+};
+
+struct ThreefryStreamPtrs { const uint32_t* p[TF_MAX_STEPS]; };
+
+template <int VEC>
+__device__ __forceinline__ void threefry_stream_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ key0,
+                                                     const uint32_t* __restrict__ key1, const ThreefryStreamPtrs& operands,
+                                                     const ThreefryStreamParams& P) {
+    const uint32_t j0 = (blockIdx.x * 256u + threadIdx.x) * VEC;
+    if (j0 >= P.h) return;
+    const uint32_t k0 = key0[0], k1 = key1[0];
+    uint32_t y[2 * VEC];                             // [0, VEC): first results, [VEC, 2 VEC): second results
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        y[j]       = P.c0 + j0 + j;
+        y[VEC + j] = P.c1 + j0 + j;
+        threefry_block(k0, k1, y[j], y[VEC + j]);
+    }
+    // The step loop stays rolled (one copy of the opcode switch). Its descriptors are read from the
+    // argument block through the kernel-argument pointer: indexing the by-value argument with a
+    // run-time value would make the compiler copy it to scratch memory. Layout of the block:
+    // out, key0, key1 (24 bytes), the operand pointers (64 bytes), then ThreefryStreamParams.
+    const char* const args = reinterpret_cast<const char*>(__builtin_amdgcn_kernarg_segment_ptr());
+    const uint32_t* const* const op_ptr = reinterpret_cast<const uint32_t* const*>(args + 24);
+    const uint32_t* const desc = reinterpret_cast<const uint32_t*>(args + 24 + 8 * TF_MAX_STEPS) + 4;
+#pragma nounroll
+    for (uint32_t k = 0; k < P.nsteps; ++k) {
+        const uint32_t op = desc[k], flags = desc[TF_MAX_STEPS + k], imm = desc[2 * TF_MAX_STEPS + k];
+        const uint32_t o = (flags & 1u) ? op_ptr[k][0] : 0u;                  // uniform address: a scalar load
+        uint32_t v[2 * VEC];
+#pragma unroll
+        for (int j = 0; j < 2 * VEC; ++j) v[j] = o;
+        ew_apply_vec<2 * VEC>(op, y, v, (flags & 2u) != 0, imm);
+    }
+    if constexpr (VEC == 4) {
+        u32x4 va, vb;
+        va.x = y[0]; va.y = y[1]; va.z = y[2]; va.w = y[3];
+        vb.x = y[4]; vb.y = y[5]; vb.z = y[6]; vb.w = y[7];
+        *reinterpret_cast<u32x4*>(out + j0) = va;
+        *reinterpret_cast<u32x4*>(out + P.h + j0) = vb;
+    } else {
+        out[j0] = y[0]; out[P.h + j0] = y[1];
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) void threefry2x32_stream_v1(uint32_t* out, const uint32_t* key0, const uint32_t* key1,
+                                                                         ThreefryStreamPtrs operands, ThreefryStreamParams P) {
+    threefry_stream_body<1>(out, key0, key1, operands, P);
+}
+// requires h % 4 == 0 and a 16-byte aligned output
+extern "C" __global__ __launch_bounds__(256) void threefry2x32_stream_v4(uint32_t* out, const uint32_t* key0, const uint32_t* key1,
+                                                                         ThreefryStreamPtrs operands, ThreefryStreamParams P) {
+    threefry_stream_body<4>(out, key0, key1, operands, P);
 }

@@ -39,6 +39,13 @@ def _reads(op) -> tp.List:
     if op.conv is not None:
         out, lhs, rhs, geom, epilogue = op.conv
         return [lhs, rhs] + [e.operand for e in epilogue]
+    if op.meta is not None:
+        if op.meta[0] == 'iota':
+            return []
+        if op.meta[0] == 'concat_part':
+            return [op.meta[2]]
+        if op.meta[0] == 'threefry':
+            return list(op.meta[2])
     return [b for b, _ in op.launch.buffers if b is not None]
 
 
@@ -156,4 +163,169 @@ def fuse_ops(all_ops, bufferpool, outvars):
         out = _out(new)
         if out is not None:
             producer[id(out._placeholder)] = len(result) - 1
-    return [op for op in result if op is not None]
+    ops = fuse_random_streams([op for op in result if op is not None], bufferpool, outvars)
+    return remove_dead_ops(ops, bufferpool, outvars)
+
+
+def _writes(op) -> tp.List:
+    if op.chain is not None or op.conv is not None:
+        return [_out(op)]
+    if op.meta is not None and op.meta[0] in ('iota', 'concat_part'):
+        return [op.meta[1]]
+    if op.meta is not None and op.meta[0] == 'threefry':
+        return list(op.meta[1])
+    return [b for b, _ in op.launch.buffers[:1] if b is not None]      #kernels write their first argument
+
+
+def remove_dead_ops(ops, bufferpool, outvars):
+    '''Drops launches none of whose results is read by a later launch or returned (the unused half
+    of a PRNG key split, for instance). The reference runs every equation; the values returned
+    are the same.'''
+    ops = list(ops)
+    while True:
+        uses = _use_counts(ops, bufferpool, outvars)
+        #an accumulating kernel (scatter-add) also reads what it writes: such a use does not keep it alive
+        dead = [i for i, op in enumerate(ops)
+                if _writes(op) and all(uses[id(b._placeholder)] - sum(1 for r in _reads(op) if r._placeholder is b._placeholder) == 0
+                                       for b in _writes(op))
+                and not any(sum(1 for o in ops if any(w._placeholder is b._placeholder for w in _writes(o))) > 1 for b in _writes(op))]
+        if not dead:
+            return ops
+        for i in dead:
+            for b in _writes(ops[i]):
+                b._placeholder.elided = True
+        ops = [op for i, op in enumerate(ops) if i not in set(dead)]
+
+
+def _use_counts(ops, bufferpool, outvars):
+    uses = collections.Counter()
+    for op in ops:
+        for b in _reads(op):
+            uses[id(b._placeholder)] += 1
+    for v in outvars:
+        b = bufferpool.get_buffer(v)
+        if b is not None:
+            uses[id(b._placeholder)] += 2
+            b.accesses.pop()
+    return uses
+
+
+def fuse_random_streams(ops, bufferpool, outvars):
+    '''Collapses the random-bits pipeline into one launch:
+
+        c = iota(2h); a, b = threefry2x32(key, c[:h], c[h:]); bits = concatenate(a, b); out = chain(bits)
+
+    where `chain` is an element-wise chain whose operands are single values (jax.random.uniform's
+    shift / or / bitcast / sub / mul / add / max). The fused kernel generates the counters in
+    registers and applies the chain before its only store, so of the iota, the two slices, the
+    block function, the two concatenate copies and the chain only one write of the result remains.
+    The arithmetic per element is unchanged.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    writers = collections.defaultdict(list)          #placeholder id -> positions of the ops that write it
+    for i, op in enumerate(ops):
+        if op.chain is not None or op.conv is not None:
+            writers[pid(_out(op))].append(i)
+        elif op.meta is not None and op.meta[0] == 'iota':
+            writers[pid(op.meta[1])].append(i)
+        elif op.meta is not None and op.meta[0] == 'concat_part':
+            writers[pid(op.meta[1])].append(i)
+        elif op.meta is not None and op.meta[0] == 'threefry':
+            for b in op.meta[1]:
+                writers[pid(b)].append(i)
+        else:
+            for b, _ in op.launch.buffers[:1]:       #kernels write their first argument
+                if b is not None:
+                    writers[pid(b)].append(i)
+    removed = set()
+    replacement = {}
+    for ti, T in enumerate(ops):
+        if T.meta is None or T.meta[0] != 'threefry' or not T.meta[3]:
+            continue
+        (aa, ab), (key0, key1, x0, x1), _ = T.meta[1:]
+        h = x0.size
+        if aa.size != h or len(aa.shape) != 1:
+            continue
+        #counters: contiguous slices of one-dimensional uint32 iotas
+        sources = []
+        for xb in (x0, x1):
+            w = writers.get(pid(xb), [])
+            if len(w) != 1 or uses[pid(xb)] != 1:
+                break
+            C = ops[w[0]]
+            if C.chain is None or C.chain.steps or len(C.chain.shape) != 1 or tuple(C.chain.first.strides) != (1,):
+                break
+            S  = C.chain.first.buffer
+            ws = writers.get(pid(S), [])
+            if len(ws) != 1 or ops[ws[0]].meta is None or ops[ws[0]].meta[0] != 'iota' or len(S.shape) != 1 or S.dtype != 'uint32':
+                break
+            sources.append((w[0], C.chain.first.offset, ws[0], S))
+        if len(sources) != 2:
+            continue
+        #results: concatenated in order into one array
+        if uses[pid(aa)] != 1 or uses[pid(ab)] != 1:
+            continue
+        cats = [i for i, op in enumerate(ops) if op.meta is not None and op.meta[0] == 'concat_part'
+                and op.meta[2]._placeholder in (aa._placeholder, ab._placeholder)]
+        if len(cats) != 2:
+            continue
+        m0, m1 = ops[cats[0]].meta, ops[cats[1]].meta
+        if m0[2]._placeholder is not aa._placeholder:
+            m0, m1 = m1, m0
+        AC = m0[1]
+        if (m0[2]._placeholder is not aa._placeholder or m1[2]._placeholder is not ab._placeholder or m1[1]._placeholder is not AC._placeholder
+                or len(AC.shape) != 1 or AC.size != 2 * h or (m0[3], m0[4], m1[3], m1[4]) != (0, 0, 0, h)
+                or sorted(writers[pid(AC)]) != sorted(cats)):
+            continue
+        #an element-wise chain on the bits whose operands are single values
+        chain_pos = None
+        if uses[pid(AC)] == 1:
+            for i in range(max(cats) + 1, len(ops)):
+                op = ops[i]
+                if any(b._placeholder is AC._placeholder for b in _reads(op)):
+                    ch = op.chain
+                    n  = 1
+                    for d in (ch.shape if ch is not None else ()):
+                        n *= d
+                    if (ch is not None and ch.first.buffer._placeholder is AC._placeholder and ch.first.offset == 0 and n == 2 * h
+                            and tuple(ch.first.strides) == K.row_major_strides(ch.shape) and len(ch.steps) <= K.TF_MAX_STEPS
+                            and all(st.op not in _SELECTS and st.op != EW['NOP'] and
+                                    (st.operand is None or (st.operand.buffer.size == 1 and st.operand.offset == 0)) for st in ch.steps)):
+                        chain_pos = i
+                    break
+        members = [sources[0][0], sources[1][0], ti] + cats + ([chain_pos] if chain_pos is not None else [])
+        if removed & set(members):
+            continue
+        last  = max(members)
+        out   = ops[chain_pos].chain.out if chain_pos is not None else AC
+        steps = list(ops[chain_pos].chain.steps) if chain_pos is not None else []
+        #a key word that is a one-element copy out of another array is read from there
+        keys = []
+        for kb in (key0, key1):
+            w = writers.get(pid(kb), [])
+            C = ops[w[0]] if len(w) == 1 else None
+            if (C is not None and C.chain is not None and not C.chain.steps and kb.size == 1 and w[0] not in removed
+                    and C.chain.first.buffer.dtype == kb.dtype):
+                keys.append((C.chain.first.buffer, C.chain.first.offset))
+                if uses[pid(kb)] == 1:
+                    members.append(w[0])
+                    kb._placeholder.elided = True
+            else:
+                keys.append((kb, 0))
+        fused = Op(_label(*[ops[i] for i in sorted(members)]),
+                   launch=K.threefry_stream(out, keys[0], keys[1], h, sources[0][1], sources[1][1], steps))
+        fused.index = ops[last].index
+        for b in [keys[0][0], keys[1][0]] + [st.operand.buffer for st in steps if st.operand is not None]:
+            b.accesses.append(fused.index)
+        for b in (x0, x1, aa, ab) + ((AC,) if chain_pos is not None else ()):
+            b._placeholder.elided = True
+        removed |= set(members)
+        replacement[last] = fused
+        #an iota nobody reads any more goes too
+        for _, _, si, S in sources:
+            uses[pid(S)] -= 1
+            if uses[pid(S)] == 0 and si not in removed:
+                removed.add(si)
+                S._placeholder.elided = True
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed or i in replacement]

@@ -205,6 +205,30 @@ def concat_part(out: Buffer, part: Buffer, dimension: int, offset_along_dim: int
                   _u32(n, part_inner, out_inner, offset_along_dim * inner), bytes_moved=8 * n)
 
 
+TF_MAX_STEPS = 8
+
+
+def threefry_stream(out: Buffer, key0: tp.Tuple[Buffer, int], key1: tp.Tuple[Buffer, int], h: int, c0: int, c1: int,
+                    steps: tp.Sequence[EwStep]) -> Launch:
+    '''out[j], out[h + j] = steps(threefry2x32(key, c0 + j, c1 + j)) for j < h: counters generated in
+    registers, the element-wise `steps` (operands: single values) applied before the only store.
+    The key words are given as (buffer, element offset).'''
+    if len(steps) > TF_MAX_STEPS:
+        raise ValueError('too many steps')
+    flags, buffers = [], []
+    for s in steps:
+        if s.operand is not None:
+            assert s.operand.buffer.size == 1 and s.operand.offset == 0
+        flags.append((1 if s.operand is not None else 0) | (2 if s.operand_left else 0))
+        buffers.append((s.operand.buffer if s.operand is not None else None, 0))
+    vec = 4 if h % 4 == 0 else 1
+    params = _u32(h, c0, c1, len(steps), *_pad([s.op for s in steps], TF_MAX_STEPS), *_pad(flags, TF_MAX_STEPS),
+                  *_pad([s.imm for s in steps], TF_MAX_STEPS))
+    return Launch(f'threefry2x32_stream_v{vec}', (_cdiv(_cdiv(h, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                  [(out, 0), (key0[0], key0[1] * 4), (key1[0], key1[1] * 4)] + _pad(buffers, TF_MAX_STEPS, (None, 0)), params,
+                  bytes_moved=8 * h)
+
+
 # --------------------------------------------------------------------------- conv / dot
 
 class ConvGeometry(tp.NamedTuple):

@@ -29,10 +29,11 @@ class Op:
     order (entries can be None), `shader` names the kernel, `equation` is the jaxpr equation it
     came from (or a label string for helper launches), as in the reference's Op tuple
     (vkjax/ops.py:28-41).'''
-    __slots__ = ('equation', 'chain', '_launch', 'conv', 'index')
+    __slots__ = ('equation', 'chain', '_launch', 'conv', 'index', 'meta')
 
-    def __init__(self, equation, launch: tp.Optional[Launch] = None, chain: tp.Optional[EwChain] = None, conv=None):
+    def __init__(self, equation, launch: tp.Optional[Launch] = None, chain: tp.Optional[EwChain] = None, conv=None, meta=None):
         self.equation = equation
+        self.meta     = meta          #(kind, ...) structure of a plain launch that a fusion pass may want to recognise
         self.chain    = chain
         self._launch  = launch
         self.conv     = conv          #(out, lhs, rhs, geometry, epilogue list) for conv/dot ops, so a fusion pass can extend it
@@ -343,7 +344,7 @@ def iota(bufferpool, equation):
     outbuf = bufferpool.get_buffer(outvar, increment_op_counter=True)
     if _kind(outbuf.dtype) == _B:
         raise NotImplementedError(equation)
-    return [Op(equation, launch=K.iota(outbuf, dimension))]
+    return [Op(equation, launch=K.iota(outbuf, dimension), meta=('iota', outbuf, dimension))]
 
 
 def concatenate(bufferpool, equation):
@@ -356,7 +357,7 @@ def concatenate(bufferpool, equation):
     ops, offset = [], 0
     for b in inbufs:
         if b.size:
-            ops.append(Op(equation, launch=K.concat_part(outbuf, b, dim, offset)))
+            ops.append(Op(equation, launch=K.concat_part(outbuf, b, dim, offset), meta=('concat_part', outbuf, b, dim, offset)))
         offset += b.shape[dim]
     return ops
 
@@ -613,7 +614,8 @@ def threefry2x32(bufferpool, equation):
         assert inbufs[0].shape == inbufs[2].shape
     if outbufs[0].size == 0:
         return []
-    return [Op(equation, launch=K.threefry2x32(*outbufs, *inbufs, key_is_scalar=key_is_scalar))]
+    return [Op(equation, launch=K.threefry2x32(*outbufs, *inbufs, key_is_scalar=key_is_scalar),
+               meta=('threefry', outbufs, inbufs, key_is_scalar))]
 
 
 import builtins as _builtins
