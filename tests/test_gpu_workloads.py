@@ -96,6 +96,38 @@ def test_gather_scatter_small_exact_and_full():
     assert np.allclose(acc, expected, rtol=1e-5, atol=1e-6)
 
 
+def test_scatter_add_rows_sorted_and_atomic_paths():
+    '''Row scatter-add through both implementations (bucketed by a counting sort of the indices,
+    and HBM atomics): integer-valued updates make every sum exact; cases cover rows that receive no
+    update, one row that receives more than 64, indices outside the table (dropped), a row length
+    that is not a multiple of 4, integer data and an operand that is not zero.'''
+    from vkjax_amd import ops
+    rng = np.random.default_rng(7)
+
+    def scatter(table, idx, updates):
+        return mj.numpy.index_add(table, idx, updates)
+
+    saved = ops.SCATTER_SORT_THRESHOLD
+    try:
+        for threshold in (0, 1 << 60):
+            ops.SCATTER_SORT_THRESHOLD = threshold
+            for rows, cols, n, dtype in ((50, 256, 400, np.float32), (9, 10, 37, np.float32), (300, 64, 200, np.int32), (4, 20, 500, np.float32)):
+                table   = rng.integers(-9, 9, size=(rows, cols)).astype(dtype)
+                idx     = rng.integers(0, rows, size=(n,)).astype(np.int32)
+                idx[: n // 3] = idx[0]                                 #one crowded row
+                updates = rng.integers(-5, 6, size=(n, cols)).astype(dtype)
+                _, _, fn = check_against_oracle(scatter, [table, idx, updates], exact=True)
+                kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+                assert any(k.startswith('scatter_rows_sum') for k in kernels) == (threshold == 0), kernels
+            #indices beyond the table (jnp's normalisation only wraps negative ones)
+            table   = np.zeros((16, 8), np.float32)
+            idx     = np.array([3, 99, 16, 15, -1, 3], np.int32)
+            updates = rng.integers(-5, 6, size=(6, 8)).astype(np.float32)
+            check_against_oracle(scatter, [table, idx, updates], exact=True)
+    finally:
+        ops.SCATTER_SORT_THRESHOLD = saved
+
+
 def test_fusion_does_not_change_a_single_bit():
     '''The fused program (chains merged, batch-norm / ReLU / residual in the convolution epilogue)
     performs the same fp32 operations in the same order as one launch per equation.'''

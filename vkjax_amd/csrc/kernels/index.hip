@@ -98,6 +98,213 @@ extern "C" __global__ __launch_bounds__(256) void scatter_add_rows(uint32_t* __r
     else atomicAdd(dst, u);
 }
 
+// ---------------------------------------------------------------------------------------------
+// scatter-add of whole rows without atomics on the data: the update rows are bucketed by target
+// row with a counting sort of their indices (three small launches over the indices), then one
+// wave per table row adds up its updates, in ascending update order, on top of the operand row and
+// writes the result once. Every update row is read exactly once, the table is read once and
+// written once, and the sum does not depend on the order in which threads happen to run (rows
+// that receive more than 64 updates are summed in blocks of 64, each block in ascending order).
+struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride; };
+
+// count[r + 1] += 1 for every in-range index; count has n_rows + 1 words and starts at zero
+extern "C" __global__ __launch_bounds__(256) void scatter_rows_count(uint32_t* __restrict__ count, const int32_t* __restrict__ idx,
+                                                                     ScatterSortParams P) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= P.n_idx) return;
+    const int32_t r = idx[(uint64_t)i * P.idx_stride];
+    if (r < 0 || r >= (int32_t)P.n_rows) return;          // updates outside the operand are dropped
+    atomicAdd(count + r + 1, 1u);
+}
+
+// in-place inclusive prefix sum over n words by one block: afterwards word r is the number of
+// updates that go to rows before r, i.e. where row r's bucket starts. The block walks the array
+// in tiles of 1024 x 16 words; a thread scans 16 consecutive words, the 1024 thread totals are
+// scanned with wave shuffles and one exchange through LDS, and a running carry links the tiles.
+extern "C" __global__ __launch_bounds__(1024) void scatter_rows_scan(uint32_t* __restrict__ data, uint32_t n) {
+    __shared__ uint32_t wave_total[16];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t carry = 0;
+    for (uint32_t tile = 0; tile < n; tile += 1024u * 16u) {
+        const uint32_t base = tile + threadIdx.x * 16u;
+        uint32_t v[16];
+        if (base + 16u <= n) {                                   // 64 aligned bytes per thread
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const u32x4 t4 = *reinterpret_cast<const u32x4*>(data + base + 4 * q);
+                v[4 * q] = t4.x; v[4 * q + 1] = t4.y; v[4 * q + 2] = t4.z; v[4 * q + 3] = t4.w;
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) v[q] = base + q < n ? data[base + q] : 0u;
+        }
+#pragma unroll
+        for (int q = 1; q < 16; ++q) v[q] += v[q - 1];
+        // inclusive scan of the thread totals across the wave
+        uint32_t t = v[15];
+#pragma unroll
+        for (uint32_t off = 1; off < 64u; off <<= 1) {
+            const uint32_t up = __shfl_up(t, off, 64);
+            if (lane >= off) t += up;
+        }
+        if (lane == 63u) wave_total[wave] = t;
+        __syncthreads();
+        uint32_t before = carry;                                 // everything before this thread's 16 words
+        for (uint32_t w = 0; w < wave; ++w) before += wave_total[w];
+        before += t - v[15];
+        uint32_t tile_total = 0;
+        for (uint32_t w = 0; w < 16u; ++w) tile_total += wave_total[w];
+        __syncthreads();                                         // wave_total is rewritten by the next tile
+        if (base + 16u <= n) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                u32x4 t4;
+                t4.x = v[4 * q] + before; t4.y = v[4 * q + 1] + before; t4.z = v[4 * q + 2] + before; t4.w = v[4 * q + 3] + before;
+                *reinterpret_cast<u32x4*>(data + base + 4 * q) = t4;
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+                if (base + q < n) data[base + q] = v[q] + before;
+        }
+        carry += tile_total;
+    }
+}
+
+// order[start[r] + k] = i for the k-th update (in order of arrival) whose index is r; cursor starts at zero
+extern "C" __global__ __launch_bounds__(256) void scatter_rows_fill(uint32_t* __restrict__ order, uint32_t* __restrict__ cursor,
+                                                                    const uint32_t* __restrict__ start, const int32_t* __restrict__ idx,
+                                                                    ScatterSortParams P) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= P.n_idx) return;
+    const int32_t r = idx[(uint64_t)i * P.idx_stride];
+    if (r < 0 || r >= (int32_t)P.n_rows) return;
+    order[start[r] + atomicAdd(cursor + r, 1u)] = i;
+}
+
+// ascending bitonic sort of one value per lane across the wave
+__device__ __forceinline__ uint32_t wave_sort(uint32_t e, uint32_t lane) {
+#pragma unroll
+    for (uint32_t k = 2; k <= 64u; k <<= 1) {
+#pragma unroll
+        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+            const uint32_t partner = __shfl_xor(e, j, 64);
+            const bool keep_min = ((lane & k) == 0u) == ((lane & j) == 0u);
+            e = keep_min ? min(e, partner) : max(e, partner);
+        }
+    }
+    return e;
+}
+
+// out[r, :] = operand[r, :] + sum over the updates i in row r's bucket of updates[i, :].
+// One wave takes 4 consecutive rows. Their buckets are adjacent in `order`, so one load fetches
+// them all (up to 64 entries, the usual case); they are sorted together under the key
+// (row, update number), and all the rows' loads of operand and update data are in flight together.
+// A wave whose rows hold more than 64 entries falls back to one row at a time, 64 entries at a time.
+// Update numbers are below 2^30 (the host sees to that).
+#define SCATTER_ROWS_PER_WAVE 4
+template <int VEC, bool IS_FLOAT>
+__device__ __forceinline__ void scatter_rows_sum_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ operand,
+                                                      const uint32_t* __restrict__ updates, const uint32_t* __restrict__ start,
+                                                      const uint32_t* __restrict__ order, const ScatterSortParams& P) {
+    constexpr int ROWS = SCATTER_ROWS_PER_WAVE;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t r0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * ROWS;
+    if (r0 >= P.n_rows) return;
+    auto add = [](uint32_t a, uint32_t b) -> uint32_t { return IS_FLOAT ? f2u(u2f(a) + u2f(b)) : a + b; };
+    // bucket boundaries: s[j] .. s[j + 1] for row r0 + j (rows beyond the table get empty buckets)
+    const uint32_t sv = start[min(r0 + lane, P.n_rows)];
+    uint32_t s[ROWS + 1];
+#pragma unroll
+    for (int j = 0; j <= ROWS; ++j) s[j] = __builtin_amdgcn_readlane(sv, j);
+    const uint32_t total = s[ROWS] - s[0];
+
+    auto load_row = [&](const uint32_t* base, uint32_t row, uint32_t c, uint32_t (&dst)[VEC]) {
+        if constexpr (VEC == 4) {
+            const u32x4 t = *reinterpret_cast<const u32x4*>(base + (uint64_t)row * P.row_len + c);
+            dst[0] = t.x; dst[1] = t.y; dst[2] = t.z; dst[3] = t.w;
+        } else {
+            dst[0] = base[(uint64_t)row * P.row_len + c];
+        }
+    };
+    auto store_row = [&](uint32_t row, uint32_t c, const uint32_t (&src)[VEC]) {
+        if constexpr (VEC == 4) {
+            u32x4 t; t.x = src[0]; t.y = src[1]; t.z = src[2]; t.w = src[3];
+            *reinterpret_cast<u32x4*>(out + (uint64_t)row * P.row_len + c) = t;
+        } else {
+            out[(uint64_t)row * P.row_len + c] = src[0];
+        }
+    };
+    // acc += updates[e(k), c ...] for k in [k0, k1), four rows requested at a time and added in order;
+    // e holds the (sorted) update numbers, one per lane
+    auto accumulate = [&](uint32_t e, uint32_t k0, uint32_t k1, uint32_t c, bool live, uint32_t (&acc)[VEC]) {
+        for (uint32_t k = k0; k < k1; k += 4u) {
+            uint32_t t[4][VEC];
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q)
+                if (k + q < k1 && live) load_row(updates, __builtin_amdgcn_readlane(e, k + q) & 0x3FFFFFFFu, c, t[q]);
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q)
+                if (k + q < k1 && live) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = add(acc[v], t[q][v]);
+                }
+        }
+    };
+
+    if (total <= 64u) {
+        uint32_t e = 0xFFFFFFFFu;
+        if (lane < total) {
+            uint32_t row = 0;
+#pragma unroll
+            for (int j = 1; j < ROWS; ++j) row += lane >= s[j] - s[0] ? 1u : 0u;
+            e = order[s[0] + lane] | row << 30;
+        }
+        if (total > 1u) e = wave_sort(e, lane);
+        for (uint32_t c0 = 0; c0 < P.row_len; c0 += 64u * VEC) {
+            const uint32_t c = c0 + lane * VEC;
+            const bool live = c < P.row_len;                   // row_len is a multiple of VEC
+            uint32_t acc[ROWS][VEC];
+#pragma unroll
+            for (int j = 0; j < ROWS; ++j)
+                if (live && r0 + j < P.n_rows) load_row(operand, r0 + j, c, acc[j]);
+#pragma unroll
+            for (int j = 0; j < ROWS; ++j) accumulate(e, s[j] - s[0], s[j + 1] - s[0], c, live, acc[j]);
+#pragma unroll
+            for (int j = 0; j < ROWS; ++j)
+                if (live && r0 + j < P.n_rows) store_row(r0 + j, c, acc[j]);
+        }
+    } else {
+        for (uint32_t j = 0; j < (uint32_t)ROWS && r0 + j < P.n_rows; ++j) {
+            const uint32_t begin = __builtin_amdgcn_readlane(sv, j), end = __builtin_amdgcn_readlane(sv, j + 1);
+            for (uint32_t c0 = 0; c0 < P.row_len; c0 += 64u * VEC) {
+                const uint32_t c = c0 + lane * VEC;
+                const bool live = c < P.row_len;
+                uint32_t acc[VEC];
+                if (live) load_row(operand, r0 + j, c, acc);
+                for (uint32_t b0 = begin; b0 < end; b0 += 64u) {
+                    const uint32_t cnt = min(64u, end - b0);
+                    uint32_t e = lane < cnt ? order[b0 + lane] : 0xFFFFFFFFu;
+                    if (cnt > 1u) e = wave_sort(e, lane);
+                    accumulate(e, 0u, cnt, c, live, acc);
+                }
+                if (live) store_row(r0 + j, c, acc);
+            }
+        }
+    }
+}
+
+#define SCATTER_SUM_KERNEL(name, VEC, IS_FLOAT)                                                                   \
+    extern "C" __global__ __launch_bounds__(256) void name(uint32_t* out, const uint32_t* operand, const uint32_t* updates, \
+                                                           const uint32_t* start, const uint32_t* order, ScatterSortParams P) { \
+        scatter_rows_sum_body<VEC, IS_FLOAT>(out, operand, updates, start, order, P);                              \
+    }
+// the _v4 variants require row_len % 4 == 0 and 16-byte aligned data pointers
+SCATTER_SUM_KERNEL(scatter_rows_sum_f_v1, 1, true)
+SCATTER_SUM_KERNEL(scatter_rows_sum_f_v4, 4, true)
+SCATTER_SUM_KERNEL(scatter_rows_sum_i_v1, 1, false)
+SCATTER_SUM_KERNEL(scatter_rows_sum_i_v4, 4, false)
+
 struct ScatterGeneralParams {
     uint32_t n_upd, upd_rank, op_rank, n_index, is_float;
     uint32_t upd_dims[IDX_MAX_RANK];

@@ -488,6 +488,27 @@ def scatter_add_rows(out: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_
                   bytes_moved=4 * (total + n_idx + out.size))
 
 
+def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, counters: Buffer, order: Buffer,
+                            n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1) -> tp.List[Launch]:
+    '''out = operand; out[idx[i], :] += updates[i, :] without atomics on the data: a counting sort of the
+    indices (`counters`: 2 * (n_rows + 1) words, `order`: n_idx words), then one wave per row sums its bucket.'''
+    assert counters.size == 2 * (n_rows + 1) and order.size == n_idx
+    params = _u32(n_idx, row_len, n_rows, idx_stride)
+    cursor = (n_rows + 1) * 4                       #byte offset of the second half of `counters`
+    vec    = 4 if row_len % 4 == 0 else 1
+    kind   = 'f' if out.dtype == np.float32 else 'i'
+    return [
+        fill(counters, 0),
+        Launch('scatter_rows_count', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(counters, 0), (idx, 0)], params, bytes_moved=8 * n_idx),
+        Launch('scatter_rows_scan', (1, 1, 1), (1024, 1, 1), [(counters, 0)], _u32(n_rows + 1), bytes_moved=8 * (n_rows + 1)),
+        Launch('scatter_rows_fill', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(order, 0), (counters, cursor), (counters, 0), (idx, 0)], params,
+               bytes_moved=16 * n_idx),
+        Launch(f'scatter_rows_sum_{kind}_v{vec}', (_cdiv(n_rows, 16), 1, 1), (BLOCK, 1, 1),     #4 waves x 4 rows per block
+               [(out, 0), (operand, 0), (updates, 0), (counters, 0), (order, 0)], params,
+               bytes_moved=4 * (n_idx * row_len + n_idx + 2 * n_rows * row_len)),
+    ]
+
+
 def scatter_add_general(out: Buffer, indices: Buffer, updates: Buffer, update_window_dims, inserted_window_dims,
                         scatter_dims_to_operand_dims) -> Launch:
     upd_rank, op_rank = len(updates.shape), len(out.shape)

@@ -578,14 +578,18 @@ def scatter_add(bufferpool, equation):
     dn = equation.params['dimension_numbers']
     uwd, iwd, sd2od = tuple(dn.update_window_dims), tuple(dn.inserted_window_dims), tuple(dn.scatter_dims_to_operand_dims)
     operand, indices, updates = [bufferpool.get_buffer(v) for v in equation.invars]
-    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    outbuf = bufferpool.get_buffer(equation.outvars[0])
+    #scratch arrays of this equation must carry its position, like its inputs and outputs: the
+    #position advances only after they have been created
+    counter_before = bufferpool.op_counter
+    bufferpool.op_counter += 1
     if _kind(operand.dtype) == _B or _kind(indices.dtype) not in (_I, _U):
         raise NotImplementedError(equation)
     if outbuf.size == 0:
         return []
-    ops = [_copy_op(equation, outbuf, EwOperand(operand, 0, K.row_major_strides(outbuf.shape)))]
+    copy = _copy_op(equation, outbuf, EwOperand(operand, 0, K.row_major_strides(outbuf.shape)))
     if updates.size == 0:
-        return ops
+        return [copy]
     n_batch = len(indices.shape) - 1
     is_rows = (iwd == (0,) and sd2od == (0,) and indices.shape[-1] == 1
                and uwd == tuple(range(n_batch, len(updates.shape)))
@@ -593,10 +597,22 @@ def scatter_add(bufferpool, equation):
     if is_rows:
         row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
         n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
-        ops.append(Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, operand.shape[0])))
-    else:
-        ops.append(Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od)))
-    return ops
+        n_rows  = operand.shape[0]
+        if n_idx * row_len >= SCATTER_SORT_THRESHOLD and n_idx < 2**30 and n_rows < 2**31 - 1:
+            #large: bucket the updates by row and sum each bucket (no atomics on the data, no copy of the operand)
+            bufferpool.op_counter = counter_before
+            counters = bufferpool.new_temporary(np.dtype('uint32'), (2 * (n_rows + 1),))
+            order    = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
+            bufferpool.op_counter = counter_before + 1
+            launches = K.scatter_add_rows_sorted(outbuf, operand, indices, updates, counters, order, n_idx, row_len, n_rows)
+            return [Op(equation, launch=l) for l in launches]
+        ops = [copy, Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, n_rows))]
+        return ops
+    return [copy, Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od))]
+
+
+#scatter-add of rows: from this many update elements on, the sorted (atomic-free) kernels are used
+SCATTER_SORT_THRESHOLD = 1 << 18
 
 
 # ------------------------------------------------------------------ rng
