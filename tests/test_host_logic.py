@@ -64,7 +64,7 @@ def test_kernel_argument_layouts_match_the_structs():
     #compiled on their own with the host compiler
     kdir  = os.path.join(ROOT, 'vkjax_amd', 'csrc', 'kernels')
     text  = ''.join(open(os.path.join(kdir, f)).read() for f in sorted(os.listdir(kdir)) if f.endswith('.hip'))
-    defs  = re.findall(r'^#define\s+(?:EW_MAX_STEPS|CONV_MAX_EPI|IDX_MAX_RANK|TF_MAX_STEPS)\s+\d+\s*$', text, re.M)
+    defs  = re.findall(r'^#define\s+(?:EW_MAX_STEPS|CONV_MAX_EPI|CONV_MAX_DERIVED|IDX_MAX_RANK|TF_MAX_STEPS)\s+\d+\s*$', text, re.M)
     decls = re.findall(r'^struct\s+\w+\s*\{[^}]*\};', text, re.M)
     names = [re.match(r'struct\s+(\w+)', d).group(1) for d in decls]
     src   = '#include <cstdio>\n#include <cstdint>\n' + '\n'.join(defs) + '\n' + '\n'.join(decls) + '\nint main(){\n' \
@@ -98,11 +98,14 @@ def test_kernel_argument_layouts_match_the_structs():
         'ThreefryStreamParams': K.threefry_stream(Buffer(None, np.dtype('uint32'), (16,)), (Buffer(None, np.dtype('uint32'), (2,)), 0),
                                                   (Buffer(None, np.dtype('uint32'), (2,)), 1), 8, 0, 8, []),
     }
+    #the convolution kernel takes two parameter structs, one after the other
+    sizes['ConvParams'] += sizes['ConvDerived']
     for struct, launch in launches.items():
         assert len(launch.params) == sizes[struct], (struct, len(launch.params), sizes[struct])
     assert sizes['ConvEpiPtrs'] == 8 * K.CONV_MAX_EPI and sizes['ThreefryStreamPtrs'] == 8 * K.TF_MAX_STEPS
     assert len(launches['ThreefryStreamParams'].buffers) == 3 + K.TF_MAX_STEPS
-    assert len(launches['ConvParams'].buffers) == 3 + K.CONV_MAX_EPI and len(launches['EwParams'].buffers) == 1 + K.EW_MAX_STEPS
+    assert sizes['ConvDerivedPtrs'] == 8 * (K.CONV_MAX_DERIVED + 1)
+    assert len(launches['ConvParams'].buffers) == 3 + K.CONV_MAX_EPI + K.CONV_MAX_DERIVED + 1 and len(launches['EwParams'].buffers) == 1 + K.EW_MAX_STEPS
 
 
 # ------------------------------------------------------------------ Function: trace cache

@@ -74,6 +74,20 @@ struct ConvParams {
 
 struct ConvEpiPtrs { const float* p[CONV_MAX_EPI]; };
 
+// One per-feature epilogue operand may be computed instead of read: the value for column n is
+//     v = first[n]; v = op_k(v, operand_k[n]) for k < nsteps      (each array a vector [N] or a single value)
+// which lets the small chain that prepares a batch-norm scale (gamma * rsqrt(var + eps)) run inside
+// the convolution that consumes it instead of as a launch of its own.
+#define CONV_MAX_DERIVED 3
+struct ConvDerivedPtrs { const float* p[CONV_MAX_DERIVED + 1]; };   // first, then the operand of each step (null where a step has none)
+struct ConvDerived {
+    uint32_t step;                          // the epilogue step whose operand this is
+    uint32_t nsteps;                        // 0: nothing is derived
+    uint32_t vector_mask;                   // bit k: array k is a vector [N] (else one value)
+    uint32_t op[CONV_MAX_DERIVED];          // add / sub / mul / div / max / min / neg / rsqrt / sqrt, float
+    uint32_t left[CONV_MAX_DERIVED];        // the operand is the left argument
+};
+
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
@@ -106,7 +120,7 @@ __device__ __forceinline__ int magic_div(int n, uint32_t magic, uint32_t shift) 
 template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST, bool LEAN>
 __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
                                                const float* __restrict__ w, const ConvEpiPtrs& epi,
-                                               const ConvParams& Pk) {
+                                               const ConvDerivedPtrs& Dp, const ConvParams& Pk, const ConvDerived& Dk) {
     constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, NT = 64 * WGM * WGN;
     constexpr int LDA = BK + 4, LDB = BN + 4;
     __shared__ __attribute__((aligned(16))) float As[BM * LDA];
@@ -177,8 +191,42 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
         for (int e = 0; e < CONV_MAX_EPI; ++e) {
             const uint32_t kind = step_desc(e) >> 8;             // 0 beyond the last step
             e_reg[e] = 0.f;
-            if (kind == 1) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], 4u), 0u);
-            else if (kind == 2) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], (uint32_t)P.N * 4u), (uint32_t)(n0 + tid) * 4u);
+            // (a step whose operand is derived below has no array: a descriptor of size 0 reads nothing)
+            const uint32_t present = epi.p[e] != nullptr ? 1u : 0u;
+            if (kind == 1) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], 4u * present), 0u);
+            else if (kind == 2) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], (uint32_t)P.N * 4u * present), (uint32_t)(n0 + tid) * 4u);
+        }
+        if (Dk.nsteps) {
+            // the derived operand: same arithmetic, operation by operation, as the element-wise kernel
+            float in[CONV_MAX_DERIVED + 1];
+#pragma unroll
+            for (int k = 0; k <= CONV_MAX_DERIVED; ++k) {
+                const bool vec = (Dk.vector_mask >> k) & 1u;
+                in[k] = buffer_load_x1(make_rsrc(Dp.p[k], Dp.p[k] == nullptr ? 0u : vec ? (uint32_t)P.N * 4u : 4u),
+                                       vec ? (uint32_t)(n0 + tid) * 4u : 0u);
+            }
+            float v = in[0];
+#pragma unroll
+            for (int k = 0; k < CONV_MAX_DERIVED; ++k) {
+                if (k < (int)Dk.nsteps) {
+                    const float a = Dk.left[k] ? in[k + 1] : v, b = Dk.left[k] ? v : in[k + 1];
+                    switch (Dk.op[k]) {
+                        case CEW_ADD_F:   v = a + b; break;
+                        case CEW_SUB_F:   v = a - b; break;
+                        case CEW_MUL_F:   v = a * b; break;
+                        case CEW_DIV_F:   v = a / b; break;
+                        case CEW_MAX_F:   v = (a > b || a != a) ? a : b; break;
+                        case CEW_MIN_F:   v = (a < b || a != a) ? a : b; break;
+                        case CEW_NEG_F:   v = -v; break;
+                        case CEW_RSQRT_F: v = 1.0f / sqrtf(v); break;
+                        case CEW_SQRT_F:  v = sqrtf(v); break;
+                        default: break;
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < CONV_MAX_EPI; ++e)
+                if (e == (int)Dk.step) e_reg[e] = v;
         }
     }
     // the first full-size operand (a residual input) is fetched for a whole tile at once, while
@@ -634,8 +682,8 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 #define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF, LEAN)                                               \
     extern "C" __global__ __launch_bounds__(64 * WGM * WGN) __attribute__((amdgpu_waves_per_eu(2))) void name( \
         float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
-        ConvEpiPtrs epi, ConvParams P) {                                                                     \
-        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF, LEAN>(out, x, w, epi, P);                               \
+        ConvEpiPtrs epi, ConvDerivedPtrs dp, ConvParams P, ConvDerived D) {                                  \
+        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF, LEAN>(out, x, w, epi, dp, P, D);                        \
     }
 
 // name = conv_gemm_<BM>x<BN>x<BK>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads),

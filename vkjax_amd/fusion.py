@@ -38,7 +38,11 @@ def _reads(op) -> tp.List:
         return [o.buffer for o in op.chain.operands() if o is not None]
     if op.conv is not None:
         out, lhs, rhs, geom, epilogue = op.conv
-        return [lhs, rhs] + [e.operand for e in epilogue]
+        reads = [lhs, rhs] + [e.operand for e in epilogue if e.operand is not None]
+        for e in epilogue:
+            if e.derived is not None:
+                reads += [e.derived.first] + [st[1] for st in e.derived.steps if st[1] is not None]
+        return reads
     if op.meta is not None:
         if op.meta[0] == 'iota':
             return []
@@ -164,7 +168,81 @@ def fuse_ops(all_ops, bufferpool, outvars):
         if out is not None:
             producer[id(out._placeholder)] = len(result) - 1
     ops = fuse_random_streams([op for op in result if op is not None], bufferpool, outvars)
+    ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
     return remove_dead_ops(ops, bufferpool, outvars)
+
+
+def fuse_derived_epilogue_operands(ops, bufferpool, outvars):
+    '''A per-feature operand of a convolution epilogue that is itself the result of a short chain over
+    per-feature vectors and single values (the batch-norm scale gamma * rsqrt(var + eps)) is computed
+    by the convolution kernel while it stages its epilogue operands; the chain's own launch and its
+    result array go away. One such operand per convolution; the arithmetic is unchanged.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    producer = {pid(op.chain.out): i for i, op in enumerate(ops) if op.chain is not None}
+    allowed  = {EW[name] for name in K.CONV_DERIVED_OPS}
+    unary    = {EW['NEG_F'], EW['RSQRT_F'], EW['SQRT_F']}
+    removed  = set()
+    result   = list(ops)
+    for ci, op in enumerate(ops):
+        if op.conv is None:
+            continue
+        out, lhs, rhs, geom, epilogue = op.conv
+        N = geom.N
+        for ei, e in enumerate(epilogue):
+            if e.kind != 2 or e.derived is not None or e.operand is None:
+                continue
+            pi = producer.get(pid(e.operand))
+            if pi is None or pi >= ci or pi in removed or uses[pid(e.operand)] != 1:
+                continue
+            chain = ops[pi].chain
+            n = 1
+            for d in chain.shape:
+                n *= d
+            if n != N or not (1 <= len(chain.steps) <= K.CONV_MAX_DERIVED):
+                continue
+
+            def per_feature(o):
+                '''(buffer) if the operand is one value or walks N contiguous values, else None'''
+                if o.offset != 0:
+                    return None
+                if o.buffer.size == 1:
+                    return o.buffer
+                if o.buffer.size == N and tuple(o.strides) == K.row_major_strides(chain.shape):
+                    return o.buffer
+                return None
+            first = per_feature(chain.first)
+            steps = []
+            for st in chain.steps:
+                if st.op not in allowed or st.imm:
+                    steps = None
+                    break
+                if st.op in unary:
+                    if st.operand is not None:
+                        steps = None
+                        break
+                    steps.append((st.op, None, False))
+                else:
+                    b = per_feature(st.operand) if st.operand is not None else None
+                    if b is None:
+                        steps = None
+                        break
+                    steps.append((st.op, b, bool(st.operand_left)))
+            if first is None or steps is None:
+                continue
+            derived  = K.ConvDerivedOperand(first, tuple(steps))
+            new_epi  = list(epilogue)
+            new_epi[ei] = e._replace(operand=None, derived=derived)
+            fused = Op(_label(ops[pi], op), conv=(out, lhs, rhs, geom, new_epi))
+            fused.index = op.index
+            for b in [first] + [st[1] for st in steps if st[1] is not None]:
+                b.accesses.append(fused.index)
+            e.operand._placeholder.elided = True
+            removed.add(pi)
+            result[ci] = fused
+            break
+    return [op for i, op in enumerate(result) if i not in removed]
 
 
 def _writes(op) -> tp.List:

@@ -246,11 +246,23 @@ class ConvGeometry(tp.NamedTuple):
     def K(self): return self.KH * self.KW * self.Cin
 
 
+class ConvDerivedOperand(tp.NamedTuple):
+    '''A per-feature epilogue operand that the kernel computes instead of reading: `first` and the
+    step operands are buffers of N values or of one value.'''
+    first: Buffer
+    steps: tp.Tuple[tp.Tuple[int, tp.Optional[Buffer], bool], ...]       #(opcode, operand or None, operand is the left argument)
+
+
 class ConvEpilogueStep(tp.NamedTuple):
     op:           int
     kind:         int                    #1 scalar, 2 per-feature vector [N], 3 full tensor laid out like the output
-    operand:      Buffer
+    operand:      tp.Optional[Buffer]    #None when `derived` says how to compute it
     operand_left: bool = False
+    derived:      tp.Optional[ConvDerivedOperand] = None
+
+
+CONV_MAX_DERIVED = 3
+CONV_DERIVED_OPS = ('ADD_F', 'SUB_F', 'MUL_F', 'DIV_F', 'MAX_F', 'MIN_F', 'NEG_F', 'RSQRT_F', 'SQRT_F')
 
 
 #(tag, BM, BN, threads, resident blocks per CU, relative MFMA efficiency of the tile shape)
@@ -392,10 +404,22 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
                    *g.xs[:3], tiles_m, tiles_n)
               + _u32(flags, *descs, x_bytes, w_bytes, out.size * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
               + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os))
+    derived_ptrs, derived_desc = [(None, 0)] * (CONV_MAX_DERIVED + 1), _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
+    for i, e in enumerate(epilogue):
+        if e.derived is not None:
+            d = e.derived
+            assert e.kind == 2 and len(d.steps) <= CONV_MAX_DERIVED and derived_desc == _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
+            arrays = [d.first] + [st[1] for st in d.steps]
+            assert all(a is None or a.size in (1, N) for a in arrays)
+            derived_ptrs = _pad([(a, 0) for a in arrays], CONV_MAX_DERIVED + 1, (None, 0))
+            mask = sum(1 << k for k, a in enumerate(arrays) if a is not None and a.size == N and N != 1)
+            derived_desc = _u32(i, len(d.steps), mask, *_pad([st[0] for st in d.steps], CONV_MAX_DERIVED),
+                                *_pad([int(st[2]) for st in d.steps], CONV_MAX_DERIVED))
+    params += derived_desc
     buffers = [(out, 0), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
-    buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
+    buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0)) + derived_ptrs
     kernel  = f'conv_gemm_{tag}x{bk}_' + ('lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
-    nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue)
+    nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
     return Launch(kernel, (_cdiv(tiles_m, chunk) * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
                   bytes_moved=nbytes, flops=2 * M * N * K)
 
