@@ -32,7 +32,7 @@ UNITS = {'resnet50': ('images/sec', 'batch'), 'mlp': ('samples/sec', 'batch'), '
 
 
 def kernel_family(name: str) -> str:
-    for prefix in ('conv_gemm', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_3d'):
+    for prefix in ('conv_gemm', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows'):
         if name.startswith(prefix):
             return prefix
     return name

@@ -1,0 +1,63 @@
+'''Reductions on the GPU against the numpy oracle: both kernels (contiguous rows, strided columns),
+16-byte and 4-byte loads, reductions split into ranges with a second launch, index-returning
+reductions with ties and NaNs. Integer-valued data keeps float sums exact, so every case is
+compared bit for bit.'''
+import numpy as np
+import pytest
+
+from vkjax_amd import minijax as mj
+from tests.common import check_against_oracle
+
+pytestmark = pytest.mark.gpu
+jnp = mj.numpy
+rng = np.random.RandomState(99)
+
+
+def ints(shape, lo=-2, hi=3, dtype=np.float32):
+    return rng.randint(lo, hi, size=shape).astype(dtype)
+
+
+CASES = [
+    #(shape, axes, expected kernel prefix, expected number of launches)
+    ((3, 100003), (1,), 'reduce_rows', 2), ((2, 1 << 20), (1,), 'reduce_rows', 2), ((65, 1000), (1,), 'reduce_rows', 1),
+    ((70000, 7), (1,), 'reduce_rows', 1), ((100000, 12), (0,), 'reduce_cols', 2), ((99999, 13), (0,), 'reduce_cols', 2),
+    ((16, 5000, 24), (1,), 'reduce_cols', 2), ((1 << 22,), (0,), 'reduce_rows', 2), ((5, 7, 9, 64), (1, 2), 'reduce_cols', 1),
+    ((64, 7, 7, 2048), (1, 2), 'reduce_cols', 1), ((300, 300), (0, 1), 'reduce_rows', 2),
+]
+
+
+@pytest.mark.parametrize('shape,axes,kernel,launches', CASES)
+def test_sum_max_min_exact(shape, axes, kernel, launches):
+    x = ints(shape)
+    for name, f in (('sum', lambda x: jnp.sum(x, axis=axes)), ('max', lambda x: jnp.max(x, axis=axes)), ('min', lambda x: jnp.min(x, axis=axes))):
+        print(f'{name} {shape} axes {axes}', flush=True)
+        _, _, fn = check_against_oracle(f, [x], exact=True)
+        kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+        assert all(k.startswith(kernel) for k in kernels) and len(kernels) == launches, kernels
+
+
+def test_integer_and_product_reductions():
+    check_against_oracle(lambda x: jnp.sum(x, axis=0), [ints((50000, 6), -1000, 1000, np.int32)], exact=True)
+    check_against_oracle(lambda x: jnp.max(x, axis=1), [ints((9, 70001), -10**9, 10**9, np.int32)], exact=True)
+    check_against_oracle(lambda x: jnp.min(x, axis=0), [rng.randint(0, 2**31, size=(40000, 3)).astype(np.uint32)], exact=True)
+    x = np.ones((4, 30000), np.float32)
+    x[:, ::1000] = 2.0                                      #products of powers of two are exact
+    check_against_oracle(lambda x: jnp.prod(x, axis=1), [x], exact=True)
+
+
+@pytest.mark.parametrize('shape,axis', [((7, 100001), 1), ((65536 + 3, 10), 1), ((50001, 9), 0), ((4, 3000, 8), 1)])
+def test_argmax_argmin_ties_and_nans(shape, axis):
+    x = ints(shape, -3, 4)                                   #many ties: the first occurrence must win
+    check_against_oracle(lambda x: jnp.argmax(x, axis=axis), [x], exact=True)
+    check_against_oracle(lambda x: jnp.argmin(x, axis=axis), [x], exact=True)
+    x = rng.random_sample(shape).astype(np.float32)
+    x[tuple(rng.randint(0, s, size=20) for s in shape)] = np.nan      #a NaN beats every number
+    check_against_oracle(lambda x: jnp.argmax(x, axis=axis), [x], exact=True)
+    check_against_oracle(lambda x: jnp.max(x, axis=axis), [x], exact=True)
+
+
+def test_float_sum_within_tolerance():
+    x = rng.random_sample((3, 1 << 21)).astype(np.float32)
+    check_against_oracle(lambda x: jnp.sum(x, axis=1), [x], rtol=1e-5, atol=0)
+    x = rng.random_sample((1 << 18, 24)).astype(np.float32)
+    check_against_oracle(lambda x: jnp.sum(x, axis=0), [x], rtol=1e-5, atol=0)

@@ -85,7 +85,7 @@ def test_kernel_argument_layouts_match_the_structs():
     launches = {
         'EwParams': K.lower_ew_chain(chain), 'IotaParams': K.iota(i(8), 0), 'FillParams': K.fill(b(8), 0),
         'ConcatParams': K.concat_part(b(4, 8), b(4, 3), 1, 0), 'ConvParams': K.conv_gemm(b(1, 4, 4, 8), b(1, 4, 4, 4), b(1, 1, 4, 8), geom),
-        'Reduce3dParams': K.reduce_3d(b(4), b(4, 8), 4, 8, 1, 'reduce_sum'),
+        'ReduceParams': K.reduce(b(4), b(4, 8), 4, 8, 1, 'reduce_sum')[0],
         'ReduceGeneralParams': K.reduce_general(b(4), b(4, 8), [(4, 8)], [(8, 1)], 'reduce_sum'),
         'PoolParams': K.pool(b(1, 2, 2, 4), b(1, 4, 4, 4), 'reduce_max', (1, 2, 2, 1), (1, 2, 2, 1), (0, 0, 0, 0), (1, 1, 1, 1)),
         'GatherRowsParams': K.gather_rows(b(3, 8), b(4, 8), i(3, 1), 3, 8, 4),

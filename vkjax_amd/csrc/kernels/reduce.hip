@@ -1,8 +1,6 @@
 // Reductions (sum / prod / max / min, argmax / argmin) and window reductions (max / sum pooling).
 //
-// reduce_3d views the operand as [outer, R, inner] and reduces R. A block is TI x TR threads
-// (TI*TR = 256): TI consecutive `inner` positions times TR interleaved slices of R, so global
-// loads are contiguous whichever of the two is the fast axis; slices are combined through LDS.
+// reduce_rows / reduce_cols view the operand as [outer, R, inner] and reduce R (see below).
 // reduce_general handles reductions whose kept and reduced dimensions interleave more than once
 // (one wave per output element, butterfly combine).
 // They supersede the reference's serial one-thread-per-output kernels reduce_sum/max/min/prod.comp,
@@ -56,46 +54,191 @@ __device__ __forceinline__ bool arg_better(bool is_max, uint32_t ty, uint32_t va
     return ia < ib;
 }
 
-struct Reduce3dParams { uint32_t outer, R, inner, op, type, TI, TR; };
+// ---------------------------------------------------------------------------------------------
+// Reductions of the canonical form [outer, R, inner] -> [outer, inner].
+//
+// reduce_rows (inner == 1): a wave owns one (row, split) pair and streams its part of the row with
+// 16-byte loads, four in flight per lane; lanes are combined with a butterfly.
+// reduce_cols (inner > 1): a block owns TI*VEC consecutive `inner` positions and one split of R;
+// its TR thread rows walk R interleaved, so every wave-level load is contiguous along `inner`;
+// thread rows are combined through LDS.
+// Splits: when outer x inner alone would not fill the GPU, R is cut into `nsplit` ranges of
+// `r_chunk` rows that different waves / blocks reduce; the partial results [outer, nsplit, inner]
+// are then reduced by a second launch of the same kernel. (Index-returning reductions run unsplit.)
+// MODE picks the combine at compile time: 0 float sum, 1 float max (NaN wins), 2 whatever op/type say,
+// 3 / 4 float argmax / argmin.
+struct ReduceParams { uint32_t outer, R, inner, op, type, r_chunk, nsplit, TI; };
 
-extern "C" __global__ __launch_bounds__(256) void reduce_3d(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
-                                                            Reduce3dParams P) {
-    __shared__ uint32_t s_val[256];
-    __shared__ uint32_t s_idx[256];
-    const uint32_t tid = threadIdx.x, ti = tid % P.TI, tr = tid / P.TI;
-    const uint32_t i = blockIdx.x * P.TI + ti, o = blockIdx.y;
-    const bool is_arg = P.op >= RED_ARGMAX, is_max = P.op == RED_ARGMAX;
-    uint32_t acc = red_identity(P.op, P.type), best_i = 0xFFFFFFFFu, best_v = 0;
-    if (i < P.inner) {
-        const uint32_t* p = in + ((uint64_t)o * P.R) * P.inner + i;
-        for (uint32_t r = tr; r < P.R; r += P.TR) {
-            const uint32_t v = p[(uint64_t)r * P.inner];
-            if (is_arg) {
-                if (best_i == 0xFFFFFFFFu || arg_better(is_max, P.type, v, r, best_v, best_i)) { best_v = v; best_i = r; }
+template <int MODE>
+__device__ __forceinline__ uint32_t red_step(uint32_t op, uint32_t ty, uint32_t a, uint32_t b) {
+    if constexpr (MODE == 0) return f2u(u2f(a) + u2f(b));
+    else if constexpr (MODE == 1) { const float x = u2f(a), y = u2f(b); return (x > y || x != x) ? a : b; }
+    else return red_combine(op, ty, a, b);
+}
+
+template <int VEC, int MODE>
+__device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint64_t unit = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (unit >= (uint64_t)P.outer * P.nsplit) return;                 // whole wave leaves together
+    const uint32_t o = (uint32_t)(unit / P.nsplit), sp = (uint32_t)(unit - (uint64_t)o * P.nsplit);
+    const uint32_t r_lo = sp * P.r_chunk, r_hi = min(P.R, r_lo + P.r_chunk);
+    const uint32_t* row = in + (uint64_t)o * P.R;
+    const bool is_arg = MODE >= 3 || (MODE == 2 && P.op >= RED_ARGMAX), is_max = MODE == 3 || (MODE == 2 && P.op == RED_ARGMAX);
+    const uint32_t ident = MODE == 0 ? 0u : MODE == 1 ? 0xFF800000u : red_identity(P.op, P.type);
+    uint32_t acc[4] = {ident, ident, ident, ident}, best_i = 0xFFFFFFFFu, best_v = 0;
+    auto take = [&](uint32_t v, uint32_t r, int slot) {
+        if constexpr (MODE >= 3) {
+            // float argmax / argmin: a lane meets its elements in ascending index order, so on a tie the
+            // earlier one stays; a NaN replaces any number and is never replaced
+            const float x = u2f(v), y = u2f(best_v);
+            const bool better = (MODE == 3 ? x > y : x < y) || (x != x && y == y) || best_i == 0xFFFFFFFFu;
+            best_v = better ? v : best_v;
+            best_i = better ? r : best_i;
+        } else if (is_arg) {
+            if (best_i == 0xFFFFFFFFu || arg_better(is_max, P.type, v, r, best_v, best_i)) { best_v = v; best_i = r; }
+        } else {
+            acc[slot] = red_step<MODE>(P.op, P.type, acc[slot], v);
+        }
+    };
+    if constexpr (VEC == 4) {
+        // r_lo, R and the row starts are multiples of 4 (the host checks); four loads in flight per lane
+        uint32_t r = r_lo + lane * 4u;
+        for (; r + 3u * 256u < r_hi; r += 4u * 256u) {
+            u32x4 v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = *reinterpret_cast<const u32x4*>(row + r + q * 256u);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                take(v[q].x, r + q * 256u, 0); take(v[q].y, r + q * 256u + 1u, 1); take(v[q].z, r + q * 256u + 2u, 2); take(v[q].w, r + q * 256u + 3u, 3);
+            }
+        }
+        for (; r < r_hi; r += 256u) {                                    // r_hi - r_lo is a multiple of 4 too
+            const u32x4 v = *reinterpret_cast<const u32x4*>(row + r);
+            take(v.x, r, 0); take(v.y, r + 1u, 1); take(v.z, r + 2u, 2); take(v.w, r + 3u, 3);
+        }
+    } else {
+        uint32_t r = r_lo + lane;
+        for (; r + 3u * 64u < r_hi; r += 4u * 64u) {
+            uint32_t v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = row[r + q * 64u];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) take(v[q], r + q * 64u, q);
+        }
+        for (; r < r_hi; r += 64u) take(row[r], r, 0);
+    }
+    uint32_t a = acc[0];
+    if (!is_arg) {
+        a = red_step<MODE>(P.op, P.type, red_step<MODE>(P.op, P.type, acc[0], acc[1]), red_step<MODE>(P.op, P.type, acc[2], acc[3]));
+    }
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        if (is_arg) {
+            const uint32_t vi = __shfl_xor(best_i, s, 64), vv = __shfl_xor(best_v, s, 64);
+            if (vi != 0xFFFFFFFFu && (best_i == 0xFFFFFFFFu || arg_better(is_max, P.type, vv, vi, best_v, best_i))) { best_v = vv; best_i = vi; }
+        } else {
+            a = red_step<MODE>(P.op, P.type, a, __shfl_xor(a, s, 64));
+        }
+    }
+    if (lane == 0) out[unit] = is_arg ? (best_i == 0xFFFFFFFFu ? 0u : best_i) : a;
+}
+
+template <int VEC, int MODE>
+__device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P) {
+    __shared__ uint32_t s_val[256 * VEC];
+    __shared__ uint32_t s_idx[256 * VEC];
+    const uint32_t TI = P.TI, TR = 256u / TI;
+    const uint32_t tid = threadIdx.x, ti = tid % TI, tr = tid / TI;
+    // block -> (inner tile, split, outer row)
+    const uint32_t tiles_i = (P.inner + TI * VEC - 1u) / (TI * VEC);
+    const uint32_t it = blockIdx.x % tiles_i, rest = blockIdx.x / tiles_i;
+    const uint32_t sp = rest % P.nsplit, o = rest / P.nsplit;
+    const uint32_t i = (it * TI + ti) * VEC;
+    const uint32_t r_lo = sp * P.r_chunk, r_hi = min(P.R, r_lo + P.r_chunk);
+    const bool is_arg = MODE >= 3 || (MODE == 2 && P.op >= RED_ARGMAX), is_max = MODE == 3 || (MODE == 2 && P.op == RED_ARGMAX);
+    const uint32_t ident = MODE == 0 ? 0u : MODE == 1 ? 0xFF800000u : red_identity(P.op, P.type);
+    uint32_t acc[VEC], best_i[VEC], best_v[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { acc[j] = ident; best_i[j] = 0xFFFFFFFFu; best_v[j] = 0; }
+    auto take = [&](uint32_t v, uint32_t r, int j) {
+        if constexpr (MODE >= 3) {
+            const float x = u2f(v), y = u2f(best_v[j]);
+            const bool better = (MODE == 3 ? x > y : x < y) || (x != x && y == y) || best_i[j] == 0xFFFFFFFFu;
+            best_v[j] = better ? v : best_v[j];
+            best_i[j] = better ? r : best_i[j];
+        } else if (is_arg) {
+            if (best_i[j] == 0xFFFFFFFFu || arg_better(is_max, P.type, v, r, best_v[j], best_i[j])) { best_v[j] = v; best_i[j] = r; }
+        } else {
+            acc[j] = red_step<MODE>(P.op, P.type, acc[j], v);
+        }
+    };
+    if (i < P.inner) {                                                // inner is a multiple of VEC
+        const uint32_t* p = in + (uint64_t)o * P.R * P.inner + i;
+        uint32_t r = r_lo + tr;
+        for (; r + 3u * TR < r_hi; r += 4u * TR) {                    // four loads in flight per thread
+            uint32_t v[4][VEC];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if constexpr (VEC == 4) {
+                    const u32x4 t = *reinterpret_cast<const u32x4*>(p + (uint64_t)(r + q * TR) * P.inner);
+                    v[q][0] = t.x; v[q][1] = t.y; v[q][2] = t.z; v[q][3] = t.w;
+                } else {
+                    v[q][0] = p[(uint64_t)(r + q * TR) * P.inner];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) take(v[q][j], r + q * TR, j);
+        }
+        for (; r < r_hi; r += TR) {
+            if constexpr (VEC == 4) {
+                const u32x4 t = *reinterpret_cast<const u32x4*>(p + (uint64_t)r * P.inner);
+                take(t.x, r, 0); take(t.y, r, 1); take(t.z, r, 2); take(t.w, r, 3);
             } else {
-                acc = red_combine(P.op, P.type, acc, v);
+                take(p[(uint64_t)r * P.inner], r, 0);
             }
         }
     }
-    s_val[tid] = is_arg ? best_v : acc;
-    s_idx[tid] = best_i;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { s_val[tid * VEC + j] = is_arg ? best_v[j] : acc[j]; s_idx[tid * VEC + j] = best_i[j]; }
     __syncthreads();
-    for (uint32_t s = P.TR >> 1; s >= 1; s >>= 1) {
+    for (uint32_t s = TR >> 1; s >= 1; s >>= 1) {
         if (tr < s) {
-            const uint32_t other = tid + s * P.TI;
-            if (is_arg) {
-                const uint32_t vi = s_idx[other], vv = s_val[other];
-                if (vi != 0xFFFFFFFFu && (s_idx[tid] == 0xFFFFFFFFu || arg_better(is_max, P.type, vv, vi, s_val[tid], s_idx[tid]))) {
-                    s_val[tid] = vv; s_idx[tid] = vi;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const uint32_t mine = tid * VEC + j, other = (tid + s * TI) * VEC + j;
+                if (is_arg) {
+                    const uint32_t vi = s_idx[other], vv = s_val[other];
+                    if (vi != 0xFFFFFFFFu && (s_idx[mine] == 0xFFFFFFFFu || arg_better(is_max, P.type, vv, vi, s_val[mine], s_idx[mine]))) {
+                        s_val[mine] = vv; s_idx[mine] = vi;
+                    }
+                } else {
+                    s_val[mine] = red_step<MODE>(P.op, P.type, s_val[mine], s_val[other]);
                 }
-            } else {
-                s_val[tid] = red_combine(P.op, P.type, s_val[tid], s_val[other]);
             }
         }
         __syncthreads();
     }
-    if (tr == 0 && i < P.inner) out[(uint64_t)o * P.inner + i] = is_arg ? (s_idx[tid] == 0xFFFFFFFFu ? 0u : s_idx[tid]) : s_val[tid];
+    if (tr == 0 && i < P.inner) {
+        uint32_t* dst = out + ((uint64_t)o * P.nsplit + sp) * P.inner + i;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) dst[j] = is_arg ? (s_idx[tid * VEC + j] == 0xFFFFFFFFu ? 0u : s_idx[tid * VEC + j]) : s_val[tid * VEC + j];
+    }
 }
+
+#define REDUCE_KERNELS(tag, MODE)                                                                                              \
+    extern "C" __global__ __launch_bounds__(256) void reduce_rows_##tag##_v1(uint32_t* out, const uint32_t* in, ReduceParams P) { reduce_rows_body<1, MODE>(out, in, P); } \
+    extern "C" __global__ __launch_bounds__(256) void reduce_rows_##tag##_v4(uint32_t* out, const uint32_t* in, ReduceParams P) { reduce_rows_body<4, MODE>(out, in, P); } \
+    extern "C" __global__ __launch_bounds__(256) void reduce_cols_##tag##_v1(uint32_t* out, const uint32_t* in, ReduceParams P) { reduce_cols_body<1, MODE>(out, in, P); } \
+    extern "C" __global__ __launch_bounds__(256) void reduce_cols_##tag##_v4(uint32_t* out, const uint32_t* in, ReduceParams P) { reduce_cols_body<4, MODE>(out, in, P); }
+// the _v4 variants need R % 4 == 0, r_chunk % 4 == 0 (rows) or inner % 4 == 0 (cols) and 16-byte aligned pointers
+REDUCE_KERNELS(fsum, 0)
+REDUCE_KERNELS(fmax, 1)
+REDUCE_KERNELS(any, 2)
+REDUCE_KERNELS(fargmax, 3)
+REDUCE_KERNELS(fargmin, 4)
 
 struct ReduceGeneralParams {
     uint32_t n_out, n_red, op, type;
@@ -199,6 +342,54 @@ __device__ __forceinline__ void pool_body(uint32_t* __restrict__ out, const uint
     } else {
         out[e0] = acc[0];
     }
+}
+
+// The usual pooling layout, [batch, y, x, channels] with a KH x KW window over y and x only: all
+// taps of a thread's four channels are requested before the first is used (the general kernel
+// above walks the window with one load in flight), with 32-bit index arithmetic. Needs channels % 4 == 0
+// and fewer than 2^32 bytes on either side; the host checks.
+template <int KH, int KW>
+__device__ __forceinline__ void pool2d_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const PoolParams& P) {
+    const uint32_t e0 = (blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (e0 >= P.n_out) return;
+    const uint32_t C = P.out_dims[3], Wo = P.out_dims[2], Ho = P.out_dims[1];
+    uint32_t r = e0 / C;
+    const uint32_t c = e0 - r * C;
+    const uint32_t wo = r % Wo; r /= Wo;
+    const uint32_t ho = r % Ho, b = r / Ho;
+    const int32_t y0 = (int32_t)(ho * P.stride[1]) - P.pad_low[1], x0 = (int32_t)(wo * P.stride[2]) - P.pad_low[2];
+    const uint32_t ident = red_identity(P.op, P.type);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in), 0,
+        (int)(P.in_dims[0] * P.in_dims[1] * P.in_dims[2] * P.in_dims[3] * 4u), 0x00020000);
+    u32x4 v[KH][KW];
+#pragma unroll
+    for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx) {
+            const int32_t y = y0 + ky * (int32_t)P.dilation[1], x = x0 + kx * (int32_t)P.dilation[2];
+            const bool ok = (uint32_t)y < P.in_dims[1] && (uint32_t)x < P.in_dims[2];
+            const uint32_t off = ((b * P.in_dims[1] + (uint32_t)y) * P.in_dims[2] + (uint32_t)x) * C + c;
+            v[ky][kx] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off * 4u : 0x80000000u, 0, 0);   // out of range reads 0 ...
+            if (!ok) v[ky][kx] = u32x4{ident, ident, ident, ident};                                         // ... and counts as the identity
+        }
+    u32x4 acc = v[0][0];
+#pragma unroll
+    for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx) {
+            if (ky == 0 && kx == 0) continue;
+            acc.x = red_combine(P.op, P.type, acc.x, v[ky][kx].x);
+            acc.y = red_combine(P.op, P.type, acc.y, v[ky][kx].y);
+            acc.z = red_combine(P.op, P.type, acc.z, v[ky][kx].z);
+            acc.w = red_combine(P.op, P.type, acc.w, v[ky][kx].w);
+        }
+    *reinterpret_cast<u32x4*>(out + e0) = acc;
+}
+extern "C" __global__ __launch_bounds__(256) void pool2d_3x3_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, PoolParams P) {
+    pool2d_body<3, 3>(out, in, P);
+}
+extern "C" __global__ __launch_bounds__(256) void pool2d_2x2_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, PoolParams P) {
+    pool2d_body<2, 2>(out, in, P);
 }
 
 extern "C" __global__ __launch_bounds__(256) void pool_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, PoolParams P) {

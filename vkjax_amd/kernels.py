@@ -437,14 +437,52 @@ def _pow2_at_least(x: int) -> int:
     return p
 
 
-def reduce_3d(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str) -> Launch:
-    TI = min(64, _pow2_at_least(inner))
-    TR = BLOCK // TI
-    if outer > 65535:
+def plan_reduce_splits(outer: int, R: int, inner: int, op: str, compute_units: int = 256) -> int:
+    '''Into how many ranges R is cut so that outer x inner x splits fills the GPU (1 = a single launch).'''
+    if op in ('argmax', 'argmin'):
+        return 1                                   #index-returning reductions run unsplit
+    if inner == 1:
+        want  = 32 * compute_units                 #waves
+        split = min(_cdiv(want, outer), R // 4096)         #at least 16 KB per wave
+    else:
+        tiles = _cdiv(inner, 256)
+        want  = 4 * compute_units                  #blocks
+        split = min(_cdiv(want, tiles * outer), R // 64)   #at least 64 rows per block
+    return max(1, min(split, 65535))
+
+
+def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str, nsplit: int, in_offset_ok=True) -> Launch:
+    ty   = _RTYPE[inp.dtype]
+    mode = {('reduce_sum', 0): 'fsum', ('reduce_max', 0): 'fmax', ('argmax', 0): 'fargmax', ('argmin', 0): 'fargmin'}.get((op, ty), 'any')
+    r_chunk = _cdiv(_cdiv(R, nsplit), 4) * 4
+    nsplit  = _cdiv(R, r_chunk)
+    if inner == 1:
+        vec = 4 if R % 4 == 0 else 1
+        params = _u32(outer, R, 1, RED[op], ty, r_chunk, nsplit, 0)
+        return Launch(f'reduce_rows_{mode}_v{vec}', (_cdiv(outer * nsplit, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
+                      bytes_moved=4 * (outer * R + outer * nsplit)), nsplit
+    vec = 4 if inner % 4 == 0 else 1
+    TI  = min(64, _pow2_at_least(_cdiv(inner, vec)))
+    params = _u32(outer, R, inner, RED[op], ty, r_chunk, nsplit, TI)
+    blocks = _cdiv(inner, TI * vec) * nsplit * outer
+    if blocks >= 2**31:
         raise NotImplementedError(f'reduction with {outer} outer rows and inner size {inner}')
-    params = _u32(outer, R, inner, RED[op], _RTYPE[inp.dtype], TI, TR)
-    return Launch('reduce_3d', (_cdiv(inner, TI), outer, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
-                  bytes_moved=4 * (inp.size + out.size))
+    return Launch(f'reduce_cols_{mode}_v{vec}', (blocks, 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
+                  bytes_moved=4 * (outer * R * inner + outer * nsplit * inner)), nsplit
+
+
+def reduce(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str,
+           partial: tp.Optional[Buffer] = None, nsplit: int = 1) -> tp.List[Launch]:
+    '''[outer, R, inner] -> [outer, inner]. With nsplit > 1, `partial` (outer * nsplit * inner words) receives
+    the per-range results of a first launch and a second launch reduces them.'''
+    if nsplit <= 1:
+        return [_reduce_launch(out, inp, outer, R, inner, op, 1)[0]]
+    first, nsplit = _reduce_launch(partial, inp, outer, R, inner, op, nsplit)
+    if nsplit == 1:
+        return [_reduce_launch(out, inp, outer, R, inner, op, 1)[0]]
+    assert partial.size >= outer * nsplit * inner and partial.dtype == inp.dtype
+    second = _reduce_launch(out, partial, outer, nsplit, inner, op, 1)[0]
+    return [first, second]
 
 
 def reduce_general(out: Buffer, inp: Buffer, kept, reduced, op: str) -> Launch:
@@ -475,6 +513,11 @@ def pool(out: Buffer, inp: Buffer, op: str, window, strides, pad_low, dilation) 
     vec = 4 if (window[3] == 1 and strides[3] == 1 and pad_low[3] == 0 and in_dims[3] % 4 == 0
                 and in_dims[3] == out_dims[3]) else 1
     params = _u32(n, RED[op], _RTYPE[inp.dtype], *in_dims, *out_dims, *window, *strides, *dilation) + _i32(*pad_low)
+    #[batch, y, x, channels] with a 3x3 or 2x2 window over y and x: the kernel that requests all taps at once
+    if (vec == 4 and window[0] == 1 and strides[0] == 1 and pad_low[0] == 0 and in_dims[0] == out_dims[0]
+            and (window[1], window[2]) in ((3, 3), (2, 2)) and inp.size * 4 < 2**31 and n * 4 < 2**32):
+        return Launch(f'pool2d_{window[1]}x{window[2]}_v4', (_cdiv(_cdiv(n, 4), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
+                      bytes_moved=4 * (inp.size + out.size))
     return Launch(f'pool_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
                   bytes_moved=4 * (inp.size + out.size))
 

@@ -510,8 +510,14 @@ def reduce_op(bufferpool, equation):
         outer = groups[0][1] if not roles[0] else 1
         inner = groups[-1][1] if not roles[-1] else 1
         R     = [g[1] for g in groups if g[0]][0]
-        if outer <= 65535:
-            return [Op(equation, launch=K.reduce_3d(outbuf, inbuf, outer, R, inner, name))]
+        nsplit = K.plan_reduce_splits(outer, R, inner, name)
+        partial = None
+        if nsplit > 1:
+            #scratch of this equation carries its position, like its operands
+            bufferpool.op_counter -= 1
+            partial = bufferpool.new_temporary(inbuf.dtype, (outer * nsplit * inner,))
+            bufferpool.op_counter += 1
+        return [Op(equation, launch=l) for l in K.reduce(outbuf, inbuf, outer, R, inner, name, partial, nsplit)]
     kept    = [(g[1], g[2]) for g in groups if not g[0]]
     reduced = [(g[1], g[2]) for g in groups if g[0]]
     return [Op(equation, launch=K.reduce_general(outbuf, inbuf, kept, reduced, name))]
