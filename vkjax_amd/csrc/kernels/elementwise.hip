@@ -20,11 +20,15 @@ struct EwParams {
     uint32_t nsteps;                   // 1..8; step 0 is the initial load
     uint32_t op[EW_MAX_STEPS];         // opcode of step k (op[0] ignored)
     uint32_t flags[EW_MAX_STEPS];      // bit0: step has an operand; bit1: operand is the LEFT argument;
-                                       // bit2: the operand's fastest stride is 1 (else 0: one value per vector)
+                                       // bit2: the operand's fastest stride is 1 (else 0: one value per vector);
+                                       // bits 4-5: how the operand is addressed: 0 through its strides, 1 like the
+                                       // output (element = base + linear index), 2 by the fastest dimension only
+                                       // (element = base + coordinate), 3 a single element (base)
     uint32_t imm[EW_MAX_STEPS];        // immediate (integer_pow exponent)
     int32_t  stride[EW_MAX_STEPS][4];  // operand strides per collapsed dim, in elements
     uint32_t nbytes[EW_MAX_STEPS];     // bytes readable from each operand pointer (0 = no operand)
     uint32_t base[EW_MAX_STEPS];       // element offset of output element 0 in each operand
+    uint32_t dim_magic[4], dim_shift[4];   // n / dims[d] = mulhi(n, magic) >> shift for n < 2^31; magic 0: dims[d] == 1
 };
 
 // Keeps a kernel argument in a scalar register from this point on. Used on every argument at
@@ -41,8 +45,13 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     uint32_t dims[4], op[NS], flags[NS], imm[NS], nbytes[NS], base[NS];
     int32_t  stride[NS][4];
     EW_PIN(n); EW_PIN(ndim); EW_PIN(nsteps);
+    uint32_t dim_magic[4], dim_shift[4];
 #pragma unroll
-    for (int d = 0; d < 4; ++d) { dims[d] = P.dims[d]; EW_PIN(dims[d]); }
+    for (int d = 0; d < 4; ++d) {
+        dims[d] = P.dims[d]; dim_magic[d] = P.dim_magic[d]; dim_shift[d] = P.dim_shift[d];
+        EW_PIN(dims[d]);
+        if (d >= 1) { EW_PIN(dim_magic[d]); EW_PIN(dim_shift[d]); }
+    }
 #pragma unroll
     for (int k = 0; k < NS; ++k) {
         flags[k] = P.flags[k]; nbytes[k] = P.nbytes[k]; base[k] = P.base[k];
@@ -52,55 +61,69 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
         for (int d = 0; d < 4; ++d) { stride[k][d] = P.stride[k][d]; EW_PIN(stride[k][d]); }
     }
 
-    const uint32_t v  = blockIdx.x * 256u + threadIdx.x;
-    const uint32_t i0 = v * VEC;                   // the host keeps n below 2^31
-    if (i0 >= n) return;
+    // A thread works on U vectors, 256 vectors apart (so that a wave's loads stay contiguous). All
+    // loads of all U vectors are requested before any is used: with one vector per thread the bytes a
+    // CU has in flight do not cover the memory latency once a chain has several operands.
+    constexpr int U = (NS == 4 || NS == 6) ? 2 : 1;
+    constexpr int W = U * VEC;                                    // values per thread
+    const uint32_t first = (blockIdx.x * U * 256u + threadIdx.x) * VEC;     // the host keeps n below 2^31
+    if (first >= n) return;
 
-    // coordinates of the first element of this vector in the collapsed output space
-    uint32_t c[4] = {0, 0, 0, 0};
-    {
-        uint32_t r = i0;
-        if (ndim > 1) {
-#pragma unroll
-            for (int d = 3; d >= 1; --d) {
-                if (d < (int)ndim) { const uint32_t q = r / dims[d]; c[d] = r - q * dims[d]; r = q; }
-            }
-        }
-        c[0] = r;
-    }
     // Every operand is read through a buffer descriptor with one branch-free load per slot: 16 bytes
     // (of which only the first dword is used where the operand is constant along the vector), or
-    // nothing at all for an empty slot, whose descriptor has size 0. All loads are in flight
-    // together; they are consumed after a single wait.
-    uint32_t vals[NS][VEC];
-    if constexpr (VEC == 4) {
-        u32x4 vec[NS];
+    // nothing at all for an empty slot, whose descriptor has size 0.
+    uint32_t vals[NS][W];
 #pragma unroll
-        for (int k = 0; k < NS; ++k) {
-            uint32_t idx = base[k] + c[0] * (uint32_t)stride[k][0];   // wraps correctly for negative strides
+    for (int u = 0; u < U; ++u) {
+        const uint32_t i0 = first + u * 256u * VEC;
+        // coordinates of the first element of this vector in the collapsed output space (divisions by
+        // multiply-high with constants from the host)
+        uint32_t c[4] = {0, 0, 0, 0};
+        {
+            uint32_t r = i0;
+            if (ndim > 1) {
+#pragma unroll
+                for (int d = 3; d >= 1; --d) {
+                    if (d < (int)ndim) {
+                        const uint32_t magic = dim_magic[d], shift = dim_shift[d];
+                        const uint32_t q = magic ? __umulhi(r, magic) >> shift : r;
+                        c[d] = r - q * dims[d]; r = q;
+                    }
+                }
+            }
+            c[0] = r;
+        }
+        // element index of this vector in operand k. Most operands are addressed in one of three simple
+        // ways, told apart by a wave-uniform flag; 32-bit multiplies run at a quarter of the rate of adds.
+        auto operand_index = [&](int k) -> uint32_t {
+            const uint32_t how = (flags[k] >> 4) & 3u;
+            if (how == 1u) return base[k] + i0;
+            if (how == 3u) return base[k];
+            uint32_t last = c[0];
+#pragma unroll
+            for (int d = 1; d < 4; ++d) last = d < (int)ndim ? c[d] : last;
+            if (how == 2u) return base[k] + last;
+            uint32_t idx = base[k] + c[0] * (uint32_t)stride[k][0];       // wraps correctly for negative strides
             if (ndim > 1) {
 #pragma unroll
                 for (int d = 1; d < 4; ++d) idx += c[d] * (uint32_t)stride[k][d];
             }
+            return idx;
+        };
+#pragma unroll
+        for (int k = 0; k < NS; ++k) {
+            const uint32_t idx = operand_index(k);
             const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, (int)nbytes[k], 0x00020000);
-            vec[k] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 4u, 0, 0);
-        }
-#pragma unroll
-        for (int k = 0; k < NS; ++k) {
-            const bool is_vec = (flags[k] & 4u) != 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) vals[k][j] = is_vec ? vec[k][j] : vec[k][0];
-        }
-    } else {
-#pragma unroll
-        for (int k = 0; k < NS; ++k) {
-            uint32_t idx = base[k] + c[0] * (uint32_t)stride[k][0];
-            if (ndim > 1) {
-#pragma unroll
-                for (int d = 1; d < 4; ++d) idx += c[d] * (uint32_t)stride[k][d];
+            if constexpr (VEC == 4) {
+                const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 4u, 0, 0);
+                const bool is_vec = (flags[k] & 4u) != 0;
+                vals[k][u * 4 + 0] = t.x;
+                vals[k][u * 4 + 1] = is_vec ? t.y : t.x;
+                vals[k][u * 4 + 2] = is_vec ? t.z : t.x;
+                vals[k][u * 4 + 3] = is_vec ? t.w : t.x;
+            } else {
+                vals[k][u] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, idx * 4u, 0, 0);
             }
-            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, (int)nbytes[k], 0x00020000);
-            vals[k][0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, idx * 4u, 0, 0);
         }
     }
 
@@ -108,9 +131,9 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
 #pragma unroll
     for (int k = 0; k < NS; ++k) { op[k] = P.op[k]; imm[k] = P.imm[k]; EW_PIN(op[k]); EW_PIN(imm[k]); }
 
-    uint32_t acc[VEC];
+    uint32_t acc[W];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = vals[0][j];
+    for (int j = 0; j < W; ++j) acc[j] = vals[0][j];
 
 #pragma unroll
     for (int k = 1; k < NS; ++k) {
@@ -119,23 +142,29 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
                 // three-input select: this step's operand and the next step's operand (a NOP carrier)
                 const int k2 = (k + 1 < NS) ? k + 1 : k;
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
+                for (int j = 0; j < W; ++j) {
                     const uint32_t s = vals[k][j], t = vals[k2][j];
                     acc[j] = op[k] == EW_SEL_P ? (acc[j] ? s : t)       // acc is the predicate
                            : op[k] == EW_SEL_T ? (s ? acc[j] : t)       // acc is on_true, s the predicate
                                                : (s ? t : acc[j]);      // acc is on_false, s the predicate
                 }
             } else {
-                ew_apply_vec<VEC>(op[k], acc, vals[k], (flags[k] & 2u) != 0, imm[k]);
+                ew_apply_vec<W>(op[k], acc, vals[k], (flags[k] & 2u) != 0, imm[k]);
             }
         }
     }
 
-    if constexpr (VEC == 4) {
-        u32x4 t; t.x = acc[0]; t.y = acc[1]; t.z = acc[2]; t.w = acc[3];
-        *reinterpret_cast<u32x4*>(out + i0) = t;
-    } else {
-        out[i0] = acc[0];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t i0 = first + u * 256u * VEC;
+        if (i0 < n) {
+            if constexpr (VEC == 4) {
+                u32x4 t; t.x = acc[u * 4]; t.y = acc[u * 4 + 1]; t.z = acc[u * 4 + 2]; t.w = acc[u * 4 + 3];
+                *reinterpret_cast<u32x4*>(out + i0) = t;
+            } else {
+                out[i0] = acc[u];
+            }
+        }
     }
 }
 
@@ -163,18 +192,33 @@ EW_KERNEL(ew_chain_v4_s8, 4, 8)
 struct IotaParams { uint32_t n, inner, size, to_float; };
 
 // out[i] = (i / inner) % size   (reference: vkjax/shaders/iota.comp:8-11 for the 1-D case)
-extern "C" __global__ __launch_bounds__(256) void iota_nd(uint32_t* __restrict__ out, IotaParams P) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+// Four consecutive elements per thread (16-byte stores); VEC = 4 needs n % 4 == 0.
+template <int VEC>
+__device__ __forceinline__ void iota_body(uint32_t* __restrict__ out, const IotaParams& P) {
+    const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * VEC;
     if (i >= P.n) return;
-    const uint32_t v = (i / P.inner) % P.size;
-    out[i] = P.to_float ? f2u((float)v) : v;
+    uint32_t v[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        const uint32_t x = ((i + j) / P.inner) % P.size;
+        v[j] = P.to_float ? f2u((float)x) : x;
+    }
+    if constexpr (VEC == 4) { u32x4 t; t.x = v[0]; t.y = v[1]; t.z = v[2]; t.w = v[3]; *reinterpret_cast<u32x4*>(out + i) = t; }
+    else out[i] = v[0];
 }
+extern "C" __global__ __launch_bounds__(256) void iota_nd_v1(uint32_t* __restrict__ out, IotaParams P) { iota_body<1>(out, P); }
+extern "C" __global__ __launch_bounds__(256) void iota_nd_v4(uint32_t* __restrict__ out, IotaParams P) { iota_body<4>(out, P); }
 
 struct FillParams { uint32_t n, value; };
 
+// (16-byte stores for whole groups of four, single words for the tail)
 extern "C" __global__ __launch_bounds__(256) void fill_u32(uint32_t* __restrict__ out, FillParams P) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < P.n) out[i] = P.value;
+    const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (i + 3u < P.n) {
+        *reinterpret_cast<u32x4*>(out + i) = u32x4{P.value, P.value, P.value, P.value};
+    } else {
+        for (uint32_t j = i; j < P.n; ++j) out[j] = P.value;
+    }
 }
 
 struct ConcatParams { uint32_t n, part_inner, out_inner, out_offset; };
@@ -182,10 +226,19 @@ struct ConcatParams { uint32_t n, part_inner, out_inner, out_offset; };
 // One operand of a concatenation: the operand is [outer, part_inner], the output
 // [outer, out_inner]; operand row r lands at out[r*out_inner + out_offset ...].
 // (reference: vkjax/shaders/concatenate.comp:9-25, two operands on the last axis only)
-extern "C" __global__ __launch_bounds__(256) void concat_part(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
-                                                              ConcatParams P) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+// VEC = 4 needs part_inner, out_inner and out_offset to be multiples of 4.
+template <int VEC>
+__device__ __forceinline__ void concat_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ConcatParams& P) {
+    const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * VEC;
     if (i >= P.n) return;
     const uint32_t r = i / P.part_inner, c = i - r * P.part_inner;
-    out[(uint64_t)r * P.out_inner + P.out_offset + c] = in[i];
+    uint32_t* dst = out + (uint64_t)r * P.out_inner + P.out_offset + c;
+    if constexpr (VEC == 4) *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(in + i);
+    else *dst = in[i];
+}
+extern "C" __global__ __launch_bounds__(256) void concat_part_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, ConcatParams P) {
+    concat_body<1>(out, in, P);
+}
+extern "C" __global__ __launch_bounds__(256) void concat_part_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, ConcatParams P) {
+    concat_body<4>(out, in, P);
 }

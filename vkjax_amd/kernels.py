@@ -147,6 +147,7 @@ def lower_ew_chain(chain: EwChain) -> Launch:
             vec = 1
         elif st[-1] == 1 and (o.offset % 4 or any(s % 4 for s in st[:-1])):
             vec = 1
+    magics = [_magic_division(d) for d in _pad(dims, 4, 1)]
     ops, flags, imms, stride_rows, buffers, extents, bases = [], [], [], [], [], [], []
     it = iter(strides)
     for k, o in enumerate(operands):
@@ -166,6 +167,13 @@ def lower_ew_chain(chain: EwChain) -> Launch:
             extents.append(o.buffer.size * 4)
             bases.append(o.offset)
             flag |= 1 | (4 if st[-1] == 1 else 0)
+            #simple addressing patterns the kernel resolves without multiplications
+            if all(s == 0 for s in st):
+                flag |= 3 << 4
+            elif tuple(st) == row_major_strides(dims):
+                flag |= 1 << 4
+            elif st[-1] == 1 and all(s == 0 for s in st[:-1]):
+                flag |= 2 << 4
             stride_rows.append(_pad(st, 4))
             buffers.append((o.buffer, 0))
         flags.append(flag)
@@ -174,12 +182,14 @@ def lower_ew_chain(chain: EwChain) -> Launch:
         buffers.append((None, 0))
     params = (_u32(n, ndim, *_pad(dims, 4, 1), nsteps, *_pad(ops, EW_MAX_STEPS), *_pad(flags, EW_MAX_STEPS),
                    *_pad(imms, EW_MAX_STEPS))
-              + _i32(*[s for row in stride_rows for s in row]) + _u32(*_pad(extents, EW_MAX_STEPS), *_pad(bases, EW_MAX_STEPS)))
+              + _i32(*[s for row in stride_rows for s in row]) + _u32(*_pad(extents, EW_MAX_STEPS), *_pad(bases, EW_MAX_STEPS))
+              + _u32(*[m for m, _ in magics], *[sh for _, sh in magics]))
     nbytes = 4 * n + sum(4 * min(n, o.buffer.size) for o in present)
     if n >= 2**31:
         raise NotImplementedError(f'element-wise op over {n} elements exceeds 32-bit indexing')
     slots = 2 if nsteps <= 2 else 4 if nsteps <= 4 else 6 if nsteps <= 6 else 8
-    return Launch(f'ew_chain_v{vec}_s{slots}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+    per_thread = {2: 1, 4: 2, 6: 2, 8: 1}[slots]               #vectors a thread works on (the kernel's U)
+    return Launch(f'ew_chain_v{vec}_s{slots}', (_cdiv(_cdiv(n, vec), BLOCK * per_thread), 1, 1), (BLOCK, 1, 1),
                   [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
 
 
@@ -187,21 +197,23 @@ def iota(out: Buffer, dimension: int) -> Launch:
     n     = out.size
     inner = int(np.prod(out.shape[dimension + 1:], dtype=np.int64))
     size  = out.shape[dimension]
-    return Launch('iota_nd', (_cdiv(n, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0)],
+    vec   = 4 if n % 4 == 0 else 1
+    return Launch(f'iota_nd_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0)],
                   _u32(n, inner, size, int(out.dtype == np.float32)), bytes_moved=4 * n)
 
 
 def fill(out: Buffer, word: int) -> Launch:
     n = out.size
-    return Launch('fill_u32', (_cdiv(n, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0)], _u32(n, word), bytes_moved=4 * n)
+    return Launch('fill_u32', (_cdiv(_cdiv(n, 4), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0)], _u32(n, word), bytes_moved=4 * n)
 
 
 def concat_part(out: Buffer, part: Buffer, dimension: int, offset_along_dim: int) -> Launch:
     inner      = int(np.prod(out.shape[dimension + 1:], dtype=np.int64))
     part_inner = part.shape[dimension] * inner
     out_inner  = out.shape[dimension] * inner
-    n = part.size
-    return Launch('concat_part', (_cdiv(n, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (part, 0)],
+    n   = part.size
+    vec = 4 if (part_inner % 4 == 0 and out_inner % 4 == 0 and (offset_along_dim * inner) % 4 == 0) else 1
+    return Launch(f'concat_part_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (part, 0)],
                   _u32(n, part_inner, out_inner, offset_along_dim * inner), bytes_moved=8 * n)
 
 
