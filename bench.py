@@ -47,6 +47,7 @@ def main():
     ap.add_argument('--batch', type=int, default=None)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-fuse', action='store_true')
+    ap.add_argument('--graph', action='store_true', help='replay the launches as one captured HIP graph')
     ap.add_argument('--profile-iters', type=int, default=3)
     ap.add_argument('--dump-launches', default=None, help='write one line per launch (kernel, grid, FLOP, bytes, ms) to this file')
     ap.add_argument('--calibration-copy', action='store_true',
@@ -71,7 +72,7 @@ def main():
     props  = dev.get_device_properties()
 
     t0 = time.perf_counter()
-    wrapped = vkjax_amd.wrap(fn, frontend='minijax', fuse=not args.no_fuse)
+    wrapped = vkjax_amd.wrap(fn, frontend='minijax', fuse=not args.no_fuse, graph=args.graph)
     interp, _ = wrapped._get_or_create_jaxpr_interpreter(tuple(inputs))
     build_s = time.perf_counter() - t0
     interp.upload_inputs(*inputs)

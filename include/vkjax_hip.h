@@ -112,6 +112,13 @@ int vkj_seq_eval(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t fl
  * stream; *ms_total receives the elapsed device time of all iterations. Used for
  * measurement with inputs resident in HBM. No counterpart in the reference. */
 int vkj_seq_replay(vkj_handle seq, int iters, float* ms_total);
+/* Makes vkj_seq_eval and vkj_seq_replay issue the launches of this sequence as ONE captured HIP
+ * graph (built at the next use, rebuilt after further recording) instead of one launch call
+ * each; uploads, downloads and profiling events stay outside the graph. enable = 0 returns to
+ * individual launches. A sequence created with timestamps never uses a graph. The counterpart
+ * in the reference is the Vulkan command buffer the sequence is recorded into once
+ * (vkjax/kompute_jaxpr_interpreter.py:49-63). */
+int vkj_seq_use_graph(vkj_handle seq, int enable);
 /* sequence.get_timestamps()           reference: vkjax/kompute_jaxpr_interpreter.py:91-95
  * Milliseconds since the first timestamp of the last vkj_seq_eval; *count receives the
  * number of timestamps available (steps + 1). */

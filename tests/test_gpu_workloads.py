@@ -178,3 +178,24 @@ def test_function_semantics_on_device():
     assert len(vk_func._jaxpr_interpreters) == 3
     with pytest.raises(TypeError):
         list(vk_func._jaxpr_interpreters.values())[0].run(1, 2)
+
+
+def test_graph_replay_matches_individual_launches():
+    '''The launches of a sequence issued as one captured HIP graph: several replays, with other work
+    and synchronisations of the same program in between, each compared bit for bit with the result
+    of the individually launched sequence; new inputs are picked up by every replay.'''
+    rng = np.random.default_rng(11)
+    for f, make in ((W.mlp, W.mlp_inputs), (W.conv_block, lambda: W.conv_block_inputs(batch=3, size=20, channels=24)),
+                    (lambda key: W.rng_uniform(key, (64, 48)), W.rng_inputs)):
+        plain = vkjax_amd.wrap(f, frontend='minijax')
+        graph = vkjax_amd.wrap(f, frontend='minijax', graph=True)
+        for rep in range(4):
+            args = make()
+            if rep:                                   #different data every time
+                args = [a + np.asarray(rep, dtype=a.dtype) if isinstance(a, np.ndarray) and a.dtype == np.float32 else a for a in args]
+            expected = plain(*args)
+            got = graph(*args)
+            assert_tree_close(got, expected, exact=True, what=f'graph replay {rep}')
+            plain(*make())                            #unrelated eager work between graph launches
+        interp = list(graph._jaxpr_interpreters.values())[0]
+        assert interp.graph

@@ -96,6 +96,9 @@ struct Seq {
     std::vector<Launch>   launches;
     std::vector<hipEvent_t> stamps;   // profiling: 1 + number of steps
     int                   stamps_valid = 0;
+    bool                  want_graph = false;     // issue the launches as one captured graph
+    bool                  graph_failed = false;   // capture did not work once: keep to plain launches
+    hipGraphExec_t        graph_exec = nullptr;
 };
 
 // Handles are keys into a process-wide table, never raw addresses, so that a stale or made-up
@@ -142,6 +145,41 @@ int issue_launch(Ctx* c, Launch& l) {
         g_last_error = "launch of " + l.fn->name + ": " + hipGetErrorString(e);
         return (int)e;
     }
+    return 0;
+}
+
+void drop_graph(Seq* s) {
+    if (s->graph_exec) { hipGraphExecDestroy(s->graph_exec); s->graph_exec = nullptr; }
+    s->graph_failed = false;
+}
+
+// All launches of a sequence, once: as its captured graph when that is asked for, else one by one.
+int issue_all(Ctx* c, Seq* s) {
+    if (s->want_graph && !s->profiling && !s->graph_failed && s->launches.size() > 1) {
+        if (!s->graph_exec) {
+            hipGraph_t graph = nullptr;
+            hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
+            if (e == hipSuccess) {
+                int r = 0;
+                for (auto& l : s->launches) if ((r = issue_launch(c, l))) break;
+                hipError_t e2 = hipStreamEndCapture(c->stream, &graph);
+                if (r == 0 && e2 == hipSuccess && graph) e = hipGraphInstantiate(&s->graph_exec, graph, nullptr, nullptr, 0);
+                else e = e2 == hipSuccess ? hipErrorUnknown : e2;
+                if (graph) hipGraphDestroy(graph);
+            }
+            if (e != hipSuccess || !s->graph_exec) {
+                (void)hipGetLastError();
+                s->graph_exec = nullptr;
+                s->graph_failed = true;
+            }
+        }
+        if (s->graph_exec) {
+            HIP_TRY(hipGraphLaunch(s->graph_exec, c->stream));
+            return 0;
+        }
+    }
+    for (auto& l : s->launches)
+        if (int r = issue_launch(c, l)) return r;
     return 0;
 }
 
@@ -366,6 +404,7 @@ int vkj_seq_destroy(vkj_handle sh) {
     for (auto& t : s->uploads)   if (t.staging) hipHostFree(t.staging);
     for (auto& t : s->downloads) if (t.staging) hipHostFree(t.staging);
     for (auto e : s->stamps) hipEventDestroy(e);
+    drop_graph(s);
     retire(s);
     delete s;
     return 0;
@@ -427,6 +466,7 @@ int vkj_seq_record_launch(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], 
         memcpy(l.kernarg.data() + buf_arg_offsets[i], &addr, 8);
     }
     s->launches.push_back(std::move(l));
+    drop_graph(s);                                  // a captured graph no longer matches the sequence
     return 0;
 }
 
@@ -466,9 +506,13 @@ int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t fla
         HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
     }
     if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[1], c->stream));
-    for (size_t i = 0; i < s->launches.size(); i++) {
-        if (int r = issue_launch(c, s->launches[i])) return r;
-        if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[2 + i], c->stream));
+    if (s->profiling) {
+        for (size_t i = 0; i < s->launches.size(); i++) {
+            if (int r = issue_launch(c, s->launches[i])) return r;
+            HIP_TRY(hipEventRecord(s->stamps[2 + i], c->stream));
+        }
+    } else if (int r = issue_all(c, s)) {
+        return r;
     }
     if (down) for (auto& t : s->downloads) {
         if (!t.nbytes) continue;
@@ -489,13 +533,20 @@ int vkj_seq_replay(vkj_handle sh, int iters, float* ms_total) {
     if (int r = use(c)) return r;
     HIP_TRY(hipEventRecord(c->ev_begin, c->stream));
     for (int it = 0; it < iters; it++)
-        for (auto& l : s->launches)
-            if (int r = issue_launch(c, l)) return r;
+        if (int r = issue_all(c, s)) return r;
     HIP_TRY(hipEventRecord(c->ev_end, c->stream));
     HIP_TRY(hipEventSynchronize(c->ev_end));
     float ms = 0.f;
     HIP_TRY(hipEventElapsedTime(&ms, c->ev_begin, c->ev_end));
     if (ms_total) *ms_total = ms;
+    return 0;
+}
+
+int vkj_seq_use_graph(vkj_handle sh, int enable) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_use_graph: bad handle");
+    s->want_graph = enable != 0;
+    if (!s->want_graph) drop_graph(s);
     return 0;
 }
 

@@ -60,6 +60,7 @@ _PROTOTYPES = {
     'vkj_seq_num_steps':       (C.c_int, [_H, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     'vkj_seq_eval':            (C.c_int, [_H, C.POINTER(C.c_void_p), C.c_int, C.c_uint32]),
     'vkj_seq_replay':          (C.c_int, [_H, C.c_int, C.POINTER(C.c_float)]),
+    'vkj_seq_use_graph':       (C.c_int, [_H, C.c_int]),
     'vkj_seq_timestamps':      (C.c_int, [_H, C.POINTER(C.c_float), C.c_int, C.POINTER(C.c_int)]),
 }
 
@@ -285,6 +286,10 @@ class Sequence:
         ms = C.c_float(0)
         _check(self.device.lib.vkj_seq_replay(self.handle, iters, C.byref(ms)), 'vkj_seq_replay')
         return ms.value
+
+    def use_graph(self, enable: bool = True):
+        '''Issue the recorded launches as one captured HIP graph from the next eval / replay on.'''
+        _check(self.device.lib.vkj_seq_use_graph(self.handle, int(bool(enable))), 'vkj_seq_use_graph')
 
     def get_timestamps(self) -> np.ndarray:
         n = C.c_int(0)

@@ -21,8 +21,10 @@ from .minijax import core, tree_util
 
 class JaxprInterpreter:
     def __init__(self, jaxpr, static_argnums: tp.Tuple[int, ...] = (), profiling: bool = False,
-                 reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False):
+                 reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False, graph: bool = False):
         self.jaxpr          = jaxpr
+        #graph=True replays the launches as one captured HIP graph (never with profiling)
+        self.graph          = graph and not profiling
         self.static_argnums = tuple(static_argnums)
         self.profiling      = profiling
         self.fuse           = fuse
@@ -69,6 +71,8 @@ class JaxprInterpreter:
             for (b, _), (t, _) in zip(launch.buffers, bufs):
                 assert b is None or t is not None, f'{op}: buffer without storage'
             self.sequence.record_launch(launch.kernel, launch.grid, launch.block, bufs, launch.params, launch.lds)
+        if self.graph:
+            self.sequence.use_graph(True)
         self._output_slots = []
         self._output_arrays = []
         for b in self.output_buffers:
