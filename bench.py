@@ -47,6 +47,8 @@ def main():
     ap.add_argument('--batch', type=int, default=None)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-fuse', action='store_true')
+    ap.add_argument('--end-to-end', action='store_true',
+                    help='also time whole calls through wrap() (uploads, launches, downloads, Python), median of 5')
     ap.add_argument('--graph', action='store_true', help='replay the launches as one captured HIP graph')
     ap.add_argument('--profile-iters', type=int, default=3)
     ap.add_argument('--dump-launches', default=None, help='write one line per launch (kernel, grid, FLOP, bytes, ms) to this file')
@@ -155,6 +157,23 @@ def main():
 
     roofline['traffic'] = measured_hbm_traffic(args.workload, dominant)
 
+    #end-to-end calls through wrap(): host arrays in, host arrays out, uploads and Python included;
+    #once copying every argument per call (what the reference does), once with the weights resident
+    end_to_end = {}
+    if args.end_to_end:
+        import statistics
+        for label, kw in (('all_arguments_copied_ms', {}), ('weights_resident_ms', dict(resident_argnums=(0,)))):
+            if label == 'weights_resident_ms' and not isinstance(inputs[0], dict):
+                continue
+            f = vkjax_amd.wrap(fn, frontend='minijax', fuse=not args.no_fuse, **kw)
+            f(*inputs)
+            times = []
+            for _ in range(5):
+                t0 = time.perf_counter()
+                f(*inputs)
+                times.append((time.perf_counter() - t0) * 1e3)
+            end_to_end[label] = round(statistics.median(times), 3)
+
     cpu_baseline = None
     if not args.no_cpu_baseline:
         cpu_baseline = time_cpu_baseline(args.workload, fn, make_inputs, kwargs)
@@ -167,7 +186,8 @@ def main():
         'config': {'workload': args.workload, 'input_shape': list(leaves[-1].shape) if hasattr(leaves[-1], 'shape') else None,
                    'launches_per_step': len(interp.launches), 'fused': interp.fuse, 'inputs_resident_in_hbm': True,
                    'device': props['device_name'], 'arch': props['arch'], 'compute_units': props['compute_units'],
-                   'hbm_bytes_allocated': interp.bufferpool.total_device_bytes(), 'build_seconds': round(build_s, 2)},
+                   'hbm_bytes_allocated': interp.bufferpool.total_device_bytes(), 'build_seconds': round(build_s, 2),
+                   **({'end_to_end_call': end_to_end} if end_to_end else {})},
         'roofline': roofline, 'kernels': kernels, 'cpu_baseline': cpu_baseline,
     }
     print(json.dumps(out))

@@ -38,7 +38,8 @@ enum {
 enum {
     VKJ_EVAL_DEFAULT        = 0,
     VKJ_EVAL_SKIP_UPLOADS   = 1,   /* inputs are already resident in HBM */
-    VKJ_EVAL_SKIP_DOWNLOADS = 2
+    VKJ_EVAL_SKIP_DOWNLOADS = 2,
+    VKJ_EVAL_NULL_IS_RESIDENT = 4  /* an upload slot whose host pointer is NULL is skipped: its buffer keeps what it holds */
 };
 
 typedef struct vkj_props {

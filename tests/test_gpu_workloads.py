@@ -199,3 +199,23 @@ def test_graph_replay_matches_individual_launches():
             plain(*make())                            #unrelated eager work between graph launches
         interp = list(graph._jaxpr_interpreters.values())[0]
         assert interp.graph
+
+
+def test_resident_arguments_are_uploaded_once():
+    '''resident_argnums: a weight leaf is uploaded when the object passed for it changes, and only
+    then; other arguments are copied on every call as in the reference.'''
+    params, x = W.mlp_inputs()
+    plain    = vkjax_amd.wrap(W.mlp, frontend='minijax')
+    resident = vkjax_amd.wrap(W.mlp, frontend='minijax', resident_argnums=(0,))
+    assert_tree_close(resident(params, x), plain(params, x), exact=True, what='first call')
+    x2 = x[::-1].copy()
+    assert_tree_close(resident(params, x2), plain(params, x2), exact=True, what='new activations, same weights')
+    #a replaced leaf is picked up, the untouched ones stay where they are
+    from vkjax_amd.minijax import tree_util
+    leaves, structure = tree_util.tree_flatten(params)
+    leaves2 = list(leaves)
+    leaves2[0] = leaves[0] * np.float32(0.5)
+    params2 = tree_util.tree_unflatten(structure, leaves2)
+    assert_tree_close(resident(params2, x2), plain(params2, x2), exact=True, what='one weight replaced')
+    interp = list(resident._jaxpr_interpreters.values())[0]
+    assert len(interp._resident_leaves) == len(leaves)

@@ -486,7 +486,9 @@ int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t fla
     if (int r = use(c)) return r;
     const bool up = !(flags & VKJ_EVAL_SKIP_UPLOADS), down = !(flags & VKJ_EVAL_SKIP_DOWNLOADS);
     auto slot_ok = [&](const Transfer& t) { return t.nbytes == 0 || (host_ptrs && t.slot < nslots && host_ptrs[t.slot]); };
-    if (up)   for (auto& t : s->uploads)   if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for upload slot %d", t.slot);
+    const bool null_resident = flags & VKJ_EVAL_NULL_IS_RESIDENT;
+    if (up)   for (auto& t : s->uploads)   if (!slot_ok(t) && !(null_resident && host_ptrs && t.slot < nslots))
+        return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for upload slot %d", t.slot);
     if (down) for (auto& t : s->downloads) if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for download slot %d", t.slot);
 
     size_t nstamps = 0;
@@ -501,7 +503,7 @@ int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t fla
         HIP_TRY(hipEventRecord(s->stamps[0], c->stream));
     }
     if (up) for (auto& t : s->uploads) {
-        if (!t.nbytes) continue;
+        if (!t.nbytes || !host_ptrs[t.slot]) continue;
         memcpy(t.staging, host_ptrs[t.slot], t.nbytes);
         HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
     }

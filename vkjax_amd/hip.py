@@ -21,6 +21,7 @@ KERNEL_MODULES = ('elementwise', 'conv_gemm', 'reduce', 'index', 'threefry')
 
 EVAL_SKIP_UPLOADS   = 1
 EVAL_SKIP_DOWNLOADS = 2
+EVAL_NULL_IS_RESIDENT = 4
 
 
 class Props(C.Structure):

@@ -21,8 +21,14 @@ from .minijax import core, tree_util
 
 class JaxprInterpreter:
     def __init__(self, jaxpr, static_argnums: tp.Tuple[int, ...] = (), profiling: bool = False,
-                 reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False, graph: bool = False):
+                 reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False, graph: bool = False,
+                 resident_argnums: tp.Tuple[int, ...] = ()):
         self.jaxpr          = jaxpr
+        #Arguments named here (weights, tables) stay in HBM between calls: a leaf is uploaded when the
+        #object passed for it is not the one uploaded last. Changing such an array in place is not
+        #noticed (the reference copies every argument on every call, vkjax/kompute_jaxpr_interpreter.py:72-75).
+        self.resident_argnums = tuple(resident_argnums)
+        self._resident_leaves = {}
         #graph=True replays the launches as one captured HIP graph (never with profiling)
         self.graph          = graph and not profiling
         self.static_argnums = tuple(static_argnums)
@@ -83,22 +89,32 @@ class JaxprInterpreter:
             self._output_slots.append(self.sequence.record_download(b.tensor, b.nbytes()))
             self._output_arrays.append(np.zeros(b.size, dtype=np.uint32))
 
-    def _flatten_args(self, X):
-        X = tree_util.tree_leaves([x for i, x in enumerate(X) if i not in self.static_argnums])
-        if len(self.input_buffers) != len(X):
-            raise TypeError(f'Expected {len(self.input_buffers)} input arguments, received {len(X)}')
-        return X
+    def _flatten_args(self, X, with_residency: bool = False):
+        leaves, resident = [], []
+        for i, x in enumerate(X):
+            if i in self.static_argnums:
+                continue
+            these = tree_util.tree_leaves([x])
+            leaves   += these
+            resident += [i in self.resident_argnums] * len(these)
+        if len(self.input_buffers) != len(leaves):
+            raise TypeError(f'Expected {len(self.input_buffers)} input arguments, received {len(leaves)}')
+        return (leaves, resident) if with_residency else leaves
 
     def run(self, *X, return_all=False):
         '''Executes a previously recorded sequence with actual data'''
-        X = self._flatten_args(X)
+        X, resident = self._flatten_args(X, with_residency=True)
         if self.sequence is None:
             raise RuntimeError('this interpreter was built with plan_only=True and has no device to run on')
         host = [None] * self.sequence.n_slots
         keep = []
-        for slot, x, var in zip(self._input_slots, X, self.jaxpr.jaxpr.invars):
+        for k, (slot, x, var) in enumerate(zip(self._input_slots, X, self.jaxpr.jaxpr.invars)):
             if slot is None:
                 continue
+            if resident[k]:
+                if self._resident_leaves.get(k) is x:
+                    continue                                    #already in HBM
+                self._resident_leaves[k] = x
             words = to_device_words(np.asarray(x), core.canonicalize_dtype(var.aval.dtype))
             if words.size != int(np.prod(var.aval.shape, dtype=np.int64)):
                 raise TypeError(f'argument of shape {np.shape(x)} does not match the traced shape {var.aval.shape}')
@@ -107,7 +123,7 @@ class JaxprInterpreter:
         for slot, arr in zip(self._output_slots, self._output_arrays):
             if slot is not None:
                 host[slot] = arr
-        self.sequence.eval(host)
+        self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT if self.resident_argnums else 0)
 
         output_values = []
         for b, arr in zip(self.output_buffers, self._output_arrays):
