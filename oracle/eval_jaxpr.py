@@ -13,15 +13,23 @@ _CALLS = {
     'xla_call':              lambda params: params['call_jaxpr'],
     'core_call':             lambda params: params['call_jaxpr'],
     'pjit':                  lambda params: params['jaxpr'],
+    'jit':                   lambda params: params['jaxpr'],
     'closed_call':           lambda params: params['call_jaxpr'],
     'custom_jvp_call_jaxpr': lambda params: params['fun_jaxpr'],
     'custom_jvp_call':       lambda params: params['call_jaxpr'],
 }
 
 
+def _physical(aval):
+    '''A typed key array is held as its uint32 words: one more trailing dimension of 2.'''
+    if type(aval.dtype).__name__ == 'KeyTy':
+        return tuple(aval.shape) + (2,), np.dtype('uint32')
+    return tuple(aval.shape), aval.dtype
+
+
 def _canon_input(x, aval):
-    x = np.asarray(x)
-    return np.asarray(x, dtype=aval.dtype).reshape(aval.shape)
+    shape, dtype = _physical(aval)
+    return np.asarray(np.asarray(x), dtype=dtype).reshape(shape)
 
 
 def eval_jaxpr(jaxpr, consts, *args, return_env=False):
@@ -60,8 +68,9 @@ def eval_jaxpr(jaxpr, consts, *args, return_env=False):
                 outvals = [outvals]
         for v, val in zip(eqn.outvars, outvals):
             val = np.asarray(val)
-            assert val.shape == tuple(v.aval.shape), (name, val.shape, v.aval.shape)
-            assert val.dtype == v.aval.dtype, (name, val.dtype, v.aval.dtype)
+            shape, dtype = _physical(v.aval)
+            assert val.shape == shape, (name, val.shape, shape)
+            assert val.dtype == dtype, (name, val.dtype, dtype)
             env[v] = val
 
     outs = [read(v) for v in jaxpr.outvars]

@@ -24,7 +24,10 @@ written from vkjax/shaders/conv2d.comp:44-95, against torch.nn.functional.conv2d
 and against the delta-kernel and 1x1 == GEMM special cases; reduce_window against brute force
 and torch max_pool2d / avg_pool2d; gather / scatter-add against brute-force loops over the
 XLA index rule and numpy fancy indexing / np.add.at; reductions and elementwise ops against
-closed forms and hand-computed values. Parity unpinned: the *jaxpr expansions* (which
+closed forms and hand-computed values; the key primitives of newer jax versions (random_bits,
+random_split, ...) in the original counter layout against that same expansion and in the
+partitionable layout against the values jax's documentation prints (tests/test_key_primitives.py).
+Parity unpinned: the *jaxpr expansions* (which
 primitives jax emits for jnp.dot, softmax, indexing, random.uniform) - they are produced by
 jax, which is not importable here, and are restated from the reference's accepted-parameter
 lists only.
@@ -164,6 +167,52 @@ acosh, asinh, atanh = _un64(np.arccosh), _un64(np.arcsinh), _un64(np.arctanh)
 ceil, floor = _un64(np.ceil), _un64(np.floor)
 
 
+logistic = _un64(lambda x: 1.0 / (1.0 + np.exp(-x)))
+log1p, expm1, exp2, cbrt = _un64(np.log1p), _un64(np.expm1), _un64(np.exp2), _un64(np.cbrt)
+
+
+def atan2(a, b):
+    return np.arctan2(_canon(a).astype(np.float64), _canon(b).astype(np.float64)).astype(f32)
+
+
+def is_finite(x):
+    return np.isfinite(_canon(x))
+
+
+def round(x, rounding_method=0, **_):
+    '''rounding_method 0: halves away from zero; 1: halves to even (jax.lax.RoundingMethod).'''
+    x = _canon(x).astype(np.float64)
+    if int(getattr(rounding_method, 'value', rounding_method)) == 1:
+        return np.rint(x).astype(f32)
+    return (np.sign(x) * np.floor(np.abs(x) + 0.5)).astype(f32)
+
+
+def square(x):
+    return mul(x, x)
+
+
+def clamp(lo, x, hi):
+    return globals()['min'](globals()['max'](x, lo), hi)
+
+
+def population_count(x):
+    x = _canon(x)
+    return np.array([bin(int(v) & 0xFFFFFFFF).count('1') for v in x.reshape(-1)], dtype=x.dtype).reshape(x.shape)
+
+
+def clz(x):
+    x = _canon(x)
+    return np.array([32 - (int(v) & 0xFFFFFFFF).bit_length() for v in x.reshape(-1)], dtype=x.dtype).reshape(x.shape)
+
+
+def _not(x):
+    x = _canon(x)
+    return ~x
+
+
+globals()['not'] = _not
+
+
 def erf(x):
     from scipy import special
     return special.erf(_canon(x).astype(np.float64)).astype(f32)
@@ -252,6 +301,15 @@ def broadcast_in_dim(x, shape, broadcast_dimensions, **_):
 def reshape(x, new_sizes, dimensions=None, **_):
     assert dimensions is None
     return _canon(x).reshape(new_sizes)
+
+
+def split(x, sizes, axis, **_):
+    edges = np.cumsum([0] + [int(n) for n in sizes])
+    return [np.take(x, np.arange(edges[i], edges[i + 1]), axis=axis) for i in range(len(sizes))]
+
+
+def expand_dims(x, dimensions, **_):
+    return np.expand_dims(x, tuple(dimensions))
 
 
 def squeeze(x, dimensions, **_):
@@ -529,3 +587,67 @@ def threefry2x32(key0, key1, x0, x1):
         a = (a + ks[(i + 1) % 3]) & M
         b = (b + ks[(i + 2) % 3] + np.uint64(i + 1)) & M
     return a.astype(u32), b.astype(u32)
+
+
+# Key primitives of newer jax versions (jax/_src/prng.py: threefry_seed, threefry_split,
+# threefry_fold_in, threefry_random_bits). A key array is held as its uint32 words, shape
+# (..., 2). Both counter layouts of jax are restated; which one applies is jax's configuration
+# flag `jax_threefry_partitionable`, mirrored here by THREEFRY_PARTITIONABLE. Pins: the original
+# layout against the published split(PRNGKey(0)) / uniform(PRNGKey(0)) values, the partitionable
+# layout against the values jax's documentation prints for uniform(key(0)) = 0.947667 and
+# uniform(split(key(0))[1]) = 0.00729382.
+THREEFRY_PARTITIONABLE = False
+
+
+def random_wrap(x, **_):
+    return np.asarray(x, u32)
+
+
+def random_unwrap(x, **_):
+    return np.asarray(x, u32)
+
+
+def random_seed(seeds, **_):
+    seeds = _canon(seeds)
+    low   = (seeds.astype(np.int64) & 0xFFFFFFFF).astype(u32)
+    return np.stack([np.zeros_like(low), low], axis=-1)
+
+
+def _threefry_2x32_flat(key, counts):
+    '''jax's threefry_2x32: the flat counters are split into two halves (one zero appended when
+    the count is odd), run through the block function, joined again and trimmed.'''
+    n    = counts.size
+    flat = np.concatenate([counts.reshape(-1), np.zeros(n % 2, u32)])
+    a, b = threefry2x32(key[0], key[1], flat[:flat.size // 2], flat[flat.size // 2:])
+    return np.concatenate([a, b])[:n].reshape(counts.shape)
+
+
+def _single_key(keys):
+    keys = np.asarray(keys, u32)
+    if keys.shape != (2,):
+        raise NotImplementedError('batched keys')
+    return keys
+
+
+def random_bits(keys, bit_width, shape, **_):
+    assert bit_width == 32
+    key = _single_key(keys)
+    n   = int(np.prod(shape, dtype=np.int64))
+    if THREEFRY_PARTITIONABLE:
+        hi, lo = threefry2x32(key[0], key[1], np.zeros(n, u32), np.arange(n, dtype=u32))
+        return (hi ^ lo).reshape(shape)
+    return _threefry_2x32_flat(key, np.arange(n, dtype=u32)).reshape(shape)
+
+
+def random_split(keys, shape, **_):
+    key = _single_key(keys)
+    num = int(np.prod(shape, dtype=np.int64))
+    if THREEFRY_PARTITIONABLE:
+        hi, lo = threefry2x32(key[0], key[1], np.zeros(num, u32), np.arange(num, dtype=u32))
+        return np.stack([hi, lo], axis=-1).reshape(tuple(shape) + (2,))
+    return _threefry_2x32_flat(key, np.arange(2 * num, dtype=u32)).reshape(tuple(shape) + (2,))
+
+
+def random_fold_in(keys, msgs, **_):
+    key = _single_key(keys)
+    return _threefry_2x32_flat(key, np.array([0, np.asarray(msgs, u32).reshape(())], dtype=u32))

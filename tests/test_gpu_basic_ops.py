@@ -211,6 +211,40 @@ param_matrix = [
     (lax.nextafter, 'nextafter(X,Y)',   [random([77, 101]) * 2 - 1, random([77, 101])]),
 ]
 
+#names newer jax versions trace (jax.nn.sigmoid -> logistic, x**2 -> square, jnp.logical_not -> not, jnp.split -> split, ...)
+def split0(x): return lax.split(x, (3, 0, 90, 6), axis=1)
+def split1(x): return [p * 2.0 for p in lax.split(x + 1.0, (5, 2), axis=0)]
+def clamp0(x): return lax.clamp(-0.25, x, 0.5)
+def clamp1(lo, x, hi): return lax.clamp(lo, x, hi)
+def round_even(x): return lax.round(x, 1)
+_special = np.array([0.0, -0.0, 1.5, -2.5, np.inf, -np.inf, np.nan, 3e38, 1e-45] * 13, np.float32)
+_halves  = np.concatenate([np.arange(-20, 20) + 0.5, random([500]) * 20 - 10, [0.0, -0.0, 2.5, 3.5, -2.5]]).astype(np.float32)
+
+param_matrix += [
+    (lax.logistic, 'logistic',          [random([77, 101]) * 20 - 10]),
+    (lax.log1p, 'log1p',                [random([77, 101]) * 2 - 0.99]),
+    (lax.log1p, 'log1p tiny',           [(random([77, 101]) * 2 - 1) * 1e-6]),
+    (lax.expm1, 'expm1',                [random([77, 101]) * 4 - 2]),
+    (lax.expm1, 'expm1 tiny',           [(random([77, 101]) * 2 - 1) * 1e-6]),
+    (lax.exp2, 'exp2',                  [random([77, 101]) * 40 - 20]),
+    (lax.cbrt, 'cbrt',                  [random([77, 101]) * 2000 - 1000]),
+    (lax.atan2, 'atan2',                [random([77, 101]) * 2 - 1, random([77, 101]) * 2 - 1]),
+    (lax.is_finite, 'is_finite',        [_special]),
+    (lax.bitwise_not, 'not bool',       [random([77, 101]) > 0.5]),
+    (lax.bitwise_not, 'not int',        [randint(-2**31, 2**31, size=[77, 101])]),
+    (lax.population_count, 'popcount',  [randint(0, 2**32, size=[77, 101], dtype=np.uint64).astype(np.uint32)]),
+    (lax.clz, 'clz',                    [np.concatenate([[0, 1, 2**31, 2**32 - 1], 2**randint(0, 32, size=500) - 1]).astype(np.uint32)]),
+    (lax.square, 'square float',        [random([77, 101]) * 20 - 10]),
+    (lax.square, 'square int',          [randint(-100000, 100000, size=[77, 101])]),
+    (lax.round, 'round away',           [_halves]),
+    (round_even, 'round even',          [_halves]),
+    (clamp0, 'clamp scalars',           [random([77, 101]) * 2 - 1]),
+    (clamp1, 'clamp arrays',            [random([77, 101]) - 1, random([77, 101]) * 2 - 1, random([77, 101])]),
+    (clamp0, 'clamp int',               [randint(-5, 5, size=[77, 101])]),
+    (split0, 'split axis 1',            [random([7, 99, 5])]),
+    (split1, 'split + chains',          [random([7, 33])]),
+]
+
 for fname in ['cos', 'sin', 'tan', 'cosh', 'sinh', 'tanh', 'acos', 'asin', 'atan', 'acosh', 'asinh', 'atanh',
               'ceil', 'floor', 'sign']:
     param_matrix += [(getattr(lax, fname), fname, [random([77, 101]) * 2 - 1])]
@@ -223,6 +257,10 @@ TOLERANCES = {
     'sin':           (1e-5, 1e-6),
     'sinh':          (1e-5, 1e-6),
     'tan':           (1e-5, 1e-6),
+    'log1p tiny':    (1e-5, 1e-12),
+    'expm1 tiny':    (1e-5, 1e-12),
+    'expm1':         (1e-5, 1e-7),
+    'atan2':         (1e-5, 1e-7),
     #dot: north-star tolerance for contractions
     'dot0 x@y': (1e-4, 1e-8), 'dot1 x@const': (1e-4, 1e-8), 'dot axes=(0,0)': (1e-4, 1e-8),
     'dot axes=(1,1)': (1e-4, 1e-8), 'dot axes=(0,1)': (1e-4, 1e-8), 'reshape_dot': (1e-4, 1e-8),

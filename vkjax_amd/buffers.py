@@ -156,7 +156,8 @@ class BufferPool:
         if varhash not in self.buffers:
             if _is_unit(var.aval):
                 return None
-            self.buffers[varhash] = Buffer(None, core.canonicalize_dtype(var.aval.dtype), var.aval.shape)
+            shape, dtype = core.physical(var.aval)
+            self.buffers[varhash] = Buffer(None, dtype, shape)
         b = self.buffers[varhash]
         if b is None:
             return None
@@ -214,13 +215,13 @@ class BufferPool:
         return None
 
     def _create_tensor(self, var, initial_value=None):
-        dtype = core.canonicalize_dtype(var.aval.dtype)
+        shape, dtype = core.physical(var.aval)
         if core.is_literal(var):
             initial_value = var.val
         if initial_value is None:
-            return self.device.alloc(max(int(np.prod(var.aval.shape, dtype=np.int64)) * 4, 4))
+            return self.device.alloc(max(int(np.prod(shape, dtype=np.int64)) * 4, 4))
         initial_value = np.asarray(initial_value)
-        assert initial_value.size == int(np.prod(var.aval.shape, dtype=np.int64)), (initial_value.shape, var.aval.shape)
+        assert initial_value.size == int(np.prod(shape, dtype=np.int64)), (initial_value.shape, shape)
         return self.device.tensor(to_device_words(initial_value, dtype))
 
     def unique_tensors(self) -> set:

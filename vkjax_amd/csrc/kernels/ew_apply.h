@@ -51,6 +51,19 @@ __device__ __noinline__ uint32_t ew_apply_rare(uint32_t op, uint32_t a, uint32_t
         case EW_ACOSH_F:     return f2u(acoshf(x));
         case EW_ASINH_F:     return f2u(asinhf(x));
         case EW_ATANH_F:     return f2u(atanhf(x));
+        case EW_LOGISTIC_F:  return f2u(1.0f / (1.0f + expf(-x)));
+        case EW_LOG1P_F:     return f2u(log1pf(x));
+        case EW_EXPM1_F:     return f2u(expm1f(x));
+        case EW_EXP2_F:      return f2u(exp2f(x));
+        case EW_ISFINITE_F:  return (a & 0x7F800000u) != 0x7F800000u;
+        case EW_NOT_X:       return ~a;
+        case EW_NOT_B:       return a == 0u;
+        case EW_ROUND_AWAY_F: return f2u(roundf(x));           // halves away from zero
+        case EW_ROUND_EVEN_F: return f2u(rintf(x));            // halves to even (default rounding mode)
+        case EW_ATAN2_F:     return f2u(atan2f(x, y));
+        case EW_CBRT_F:      return f2u(cbrtf(x));
+        case EW_POPCNT_X:    return (uint32_t)__popc(a);
+        case EW_CLZ_X:       return a == 0u ? 32u : (uint32_t)__clz((int)a);
         case EW_DIV_I: { int32_t p = (int32_t)a, q = (int32_t)b;
                          return q == 0 ? 0xFFFFFFFFu : (p == INT32_MIN && q == -1) ? (uint32_t)INT32_MIN : (uint32_t)(p / q); }
         case EW_DIV_U:       return b == 0 ? 0xFFFFFFFFu : a / b;

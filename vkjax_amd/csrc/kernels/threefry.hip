@@ -84,63 +84,106 @@ extern "C" __global__ __launch_bounds__(256) void threefry2x32_v4(uint32_t* out0
 #define TF_MAX_STEPS 8
 
 struct ThreefryStreamParams {
-    uint32_t h;                        // elements per half: the output has 2h
-    uint32_t c0, c1;                   // first counter of each half
+    uint32_t h;                        // blocks to run (halves layout: the output has up to 2h elements)
+    uint32_t c0, c1;                   // first counter of each word
     uint32_t nsteps;                   // element-wise steps applied to the bits (0..8)
     uint32_t op[TF_MAX_STEPS];         // opcode of step k
     uint32_t flags[TF_MAX_STEPS];      // bit0: the step has an operand (a single value); bit1: it is the LEFT argument
     uint32_t imm[TF_MAX_STEPS];        // immediate of step k (integer_pow exponent)
+    uint32_t n;                        // halves layout: elements of the output (2h, or 2h - 1 for an odd-sized draw)
 };
 
 struct ThreefryStreamPtrs { const uint32_t* p[TF_MAX_STEPS]; };
 
-template <int VEC>
-__device__ __forceinline__ void threefry_stream_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ key0,
-                                                     const uint32_t* __restrict__ key1, const ThreefryStreamPtrs& operands,
-                                                     const ThreefryStreamParams& P) {
-    const uint32_t j0 = (blockIdx.x * 256u + threadIdx.x) * VEC;
-    if (j0 >= P.h) return;
-    const uint32_t k0 = key0[0], k1 = key1[0];
-    uint32_t y[2 * VEC];                             // [0, VEC): first results, [VEC, 2 VEC): second results
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-        y[j]       = P.c0 + j0 + j;
-        y[VEC + j] = P.c1 + j0 + j;
-        threefry_block(k0, k1, y[j], y[VEC + j]);
-    }
-    // The step loop stays rolled (one copy of the opcode switch). Its descriptors are read from the
-    // argument block through the kernel-argument pointer: indexing the by-value argument with a
-    // run-time value would make the compiler copy it to scratch memory. Layout of the block:
-    // out, key0, key1 (24 bytes), the operand pointers (64 bytes), then ThreefryStreamParams.
+// Counter layouts of the stream kernels:
+//   HALVES  x0 = c0 + j, x1 = c1 + j;  out[j] = y0, out[h + j] = y1      (jax's original layout; an
+//           odd-sized draw pads the counters with one zero and drops the last result, so the x1
+//           counter of element n is 0 and that element is not stored)
+//   XOR     x0 = c0, x1 = c1 + j;      out[j] = y0 ^ y1                   (jax's partitionable layout:
+//           the 64-bit flat index of the element is the counter, 32 bits per word)
+//   PAIRS   x0 = c0, x1 = c1 + j;      out[2j] = y0, out[2j + 1] = y1     (partitionable key split)
+enum { TF_HALVES = 0, TF_XOR = 1, TF_PAIRS = 2 };
+
+// Applies the element-wise steps to y. The step loop stays rolled (one copy of the opcode switch).
+// Its descriptors are read from the argument block through the kernel-argument pointer: indexing
+// the by-value argument with a run-time value would make the compiler copy it to scratch memory.
+// Layout of the block: out, key0, key1 (24 bytes), the operand pointers (64 bytes), then
+// ThreefryStreamParams.
+template <int NV>
+__device__ __forceinline__ void threefry_stream_steps(uint32_t (&y)[NV], uint32_t nsteps) {
     const char* const args = reinterpret_cast<const char*>(__builtin_amdgcn_kernarg_segment_ptr());
     const uint32_t* const* const op_ptr = reinterpret_cast<const uint32_t* const*>(args + 24);
     const uint32_t* const desc = reinterpret_cast<const uint32_t*>(args + 24 + 8 * TF_MAX_STEPS) + 4;
 #pragma nounroll
-    for (uint32_t k = 0; k < P.nsteps; ++k) {
+    for (uint32_t k = 0; k < nsteps; ++k) {
         const uint32_t op = desc[k], flags = desc[TF_MAX_STEPS + k], imm = desc[2 * TF_MAX_STEPS + k];
         const uint32_t o = (flags & 1u) ? op_ptr[k][0] : 0u;                  // uniform address: a scalar load
-        uint32_t v[2 * VEC];
+        uint32_t v[NV];
 #pragma unroll
-        for (int j = 0; j < 2 * VEC; ++j) v[j] = o;
-        ew_apply_vec<2 * VEC>(op, y, v, (flags & 2u) != 0, imm);
-    }
-    if constexpr (VEC == 4) {
-        u32x4 va, vb;
-        va.x = y[0]; va.y = y[1]; va.z = y[2]; va.w = y[3];
-        vb.x = y[4]; vb.y = y[5]; vb.z = y[6]; vb.w = y[7];
-        *reinterpret_cast<u32x4*>(out + j0) = va;
-        *reinterpret_cast<u32x4*>(out + P.h + j0) = vb;
-    } else {
-        out[j0] = y[0]; out[P.h + j0] = y[1];
+        for (int j = 0; j < NV; ++j) v[j] = o;
+        ew_apply_vec<NV>(op, y, v, (flags & 2u) != 0, imm);
     }
 }
 
-extern "C" __global__ __launch_bounds__(256) void threefry2x32_stream_v1(uint32_t* out, const uint32_t* key0, const uint32_t* key1,
-                                                                         ThreefryStreamPtrs operands, ThreefryStreamParams P) {
-    threefry_stream_body<1>(out, key0, key1, operands, P);
+template <int VEC, int MODE>
+__device__ __forceinline__ void threefry_stream_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ key0,
+                                                     const uint32_t* __restrict__ key1, const ThreefryStreamParams& P) {
+    const uint32_t j0 = (blockIdx.x * 256u + threadIdx.x) * VEC;
+    if (j0 >= P.h) return;
+    const uint32_t k0 = key0[0], k1 = key1[0];
+    if constexpr (MODE == TF_HALVES) {
+        uint32_t y[2 * VEC];                         // [0, VEC): first results, [VEC, 2 VEC): second results
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            y[j]       = P.c0 + j0 + j;
+            y[VEC + j] = P.c1 + j0 + j;
+            if (VEC == 1 && P.h + j0 >= P.n) y[VEC] = 0u;           // the padding counter of an odd-sized draw
+            threefry_block(k0, k1, y[j], y[VEC + j]);
+        }
+        threefry_stream_steps<2 * VEC>(y, P.nsteps);
+        if constexpr (VEC == 4) {
+            u32x4 va, vb;
+            va.x = y[0]; va.y = y[1]; va.z = y[2]; va.w = y[3];
+            vb.x = y[4]; vb.y = y[5]; vb.z = y[6]; vb.w = y[7];
+            *reinterpret_cast<u32x4*>(out + j0) = va;
+            *reinterpret_cast<u32x4*>(out + P.h + j0) = vb;
+        } else {
+            out[j0] = y[0];
+            if (P.h + j0 < P.n) out[P.h + j0] = y[1];
+        }
+    } else {
+        uint32_t y[VEC], z[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            y[j] = P.c0;
+            z[j] = P.c1 + j0 + j;
+            threefry_block(k0, k1, y[j], z[j]);
+        }
+        if constexpr (MODE == TF_PAIRS) {
+            static_assert(VEC == 1, "pairs are written one block per thread");
+            out[2 * j0] = y[0]; out[2 * j0 + 1] = z[0];
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) y[j] ^= z[j];
+            threefry_stream_steps<VEC>(y, P.nsteps);
+            if constexpr (VEC == 4) {
+                u32x4 va;
+                va.x = y[0]; va.y = y[1]; va.z = y[2]; va.w = y[3];
+                *reinterpret_cast<u32x4*>(out + j0) = va;
+            } else {
+                out[j0] = y[0];
+            }
+        }
+    }
 }
-// requires h % 4 == 0 and a 16-byte aligned output
-extern "C" __global__ __launch_bounds__(256) void threefry2x32_stream_v4(uint32_t* out, const uint32_t* key0, const uint32_t* key1,
-                                                                         ThreefryStreamPtrs operands, ThreefryStreamParams P) {
-    threefry_stream_body<4>(out, key0, key1, operands, P);
-}
+
+#define TF_STREAM_KERNEL(name, VEC, MODE)                                                                              \
+    extern "C" __global__ __launch_bounds__(256) void name(uint32_t* out, const uint32_t* key0, const uint32_t* key1,  \
+                                                           ThreefryStreamPtrs operands, ThreefryStreamParams P) {      \
+        threefry_stream_body<VEC, MODE>(out, key0, key1, P);                                                           \
+    }
+TF_STREAM_KERNEL(threefry2x32_stream_v1, 1, TF_HALVES)
+TF_STREAM_KERNEL(threefry2x32_stream_v4, 4, TF_HALVES)          // requires h % 4 == 0, n == 2h and a 16-byte aligned output
+TF_STREAM_KERNEL(threefry2x32_stream_xor_v1, 1, TF_XOR)
+TF_STREAM_KERNEL(threefry2x32_stream_xor_v4, 4, TF_XOR)         // requires h % 4 == 0 and a 16-byte aligned output
+TF_STREAM_KERNEL(threefry2x32_stream_pairs_v1, 1, TF_PAIRS)

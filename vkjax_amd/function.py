@@ -12,7 +12,7 @@ import numpy as np
 
 from . import minijax
 from .jaxpr_interpreter import JaxprInterpreter
-from .minijax import tree_util
+from .minijax import core, tree_util
 
 
 def _pick_frontend(frontend: tp.Optional[str]):
@@ -68,7 +68,11 @@ class Function:
     def _restore_shapes(self, x, targetshapes):
         structure = self._tree.tree_structure(targetshapes)
         x         = self._tree.tree_unflatten(structure, x)
-        return self._tree.tree_map(lambda a, shapestruct: np.asarray(a).reshape(shapestruct.shape), x, targetshapes)
+        #typed PRNG keys come back as their uint32 words, with the key's words as a trailing dimension
+        def restore(a, shapestruct):
+            a = np.asarray(a)
+            return a if core.is_key_dtype(shapestruct.dtype) else a.reshape(shapestruct.shape)
+        return self._tree.tree_map(restore, x, targetshapes)
 
 
 def wrap(function: tp.Callable, *args, **kwargs) -> Function:

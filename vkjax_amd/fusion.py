@@ -50,6 +50,8 @@ def _reads(op) -> tp.List:
             return [op.meta[2]]
         if op.meta[0] == 'threefry':
             return list(op.meta[2])
+        if op.meta[0] == 'random_stream':
+            return [b for b, _ in op.launch.buffers[1:] if b is not None]
     return [b for b, _ in op.launch.buffers if b is not None]
 
 
@@ -168,8 +170,47 @@ def fuse_ops(all_ops, bufferpool, outvars):
         if out is not None:
             producer[id(out._placeholder)] = len(result) - 1
     ops = fuse_random_streams([op for op in result if op is not None], bufferpool, outvars)
+    ops = fuse_stream_chains(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
     return remove_dead_ops(ops, bufferpool, outvars)
+
+
+def fuse_stream_chains(ops, bufferpool, outvars):
+    '''A launch that generates random words (random_bits lowered directly) followed by an
+    element-wise chain over exactly those words whose operands are single values: the chain is
+    applied by the generating kernel before its only store.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    removed, replacement = set(), {}
+    for si, S in enumerate(ops):
+        if S.meta is None or S.meta[0] != 'random_stream':
+            continue
+        _, out, layout, key0, key1, h, c0, c1, n = S.meta
+        if layout == 'pairs' or uses[pid(out)] != 1:
+            continue
+        for i in range(si + 1, len(ops)):
+            op = ops[i]
+            if not any(b._placeholder is out._placeholder for b in _reads(op)):
+                continue
+            ch = op.chain
+            size = 1
+            for d in (ch.shape if ch is not None else ()):
+                size *= d
+            if (ch is not None and ch.first.buffer._placeholder is out._placeholder and ch.first.offset == 0 and size == out.size
+                    and tuple(ch.first.strides) == K.row_major_strides(ch.shape) and len(ch.steps) <= K.TF_MAX_STEPS
+                    and all(st.op not in _SELECTS and st.op != EW['NOP'] and
+                            (st.operand is None or (st.operand.buffer.size == 1 and st.operand.offset == 0)) for st in ch.steps)):
+                fused = Op(_label(S, op), launch=K.threefry_stream(ch.out, key0, key1, h, c0, c1, list(ch.steps), layout=layout, n=n),
+                           meta=('random_stream', ch.out, layout, key0, key1, h, c0, c1, n))
+                fused.index = op.index
+                for b in [key0[0], key1[0]] + [st.operand.buffer for st in ch.steps if st.operand is not None]:
+                    b.accesses.append(fused.index)
+                out._placeholder.elided = True
+                removed.add(si)
+                replacement[i] = fused
+            break
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
 
 
 def fuse_derived_epilogue_operands(ops, bufferpool, outvars):

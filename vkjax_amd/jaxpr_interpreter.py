@@ -115,9 +115,7 @@ class JaxprInterpreter:
                 if self._resident_leaves.get(k) is x:
                     continue                                    #already in HBM
                 self._resident_leaves[k] = x
-            words = to_device_words(np.asarray(x), core.canonicalize_dtype(var.aval.dtype))
-            if words.size != int(np.prod(var.aval.shape, dtype=np.int64)):
-                raise TypeError(f'argument of shape {np.shape(x)} does not match the traced shape {var.aval.shape}')
+            words = _device_words_of_argument(x, var.aval)
             host[slot] = words
             keep.append(words)
         for slot, arr in zip(self._output_slots, self._output_arrays):
@@ -142,7 +140,7 @@ class JaxprInterpreter:
         X = self._flatten_args(X)
         for b, x, var in zip(self.input_buffers, X, self.jaxpr.jaxpr.invars):
             if b is not None and b.size:
-                b.tensor.upload(to_device_words(np.asarray(x), core.canonicalize_dtype(var.aval.dtype)))
+                b.tensor.upload(_device_words_of_argument(x, var.aval))
 
     def replay(self, iters: int = 1) -> float:
         '''Run only the kernels of the recorded sequence `iters` times on whatever the input
@@ -157,6 +155,18 @@ class JaxprInterpreter:
         deltas     = np.diff(timestamps)
         labels     = ['data2device'] + [op.equation for op in self.all_ops] + ['data2host']
         return list(zip(labels, deltas))
+
+
+def _device_words_of_argument(x, aval) -> np.ndarray:
+    shape, dtype = core.physical(aval)
+    if core.is_key_dtype(getattr(x, 'dtype', None)):
+        #a typed key array of jax: its uint32 words are what the device holds
+        import jax
+        x = jax.random.key_data(x)
+    words = to_device_words(np.asarray(x), dtype)
+    if words.size != int(np.prod(shape, dtype=np.int64)):
+        raise TypeError(f'argument of shape {np.shape(x)} does not match the traced shape {shape}')
+    return words
 
 
 def get_maximum_workgroup_size(mgr) -> int:

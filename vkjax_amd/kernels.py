@@ -221,24 +221,33 @@ TF_MAX_STEPS = 8
 
 
 def threefry_stream(out: Buffer, key0: tp.Tuple[Buffer, int], key1: tp.Tuple[Buffer, int], h: int, c0: int, c1: int,
-                    steps: tp.Sequence[EwStep]) -> Launch:
-    '''out[j], out[h + j] = steps(threefry2x32(key, c0 + j, c1 + j)) for j < h: counters generated in
-    registers, the element-wise `steps` (operands: single values) applied before the only store.
-    The key words are given as (buffer, element offset).'''
+                    steps: tp.Sequence[EwStep], layout: str = 'halves', n: tp.Optional[int] = None) -> Launch:
+    '''Random words from counters generated in registers, the element-wise `steps` (operands: single
+    values) applied before the only store. `h` blocks are run; the key words are given as
+    (buffer, element offset). Layouts:
+      halves  out[j], out[h + j] = steps(threefry2x32(key, c0 + j, c1 + j)); `n` (2h or 2h - 1) is the
+              number of elements stored, and with n == 2h - 1 the last x1 counter is 0
+      xor     out[j] = steps(y0 ^ y1) with y = threefry2x32(key, c0, c1 + j)
+      pairs   out[2j], out[2j + 1] = threefry2x32(key, c0, c1 + j)  (no steps)'''
     if len(steps) > TF_MAX_STEPS:
         raise ValueError('too many steps')
+    if layout == 'pairs' and steps:
+        raise ValueError('the pairs layout takes no steps')
+    n = 2 * h if n is None else n
+    assert layout != 'halves' or n in (2 * h, 2 * h - 1)
     flags, buffers = [], []
     for s in steps:
         if s.operand is not None:
             assert s.operand.buffer.size == 1 and s.operand.offset == 0
         flags.append((1 if s.operand is not None else 0) | (2 if s.operand_left else 0))
         buffers.append((s.operand.buffer if s.operand is not None else None, 0))
-    vec = 4 if h % 4 == 0 else 1
+    vec = 4 if h % 4 == 0 and (n == 2 * h if layout == 'halves' else layout == 'xor') else 1
     params = _u32(h, c0, c1, len(steps), *_pad([s.op for s in steps], TF_MAX_STEPS), *_pad(flags, TF_MAX_STEPS),
-                  *_pad([s.imm for s in steps], TF_MAX_STEPS))
-    return Launch(f'threefry2x32_stream_v{vec}', (_cdiv(_cdiv(h, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                  *_pad([s.imm for s in steps], TF_MAX_STEPS), n)
+    kernel = {'halves': 'threefry2x32_stream', 'xor': 'threefry2x32_stream_xor', 'pairs': 'threefry2x32_stream_pairs'}[layout]
+    return Launch(f'{kernel}_v{vec}', (_cdiv(_cdiv(h, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                   [(out, 0), (key0[0], key0[1] * 4), (key1[0], key1[1] * 4)] + _pad(buffers, TF_MAX_STEPS, (None, 0)), params,
-                  bytes_moved=8 * h)
+                  bytes_moved=4 * (h if layout == 'xor' else n))
 
 
 # --------------------------------------------------------------------------- conv / dot

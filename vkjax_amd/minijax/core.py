@@ -32,12 +32,55 @@ def canonicalize_dtype(dtype) -> np.dtype:
     return dtype
 
 
+class KeyTy:
+    '''Element type of typed PRNG key arrays (jax prints it as `key<fry>`): one element is a
+    whole threefry key, stored as `key_shape` trailing uint32 words. Newer jax versions route
+    `jax.random` through the primitives random_wrap / random_bits / random_split / ... whose
+    operands carry this type.'''
+    name      = 'key<fry>'
+    key_shape = (2,)
+    impl_name = 'threefry2x32'
+
+    def __eq__(self, other):
+        return type(other).__name__ == 'KeyTy' and key_words_shape(other) == self.key_shape
+
+    def __hash__(self):
+        return hash(self.name)
+
+    def __repr__(self):
+        return self.name
+
+
+key_fry = KeyTy()
+
+
+def is_key_dtype(dtype) -> bool:
+    '''True for KeyTy above and for jax's own key element type (matched by class name).'''
+    return type(dtype).__name__ == 'KeyTy'
+
+
+def key_words_shape(dtype) -> tp.Tuple[int, ...]:
+    '''Trailing uint32 words of one key. Only the threefry implementation is supported.'''
+    impl = getattr(dtype, '_impl', dtype)
+    name = getattr(impl, 'name', None) if impl is not dtype else dtype.impl_name
+    if name != 'threefry2x32':
+        raise NotImplementedError(f'PRNG implementation {name}: only threefry2x32 keys are supported')
+    return tuple(impl.key_shape)
+
+
+def physical(aval) -> tp.Tuple[tp.Tuple[int, ...], np.dtype]:
+    '''(shape, dtype) of the device array that holds a value of this abstract type.'''
+    if is_key_dtype(aval.dtype):
+        return tuple(aval.shape) + key_words_shape(aval.dtype), np.dtype('uint32')
+    return tuple(aval.shape), canonicalize_dtype(aval.dtype)
+
+
 class ShapedArray:
     __slots__ = ('shape', 'dtype', 'weak_type')
 
     def __init__(self, shape, dtype, weak_type=False):
         self.shape     = tuple(int(s) for s in shape)
-        self.dtype     = np.dtype(dtype)
+        self.dtype     = dtype if is_key_dtype(dtype) else np.dtype(dtype)
         self.weak_type = bool(weak_type)
 
     @property
@@ -55,7 +98,7 @@ class ShapedArray:
         return hash((self.shape, self.dtype))
 
     def __repr__(self):
-        short = {'float32': 'f32', 'int32': 'i32', 'uint32': 'u32', 'bool': 'bool'}[self.dtype.name]
+        short = {'float32': 'f32', 'int32': 'i32', 'uint32': 'u32', 'bool': 'bool'}.get(self.dtype.name, self.dtype.name)
         return f'{short}[{",".join(map(str, self.shape))}]'
 
     def str_short(self):
@@ -68,7 +111,7 @@ class ShapeDtypeStruct:
 
     def __init__(self, shape, dtype):
         self.shape = tuple(shape)
-        self.dtype = np.dtype(dtype)
+        self.dtype = dtype if is_key_dtype(dtype) else np.dtype(dtype)
 
     def __repr__(self):
         return f'ShapeDtypeStruct(shape={self.shape}, dtype={self.dtype.name})'

@@ -98,6 +98,31 @@ cos, sin, tan, cosh, sinh, tanh = map(_unary_f32, ('cos', 'sin', 'tan', 'cosh', 
 acos, asin, atan, acosh, asinh, atanh = map(_unary_f32, ('acos', 'asin', 'atan', 'acosh', 'asinh', 'atanh'))
 ceil, floor = map(_unary_f32, ('ceil', 'floor'))
 sqrt = _unary_f32('sqrt')
+logistic, log1p, expm1, exp2, cbrt = map(_unary_f32, ('logistic', 'log1p', 'expm1', 'exp2', 'cbrt'))
+def atan2(x, y): return _binary('atan2', x, y, allowed=(_f32,))
+
+
+def is_finite(x):
+    if dtype_of(x)[0] != _f32:
+        raise TypeError('is_finite needs float32')
+    return emit('is_finite', [x], [_aval(_shape(x), _bool)])
+
+
+def round(x, rounding_method: int = 0):
+    '''rounding_method 0: halves away from zero, 1: halves to even (jax.lax.RoundingMethod).'''
+    if dtype_of(x)[0] != _f32:
+        raise TypeError('round needs float32')
+    return emit('round', [x], [_aval(_shape(x), _f32)], dict(rounding_method=int(rounding_method)))
+
+
+def clamp(lo, x, hi):
+    '''min(max(x, lo), hi); the bounds are scalars or have x's shape.'''
+    dtype = dtype_of(x)[0]
+    lo, hi = _as_dtype(lo, dtype), _as_dtype(hi, dtype)
+    for b in (lo, hi):
+        if _shape(b) not in ((), _shape(x)):
+            raise TypeError('clamp bounds must be scalars or match the operand')
+    return emit('clamp', [lo, x, hi], [_aval(_shape(x), dtype)])
 
 
 def _unary_any(name):
@@ -108,6 +133,21 @@ def _unary_any(name):
 
 
 neg, abs, sign = map(_unary_any, ('neg', 'abs', 'sign'))
+square = _unary_any('square')
+
+
+def _unary_int(name, allowed):
+    def op(x):
+        if dtype_of(x)[0] not in allowed:
+            raise TypeError(f'{name} does not accept {dtype_of(x)[0]}')
+        return emit(name, [x], [_aval(_shape(x), dtype_of(x)[0])])
+    op.__name__ = name
+    return op
+
+
+bitwise_not      = _unary_int('not', (_i32, _u32, _bool))
+population_count = _unary_int('population_count', (_i32, _u32))
+clz              = _unary_int('clz', (_i32, _u32))
 
 
 def integer_pow(x, y: int):
@@ -188,6 +228,17 @@ def expand_dims(x, dimensions):
     for d in dims:
         xs.insert(d, 1)
     return reshape(x, xs)
+
+
+def split(x, sizes, axis: int = 0):
+    '''Pieces of `x` along `axis` with the given sizes (the `split` primitive of newer jax).'''
+    xs    = _shape(x)
+    axis  = axis % len(xs)
+    sizes = tuple(int(n) for n in sizes)
+    if builtins.sum(sizes) != xs[axis]:
+        raise TypeError(f'split sizes {sizes} do not add up to {xs[axis]}')
+    avals = [_aval(xs[:axis] + (n,) + xs[axis + 1:], dtype_of(x)[0]) for n in sizes]
+    return emit('split', [x], avals, dict(sizes=sizes, axis=axis), multiple_results=True)
 
 
 def iota(dtype, size: int):
@@ -421,3 +472,51 @@ def threefry2x32(key0, key1, x0, x1):
         raise TypeError('threefry2x32: key halves / data halves must have equal shapes')
     shape = _shape(x0)
     return emit('threefry2x32', [key0, key1, x0, x1], [_aval(shape, _u32), _aval(shape, _u32)], multiple_results=True)
+
+
+
+# typed keys: the primitives newer jax versions emit for jax.random (jax/_src/prng.py); a key
+# array's element is a whole threefry key, see core.KeyTy
+
+def _is_key(x) -> bool:
+    return isinstance(x, Tracer) and core.is_key_dtype(x.dtype)
+
+
+def random_seed(seeds, impl='fry'):
+    if dtype_of(seeds)[0] not in (_i32, _u32):
+        raise TypeError('random_seed takes integers')
+    return emit('random_seed', [seeds], [_aval(_shape(seeds), core.key_fry)], dict(impl=impl))
+
+
+def random_wrap(key_data, impl='fry'):
+    if dtype_of(key_data)[0] != _u32 or _shape(key_data)[-1:] != core.key_fry.key_shape:
+        raise TypeError('random_wrap takes uint32[..., 2]')
+    return emit('random_wrap', [key_data], [_aval(_shape(key_data)[:-1], core.key_fry)], dict(impl=impl))
+
+
+def random_unwrap(keys):
+    if not _is_key(keys):
+        raise TypeError('random_unwrap takes a key array')
+    return emit('random_unwrap', [keys], [_aval(_shape(keys) + core.key_fry.key_shape, _u32)])
+
+
+def random_bits(keys, bit_width: int, shape):
+    if not _is_key(keys):
+        raise TypeError('random_bits takes a key array')
+    if bit_width != 32:
+        raise NotImplementedError('random_bits: 32-bit words only (all device data is 32 bits wide)')
+    shape = tuple(int(n) for n in shape)
+    return emit('random_bits', [keys], [_aval(_shape(keys) + shape, _u32)], dict(bit_width=32, shape=shape))
+
+
+def random_split(keys, shape):
+    if not _is_key(keys):
+        raise TypeError('random_split takes a key array')
+    shape = tuple(int(n) for n in shape)
+    return emit('random_split', [keys], [_aval(_shape(keys) + shape, core.key_fry)], dict(shape=shape))
+
+
+def random_fold_in(keys, msgs):
+    if not _is_key(keys) or dtype_of(msgs)[0] != _u32 or _shape(msgs) != _shape(keys):
+        raise TypeError('random_fold_in takes a key array and uint32 data of the same shape')
+    return emit('random_fold_in', [keys, msgs], [_aval(_shape(keys), core.key_fry)])

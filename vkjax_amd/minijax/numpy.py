@@ -243,6 +243,22 @@ def getitem(x, index):
     def is_array(i):
         return isinstance(i, Tracer) or (isinstance(i, (np.ndarray, list)) and np.ndim(i) > 0)
 
+    if isinstance(x, Tracer) and core.is_key_dtype(x.dtype):
+        #key arrays: static integers and unit-stride slices, as slice + squeeze (what newer jax traces)
+        start, limit, dropped = [], [], []
+        for ax, i in enumerate(index):
+            if isinstance(i, (int, np.integer)):
+                i = int(i) + (xs[ax] if i < 0 else 0)
+                if not 0 <= i < xs[ax]:
+                    raise IndexError(f'index {i} out of bounds for axis {ax} with size {xs[ax]}')
+                start.append(i); limit.append(i + 1); dropped.append(ax)
+            elif isinstance(i, builtins.slice) and i.step in (None, 1):
+                s, l, _ = i.indices(xs[ax])
+                start.append(s); limit.append(builtins.max(l, s))
+            else:
+                raise NotImplementedError('key arrays take integers and unit-stride slices as indices')
+        return lax.squeeze(lax.slice(x, start, limit), dropped)
+
     arrays = [i for i in index if is_array(i)]
     if len(arrays) > 1 or (arrays and builtins.any(isinstance(i, (int, np.integer)) for i in index)):
         raise NotImplementedError('indexing with more than one array (or arrays mixed with ints)')

@@ -2,7 +2,12 @@
 (non-partitionable) implementation: counters are `iota(n)`, the first half feeds
 word 0 and the second half word 1 of the block function; odd sizes are padded with one
 zero counter and trimmed. `split(key, n)` is `threefry(key, iota(2n)).reshape(n, 2)`.
-(Primitive: reference vkjax/ops.py:550-560, vkjax/shaders/threefry2x32.comp.)'''
+(Primitive: reference vkjax/ops.py:550-560, vkjax/shaders/threefry2x32.comp.)
+
+Newer jax versions do not expand these functions while tracing: they emit the key primitives
+random_wrap / random_bits / random_split / random_fold_in / random_unwrap and leave the
+expansion to the backend. `key_primitives(True)` makes this module trace that way, and typed
+keys made by `key()` / `wrap_key_data()` always do.'''
 import numpy as np
 
 from . import lax, numpy as mnp
@@ -23,6 +28,42 @@ def _key_halves(key):
     return k0, k1
 
 
+_EMIT_KEY_PRIMITIVES = False
+
+
+def key_primitives(enable: bool) -> bool:
+    '''Trace split / random_bits / fold_in as key primitives instead of expanding them. Returns the previous setting.'''
+    global _EMIT_KEY_PRIMITIVES
+    previous, _EMIT_KEY_PRIMITIVES = _EMIT_KEY_PRIMITIVES, bool(enable)
+    return previous
+
+
+def _is_typed(key) -> bool:
+    return isinstance(key, Tracer) and lax.core.is_key_dtype(key.dtype)
+
+
+def key(seed):
+    '''A typed key from an integer seed (traced values only).'''
+    return lax.random_seed(seed)
+
+
+def wrap_key_data(data):
+    return lax.random_wrap(data)
+
+
+def key_data(keys):
+    return lax.random_unwrap(keys) if _is_typed(keys) else keys
+
+
+def fold_in(key, data):
+    data = lax.convert_element_type(data, np.uint32) if isinstance(data, Tracer) else np.uint32(data)
+    if _is_typed(key):
+        return lax.random_fold_in(key, data)
+    if _EMIT_KEY_PRIMITIVES:
+        return lax.random_unwrap(lax.random_fold_in(lax.random_wrap(key), data))
+    return threefry_2x32(key, mnp.concatenate([np.zeros((1,), np.uint32), mnp.reshape(data, (1,))]))
+
+
 def threefry_2x32(key, count):
     '''Apply the block function to a flat uint32 counter array of any length.'''
     k0, k1 = _key_halves(key)
@@ -40,11 +81,19 @@ def threefry_2x32(key, count):
 
 
 def split(key, num: int = 2):
+    if _is_typed(key):
+        return lax.random_split(key, (num,))
+    if _EMIT_KEY_PRIMITIVES:
+        return lax.random_unwrap(lax.random_split(lax.random_wrap(key), (num,)))
     counts = lax.iota(np.uint32, num * 2)
     return mnp.reshape(threefry_2x32(key, counts), (num, 2))
 
 
 def random_bits(key, shape):
+    if _is_typed(key):
+        return lax.random_bits(key, 32, tuple(shape))
+    if _EMIT_KEY_PRIMITIVES:
+        return lax.random_bits(lax.random_wrap(key), 32, tuple(shape))
     size = int(np.prod(shape, dtype=np.int64))
     bits = threefry_2x32(key, lax.iota(np.uint32, size))
     return mnp.reshape(bits, tuple(shape))

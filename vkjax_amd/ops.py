@@ -126,6 +126,7 @@ _BINARY = {
     'shift_right_arithmetic': {_I: 'SHR_A', _U: 'SHR_A'},
 }
 _BINARY['add_any'] = _BINARY['add']
+_BINARY['atan2']   = {_F: 'ATAN2_F'}
 
 _UNARY = {
     'exp': {_F: 'EXP_F'}, 'log': {_F: 'LOG_F'}, 'rsqrt': {_F: 'RSQRT_F'}, 'sqrt': {_F: 'SQRT_F'},
@@ -138,6 +139,10 @@ _UNARY = {
     'acos': {_F: 'ACOS_F'}, 'asin': {_F: 'ASIN_F'}, 'atan': {_F: 'ATAN_F'},
     'acosh': {_F: 'ACOSH_F'}, 'asinh': {_F: 'ASINH_F'}, 'atanh': {_F: 'ATANH_F'},
     'ceil': {_F: 'CEIL_F'}, 'floor': {_F: 'FLOOR_F'},
+    'logistic': {_F: 'LOGISTIC_F'}, 'log1p': {_F: 'LOG1P_F'}, 'expm1': {_F: 'EXPM1_F'}, 'exp2': {_F: 'EXP2_F'},
+    'cbrt': {_F: 'CBRT_F'}, 'is_finite': {_F: 'ISFINITE_F'},
+    'not': {_I: 'NOT_X', _U: 'NOT_X', _B: 'NOT_B'},
+    'population_count': {_I: 'POPCNT_X', _U: 'POPCNT_X'}, 'clz': {_I: 'CLZ_X', _U: 'CLZ_X'},
 }
 
 
@@ -175,7 +180,7 @@ add = sub = mul = div = max = min = element_wise_binary_op
 gt = ge = lt = le = eq = ne = element_wise_binary_op
 add_any = pow = rem = nextafter = element_wise_binary_op
 shift_left = shift_right_logical = shift_right_arithmetic = element_wise_binary_op
-xor = element_wise_binary_op
+xor = atan2 = element_wise_binary_op
 globals()['or']  = element_wise_binary_op
 globals()['and'] = element_wise_binary_op
 
@@ -196,6 +201,44 @@ def element_wise_unary_op(bufferpool: BufferPool, equation):
 exp = log = neg = abs = rsqrt = sqrt = erf = erf_inv = sign = element_wise_unary_op
 cos = sin = tan = cosh = sinh = tanh = element_wise_unary_op
 acos = asin = atan = acosh = asinh = atanh = ceil = floor = element_wise_unary_op
+#names newer jax versions emit (jax.nn.sigmoid -> logistic, jnp.logical_not -> not, ...)
+logistic = log1p = expm1 = exp2 = cbrt = is_finite = population_count = clz = element_wise_unary_op
+globals()['not'] = element_wise_unary_op
+
+
+def square(bufferpool, equation):
+    '''x * x in the operand's own type (newer jax traces jnp.square / x**2 as `square`).'''
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    kind   = _kind(inbuf.dtype)
+    if kind == _B:
+        return noop(bufferpool, equation)
+    outbuf  = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    operand = K.broadcast_operand(inbuf, outbuf.shape)
+    return [Op(equation, chain=EwChain(outbuf, outbuf.shape, operand, [EwStep(EW['MUL_F' if kind == _F else 'MUL_I'], operand)]))]
+
+
+def round(bufferpool, equation):
+    '''rounding_method 0 (AWAY_FROM_ZERO) or 1 (TO_NEAREST_EVEN), given as an int or as jax's enum.'''
+    method = equation.params.get('rounding_method', 0)
+    method = int(getattr(method, 'value', method))
+    if method not in (0, 1):
+        raise NotImplementedError(equation)
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    if _kind(inbuf.dtype) != _F:
+        raise NotImplementedError(equation)
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    opcode = EW['ROUND_EVEN_F' if method else 'ROUND_AWAY_F']
+    return [Op(equation, chain=EwChain(outbuf, outbuf.shape, K.broadcast_operand(inbuf, outbuf.shape), [EwStep(opcode)]))]
+
+
+def clamp(bufferpool, equation):
+    '''clamp(lo, x, hi) = min(max(x, lo), hi); scalar bounds are read in place.'''
+    lo, x, hi = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    shape  = outbuf.shape
+    steps  = [EwStep(_opcode(_BINARY, 'max', x.dtype, equation), K.broadcast_operand(lo, shape)),
+              EwStep(_opcode(_BINARY, 'min', x.dtype, equation), K.broadcast_operand(hi, shape))]
+    return [Op(equation, chain=EwChain(outbuf, shape, K.broadcast_operand(x, shape), steps))]
 
 
 def integer_pow(bufferpool, equation):
@@ -262,13 +305,16 @@ def noop(bufferpool, equation):
     assert len(equation.invars) == len(equation.outvars) == 1
     inbuf  = bufferpool.get_buffer(equation.invars[0])
     outvar = equation.outvars[0]
-    outbuf = inbuf.view(core.canonicalize_dtype(outvar.aval.dtype), outvar.aval.shape)
+    shape, dtype = core.physical(outvar.aval)
+    outbuf = inbuf.view(dtype, shape)
     bufferpool.set_buffer(outvar, outbuf)
     return []
 
 
-stop_gradient = squeeze = bitcast_convert_type = noop
+stop_gradient = squeeze = expand_dims = bitcast_convert_type = noop
 copy = copy_p = optimization_barrier = noop
+#a typed key array and its uint32 words are the same device array
+random_wrap = random_unwrap = noop
 
 
 def reshape(bufferpool, equation):
@@ -312,8 +358,10 @@ def slice(bufferpool, equation):
     inbuf  = bufferpool.get_buffer(equation.invars[0])
     outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
     n       = len(inbuf.shape)
-    start   = equation.params['start_indices']
-    strides = equation.params['strides'] or (1,) * n
+    #a key array has its words as one more (whole) trailing dimension
+    extra   = n - len(equation.params['start_indices'])
+    start   = tuple(equation.params['start_indices']) + (0,) * extra
+    strides = tuple(equation.params['strides'] or (1,) * (n - extra)) + (1,) * extra
     in_strides = K.row_major_strides(inbuf.shape)
     offset  = sum(int(s) * st for s, st in zip(start, in_strides))
     return [_copy_op(equation, outbuf, EwOperand(inbuf, offset, tuple(int(k) * st for k, st in zip(strides, in_strides))))]
@@ -362,6 +410,21 @@ def concatenate(bufferpool, equation):
     return ops
 
 
+def split(bufferpool, equation):
+    '''split[sizes, axis] of newer jax: every piece is a strided copy out of the operand.'''
+    axis   = int(equation.params['axis'])
+    inbuf  = bufferpool.get_buffer(equation.invars[0])
+    in_strides = K.row_major_strides(inbuf.shape)
+    ops, start = [], 0
+    for outvar, size in zip(equation.outvars, equation.params['sizes']):
+        if not core.is_dropped(outvar) and int(size):
+            outbuf = bufferpool.get_buffer(outvar)
+            ops.append(_copy_op(equation, outbuf, EwOperand(inbuf, start * in_strides[axis], tuple(in_strides))))
+        start += int(size)
+    bufferpool.op_counter += 1
+    return ops
+
+
 # ------------------------------------------------------------------ nested calls (inlined)
 
 def _inline_call(bufferpool, equation, jaxpr, consts=()):
@@ -400,6 +463,9 @@ core_call = closed_call = remat = xla_call
 def pjit(bufferpool, equation):
     closed = equation.params['jaxpr']
     return _inline_call(bufferpool, equation, closed, getattr(closed, 'consts', ()))
+
+
+jit = pjit      #the primitive's name in the newest jax versions
 
 
 def custom_jvp_call_jaxpr(bufferpool, equation):
@@ -638,6 +704,106 @@ def threefry2x32(bufferpool, equation):
         return []
     return [Op(equation, launch=K.threefry2x32(*outbufs, *inbufs, key_is_scalar=key_is_scalar),
                meta=('threefry', outbufs, inbufs, key_is_scalar))]
+
+
+# Key primitives of newer jax versions (jax/_src/prng.py): jax.random.* is traced as
+# random_wrap -> random_bits / random_split / random_fold_in -> random_unwrap and the backend expands
+# them. Only the threefry implementation and single (unbatched) keys are supported. The counter
+# layout follows jax's `jax_threefry_partitionable` setting:
+#   original       bits = threefry_2x32(key, iota(n)) (halves layout, odd sizes padded with a zero counter)
+#                  split = threefry_2x32(key, iota(2 num)).reshape(num, 2)
+#   partitionable  the counter of element i is its 64-bit flat index (high word, low word);
+#                  bits = y0 ^ y1, split = stack(y0, y1)
+
+#None: follow jax's configuration where jax can be imported, otherwise the original layout
+THREEFRY_PARTITIONABLE: tp.Optional[bool] = None
+
+
+def threefry_partitionable() -> bool:
+    if THREEFRY_PARTITIONABLE is not None:
+        return bool(THREEFRY_PARTITIONABLE)
+    try:
+        import jax
+        return bool(jax.config.jax_threefry_partitionable)
+    except (ImportError, AttributeError):
+        return False
+
+
+def _single_key(bufferpool, equation) -> Buffer:
+    keyvar = equation.invars[0]
+    if tuple(keyvar.aval.shape) != ():
+        raise NotImplementedError(f'batched keys are not supported: {equation}')
+    core.key_words_shape(keyvar.aval.dtype)            #raises for implementations other than threefry
+    return bufferpool.get_buffer(keyvar)
+
+
+def _stream_op(equation, outbuf, layout, key, h, c0, c1, n):
+    k0, k1 = (key, 0), (key, 1)
+    return Op(equation, launch=K.threefry_stream(outbuf, k0, k1, h, c0, c1, [], layout=layout, n=n),
+              meta=('random_stream', outbuf, layout, k0, k1, h, c0, c1, n))
+
+
+def random_bits(bufferpool, equation):
+    if int(equation.params['bit_width']) != 32:
+        raise NotImplementedError(f'only 32-bit random words exist on the device: {equation}')
+    key    = _single_key(bufferpool, equation)
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    n      = outbuf.size
+    if n == 0:
+        return []
+    if n >= 2**32:
+        raise NotImplementedError(equation)
+    if threefry_partitionable():
+        return [_stream_op(equation, outbuf, 'xor', key, n, 0, 0, n)]
+    h = (n + 1) // 2
+    return [_stream_op(equation, outbuf, 'halves', key, h, 0, h, n)]
+
+
+def random_split(bufferpool, equation):
+    key    = _single_key(bufferpool, equation)
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    num    = outbuf.size // 2
+    if num == 0:
+        return []
+    if threefry_partitionable():
+        return [_stream_op(equation, outbuf, 'pairs', key, num, 0, 0, 2 * num)]
+    return [_stream_op(equation, outbuf, 'halves', key, num, 0, num, 2 * num)]
+
+
+def _inline_traced(bufferpool, equation, function, *example_arguments):
+    '''Lowers an equation through its expansion into primitives that exist here.'''
+    from . import minijax
+    closed = minijax.make_jaxpr(function)(*example_arguments)
+    return _inline_call(bufferpool, equation, closed, closed.consts)
+
+
+def random_fold_in(bufferpool, equation):
+    '''fold_in(key, data) = threefry_2x32(key, [0, data]) in both counter layouts.'''
+    from .minijax import lax, numpy as mnp
+    _single_key(bufferpool, equation)
+
+    def expansion(key, data):
+        k0 = lax.reshape(lax.slice(key, (0,), (1,)), ())
+        k1 = lax.reshape(lax.slice(key, (1,), (2,)), ())
+        y0, y1 = lax.threefry2x32(k0, k1, np.zeros((1,), np.uint32), mnp.reshape(data, (1,)))
+        return mnp.concatenate([y0, y1])
+    return _inline_traced(bufferpool, equation, expansion, np.zeros(2, np.uint32), np.uint32(0))
+
+
+def random_seed(bufferpool, equation):
+    '''Key words (seed >> 32, seed & 0xFFFFFFFF) of a 32-bit seed: (0, seed).'''
+    from .minijax import lax, numpy as mnp
+    core.key_words_shape(equation.outvars[0].aval.dtype)
+    seedvar = equation.invars[0]
+    shape   = tuple(seedvar.aval.shape)
+    dtype   = core.canonicalize_dtype(seedvar.aval.dtype)
+    if _kind(dtype) not in (_I, _U):
+        raise NotImplementedError(equation)
+
+    def expansion(seed):
+        low = mnp.reshape(lax.convert_element_type(seed, np.uint32), shape + (1,))
+        return mnp.concatenate([np.zeros(shape + (1,), np.uint32), low], axis=-1)
+    return _inline_traced(bufferpool, equation, expansion, np.zeros(shape, dtype))
 
 
 import builtins as _builtins
