@@ -16,8 +16,9 @@ INCLUDE = os.path.join(ROOT, 'include')
 HIPCC   = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
 ARCH    = 'gfx950'
 
-#packed fp32 instructions are switched off for all device code
-DEVICE_FLAGS = ['-O3', f'--offload-arch={ARCH}', '--genco', '-munsafe-fp-atomics',
+#packed fp32 instructions are switched off for all device code; no contraction of a multiply and an
+#add into a fused multiply-add: every element-wise step rounds on its own, fused into another kernel or not
+DEVICE_FLAGS = ['-O3', f'--offload-arch={ARCH}', '--genco', '-munsafe-fp-atomics', '-ffp-contract=off',
                 '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops', '-Wno-pass-failed']
 
 KERNEL_SOURCES = ['elementwise', 'conv_gemm', 'reduce', 'index', 'threefry']

@@ -125,12 +125,34 @@ __device__ __forceinline__ void threefry_stream_steps(uint32_t (&y)[NV], uint32_
     }
 }
 
-template <int VEC, int MODE>
+// The chain of jax.random.uniform, known at compile time: the opcode switch folds away and the six
+// single-value operands are fetched before the block function runs instead of one dependent pair
+// of scalar loads per step. (bits >> 9 | 0x3F800000, as float - 1, * (max - min), + min, max(min, .))
+template <int NV>
+__device__ __forceinline__ void threefry_uniform_steps(uint32_t (&y)[NV], const uint32_t (&o)[6]) {
+    constexpr uint32_t ops[6] = {EW_SHR_L, EW_OR_X, EW_SUB_F, EW_MUL_F, EW_ADD_F, EW_MAX_F};
+#pragma unroll
+    for (int k = 0; k < 6; ++k) {
+        uint32_t v[NV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j) v[j] = o[k];
+        ew_apply_vec<NV>(ops[k], y, v, k == 5, 0u);
+    }
+}
+
+template <int VEC, int MODE, bool UNIFORM = false>
 __device__ __forceinline__ void threefry_stream_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ key0,
                                                      const uint32_t* __restrict__ key1, const ThreefryStreamParams& P) {
     const uint32_t j0 = (blockIdx.x * 256u + threadIdx.x) * VEC;
     if (j0 >= P.h) return;
     const uint32_t k0 = key0[0], k1 = key1[0];
+    uint32_t o[6] = {};
+    if constexpr (UNIFORM) {
+        const char* const args = reinterpret_cast<const char*>(__builtin_amdgcn_kernarg_segment_ptr());
+        const uint32_t* const* const op_ptr = reinterpret_cast<const uint32_t* const*>(args + 24);
+#pragma unroll
+        for (int k = 0; k < 6; ++k) o[k] = op_ptr[k][0];
+    }
     if constexpr (MODE == TF_HALVES) {
         uint32_t y[2 * VEC];                         // [0, VEC): first results, [VEC, 2 VEC): second results
 #pragma unroll
@@ -140,7 +162,8 @@ __device__ __forceinline__ void threefry_stream_body(uint32_t* __restrict__ out,
             if (VEC == 1 && P.h + j0 >= P.n) y[VEC] = 0u;           // the padding counter of an odd-sized draw
             threefry_block(k0, k1, y[j], y[VEC + j]);
         }
-        threefry_stream_steps<2 * VEC>(y, P.nsteps);
+        if constexpr (UNIFORM) threefry_uniform_steps<2 * VEC>(y, o);
+        else threefry_stream_steps<2 * VEC>(y, P.nsteps);
         if constexpr (VEC == 4) {
             u32x4 va, vb;
             va.x = y[0]; va.y = y[1]; va.z = y[2]; va.w = y[3];
@@ -165,7 +188,8 @@ __device__ __forceinline__ void threefry_stream_body(uint32_t* __restrict__ out,
         } else {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) y[j] ^= z[j];
-            threefry_stream_steps<VEC>(y, P.nsteps);
+            if constexpr (UNIFORM) threefry_uniform_steps<VEC>(y, o);
+            else threefry_stream_steps<VEC>(y, P.nsteps);
             if constexpr (VEC == 4) {
                 u32x4 va;
                 va.x = y[0]; va.y = y[1]; va.z = y[2]; va.w = y[3];
@@ -177,13 +201,16 @@ __device__ __forceinline__ void threefry_stream_body(uint32_t* __restrict__ out,
     }
 }
 
-#define TF_STREAM_KERNEL(name, VEC, MODE)                                                                              \
+#define TF_STREAM_KERNEL(name, VEC, MODE, ...)                                                                         \
     extern "C" __global__ __launch_bounds__(256) void name(uint32_t* out, const uint32_t* key0, const uint32_t* key1,  \
                                                            ThreefryStreamPtrs operands, ThreefryStreamParams P) {      \
-        threefry_stream_body<VEC, MODE>(out, key0, key1, P);                                                           \
+        threefry_stream_body<VEC, MODE, ##__VA_ARGS__>(out, key0, key1, P);                                            \
     }
 TF_STREAM_KERNEL(threefry2x32_stream_v1, 1, TF_HALVES)
 TF_STREAM_KERNEL(threefry2x32_stream_v4, 4, TF_HALVES)          // requires h % 4 == 0, n == 2h and a 16-byte aligned output
 TF_STREAM_KERNEL(threefry2x32_stream_xor_v1, 1, TF_XOR)
 TF_STREAM_KERNEL(threefry2x32_stream_xor_v4, 4, TF_XOR)         // requires h % 4 == 0 and a 16-byte aligned output
 TF_STREAM_KERNEL(threefry2x32_stream_pairs_v1, 1, TF_PAIRS)
+// the steps are exactly jax.random.uniform's chain, every step with an operand (see threefry_uniform_steps)
+TF_STREAM_KERNEL(threefry2x32_stream_uniform_v4, 4, TF_HALVES, true)
+TF_STREAM_KERNEL(threefry2x32_stream_xor_uniform_v4, 4, TF_XOR, true)

@@ -220,6 +220,9 @@ def concat_part(out: Buffer, part: Buffer, dimension: int, offset_along_dim: int
 TF_MAX_STEPS = 8
 
 
+_UNIFORM_CHAIN_OPS = [EW[name] for name in ('SHR_L', 'OR_X', 'SUB_F', 'MUL_F', 'ADD_F', 'MAX_F')]
+
+
 def threefry_stream(out: Buffer, key0: tp.Tuple[Buffer, int], key1: tp.Tuple[Buffer, int], h: int, c0: int, c1: int,
                     steps: tp.Sequence[EwStep], layout: str = 'halves', n: tp.Optional[int] = None) -> Launch:
     '''Random words from counters generated in registers, the element-wise `steps` (operands: single
@@ -245,6 +248,9 @@ def threefry_stream(out: Buffer, key0: tp.Tuple[Buffer, int], key1: tp.Tuple[Buf
     params = _u32(h, c0, c1, len(steps), *_pad([s.op for s in steps], TF_MAX_STEPS), *_pad(flags, TF_MAX_STEPS),
                   *_pad([s.imm for s in steps], TF_MAX_STEPS), n)
     kernel = {'halves': 'threefry2x32_stream', 'xor': 'threefry2x32_stream_xor', 'pairs': 'threefry2x32_stream_pairs'}[layout]
+    #jax.random.uniform's chain has a kernel of its own with the steps compiled in
+    if vec == 4 and [s.op for s in steps] == _UNIFORM_CHAIN_OPS and flags == [1, 1, 1, 1, 1, 3] and all(s.imm == 0 for s in steps):
+        kernel += '_uniform'
     return Launch(f'{kernel}_v{vec}', (_cdiv(_cdiv(h, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                   [(out, 0), (key0[0], key0[1] * 4), (key1[0], key1[1] * 4)] + _pad(buffers, TF_MAX_STEPS, (None, 0)), params,
                   bytes_moved=4 * (h if layout == 'xor' else n))
