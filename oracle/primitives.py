@@ -36,7 +36,10 @@ import math
 
 import numpy as np
 
+import builtins
+
 f32, i32, u32 = np.float32, np.int32, np.uint32
+builtins_max, builtins_min = builtins.max, builtins.min
 _EW_ERR = dict(over='ignore', invalid='ignore', divide='ignore')
 
 
@@ -484,6 +487,53 @@ def reduce_window_sum(x, window_dimensions, window_strides, padding, **kw):
     '''Window sum with 0 outside the array (average pooling divides it by the window size
     afterwards). No counterpart in the reference's primitive set.'''
     return _reduce_window(x, 0, np.add, window_dimensions, window_strides, padding, **kw)
+
+
+def select_and_scatter_add(source, operand, select_prim, window_dimensions, window_strides, padding, **_):
+    '''XLA select-and-scatter with addition (the gradient of a max/min pooling): every window of
+    `operand` selects one of its elements, and the window's `source` value is added to the result
+    at that position; the result has operand's shape and starts at 0. Selection follows XLA's
+    evaluator: the window is scanned in row-major order over the positions inside the array
+    (padding is never selected), the first one is taken, and a later one replaces it whenever
+    select(selected, candidate) is false, with select = `ge` (max pooling) or `le` (min pooling);
+    ties keep the earlier position. Windows are visited in row-major order, and sums follow it.'''
+    name = getattr(select_prim, 'name', str(select_prim))
+    keep = {'ge': lambda a, b: a >= b, 'le': lambda a, b: a <= b}[name]
+    source, operand = _canon(source), _canon(operand)
+    out = np.zeros(operand.shape, np.float64)
+    for o in np.ndindex(*source.shape):
+        selected = None
+        for t in np.ndindex(*window_dimensions):
+            pos = tuple(o[d] * window_strides[d] - padding[d][0] + t[d] for d in range(operand.ndim))
+            if any(p < 0 or p >= operand.shape[d] for d, p in enumerate(pos)):
+                continue
+            if selected is None or not keep(operand[selected], operand[pos]):
+                selected = pos
+        if selected is not None:
+            #float32 accumulation in visiting order, as a sequential scatter would do
+            out[selected] = np.float32(np.float32(out[selected]) + source[o])
+    return out.astype(f32)
+
+
+def pad(x, padding_value, padding_config, **_):
+    '''XLA pad: (low, high, interior) per dimension; negative low/high crop.'''
+    x = _canon(x)
+    value = np.asarray(padding_value, dtype=x.dtype).reshape(())
+    for d, (lo, hi, interior) in enumerate(padding_config):
+        n = x.shape[d]
+        dilated = np.full(x.shape[:d] + (builtins_max(n + (n - 1) * interior, 0),) + x.shape[d + 1:], value, x.dtype)
+        idx = [np.s_[:]] * x.ndim
+        idx[d] = np.s_[::interior + 1]
+        dilated[tuple(idx)] = x
+        m = dilated.shape[d]
+        grown = np.full(x.shape[:d] + (builtins_max(m + lo + hi, 0),) + x.shape[d + 1:], value, x.dtype)
+        src_lo, dst_lo = builtins_max(-lo, 0), builtins_max(lo, 0)
+        length = builtins_max(builtins_min(m - src_lo - builtins_max(-hi, 0), grown.shape[d] - dst_lo), 0)
+        src, dst = [np.s_[:]] * x.ndim, [np.s_[:]] * x.ndim
+        src[d], dst[d] = np.s_[src_lo:src_lo + length], np.s_[dst_lo:dst_lo + length]
+        grown[tuple(dst)] = dilated[tuple(src)]
+        x = grown
+    return x
 
 
 # ------------------------------------------------------------------ indexing

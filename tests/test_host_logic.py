@@ -64,7 +64,7 @@ def test_kernel_argument_layouts_match_the_structs():
     #compiled on their own with the host compiler
     kdir  = os.path.join(ROOT, 'vkjax_amd', 'csrc', 'kernels')
     text  = ''.join(open(os.path.join(kdir, f)).read() for f in sorted(os.listdir(kdir)) if f.endswith('.hip'))
-    defs  = re.findall(r'^#define\s+(?:EW_MAX_STEPS|CONV_MAX_EPI|CONV_MAX_DERIVED|IDX_MAX_RANK|TF_MAX_STEPS)\s+\d+\s*$', text, re.M)
+    defs  = re.findall(r'^#define\s+(?:EW_MAX_STEPS|CONV_MAX_EPI|CONV_MAX_DERIVED|IDX_MAX_RANK|TF_MAX_STEPS|PAD_MAX_RANK)\s+\d+\s*$', text, re.M)
     decls = re.findall(r'^struct\s+\w+\s*\{[^}]*\};', text, re.M)
     names = [re.match(r'struct\s+(\w+)', d).group(1) for d in decls]
     src   = '#include <cstdio>\n#include <cstdint>\n' + '\n'.join(defs) + '\n' + '\n'.join(decls) + '\nint main(){\n' \
@@ -88,6 +88,7 @@ def test_kernel_argument_layouts_match_the_structs():
         'ReduceParams': K.reduce(b(4), b(4, 8), 4, 8, 1, 'reduce_sum')[0],
         'ReduceGeneralParams': K.reduce_general(b(4), b(4, 8), [(4, 8)], [(8, 1)], 'reduce_sum'),
         'PoolParams': K.pool(b(1, 2, 2, 4), b(1, 4, 4, 4), 'reduce_max', (1, 2, 2, 1), (1, 2, 2, 1), (0, 0, 0, 0), (1, 1, 1, 1)),
+        'PadParams': K.pad(b(6, 8), b(4, 8), b(), ((1, 1, 0), (0, 0, 0))),
         'GatherRowsParams': K.gather_rows(b(3, 8), b(4, 8), i(3, 1), 3, 8, 4),
         'GatherGeneralParams': K.gather_general(b(3, 8), b(4, 8), i(3, 1), (1,), (0,), (0,), (1, 8)),
         'ScatterRowsParams': K.scatter_add_rows(b(4, 8), i(3, 1), b(3, 8), 3, 8, 4),

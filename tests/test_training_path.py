@@ -1,0 +1,250 @@
+'''Training-path programs: the primitives autodiff adds to a jaxpr (pad, select_and_scatter_add, convolutions
+with lhs / rhs dilation, reversed kernels and permuted dimension numbers, transposed dot_generals, add_any) and
+whole SGD steps, the way the reference runs them in tests/test_elegy_mlp.py:87-129 and
+tests/test_elegy_conv.py:51-94. CPU part: the differentiation rules and the oracle against torch autograd
+(an independent implementation); GPU part: the HIP path against the oracle on the same programs.'''
+import numpy as np
+import pytest
+
+from oracle import primitives as P
+from oracle.eval_jaxpr import eval_closed_jaxpr
+from tests.common import check_against_oracle
+from vkjax_amd import minijax as mj, workloads as W
+from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
+
+lax, jnp, nn = mj.lax, mj.numpy, mj.nn
+rng = np.random.RandomState(99)
+random = lambda shape: rng.random_sample(shape).astype(np.float32)
+
+
+def pad0(x): return lax.pad(x, 0.0, ((1, 2, 0), (0, 0, 0)))
+def pad1(x): return lax.pad(x, -1.5, ((0, 0, 0), (2, 1, 1), (1, 0, 2), (0, 0, 0)))
+def pad2(x): return lax.pad(x, 7.0, ((-1, 2, 0), (1, -2, 1), (0, 3, 0)))
+def pad3(x, v): return lax.pad(x, v, ((0, 0, 3),))
+def pad4(x): return lax.pad(x + 1, 0, ((2, 2, 1), (0, 1, 0)))
+def pool_grad(window, strides, padding, select=None):
+    def f(g, x): return lax.select_and_scatter_add(g, x, select or lax.ge_p, window, strides, padding)
+    return f
+
+def _pooled(shape, window, strides, padding):
+    return [(n + lo + hi - w) // s + 1 for n, w, s, (lo, hi) in zip(shape, window, strides, padding)]
+
+_P = ((0, 0), (0, 1), (0, 1), (0, 0))
+_SAME = ((0, 0), (1, 1), (1, 1), (0, 0))
+_ties = np.round(random([2, 9, 9, 8]) * 3)          #many equal values: the first position of a window must win
+pool_cases = [
+    ('3x3 s2 pad hi C8',   (1, 3, 3, 1), (1, 2, 2, 1), _P,    random([2, 11, 12, 8]) - 0.5, None),
+    ('3x3 s2 SAME C5',     (1, 3, 3, 1), (1, 2, 2, 1), _SAME, random([2, 9, 10, 5]) - 0.5, None),
+    ('2x2 s2 C4',          (1, 2, 2, 1), (1, 2, 2, 1), ((0, 0),) * 4, random([3, 8, 6, 4]), None),
+    ('3x3 s1 ties',        (1, 3, 3, 1), (1, 1, 1, 1), _SAME, _ties, None),
+    ('min pooling',        (1, 2, 2, 1), (1, 1, 1, 1), ((0, 0),) * 4, random([2, 6, 7, 4]), lax.le_p),
+    ('window over all dims', (2, 2, 1, 3), (1, 2, 1, 2), ((1, 0), (0, 0), (0, 0), (1, 1)), random([3, 6, 4, 7]), None),
+    ('2-D array',          (3, 2), (2, 1), ((1, 1), (0, 1)), random([13, 9]), None),
+]
+pad_cases = [(pad0, [random([5, 8])]), (pad1, [random([2, 5, 6, 8])]), (pad2, [random([4, 7, 5])]),
+             (pad3, [np.arange(9, dtype=np.int32), np.int32(-7)]), (pad4, [random([6, 12])])]
+
+
+def small_convnet_inputs():
+    return W.convnet_train_inputs(batch=3, size=16, channels=(3, 8, 12), classes=5)
+
+
+def small_mlp_inputs():
+    return W.mlp_train_inputs(batch=16, sizes=(40, 32, 24, 5))
+
+
+# ------------------------------------------------------------------ CPU: pins of the oracle and of the differentiation rules
+
+def test_select_and_scatter_add_oracle_equals_torch_max_pool_backward():
+    torch = pytest.importorskip('torch')
+    x = random([2, 9, 11, 3])
+    xt = torch.tensor(x.transpose(0, 3, 1, 2), requires_grad=True)
+    y = torch.nn.functional.max_pool2d(xt, 3, 2, padding=1)
+    g = random(tuple(y.shape))
+    y.backward(torch.tensor(g))
+    mine = P.select_and_scatter_add(g.transpose(0, 2, 3, 1), x, lax.ge_p, (1, 3, 3, 1), (1, 2, 2, 1), _SAME)
+    assert np.array_equal(mine, xt.grad.numpy().transpose(0, 2, 3, 1))
+    #ties: the whole cotangent of a window goes to its first maximum
+    flat = P.select_and_scatter_add(np.ones((1, 1), np.float32), np.zeros((2, 2), np.float32), lax.ge_p, (2, 2), (1, 1), ((0, 0), (0, 0)))
+    assert flat.tolist() == [[1, 0], [0, 0]]
+
+
+def test_pad_oracle_against_numpy_and_brute_force():
+    x = random([3, 5, 4])
+    assert np.array_equal(P.pad(x, 0.0, ((1, 2, 0), (3, 0, 0), (0, 1, 0))), np.pad(x, ((1, 2), (3, 0), (0, 1))))
+    config = ((1, 2, 0), (0, 0, 1), (-1, 1, 2))
+    shape = [n + (n - 1) * it + lo + hi for n, (lo, hi, it) in zip(x.shape, config)]
+    brute = np.full(shape, 7.0, np.float32)
+    for idx in np.ndindex(*x.shape):
+        o = tuple(lo + i * (it + 1) for i, (lo, hi, it) in zip(idx, config))
+        if all(0 <= p < s for p, s in zip(o, shape)):
+            brute[o] = x[idx]
+    assert np.array_equal(P.pad(x, 7.0, config), brute)
+
+
+def _torch_convnet_grads(params, x, onehot):
+    import torch
+    F = torch.nn.functional
+    T = lambda a: torch.tensor(a, dtype=torch.float64, requires_grad=True)
+    tp, xt = {k: T(v) for k, v in params.items()}, T(x)
+    y = F.conv2d(xt.permute(0, 3, 1, 2), tp['w1'].permute(3, 2, 0, 1), stride=2, padding=1)
+    y = torch.relu(y * tp['scale'][None, :, None, None] + tp['shift'][None, :, None, None])
+    y = F.max_pool2d(F.pad(y, (0, 1, 0, 1), value=-np.inf), 3, 2)
+    y = torch.relu(F.conv2d(y, tp['w2'].permute(3, 2, 0, 1), padding=1))
+    y = F.avg_pool2d(y, 2, 2).mean(dim=(2, 3))
+    loss = F.cross_entropy(y @ tp['w3'] + tp['b3'], torch.tensor(onehot.argmax(1)))
+    loss.backward()
+    return float(loss), {k: v.grad.numpy() for k, v in tp.items()}, xt.grad.numpy()
+
+
+def test_convnet_gradients_equal_torch_autograd():
+    pytest.importorskip('torch')
+    params, x, onehot = small_convnet_inputs()
+    f = lambda p, x, o: mj.value_and_grad(W.convnet_loss, argnums=(0, 1))(p, x, o)
+    closed = mj.make_jaxpr(f)(params, x, onehot)
+    names = set(e.primitive.name for e in closed.jaxpr.eqns)
+    assert {'select_and_scatter_add', 'pad', 'rev', 'add_any', 'conv_general_dilated'} <= names
+    outs = eval_closed_jaxpr(closed, *mj.tree_leaves([params, x, onehot]))
+    loss, grads, gx = _torch_convnet_grads(params, x, onehot)
+    assert abs(float(outs[0]) - loss) < 1e-6
+    for name, g in zip(sorted(params), outs[1:]):
+        assert np.allclose(g, grads[name], rtol=1e-4, atol=1e-7), name
+    assert np.allclose(outs[-1], gx, rtol=1e-4, atol=1e-7)
+
+
+def test_conv_gradient_with_padding_beyond_kernel_equals_torch():
+    '''Padding >= kernel size makes the input gradient a convolution with negative (cropping) padding.'''
+    torch = pytest.importorskip('torch')
+    F = torch.nn.functional
+    x, w = random([2, 9, 8, 4]) - 0.5, random([3, 2, 4, 8]) - 0.5
+    padding = ((3, 1), (2, 0))
+    def loss(x, w):
+        y = lax.conv_general_dilated(x, w, window_strides=(1, 1), padding=padding, dimension_numbers=W.NHWC)
+        return jnp.sum(y * y) * 0.5
+    closed = mj.make_jaxpr(lambda x, w: mj.grad(loss, argnums=(0, 1))(x, w))(x, w)
+    assert any(e.primitive.name == 'conv_general_dilated' and min(min(p) for p in e.params['padding']) < 0 for e in closed.jaxpr.eqns)
+    gx, gw = eval_closed_jaxpr(closed, x, w)
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    y = F.conv2d(F.pad(xt.permute(0, 3, 1, 2), (2, 0, 3, 1)), wt.permute(3, 2, 0, 1))
+    (y * y).sum().mul(0.5).backward()
+    assert np.allclose(gx, xt.grad.numpy(), rtol=1e-4, atol=1e-6) and np.allclose(gw, wt.grad.numpy(), rtol=1e-4, atol=1e-6)
+
+
+def test_mlp_gradients_equal_torch_autograd():
+    torch = pytest.importorskip('torch')
+    params, x, onehot = small_mlp_inputs()
+    closed = mj.make_jaxpr(lambda p, x, o: mj.value_and_grad(W.mlp_loss)(p, x, o))(params, x, onehot)
+    outs = eval_closed_jaxpr(closed, *mj.tree_leaves([params, x, onehot]))
+    T = lambda a: torch.tensor(a, dtype=torch.float64, requires_grad=True)
+    tp = {k: T(v) for k, v in params.items()}
+    h = torch.relu(torch.tensor(x, dtype=torch.float64) @ tp['w1'] + tp['b1'])
+    h = torch.relu(h @ tp['w2'] + tp['b2'])
+    loss = torch.nn.functional.cross_entropy(h @ tp['w3'] + tp['b3'], torch.tensor(onehot.argmax(1)))
+    loss.backward()
+    assert abs(float(outs[0]) - float(loss)) < 1e-6
+    for name, g in zip(sorted(params), outs[1:]):
+        assert np.allclose(g, tp[name].grad.numpy(), rtol=1e-4, atol=1e-7), name
+
+
+def test_gradient_rules_of_other_primitives_equal_torch_autograd():
+    '''Rules not reached by the two networks: div, sqrt, rsqrt, logistic, integer_pow, reduce_max, transpose,
+    slice, concatenate, gather, min, select.'''
+    torch = pytest.importorskip('torch')
+    def f(a, b, idx):
+        t = lax.transpose(a, (1, 0))[1:4:2, :]                               #[2, 5]
+        u = jnp.concatenate([t, lax.sqrt(b[:2] + 2.0)], axis=0)              #[4, 5]
+        v = lax.logistic(u) / (1.5 + lax.integer_pow(u, 2)) + lax.rsqrt(u * u + 1.0)
+        w = jnp.minimum(v, 0.9 * jnp.max(v, axis=1, keepdims=True))
+        rows = b[idx]                                                        #gather [3, 5]
+        s = lax.select(lax.gt(rows, 0.5), rows * rows, -rows)
+        return jnp.sum(w * w) + jnp.sum(s) * 0.25
+    a, b = random([5, 6]) + 0.1, random([4, 5])
+    idx = np.array([3, 0, 3], np.int32)
+    closed = mj.make_jaxpr(lambda a, b, i: mj.value_and_grad(f, argnums=(0, 1))(a, b, i))(a, b, idx)
+    value, ga, gb = eval_closed_jaxpr(closed, a, b, idx)
+    at, bt = (torch.tensor(v, dtype=torch.float64, requires_grad=True) for v in (a, b))
+    t = at.T[1:4:2, :]
+    u = torch.cat([t, torch.sqrt(bt[:2] + 2.0)], dim=0)
+    v = torch.sigmoid(u) / (1.5 + u ** 2) + torch.rsqrt(u * u + 1.0)
+    w = torch.minimum(v, 0.9 * v.amax(dim=1, keepdim=True))
+    rows = bt[torch.tensor(idx, dtype=torch.long)]
+    s = torch.where(rows > 0.5, rows * rows, -rows)
+    total = (w * w).sum() + s.sum() * 0.25
+    total.backward()
+    assert abs(float(value) - float(total)) < 1e-5
+    assert np.allclose(ga, at.grad.numpy(), rtol=1e-4, atol=1e-6) and np.allclose(gb, bt.grad.numpy(), rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize('name', ['mlp_train', 'convnet_train'])
+def test_training_steps_plan_at_full_size(name):
+    fn, make_inputs = W.WORKLOADS[name]
+    interp = JaxprInterpreter(mj.make_jaxpr(fn)(*make_inputs()), plan_only=True)
+    kernels = [l.kernel for l in interp.launches]
+    assert any(k.startswith('conv_gemm') for k in kernels)
+    if name == 'convnet_train':
+        assert 'select_scatter_add_v4' in kernels and any(k.startswith('pad_nd') for k in kernels)
+
+
+@pytest.mark.parametrize('f,args', pad_cases, ids=[c[0].__name__ for c in pad_cases])
+def test_pad_plans(f, args):
+    JaxprInterpreter(mj.make_jaxpr(f)(*args), plan_only=True)
+
+
+# ------------------------------------------------------------------ GPU parity
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('f,args', pad_cases, ids=[c[0].__name__ for c in pad_cases])
+def test_pad_hip(f, args):
+    print(f'case: {f.__name__}', flush=True)
+    check_against_oracle(f, args, exact=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('desc,window,strides,padding,x,select', pool_cases, ids=[c[0] for c in pool_cases])
+def test_select_and_scatter_add_hip(desc, window, strides, padding, x, select):
+    print(f'case: {desc}', flush=True)
+    g = random(_pooled(x.shape, window, strides, padding)) + 0.25
+    check_against_oracle(pool_grad(window, strides, padding, select), [g, x], exact=True)
+
+
+@pytest.mark.gpu
+def test_conv_gradient_forms_hip():
+    '''Input and kernel gradients of strided, padded and dilated convolutions (the convolutions autodiff emits:
+    lhs dilation, rhs dilation, reversed kernels, permuted dimension numbers, padding that can be negative).'''
+    cases = [((2, 9, 10, 4), (3, 3, 4, 6), (2, 2), ((1, 1), (1, 1)), (1, 1)),
+             ((2, 12, 11, 8), (3, 2, 8, 16), (1, 2), ((0, 2), (1, 0)), (2, 1)),
+             ((1, 8, 8, 3), (1, 1, 3, 5), (2, 2), ((0, 0), (0, 0)), (1, 1)),
+             ((2, 10, 9, 16), (3, 3, 16, 8), (3, 2), ((2, 1), (0, 1)), (1, 1)),
+             ((2, 9, 8, 4), (3, 2, 4, 8), (1, 1), ((3, 1), (2, 0)), (1, 1))]        #padding >= kernel size: the input gradient crops
+    for xs, ws, strides, padding, rhs_dilation in cases:
+        print(f'case: conv gradients x{xs} w{ws} strides{strides} padding{padding} rhs_dilation{rhs_dilation}', flush=True)
+        def loss(x, w):
+            y = lax.conv_general_dilated(x, w, window_strides=strides, padding=padding, rhs_dilation=rhs_dilation, dimension_numbers=W.NHWC)
+            return jnp.sum(y * y) * 0.5
+        f = lambda x, w: mj.grad(loss, argnums=(0, 1))(x, w)
+        check_against_oracle(f, [random(xs) - 0.5, random(ws) - 0.5], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('name,make_inputs', [('mlp_train', small_mlp_inputs), ('convnet_train', small_convnet_inputs)])
+def test_training_step_hip_matches_oracle(name, make_inputs):
+    '''One SGD step: loss and every updated parameter against the oracle (reference tests/test_elegy_mlp.py:87-129
+    compares exactly these after train_on_batch, rtol 1e-5 / atol 1e-6 there; contractions here use the tolerance
+    of dot / conv).'''
+    print(f'case: {name}', flush=True)
+    fn, _ = W.WORKLOADS[name]
+    for fuse in (True, False):
+        check_against_oracle(fn, make_inputs(), rtol=1e-4, atol=1e-6, fuse=fuse)
+
+
+@pytest.mark.gpu
+def test_repeated_training_steps_reduce_the_loss():
+    import vkjax_amd
+    params, x, onehot = small_mlp_inputs()
+    step = vkjax_amd.wrap(lambda p, x, o: W.mlp_train_step(p, x, o, lr=0.2), frontend='minijax')
+    losses = []
+    for _ in range(10):
+        loss, params = step(params, x, onehot)
+        losses.append(float(loss))
+    assert losses[-1] < 0.7 * losses[0], losses

@@ -242,3 +242,49 @@ extern "C" __global__ __launch_bounds__(256) void concat_part_v1(uint32_t* __res
 extern "C" __global__ __launch_bounds__(256) void concat_part_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, ConcatParams P) {
     concat_body<4>(out, in, P);
 }
+
+// XLA pad: out = value everywhere except at low + i * (interior + 1) along every dimension, where it
+// is in[i]; negative low / high crop. One output element per thread (four with VEC = 4, which needs
+// the last dimension untouched by the padding and divisible by 4). Up to 6 dimensions (unused = 1).
+#define PAD_MAX_RANK 6
+struct PadParams {
+    uint32_t n;                           // output elements
+    uint32_t out_dims[PAD_MAX_RANK], in_dims[PAD_MAX_RANK];
+    int32_t  low[PAD_MAX_RANK];
+    uint32_t step[PAD_MAX_RANK];          // interior + 1
+};
+
+template <int VEC>
+__device__ __forceinline__ void pad_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                         const uint32_t* __restrict__ value, const PadParams& P) {
+    const uint64_t e0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * VEC;
+    if (e0 >= P.n) return;
+    uint64_t r = e0, off = 0, mul = 1;
+    bool inside = true;
+#pragma unroll
+    for (int d = PAD_MAX_RANK - 1; d >= 0; --d) {
+        const uint64_t q = r / P.out_dims[d];
+        const int64_t  p = (int64_t)(r - q * P.out_dims[d]) - P.low[d];
+        r = q;
+        const int64_t i = p / (int64_t)P.step[d];
+        inside = inside && p >= 0 && i * (int64_t)P.step[d] == p && i < (int64_t)P.in_dims[d];
+        off += (uint64_t)i * mul;
+        mul *= P.in_dims[d];
+    }
+    const uint32_t v = value[0];
+    if constexpr (VEC == 4) {
+        u32x4 q = u32x4{v, v, v, v};
+        if (inside) q = *reinterpret_cast<const u32x4*>(in + off);
+        *reinterpret_cast<u32x4*>(out + e0) = q;
+    } else {
+        out[e0] = inside ? in[off] : v;
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void pad_nd_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                            const uint32_t* __restrict__ value, PadParams P) {
+    pad_body<1>(out, in, value, P);
+}
+extern "C" __global__ __launch_bounds__(256) void pad_nd_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                            const uint32_t* __restrict__ value, PadParams P) {
+    pad_body<4>(out, in, value, P);
+}

@@ -398,3 +398,109 @@ extern "C" __global__ __launch_bounds__(256) void pool_v1(uint32_t* __restrict__
 extern "C" __global__ __launch_bounds__(256) void pool_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, PoolParams P) {
     pool_body<4>(out, in, P);
 }
+
+// ---------------------------------------------------------------------------------------------
+// select_and_scatter_add: the gradient of a max (or min) pooling. Every window of `operand` selects
+// one of its elements (scan in row-major order over the positions inside the array, the first is
+// taken, a later one replaces it when !(selected >= candidate), resp. <=); the window's `source`
+// value is added at that position. Written as a gather so that no atomics are needed and the sums
+// have a fixed order: one thread per operand element (four with VEC = 4) walks the windows that
+// contain it in row-major order, repeats each window's selection and adds the source value when the
+// selection is its own element. Re-reads of the operand (window size x windows per element) hit
+// the caches; HBM sees operand + source once and the result once.
+// PoolParams: in_dims = operand, out_dims = source, n_out = operand elements, op = RED_MAX (ge) or
+// RED_MIN (le); dilation is not used. VEC = 4 has the same conditions as for pooling.
+template <int VEC>
+__device__ __forceinline__ void select_scatter_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                    const uint32_t* __restrict__ operand, const PoolParams& P) {
+    const uint64_t e0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * VEC;
+    if (e0 >= P.n_out) return;
+    int32_t c[4];
+    {
+        uint64_t r = e0;
+#pragma unroll
+        for (int d = 3; d >= 1; --d) { const uint64_t q = r / P.in_dims[d]; c[d] = (int32_t)(r - q * P.in_dims[d]); r = q; }
+        c[0] = (int32_t)r;
+    }
+    // windows that contain the element: o * stride - pad <= c < o * stride - pad + window
+    int32_t lo[4], hi[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const int32_t s = (int32_t)P.stride[d], a = c[d] + P.pad_low[d];
+        const int32_t first = a - (int32_t)P.window[d] + 1;
+        lo[d] = first <= 0 ? 0 : (first + s - 1) / s;
+        hi[d] = a < 0 ? -1 : a / s;
+        if (hi[d] > (int32_t)P.out_dims[d] - 1) hi[d] = (int32_t)P.out_dims[d] - 1;
+    }
+    if constexpr (VEC == 4) { lo[3] = hi[3] = 0; }           // the last dimension is not windowed: handled per lane element
+    const bool want_max = P.op == RED_MAX;
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.0f;
+    for (int32_t o0 = lo[0]; o0 <= hi[0]; ++o0)
+    for (int32_t o1 = lo[1]; o1 <= hi[1]; ++o1)
+    for (int32_t o2 = lo[2]; o2 <= hi[2]; ++o2)
+    for (int32_t o3 = lo[3]; o3 <= hi[3]; ++o3) {
+        float sel[VEC];
+        bool  mine[VEC], have = false;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) { sel[j] = 0.0f; mine[j] = false; }
+        const uint32_t w3 = VEC == 4 ? 1u : P.window[3];
+        for (uint32_t t0 = 0; t0 < P.window[0]; ++t0) {
+            const int32_t k0 = o0 * (int32_t)P.stride[0] - P.pad_low[0] + (int32_t)t0;
+            if (k0 < 0 || k0 >= (int32_t)P.in_dims[0]) continue;
+            for (uint32_t t1 = 0; t1 < P.window[1]; ++t1) {
+                const int32_t k1 = o1 * (int32_t)P.stride[1] - P.pad_low[1] + (int32_t)t1;
+                if (k1 < 0 || k1 >= (int32_t)P.in_dims[1]) continue;
+                for (uint32_t t2 = 0; t2 < P.window[2]; ++t2) {
+                    const int32_t k2 = o2 * (int32_t)P.stride[2] - P.pad_low[2] + (int32_t)t2;
+                    if (k2 < 0 || k2 >= (int32_t)P.in_dims[2]) continue;
+                    for (uint32_t t3 = 0; t3 < w3; ++t3) {
+                        const int32_t k3 = VEC == 4 ? c[3] : o3 * (int32_t)P.stride[3] - P.pad_low[3] + (int32_t)t3;
+                        if (k3 < 0 || k3 >= (int32_t)P.in_dims[3]) continue;
+                        const uint64_t off = (((uint64_t)k0 * P.in_dims[1] + k1) * P.in_dims[2] + k2) * P.in_dims[3] + k3;
+                        const bool me = k0 == c[0] && k1 == c[1] && k2 == c[2] && (VEC == 4 || k3 == c[3]);
+                        float v[VEC];
+                        if constexpr (VEC == 4) {
+                            const u32x4 q = *reinterpret_cast<const u32x4*>(operand + off);
+                            v[0] = u2f(q.x); v[1] = u2f(q.y); v[2] = u2f(q.z); v[3] = u2f(q.w);
+                        } else {
+                            v[0] = u2f(operand[off]);
+                        }
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) {
+                            const bool keep = have && (want_max ? sel[j] >= v[j] : sel[j] <= v[j]);
+                            if (!keep) { sel[j] = v[j]; mine[j] = me; }
+                        }
+                        have = true;
+                    }
+                }
+            }
+        }
+        const uint64_t soff = (((uint64_t)o0 * P.out_dims[1] + o1) * P.out_dims[2] + o2) * P.out_dims[3] + (VEC == 4 ? c[3] : o3);
+        if constexpr (VEC == 4) {
+            const u32x4 g = *reinterpret_cast<const u32x4*>(source + soff);
+            if (mine[0]) acc[0] += u2f(g.x);
+            if (mine[1]) acc[1] += u2f(g.y);
+            if (mine[2]) acc[2] += u2f(g.z);
+            if (mine[3]) acc[3] += u2f(g.w);
+        } else {
+            if (mine[0]) acc[0] += u2f(source[soff]);
+        }
+    }
+    if constexpr (VEC == 4) {
+        u32x4 r; r.x = f2u(acc[0]); r.y = f2u(acc[1]); r.z = f2u(acc[2]); r.w = f2u(acc[3]);
+        *reinterpret_cast<u32x4*>(out + e0) = r;
+    } else {
+        out[e0] = f2u(acc[0]);
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) void select_scatter_add_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                                        const uint32_t* __restrict__ operand, PoolParams P) {
+    select_scatter_body<1>(out, source, operand, P);
+}
+extern "C" __global__ __launch_bounds__(256) void select_scatter_add_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                                        const uint32_t* __restrict__ operand, PoolParams P) {
+    select_scatter_body<4>(out, source, operand, P);
+}

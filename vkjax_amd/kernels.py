@@ -404,7 +404,8 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     #the 16-byte A path keeps the validity of a row's taps in one 32-bit mask and addresses the
     #input from (PH, PW) positions before its start
     x_bias = (g.PH * g.xs[1] + g.PW * g.xs[2]) * 4
-    a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0
+    #(negative padding, i.e. cropping, goes through the generic loader's coordinate checks)
+    a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0 and g.PH >= 0 and g.PW >= 0
               and all(s % 4 == 0 and s >= 0 for s in g.xs[:3]) and (not needs_masks or g.KH * g.KW <= 32)
               and (lhs.size - lhs_offset) * 4 + x_bias <= 2**31)
     b_fast = (g.ws[3] == 1 and N % 4 == 0 and rhs_offset % 4 == 0
@@ -547,6 +548,46 @@ def pool(out: Buffer, inp: Buffer, op: str, window, strides, pad_low, dilation) 
                       bytes_moved=4 * (inp.size + out.size))
     return Launch(f'pool_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
                   bytes_moved=4 * (inp.size + out.size))
+
+
+def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, op: str, window, strides, pad_low) -> Launch:
+    '''Gradient of a max (`op` = 'reduce_max': select with ge) or min pooling; see select_scatter_body in reduce.hip.'''
+    rank = len(operand.shape)
+    if rank > 4:
+        raise NotImplementedError('select_and_scatter_add over more than 4 dimensions')
+    lead     = 4 - rank
+    in_dims  = [1] * lead + list(operand.shape)
+    out_dims = [1] * lead + list(source.shape)
+    window   = [1] * lead + list(window)
+    strides  = [1] * lead + list(strides)
+    pad_low  = [0] * lead + list(pad_low)
+    n   = operand.size
+    vec = 4 if (window[3] == 1 and strides[3] == 1 and pad_low[3] == 0 and in_dims[3] % 4 == 0
+                and in_dims[3] == out_dims[3]) else 1
+    if max(in_dims) >= 2**31 or any(abs(p) >= 2**30 for p in pad_low):
+        raise NotImplementedError('select_and_scatter_add: dimension too large')
+    params = _u32(n, RED[op], _RTYPE[operand.dtype], *in_dims, *out_dims, *window, *strides, 1, 1, 1, 1) + _i32(*pad_low)
+    return Launch(f'select_scatter_add_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                  [(out, 0), (source, 0), (operand, 0)], params, bytes_moved=4 * (2 * operand.size + source.size))
+
+
+PAD_MAX_RANK = 6
+
+
+def pad(out: Buffer, inp: Buffer, value: Buffer, padding_config) -> Launch:
+    rank = len(inp.shape)
+    if rank > PAD_MAX_RANK:
+        raise NotImplementedError('pad with rank > 6')
+    lead = PAD_MAX_RANK - rank
+    config   = [(0, 0, 0)] * lead + [tuple(int(v) for v in c) for c in padding_config]
+    in_dims  = [1] * lead + list(inp.shape)
+    out_dims = [1] * lead + list(out.shape)
+    #an empty operand contributes nothing: give the kernel a dimension no index can fall into
+    in_dims  = [max(d, 0) for d in in_dims]
+    vec = 4 if (config[-1] == (0, 0, 0) and out_dims[-1] % 4 == 0) else 1
+    params = _u32(out.size, *out_dims, *in_dims) + _i32(*[c[0] for c in config]) + _u32(*[c[2] + 1 for c in config])
+    return Launch(f'pad_nd_v{vec}', (_cdiv(_cdiv(out.size, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                  [(out, 0), (inp, 0), (value, 0)], params, bytes_moved=4 * (inp.size + out.size))
 
 
 # --------------------------------------------------------------------------- gather / scatter / rng

@@ -422,6 +422,37 @@ def reduce_window(x, init_value, computation, window_dimensions, window_strides,
                      window_dilation=tuple(window_dilation or (1,) * len(xs))))
 
 
+def select_and_scatter_add(source, operand, select_prim, window_dimensions, window_strides, padding):
+    '''The gradient of a max/min pooling as autodiff emits it (`select_prim` is `ge_p` or `le_p`).'''
+    xs = _shape(operand)
+    wd = tuple(int(w) for w in window_dimensions)
+    ws = tuple(int(s) for s in window_strides)
+    padding = tuple((int(lo), int(hi)) for lo, hi in padding)
+    pooled  = tuple(builtins.max((n + lo + hi - w) // s + 1, 0) for n, w, s, (lo, hi) in zip(xs, wd, ws, padding))
+    if _shape(source) != pooled:
+        raise TypeError(f'select_and_scatter_add: source {_shape(source)} does not match the pooled shape {pooled}')
+    if dtype_of(source)[0] != _f32 or dtype_of(operand)[0] != _f32:
+        raise TypeError('select_and_scatter_add takes float32 operands')
+    if getattr(select_prim, 'name', None) not in ('ge', 'le'):
+        raise NotImplementedError('select_and_scatter_add selects with ge or le')
+    return emit('select_and_scatter_add', [source, operand], [_aval(xs, _f32)],
+                dict(select_prim=select_prim, window_dimensions=wd, window_strides=ws, padding=padding))
+
+
+ge_p, le_p = core.Primitive('ge'), core.Primitive('le')
+
+
+def pad(x, padding_value, padding_config):
+    '''(low, high, interior) per dimension; negative low/high crop.'''
+    dtype  = dtype_of(x)[0]
+    config = tuple((int(lo), int(hi), int(it)) for lo, hi, it in padding_config)
+    xs     = _shape(x)
+    if len(config) != len(xs) or builtins.any(it < 0 for _, _, it in config):
+        raise TypeError('pad needs one (low, high, interior >= 0) triple per dimension')
+    shape  = tuple(builtins.max(n + builtins.max(n - 1, 0) * it + lo + hi, 0) for n, (lo, hi, it) in zip(xs, config))
+    return emit('pad', [x, _as_dtype(padding_value, dtype)], [_aval(shape, dtype)], dict(padding_config=config))
+
+
 # ---------------------------------------------------------------- indexing
 
 def gather(operand, start_indices, dimension_numbers: GatherDimensionNumbers, slice_sizes,

@@ -620,6 +620,32 @@ def reduce_window_sum(bufferpool, equation):
 
 # ------------------------------------------------------------------ indexing
 
+def select_and_scatter_add(bufferpool, equation):
+    '''Gradient of reduce_window_max / min as autodiff emits it: operands (source, operand),
+    select_prim ge or le.'''
+    params = equation.params
+    select = getattr(params['select_prim'], 'name', str(params['select_prim']))
+    if select not in ('ge', 'le'):
+        raise NotImplementedError(equation)
+    source, operand = [bufferpool.get_buffer(v) for v in equation.invars]
+    if _kind(operand.dtype) != _F or _kind(source.dtype) != _F:
+        raise NotImplementedError(equation)
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    if outbuf.size == 0:
+        return []
+    pad_low = [int(lo) for lo, _ in params['padding']]
+    return [Op(equation, launch=K.select_scatter_add(outbuf, source, operand, 'reduce_max' if select == 'ge' else 'reduce_min',
+                                                     params['window_dimensions'], params['window_strides'], pad_low))]
+
+
+def pad(bufferpool, equation):
+    inbuf, value = [bufferpool.get_buffer(v) for v in equation.invars]
+    outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
+    if outbuf.size == 0:
+        return []
+    return [Op(equation, launch=K.pad(outbuf, inbuf, value, equation.params['padding_config']))]
+
+
 def gather(bufferpool, equation):
     params = equation.params
     dn     = params['dimension_numbers']

@@ -174,6 +174,66 @@ def gather_scatter_inputs(seed=5, rows=65536, cols=256, n0=8192, n1=32):
     return [table, idx, updates]
 
 
+# ------------------------------------------------------------------ training steps (forward, backward, SGD update)
+
+def softmax_cross_entropy(logits, onehot):
+    z    = logits - lax.stop_gradient(jnp.max(logits, axis=1, keepdims=True))
+    logp = z - jnp.log(jnp.sum(jnp.exp(z), axis=1, keepdims=True))
+    return -jnp.mean(jnp.sum(onehot * logp, axis=1))
+
+
+def _sgd(params, grads, lr):
+    return mj.tree_multimap(lambda p, g: p - np.float32(lr) * g, params, grads)
+
+
+def mlp_loss(params, x, onehot):
+    h = nn.relu(jnp.dot(x, params['w1']) + params['b1'])
+    h = nn.relu(jnp.dot(h, params['w2']) + params['b2'])
+    return softmax_cross_entropy(jnp.dot(h, params['w3']) + params['b3'], onehot)
+
+
+def mlp_train_step(params, x, onehot, lr=0.05):
+    '''One SGD step of the MLP on a batch: returns (loss, updated parameters). The backward pass is the
+    program autodiff produces (transposed dot_generals, relu masks, bias gradients as reduce_sum).'''
+    loss, grads = mj.value_and_grad(mlp_loss)(params, x, onehot)
+    return loss, _sgd(params, grads, lr)
+
+
+def mlp_train_inputs(seed=6, batch=256, sizes=(784, 512, 512, 10)):
+    params, x = mlp_inputs(seed, batch, sizes)
+    rng = np.random.default_rng(seed + 1000)
+    onehot = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], size=batch)]
+    return [params, x, onehot]
+
+
+def convnet_loss(params, x, onehot):
+    '''A small convolutional classifier that exercises every gradient form of the path: strided 3x3 convolution,
+    per-channel scale and shift, relu, 3x3/2 max pooling, 3x3 convolution, 2x2 average pooling, global mean, dense.'''
+    y = lax.conv_general_dilated(x, params['w1'], window_strides=(2, 2), padding=((1, 1), (1, 1)), dimension_numbers=NHWC)
+    y = nn.relu(y * params['scale'] + params['shift'])
+    y = lax.reduce_window(y, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (0, 1), (0, 1), (0, 0)))
+    y = nn.relu(lax.conv_general_dilated(y, params['w2'], window_strides=(1, 1), padding=((1, 1), (1, 1)), dimension_numbers=NHWC))
+    y = lax.reduce_window(y, 0.0, lax.add, (1, 2, 2, 1), (1, 2, 2, 1), 'VALID') / 4.0
+    y = jnp.mean(y, axis=(1, 2))
+    return softmax_cross_entropy(jnp.dot(y, params['w3']) + params['b3'], onehot)
+
+
+def convnet_train_step(params, x, onehot, lr=0.05):
+    loss, grads = mj.value_and_grad(convnet_loss)(params, x, onehot)
+    return loss, _sgd(params, grads, lr)
+
+
+def convnet_train_inputs(seed=7, batch=64, size=64, channels=(3, 64, 128), classes=10):
+    rng = np.random.default_rng(seed)
+    c0, c1, c2 = channels
+    params = dict(w1=he_normal(rng, (3, 3, c0, c1), 9 * c0), scale=(0.5 + rng.random(c1, dtype=np.float32)).astype(np.float32),
+                  shift=(0.1 * rng.standard_normal(c1, dtype=np.float32)).astype(np.float32),
+                  w2=he_normal(rng, (3, 3, c1, c2), 9 * c1), w3=he_normal(rng, (c2, classes), c2), b3=np.zeros((classes,), np.float32))
+    x = rng.random((batch, size, size, c0), dtype=np.float32)
+    onehot = np.eye(classes, dtype=np.float32)[rng.integers(0, classes, size=batch)]
+    return [params, x, onehot]
+
+
 WORKLOADS: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable]] = {
     'affine':         (affine, affine_inputs),
     'mlp':            (mlp, mlp_inputs),
@@ -181,4 +241,6 @@ WORKLOADS: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable]] = {
     'resnet50':       (resnet50, resnet50_inputs),
     'rng_uniform':    (rng_uniform, rng_inputs),
     'gather_scatter': (gather_scatter, gather_scatter_inputs),
+    'mlp_train':      (mlp_train_step, mlp_train_inputs),
+    'convnet_train':  (convnet_train_step, convnet_train_inputs),
 }
