@@ -28,11 +28,14 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS          = 8000.0
 
 UNITS = {'resnet50': ('images/sec', 'batch'), 'mlp': ('samples/sec', 'batch'), 'conv_block': ('images/sec', 'batch'),
-         'affine': ('calls/sec', None), 'rng_uniform': ('Gsamples/sec', None), 'gather_scatter': ('Grows/sec', None)}
+         'affine': ('calls/sec', None), 'rng_uniform': ('Gsamples/sec', None), 'gather_scatter': ('Grows/sec', None),
+         'mlp_train': ('samples/sec', 'batch'), 'convnet_train': ('images/sec', 'batch')}
+BATCHED = ('resnet50', 'mlp', 'conv_block', 'mlp_train', 'convnet_train')
 
 
 def kernel_family(name: str) -> str:
-    for prefix in ('conv_gemm', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows'):
+    for prefix in ('conv_gemm', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows',
+                   'select_scatter', 'pad_nd'):
         if name.startswith(prefix):
             return prefix
     return name
@@ -98,7 +101,7 @@ def main():
     ms_per_step = wall_s * 1e3 / args.steps
 
     leaves = tree_util.tree_leaves(inputs)
-    if args.workload in ('resnet50', 'mlp', 'conv_block'):
+    if args.workload in BATCHED:
         units_per_step = leaves[-1].shape[0]
     elif args.workload == 'rng_uniform':
         units_per_step = 4096 * 4096 / 1e9
@@ -217,6 +220,9 @@ def time_cpu_baseline(workload, fn, make_inputs, kwargs):
     if workload == 'resnet50':
         sample_kwargs['batch'] = 4
         sample = 'batch 4 of the same 224x224x3 ResNet-50 forward'
+    if workload == 'convnet_train':
+        sample_kwargs['batch'] = 1
+        sample = 'batch 1 of the same training step (the pooling gradient of the oracle is a python loop)'
     inputs = make_inputs(**sample_kwargs)
     closed = mj.make_jaxpr(fn)(*inputs)
     leaves = tree_util.tree_leaves(inputs)
@@ -227,7 +233,7 @@ def time_cpu_baseline(workload, fn, make_inputs, kwargs):
         t_total += time.perf_counter() - t0
         reps += 1
     per_call = t_total / reps
-    if workload in ('resnet50', 'mlp', 'conv_block'):
+    if workload in BATCHED:
         units = leaves[-1].shape[0]
     elif workload == 'rng_uniform':
         units = 4096 * 4096 / 1e9

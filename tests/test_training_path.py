@@ -226,6 +226,60 @@ def test_conv_gradient_forms_hip():
         check_against_oracle(f, [random(xs) - 0.5, random(ws) - 0.5], rtol=1e-4, atol=1e-5)
 
 
+WGRAD_CASES = [   #x, kernel, strides, padding, rhs_dilation; the loader variant in the name
+    ('aa', (4, 12, 12, 8), (3, 3, 8, 16), (1, 1), ((1, 1), (1, 1)), (1, 1)),
+    ('aa strided', (3, 17, 15, 4), (3, 3, 4, 8), (2, 2), ((1, 1), (0, 1)), (1, 1)),
+    ('sa stem', (2, 20, 20, 3), (7, 7, 3, 8), (2, 2), ((3, 3), (3, 3)), (1, 1)),
+    ('as', (2, 10, 10, 8), (1, 1, 8, 10), (1, 1), ((0, 0), (0, 0)), (1, 1)),
+    ('ss dilated', (2, 13, 11, 5), (2, 3, 5, 7), (1, 1), ((1, 1), (2, 2)), (2, 2)),
+    ('aa wide', (2, 10, 10, 72), (3, 3, 72, 136), (1, 1), ((1, 1), (1, 1)), (1, 1)),
+]
+
+
+def _kernel_gradient_function(strides, padding, rhs_dilation):
+    def loss(x, w):
+        y = lax.conv_general_dilated(x, w, window_strides=strides, padding=padding, rhs_dilation=rhs_dilation, dimension_numbers=W.NHWC)
+        return jnp.sum(y * y) * 0.5
+    return lambda x, w: mj.grad(loss, argnums=1)(x, w)
+
+
+@pytest.mark.parametrize('case', WGRAD_CASES, ids=[c[0] for c in WGRAD_CASES])
+def test_kernel_gradients_take_the_wgrad_kernel(case):
+    name, xs, ws, strides, padding, rhs_dilation = case
+    closed = mj.make_jaxpr(_kernel_gradient_function(strides, padding, rhs_dilation))(random(xs), random(ws))
+    kernels = [l.kernel for l in JaxprInterpreter(closed, plan_only=True).launches]
+    assert f'wgrad_gemm_64x64_{name[:2]}' in kernels, kernels
+
+
+def test_dense_layer_weight_gradient_takes_the_wgrad_kernel():
+    closed = mj.make_jaxpr(lambda x, g: lax.dot_general(x, g, (((0,), (0,)), ((), ()))))(random([256, 40]), random([256, 10]))
+    kernels = [l.kernel for l in JaxprInterpreter(closed, plan_only=True).launches]
+    assert kernels[0] == 'wgrad_gemm_64x64_as' and (len(kernels) == 1 or kernels[1].startswith('reduce_cols')), kernels
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('case', WGRAD_CASES, ids=[c[0] for c in WGRAD_CASES])
+def test_kernel_gradient_hip(case):
+    name, xs, ws, strides, padding, rhs_dilation = case
+    print(f'case: kernel gradient {name} x{xs} w{ws}', flush=True)
+    #integer-valued operands: every product and partial sum is exact, so the result does not depend on the split
+    x = np.round(random(xs) * 8 - 4).astype(np.float32)
+    w = np.round(random(ws) * 4 - 2).astype(np.float32)
+    check_against_oracle(_kernel_gradient_function(strides, padding, rhs_dilation), [x, w], exact=True)
+    check_against_oracle(_kernel_gradient_function(strides, padding, rhs_dilation), [random(xs) - 0.5, random(ws) - 0.5], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_rows_contracted_dot_hip():
+    for k, m, n in ((256, 40, 10), (1000, 65, 64), (4096, 128, 256), (130, 3, 5)):
+        print(f'case: x^T g with {k} rows, {m} x {n}', flush=True)
+        f = lambda x, g: lax.dot_general(x, g, (((0,), (0,)), ((), ())))
+        x = np.round(random([k, m]) * 8 - 4).astype(np.float32)
+        g = np.round(random([k, n]) * 8 - 4).astype(np.float32)
+        check_against_oracle(f, [x, g], exact=True)
+        check_against_oracle(f, [random([k, m]) - 0.5, random([k, n]) - 0.5], rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize('name,make_inputs', [('mlp_train', small_mlp_inputs), ('convnet_train', small_convnet_inputs)])
 def test_training_step_hip_matches_oracle(name, make_inputs):

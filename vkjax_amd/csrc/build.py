@@ -21,7 +21,7 @@ ARCH    = 'gfx950'
 DEVICE_FLAGS = ['-O3', f'--offload-arch={ARCH}', '--genco', '-munsafe-fp-atomics', '-ffp-contract=off',
                 '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops', '-Wno-pass-failed']
 
-KERNEL_SOURCES = ['elementwise', 'conv_gemm', 'reduce', 'index', 'threefry']
+KERNEL_SOURCES = ['elementwise', 'conv_gemm', 'wgrad_gemm', 'reduce', 'index', 'threefry']
 
 
 def shim_path():

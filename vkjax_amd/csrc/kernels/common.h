@@ -19,3 +19,22 @@ __device__ __forceinline__ T wave_allreduce(T v, F f) {
     for (int off = 32; off >= 1; off >>= 1) v = f(v, __shfl_xor(v, off, VKJ_WAVE));
     return v;
 }
+
+// Buffer-descriptor access: loads beyond `bytes` return 0 and stores there are dropped, so a lane
+// that must not touch memory is given an offset of 0x80000000.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+// voff: per-lane byte offset, soff: wave-uniform byte offset; the range check covers their sum
+__device__ __forceinline__ f32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ float buffer_load_x1(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, voff, soff, 0);
+}
+__device__ __forceinline__ int magic_div(int n, uint32_t magic, uint32_t shift) {
+    return magic ? (int)(__umulhi((uint32_t)n, magic) >> shift) : n;
+}

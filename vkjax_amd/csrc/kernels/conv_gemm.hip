@@ -88,23 +88,6 @@ struct ConvDerived {
     uint32_t left[CONV_MAX_DERIVED];        // the operand is the left argument
 };
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
-}
-// voff: per-lane byte offset, soff: wave-uniform byte offset; the range check covers their sum
-__device__ __forceinline__ f32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
-    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
-}
-__device__ __forceinline__ float buffer_load_x1(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
-}
-__device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, voff, soff, 0);
-}
-__device__ __forceinline__ int magic_div(int n, uint32_t magic, uint32_t shift) {
-    return magic ? (int)(__umulhi((uint32_t)n, magic) >> shift) : n;
-}
-
 // Optional per-block phase time stamps (profiling builds only): slot s of block b lands in
 // ((uint64*)epi.p[CONV_MAX_EPI - 1])[16 * b + s].
 #ifdef CONV_PHASE_STAMPS

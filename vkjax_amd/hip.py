@@ -17,7 +17,7 @@ _PKG    = os.path.dirname(os.path.abspath(__file__))
 LIBDIR  = os.path.join(_PKG, 'lib')
 LIBPATH = os.path.join(LIBDIR, 'libvkjax_hip.so')
 
-KERNEL_MODULES = ('elementwise', 'conv_gemm', 'reduce', 'index', 'threefry')
+KERNEL_MODULES = ('elementwise', 'conv_gemm', 'wgrad_gemm', 'reduce', 'index', 'threefry')
 
 EVAL_SKIP_UPLOADS   = 1
 EVAL_SKIP_DOWNLOADS = 2

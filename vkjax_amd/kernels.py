@@ -273,6 +273,43 @@ class ConvGeometry(tp.NamedTuple):
     def K(self): return self.KH * self.KW * self.Cin
 
 
+class WgradGeometry(tp.NamedTuple):
+    '''Kernel gradient of an NHWC / HWIO convolution in the forward convolution's own terms: X is
+    [images, H, W, C], the output cotangent G is [images, Ho, Wo, N], the result [KH, KW, C, N]
+    (see csrc/kernels/wgrad_gemm.hip). A product X^T G of row-major matrices is the 1x1 case.'''
+    images: int; Ho: int; Wo: int; H: int; W: int; C: int; KH: int; KW: int; N: int
+    SH: int = 1; SW: int = 1; PH: int = 0; PW: int = 0; DH: int = 1; DW: int = 1
+
+    @property
+    def pixels(self): return self.images * self.Ho * self.Wo
+    @property
+    def M(self): return self.KH * self.KW * self.C
+
+
+def choose_wgrad_splits(g: WgradGeometry, compute_units: int = 256) -> int:
+    '''Slices of the contraction: enough blocks to fill the chip several times over, at least four
+    k steps of 32 pixels per slice.'''
+    tiles = _cdiv(g.M, 64) * _cdiv(g.N, 64)
+    want  = _cdiv(4 * compute_units, tiles)
+    return max(1, min(want, g.pixels // 128, 1024))
+
+
+def wgrad_gemm(out: Buffer, x: Buffer, cot: Buffer, g: WgradGeometry, splits: int) -> Launch:
+    '''`out` holds `splits` partial results of M * N elements each (the result itself when splits == 1).'''
+    for name, b in (('input', x), ('cotangent', cot)):
+        if b.size * 4 >= 2**31:
+            raise NotImplementedError(f'kernel gradient: {name} of {b.size * 4} bytes exceeds the 2 GiB the kernel addresses')
+    assert x.size == g.images * g.H * g.W * g.C and cot.size == g.pixels * g.N and out.size == splits * g.M * g.N
+    per_split = _cdiv(_cdiv(g.pixels, splits), 32) * 32
+    assert per_split * splits >= g.pixels
+    magics = [v for d in (g.Ho * g.Wo, g.Wo, g.C, g.KW) for v in _magic_division(d)]
+    params = _i32(g.pixels, g.M, g.N, g.Ho, g.Wo, g.H, g.W, g.C, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW, per_split) \
+           + _u32(*magics, x.size * 4, cot.size * 4)
+    kernel = 'wgrad_gemm_64x64_' + ('a' if g.C % 4 == 0 else 's') + ('a' if g.N % 4 == 0 else 's')
+    return Launch(kernel, (_cdiv(g.N, 64), _cdiv(g.M, 64), splits), (256, 1, 1), [(out, 0), (x, 0), (cot, 0)], params,
+                  bytes_moved=4 * (x.size + cot.size + out.size), flops=2 * g.pixels * g.M * g.N)
+
+
 class ConvDerivedOperand(tp.NamedTuple):
     '''A per-feature epilogue operand that the kernel computes instead of reading: `first` and the
     step operands are buffers of N values or of one value.'''

@@ -483,6 +483,23 @@ custom_vjp_call = custom_vjp_call_jaxpr = custom_jvp_call
 
 # ------------------------------------------------------------------ contractions
 
+#contractions at least this long over the slowest dimension of both operands go to the kernel-gradient GEMM
+WGRAD_MIN_PIXELS = 128
+
+
+def _wgrad_ops(bufferpool, equation, outbuf, x, cot, wg: 'K.WgradGeometry'):
+    '''X^T G over the pixels, split over the contraction; the slices are added by a column reduction.'''
+    splits = K.choose_wgrad_splits(wg)
+    if splits == 1:
+        return [Op(equation, launch=K.wgrad_gemm(outbuf, x, cot, wg, 1))]
+    position = bufferpool.op_counter
+    bufferpool.op_counter -= 1                  #the temporary lives at the equation's own position
+    partial = bufferpool.new_temporary(np.float32, (splits, wg.M * wg.N))
+    bufferpool.op_counter = position
+    launches = [K.wgrad_gemm(partial, x, cot, wg, splits)] + K.reduce(outbuf, partial, 1, splits, wg.M * wg.N, 'reduce_sum')
+    return [Op(equation, launch=l) for l in launches]
+
+
 def dot_general(bufferpool, equation):
     '''2-D x 2-D, one contracting dimension per side, no batch dimensions, float32
     (reference: vkjax/ops.py:277-297). Lowered onto the implicit-GEMM kernel with a 1x1 window.'''
@@ -500,6 +517,12 @@ def dot_general(bufferpool, equation):
     M, N = outbuf.shape
     Kc   = lhs.shape[lc[0]]
     lst, rst = K.row_major_strides(lhs.shape), K.row_major_strides(rhs.shape)
+    if outbuf.size == 0:
+        return []
+    if tuple(lc) == (0,) and tuple(rc) == (0,) and Kc >= WGRAD_MIN_PIXELS:
+        #both operands contracted over their rows (a dense layer's weight gradient): read along the rows
+        wg = K.WgradGeometry(images=1, Ho=Kc, Wo=1, H=Kc, W=1, C=M, KH=1, KW=1, N=N)
+        return _wgrad_ops(bufferpool, equation, outbuf, lhs, rhs, wg)
     geom = K.ConvGeometry(batch=1, Ho=M, Wo=1, N=N, H=M, W=1, Cin=Kc, KH=1, KW=1,
                           xs=(0, lst[1 - lc[0]], 0, lst[lc[0]]),
                           ws=(rst[rc[0]] * Kc, rst[rc[0]] * Kc, rst[rc[0]], rst[1 - rc[0]]),
@@ -537,7 +560,25 @@ def conv_general_dilated(bufferpool, equation):
                           os=(os_[0], os_[2], os_[3], os_[1]))
     if outbuf.size == 0:
         return []
+    wg = _as_kernel_gradient(geom)
+    if wg is not None:
+        return _wgrad_ops(bufferpool, equation, outbuf, lhs, rhs, wg)
     return [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+
+
+def _as_kernel_gradient(g: 'K.ConvGeometry') -> tp.Optional['K.WgradGeometry']:
+    '''The convolution autodiff emits for the kernel gradient of an NHWC / HWIO convolution: its "batch" is
+    the forward input's (contiguous) feature dimension, its contraction runs over the forward batch and
+    over the cotangent's pixels, which act as the window. Returns that convolution in forward terms, or
+    None when the operands are laid out differently.'''
+    images, C, N = g.Cin, g.batch, g.N
+    x_dense   = g.xs == (1, g.W * C, C, g.H * g.W * C)
+    cot_dense = g.ws == (g.KW * N, N, g.KH * g.KW * N, 1)
+    out_dense = g.os == (N, g.Wo * C * N, C * N, 1)
+    if not (x_dense and cot_dense and out_dense and g.LH == 1 and g.LW == 1 and images * g.KH * g.KW >= WGRAD_MIN_PIXELS):
+        return None
+    return K.WgradGeometry(images=images, Ho=g.KH, Wo=g.KW, H=g.H, W=g.W, C=C, KH=g.Ho, KW=g.Wo, N=N,
+                           SH=g.DH, SW=g.DW, PH=g.PH, PW=g.PW, DH=g.SH, DW=g.SW)
 
 
 # ------------------------------------------------------------------ reductions
