@@ -7,6 +7,9 @@ something computed by this repository's code:
   * `jax.random.split(jax.random.PRNGKey(0))` and `jax.random.uniform(jax.random.PRNGKey(0))`
     as printed in the JAX documentation ("Pseudo random numbers in JAX") for the original,
     non-partitionable threefry layout.
+  * `jax.random.normal(PRNGKey(0), (1,))` = [-0.20584226] (JAX documentation, "JAX PRNG design") and the ten
+    values `random.normal(random.PRNGKey(0), (10,))` prints in the JAX quickstart; `uniform(key(0))` = 0.947667
+    and `uniform(split(key(0))[1])` = 0.00729382 from the jax.random module documentation (partitionable layout).
   * The literal expectations of the reference's own tests: f(65) == 66, f(-5) == -4
     (tests/test_function.py:15-16), shift_right_logical(1, 32) == 0 (tests/test_basic_ops.py:150-151,305),
     buffer-reuse counts 2 and 8 (tests/test_bufferpool.py:40,63).
@@ -23,6 +26,10 @@ KNOWN = {
     ],
     'jax_random_split_PRNGKey0': [[4146024105, 967050713], [2718843009, 1272950319]],
     'jax_random_uniform_PRNGKey0': {'bits': 1797259609, 'value': 0.41845703},
+    'jax_random_normal_PRNGKey0': {'shape_1': [-0.20584226],
+                                   'shape_10': [-0.3721109, 0.26423115, -0.18252768, -0.7368197, -0.44030377, -0.1521442,
+                                                -0.67135346, -0.5908641, 0.73168886, 0.5673026]},
+    'jax_random_partitionable_key0': {'uniform': 0.947667, 'uniform_of_second_subkey': 0.00729382},
     'reference_test_literals': {'func0_65': 66, 'func0_minus5': -4, 'shift_right_logical_1_32': 0,
                                 'bufferpool_lowlevel_unique_tensors': 2, 'bufferpool_highlevel_unique_tensors': 8,
                                 'bufferpool_lowlevel_accesses': [[0, 2], [1], [3]]},

@@ -1,6 +1,9 @@
 '''The key primitives newer jax versions trace for jax.random (random_seed / random_wrap /
 random_bits / random_split / random_fold_in / random_unwrap): oracle pins and launch plans on
 the CPU, parity of the HIP path on the GPU. Both counter layouts of jax are covered.'''
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -80,11 +83,12 @@ def test_oracle_partitionable_layout_matches_documented_jax_values():
     try:
         key0 = P.random_seed(np.int32(0))
         assert key0.tolist() == [0, 0]
+        published = json.load(open(os.path.join(os.path.dirname(__file__), 'golden', 'known_answers.json')))['jax_random_partitionable_key0']
         bits = P.random_bits(key0, 32, ())
-        assert np.float32((int(bits) >> 9) * 2.0**-23) == np.float32(0.947667)
+        assert np.float32((int(bits) >> 9) * 2.0**-23) == np.float32(published['uniform'])
         subkey = P.random_split(key0, (2,))[1]
         bits = P.random_bits(subkey, 32, ())
-        assert abs(np.float32((int(bits) >> 9) * 2.0**-23) - np.float32(0.00729382)) < 5e-9
+        assert abs(np.float32((int(bits) >> 9) * 2.0**-23) - np.float32(published['uniform_of_second_subkey'])) < 5e-9
         #closed form: element i of a draw is the xor of the block function's words on the counter (0, i)
         draw = P.random_bits(KEY, 32, (3, 5))
         for i in range(15):
@@ -126,6 +130,17 @@ def test_hip_matches_oracle(layout, f, args):
     print(f'case: {f.__name__} partitionable={layout}', flush=True)
     for fuse in (True, False):
         check_against_oracle(f, args, exact=True, fuse=fuse)
+
+
+@pytest.mark.gpu
+def test_normal_draw_hip(layout):
+    '''uniform -> erf_inv -> * sqrt(2) folded into the generating kernel; tolerance of element-wise float work.'''
+    def draw(key): return mrandom.normal(key, (257, 129))
+    print(f'case: normal draw partitionable={layout}', flush=True)
+    y, ytrue, fn = check_against_oracle(draw, [KEY], rtol=1e-5, atol=1e-6)
+    assert abs(float(y.mean())) < 0.02 and abs(float(y.std()) - 1.0) < 0.02
+    interp = next(iter(fn._jaxpr_interpreters.values()))
+    assert len(interp.launches) <= 2, [l.kernel for l in interp.launches]      #the generating kernel and, at most, the tail of the chain
 
 
 @pytest.mark.gpu

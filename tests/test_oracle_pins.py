@@ -55,6 +55,16 @@ def test_split_and_uniform_match_published_jax_values():
     assert np.float32(u) == np.float32((int(bits) >> 9) * 2.0 ** -23)
 
 
+def test_normal_matches_published_jax_values():
+    '''jax's documentation prints random.normal(PRNGKey(0), (1,)) = [-0.20584226] and the ten values of
+    random.normal(PRNGKey(0), (10,)) in its quickstart; they pin the uniform -> erf_inv path end to end.'''
+    key = mj.random.PRNGKey(0)
+    for shape, name in (((1,), 'shape_1'), ((10,), 'shape_10')):
+        closed = mj.make_jaxpr(lambda k: mj.random.normal(k, shape))(key)
+        (x,) = eval_closed_jaxpr(closed, key)
+        assert np.allclose(x, np.float32(GOLDEN['jax_random_normal_PRNGKey0'][name]), rtol=2e-6, atol=0)
+
+
 def test_random_bits_odd_sizes_pad_and_trim():
     key = mj.random.PRNGKey(42)
     for n in (1, 2, 5, 6, 33):

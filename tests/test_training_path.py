@@ -183,7 +183,7 @@ def test_training_steps_plan_at_full_size(name):
     kernels = [l.kernel for l in interp.launches]
     assert any(k.startswith('conv_gemm') for k in kernels)
     if name == 'convnet_train':
-        assert 'select_scatter_add_v4' in kernels and any(k.startswith('pad_nd') for k in kernels)
+        assert 'select_window_v4' in kernels and 'scatter_selected_v4' in kernels and any(k.startswith('pad_nd') for k in kernels)
 
 
 @pytest.mark.parametrize('f,args', pad_cases, ids=[c[0].__name__ for c in pad_cases])

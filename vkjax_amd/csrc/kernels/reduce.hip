@@ -403,16 +403,65 @@ extern "C" __global__ __launch_bounds__(256) void pool_v4(uint32_t* __restrict__
 // select_and_scatter_add: the gradient of a max (or min) pooling. Every window of `operand` selects
 // one of its elements (scan in row-major order over the positions inside the array, the first is
 // taken, a later one replaces it when !(selected >= candidate), resp. <=); the window's `source`
-// value is added at that position. Written as a gather so that no atomics are needed and the sums
-// have a fixed order: one thread per operand element (four with VEC = 4) walks the windows that
-// contain it in row-major order, repeats each window's selection and adds the source value when the
-// selection is its own element. Re-reads of the operand (window size x windows per element) hit
-// the caches; HBM sees operand + source once and the result once.
-// PoolParams: in_dims = operand, out_dims = source, n_out = operand elements, op = RED_MAX (ge) or
-// RED_MIN (le); dilation is not used. VEC = 4 has the same conditions as for pooling.
+// value is added at that position. Two passes, no atomics, sums in a fixed order:
+//   select_window   one thread per window (four channels with VEC = 4) repeats the scan and stores
+//                   the row-major number of the selected tap inside the window (0xFFFFFFFF: the
+//                   window lies entirely outside the array);
+//   scatter_selected one thread per operand element walks the windows that contain it in row-major
+//                   order and adds the source value of those whose selected tap is this element.
+// HBM sees the operand once, the result once and the two small window-sized arrays a few times.
+// PoolParams: in_dims = operand, out_dims = source / selection, op = RED_MAX (ge) or RED_MIN (le);
+// dilation is not used. VEC = 4 has the same conditions as for pooling.
 template <int VEC>
-__device__ __forceinline__ void select_scatter_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
-                                                    const uint32_t* __restrict__ operand, const PoolParams& P) {
+__device__ __forceinline__ void select_window_body(uint32_t* __restrict__ sel_out, const uint32_t* __restrict__ operand, const PoolParams& P) {
+    const uint64_t e0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * VEC;
+    if (e0 >= P.n_out) return;
+    int32_t o[4];
+    {
+        uint64_t r = e0;
+#pragma unroll
+        for (int d = 3; d >= 1; --d) { const uint64_t q = r / P.out_dims[d]; o[d] = (int32_t)(r - q * P.out_dims[d]); r = q; }
+        o[0] = (int32_t)r;
+    }
+    const bool want_max = P.op == RED_MAX;
+    float sel[VEC];
+    uint32_t pick[VEC];
+    bool have = false;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { sel[j] = 0.0f; pick[j] = 0xFFFFFFFFu; }
+    const uint32_t w3 = VEC == 4 ? 1u : P.window[3];
+    uint32_t tap = 0;
+    for (uint32_t t0 = 0; t0 < P.window[0]; ++t0)
+    for (uint32_t t1 = 0; t1 < P.window[1]; ++t1)
+    for (uint32_t t2 = 0; t2 < P.window[2]; ++t2)
+    for (uint32_t t3 = 0; t3 < w3; ++t3, ++tap) {
+        const int32_t k0 = o[0] * (int32_t)P.stride[0] - P.pad_low[0] + (int32_t)t0;
+        const int32_t k1 = o[1] * (int32_t)P.stride[1] - P.pad_low[1] + (int32_t)t1;
+        const int32_t k2 = o[2] * (int32_t)P.stride[2] - P.pad_low[2] + (int32_t)t2;
+        const int32_t k3 = VEC == 4 ? o[3] : o[3] * (int32_t)P.stride[3] - P.pad_low[3] + (int32_t)t3;
+        if ((uint32_t)k0 >= P.in_dims[0] || (uint32_t)k1 >= P.in_dims[1] || (uint32_t)k2 >= P.in_dims[2] || (uint32_t)k3 >= P.in_dims[3]) continue;
+        const uint64_t off = (((uint64_t)k0 * P.in_dims[1] + k1) * P.in_dims[2] + k2) * P.in_dims[3] + k3;
+        float v[VEC];
+        if constexpr (VEC == 4) {
+            const u32x4 q = *reinterpret_cast<const u32x4*>(operand + off);
+            v[0] = u2f(q.x); v[1] = u2f(q.y); v[2] = u2f(q.z); v[3] = u2f(q.w);
+        } else {
+            v[0] = u2f(operand[off]);
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const bool keep = have && (want_max ? sel[j] >= v[j] : sel[j] <= v[j]);
+            if (!keep) { sel[j] = v[j]; pick[j] = tap; }
+        }
+        have = true;
+    }
+    if constexpr (VEC == 4) *reinterpret_cast<u32x4*>(sel_out + e0) = u32x4{pick[0], pick[1], pick[2], pick[3]};
+    else sel_out[e0] = pick[0];
+}
+
+template <int VEC>
+__device__ __forceinline__ void scatter_selected_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                      const uint32_t* __restrict__ selected, const PoolParams& P) {
     const uint64_t e0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * VEC;
     if (e0 >= P.n_out) return;
     int32_t c[4];
@@ -433,7 +482,7 @@ __device__ __forceinline__ void select_scatter_body(uint32_t* __restrict__ out, 
         if (hi[d] > (int32_t)P.out_dims[d] - 1) hi[d] = (int32_t)P.out_dims[d] - 1;
     }
     if constexpr (VEC == 4) { lo[3] = hi[3] = 0; }           // the last dimension is not windowed: handled per lane element
-    const bool want_max = P.op == RED_MAX;
+    const uint32_t w3 = VEC == 4 ? 1u : P.window[3];
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.0f;
@@ -441,51 +490,22 @@ __device__ __forceinline__ void select_scatter_body(uint32_t* __restrict__ out, 
     for (int32_t o1 = lo[1]; o1 <= hi[1]; ++o1)
     for (int32_t o2 = lo[2]; o2 <= hi[2]; ++o2)
     for (int32_t o3 = lo[3]; o3 <= hi[3]; ++o3) {
-        float sel[VEC];
-        bool  mine[VEC], have = false;
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) { sel[j] = 0.0f; mine[j] = false; }
-        const uint32_t w3 = VEC == 4 ? 1u : P.window[3];
-        for (uint32_t t0 = 0; t0 < P.window[0]; ++t0) {
-            const int32_t k0 = o0 * (int32_t)P.stride[0] - P.pad_low[0] + (int32_t)t0;
-            if (k0 < 0 || k0 >= (int32_t)P.in_dims[0]) continue;
-            for (uint32_t t1 = 0; t1 < P.window[1]; ++t1) {
-                const int32_t k1 = o1 * (int32_t)P.stride[1] - P.pad_low[1] + (int32_t)t1;
-                if (k1 < 0 || k1 >= (int32_t)P.in_dims[1]) continue;
-                for (uint32_t t2 = 0; t2 < P.window[2]; ++t2) {
-                    const int32_t k2 = o2 * (int32_t)P.stride[2] - P.pad_low[2] + (int32_t)t2;
-                    if (k2 < 0 || k2 >= (int32_t)P.in_dims[2]) continue;
-                    for (uint32_t t3 = 0; t3 < w3; ++t3) {
-                        const int32_t k3 = VEC == 4 ? c[3] : o3 * (int32_t)P.stride[3] - P.pad_low[3] + (int32_t)t3;
-                        if (k3 < 0 || k3 >= (int32_t)P.in_dims[3]) continue;
-                        const uint64_t off = (((uint64_t)k0 * P.in_dims[1] + k1) * P.in_dims[2] + k2) * P.in_dims[3] + k3;
-                        const bool me = k0 == c[0] && k1 == c[1] && k2 == c[2] && (VEC == 4 || k3 == c[3]);
-                        float v[VEC];
-                        if constexpr (VEC == 4) {
-                            const u32x4 q = *reinterpret_cast<const u32x4*>(operand + off);
-                            v[0] = u2f(q.x); v[1] = u2f(q.y); v[2] = u2f(q.z); v[3] = u2f(q.w);
-                        } else {
-                            v[0] = u2f(operand[off]);
-                        }
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) {
-                            const bool keep = have && (want_max ? sel[j] >= v[j] : sel[j] <= v[j]);
-                            if (!keep) { sel[j] = v[j]; mine[j] = me; }
-                        }
-                        have = true;
-                    }
-                }
-            }
-        }
-        const uint64_t soff = (((uint64_t)o0 * P.out_dims[1] + o1) * P.out_dims[2] + o2) * P.out_dims[3] + (VEC == 4 ? c[3] : o3);
+        // this element's tap number inside the window
+        const uint32_t t0 = (uint32_t)(c[0] + P.pad_low[0] - o0 * (int32_t)P.stride[0]);
+        const uint32_t t1 = (uint32_t)(c[1] + P.pad_low[1] - o1 * (int32_t)P.stride[1]);
+        const uint32_t t2 = (uint32_t)(c[2] + P.pad_low[2] - o2 * (int32_t)P.stride[2]);
+        const uint32_t t3 = VEC == 4 ? 0u : (uint32_t)(c[3] + P.pad_low[3] - o3 * (int32_t)P.stride[3]);
+        const uint32_t tap = ((t0 * P.window[1] + t1) * P.window[2] + t2) * w3 + t3;
+        const uint64_t woff = (((uint64_t)o0 * P.out_dims[1] + o1) * P.out_dims[2] + o2) * P.out_dims[3] + (VEC == 4 ? c[3] : o3);
         if constexpr (VEC == 4) {
-            const u32x4 g = *reinterpret_cast<const u32x4*>(source + soff);
-            if (mine[0]) acc[0] += u2f(g.x);
-            if (mine[1]) acc[1] += u2f(g.y);
-            if (mine[2]) acc[2] += u2f(g.z);
-            if (mine[3]) acc[3] += u2f(g.w);
+            const u32x4 s = *reinterpret_cast<const u32x4*>(selected + woff);
+            const u32x4 g = *reinterpret_cast<const u32x4*>(source + woff);
+            if (s.x == tap) acc[0] += u2f(g.x);
+            if (s.y == tap) acc[1] += u2f(g.y);
+            if (s.z == tap) acc[2] += u2f(g.z);
+            if (s.w == tap) acc[3] += u2f(g.w);
         } else {
-            if (mine[0]) acc[0] += u2f(source[soff]);
+            if (selected[woff] == tap) acc[0] += u2f(source[woff]);
         }
     }
     if constexpr (VEC == 4) {
@@ -496,11 +516,17 @@ __device__ __forceinline__ void select_scatter_body(uint32_t* __restrict__ out, 
     }
 }
 
-extern "C" __global__ __launch_bounds__(256) void select_scatter_add_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
-                                                                        const uint32_t* __restrict__ operand, PoolParams P) {
-    select_scatter_body<1>(out, source, operand, P);
+extern "C" __global__ __launch_bounds__(256) void select_window_v1(uint32_t* __restrict__ sel, const uint32_t* __restrict__ operand, PoolParams P) {
+    select_window_body<1>(sel, operand, P);
 }
-extern "C" __global__ __launch_bounds__(256) void select_scatter_add_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
-                                                                        const uint32_t* __restrict__ operand, PoolParams P) {
-    select_scatter_body<4>(out, source, operand, P);
+extern "C" __global__ __launch_bounds__(256) void select_window_v4(uint32_t* __restrict__ sel, const uint32_t* __restrict__ operand, PoolParams P) {
+    select_window_body<4>(sel, operand, P);
+}
+extern "C" __global__ __launch_bounds__(256) void scatter_selected_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                                      const uint32_t* __restrict__ selected, PoolParams P) {
+    scatter_selected_body<1>(out, source, selected, P);
+}
+extern "C" __global__ __launch_bounds__(256) void scatter_selected_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                                      const uint32_t* __restrict__ selected, PoolParams P) {
+    scatter_selected_body<4>(out, source, selected, P);
 }

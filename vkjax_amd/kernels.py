@@ -587,8 +587,9 @@ def pool(out: Buffer, inp: Buffer, op: str, window, strides, pad_low, dilation) 
                   bytes_moved=4 * (inp.size + out.size))
 
 
-def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, op: str, window, strides, pad_low) -> Launch:
-    '''Gradient of a max (`op` = 'reduce_max': select with ge) or min pooling; see select_scatter_body in reduce.hip.'''
+def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, selected: Buffer, op: str, window, strides, pad_low) -> tp.List[Launch]:
+    '''Gradient of a max (`op` = 'reduce_max': select with ge) or min pooling in two launches: the selected tap
+    of every window into `selected` (uint32, source's shape), then the per-element sums; see reduce.hip.'''
     rank = len(operand.shape)
     if rank > 4:
         raise NotImplementedError('select_and_scatter_add over more than 4 dimensions')
@@ -598,14 +599,18 @@ def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, op: str, wi
     window   = [1] * lead + list(window)
     strides  = [1] * lead + list(strides)
     pad_low  = [0] * lead + list(pad_low)
-    n   = operand.size
     vec = 4 if (window[3] == 1 and strides[3] == 1 and pad_low[3] == 0 and in_dims[3] % 4 == 0
                 and in_dims[3] == out_dims[3]) else 1
     if max(in_dims) >= 2**31 or any(abs(p) >= 2**30 for p in pad_low):
         raise NotImplementedError('select_and_scatter_add: dimension too large')
-    params = _u32(n, RED[op], _RTYPE[operand.dtype], *in_dims, *out_dims, *window, *strides, 1, 1, 1, 1) + _i32(*pad_low)
-    return Launch(f'select_scatter_add_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
-                  [(out, 0), (source, 0), (operand, 0)], params, bytes_moved=4 * (2 * operand.size + source.size))
+    assert tuple(selected.shape) == tuple(source.shape) and selected.dtype == np.uint32
+    tail = _u32(RED[op], _RTYPE[operand.dtype], *in_dims, *out_dims, *window, *strides, 1, 1, 1, 1) + _i32(*pad_low)
+    n_win, n = source.size, operand.size
+    first  = Launch(f'select_window_v{vec}', (_cdiv(_cdiv(n_win, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                    [(selected, 0), (operand, 0)], _u32(n_win) + tail, bytes_moved=4 * (operand.size + source.size))
+    second = Launch(f'scatter_selected_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+                    [(out, 0), (source, 0), (selected, 0)], _u32(n) + tail, bytes_moved=4 * (operand.size + 2 * source.size))
+    return [first, second]
 
 
 PAD_MAX_RANK = 6

@@ -109,3 +109,13 @@ def uniform(key, shape=(), dtype=np.float32, minval=0.0, maxval=1.0):
     floats = lax.sub(lax.bitcast_convert_type(fbits, np.float32), np.float32(1.0))
     scaled = lax.add(lax.mul(floats, np.float32(maxval - minval)), np.float32(minval))
     return lax.max(np.float32(minval), mnp.reshape(scaled, shape))
+
+
+def normal(key, shape=(), dtype=np.float32):
+    '''Standard normal samples the way jax.random.normal draws them: uniform on (-1, 1), then
+    sqrt(2) * erf_inv.'''
+    if np.dtype(dtype) != np.float32:
+        raise NotImplementedError('normal: float32 only')
+    lo = np.nextafter(np.float32(-1.0), np.float32(0.0))
+    u  = uniform(key, shape, dtype, minval=lo, maxval=1.0)
+    return lax.mul(np.float32(np.sqrt(2)), lax.erf_inv(u))

@@ -527,7 +527,8 @@ def dot_general(bufferpool, equation):
                           xs=(0, lst[1 - lc[0]], 0, lst[lc[0]]),
                           ws=(rst[rc[0]] * Kc, rst[rc[0]] * Kc, rst[rc[0]], rst[1 - rc[0]]),
                           os=(M * N, N, N, 1))
-    return [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+    ops, rhs, geom = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
+    return ops + [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
 
 
 def conv_general_dilated(bufferpool, equation):
@@ -563,7 +564,24 @@ def conv_general_dilated(bufferpool, equation):
     wg = _as_kernel_gradient(geom)
     if wg is not None:
         return _wgrad_ops(bufferpool, equation, outbuf, lhs, rhs, wg)
-    return [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+    ops, rhs, geom = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
+    return ops + [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+
+
+def _with_dense_kernel(bufferpool, equation, rhs: Buffer, geom: 'K.ConvGeometry', lhs: Buffer, outbuf: Buffer):
+    '''A kernel operand that is not laid out [ky, kx, in, out] with `out` contiguous (the swapped and reversed
+    kernel of an input gradient, a transposed weight matrix) is copied into that layout first when it is no
+    bigger than the activations: the GEMM kernel then reads it with 16-byte loads. Returns (ops, rhs, geometry).'''
+    N, dense = geom.N, (geom.KW * geom.Cin * geom.N, geom.Cin * geom.N, geom.N, 1)
+    if geom.ws == dense or N % 4 != 0 or geom.M < 256 or rhs.size > lhs.size + outbuf.size or builtins_min(geom.ws) < 0:
+        return [], rhs, geom
+    position = bufferpool.op_counter
+    bufferpool.op_counter -= 1                  #the copy lives at the equation's own position
+    shape = (geom.KH, geom.KW, geom.Cin, N)
+    copy  = bufferpool.new_temporary(np.float32, shape)
+    bufferpool.op_counter = position
+    op = Op(equation, chain=EwChain(copy, shape, EwOperand(rhs, 0, tuple(geom.ws)), []))
+    return [op], copy, geom._replace(ws=dense)
 
 
 def _as_kernel_gradient(g: 'K.ConvGeometry') -> tp.Optional['K.WgradGeometry']:
@@ -675,8 +693,13 @@ def select_and_scatter_add(bufferpool, equation):
     if outbuf.size == 0:
         return []
     pad_low = [int(lo) for lo, _ in params['padding']]
-    return [Op(equation, launch=K.select_scatter_add(outbuf, source, operand, 'reduce_max' if select == 'ge' else 'reduce_min',
-                                                     params['window_dimensions'], params['window_strides'], pad_low))]
+    position = bufferpool.op_counter
+    bufferpool.op_counter -= 1                  #the temporary lives at the equation's own position
+    selected = bufferpool.new_temporary(np.uint32, source.shape)
+    bufferpool.op_counter = position
+    launches = K.select_scatter_add(outbuf, source, operand, selected, 'reduce_max' if select == 'ge' else 'reduce_min',
+                                    params['window_dimensions'], params['window_strides'], pad_low)
+    return [Op(equation, launch=l) for l in launches]
 
 
 def pad(bufferpool, equation):
@@ -875,3 +898,4 @@ def random_seed(bufferpool, equation):
 
 import builtins as _builtins
 builtins_max = _builtins.max
+builtins_min = _builtins.min
