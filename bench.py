@@ -29,8 +29,8 @@ PEAK_HBM_GBS          = 8000.0
 
 UNITS = {'resnet50': ('images/sec', 'batch'), 'mlp': ('samples/sec', 'batch'), 'conv_block': ('images/sec', 'batch'),
          'affine': ('calls/sec', None), 'rng_uniform': ('Gsamples/sec', None), 'gather_scatter': ('Grows/sec', None),
-         'mlp_train': ('samples/sec', 'batch'), 'convnet_train': ('images/sec', 'batch')}
-BATCHED = ('resnet50', 'mlp', 'conv_block', 'mlp_train', 'convnet_train')
+         'mlp_train': ('samples/sec', 'batch'), 'convnet_train': ('images/sec', 'batch'), 'resnet50_train': ('images/sec', 'batch')}
+BATCHED = ('resnet50', 'mlp', 'conv_block', 'mlp_train', 'convnet_train', 'resnet50_train')
 
 
 def kernel_family(name: str) -> str:
@@ -220,6 +220,9 @@ def time_cpu_baseline(workload, fn, make_inputs, kwargs):
     if workload == 'resnet50':
         sample_kwargs['batch'] = 4
         sample = 'batch 4 of the same 224x224x3 ResNet-50 forward'
+    if workload == 'resnet50_train':
+        sample_kwargs['batch'] = 1
+        sample = 'batch 1 of the same training step'
     if workload == 'convnet_train':
         sample_kwargs['batch'] = 1
         sample = 'batch 1 of the same training step (the pooling gradient of the oracle is a python loop)'

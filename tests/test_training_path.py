@@ -49,6 +49,10 @@ def small_convnet_inputs():
     return W.convnet_train_inputs(batch=3, size=16, channels=(3, 8, 12), classes=5)
 
 
+def tiny_resnet_inputs():
+    return W.resnet50_train_inputs(batch=2, size=32, num_classes=10, width_scale=0.125)
+
+
 def small_mlp_inputs():
     return W.mlp_train_inputs(batch=16, sizes=(40, 32, 24, 5))
 
@@ -281,15 +285,18 @@ def test_rows_contracted_dot_hip():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('name,make_inputs', [('mlp_train', small_mlp_inputs), ('convnet_train', small_convnet_inputs)])
+@pytest.mark.parametrize('name,make_inputs', [('mlp_train', small_mlp_inputs), ('convnet_train', small_convnet_inputs),
+                                              ('resnet50_train', tiny_resnet_inputs)])
 def test_training_step_hip_matches_oracle(name, make_inputs):
     '''One SGD step: loss and every updated parameter against the oracle (reference tests/test_elegy_mlp.py:87-129
     compares exactly these after train_on_batch, rtol 1e-5 / atol 1e-6 there; contractions here use the tolerance
     of dot / conv).'''
     print(f'case: {name}', flush=True)
     fn, _ = W.WORKLOADS[name]
+    #the 53-layer network accumulates the rounding differences of its contractions: the tolerance of its logits
+    rtol, atol = (1e-3, 1e-5) if name == 'resnet50_train' else (1e-4, 1e-6)
     for fuse in (True, False):
-        check_against_oracle(fn, make_inputs(), rtol=1e-4, atol=1e-6, fuse=fuse)
+        check_against_oracle(fn, make_inputs(), rtol=rtol, atol=atol, fuse=fuse)
 
 
 @pytest.mark.gpu

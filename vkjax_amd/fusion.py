@@ -133,9 +133,45 @@ def fuse_ops(all_ops, bufferpool, outvars):
         for b in _reads(op):
             b.accesses.append(index)
 
+    def fold_copies(op):
+        '''An operand that is the full-size result of a pure copy (a broadcast, slice, transpose or reversal
+        that was given a launch of its own) is read through that copy's strides instead; the copy goes away
+        once nothing reads its result any more.'''
+        chain, changed = op.chain, False
+        first, steps = chain.first, list(chain.steps)
+        for k, o in enumerate(chain.operands()):
+            if o is None:
+                continue
+            pid = id(o.buffer._placeholder)
+            pos = producer.get(pid)
+            prod = result[pos] if pos is not None else None
+            if (prod is None or prod.chain is None or prod.chain.steps or tuple(prod.chain.shape) != tuple(chain.shape)
+                    or not _is_full_contiguous(o, chain.shape)):
+                continue
+            source = prod.chain.first
+            if k == 0:
+                first = source
+            else:
+                steps[k - 1] = steps[k - 1]._replace(operand=source)
+            changed = True
+            uses[pid] -= 1
+            uses[id(source.buffer._placeholder)] += 1
+            source.buffer.accesses.append(op.index)
+            if uses[pid] == 0:
+                uses[id(source.buffer._placeholder)] -= 1
+                _out(prod)._placeholder.elided = True
+                result[pos] = None
+                del producer[pid]
+        if changed:
+            new = Op(op.equation, chain=EwChain(chain.out, chain.shape, first, steps))
+            new.index = op.index
+            return new
+        return op
+
     for op in all_ops:
         fused = None
         if op.chain is not None:
+            op = fold_copies(op)
             for cand in [o for o in op.chain.operands()[:2] if o is not None]:
                 pid = id(cand.buffer._placeholder)
                 pos = producer.get(pid)

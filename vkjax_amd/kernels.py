@@ -425,7 +425,7 @@ def _magic_division(d: int) -> tp.Tuple[int, int]:
 
 
 def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: tp.Sequence[ConvEpilogueStep] = (),
-              compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0) -> Launch:
+              compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0, out_offset: int = 0) -> Launch:
     if len(epilogue) > CONV_MAX_EPI:
         raise ValueError('too many epilogue steps')
     g = _flatten_pointwise(g)
@@ -467,7 +467,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
         descs[i // 3] |= ((e.op * 2 + int(e.operand_left)) | e.kind << 8) << (10 * (i % 3))
     params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW,
                    *g.xs[:3], tiles_m, tiles_n)
-              + _u32(flags, *descs, x_bytes, w_bytes, out.size * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
+              + _u32(flags, *descs, x_bytes, w_bytes, (out.size - out_offset) * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
               + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os))
     derived_ptrs, derived_desc = [(None, 0)] * (CONV_MAX_DERIVED + 1), _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
     for i, e in enumerate(epilogue):
@@ -481,7 +481,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
             derived_desc = _u32(i, len(d.steps), mask, *_pad([st[0] for st in d.steps], CONV_MAX_DERIVED),
                                 *_pad([int(st[2]) for st in d.steps], CONV_MAX_DERIVED))
     params += derived_desc
-    buffers = [(out, 0), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
+    buffers = [(out, out_offset * 4), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
     buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0)) + derived_ptrs
     kernel  = f'conv_gemm_{tag}x{bk}_' + ('lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)

@@ -27,8 +27,13 @@ def _shape(x):
     return tuple(x.shape) if isinstance(x, Tracer) else tuple(np.shape(x))
 
 
+def _full(shape, value):
+    '''A constant array as jax's rules make it: a broadcast of a scalar literal (no storage of its own).'''
+    return lax.broadcast_in_dim(np.float32(value), tuple(shape), ()) if tuple(shape) else np.float32(value)
+
+
 def _zeros_like(x):
-    return np.zeros(_shape(x), np.float32)
+    return _full(_shape(x), 0.0)
 
 
 def _sum_to_shape(g, shape):
@@ -43,7 +48,7 @@ def _sum_to_shape(g, shape):
 
 
 def _indicator(pred, yes, no, shape):
-    return lax.select(pred, np.full(shape, yes, np.float32), np.full(shape, no, np.float32))
+    return lax.select(pred, _full(shape, yes), _full(shape, no))
 
 
 # ---------------------------------------------------------------- rules: (cotangent(s) of the result, operands, result, params) -> operand cotangents
@@ -130,7 +135,7 @@ def _logistic(g, x, out):
 def _integer_pow(g, x, out, y):
     if y == 0:
         return (None,)
-    return (lax.mul(g, lax.mul(np.float32(y), lax.integer_pow(x, y - 1) if y != 1 else np.ones(_shape(x), np.float32))),)
+    return (lax.mul(g, lax.mul(np.float32(y), lax.integer_pow(x, y - 1) if y != 1 else _full(_shape(x), 1.0))),)
 
 
 @_rule('square')

@@ -527,7 +527,7 @@ def dot_general(bufferpool, equation):
                           xs=(0, lst[1 - lc[0]], 0, lst[lc[0]]),
                           ws=(rst[rc[0]] * Kc, rst[rc[0]] * Kc, rst[rc[0]], rst[1 - rc[0]]),
                           os=(M * N, N, N, 1))
-    ops, rhs, geom = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
+    ops, rhs, geom, _ = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
     return ops + [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
 
 
@@ -564,24 +564,61 @@ def conv_general_dilated(bufferpool, equation):
     wg = _as_kernel_gradient(geom)
     if wg is not None:
         return _wgrad_ops(bufferpool, equation, outbuf, lhs, rhs, wg)
-    ops, rhs, geom = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
+    if (geom.LH > 1 or geom.LW > 1) and geom.SH == geom.SW == 1 and geom.DH == geom.DW == 1:
+        return _dilated_input_convolution(bufferpool, equation, outbuf, lhs, rhs, geom)
+    ops, rhs, geom, _ = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
     return ops + [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
 
 
-def _with_dense_kernel(bufferpool, equation, rhs: Buffer, geom: 'K.ConvGeometry', lhs: Buffer, outbuf: Buffer):
+def _with_dense_kernel(bufferpool, equation, rhs: Buffer, geom: 'K.ConvGeometry', lhs: Buffer, outbuf: Buffer, rhs_offset: int = 0):
     '''A kernel operand that is not laid out [ky, kx, in, out] with `out` contiguous (the swapped and reversed
-    kernel of an input gradient, a transposed weight matrix) is copied into that layout first when it is no
-    bigger than the activations: the GEMM kernel then reads it with 16-byte loads. Returns (ops, rhs, geometry).'''
+    kernel of an input gradient, a transposed weight matrix, every other tap of a kernel) is copied into that
+    layout first when it is no bigger than the activations: the GEMM kernel then reads it with 16-byte loads.
+    Returns (ops, rhs, geometry, rhs offset).'''
     N, dense = geom.N, (geom.KW * geom.Cin * geom.N, geom.Cin * geom.N, geom.N, 1)
-    if geom.ws == dense or N % 4 != 0 or geom.M < 256 or rhs.size > lhs.size + outbuf.size or builtins_min(geom.ws) < 0:
-        return [], rhs, geom
+    if ((geom.ws == dense and rhs_offset % 4 == 0) or N % 4 != 0 or geom.M < 256 or geom.K * N > lhs.size + outbuf.size
+            or builtins_min(geom.ws) < 0):
+        return [], rhs, geom, rhs_offset
     position = bufferpool.op_counter
     bufferpool.op_counter -= 1                  #the copy lives at the equation's own position
     shape = (geom.KH, geom.KW, geom.Cin, N)
     copy  = bufferpool.new_temporary(np.float32, shape)
     bufferpool.op_counter = position
-    op = Op(equation, chain=EwChain(copy, shape, EwOperand(rhs, 0, tuple(geom.ws)), []))
-    return [op], copy, geom._replace(ws=dense)
+    op = Op(equation, chain=EwChain(copy, shape, EwOperand(rhs, rhs_offset, tuple(geom.ws)), []))
+    return [op], copy, geom._replace(ws=dense), 0
+
+
+def _dilated_input_convolution(bufferpool, equation, outbuf: Buffer, lhs: Buffer, rhs: Buffer, g: 'K.ConvGeometry'):
+    '''A convolution over an lhs-dilated input (the input gradient of a strided convolution) touches a real
+    input element only at every LH-th (LW-th) position, and which kernel taps meet real elements depends only
+    on the output position modulo the dilation. So it is computed as LH * LW ordinary convolutions, one per
+    residue class of output positions, each with the kernel taps of its class and writing every LH-th
+    (LW-th) output position; classes that meet no tap are zero. The multiplications with the inserted zeros,
+    (1 - 1 / (LH * LW)) of the total, are never issued.'''
+    def classes(L, P, taps, out_size):
+        result = []
+        for a in range(builtins_min(L, out_size)):
+            r0 = (P - a) % L
+            n  = len(range(r0, taps, L))
+            result.append((a, r0, n, (a + r0 - P) // L, -(-(out_size - a) // L)))     #class, first tap, taps, input shift, positions
+        return result
+    ops, launches = [], []
+    rows, cols = classes(g.LH, g.PH, g.KH, g.Ho), classes(g.LW, g.PW, g.KW, g.Wo)
+    if any(n == 0 for _, _, n, _, _ in rows + cols):
+        ops.append(Op(equation, launch=K.fill(outbuf, 0)))
+    for ah, rh, nh, ch, th in rows:
+        for aw, rw, nw, cw, tw in cols:
+            if nh == 0 or nw == 0:
+                continue
+            sub = g._replace(Ho=th, Wo=tw, KH=nh, KW=nw, PH=-ch, PW=-cw, LH=1, LW=1,
+                             ws=(g.ws[0] * g.LH, g.ws[1] * g.LW, g.ws[2], g.ws[3]),
+                             os=(g.os[0], g.os[1] * g.LH, g.os[2] * g.LW, g.os[3]))
+            copies, kernel, sub, kernel_offset = _with_dense_kernel(bufferpool, equation, rhs, sub, lhs, outbuf,
+                                                                    rh * g.ws[0] + rw * g.ws[1])
+            ops += copies
+            ops.append(Op(equation, launch=K.conv_gemm(outbuf, lhs, kernel, sub, rhs_offset=kernel_offset,
+                                                       out_offset=ah * g.os[1] + aw * g.os[2])))
+    return ops
 
 
 def _as_kernel_gradient(g: 'K.ConvGeometry') -> tp.Optional['K.WgradGeometry']:

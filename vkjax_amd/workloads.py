@@ -234,6 +234,25 @@ def convnet_train_inputs(seed=7, batch=64, size=64, channels=(3, 64, 128), class
     return [params, x, onehot]
 
 
+def resnet50_loss(params, x, onehot):
+    logits, _ = resnet50(params, x)
+    return softmax_cross_entropy(logits, onehot)
+
+
+def resnet50_train_step(params, x, onehot, lr=0.01):
+    '''One SGD step of ResNet-50 with its batch-norm layers in inference mode (fixed statistics): gradients
+    of every convolution kernel, scale, shift and of the dense layer.'''
+    loss, grads = mj.value_and_grad(resnet50_loss)(params, x, onehot)
+    return loss, _sgd(params, grads, lr)
+
+
+def resnet50_train_inputs(seed=4, batch=64, size=224, num_classes=1000, width_scale=1.0):
+    params, x = resnet50_inputs(seed, batch, size, num_classes, width_scale)
+    rng = np.random.default_rng(seed + 2000)
+    onehot = np.eye(num_classes, dtype=np.float32)[rng.integers(0, num_classes, size=batch)]
+    return [params, x, onehot]
+
+
 WORKLOADS: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable]] = {
     'affine':         (affine, affine_inputs),
     'mlp':            (mlp, mlp_inputs),
@@ -243,4 +262,5 @@ WORKLOADS: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable]] = {
     'gather_scatter': (gather_scatter, gather_scatter_inputs),
     'mlp_train':      (mlp_train_step, mlp_train_inputs),
     'convnet_train':  (convnet_train_step, convnet_train_inputs),
+    'resnet50_train': (resnet50_train_step, resnet50_train_inputs),
 }
