@@ -34,7 +34,7 @@ BATCHED = ('resnet50', 'mlp', 'conv_block', 'mlp_train', 'convnet_train', 'resne
 
 
 def kernel_family(name: str) -> str:
-    for prefix in ('conv_gemm', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows',
+    for prefix in ('conv_gemm', 'wgrad_gemm', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows',
                    'select_window', 'scatter_selected', 'pad_nd'):
         if name.startswith(prefix):
             return prefix
@@ -203,7 +203,9 @@ def measured_hbm_traffic(workload, family):
     Counters cannot be collected from inside this process.'''
     import glob, re
     here = os.path.dirname(os.path.abspath(__file__))
-    for path in sorted(glob.glob(os.path.join(here, 'profiles', f'*{workload}*.txt'))):
+    #summaries are named <kernels>_<workload>.txt (the headline one: <kernels>_resnet50_bs64.txt)
+    paths = glob.glob(os.path.join(here, 'profiles', f'*_{workload}.txt')) + glob.glob(os.path.join(here, 'profiles', f'*_{workload}_bs64.txt'))
+    for path in sorted(paths):
         m = re.search(rf'^hbm_traffic_bytes_per_launch {re.escape(family)} (\d+)', open(path).read(), re.M)
         if m:
             return int(m.group(1))
