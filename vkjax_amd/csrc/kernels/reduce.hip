@@ -144,8 +144,15 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
     if (lane == 0) out[unit] = is_arg ? (best_i == 0xFFFFFFFFu ? 0u : best_i) : a;
 }
 
-template <int VEC, int MODE>
-__device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P) {
+// PRO: what is reduced. 0 the operand itself; 1 its product with a second array of the same shape;
+// 2 its product with a vector over `inner`; 3 its negation (float). The element-wise producer of a
+// reduction's operand (the `g * x` and `-g` of a batch-norm backward pass) is applied while loading,
+// with the same roundings as a separate pass, so that array never exists.
+enum { PRO_NONE = 0, PRO_MUL = 1, PRO_MULV = 2, PRO_NEG = 3 };
+
+template <int VEC, int MODE, int PRO = PRO_NONE>
+__device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P,
+                                                 const uint32_t* __restrict__ in2 = nullptr) {
     __shared__ uint32_t s_val[256 * VEC];
     __shared__ uint32_t s_idx[256 * VEC];
     const uint32_t TI = P.TI, TR = 256u / TI;
@@ -174,31 +181,44 @@ __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, con
         }
     };
     if (i < P.inner) {                                                // inner is a multiple of VEC
-        const uint32_t* p = in + (uint64_t)o * P.R * P.inner + i;
+        const uint32_t* p  = in + (uint64_t)o * P.R * P.inner + i;
+        const uint32_t* p2 = PRO == PRO_MUL ? in2 + (uint64_t)o * P.R * P.inner + i : nullptr;
+        uint32_t w[VEC];                                              // PRO_MULV: this thread's part of the vector
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) w[j] = PRO == PRO_MULV ? in2[i + j] : 0u;
+        auto fetch = [&](uint32_t row, uint32_t (&v)[VEC]) {
+            const uint64_t off = (uint64_t)row * P.inner;
+            uint32_t b[VEC];
+            if constexpr (VEC == 4) {
+                const u32x4 t = *reinterpret_cast<const u32x4*>(p + off);
+                v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+                if constexpr (PRO == PRO_MUL) { const u32x4 u = *reinterpret_cast<const u32x4*>(p2 + off); b[0] = u.x; b[1] = u.y; b[2] = u.z; b[3] = u.w; }
+            } else {
+                v[0] = p[off];
+                if constexpr (PRO == PRO_MUL) b[0] = p2[off];
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                if constexpr (PRO == PRO_MUL)  v[j] = f2u(u2f(v[j]) * u2f(b[j]));
+                if constexpr (PRO == PRO_MULV) v[j] = f2u(u2f(v[j]) * u2f(w[j]));
+                if constexpr (PRO == PRO_NEG)  v[j] ^= 0x80000000u;
+            }
+        };
         uint32_t r = r_lo + tr;
         for (; r + 3u * TR < r_hi; r += 4u * TR) {                    // four loads in flight per thread
             uint32_t v[4][VEC];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                if constexpr (VEC == 4) {
-                    const u32x4 t = *reinterpret_cast<const u32x4*>(p + (uint64_t)(r + q * TR) * P.inner);
-                    v[q][0] = t.x; v[q][1] = t.y; v[q][2] = t.z; v[q][3] = t.w;
-                } else {
-                    v[q][0] = p[(uint64_t)(r + q * TR) * P.inner];
-                }
-            }
+            for (int q = 0; q < 4; ++q) fetch(r + q * TR, v[q]);
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) take(v[q][j], r + q * TR, j);
         }
         for (; r < r_hi; r += TR) {
-            if constexpr (VEC == 4) {
-                const u32x4 t = *reinterpret_cast<const u32x4*>(p + (uint64_t)r * P.inner);
-                take(t.x, r, 0); take(t.y, r, 1); take(t.z, r, 2); take(t.w, r, 3);
-            } else {
-                take(p[(uint64_t)r * P.inner], r, 0);
-            }
+            uint32_t v[VEC];
+            fetch(r, v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) take(v[j], r, j);
         }
     }
 #pragma unroll
@@ -233,7 +253,13 @@ __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, con
     extern "C" __global__ __launch_bounds__(256) void reduce_rows_##tag##_v4(uint32_t* out, const uint32_t* in, ReduceParams P) { reduce_rows_body<4, MODE>(out, in, P); } \
     extern "C" __global__ __launch_bounds__(256) void reduce_cols_##tag##_v1(uint32_t* out, const uint32_t* in, ReduceParams P) { reduce_cols_body<1, MODE>(out, in, P); } \
     extern "C" __global__ __launch_bounds__(256) void reduce_cols_##tag##_v4(uint32_t* out, const uint32_t* in, ReduceParams P) { reduce_cols_body<4, MODE>(out, in, P); }
+#define REDUCE_COLS_PROLOGUE_KERNELS(tag, PRO)                                                                                 \
+    extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v1(uint32_t* out, const uint32_t* in, const uint32_t* in2, ReduceParams P) { reduce_cols_body<1, 0, PRO>(out, in, P, in2); } \
+    extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v4(uint32_t* out, const uint32_t* in, const uint32_t* in2, ReduceParams P) { reduce_cols_body<4, 0, PRO>(out, in, P, in2); }
 // the _v4 variants need R % 4 == 0, r_chunk % 4 == 0 (rows) or inner % 4 == 0 (cols) and 16-byte aligned pointers
+REDUCE_COLS_PROLOGUE_KERNELS(mul, PRO_MUL)
+REDUCE_COLS_PROLOGUE_KERNELS(mulv, PRO_MULV)
+REDUCE_COLS_PROLOGUE_KERNELS(neg, PRO_NEG)
 REDUCE_KERNELS(fsum, 0)
 REDUCE_KERNELS(fmax, 1)
 REDUCE_KERNELS(any, 2)

@@ -207,8 +207,65 @@ def fuse_ops(all_ops, bufferpool, outvars):
             producer[id(out._placeholder)] = len(result) - 1
     ops = fuse_random_streams([op for op in result if op is not None], bufferpool, outvars)
     ops = fuse_stream_chains(ops, bufferpool, outvars)
+    ops = fuse_reduce_prologues(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
     return remove_dead_ops(ops, bufferpool, outvars)
+
+
+def fuse_reduce_prologues(ops, bufferpool, outvars):
+    '''A float column sum whose operand is, and is only, the result of `a * b` (b of the same shape or a
+    vector over the columns) or of `-a` reads a (and b) itself and applies the step while loading: the
+    pairs `multiply -> reduce_sum` and `negate -> reduce_sum` of a batch-norm backward pass lose a full-size
+    array each. Values are unchanged (same products, same order of additions).'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    chain_writer = {pid(op.chain.out): i for i, op in enumerate(ops) if op.chain is not None}
+    removed, replacement = set(), {}
+    for i, R in enumerate(ops):
+        if R.meta is None or R.meta[0] != 'reduce':
+            continue
+        _, out, inp, outer, rows, inner, name, partial, nsplit = R.meta
+        w = chain_writer.get(pid(inp))
+        if name != 'reduce_sum' or inner <= 1 or inp.dtype != 'float32' or w is None or w > i or w in removed or uses[pid(inp)] != 1:
+            continue
+        ch = ops[w].chain
+        size = 1
+        for d in ch.shape:
+            size *= d
+        if size != outer * rows * inner or len(ch.steps) != 1 or not _is_full_contiguous_any_shape(ch.first, ch.shape):
+            continue
+        step, prologue = ch.steps[0], None
+        if step.op == EW['NEG_F'] and step.operand is None:
+            prologue = ('neg', None)
+        elif step.op == EW['MUL_F'] and step.operand is not None:
+            o = step.operand
+            if _is_full_contiguous_any_shape(o, ch.shape):
+                prologue = ('mul', o.buffer)
+            elif (o.offset == 0 and o.buffer.size == inner and ch.shape[-1] == inner
+                  and tuple(o.strides) == (0,) * (len(ch.shape) - 1) + (1,)):
+                prologue = ('mulv', o.buffer)
+        if prologue is None:
+            continue
+        source = ch.first.buffer
+        launch = K.reduce(out, source, outer, rows, inner, name, partial, nsplit, prologue=prologue)[0]
+        fused  = Op(_label(ops[w], R), launch=launch, meta=None)
+        fused.index = R.index
+        for b in (source, prologue[1]):
+            if b is not None:
+                b.accesses.append(R.index)
+        ch.out._placeholder.elided = True
+        removed.add(w)
+        replacement[i] = fused
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
+
+
+def _is_full_contiguous_any_shape(operand: EwOperand, shape) -> bool:
+    '''The operand covers `shape` densely in row-major order (its buffer may carry another shape of the same size).'''
+    size = 1
+    for d in shape:
+        size *= d
+    return operand.offset == 0 and operand.buffer.size == size and tuple(operand.strides) == K.row_major_strides(shape)
 
 
 def fuse_stream_chains(ops, bufferpool, outvars):

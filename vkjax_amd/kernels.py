@@ -516,7 +516,8 @@ def plan_reduce_splits(outer: int, R: int, inner: int, op: str, compute_units: i
     return max(1, min(split, 65535))
 
 
-def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str, nsplit: int, in_offset_ok=True) -> Launch:
+def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str, nsplit: int, in_offset_ok=True,
+                   prologue: tp.Optional[tp.Tuple[str, tp.Optional[Buffer]]] = None) -> Launch:
     ty   = _RTYPE[inp.dtype]
     mode = {('reduce_sum', 0): 'fsum', ('reduce_max', 0): 'fmax', ('argmax', 0): 'fargmax', ('argmin', 0): 'fargmin'}.get((op, ty), 'any')
     r_chunk = _cdiv(_cdiv(R, nsplit), 4) * 4
@@ -532,19 +533,28 @@ def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op:
     blocks = _cdiv(inner, TI * vec) * nsplit * outer
     if blocks >= 2**31:
         raise NotImplementedError(f'reduction with {outer} outer rows and inner size {inner}')
+    if prologue is not None:
+        #the operand's element-wise producer applied while loading: ('mul', array of the same shape),
+        #('mulv', vector over inner) or ('neg', None); float column sums only
+        kind, second = prologue
+        assert mode == 'fsum' and kind in ('mul', 'mulv', 'neg') and (second is None) == (kind == 'neg')
+        assert second is None or second.size == (outer * R * inner if kind == 'mul' else inner)
+        extra = 0 if second is None else second.size
+        return Launch(f'reduce_cols_fsum_{kind}_v{vec}', (blocks, 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0), (second, 0)], params,
+                      bytes_moved=4 * (outer * R * inner + outer * nsplit * inner + extra)), nsplit
     return Launch(f'reduce_cols_{mode}_v{vec}', (blocks, 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
                   bytes_moved=4 * (outer * R * inner + outer * nsplit * inner)), nsplit
 
 
 def reduce(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str,
-           partial: tp.Optional[Buffer] = None, nsplit: int = 1) -> tp.List[Launch]:
+           partial: tp.Optional[Buffer] = None, nsplit: int = 1, prologue=None) -> tp.List[Launch]:
     '''[outer, R, inner] -> [outer, inner]. With nsplit > 1, `partial` (outer * nsplit * inner words) receives
-    the per-range results of a first launch and a second launch reduces them.'''
+    the per-range results of a first launch and a second launch reduces them. `prologue`: see _reduce_launch.'''
     if nsplit <= 1:
-        return [_reduce_launch(out, inp, outer, R, inner, op, 1)[0]]
-    first, nsplit = _reduce_launch(partial, inp, outer, R, inner, op, nsplit)
+        return [_reduce_launch(out, inp, outer, R, inner, op, 1, prologue=prologue)[0]]
+    first, nsplit = _reduce_launch(partial, inp, outer, R, inner, op, nsplit, prologue=prologue)
     if nsplit == 1:
-        return [_reduce_launch(out, inp, outer, R, inner, op, 1)[0]]
+        return [_reduce_launch(out, inp, outer, R, inner, op, 1, prologue=prologue)[0]]
     assert partial.size >= outer * nsplit * inner and partial.dtype == inp.dtype
     second = _reduce_launch(out, partial, outer, nsplit, inner, op, 1)[0]
     return [first, second]

@@ -679,7 +679,10 @@ def reduce_op(bufferpool, equation):
             bufferpool.op_counter -= 1
             partial = bufferpool.new_temporary(inbuf.dtype, (outer * nsplit * inner,))
             bufferpool.op_counter += 1
-        return [Op(equation, launch=l) for l in K.reduce(outbuf, inbuf, outer, R, inner, name, partial, nsplit)]
+        ops = [Op(equation, launch=l) for l in K.reduce(outbuf, inbuf, outer, R, inner, name, partial, nsplit)]
+        #the launch that reads the operand can take over the operand's element-wise producer (see fusion.py)
+        ops[0].meta = ('reduce', outbuf, inbuf, outer, R, inner, name, partial, nsplit)
+        return ops
     kept    = [(g[1], g[2]) for g in groups if not g[0]]
     reduced = [(g[1], g[2]) for g in groups if g[0]]
     return [Op(equation, launch=K.reduce_general(outbuf, inbuf, kept, reduced, name))]
