@@ -61,3 +61,23 @@ def test_float_sum_within_tolerance():
     check_against_oracle(lambda x: jnp.sum(x, axis=1), [x], rtol=1e-5, atol=0)
     x = rng.random_sample((1 << 18, 24)).astype(np.float32)
     check_against_oracle(lambda x: jnp.sum(x, axis=0), [x], rtol=1e-5, atol=0)
+
+
+def test_column_sums_take_over_their_operands_multiply_or_negate():
+    '''sum(a * b), sum(a * per-column vector), sum(-a) over the leading dimensions: one launch family
+    `reduce_cols_fsum_{mul,mulv,neg}` instead of an element-wise pass plus a reduction; same values as unfused.'''
+    import vkjax_amd
+    a, b, v = ints((6, 33, 17, 64)), ints((6, 33, 17, 64)), ints((64,))
+    cases = [('mul', lambda a, b, v: jnp.sum(a * b, axis=(0, 1, 2))), ('mulv', lambda a, b, v: jnp.sum(a * v, axis=(0, 1, 2))),
+             ('neg', lambda a, b, v: jnp.sum(-a, axis=(0, 1))), ('mul', lambda a, b, v: jnp.sum(a.reshape(-1, 64) * b.reshape(-1, 64), axis=0))]
+    for kind, f in cases:
+        print(f'prologue {kind}', flush=True)
+        y, _, fn = check_against_oracle(f, [a, b, v], exact=True)
+        kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+        assert kernels[0].startswith(f'reduce_cols_fsum_{kind}_v') and not any(k.startswith('ew_chain') for k in kernels), kernels
+    #random floats: bit-identical to the unfused program
+    x, y = rng.random_sample((5000, 96)).astype(np.float32), rng.random_sample((5000, 96)).astype(np.float32)
+    f = lambda x, y: jnp.sum(x * y, axis=0)
+    fused   = vkjax_amd.wrap(f, frontend='minijax')(x, y)
+    unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)(x, y)
+    assert np.array_equal(fused, unfused)
