@@ -274,6 +274,25 @@ def test_matrix_hip_interpreter(f, desc, args):
     check_against_oracle(f, args, rtol=rtol, atol=atol)
 
 
+def test_tiled_transposes():
+    '''Copies that swap the two fastest dimensions go through the LDS-tiled kernel: ragged sizes, batches,
+    NHWC <-> NCHW, a sliced source.'''
+    cases = [(lambda x: lax.transpose(x, (1, 0)), [random([1000, 77])]),
+             (lambda x: lax.transpose(x, (1, 0)), [random([64, 64])]),
+             (lambda x: lax.transpose(x, (1, 0)), [randint(-9, 9, size=[129, 2050])]),
+             (lambda x: lax.transpose(x, (0, 2, 1)), [random([5, 70, 33])]),
+             (lambda x: lax.transpose(x, (0, 3, 1, 2)), [random([3, 17, 19, 24])]),
+             (lambda x: lax.transpose(x, (0, 2, 3, 1)), [random([3, 24, 17, 19])]),
+             (lambda x: lax.transpose(x[3:, 5:70], (1, 0)), [random([40, 100])]),
+             (lambda x: lax.transpose(x, (1, 0)) * 2.0, [random([300, 200])])]
+    for k, (f, args) in enumerate(cases):
+        print(f'case: tiled transpose {k}', flush=True)
+        _, _, fn = check_against_oracle(f, args, exact=True)
+        kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+        if k != 7:
+            assert 'transpose_tiled' in kernels, kernels
+
+
 def test_nextafter_direction():
     '''reference: tests/test_basic_ops.py:367-382'''
     import vkjax_amd

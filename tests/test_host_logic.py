@@ -90,6 +90,7 @@ def test_kernel_argument_layouts_match_the_structs():
         'PoolParams': K.pool(b(1, 2, 2, 4), b(1, 4, 4, 4), 'reduce_max', (1, 2, 2, 1), (1, 2, 2, 1), (0, 0, 0, 0), (1, 1, 1, 1)),
         'WgradParams': K.wgrad_gemm(b(2, 9 * 4 * 8), b(2, 8, 8, 4), b(2, 8, 8, 8),
                                     K.WgradGeometry(images=2, Ho=8, Wo=8, H=8, W=8, C=4, KH=3, KW=3, N=8, PH=1, PW=1), 2),
+        'TransposeParams': K.lower_ew_chain(K.EwChain(b(40, 30), (40, 30), K.EwOperand(b(30, 40), 0, (1, 40)), [])),
         'PadParams': K.pad(b(6, 8), b(4, 8), b(), ((1, 1, 0), (0, 0, 0))),
         'GatherRowsParams': K.gather_rows(b(3, 8), b(4, 8), i(3, 1), 3, 8, 4),
         'GatherGeneralParams': K.gather_general(b(3, 8), b(4, 8), i(3, 1), (1,), (0,), (0,), (1, 8)),

@@ -288,3 +288,29 @@ extern "C" __global__ __launch_bounds__(256) void pad_nd_v4(uint32_t* __restrict
                                                             const uint32_t* __restrict__ value, PadParams P) {
     pad_body<4>(out, in, value, P);
 }
+
+// Copy that swaps the two fastest dimensions: out[b, i, j] = in[b * sb + j * sj + i], out dense
+// [B, I, J]. The strided gather of the element-wise kernel touches a new cache line per element on
+// one side; here a 64 x 64 tile goes through LDS, read along i (contiguous in `in`) and written
+// along j (contiguous in `out`). Covers 2-D transposes and NHWC <-> NCHW style permutations.
+struct TransposeParams { uint32_t B, I, J, sb, sj; };
+
+extern "C" __global__ __launch_bounds__(256) void transpose_tiled(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                                  TransposeParams P) {
+    __shared__ uint32_t tile[64][65];
+    const uint32_t ti = threadIdx.x & 63u, tr = threadIdx.x >> 6;
+    const uint32_t j0 = blockIdx.x * 64u, i0 = blockIdx.y * 64u, b = blockIdx.z;
+    const uint32_t* src = in + (uint64_t)b * P.sb;
+    uint32_t* dst = out + (uint64_t)b * P.I * P.J;
+#pragma unroll
+    for (uint32_t p = 0; p < 16; ++p) {
+        const uint32_t j = j0 + tr + 4u * p, i = i0 + ti;
+        if (i < P.I && j < P.J) tile[tr + 4u * p][ti] = src[(uint64_t)j * P.sj + i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t p = 0; p < 16; ++p) {
+        const uint32_t i = i0 + tr + 4u * p, j = j0 + ti;
+        if (i < P.I && j < P.J) dst[(uint64_t)i * P.J + j] = tile[ti][tr + 4u * p];
+    }
+}

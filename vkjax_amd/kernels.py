@@ -139,6 +139,9 @@ def lower_ew_chain(chain: EwChain) -> Launch:
         raise NotImplementedError(f'element-wise access pattern with {len(dims)} irreducible dimensions: {chain.shape}')
     ndim    = len(dims)
     strides = strides[1:]
+    transposed = _as_tiled_transpose(chain, dims, strides)
+    if transposed is not None:
+        return transposed
     vec = 4
     if n % 4 or dims[-1] % 4:
         vec = 1
@@ -191,6 +194,24 @@ def lower_ew_chain(chain: EwChain) -> Launch:
     per_thread = {2: 1, 4: 2, 6: 2, 8: 1}[slots]               #vectors a thread works on (the kernel's U)
     return Launch(f'ew_chain_v{vec}_s{slots}', (_cdiv(_cdiv(n, vec), BLOCK * per_thread), 1, 1), (BLOCK, 1, 1),
                   [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
+
+
+def _as_tiled_transpose(chain: EwChain, dims, strides) -> tp.Optional[Launch]:
+    '''A pure copy whose collapsed form is out[b, i, j] = in[b * sb + j * sj + i] (the two fastest dimensions
+    trade places) goes through the LDS-tiled kernel when both of them are at least 16 long.'''
+    if chain.steps or len(dims) not in (2, 3):
+        return None
+    st = strides[0]
+    B, I, J = ([1] + list(dims))[-3:]
+    sb = st[0] if len(dims) == 3 else 0
+    if st[-2] != 1 or st[-1] < I or I < 16 or J < 16 or sb < 0 or B > 65535 or _cdiv(I, 64) > 65535:
+        return None
+    src = chain.first
+    if src.buffer.size * 4 >= 2**32:
+        return None
+    n = B * I * J
+    return Launch('transpose_tiled', (_cdiv(J, 64), _cdiv(I, 64), B), (BLOCK, 1, 1), [(chain.out, 0), (src.buffer, src.offset * 4)],
+                  _u32(B, I, J, sb, st[-1]), bytes_moved=8 * n)
 
 
 def iota(out: Buffer, dimension: int) -> Launch:
