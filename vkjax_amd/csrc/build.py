@@ -52,7 +52,7 @@ def build_shim(force=True):
     out = shim_path()
     if not force and _newer(out, [src, hdr]):
         return out
-    _run([HIPCC, '-O2', '-fPIC', '-shared', '-std=c++17', '-x', 'c++', '-D__HIP_PLATFORM_AMD__',
+    _run([HIPCC, '-O2', '-fPIC', '-shared', '-pthread', '-std=c++17', '-x', 'c++', '-D__HIP_PLATFORM_AMD__',
           f'-I{INCLUDE}', '-I/opt/rocm/include', src, '-o', out, '-L/opt/rocm/lib', '-lamdhip64',
           '-Wl,-rpath,/opt/rocm/lib'])
     return out

@@ -6,14 +6,17 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <thread>
 #include <new>
 #include <unordered_map>
 #include <string>
 #include <vector>
+#include <algorithm>
 
 namespace {
 
@@ -32,6 +35,41 @@ int fail(int code, const char* fmt, ...) {
 int hip_fail(hipError_t e, const char* what) {
     g_last_error = std::string(what) + ": " + hipGetErrorString(e);
     return (int)e > 0 ? (int)e : VKJ_EINVAL;
+}
+
+// Large uploads: the copy into the pinned staging buffer is done by a few threads, chunk by chunk,
+// while the calling thread hands every finished chunk to the DMA engine in order, so that staging
+// and transfer overlap instead of running one after the other.
+constexpr size_t STAGE_CHUNK   = 4u << 20;
+constexpr size_t STAGE_MIN     = 8u << 20;     // smaller transfers are copied inline
+constexpr int    STAGE_THREADS = 4;
+
+template <class Issue>
+int staged_upload(char* staging, const char* host, size_t nbytes, Issue&& issue) {
+    const size_t nchunks = (nbytes + STAGE_CHUNK - 1) / STAGE_CHUNK;
+    std::vector<std::atomic<int>> done(nchunks);
+    for (auto& d : done) d.store(0, std::memory_order_relaxed);
+    std::atomic<size_t> next{0};
+    auto worker = [&]() {
+        for (;;) {
+            const size_t k = next.fetch_add(1, std::memory_order_relaxed);
+            if (k >= nchunks) return;
+            const size_t off = k * STAGE_CHUNK, len = std::min(STAGE_CHUNK, nbytes - off);
+            memcpy(staging + off, host + off, len);
+            done[k].store(1, std::memory_order_release);
+        }
+    };
+    std::vector<std::thread> threads;
+    const int nthreads = (int)std::min<size_t>(STAGE_THREADS, nchunks);
+    for (int t = 0; t < nthreads; t++) threads.emplace_back(worker);
+    int status = 0;
+    for (size_t k = 0; k < nchunks; k++) {
+        while (!done[k].load(std::memory_order_acquire)) std::this_thread::yield();
+        const size_t off = k * STAGE_CHUNK, len = std::min(STAGE_CHUNK, nbytes - off);
+        if (status == 0) status = issue(off, len);
+    }
+    for (auto& t : threads) t.join();
+    return status;
 }
 
 #define HIP_TRY(expr)                                   \
@@ -504,6 +542,15 @@ int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t fla
     }
     if (up) for (auto& t : s->uploads) {
         if (!t.nbytes || !host_ptrs[t.slot]) continue;
+        if (t.nbytes >= STAGE_MIN) {
+            hipError_t err = hipSuccess;
+            const int r = staged_upload((char*)t.staging, (const char*)host_ptrs[t.slot], t.nbytes, [&](size_t off, size_t len) {
+                err = hipMemcpyAsync((char*)t.buf->dptr + t.offset + off, (char*)t.staging + off, len, hipMemcpyHostToDevice, c->stream);
+                return err == hipSuccess ? 0 : 1;
+            });
+            if (r) return hip_fail(err, "hipMemcpyAsync (staged upload)");
+            continue;
+        }
         memcpy(t.staging, host_ptrs[t.slot], t.nbytes);
         HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
     }
