@@ -341,7 +341,13 @@ def _replay(jaxpr, consts, inputs, env, order):
         name = eqn.primitive.name
         if name in _CALL_PARAMS:
             inner = eqn.params[_CALL_PARAMS[name]]
-            outs  = _replay(getattr(inner, 'jaxpr', inner), getattr(inner, 'consts', []), [read(v) for v in eqn.invars], env, order)
+            rule  = eqn.params.get('jvp_jaxpr_thunk') if name.startswith('custom_jvp') else None
+            #a call with a derivative rule of its own is one unit for the backward pass: its body is replayed
+            #for the values only
+            outs  = _replay(getattr(inner, 'jaxpr', inner), getattr(inner, 'consts', []), [read(v) for v in eqn.invars], env,
+                            order if not callable(rule) else [])
+            if callable(rule):
+                order.append(eqn)
         else:
             outs = emit(name, [read(v) for v in eqn.invars], [v.aval for v in eqn.outvars], eqn.params, eqn.primitive.multiple_results)
             outs = outs if eqn.primitive.multiple_results else [outs]
@@ -393,12 +399,16 @@ def value_and_grad(fun: tp.Callable, argnums: tp.Union[int, tp.Sequence[int]] = 
             name = eqn.primitive.name
             if name in _NOT_DIFFERENTIABLE:
                 continue
-            if name not in RULES:
-                raise NotImplementedError(f'no differentiation rule for {name}')
             operands = [value_of(v) for v in eqn.invars]
-            g = gs if eqn.primitive.multiple_results else _materialize(gs[0], outs_now[0])
-            out_arg = outs_now if eqn.primitive.multiple_results else outs_now[0]
-            in_cts = RULES[name](g, *operands, out_arg, **eqn.params)
+            if name in _CALL_PARAMS:
+                #a custom derivative rule (single result): rule(cotangent, result, *arguments)
+                in_cts = eqn.params['jvp_jaxpr_thunk'](_materialize(gs[0], outs_now[0]), outs_now[0], *operands)
+            else:
+                if name not in RULES:
+                    raise NotImplementedError(f'no differentiation rule for {name}')
+                g = gs if eqn.primitive.multiple_results else _materialize(gs[0], outs_now[0])
+                out_arg = outs_now if eqn.primitive.multiple_results else outs_now[0]
+                in_cts = RULES[name](g, *operands, out_arg, **eqn.params)
             for operand, ct in zip(operands, in_cts):
                 #a rule may hand back a thunk so that nothing is emitted for an operand nobody differentiates
                 if ct is not None and id(operand) in active:

@@ -12,6 +12,13 @@ def relu(x):
     return mnp.maximum(x, 0)
 
 
+@relu.defvjp
+def _relu_vjp(g, ans, x):
+    #jax.nn.relu's own rule: the cotangent passes where x > 0 (no share at x == 0)
+    zeros = lax.broadcast_in_dim(np.float32(0), tuple(g.shape), ()) if tuple(g.shape) else np.float32(0)
+    return (lax.select(lax.gt(x, mnp.broadcast_to(np.float32(0), tuple(x.shape)) if tuple(x.shape) else np.float32(0)), g, zeros),)
+
+
 def softmax(x, axis=-1):
     unnormalized = mnp.exp(x - lax.stop_gradient(mnp.max(x, axis, keepdims=True)))
     return unnormalized / mnp.sum(unnormalized, axis, keepdims=True)

@@ -316,9 +316,17 @@ def jit(fun: tp.Callable):
 
 def custom_jvp(fun: tp.Callable):
     '''Emits `custom_jvp_call_jaxpr` (what jax.nn.relu looks like in a jaxpr of that era;
-    reference: vkjax/ops.py:246-260). The derivative rule is not represented.'''
+    reference: vkjax/ops.py:246-260). A derivative rule can be attached with `.defvjp(rule)`,
+    `rule(cotangent, result, *arguments) -> cotangents of the arguments`; reverse-mode
+    differentiation then uses it instead of differentiating the body (the entry `jvp_jaxpr_thunk`
+    of the equation carries it; backends ignore that entry).'''
     def wrapped(*args):
-        params = dict(num_consts=0, jvp_jaxpr_thunk=None)
+        params = dict(num_consts=0, jvp_jaxpr_thunk=wrapped.vjp_rule)
         return _call_nested(fun, 'custom_jvp_call_jaxpr', 'fun_jaxpr', params, closed=True, args=args)
     wrapped.__name__ = getattr(fun, '__name__', 'custom_jvp_fn')
+    wrapped.vjp_rule = None
+    def defvjp(rule):
+        wrapped.vjp_rule = rule
+        return rule
+    wrapped.defvjp = defvjp
     return wrapped
