@@ -14,9 +14,11 @@ def relu(x):
 
 @relu.defvjp
 def _relu_vjp(g, ans, x):
-    #jax.nn.relu's own rule: the cotangent passes where x > 0 (no share at x == 0)
-    zeros = lax.broadcast_in_dim(np.float32(0), tuple(g.shape), ()) if tuple(g.shape) else np.float32(0)
-    return (lax.select(lax.gt(x, mnp.broadcast_to(np.float32(0), tuple(x.shape)) if tuple(x.shape) else np.float32(0)), g, zeros),)
+    #jax.nn.relu's own rule: the cotangent passes where x > 0 (no share at x == 0). The test is made on the
+    #result (max(x, 0) > 0 exactly where x > 0), so the backward pass does not keep the pre-activation alive
+    shape = tuple(g.shape)
+    zeros = lax.broadcast_in_dim(np.float32(0), shape, ()) if shape else np.float32(0)
+    return (lax.select(lax.gt(ans, zeros), g, zeros),)
 
 
 def softmax(x, axis=-1):
