@@ -432,6 +432,14 @@ def reduce_min(x, axes, **_):
     return _canon(x).min(axis=tuple(axes)) if len(axes) else _canon(x)
 
 
+def reduce_or(x, axes, **_):
+    return np.any(np.asarray(x, bool), axis=tuple(axes))
+
+
+def reduce_and(x, axes, **_):
+    return np.all(np.asarray(x, bool), axis=tuple(axes))
+
+
 def _arg_reduce(x, axes, index_dtype, better):
     '''Index of the first best element along one axis; a NaN is better than any number and
     the first NaN wins (XLA). The reference shader (argmax.comp:50-52) uses a strict compare,
@@ -654,6 +662,10 @@ def random_wrap(x, **_):
 
 
 def random_unwrap(x, **_):
+    return np.asarray(x, u32)
+
+
+def random_clone(x, **_):
     return np.asarray(x, u32)
 
 

@@ -241,6 +241,8 @@ param_matrix += [
     (clamp0, 'clamp scalars',           [random([77, 101]) * 2 - 1]),
     (clamp1, 'clamp arrays',            [random([77, 101]) - 1, random([77, 101]) * 2 - 1, random([77, 101])]),
     (clamp0, 'clamp int',               [randint(-5, 5, size=[77, 101])]),
+    (lambda x: lax.reduce_or(x, (1,)), 'any(axis=1)',    [random([77, 101]) > 0.99]),
+    (lambda x: lax.reduce_and(x, (0, 2)), 'all(axis=0,2)', [random([7, 11, 13]) > 0.01]),
     (split0, 'split axis 1',            [random([7, 99, 5])]),
     (split1, 'split + chains',          [random([7, 33])]),
 ]

@@ -392,6 +392,18 @@ def reduce_min(x, axes):  return _reduce('reduce_min', x, axes)
 def reduce_prod(x, axes): return _reduce('reduce_prod', x, axes)
 
 
+def reduce_or(x, axes):
+    if dtype_of(x)[0] != _bool:
+        raise TypeError('reduce_or takes booleans')
+    return _reduce('reduce_or', x, axes)
+
+
+def reduce_and(x, axes):
+    if dtype_of(x)[0] != _bool:
+        raise TypeError('reduce_and takes booleans')
+    return _reduce('reduce_and', x, axes)
+
+
 def argmax(x, axis: int, index_dtype=_i32):
     return _reduce('argmax', x, (axis,), core.canonicalize_dtype(index_dtype), dict(index_dtype=np.dtype(index_dtype)))
 

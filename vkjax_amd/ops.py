@@ -314,7 +314,7 @@ def noop(bufferpool, equation):
 stop_gradient = squeeze = expand_dims = bitcast_convert_type = noop
 copy = copy_p = optimization_barrier = noop
 #a typed key array and its uint32 words are the same device array
-random_wrap = random_unwrap = noop
+random_wrap = random_unwrap = random_clone = noop
 
 
 def reshape(bufferpool, equation):
@@ -478,7 +478,13 @@ def custom_jvp_call(bufferpool, equation):
     return _inline_call(bufferpool, equation, closed, getattr(closed, 'consts', ()))
 
 
-custom_vjp_call = custom_vjp_call_jaxpr = custom_jvp_call
+def custom_vjp_call(bufferpool, equation):
+    '''The forward function of a custom_vjp; jax versions name the parameter call_jaxpr or fun_jaxpr.'''
+    closed = equation.params['call_jaxpr'] if 'call_jaxpr' in equation.params else equation.params['fun_jaxpr']
+    return _inline_call(bufferpool, equation, closed, getattr(closed, 'consts', ()))
+
+
+custom_vjp_call_jaxpr = custom_vjp_call
 
 
 # ------------------------------------------------------------------ contractions
@@ -645,6 +651,11 @@ def reduce_op(bufferpool, equation):
     outvar, invar = equation.outvars[0], equation.invars[0]
     name   = equation.primitive.name
     inbuf  = bufferpool.get_buffer(invar)
+    if name in ('reduce_or', 'reduce_and'):
+        #jnp.any / jnp.all: on booleans (stored as 0 / 1) the maximum resp. minimum
+        if _kind(inbuf.dtype) != _B:
+            raise NotImplementedError(equation)
+        name = 'reduce_max' if name == 'reduce_or' else 'reduce_min'
     outbuf = bufferpool.get_buffer(outvar, increment_op_counter=True)
     if _kind(inbuf.dtype) == _B and name not in ('reduce_max', 'reduce_min'):
         raise NotImplementedError(equation)
@@ -688,7 +699,7 @@ def reduce_op(bufferpool, equation):
     return [Op(equation, launch=K.reduce_general(outbuf, inbuf, kept, reduced, name))]
 
 
-reduce_max = reduce_min = reduce_sum = reduce_prod = argmin = argmax = reduce_op
+reduce_max = reduce_min = reduce_sum = reduce_prod = argmin = argmax = reduce_or = reduce_and = reduce_op
 
 
 def _reduce_window(bufferpool, equation, op_name):
