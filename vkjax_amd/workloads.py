@@ -234,16 +234,44 @@ def convnet_train_inputs(seed=7, batch=64, size=64, channels=(3, 64, 128), class
     return [params, x, onehot]
 
 
-def resnet50_loss(params, x, onehot):
-    logits, _ = resnet50(params, x)
+_STATISTICS = ('mean', 'var')
+
+
+def _split_statistics(params):
+    '''(trainable arrays, batch-norm statistics) as two trees of the same nesting.'''
+    if not isinstance(params, dict):
+        return params, None
+    trainable, fixed = {}, {}
+    for k, v in params.items():
+        if k in _STATISTICS:
+            fixed[k] = v
+        else:
+            trainable[k], sub = _split_statistics(v)
+            if sub:
+                fixed[k] = sub
+    return trainable, fixed
+
+
+def _merge_statistics(trainable, fixed):
+    if not isinstance(trainable, dict):
+        return trainable
+    merged = {k: _merge_statistics(v, (fixed or {}).get(k)) for k, v in trainable.items()}
+    merged.update({k: v for k, v in (fixed or {}).items() if k not in merged})
+    return merged
+
+
+def resnet50_loss(trainable, statistics, x, onehot):
+    logits, _ = resnet50(_merge_statistics(trainable, statistics), x)
     return softmax_cross_entropy(logits, onehot)
 
 
 def resnet50_train_step(params, x, onehot, lr=0.01):
-    '''One SGD step of ResNet-50 with its batch-norm layers in inference mode (fixed statistics): gradients
-    of every convolution kernel, scale, shift and of the dense layer.'''
-    loss, grads = mj.value_and_grad(resnet50_loss)(params, x, onehot)
-    return loss, _sgd(params, grads, lr)
+    '''One SGD step of ResNet-50 with frozen batch-norm statistics: gradients and updates for every
+    convolution kernel, scale, shift and the dense layer; mean and variance stay as they are.
+    Returns (loss, updated trainable arrays).'''
+    trainable, statistics = _split_statistics(params)
+    loss, grads = mj.value_and_grad(resnet50_loss)(trainable, statistics, x, onehot)
+    return loss, _sgd(trainable, grads, lr)
 
 
 def resnet50_train_inputs(seed=4, batch=64, size=224, num_classes=1000, width_scale=1.0):
