@@ -81,3 +81,18 @@ def test_column_sums_take_over_their_operands_multiply_or_negate():
     fused   = vkjax_amd.wrap(f, frontend='minijax')(x, y)
     unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)(x, y)
     assert np.array_equal(fused, unfused)
+
+
+@pytest.mark.parametrize('shape', [(256, 10), (64, 1000), (33, 7), (5, 64), (5, 65), (3, 4092), (2, 3, 50)])
+def test_fused_softmax_equals_the_separate_launches(shape):
+    '''jax.nn.softmax's reduce_max / subtract / exp / reduce_sum / divide as one launch: same bits as the five.'''
+    import vkjax_amd
+    x = (rng.random_sample(shape) * 12 - 6).astype(np.float32)
+    f = lambda x: mj.nn.softmax(x, axis=-1)
+    print(f'softmax {shape}', flush=True)
+    y, _, fn = check_against_oracle(f, [x], rtol=1e-5, atol=1e-7)
+    kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+    assert len(kernels) == 1 and kernels[0].startswith('softmax_rows'), kernels
+    unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)(x)
+    assert np.array_equal(y, unfused)
+    assert np.allclose(y.sum(axis=-1), 1.0, atol=1e-5)

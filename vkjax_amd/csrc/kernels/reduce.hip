@@ -266,6 +266,63 @@ REDUCE_KERNELS(any, 2)
 REDUCE_KERNELS(fargmax, 3)
 REDUCE_KERNELS(fargmin, 4)
 
+// ---------------------------------------------------------------------------------------------
+// softmax over the rows of [outer, R] in one launch: out = exp(x - max(x)) / sum(exp(x - max(x))).
+// Takes the place of reduce_max -> (subtract, exp) -> reduce_sum -> divide. One wave per row; the
+// sum is accumulated in exactly the order reduce_rows uses (per-lane partial sums over the same
+// elements, combined pairwise, then the same butterfly), so the result has the same bits as the
+// four separate launches. For rows short enough to run unsplit there (the host checks R).
+struct SoftmaxParams { uint32_t outer, R; };
+
+template <int VEC, class F>
+__device__ __forceinline__ float row_sum_as_reduce_rows(F value_at, uint32_t R, uint32_t lane) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (VEC == 4) {
+        uint32_t r = lane * 4u;
+        for (; r + 3u * 256u < R; r += 4u * 256u)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] += value_at(r + q * 256u + j);
+        for (; r < R; r += 256u)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] += value_at(r + j);
+    } else {
+        uint32_t r = lane;
+        for (; r + 3u * 64u < R; r += 4u * 64u)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[q] += value_at(r + q * 64u);
+        for (; r < R; r += 64u) acc[0] += value_at(r);
+    }
+    float a = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) a = a + __shfl_xor(a, s, 64);
+    return a;
+}
+
+template <int VEC>
+__device__ __forceinline__ void softmax_rows_body(float* __restrict__ out, const float* __restrict__ in, const SoftmaxParams& P) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= P.outer) return;                                       // whole wave leaves together
+    const float* x = in + (uint64_t)row * P.R;
+    float* y = out + (uint64_t)row * P.R;
+    float m = -INFINITY;                                              // the maximum does not depend on the order; a NaN wins
+    for (uint32_t r = lane; r < P.R; r += 64u) { const float v = x[r]; m = (v > m || v != v) ? v : m; }
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) { const float o = __shfl_xor(m, s, 64); m = (m > o || m != m) ? m : o; }
+    const float total = row_sum_as_reduce_rows<VEC>([&](uint32_t r) { return expf(x[r] - m); }, P.R, lane);
+    for (uint32_t r = lane; r < P.R; r += 64u) y[r] = expf(x[r] - m) / total;
+}
+
+extern "C" __global__ __launch_bounds__(256) void softmax_rows_v1(float* __restrict__ out, const float* __restrict__ in, SoftmaxParams P) {
+    softmax_rows_body<1>(out, in, P);
+}
+// R % 4 == 0: the summation order of the 16-byte reduce_rows kernel
+extern "C" __global__ __launch_bounds__(256) void softmax_rows_v4(float* __restrict__ out, const float* __restrict__ in, SoftmaxParams P) {
+    softmax_rows_body<4>(out, in, P);
+}
+
 struct ReduceGeneralParams {
     uint32_t n_out, n_red, op, type;
     uint32_t nk, nr;

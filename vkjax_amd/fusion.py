@@ -50,7 +50,7 @@ def _reads(op) -> tp.List:
             return [op.meta[2]]
         if op.meta[0] == 'threefry':
             return list(op.meta[2])
-        if op.meta[0] == 'random_stream':
+        if op.meta[0] in ('random_stream', 'reduce'):
             return [b for b, _ in op.launch.buffers[1:] if b is not None]
     return [b for b, _ in op.launch.buffers if b is not None]
 
@@ -207,9 +207,65 @@ def fuse_ops(all_ops, bufferpool, outvars):
             producer[id(out._placeholder)] = len(result) - 1
     ops = fuse_random_streams([op for op in result if op is not None], bufferpool, outvars)
     ops = fuse_stream_chains(ops, bufferpool, outvars)
+    ops = fuse_softmax(ops, bufferpool, outvars)
     ops = fuse_reduce_prologues(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
     return remove_dead_ops(ops, bufferpool, outvars)
+
+
+def fuse_softmax(ops, bufferpool, outvars):
+    '''softmax over the last dimension as jax.nn.softmax spells it,
+
+        m = reduce_max(x) ; e = exp(x - m) ; s = reduce_sum(e) ; y = e / s
+
+    becomes one launch when m, e and s are used by nothing else. Same values, bit for bit: the fused kernel
+    adds in the order of the row reduction it replaces.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    removed, replacement = set(), {}
+
+    def per_row(operand, shape):
+        return (operand is not None and operand.offset == 0 and len(shape) >= 1
+                and tuple(operand.strides) == K.row_major_strides(shape[:-1] + (1,))[:-1] + (0,))
+
+    for i, R1 in enumerate(ops):
+        if R1.meta is None or R1.meta[0] != 'reduce' or i + 3 >= len(ops):
+            continue
+        _, m, x, outer, rows, inner, name, _, nsplit = R1.meta
+        C1, R2, C2 = ops[i + 1], ops[i + 2], ops[i + 3]
+        if (name != 'reduce_max' or inner != 1 or nsplit != 1 or x.dtype != 'float32' or not 0 < rows < K.SOFTMAX_MAX_ROW
+                or C1.chain is None or C2.chain is None or R2.meta is None or R2.meta[0] != 'reduce'):
+            continue
+        c1, c2 = C1.chain, C2.chain
+        _, s, e, outer2, rows2, inner2, name2, _, nsplit2 = R2.meta
+        flat = lambda shape: (int(np_prod(shape[:-1])), shape[-1]) if len(shape) else (1, 1)
+        if (name2 != 'reduce_sum' or (outer2, rows2, inner2, nsplit2) != (outer, rows, 1, 1)
+                or flat(c1.shape) != (outer, rows) or flat(c2.shape) != (outer, rows)
+                or c1.first.buffer._placeholder is not x._placeholder or not _is_full_contiguous_any_shape(c1.first, c1.shape)
+                or [st.op for st in c1.steps] != [EW['SUB_F'], EW['EXP_F']] or c1.steps[0].operand_left
+                or c1.steps[0].operand.buffer._placeholder is not m._placeholder or not per_row(c1.steps[0].operand, c1.shape)
+                or e._placeholder is not c1.out._placeholder
+                or c2.first.buffer._placeholder is not c1.out._placeholder or not _is_full_contiguous_any_shape(c2.first, c2.shape)
+                or [st.op for st in c2.steps] != [EW['DIV_F']] or c2.steps[0].operand_left
+                or c2.steps[0].operand.buffer._placeholder is not s._placeholder or not per_row(c2.steps[0].operand, c2.shape)
+                or uses[pid(m)] != 1 or uses[pid(c1.out)] != 2 or uses[pid(s)] != 1):
+            continue
+        fused = Op(_label(R1, C1, R2, C2), launch=K.softmax_rows(c2.out, x, outer, rows))
+        fused.index = C2.index
+        x.accesses.append(C2.index)
+        for b in (m, c1.out, s):
+            b._placeholder.elided = True
+        removed |= {i, i + 1, i + 2}
+        replacement[i + 3] = fused
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
+
+
+def np_prod(values) -> int:
+    out = 1
+    for v in values:
+        out *= int(v)
+    return out
 
 
 def fuse_reduce_prologues(ops, bufferpool, outvars):

@@ -581,6 +581,17 @@ def reduce(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str,
     return [first, second]
 
 
+SOFTMAX_MAX_ROW = 4096      #rows this short run unsplit in reduce_rows, whose summation order softmax_rows repeats
+
+
+def softmax_rows(out: Buffer, inp: Buffer, outer: int, R: int) -> Launch:
+    '''exp(x - max) / sum(exp(x - max)) over the rows of [outer, R]; see softmax_rows_body in reduce.hip.'''
+    assert 0 < R < SOFTMAX_MAX_ROW and inp.size == out.size == outer * R
+    vec = 4 if R % 4 == 0 else 1
+    return Launch(f'softmax_rows_v{vec}', (_cdiv(outer, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], _u32(outer, R),
+                  bytes_moved=8 * outer * R)
+
+
 def reduce_general(out: Buffer, inp: Buffer, kept, reduced, op: str) -> Launch:
     '''kept / reduced: lists of (size, stride) in row-major order of the output / of the reduce index.'''
     if len(kept) > 4 or len(reduced) > 4:
