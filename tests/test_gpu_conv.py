@@ -168,3 +168,38 @@ def test_lean_kernel_tile_chunks_with_epilogue(tile, bk):
                     assert [l.kernel for l in launches] == [f'conv_gemm_{tile}x{bk}_lean'], [l.kernel for l in launches]
     finally:
         K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = None
+
+
+def test_four_waves_per_tile_kernel():
+    '''Products with few output tiles: four waves share a 32 x 32 tile, each taking a quarter of every 128-long
+    k step. Dense layers with bias / ReLU, a contraction that is no multiple of 128, 1x1 and padded 3x3
+    convolutions with a batch-norm + residual + ReLU epilogue; integer-valued data, so every result is exact.'''
+    from vkjax_amd import kernels as K
+    from vkjax_amd import minijax as mj
+    lax, nn, jnp = mj.lax, mj.nn, mj.numpy
+    dn = ('NHWC', 'HWIO', 'NHWC')
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+
+    def dense(x, w, b): return nn.relu(jnp.dot(x, w) + b)
+    def plain(x, w): return jnp.dot(x, w)
+    def bn_res_relu(x, k, mean, scale, beta, res):
+        y = lax.conv_general_dilated(x, k, (1, 1), 'SAME', dimension_numbers=dn)
+        return nn.relu((y - mean) * scale + beta + res)
+
+    cases = [(dense, [ints(-4, 5, 256, 784), ints(-3, 4, 784, 512), ints(-9, 9, 512)]),
+             (dense, [ints(-4, 5, 70, 132), ints(-3, 4, 132, 36), ints(-9, 9, 36)]),
+             (plain, [ints(-4, 5, 64, 2048), ints(-2, 3, 2048, 1000)]),
+             (plain, [ints(-4, 5, 33, 256), ints(-2, 3, 256, 4)]),
+             (dense, [ints(-4, 5, 256, 512), ints(-3, 4, 512, 10), ints(-9, 9, 10)]),
+             (plain, [ints(-4, 5, 40, 388), ints(-2, 3, 388, 7)]),
+             (bn_res_relu, [ints(-4, 5, 2, 9, 7, 128), ints(-3, 4, 1, 1, 128, 72), ints(-5, 5, 72), ints(1, 4, 72), ints(-9, 9, 72), ints(-50, 50, 2, 9, 7, 72)]),
+             (bn_res_relu, [ints(-4, 5, 2, 9, 7, 256), ints(-3, 4, 3, 3, 256, 40), ints(-5, 5, 40), ints(1, 4, 40), ints(-9, 9, 40), ints(-50, 50, 2, 9, 7, 40)])]
+    K.FORCE_CONV_KSPLIT = True
+    try:
+        for f, args in cases:
+            print(f'four waves per tile: {f.__name__} {[a.shape for a in args]}', flush=True)
+            _, _, fn = check_against_oracle(f, args, exact=True)
+            launches = list(fn._jaxpr_interpreters.values())[0].launches
+            assert [l.kernel for l in launches] in (['conv_gemm_32x32x128_ks4'], ['conv_gemm_32x32x128_ks4g']), [l.kernel for l in launches]
+    finally:
+        K.FORCE_CONV_KSPLIT = None

@@ -100,11 +100,15 @@ struct ConvDerived {
 // registers, and with them resident waves, even when not taken): both operands on the 16-byte
 // path, k tiles that never straddle kernel taps, a row-major result, an epilogue that fits the
 // straight-line template.
-template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST, bool LEAN>
+template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST, bool LEAN, int KSW = 1>
 __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
                                                const float* __restrict__ w, const ConvEpiPtrs& epi,
                                                const ConvDerivedPtrs& Dp, const ConvParams& Pk, const ConvDerived& Dk) {
-    constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, NT = 64 * WGM * WGN;
+    // KSW > 1: KSW groups of WGM x WGN waves share one block tile, each taking a 1/KSW slice of every k
+    // step; their accumulators are added through LDS before the epilogue. For products whose handful of
+    // tiles would otherwise leave most of a CU's four MFMA units idle (a wave can drive only one).
+    static_assert(KSW == 1 || (LEAN && TM == 1 && TN == 1), "k-split blocks exist for the lean single-tile form only");
+    constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, NT = 64 * WGM * WGN * KSW;
     constexpr int LDA = BK + 4, LDB = BN + 4;
     __shared__ __attribute__((aligned(16))) float As[BM * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
@@ -137,7 +141,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     const bool c_contig = LEAN || (P.flags & 1u), flat_rows = P.flags & 2u, masked = P.flags & 4u;
     const int nepi = (P.flags >> 8) & 15u, epi_first_full = (int)((P.flags >> 16) & 15u) - 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN;
+    const int kw = wave / (WGM * WGN), wm = (wave % (WGM * WGN)) / WGN, wn = wave % WGN;
     const int l32 = lane & 31, half = lane >> 5;
 
     // A block works through up to `chunk` consecutive M tiles of one N tile, one after the other,
@@ -442,11 +446,11 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     // lanes 32-63 the second half. Fragments are double-buffered in registers: the LDS reads of
     // group g+1 are in flight while the MFMAs of group g execute.
     auto compute = [&]() {
-        constexpr int G = BK / 8;
+        constexpr int BKW = BK / KSW, G = BKW / 8;               // this wave's slice of the k step
         f32x4 af[2][TM];
         float bf[2][TN][4];
         auto load_frags = [&](int g, int buf) {
-            const int kk = half * (BK / 2) + g * 4;
+            const int kk = kw * BKW + half * (BKW / 2) + g * 4;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
                 af[buf][i] = *reinterpret_cast<const f32x4*>(&As[((wm * TM + i) * 32 + l32) * LDA + kk]);
@@ -529,6 +533,21 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) c[i][j][v] = acc[i][j][v];
+        if constexpr (KSW > 1) {
+            // the k slices meet in the first group of waves (the A tile's LDS space is free after the last step)
+            static_assert((KSW - 1) * WGM * WGN * 16 * 64 <= BM * LDA, "reduction buffer does not fit the A tile");
+            float* red = As + ((kw - 1) * WGM * WGN + wm * WGN + wn) * 16 * 64 + lane;
+            if (kw > 0) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) red[v * 64] = c[0][0][v];
+            }
+            __syncthreads();
+            if (kw > 0) continue;                                 // nsub == 1 for these kernels: the wave is done
+#pragma unroll
+            for (int s = 1; s < KSW; ++s)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) c[0][0][v] += As[((s - 1) * WGM * WGN + wm * WGN + wn) * 16 * 64 + v * 64 + lane];
+        }
 #ifdef CONV_PHASE_STAMPS
         if (sub == 0) {
             if (first_full >= 0) { float sink = full[0][0][0]; asm volatile("" :: "v"(sink)); }
@@ -662,11 +681,11 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 #endif
 }
 
-#define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF, LEAN)                                               \
-    extern "C" __global__ __launch_bounds__(64 * WGM * WGN) __attribute__((amdgpu_waves_per_eu(2))) void name( \
+#define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF, LEAN, ...)                                          \
+    extern "C" __global__ __launch_bounds__(64 * WGM * WGN * (1, ##__VA_ARGS__)) __attribute__((amdgpu_waves_per_eu(2))) void name( \
         float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
         ConvEpiPtrs epi, ConvDerivedPtrs dp, ConvParams P, ConvDerived D) {                                  \
-        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF, LEAN>(out, x, w, epi, dp, P, D);                        \
+        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF, LEAN, ##__VA_ARGS__>(out, x, w, epi, dp, P, D);         \
     }
 
 // name = conv_gemm_<BM>x<BN>x<BK>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads),
@@ -684,3 +703,7 @@ CONV_TILE(64x64x32, 2, 2, 1, 1, 32)
 CONV_TILE(64x64x64, 2, 2, 1, 1, 64)
 CONV_TILE(32x32x32, 1, 1, 1, 1, 32)
 CONV_TILE(32x32x64, 1, 1, 1, 1, 64)
+// one 32 x 32 tile per block, the k step of 128 split over four waves (chunk 1; see KSW above)
+CONV_KERNEL(conv_gemm_32x32x128_ks4, 1, 1, 1, 1, 128, true, true, true, 4)
+// the same with element-wise loads of the kernel operand (an output width that is no multiple of 4)
+CONV_KERNEL(conv_gemm_32x32x128_ks4g, 1, 1, 1, 1, 128, true, false, true, 4)

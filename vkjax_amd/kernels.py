@@ -362,6 +362,7 @@ FORCE_CONV_TILE: tp.Optional[str] = None
 FORCE_CONV_BK:   tp.Optional[int] = None
 FORCE_CONV_CHUNK: tp.Optional[int] = None
 FORCE_CONV_GENERAL = False          #never pick the lean kernel variant
+FORCE_CONV_KSPLIT: tp.Optional[bool] = None    #the four-waves-per-tile kernel: always (where it applies) / never
 
 
 def choose_conv_tile(M: int, N: int, compute_units: int = 256):
@@ -474,8 +475,16 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     lean = (a_fast and b_fast and c_contig and (g.Cin % bk == 0 or g.KH * g.KW == 1)
             and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL)
     flat_rows = g.batch == 1 and g.Wo == 1
+    #a product with so few 32 x 32 tiles that one wave per tile leaves most MFMA units idle: four waves per
+    #tile, each taking a quarter of every (128-long) k step
+    ksplit = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
+              (_cdiv(M, 32) * _cdiv(N, 32) <= 2 * compute_units and K >= 256 and FORCE_CONV_TILE is None and FORCE_CONV_BK is None))
+    ksplit = bool(ksplit) and a_fast and c_contig and (g.Cin % 128 == 0 or g.KH * g.KW == 1) \
+        and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL
+    if ksplit:
+        tag, bm, bn, nt, bk, lean = '32x32', 32, 32, 256, 128, True
     tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
-    chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean else 1
+    chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean and not ksplit else 1
     kinds = [e.kind for e in epilogue]
     x_bytes = (lhs.size - lhs_offset) * 4
     w_bytes = K * N * 4 if b_fast else (rhs.size - rhs_offset) * 4
@@ -504,7 +513,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     params += derived_desc
     buffers = [(out, out_offset * 4), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
     buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0)) + derived_ptrs
-    kernel  = f'conv_gemm_{tag}x{bk}_' + ('lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
+    kernel  = f'conv_gemm_{tag}x{bk}_' + (('ks4' if b_fast else 'ks4g') if ksplit else 'lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
     return Launch(kernel, (_cdiv(tiles_m, chunk) * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
                   bytes_moved=nbytes, flops=2 * M * N * K)
