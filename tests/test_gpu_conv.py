@@ -84,6 +84,7 @@ def test_dot_sizes():
 
 def reduce_window_max0(x): return lax.reduce_window(x, -jnp.inf, lax.max, (1, 2, 2, 1), (1, 1, 1, 1), 'VALID')
 def reduce_window_max1(x): return lax.reduce_window(x, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), 'SAME')
+def reduce_window_max2(x): return lax.reduce_window(x, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (0, 1), (0, 1), (0, 0)))
 def reduce_window_sum0(x): return lax.reduce_window(x, 0.0, lax.add, (1, 2, 2, 1), (1, 2, 2, 1), 'VALID')
 def reduce_window_sum1(x): return lax.reduce_window(x, 0.0, lax.add, (1, 3, 3, 1), (1, 2, 2, 1), 'SAME')
 def reduce_window_odd(x):  return lax.reduce_window(x, -jnp.inf, lax.max, (1, 3, 2, 3), (1, 2, 1, 2), ((0, 0), (1, 1), (0, 1), (1, 0)))
@@ -92,6 +93,10 @@ pool_matrix = [
     (reduce_window_max0, '2x2 no-pad',        [random([11, 100, 111, 5])], True),
     (reduce_window_max1, '3x3 +pad',          [random([77, 10, 99, 17])], True),
     (reduce_window_max1, '3x3 +pad C64',      [random([4, 56, 56, 64]) - 0.5], True),
+    (reduce_window_max1, '3x3 s2 odd sizes C8', [random([3, 15, 17, 8]) - 0.5], True),
+    (reduce_window_max1, '3x3 s2 tiny C4',    [random([2, 3, 2, 4]) - 0.5], True),
+    (reduce_window_max2, '3x3 s2 pad hi C12', [random([2, 14, 13, 12]) - 0.5], True),
+    (reduce_window_sum1, 'sum 3x3 s2 SAME C8', [np.round(random([3, 15, 17, 8]) * 8)], True),
     (reduce_window_sum0, 'sum 2x2 s2',        [random([4, 28, 28, 32])], False),
     (reduce_window_sum1, 'sum 3x3 s2 SAME',   [random([3, 15, 17, 6])], False),
     (reduce_window_odd,  'window over C too', [random([3, 15, 17, 6]) - 0.5], True),
