@@ -541,7 +541,9 @@ def plan_reduce_splits(outer: int, R: int, inner: int, op: str, compute_units: i
         split = min(_cdiv(want, outer), R // 4096)         #at least 16 KB per wave
     else:
         tiles = _cdiv(inner, 256)
-        want  = 4 * compute_units                  #blocks
+        #blocks: several per CU for arrays that stream from HBM for a while; one per CU for smaller ones, whose
+        #second launch (it reduces the per-block results) would otherwise take as long as the first
+        want  = (4 if outer * R * inner * 4 >= (128 << 20) else 1) * compute_units
         split = min(_cdiv(want, tiles * outer), R // 64)   #at least 64 rows per block
     return max(1, min(split, 65535))
 
