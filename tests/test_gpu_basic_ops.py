@@ -281,6 +281,8 @@ def test_tiled_transposes():
     NHWC <-> NCHW, a sliced source.'''
     cases = [(lambda x: lax.transpose(x, (1, 0)), [random([1000, 77])]),
              (lambda x: lax.transpose(x, (1, 0)), [random([64, 64])]),
+             (lambda x: lax.transpose(x, (1, 0)), [random([68, 1004])]),
+             (lambda x: lax.transpose(x[:, 8:48], (0, 2, 1)), [random([3, 36, 52])]),
              (lambda x: lax.transpose(x, (1, 0)), [randint(-9, 9, size=[129, 2050])]),
              (lambda x: lax.transpose(x, (0, 2, 1)), [random([5, 70, 33])]),
              (lambda x: lax.transpose(x, (0, 3, 1, 2)), [random([3, 17, 19, 24])]),
@@ -291,8 +293,8 @@ def test_tiled_transposes():
         print(f'case: tiled transpose {k}', flush=True)
         _, _, fn = check_against_oracle(f, args, exact=True)
         kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
-        if k != 7:
-            assert 'transpose_tiled' in kernels, kernels
+        if k != 9:
+            assert any(name.startswith('transpose_tiled') for name in kernels), kernels
 
 
 def test_nextafter_direction():

@@ -314,3 +314,35 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled(uint32_t* __re
         if (i < P.I && j < P.J) dst[(uint64_t)i * P.J + j] = tile[ti][tr + 4u * p];
     }
 }
+
+// The same with 16-byte global accesses on both sides: needs I, J, sj, sb and the source offset to be
+// multiples of 4. A thread reads four consecutive i of one j and, after the exchange through LDS,
+// writes four consecutive j of one i.
+extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                                     TransposeParams P) {
+    __shared__ uint32_t tile[64][65];
+    const uint32_t t16 = threadIdx.x & 15u, tr = threadIdx.x >> 4;        // 16 vectors per tile row, 16 rows per pass
+    const uint32_t j0 = blockIdx.x * 64u, i0 = blockIdx.y * 64u, b = blockIdx.z;
+    const uint32_t* src = in + (uint64_t)b * P.sb;
+    uint32_t* dst = out + (uint64_t)b * P.I * P.J;
+#pragma unroll
+    for (uint32_t p = 0; p < 4; ++p) {
+        const uint32_t j = j0 + tr + 16u * p, i = i0 + 4u * t16;
+        if (i < P.I && j < P.J) {                                         // I % 4 == 0: a vector is inside or outside as a whole
+            const u32x4 v = *reinterpret_cast<const u32x4*>(src + (uint64_t)j * P.sj + i);
+            tile[tr + 16u * p][4u * t16] = v.x; tile[tr + 16u * p][4u * t16 + 1u] = v.y;
+            tile[tr + 16u * p][4u * t16 + 2u] = v.z; tile[tr + 16u * p][4u * t16 + 3u] = v.w;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t p = 0; p < 4; ++p) {
+        const uint32_t i = i0 + tr + 16u * p, j = j0 + 4u * t16;
+        if (i < P.I && j < P.J) {
+            u32x4 v;
+            v.x = tile[4u * t16][tr + 16u * p]; v.y = tile[4u * t16 + 1u][tr + 16u * p];
+            v.z = tile[4u * t16 + 2u][tr + 16u * p]; v.w = tile[4u * t16 + 3u][tr + 16u * p];
+            *reinterpret_cast<u32x4*>(dst + (uint64_t)i * P.J + j) = v;
+        }
+    }
+}

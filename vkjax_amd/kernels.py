@@ -210,7 +210,8 @@ def _as_tiled_transpose(chain: EwChain, dims, strides) -> tp.Optional[Launch]:
     if src.buffer.size * 4 >= 2**32:
         return None
     n = B * I * J
-    return Launch('transpose_tiled', (_cdiv(J, 64), _cdiv(I, 64), B), (BLOCK, 1, 1), [(chain.out, 0), (src.buffer, src.offset * 4)],
+    vec = all(v % 4 == 0 for v in (I, J, st[-1], sb, src.offset))
+    return Launch('transpose_tiled_v4' if vec else 'transpose_tiled', (_cdiv(J, 64), _cdiv(I, 64), B), (BLOCK, 1, 1), [(chain.out, 0), (src.buffer, src.offset * 4)],
                   _u32(B, I, J, sb, st[-1]), bytes_moved=8 * n)
 
 
