@@ -61,7 +61,12 @@ int staged_upload(char* staging, const char* host, size_t nbytes, Issue&& issue)
     };
     std::vector<std::thread> threads;
     const int nthreads = (int)std::min<size_t>(STAGE_THREADS, nchunks);
-    for (int t = 0; t < nthreads; t++) threads.emplace_back(worker);
+    try {
+        for (int t = 0; t < nthreads; t++) threads.emplace_back(worker);
+    } catch (...) {
+        // no (more) threads to be had: the calling thread copies whatever is left
+    }
+    if ((int)threads.size() < nthreads) worker();
     int status = 0;
     for (size_t k = 0; k < nchunks; k++) {
         while (!done[k].load(std::memory_order_acquire)) std::this_thread::yield();
