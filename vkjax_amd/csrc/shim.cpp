@@ -77,6 +77,28 @@ int staged_upload(char* staging, const char* host, size_t nbytes, Issue&& issue)
     return status;
 }
 
+// Copy out of (or into) pinned memory with a few threads; small sizes are copied inline.
+void parallel_copy(char* dst, const char* src, size_t nbytes) {
+    if (nbytes < STAGE_MIN) { memcpy(dst, src, nbytes); return; }
+    const size_t nchunks = (nbytes + STAGE_CHUNK - 1) / STAGE_CHUNK;
+    std::atomic<size_t> next{0};
+    auto worker = [&]() {
+        for (;;) {
+            const size_t k = next.fetch_add(1, std::memory_order_relaxed);
+            if (k >= nchunks) return;
+            const size_t off = k * STAGE_CHUNK;
+            memcpy(dst + off, src + off, std::min(STAGE_CHUNK, nbytes - off));
+        }
+    };
+    std::vector<std::thread> threads;
+    try {
+        for (int t = 1; t < (int)std::min<size_t>(STAGE_THREADS, nchunks); t++) threads.emplace_back(worker);
+    } catch (...) {
+    }
+    worker();
+    for (auto& t : threads) t.join();
+}
+
 #define HIP_TRY(expr)                                   \
     do {                                                \
         hipError_t _e = (expr);                         \
@@ -575,7 +597,7 @@ int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t fla
     if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[nstamps - 1], c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
     if (down) for (auto& t : s->downloads)
-        if (t.nbytes) memcpy(host_ptrs[t.slot], t.staging, t.nbytes);
+        if (t.nbytes) parallel_copy((char*)host_ptrs[t.slot], (const char*)t.staging, t.nbytes);
     if (s->profiling) s->stamps_valid = (int)nstamps;
     return 0;
 }

@@ -80,14 +80,14 @@ class JaxprInterpreter:
         if self.graph:
             self.sequence.use_graph(True)
         self._output_slots = []
-        self._output_arrays = []
+        self._output_sizes = []
         for b in self.output_buffers:
             if b is None:
                 self._output_slots.append(None)
-                self._output_arrays.append(None)
+                self._output_sizes.append(None)
                 continue
             self._output_slots.append(self.sequence.record_download(b.tensor, b.nbytes()))
-            self._output_arrays.append(np.zeros(b.size, dtype=np.uint32))
+            self._output_sizes.append(b.size)
 
     def _flatten_args(self, X, with_residency: bool = False):
         leaves, resident = [], []
@@ -118,17 +118,19 @@ class JaxprInterpreter:
             words = _device_words_of_argument(x, var.aval)
             host[slot] = words
             keep.append(words)
-        for slot, arr in zip(self._output_slots, self._output_arrays):
+        #every call hands out fresh arrays: the runtime copies the results straight into them
+        fresh = [np.empty(n, np.uint32) if n is not None else None for n in self._output_sizes]
+        for slot, arr in zip(self._output_slots, fresh):
             if slot is not None:
                 host[slot] = arr
         self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT if self.resident_argnums else 0)
 
         output_values = []
-        for b, arr in zip(self.output_buffers, self._output_arrays):
+        for b, arr in zip(self.output_buffers, fresh):
             if b is None:
                 output_values.append(None)
                 continue
-            output_values.append(view_or_convert_from_32bit(arr.copy(), b.dtype).reshape(b.shape))
+            output_values.append(view_or_convert_from_32bit(arr, b.dtype).reshape(b.shape))
         output_values = tuple(output_values)
         if not return_all:
             return output_values
