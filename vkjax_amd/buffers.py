@@ -135,7 +135,11 @@ def to_device_words(x, dtype=None) -> np.ndarray:
 def hashable(var):
     '''Key of a variable in the pool; jax literals are unhashable but carry `.hash` (reference: vkjax/buffers.py:80-87).'''
     if core.is_literal(var):
-        return var.hash
+        h = getattr(var, 'hash', None)
+        if h is None:
+            #literal classes without a value hash: equal scalars of one dtype still share one buffer
+            h = hash((str(var.aval.dtype), np.asarray(var.val).tobytes()))
+        return h
     return var
 
 
