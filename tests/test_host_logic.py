@@ -251,3 +251,19 @@ def test_opcode_table_and_tile_choice():
         tag, bm, bn, nt = K.choose_conv_tile(m, n)
         assert tag in tags and nt in (64, 256)
     assert K.choose_conv_tile(8, 16)[1] <= 64
+
+
+def test_integer_and_float_literals_of_equal_hash_get_separate_buffers():
+    '''jax literals carry hash(value), and hash(1) == hash(1.0): the pool must still keep them apart.'''
+    from vkjax_amd.buffers import BufferPool, PlanOnlyDevice
+
+    class JaxLikeLiteral:
+        def __init__(self, val, dtype):
+            self.val, self.aval, self.hash = val, core.ShapedArray((), dtype), hash(val)
+
+    pool = BufferPool(PlanOnlyDevice())
+    one_i, one_f, one_f_again = JaxLikeLiteral(1, np.int32), JaxLikeLiteral(1.0, np.float32), JaxLikeLiteral(1.0, np.float32)
+    bi, bf, bf2 = pool.get_buffer(one_i), pool.get_buffer(one_f), pool.get_buffer(one_f_again)
+    assert bi is not bf and bf is bf2
+    assert bi.dtype == np.int32 and bf.dtype == np.float32
+    assert bi.tensor.initial_value.view(np.int32)[0] == 1 and bf.tensor.initial_value.view(np.float32)[0] == 1.0

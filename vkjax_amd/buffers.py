@@ -138,8 +138,9 @@ def hashable(var):
         h = getattr(var, 'hash', None)
         if h is None:
             #literal classes without a value hash: equal scalars of one dtype still share one buffer
-            h = hash((str(var.aval.dtype), np.asarray(var.val).tobytes()))
-        return h
+            h = hash(np.asarray(var.val).tobytes())
+        #jax hashes the bare value, and hash(1) == hash(1.0): the dtype keeps an integer and a float literal apart
+        return ('literal', str(var.aval.dtype), h)
     return var
 
 
