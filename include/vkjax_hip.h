@@ -109,6 +109,15 @@ int vkj_seq_num_steps(vkj_handle seq, int* uploads, int* launches, int* download
  * All uploads, then all launches, then all downloads, then one stream synchronisation.
  * host_ptrs[slot] supplies the host address of every recorded upload and download. */
 int vkj_seq_eval(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t flags);
+/* vkj_seq_eval that also brings in the arguments of the FOLLOWING evaluation while the device runs
+ * this one's launches: every upload slot whose next_host_ptrs entry is not NULL is staged and sent,
+ * on a second stream, to a landing buffer in HBM (allocated on first use, one per such slot), and
+ * copied on into its argument buffer once this evaluation's launches are through. The following
+ * call then passes NULL for those slots with VKJ_EVAL_NULL_IS_RESIDENT. next_host_ptrs has nslots
+ * entries or is NULL (then the call is vkj_seq_eval). The reference copies and runs strictly in
+ * turn (vkjax/kompute_jaxpr_interpreter.py:72-77); this is the overlap of the two. */
+int vkj_seq_eval_next(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t flags,
+                      void* const* next_host_ptrs);
 /* Launches only, `iters` times back to back, bracketed by two events on the context's
  * stream; *ms_total receives the elapsed device time of all iterations. Used for
  * measurement with inputs resident in HBM. No counterpart in the reference. */

@@ -219,3 +219,43 @@ def test_resident_arguments_are_uploaded_once():
     assert_tree_close(resident(params2, x2), plain(params2, x2), exact=True, what='one weight replaced')
     interp = list(resident._jaxpr_interpreters.values())[0]
     assert len(interp._resident_leaves) == len(leaves)
+
+
+def test_stream_matches_call_by_call():
+    '''Function.stream overlaps the upload of one argument tuple with the device work on the one
+    before it; its results must be those of plain calls, in order: small arguments, arguments large
+    enough for the chunked staging path (>= 8 MB), resident weights with one replaced on the way,
+    a change of signature in the middle, one tuple only, and none at all.'''
+    rng = np.random.default_rng(5)
+    def scale_shift(x, w):
+        return mj.numpy.tanh(x * w + 1.0), mj.numpy.sum(x, axis=0)
+    plain = vkjax_amd.wrap(scale_shift, frontend='minijax')
+    fast  = vkjax_amd.wrap(scale_shift, frontend='minijax')
+    small = [(rng.standard_normal((33, 17)).astype(np.float32), rng.standard_normal((17,)).astype(np.float32)) for _ in range(4)]
+    large = [(rng.standard_normal((1200, 2048)).astype(np.float32), rng.standard_normal((2048,)).astype(np.float32)) for _ in range(3)]
+    for name, tuples in [('small', small), ('large', large), ('mixed signatures', small[:2] + large[:2] + small[2:]),
+                         ('single', small[:1]), ('empty', [])]:
+        expected = [plain(*t) for t in tuples]
+        got = list(fast.stream(iter(tuples)))
+        assert len(got) == len(expected), name
+        for k, (g, e) in enumerate(zip(got, expected)):
+            assert_tree_close(g, e, exact=True, what=f'{name} [{k}]')
+    #a plain call after a stream sees its own arguments, not what the stream left behind
+    assert_tree_close(fast(*small[3]), plain(*small[3]), exact=True, what='call after stream')
+
+    params, x = W.mlp_inputs()
+    plain_mlp = vkjax_amd.wrap(W.mlp, frontend='minijax')
+    resident  = vkjax_amd.wrap(W.mlp, frontend='minijax', resident_argnums=(0,))
+    from vkjax_amd.minijax import tree_util
+    leaves, structure = tree_util.tree_flatten(params)
+    params2 = tree_util.tree_unflatten(structure, [leaves[0] * np.float32(0.5)] + list(leaves[1:]))
+    batches = [(params, x), (params, x[::-1].copy()), (params2, x), (params2, x * np.float32(2)), (params, x)]
+    expected = [plain_mlp(*t) for t in batches]
+    for k, (g, e) in enumerate(zip(resident.stream(batches), expected)):
+        assert_tree_close(g, e, exact=True, what=f'resident weights [{k}]')
+
+    #abandoning a stream half way leaves the function usable
+    it = fast.stream(iter(small))
+    next(it)
+    it.close()
+    assert_tree_close(fast(*small[0]), plain(*small[0]), exact=True, what='call after an abandoned stream')

@@ -267,3 +267,57 @@ def test_integer_and_float_literals_of_equal_hash_get_separate_buffers():
     assert bi is not bf and bf is bf2
     assert bi.dtype == np.int32 and bf.dtype == np.float32
     assert bi.tensor.initial_value.view(np.int32)[0] == 1 and bf.tensor.initial_value.view(np.float32)[0] == 1.0
+
+
+def test_ahead_iterator_keeps_order_passes_errors_on_and_lets_go():
+    '''The helper-thread iterator behind Function.stream: results come in the order of the
+    iterable, an exception raised by the iterable or by `prepare` reaches the consumer at the
+    position where it happened, and close() releases a helper that is waiting for the consumer.'''
+    import threading, time
+    from vkjax_amd.function import _Ahead
+    assert list(_Ahead(range(20), lambda i: i * i)) == [i * i for i in range(20)]
+    assert list(_Ahead([], lambda i: i)) == []
+
+    def failing(i):
+        if i == 3:
+            raise KeyError('three')
+        return i
+    got = []
+    with pytest.raises(KeyError):
+        for value in _Ahead(range(10), failing):
+            got.append(value)
+    assert got == [0, 1, 2]
+
+    def endless():
+        i = 0
+        while True:
+            yield i
+            i += 1
+    ahead = _Ahead(endless(), lambda i: i)
+    it = iter(ahead)
+    assert [next(it), next(it)] == [0, 1]
+    ahead.close()
+    ahead._thread.join(timeout=2.0)
+    assert not ahead._thread.is_alive()
+
+    # a helper parked on the consumer's event is released by close() too
+    gate = threading.Event()
+    def wait_for_consumer(i):
+        gate.wait()
+        return i
+    parked = _Ahead(range(3), wait_for_consumer, wake=gate)
+    time.sleep(0.05)
+    parked.close()
+    parked._thread.join(timeout=2.0)
+    assert not parked._thread.is_alive()
+
+
+def test_treedef_hash_and_equality():
+    from vkjax_amd.minijax import tree_util
+    a = tree_util.tree_structure(({'w': 1, 'b': [2, 3]}, None, (4,)))
+    b = tree_util.tree_structure(({'b': [0, 0], 'w': 0}, None, (0,)))
+    c = tree_util.tree_structure(({'b': (0, 0), 'w': 0}, None, (0,)))
+    d = tree_util.tree_structure([{'b': [0, 0], 'w': 0}, None, (0,)])
+    assert a == b and hash(a) == hash(b)
+    assert a != c and a != d
+    assert len({a, b, c, d}) == 3

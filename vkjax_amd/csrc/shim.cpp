@@ -114,6 +114,8 @@ struct Ctx {
     int         device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t  ev_begin = nullptr, ev_end = nullptr;
+    hipStream_t copy_stream = nullptr;   // created on first use: uploads that overlap the launches of `stream`
+    hipEvent_t  ev_landed = nullptr;
 };
 
 struct Buf {
@@ -144,6 +146,8 @@ struct Transfer {
     size_t offset, nbytes;
     int    slot;
     void*  staging;    // pinned host memory owned by the sequence
+    void*  next_staging = nullptr;   // pinned host memory and device memory for the arguments of the
+    void*  landing = nullptr;        // following evaluation, allocated when one is first handed in
 };
 
 struct Launch {
@@ -289,6 +293,8 @@ int vkj_ctx_destroy(vkj_handle h) {
     hipEventDestroy(c->ev_begin);
     hipEventDestroy(c->ev_end);
     hipStreamDestroy(c->stream);
+    if (c->copy_stream) { hipStreamSynchronize(c->copy_stream); hipStreamDestroy(c->copy_stream); }
+    if (c->ev_landed) hipEventDestroy(c->ev_landed);
     retire(c);
     delete c;
     return 0;
@@ -466,7 +472,12 @@ int vkj_seq_destroy(vkj_handle sh) {
     if (!s) return fail(VKJ_EINVAL, "vkj_seq_destroy: bad handle");
     if (int r = use(s->ctx)) return r;
     hipStreamSynchronize(s->ctx->stream);
-    for (auto& t : s->uploads)   if (t.staging) hipHostFree(t.staging);
+    if (s->ctx->copy_stream) hipStreamSynchronize(s->ctx->copy_stream);
+    for (auto& t : s->uploads) {
+        if (t.staging) hipHostFree(t.staging);
+        if (t.next_staging) hipHostFree(t.next_staging);
+        if (t.landing) hipFree(t.landing);
+    }
     for (auto& t : s->downloads) if (t.staging) hipHostFree(t.staging);
     for (auto e : s->stamps) hipEventDestroy(e);
     drop_graph(s);
@@ -545,10 +556,18 @@ int vkj_seq_num_steps(vkj_handle sh, int* uploads, int* launches, int* downloads
 }
 
 int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t flags) {
+    return vkj_seq_eval_next(sh, host_ptrs, nslots, flags, nullptr);
+}
+
+int vkj_seq_eval_next(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t flags, void* const* next_host_ptrs) {
     Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
     if (!s) return fail(VKJ_EINVAL, "vkj_seq_eval: bad handle");
     Ctx* c = s->ctx;
     if (int r = use(c)) return r;
+    if (next_host_ptrs && !c->copy_stream) {
+        HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
+        HIP_TRY(hipEventCreateWithFlags(&c->ev_landed, hipEventDisableTiming));
+    }
     const bool up = !(flags & VKJ_EVAL_SKIP_UPLOADS), down = !(flags & VKJ_EVAL_SKIP_DOWNLOADS);
     auto slot_ok = [&](const Transfer& t) { return t.nbytes == 0 || (host_ptrs && t.slot < nslots && host_ptrs[t.slot]); };
     const bool null_resident = flags & VKJ_EVAL_NULL_IS_RESIDENT;
@@ -590,11 +609,49 @@ int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t fla
     } else if (int r = issue_all(c, s)) {
         return r;
     }
+    bool landed = false;
+    if (next_host_ptrs) {
+        // While the device works through the launches: stage the following evaluation's arguments and
+        // send them, on the second stream, to landing buffers; once the launches are through, move
+        // them on into the argument buffers with device-to-device copies.
+        bool any = false;
+        for (auto& t : s->uploads) {
+            if (!t.nbytes || t.slot >= nslots || !next_host_ptrs[t.slot]) continue;
+            if (!t.landing) {
+                HIP_TRY(hipHostMalloc(&t.next_staging, t.nbytes, hipHostMallocDefault));
+                HIP_TRY(hipMalloc(&t.landing, t.nbytes));
+            }
+            hipError_t err = hipSuccess;
+            auto send = [&](size_t off, size_t len) {
+                err = hipMemcpyAsync((char*)t.landing + off, (char*)t.next_staging + off, len, hipMemcpyHostToDevice, c->copy_stream);
+                return err == hipSuccess ? 0 : 1;
+            };
+            if (t.nbytes >= STAGE_MIN) {
+                if (staged_upload((char*)t.next_staging, (const char*)next_host_ptrs[t.slot], t.nbytes, send))
+                    return hip_fail(err, "hipMemcpyAsync (staged upload of the next arguments)");
+            } else {
+                memcpy(t.next_staging, next_host_ptrs[t.slot], t.nbytes);
+                if (send(0, t.nbytes)) return hip_fail(err, "hipMemcpyAsync (upload of the next arguments)");
+            }
+            any = true;
+        }
+        landed = any;
+    }
+    // The downloads are queued after the copies above on purpose: a copy engine works through its
+    // queue in order, and a download queued first waits there for the launches, with every upload
+    // behind it, even one from the other stream, waiting as well.
     if (down) for (auto& t : s->downloads) {
         if (!t.nbytes) continue;
         HIP_TRY(hipMemcpyAsync(t.staging, (char*)t.buf->dptr + t.offset, t.nbytes, hipMemcpyDeviceToHost, c->stream));
     }
     if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[nstamps - 1], c->stream));
+    if (landed) {
+        HIP_TRY(hipEventRecord(c->ev_landed, c->copy_stream));
+        HIP_TRY(hipStreamWaitEvent(c->stream, c->ev_landed, 0));
+        for (auto& t : s->uploads)
+            if (t.nbytes && t.slot < nslots && next_host_ptrs[t.slot])
+                HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.landing, t.nbytes, hipMemcpyDeviceToDevice, c->stream));
+    }
     HIP_TRY(hipStreamSynchronize(c->stream));
     if (down) for (auto& t : s->downloads)
         if (t.nbytes) parallel_copy((char*)host_ptrs[t.slot], (const char*)t.staging, t.nbytes);

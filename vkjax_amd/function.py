@@ -6,10 +6,13 @@ reshaped to the traced shapes and re-nested, `profiling=True` returns `(output, 
 Tracing uses `jax.make_jaxpr` when jax can be imported and the stand-in tracer of
 `vkjax_amd.minijax` otherwise; a function written for one front-end must be traced with that one.
 '''
+import queue
+import threading
 import typing as tp
 
 import numpy as np
 
+from . import hip
 from . import minijax
 from .jaxpr_interpreter import JaxprInterpreter
 from .minijax import core, tree_util
@@ -28,6 +31,51 @@ def _pick_frontend(frontend: tp.Optional[str]):
     if frontend == 'minijax':
         return minijax.make_jaxpr, tree_util
     raise ValueError(f'unknown frontend {frontend}')
+
+
+class _Ahead:
+    '''Iterates over `prepare(item) for item in iterable`, with the iterable and `prepare` running on
+    a helper thread that stays up to two items ahead of the consumer. An exception raised there is
+    raised again in the consumer; close() lets the helper go when the consumer stops early.'''
+
+    def __init__(self, iterable, prepare, wake: tp.Optional[threading.Event] = None):
+        self._iterable, self._prepare, self._wake = iterable, prepare, wake
+        self._queue   = queue.Queue(maxsize=1)
+        self._closed  = threading.Event()
+        self._thread  = threading.Thread(target=self._work, name='vkjax-stream-ahead', daemon=True)
+        self._thread.start()
+
+    def _put(self, entry) -> bool:
+        while not self._closed.is_set():
+            try:
+                self._queue.put(entry, timeout=0.05)
+                return True
+            except queue.Full:
+                pass
+        return False
+
+    def _work(self):
+        try:
+            for item in self._iterable:
+                if self._closed.is_set() or not self._put(('item', self._prepare(item))):
+                    return
+            self._put(('end', None))
+        except BaseException as error:      # noqa: B902 - handed to the consumer
+            self._put(('error', error))
+
+    def __iter__(self):
+        while True:
+            kind, value = self._queue.get()
+            if kind == 'end':
+                return
+            if kind == 'error':
+                raise value
+            yield value
+
+    def close(self):
+        self._closed.set()
+        if self._wake is not None:
+            self._wake.set()               #a helper waiting for the consumer must see the close
 
 
 class Function:
@@ -51,12 +99,66 @@ class Function:
             return output
         return output, jaxpr_interpreter.get_profiling_info()
 
-    def _get_or_create_jaxpr_interpreter(self, args: tp.Tuple[tp.Any, ...]):
+    def stream(self, argument_tuples: tp.Iterable[tp.Tuple]) -> tp.Iterator[tp.Any]:
+        '''`(self(*args) for args in argument_tuples)` with the host work and the upload for each
+        tuple overlapping the device work on the one before it: a helper thread takes the tuples
+        from the iterable and flattens and converts their arguments while the calling thread waits
+        for the device; the runtime stages and uploads them during the preceding evaluation.
+        A tuple whose signature differs from its predecessor's is uploaded in its own turn.
+        No counterpart in the reference, whose calls copy, run and read back in turn
+        (vkjax/kompute_jaxpr_interpreter.py:72-81).'''
+        if self._profiling:
+            raise ValueError('stream() does not collect profiling information; call the function instead')
+        # Tracing and recording stay on the calling thread (a device context is used by one thread at
+        # a time). When the helper meets a signature that has no interpreter yet, it hands the tuple
+        # over as it is and prepares nothing further until the calling thread has dealt with it,
+        # so that what each prepared tuple assumes to be resident in HBM holds when it runs.
+        caught_up = threading.Event()
+        caught_up.set()
+
+        def prepare(args):
+            caught_up.wait()
+            args      = tuple(args)                  #what __call__ sees as *args
+            signature = self._signature(args)
+            entry     = self._jaxpr_interpreters.get(signature)
+            if entry is None:
+                caught_up.clear()
+                return [None, None, args]
+            return [entry, self._output_shapes[signature], entry._host_inputs(args)]
+
+        def resolved(item):
+            if item is not None and item[0] is None:
+                interpreter, output_shapes = self._get_or_create_jaxpr_interpreter(item[2])
+                item[:] = [interpreter, output_shapes, interpreter._host_inputs(item[2])]
+                caught_up.set()
+            return item
+
+        ahead = _Ahead(argument_tuples, prepare, wake=caught_up)
+        try:
+            items   = iter(ahead)
+            current = resolved(next(items, None))
+            while current is not None:
+                interpreter, output_shapes, host = current
+                following = resolved(next(items, None))
+                next_host = following[2] if following is not None and following[0] is interpreter else None
+                fresh     = interpreter._fresh_outputs(host)
+                interpreter.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT, next_host_arrays=next_host)
+                if next_host is not None:
+                    following[2] = [None] * interpreter.sequence.n_slots      #in place by now
+                yield self._restore_shapes(interpreter._output_values(fresh), output_shapes)
+                current = following
+        finally:
+            ahead.close()
+
+    def _signature(self, args: tp.Tuple[tp.Any, ...]):
         leaves, structure = self._tree.tree_flatten(args)
         args_shape        = tuple(np.shape(x) for x in leaves)
         args_dtype        = tuple(np.asarray(x).dtype if not hasattr(x, 'dtype') else np.dtype(x.dtype) for x in leaves)
         static_values     = tuple(repr(args[i]) for i in self._static_argnums if i < len(args))
-        shape_structure   = (args_shape, args_dtype, structure, static_values)
+        return (args_shape, args_dtype, structure, static_values)
+
+    def _get_or_create_jaxpr_interpreter(self, args: tp.Tuple[tp.Any, ...]):
+        shape_structure = self._signature(args)
         if shape_structure not in self._jaxpr_interpreters:
             #new input shapes or structure, need to re-trace
             jaxpr, output_shapes = self.jaxpr_function(*args)

@@ -60,6 +60,7 @@ _PROTOTYPES = {
     'vkj_seq_record_download': (C.c_int, [_H, _H, C.c_size_t, C.c_int, C.c_size_t]),
     'vkj_seq_num_steps':       (C.c_int, [_H, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     'vkj_seq_eval':            (C.c_int, [_H, C.POINTER(C.c_void_p), C.c_int, C.c_uint32]),
+    'vkj_seq_eval_next':       (C.c_int, [_H, C.POINTER(C.c_void_p), C.c_int, C.c_uint32, C.POINTER(C.c_void_p)]),
     'vkj_seq_replay':          (C.c_int, [_H, C.c_int, C.POINTER(C.c_float)]),
     'vkj_seq_use_graph':       (C.c_int, [_H, C.c_int]),
     'vkj_seq_timestamps':      (C.c_int, [_H, C.POINTER(C.c_float), C.c_int, C.POINTER(C.c_int)]),
@@ -276,11 +277,24 @@ class Sequence:
                                                       handles, argoffs, byteoff, n), f'vkj_seq_record_launch({kernel_name})')
         self.n_launches += 1
 
-    def eval(self, host_arrays: tp.Sequence[tp.Optional[np.ndarray]], flags: int = 0):
-        ptrs = (C.c_void_p * max(len(host_arrays), 1))()
-        for i, a in enumerate(host_arrays):
-            ptrs[i] = a.ctypes.data if a is not None else None
-        _check(self.device.lib.vkj_seq_eval(self.handle, ptrs, len(host_arrays), flags), 'vkj_seq_eval')
+    def eval(self, host_arrays: tp.Sequence[tp.Optional[np.ndarray]], flags: int = 0,
+             next_host_arrays: tp.Optional[tp.Sequence[tp.Optional[np.ndarray]]] = None):
+        '''`next_host_arrays`: the arguments of the following evaluation (None per slot that stays as
+        it is); they are uploaded while the device runs this one, and the following call passes None
+        for them with EVAL_NULL_IS_RESIDENT.'''
+        def pointers(arrays):
+            ptrs = (C.c_void_p * max(len(arrays), 1))()
+            for i, a in enumerate(arrays):
+                ptrs[i] = a.ctypes.data if a is not None else None
+            return ptrs
+        ptrs = pointers(host_arrays)
+        if next_host_arrays is None:
+            _check(self.device.lib.vkj_seq_eval(self.handle, ptrs, len(host_arrays), flags), 'vkj_seq_eval')
+            return
+        if len(next_host_arrays) != len(host_arrays):
+            raise ValueError('next_host_arrays must have one entry per slot')
+        _check(self.device.lib.vkj_seq_eval_next(self.handle, ptrs, len(host_arrays), flags, pointers(next_host_arrays)),
+               'vkj_seq_eval_next')
 
     def replay(self, iters: int = 1) -> float:
         '''Launches only; returns elapsed device milliseconds for all iterations.'''

@@ -101,13 +101,12 @@ class JaxprInterpreter:
             raise TypeError(f'Expected {len(self.input_buffers)} input arguments, received {len(leaves)}')
         return (leaves, resident) if with_residency else leaves
 
-    def run(self, *X, return_all=False):
-        '''Executes a previously recorded sequence with actual data'''
+    def _host_inputs(self, X) -> tp.List[tp.Optional[np.ndarray]]:
+        '''One entry per transfer slot: the device words of every argument that has to be copied.'''
         X, resident = self._flatten_args(X, with_residency=True)
         if self.sequence is None:
             raise RuntimeError('this interpreter was built with plan_only=True and has no device to run on')
         host = [None] * self.sequence.n_slots
-        keep = []
         for k, (slot, x, var) in enumerate(zip(self._input_slots, X, self.jaxpr.jaxpr.invars)):
             if slot is None:
                 continue
@@ -115,27 +114,53 @@ class JaxprInterpreter:
                 if self._resident_leaves.get(k) is x:
                     continue                                    #already in HBM
                 self._resident_leaves[k] = x
-            words = _device_words_of_argument(x, var.aval)
-            host[slot] = words
-            keep.append(words)
+            host[slot] = _device_words_of_argument(x, var.aval)
+        return host
+
+    def _fresh_outputs(self, host) -> tp.List[tp.Optional[np.ndarray]]:
         #every call hands out fresh arrays: the runtime copies the results straight into them
         fresh = [np.empty(n, np.uint32) if n is not None else None for n in self._output_sizes]
         for slot, arr in zip(self._output_slots, fresh):
             if slot is not None:
                 host[slot] = arr
-        self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT if self.resident_argnums else 0)
+        return fresh
 
-        output_values = []
-        for b, arr in zip(self.output_buffers, fresh):
-            if b is None:
-                output_values.append(None)
-                continue
-            output_values.append(view_or_convert_from_32bit(arr, b.dtype).reshape(b.shape))
-        output_values = tuple(output_values)
+    def _output_values(self, fresh) -> tp.Tuple:
+        return tuple(None if b is None else view_or_convert_from_32bit(arr, b.dtype).reshape(b.shape)
+                     for b, arr in zip(self.output_buffers, fresh))
+
+    def run(self, *X, return_all=False):
+        '''Executes a previously recorded sequence with actual data'''
+        host  = self._host_inputs(X)
+        fresh = self._fresh_outputs(host)
+        self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT if self.resident_argnums else 0)
+        output_values = self._output_values(fresh)
         if not return_all:
             return output_values
         all_arrays = [(var, buf.numpy() if buf is not None else None) for var, buf in self.bufferpool.buffers.items()]
         return output_values, dict(all_arrays)
+
+    def run_stream(self, argument_tuples: tp.Iterable[tp.Tuple]):
+        '''Runs the sequence on one tuple of arguments after the other and yields each result in
+        turn. While the device works on one tuple, the next one is taken from the iterable, staged
+        and uploaded, so that in the steady state a call costs the longer of the two instead of
+        their sum (the reference copies, runs and reads back strictly in turn,
+        vkjax/kompute_jaxpr_interpreter.py:72-81).'''
+        end      = object()
+        iterator = iter(argument_tuples)
+        current  = next(iterator, end)
+        if current is end:
+            return
+        host = self._host_inputs(tuple(current))
+        while True:
+            following = next(iterator, end)
+            next_host = self._host_inputs(tuple(following)) if following is not end else None
+            fresh     = self._fresh_outputs(host)
+            self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT, next_host_arrays=next_host)
+            yield self._output_values(fresh)
+            if following is end:
+                return
+            host = [None] * self.sequence.n_slots                #everything is in place already
 
     def upload_inputs(self, *X):
         '''Copy arguments into their HBM buffers without running (for measurements with resident inputs).'''

@@ -7,22 +7,25 @@ import typing as tp
 
 class TreeDef:
     '''Hashable description of a container nest; leaves are `*`.'''
-    __slots__ = ('kind', 'meta', 'children', 'num_leaves')
+    __slots__ = ('kind', 'meta', 'children', 'num_leaves', '_hash')
 
     def __init__(self, kind, meta, children):
         self.kind       = kind       #'leaf' | 'none' | 'tuple' | 'list' | 'dict'
         self.meta       = meta       #dict keys (sorted) for 'dict'
         self.children   = tuple(children)
         self.num_leaves = 1 if kind == 'leaf' else sum(c.num_leaves for c in self.children)
+        self._hash      = hash((kind, meta, tuple(c._hash for c in self.children)))   #children are hashed once
 
     def _key(self):
         return (self.kind, self.meta, self.children)
 
     def __eq__(self, other):
-        return isinstance(other, TreeDef) and self._key() == other._key()
+        if self is other:
+            return True
+        return isinstance(other, TreeDef) and self._hash == other._hash and self._key() == other._key()
 
     def __hash__(self):
-        return hash(self._key())
+        return self._hash
 
     def __repr__(self):
         if self.kind == 'leaf':
@@ -33,6 +36,9 @@ class TreeDef:
             return '{' + ', '.join(f'{k!r}: {c!r}' for k, c in zip(self.meta, self.children)) + '}'
         inner = ', '.join(map(repr, self.children))
         return f'({inner})' if self.kind == 'tuple' else f'[{inner}]'
+
+
+_LEAF = TreeDef('leaf', None, ())
 
 
 def tree_flatten(tree) -> tp.Tuple[list, TreeDef]:
@@ -49,7 +55,7 @@ def tree_flatten(tree) -> tp.Tuple[list, TreeDef]:
             keys = tuple(sorted(x.keys()))
             return TreeDef('dict', keys, [rec(x[k]) for k in keys])
         leaves.append(x)
-        return TreeDef('leaf', None, ())
+        return _LEAF
 
     treedef = rec(tree)
     return leaves, treedef
