@@ -35,7 +35,7 @@ BATCHED = ('resnet50', 'mlp', 'conv_block', 'mlp_train', 'convnet_train', 'resne
 
 def kernel_family(name: str) -> str:
     for prefix in ('conv_gemm', 'wgrad_gemm', 'softmax_rows', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows',
-                   'select_window', 'scatter_selected', 'pad_nd'):
+                   'select_window', 'scatter_selected', 'pad_nd', 'scale_relu_backward', 'scale_backward', 'transpose_tiled'):
         if name.startswith(prefix):
             return prefix
     return name

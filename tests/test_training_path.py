@@ -8,8 +8,8 @@ import pytest
 
 from oracle import primitives as P
 from oracle.eval_jaxpr import eval_closed_jaxpr
-from tests.common import check_against_oracle
-from vkjax_amd import minijax as mj, workloads as W
+from tests.common import check_against_oracle, assert_tree_close
+from vkjax_amd import kernels as K, minijax as mj, workloads as W
 from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
 
 lax, jnp, nn = mj.lax, mj.numpy, mj.nn
@@ -309,3 +309,69 @@ def test_repeated_training_steps_reduce_the_loss():
         loss, params = step(params, x, onehot)
         losses.append(float(loss))
     assert losses[-1] < 0.7 * losses[0], losses
+
+
+def _scale_shift_relu_net(batch=6, size=10, channels=(8, 12, 12), seed=3):
+    '''Three layers of 1x1 convolution -> per-channel scale and shift -> ReLU with a residual connection around
+    the last one, and a squared-error loss: the shapes of a batch norm with fixed statistics in a residual block.'''
+    rng = np.random.default_rng(seed)
+    params = []
+    cin = 4
+    for c in channels:
+        params.append({'w': (rng.standard_normal((1, 1, cin, c)) / np.sqrt(cin)).astype(np.float32),
+                       'scale': (1 + 0.1 * rng.standard_normal(c)).astype(np.float32), 'bias': (0.1 * rng.standard_normal(c)).astype(np.float32),
+                       'mean': (0.1 * rng.standard_normal(c)).astype(np.float32), 'var': (1 + 0.1 * rng.random(c)).astype(np.float32)})
+        cin = c
+    x = rng.standard_normal((batch, size, size, 4)).astype(np.float32)
+    return params, x
+
+
+def _scale_shift_relu_loss(trainable, fixed, x):
+    h = x
+    for k, (p, s) in enumerate(zip(trainable, fixed)):
+        y = mj.lax.conv_general_dilated(h, p['w'], (1, 1), 'VALID', dimension_numbers=('NHWC', 'HWIO', 'NHWC'))
+        y = (y - s['mean']) * (p['scale'] * mj.lax.rsqrt(s['var'] + 1e-5)) + p['bias']
+        h = mj.nn.relu(y + h) if k == 2 else mj.nn.relu(y)
+    return mj.numpy.sum(h * h)
+
+
+def _scale_shift_relu_step(params, x):
+    trainable = [{k: p[k] for k in ('w', 'scale', 'bias')} for p in params]
+    fixed     = [{k: p[k] for k in ('mean', 'var')} for p in params]
+    loss, grads = mj.value_and_grad(_scale_shift_relu_loss)(trainable, fixed, x)
+    new = [{k: p[k] - np.float32(0.01) * g[k] for k in p} for p, g in zip(trainable, grads)]
+    return loss, new
+
+
+def test_scale_relu_backward_and_small_chain_batches_are_planned():
+    import vkjax_amd
+    f = vkjax_amd.wrap(_scale_shift_relu_step, frontend='minijax', plan_only=True)
+    interp, _ = f._get_or_create_jaxpr_interpreter(_scale_shift_relu_net())
+    kernels = [l.kernel for l in interp.launches]
+    assert sum(k.startswith('scale_relu_backward') for k in kernels) == 2, kernels       #the two plain layers
+    assert sum(k.startswith('scale_backward') for k in kernels) == 1, kernels            #the one whose cotangent the shortcut shares
+    assert any(k.startswith('ew_chain_batch') for k in kernels), kernels
+    plain = vkjax_amd.wrap(_scale_shift_relu_step, frontend='minijax', plan_only=True, fuse=False)
+    unfused, _ = plain._get_or_create_jaxpr_interpreter(_scale_shift_relu_net())
+    assert len(kernels) < len(unfused.launches) - 20
+    #the table of a batch launch: one 432-byte entry per member, first workgroups ascending from 0
+    batch = next(l for l in interp.launches if l.members)
+    table = K.ew_batch_table(batch, lambda b: 0x1000)
+    assert table.nbytes == 432 * len(batch.members)
+    firsts = table.reshape(len(batch.members), 108)[:, 0]
+    assert firsts[0] == 0 and list(firsts) == list(np.cumsum([0] + [m.grid[0] for m in batch.members[:-1]]))
+    assert batch.grid[0] == sum(m.grid[0] for m in batch.members)
+
+
+@pytest.mark.gpu
+def test_scale_relu_backward_and_small_chain_batches_keep_every_bit():
+    '''The fused backward pass of scale/shift/ReLU adds in the order of the column sums it replaces, and batching
+    small chains only changes which launch evaluates them: the step's results equal the unfused ones exactly,
+    and both are within tolerance of the oracle. Second size: columns not a multiple of four (the v1 kernels).'''
+    import vkjax_amd
+    for kwargs in (dict(), dict(batch=3, size=7, channels=(6, 10, 10), seed=8)):
+        args = _scale_shift_relu_net(**kwargs)
+        fused   = vkjax_amd.wrap(_scale_shift_relu_step, frontend='minijax')(*args)
+        unfused = vkjax_amd.wrap(_scale_shift_relu_step, frontend='minijax', fuse=False)(*args)
+        assert_tree_close(fused, unfused, exact=True, what=f'fused against unfused {kwargs}')
+        check_against_oracle(_scale_shift_relu_step, args, rtol=1e-4, atol=1e-5)

@@ -35,12 +35,13 @@ struct EwParams {
 // the top of the kernel so that the scalar loads of the argument block are issued together and
 // waited for once, instead of one round trip per operand slot further down. The 8-slot
 // instantiation would run out of scalar registers and leaves its arguments to be fetched on demand.
-#define EW_PIN(x) do { if constexpr (NS <= 6) asm volatile("" : "+s"(x)); } while (0)
+#define EW_PIN(x) do { if constexpr (PIN && NS <= 6) asm volatile("" : "+s"(x)); } while (0)
 
 // NS = number of step slots this instantiation looks at (the chain has at most NS steps).
-template <int VEC, int NS>
+// `block` is the index of this workgroup within the chain's own grid.
+template <int VEC, int NS, bool PIN = true>
 __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const uint32_t* const (&in)[EW_MAX_STEPS],
-                                              const EwParams& P) {
+                                              const EwParams& P, const uint32_t block) {
     uint32_t n = P.n, ndim = P.ndim, nsteps = P.nsteps;
     uint32_t dims[4], op[NS], flags[NS], imm[NS], nbytes[NS], base[NS];
     int32_t  stride[NS][4];
@@ -56,7 +57,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     for (int k = 0; k < NS; ++k) {
         flags[k] = P.flags[k]; nbytes[k] = P.nbytes[k]; base[k] = P.base[k];
         EW_PIN(flags[k]); EW_PIN(nbytes[k]); EW_PIN(base[k]);
-        if constexpr (NS <= 6) asm volatile("" :: "s"(in[k]));
+        if constexpr (PIN && NS <= 6) asm volatile("" :: "s"(in[k]));
 #pragma unroll
         for (int d = 0; d < 4; ++d) { stride[k][d] = P.stride[k][d]; EW_PIN(stride[k][d]); }
     }
@@ -66,7 +67,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     // CU has in flight do not cover the memory latency once a chain has several operands.
     constexpr int U = (NS == 4 || NS == 6) ? 2 : 1;
     constexpr int W = U * VEC;                                    // values per thread
-    const uint32_t first = (blockIdx.x * U * 256u + threadIdx.x) * VEC;     // the host keeps n below 2^31
+    const uint32_t first = (block * U * 256u + threadIdx.x) * VEC;          // the host keeps n below 2^31
     if (first >= n) return;
 
     // Every operand is read through a buffer descriptor with one branch-free load per slot: 16 bytes
@@ -174,7 +175,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
         const uint32_t* in3, const uint32_t* in4, const uint32_t* in5, const uint32_t* in6,             \
         const uint32_t* in7, EwParams P) {                                                              \
         const uint32_t* const in[EW_MAX_STEPS] = {in0, in1, in2, in3, in4, in5, in6, in7};              \
-        ew_chain_body<VEC, NS>(out, in, P);                                                             \
+        ew_chain_body<VEC, NS>(out, in, P, blockIdx.x);                                                 \
     }
 
 // ew_chain_v4* requires: n % 4 == 0, dims[ndim-1] % 4 == 0, every operand's fastest stride in {0, 1},
@@ -188,6 +189,41 @@ EW_KERNEL(ew_chain_v4_s2, 4, 2)
 EW_KERNEL(ew_chain_v4_s4, 4, 4)
 EW_KERNEL(ew_chain_v4_s6, 4, 6)
 EW_KERNEL(ew_chain_v4_s8, 4, 8)
+
+// Several small, mutually independent chains in ONE launch: a program with many little vectors
+// (per-channel statistics, parameter updates) otherwise pays one launch latency for each of them.
+// The host writes one entry per chain into a table in device memory; workgroup b belongs to the
+// last entry whose first_block is <= b and evaluates that entry's chain as block b - first_block
+// of the chain's own grid. Entries are sorted by first_block, entry 0 starts at block 0.
+struct EwBatchEntry {
+    uint32_t        first_block, pad0;
+    uint32_t*       out;
+    const uint32_t* in[EW_MAX_STEPS];
+    EwParams        P;
+    uint32_t        pad1;
+};
+static_assert(sizeof(EwBatchEntry) == 432, "the host lays the table out with 432-byte entries");
+
+template <int VEC, int NS>
+__device__ __forceinline__ void ew_batch_body(const EwBatchEntry* __restrict__ table, uint32_t entries) {
+    uint32_t lo = 0, hi = entries;
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (table[mid].first_block <= blockIdx.x) lo = mid; else hi = mid;
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    const EwBatchEntry& e = table[lo];
+    ew_chain_body<VEC, NS, false>(e.out, e.in, e.P, blockIdx.x - e.first_block);
+}
+
+#define EW_BATCH_KERNEL(name, VEC, NS)                                                                \
+    extern "C" __global__ __launch_bounds__(256) void name(const EwBatchEntry* __restrict__ table, uint32_t entries) { \
+        ew_batch_body<VEC, NS>(table, entries);                                                         \
+    }
+EW_BATCH_KERNEL(ew_chain_batch_v1_s2, 1, 2)
+EW_BATCH_KERNEL(ew_chain_batch_v1_s4, 1, 4)
+EW_BATCH_KERNEL(ew_chain_batch_v4_s2, 4, 2)
+EW_BATCH_KERNEL(ew_chain_batch_v4_s4, 4, 4)
 
 struct IotaParams { uint32_t n, inner, size, to_float; };
 

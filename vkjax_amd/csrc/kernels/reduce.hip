@@ -267,6 +267,117 @@ REDUCE_KERNELS(fargmax, 3)
 REDUCE_KERNELS(fargmin, 4)
 
 // ---------------------------------------------------------------------------------------------
+// Backward pass of  y = max(x * k + b, 0)  (a per-channel scale and shift followed by ReLU, k and b
+// vectors over the fastest dimension) in one pass over the arrays. Autodiff spells it
+//     m  = ans > t ? g : z          (t, z single values; ans the forward result, g its cotangent)
+//     db = sum over rows of m       dk = sum over rows of m * x       dx = m * k
+// as two element-wise launches, two more that only feed the column sums, and the two sums: nine
+// passes over arrays of the activation's size. Here every element of ans, g and x is read once, dx
+// written once, and both sums accumulated on the way: four passes. The sums run over exactly the
+// rows, in exactly the order, of reduce_cols_body with the same ReduceParams (per-thread running
+// sums over rows r_lo + tr, + TR, ..., then the same tree over tr in LDS), so sum_m and sum_mx hold
+// the bits the separate launches would have produced, partial results per row range included.
+// SELECT = false: m is g itself (no activation between the scale and what follows; ans, thr and alt unused).
+template <int VEC, bool SELECT>
+__device__ __forceinline__ void scale_relu_backward_body(float* __restrict__ dx, float* __restrict__ sum_m, float* __restrict__ sum_mx,
+                                                         const float* __restrict__ ans, const float* __restrict__ thr,
+                                                         const float* __restrict__ g, const float* __restrict__ alt,
+                                                         const float* __restrict__ x, const float* __restrict__ kvec,
+                                                         const ReduceParams& P) {
+    __shared__ float s_m[256 * VEC];
+    __shared__ float s_x[256 * VEC];
+    const uint32_t TI = P.TI, TR = 256u / TI;
+    const uint32_t tid = threadIdx.x, ti = tid % TI, tr = tid / TI;
+    const uint32_t tiles_i = (P.inner + TI * VEC - 1u) / (TI * VEC);
+    const uint32_t it = blockIdx.x % tiles_i, rest = blockIdx.x / tiles_i;
+    const uint32_t sp = rest % P.nsplit, o = rest / P.nsplit;
+    const uint32_t i = (it * TI + ti) * VEC;
+    const uint32_t r_lo = sp * P.r_chunk, r_hi = min(P.R, r_lo + P.r_chunk);
+    float acc_m[VEC], acc_x[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { acc_m[j] = 0.f; acc_x[j] = 0.f; }
+    if (i < P.inner) {                                                // inner is a multiple of VEC
+        const float t = SELECT ? thr[0] : 0.f, z = SELECT ? alt[0] : 0.f;
+        const uint64_t base = (uint64_t)o * P.R * P.inner + i;
+        float kv[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) kv[j] = kvec[i + j];
+        auto fetch = [&](uint32_t row, float (&a)[VEC], float (&c)[VEC], float (&v)[VEC]) {
+            const uint64_t off = base + (uint64_t)row * P.inner;
+            if constexpr (VEC == 4) {
+                const f32x4 tc = *reinterpret_cast<const f32x4*>(g + off), tv = *reinterpret_cast<const f32x4*>(x + off);
+                c[0] = tc.x; c[1] = tc.y; c[2] = tc.z; c[3] = tc.w;
+                v[0] = tv.x; v[1] = tv.y; v[2] = tv.z; v[3] = tv.w;
+                if constexpr (SELECT) {
+                    const f32x4 ta = *reinterpret_cast<const f32x4*>(ans + off);
+                    a[0] = ta.x; a[1] = ta.y; a[2] = ta.z; a[3] = ta.w;
+                }
+            } else {
+                c[0] = g[off]; v[0] = x[off];
+                if constexpr (SELECT) a[0] = ans[off];
+            }
+        };
+        auto take = [&](uint32_t row, const float (&a)[VEC], const float (&c)[VEC], const float (&v)[VEC]) {
+            float m[VEC], d[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                m[j] = SELECT ? (a[j] > t ? c[j] : z) : c[j];
+                d[j] = m[j] * kv[j];
+                acc_m[j] = acc_m[j] + m[j];
+                acc_x[j] = acc_x[j] + m[j] * v[j];
+            }
+            const uint64_t off = base + (uint64_t)row * P.inner;
+            if constexpr (VEC == 4) *reinterpret_cast<f32x4*>(dx + off) = f32x4{d[0], d[1], d[2], d[3]};
+            else dx[off] = d[0];
+        };
+        uint32_t r = r_lo + tr;
+        for (; r + 3u * TR < r_hi; r += 4u * TR) {                    // four rows in flight per thread
+            float a[4][VEC], c[4][VEC], v[4][VEC];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) fetch(r + q * TR, a[q], c[q], v[q]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) take(r + q * TR, a[q], c[q], v[q]);
+        }
+        for (; r < r_hi; r += TR) {
+            float a[VEC], c[VEC], v[VEC];
+            fetch(r, a, c, v);
+            take(r, a, c, v);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { s_m[tid * VEC + j] = acc_m[j]; s_x[tid * VEC + j] = acc_x[j]; }
+    __syncthreads();
+    for (uint32_t s = TR >> 1; s >= 1; s >>= 1) {
+        if (tr < s) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const uint32_t mine = tid * VEC + j, other = (tid + s * TI) * VEC + j;
+                s_m[mine] = s_m[mine] + s_m[other];
+                s_x[mine] = s_x[mine] + s_x[other];
+            }
+        }
+        __syncthreads();
+    }
+    if (tr == 0 && i < P.inner) {
+        const uint64_t dst = ((uint64_t)o * P.nsplit + sp) * P.inner + i;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) { sum_m[dst + j] = s_m[tid * VEC + j]; sum_mx[dst + j] = s_x[tid * VEC + j]; }
+    }
+}
+
+#define SCALE_RELU_BACKWARD_KERNEL(name, VEC, SELECT)                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void name(float* dx, float* sum_m, float* sum_mx, const float* ans,   \
+                                                           const float* thr, const float* g, const float* alt,        \
+                                                           const float* x, const float* kvec, ReduceParams P) {       \
+        scale_relu_backward_body<VEC, SELECT>(dx, sum_m, sum_mx, ans, thr, g, alt, x, kvec, P);                              \
+    }
+// _v4 needs inner % 4 == 0 and 16-byte aligned arrays
+SCALE_RELU_BACKWARD_KERNEL(scale_relu_backward_v1, 1, true)
+SCALE_RELU_BACKWARD_KERNEL(scale_relu_backward_v4, 4, true)
+SCALE_RELU_BACKWARD_KERNEL(scale_backward_v1, 1, false)
+SCALE_RELU_BACKWARD_KERNEL(scale_backward_v4, 4, false)
+
+// ---------------------------------------------------------------------------------------------
 // softmax over the rows of [outer, R] in one launch: out = exp(x - max(x)) / sum(exp(x - max(x))).
 // Takes the place of reduce_max -> (subtract, exp) -> reduce_sum -> divide. One wave per row; the
 // sum is accumulated in exactly the order reduce_rows uses (per-lane partial sums over the same

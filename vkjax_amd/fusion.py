@@ -208,9 +208,11 @@ def fuse_ops(all_ops, bufferpool, outvars):
     ops = fuse_random_streams([op for op in result if op is not None], bufferpool, outvars)
     ops = fuse_stream_chains(ops, bufferpool, outvars)
     ops = fuse_softmax(ops, bufferpool, outvars)
+    ops = fuse_scale_relu_backward(ops, bufferpool, outvars)
     ops = fuse_reduce_prologues(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
-    return remove_dead_ops(ops, bufferpool, outvars)
+    ops = remove_dead_ops(ops, bufferpool, outvars)
+    return batch_small_chains(ops)
 
 
 def fuse_softmax(ops, bufferpool, outvars):
@@ -313,6 +315,113 @@ def fuse_reduce_prologues(ops, bufferpool, outvars):
         ch.out._placeholder.elided = True
         removed.add(w)
         replacement[i] = fused
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
+
+
+def fuse_scale_relu_backward(ops, bufferpool, outvars):
+    '''The backward pass of a per-channel scale and shift followed by ReLU (a batch norm with fixed statistics
+    and its activation), as reverse-mode differentiation emits it:
+
+        m = select(ans > t, g, z) ; db = sum_rows(m) ; dx = m * k ; p = m * x ; dk = sum_rows(p)
+
+    with m read by nothing else and p only by its sum, becomes ONE launch that reads ans, g and x once and
+    writes dx and both column sums (their first stage, when the sums are split over row ranges). The sums are
+    taken in the order of the reduce_cols launches they replace, so every value keeps its bits.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    last_writer: tp.Dict[int, int] = {}
+    for i, op in enumerate(ops):
+        for b in _may_write(op):
+            last_writer[pid(b)] = i
+    readers: tp.Dict[int, tp.List[int]] = {}
+    for i, op in enumerate(ops):
+        for b in _reads(op):
+            readers.setdefault(pid(b), []).append(i)
+    single = lambda o: o is not None and all(st == 0 for st in o.strides)
+    removed, replacement = set(), {}
+
+    def column_sum_of(i, buffer):
+        '''(rows, inner, nsplit) when ops[i] is the float sum over the rows of `buffer` seen as [rows, inner].'''
+        R = ops[i]
+        if R.meta is None or R.meta[0] != 'reduce':
+            return None
+        _, out, inp, outer, rows, inner, name, partial, nsplit = R.meta
+        if (name != 'reduce_sum' or outer != 1 or inner <= 1 or inp.dtype != 'float32' or inp._placeholder is not buffer._placeholder
+                or rows * inner != buffer.size or not R.launch.kernel.startswith('reduce_cols_fsum_v')):
+            return None
+        return rows, inner, nsplit
+
+    def select_chain(op):
+        ch = op.chain
+        return (ch is not None and [st.op for st in ch.steps] == [EW['GT_F'], EW['SEL_P'], EW['NOP']] and not ch.steps[0].operand_left
+                and single(ch.steps[0].operand) and single(ch.steps[2].operand)
+                and _is_full_contiguous_any_shape(ch.first, ch.shape) and _is_full_contiguous_any_shape(ch.steps[1].operand, ch.shape)
+                and ch.out.dtype == 'float32' and ch.first.buffer.dtype == 'float32')
+
+    chain_writer = {pid(op.chain.out): i for i, op in enumerate(ops) if op.chain is not None}
+    for R1, first_sum in enumerate(ops):
+        if first_sum.meta is None or first_sum.meta[0] != 'reduce':
+            continue
+        m = first_sum.meta[2]
+        geometry = column_sum_of(R1, m)
+        if geometry is None:
+            continue
+        rows, inner, nsplit = geometry
+        C, P = None, None
+        #several such backward passes can share one m (two branches of a residual block): each sum
+        #goes with the first scaling and the first product that follow it
+        for r in sorted(readers.get(pid(m), [])):
+            other = ops[r].chain
+            if r < R1 or other is None or [st.op for st in other.steps] != [EW['MUL_F']] or other.shape[-1] != inner or other.out.size != m.size:
+                continue
+            a, b = other.first, other.steps[0].operand
+            if b is not None and a.buffer._placeholder is not m._placeholder:
+                a, b = b, a
+            if b is None or a.buffer._placeholder is not m._placeholder or not _is_full_contiguous_any_shape(a, other.shape):
+                continue
+            if _is_full_contiguous_any_shape(b, other.shape) and b.buffer.dtype == 'float32':
+                P = P or (r, b.buffer)
+            elif (b.offset == 0 and b.buffer.size == inner and b.buffer.dtype == 'float32'
+                  and tuple(b.strides) == (0,) * (len(other.shape) - 1) + (1,)):
+                C = C or (r, b.buffer)
+        if C is None or P is None or C[0] == P[0]:
+            continue
+        p_out = ops[P[0]].chain.out
+        R2 = [r for r in readers.get(pid(p_out), []) if column_sum_of(r, p_out) is not None]
+        if uses[pid(p_out)] != 1 or len(R2) != 1 or column_sum_of(R2[0], p_out) != geometry:
+            continue
+        R2 = R2[0]
+        if ops[R1].launch.kernel != ops[R2].launch.kernel or ops[R1].launch.params != ops[R2].launch.params:
+            continue
+        x, k = P[1], C[1]
+        # with the select: where the select stood, if the three launches above are all that read its result
+        M = chain_writer.get(pid(m))
+        with_select = M is not None and M < min(R1, C[0], P[0]) and select_chain(ops[M]) and uses[pid(m)] == 3
+        position = M if with_select else min(R1, C[0], P[0])
+        involved = [R1, C[0], P[0], R2] + ([M] if with_select else [])
+        if any(j in removed or j in replacement for j in involved):
+            continue
+        #everything the merged launch reads has to exist where the first of the launches it replaces stood
+        sources = [x, k] + ([o.buffer for o in ops[M].chain.operands()] if with_select else [m])
+        if any(last_writer.get(pid(b), -1) >= position for b in sources):
+            continue
+        dx, sum_m, sum_mx = ops[C[0]].chain.out, ops[R1].launch.buffers[0][0], ops[R2].launch.buffers[0][0]
+        if with_select:
+            ch = ops[M].chain
+            launch = K.scale_relu_backward(ops[R1].launch, dx, sum_m, sum_mx, x, k, ch.steps[1].operand.buffer,
+                                           select=(ch.first.buffer, ch.steps[0].operand.buffer, ch.steps[2].operand.buffer))
+            m._placeholder.elided = True
+        else:
+            launch = K.scale_relu_backward(ops[R1].launch, dx, sum_m, sum_mx, x, k, m)
+        fused = Op(_label(*[ops[j] for j in sorted(involved)]), launch=launch)
+        fused.index = ops[position].index
+        for b, _ in launch.buffers:
+            if b is not None:
+                b.accesses.append(fused.index)
+        p_out._placeholder.elided = True
+        removed |= set(involved) - {position}
+        replacement[position] = fused
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
 
 
@@ -597,3 +706,115 @@ def fuse_random_streams(ops, bufferpool, outvars):
                 removed.add(si)
                 S._placeholder.elided = True
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed or i in replacement]
+
+
+def _is_small_chain(op) -> bool:
+    return (op.chain is not None and op.launch.kernel in K.EW_BATCH_KERNELS
+            and op.launch.grid[0] <= K.EW_BATCH_MAX_BLOCKS)
+
+
+def _may_write(op) -> tp.List:
+    '''Buffers an op may change: its result where the op's structure is known, else everything it touches.'''
+    if op.chain is not None or op.conv is not None or (op.meta is not None and op.meta[0] in ('iota', 'concat_part', 'threefry', 'reduce')):
+        return _writes(op)
+    return [b for b, _ in op.launch.buffers if b is not None]
+
+
+def _touched(op) -> tp.List:
+    if op.chain is not None or op.conv is not None:
+        return _reads(op) + _writes(op)
+    return [b for b, _ in op.launch.buffers if b is not None]
+
+
+BATCH_MIN_GAIN = 4          #launches a program must save before its small chains are moved and batched
+
+
+def batch_small_chains(ops):
+    '''Programs with many little vectors (per-channel statistics, parameter updates of a training step)
+    spend most of their launches on element-wise chains of a few workgroups, each paying a full launch
+    latency. This pass
+
+    1. moves every such chain that depends only on program inputs (or on chains moved before it) to the
+       front, and every one whose result nothing but other moved chains reads to the end,
+    2. sorts each run of consecutive small chains into dependency levels (read-after-write, write-after-read
+       and write-after-write on the buffers) and turns every level's chains of one kernel variant into ONE
+       launch of ew_chain_batch_*, and
+    3. rebuilds the buffers' access positions from the final order, since storage is shared between
+       buffers by those positions.
+
+    Every chain computes what it computed before; only the order of independent launches changes.'''
+    from .ops import Op
+    pid = lambda b: id(b._placeholder)
+    small = [_is_small_chain(op) for op in ops]
+    if sum(small) < BATCH_MIN_GAIN + 1:
+        return ops
+
+    # 1a. to the front
+    written, touched, front = set(), set(), set()
+    for i, op in enumerate(ops):
+        if small[i] and not any(pid(b) in written for b in _reads(op)) and pid(_out(op)) not in touched:
+            front.add(i)
+            continue
+        written |= {pid(b) for b in _may_write(op)}
+        touched |= {pid(b) for b in _touched(op)}
+    # 1b. to the end
+    written, touched, back = set(), set(), set()
+    for i in reversed(range(len(ops))):
+        op = ops[i]
+        if i not in front and small[i] and pid(_out(op)) not in touched and not any(pid(b) in written for b in _reads(op)):
+            back.add(i)
+            continue
+        written |= {pid(b) for b in _may_write(op)}
+        touched |= {pid(b) for b in _touched(op)}
+    order = ([i for i in range(len(ops)) if i in front] + [i for i in range(len(ops)) if i not in front and i not in back]
+             + [i for i in range(len(ops)) if i in back])
+    moved = [ops[i] for i in order]
+
+    # 2. runs of small chains -> levels -> batches
+    result, saved, i = [], 0, 0
+    while i < len(moved):
+        if not _is_small_chain(moved[i]):
+            result.append(moved[i])
+            i += 1
+            continue
+        j = i
+        while j < len(moved) and _is_small_chain(moved[j]):
+            j += 1
+        run, level = moved[i:j], []
+        for k, op in enumerate(run):
+            reads, out = {pid(b) for b in _reads(op)}, pid(_out(op))
+            lv = 0
+            for q in range(k):
+                q_reads, q_out = {pid(b) for b in _reads(run[q])}, pid(_out(run[q]))
+                if q_out in reads or q_out == out or out in q_reads:
+                    lv = max(lv, level[q] + 1)
+            level.append(lv)
+        for lv in range(max(level) + 1):
+            by_kernel: tp.Dict[str, list] = {}
+            for k, op in enumerate(run):
+                if level[k] == lv:
+                    by_kernel.setdefault(op.launch.kernel, []).append(op)
+            for group in by_kernel.values():
+                if len(group) == 1:
+                    result.append(group[0])
+                    continue
+                batch = Op(_label(*group), launch=K.ew_chain_batch([op.launch for op in group]))
+                batch.index = min(op.index for op in group)
+                result.append(batch)
+                saved += len(group) - 1
+        i = j
+    if saved < BATCH_MIN_GAIN:
+        return ops
+
+    # 3. access positions of every buffer in the order the launches now have
+    fresh: tp.Dict[int, tp.Tuple[list, list]] = {}
+    for position, op in enumerate(result):
+        launches = op.launch.members or (op.launch,)
+        for launch in launches:
+            for b, _ in launch.buffers:
+                if b is not None:
+                    fresh.setdefault(id(b.accesses), (b.accesses, []))[1].append(position)
+        op.index = position
+    for accesses, positions in fresh.values():
+        accesses[:] = positions
+    return result

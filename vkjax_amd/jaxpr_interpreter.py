@@ -14,6 +14,7 @@ import numpy as np
 
 from . import fusion
 from . import hip
+from . import kernels as K
 from . import ops
 from .buffers import BufferPool, PlanOnlyDevice, to_device_words, view_or_convert_from_32bit
 from .minijax import core, tree_util
@@ -72,7 +73,14 @@ class JaxprInterpreter:
         self._input_slots = []
         for b in self.input_buffers:
             self._input_slots.append(self.sequence.record_upload(b.tensor, b.nbytes()) if b is not None else None)
+        self._batch_tables = []
         for op, launch in zip(self.all_ops, self.launches):
+            if launch.members:
+                #a batch of small launches reads its members' arguments from a table in HBM
+                table = self.mgr.tensor(K.ew_batch_table(launch, lambda b: b.tensor.device_ptr()))
+                self._batch_tables.append(table)
+                self.sequence.record_launch(launch.kernel, launch.grid, launch.block, [(table, 0)], launch.params, launch.lds)
+                continue
             bufs = [((b.tensor if b is not None else None), off) for b, off in launch.buffers]
             for (b, _), (t, _) in zip(launch.buffers, bufs):
                 assert b is None or t is not None, f'{op}: buffer without storage'

@@ -38,6 +38,9 @@ class Launch(tp.NamedTuple):
     #algorithmic work of this launch, for roofline accounting
     bytes_moved: int = 0
     flops:       int = 0
+    #a batch launch: the launches it evaluates, described to the kernel by a table in device memory
+    #that is written when the launch is recorded (it holds device addresses)
+    members: tp.Tuple['Launch', ...] = ()
 
 
 def _u32(*values) -> bytes:
@@ -194,6 +197,34 @@ def lower_ew_chain(chain: EwChain) -> Launch:
     per_thread = {2: 1, 4: 2, 6: 2, 8: 1}[slots]               #vectors a thread works on (the kernel's U)
     return Launch(f'ew_chain_v{vec}_s{slots}', (_cdiv(_cdiv(n, vec), BLOCK * per_thread), 1, 1), (BLOCK, 1, 1),
                   [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
+
+
+EW_BATCH_KERNELS     = ('ew_chain_v1_s2', 'ew_chain_v1_s4', 'ew_chain_v4_s2', 'ew_chain_v4_s4')
+EW_BATCH_ENTRY_BYTES = 432
+EW_BATCH_MAX_BLOCKS  = 16          #chains of more workgroups than this keep a launch of their own
+
+
+def ew_chain_batch(members: tp.Sequence[Launch]) -> Launch:
+    '''One launch for several small element-wise chains that do not depend on one another and lower
+    to the same kernel variant.'''
+    kernel = members[0].kernel
+    assert kernel in EW_BATCH_KERNELS and all(m.kernel == kernel and not m.members for m in members), [m.kernel for m in members]
+    return Launch(kernel.replace('ew_chain_', 'ew_chain_batch_'), (sum(m.grid[0] for m in members), 1, 1), (BLOCK, 1, 1), [],
+                  _u32(len(members)), bytes_moved=sum(m.bytes_moved for m in members), members=tuple(members))
+
+
+def ew_batch_table(launch: Launch, device_address: tp.Callable[[Buffer], int]) -> np.ndarray:
+    '''The table of a batch launch as uint32 words: per member {first workgroup, 0, address of the result,
+    addresses of the 8 operand slots (0 = none), the member's parameter block, 0}.'''
+    rows, first = [], 0
+    for m in launch.members:
+        assert len(m.buffers) == 1 + EW_MAX_STEPS and len(m.params) == EW_BATCH_ENTRY_BYTES - 8 - 8 * (1 + EW_MAX_STEPS) - 4
+        addresses = [device_address(b) + off if b is not None else 0 for b, off in m.buffers]
+        rows.append(_u32(first, 0) + np.asarray(addresses, dtype=np.uint64).tobytes() + m.params + _u32(0))
+        first += m.grid[0]
+    table = b''.join(rows)
+    assert len(table) == EW_BATCH_ENTRY_BYTES * len(launch.members)
+    return np.frombuffer(table, dtype=np.uint32).copy()
 
 
 def _as_tiled_transpose(chain: EwChain, dims, strides) -> tp.Optional[Launch]:
@@ -591,6 +622,23 @@ def reduce(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str,
     assert partial.size >= outer * nsplit * inner and partial.dtype == inp.dtype
     second = _reduce_launch(out, partial, outer, nsplit, inner, op, 1)[0]
     return [first, second]
+
+
+def scale_relu_backward(column_sum: Launch, dx: Buffer, sum_m: Buffer, sum_mx: Buffer, x: Buffer, scale: Buffer, cotangent: Buffer,
+                        select: tp.Optional[tp.Tuple[Buffer, Buffer, Buffer]] = None) -> Launch:
+    '''dx = m * scale (scale a vector over the columns), and sum_m, sum_mx receive what `column_sum`, a reduce_cols
+    launch over an array of that shape, would write for m and for m * x (same grid, same parameters, same order
+    of additions). m is the cotangent itself, or with select = (ans, threshold, otherwise), two single values:
+    ans > threshold ? cotangent : otherwise.'''
+    assert column_sum.kernel in ('reduce_cols_fsum_v1', 'reduce_cols_fsum_v4'), column_sum.kernel
+    n = cotangent.size
+    assert dx.size == x.size == n
+    ans, threshold, otherwise = select if select is not None else (None, None, None)
+    assert select is None or (ans.size == n and threshold.size == otherwise.size == 1)
+    name = 'scale_relu_backward_' if select is not None else 'scale_backward_'
+    return Launch(name + column_sum.kernel[-2:], column_sum.grid, column_sum.block,
+                  [(dx, 0), (sum_m, 0), (sum_mx, 0), (ans, 0), (threshold, 0), (cotangent, 0), (otherwise, 0), (x, 0), (scale, 0)],
+                  column_sum.params, bytes_moved=4 * ((4 if select is not None else 3) * n + 2 * scale.size))
 
 
 SOFTMAX_MAX_ROW = 4096      #rows this short run unsplit in reduce_rows, whose summation order softmax_rows repeats
