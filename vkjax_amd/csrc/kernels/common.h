@@ -38,3 +38,12 @@ __device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t 
 __device__ __forceinline__ int magic_div(int n, uint32_t magic, uint32_t shift) {
     return magic ? (int)(__umulhi((uint32_t)n, magic) >> shift) : n;
 }
+
+// Consecutive workgroup ids are handed to the 8 XCDs in turn, and every XCD has an L2 of its own.
+// This renumbers the workgroups of a 1-D grid so that each XCD works through a contiguous range:
+// kernels whose neighbouring workgroups read overlapping data (windows, halos) then find the
+// overlap in their own L2 instead of fetching it once per XCD. A bijection on [0, gridDim.x).
+__device__ __forceinline__ uint32_t xcd_contiguous_block() {
+    const uint32_t b = blockIdx.x, per = gridDim.x / 8u;
+    return (per > 0u && b < per * 8u) ? (b & 7u) * per + (b >> 3) : b;
+}

@@ -490,7 +490,7 @@ struct PoolParams {
 
 template <int VEC>
 __device__ __forceinline__ void pool_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const PoolParams& P) {
-    const uint64_t e0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * VEC;
+    const uint64_t e0 = ((uint64_t)xcd_contiguous_block() * 256u + threadIdx.x) * VEC;
     if (e0 >= P.n_out) return;
     uint32_t oc[4];
     {
@@ -544,7 +544,7 @@ __device__ __forceinline__ void pool_body(uint32_t* __restrict__ out, const uint
 // and fewer than 2^32 bytes on either side; the host checks.
 template <int KH, int KW>
 __device__ __forceinline__ void pool2d_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const PoolParams& P) {
-    const uint32_t e0 = (blockIdx.x * 256u + threadIdx.x) * 4u;
+    const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u;
     if (e0 >= P.n_out) return;
     const uint32_t C = P.out_dims[3], Wo = P.out_dims[2], Ho = P.out_dims[1];
     uint32_t r = e0 / C;
