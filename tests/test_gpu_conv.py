@@ -208,3 +208,39 @@ def test_four_waves_per_tile_kernel():
             assert [l.kernel for l in launches] in (['conv_gemm_32x32x128_ks4'], ['conv_gemm_32x32x128_ks4g']), [l.kernel for l in launches]
     finally:
         K.FORCE_CONV_KSPLIT = None
+
+
+def test_convolution_with_a_second_result():
+    '''A convolution result that is returned (or read later) AND continued by an element-wise chain: one launch
+    stores both, the value before the chain or after its `- vector` step and the chain's result. Integer-valued
+    data, so both are exact; lean and general kernel variants, an output tile that is not full, and a chain of
+    five steps with a residual operand.'''
+    from vkjax_amd import minijax as mj
+    lax, nn = mj.lax, mj.nn
+    dn = ('NHWC', 'HWIO', 'NHWC')
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+
+    def centred_and_activated(x, k, mean, scale, beta):
+        y = lax.conv_general_dilated(x, k, (1, 1), 'SAME', dimension_numbers=dn) - mean
+        return y, nn.relu(y * scale + beta)
+    def raw_and_activated(x, k, scale, beta):
+        y = lax.conv_general_dilated(x, k, (1, 1), 'SAME', dimension_numbers=dn)
+        return y, nn.relu(y * scale + beta)
+    def centred_residual(x, k, mean, scale, beta, res):
+        y = lax.conv_general_dilated(x, k, (2, 2), 'SAME', dimension_numbers=dn) - mean
+        return nn.relu(y * scale + beta + res), y
+
+    cases = [(centred_and_activated, [ints(-4, 5, 2, 9, 7, 64), ints(-3, 4, 3, 3, 64, 128), ints(-5, 5, 128), ints(1, 4, 128), ints(-9, 9, 128)]),
+             (centred_and_activated, [ints(-4, 5, 3, 6, 5, 12), ints(-3, 4, 1, 1, 12, 40), ints(-5, 5, 40), ints(1, 4, 40), ints(-9, 9, 40)]),
+             (centred_and_activated, [ints(-4, 5, 1, 8, 8, 3), ints(-3, 4, 3, 3, 3, 8), ints(-5, 5, 8), ints(1, 4, 8), ints(-9, 9, 8)]),
+             (raw_and_activated, [ints(-4, 5, 2, 9, 7, 64), ints(-3, 4, 1, 1, 64, 64), ints(1, 4, 64), ints(-9, 9, 64)]),
+             (centred_residual, [ints(-4, 5, 2, 10, 8, 32), ints(-3, 4, 3, 3, 32, 64), ints(-5, 5, 64), ints(1, 4, 64), ints(-9, 9, 64),
+                                 ints(-50, 50, 2, 5, 4, 64)])]
+    for f, args in cases:
+        print(f'second result: {f.__name__} {[a.shape for a in args]}', flush=True)
+        _, _, fn = check_against_oracle(f, args, exact=True)
+        launches = list(fn._jaxpr_interpreters.values())[0].launches
+        assert len(launches) == 1 and launches[0].kernel.startswith('conv_gemm'), [l.kernel for l in launches]
+        flags = int(np.frombuffer(launches[0].params, dtype=np.uint32)[21])
+        assert (flags >> 12) & 15 in (1, 2), hex(flags)
+        check_against_oracle(f, args, exact=True, fuse=False)

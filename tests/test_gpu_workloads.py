@@ -32,6 +32,12 @@ def test_resnet50_reduced_width():
     assert labels.dtype == np.int32
 
 
+def test_resnet50_reduced_width_single_image():
+    '''Batch of one (dimensions of size 1 in every activation).'''
+    args = W.resnet50_inputs(batch=1, size=64, num_classes=40, width_scale=0.25)
+    check_against_oracle(W.resnet50, args, rtol=1e-3, atol=1e-4)
+
+
 def test_resnet50_full_width_batch2():
     '''rtol 1e-3 on the logits. With random He-normal weights the logits reach several thousand while
     individual ones pass through zero, so the absolute floor is tied to their scale: 1e-5 of the

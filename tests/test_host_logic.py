@@ -321,3 +321,16 @@ def test_treedef_hash_and_equality():
     assert a == b and hash(a) == hash(b)
     assert a != c and a != d
     assert len({a, b, c, d}) == 3
+
+
+def test_batch_of_one_fuses_like_any_other():
+    '''Strides of dimensions of size 1 are never used; a leading batch dimension of 1 must not keep element-wise
+    chains from joining each other or a convolution's epilogue.'''
+    import vkjax_amd
+    from vkjax_amd import workloads as W
+    counts = []
+    for batch in (1, 2):
+        fn = vkjax_amd.wrap(W.resnet50, frontend='minijax', plan_only=True)
+        interp, _ = fn._get_or_create_jaxpr_interpreter(tuple(W.resnet50_inputs(batch=batch, size=64, num_classes=40, width_scale=0.25)))
+        counts.append(len(interp.launches))
+    assert counts[0] == counts[1] == 58, counts

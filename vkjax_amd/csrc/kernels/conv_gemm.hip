@@ -56,7 +56,10 @@ struct ConvParams {
     uint32_t flags;                 // bit0: out is row-major [M, N]; bit1: m is the row index itself
                                     // (batch = Wo = 1: no row decode); bit2: some kernel taps of some
                                     // rows fall outside the input; bits 8-11: number of epilogue
-                                    // steps; bits 16-19: 1 + index of the first kind-3 step, or 0;
+                                    // steps; bits 12-15: 0, or 1 + t: the value after t template steps
+                                    // (t = 0, or t = 1 after `acc - vector`) is ALSO stored, laid out like
+                                    // out, to the array the last epilogue pointer slot names;
+                                    // bits 16-19: 1 + index of the first kind-3 step, or 0;
                                     // bits 20-24: the steps are, in this order, a subset of
                                     // (acc - vector, * vector, + vector, + full tensor, max(acc, scalar)):
                                     // bit 20+k set = template step k is present;
@@ -560,6 +563,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
             // as straight-line code: every step is one pass over a sub-tile's 16 values, in place.
             const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u),
                       e_max = __builtin_popcount(slots & 15u);
+            const int tap = (int)((P.flags >> 12) & 15u) - 1;          // -1: no second result
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -571,11 +575,17 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
                     float ov[16];
                     if ((slots & 8u) && !(PREFETCH_FULL && first_full >= 0))
                         sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(f_rsrc, vo, so); });
+                    // a second result: the value as it stands before or after the first step
+#define CONV_TAP_STORE() sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) {                                   \
+                            buffer_store_x1(y[v], make_rsrc(epi.p[CONV_MAX_EPI - 1], P.out_bytes), vo, so); })
+                    if (tap == 0) CONV_TAP_STORE();
                     if (slots & 1u) {
                         const float o = Es[col];
 #pragma unroll
                         for (int v = 0; v < 16; ++v) y[v] = y[v] - o;
+                        if (tap == 1) CONV_TAP_STORE();
                     }
+#undef CONV_TAP_STORE
                     if (slots & 2u) {
                         const float o = Es[e_mul * BN + col];
 #pragma unroll

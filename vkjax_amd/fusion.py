@@ -38,7 +38,7 @@ def _reads(op) -> tp.List:
         return [o.buffer for o in op.chain.operands() if o is not None]
     if op.conv is not None:
         out, lhs, rhs, geom, epilogue = op.conv
-        reads = [lhs, rhs] + [e.operand for e in epilogue if e.operand is not None]
+        reads = [lhs, rhs] + [e.operand for e in epilogue if e.operand is not None and e.op != K.CONV_TAP]
         for e in epilogue:
             if e.derived is not None:
                 reads += [e.derived.first] + [st[1] for st in e.derived.steps if st[1] is not None]
@@ -63,9 +63,13 @@ def _out(op):
     return None
 
 
+def _walks_densely(strides, shape) -> bool:
+    '''The strides are the row-major ones of `shape`; the stride of a dimension of size 1 is never used and may be anything.'''
+    return len(strides) == len(shape) and all(n == 1 or s == r for s, r, n in zip(strides, K.row_major_strides(shape), shape))
+
+
 def _is_full_contiguous(operand: EwOperand, shape) -> bool:
-    return (operand.offset == 0 and tuple(operand.buffer.shape) == tuple(shape)
-            and tuple(operand.strides) == K.row_major_strides(shape))
+    return operand.offset == 0 and tuple(operand.buffer.shape) == tuple(shape) and _walks_densely(operand.strides, shape)
 
 
 def _label(*ops):
@@ -168,6 +172,22 @@ def fuse_ops(all_ops, bufferpool, outvars):
             return new
         return op
 
+    def conv_with_second_result(prod, op, pid):
+        out, lhs, rhs, geom, epilogue = prod.conv
+        steps = _continuation_steps(op.chain, out)
+        if steps is None or tuple(out.shape) != tuple(op.chain.shape) or op.chain.out.size != out.size:
+            return None
+        extra = _epilogue_steps(steps, geom, op.chain.shape)
+        if extra is None or not K.conv_tap_supported(epilogue, extra):
+            return None
+        tap = K.ConvEpilogueStep(K.CONV_TAP, 3, out)
+        fused = Op(_label(prod, op), conv=(op.chain.out, lhs, rhs, geom, list(epilogue) + [tap] + extra))
+        fused.index = op.index
+        extend_lifetimes(prod, op.index)
+        out.accesses.append(op.index)
+        uses[pid] -= 1
+        return fused
+
     for op in all_ops:
         fused = None
         if op.chain is not None:
@@ -175,9 +195,18 @@ def fuse_ops(all_ops, bufferpool, outvars):
             for cand in [o for o in op.chain.operands()[:2] if o is not None]:
                 pid = id(cand.buffer._placeholder)
                 pos = producer.get(pid)
-                if pos is None or uses[pid] != 1 or result[pos] is None:
+                if pos is None or result[pos] is None:
                     continue
                 prod = result[pos]
+                if uses[pid] != 1:
+                    #a convolution whose result something else reads as well can still take the chain over,
+                    #by storing both: its result as it was, and the chain's
+                    if prod.conv is not None and _out(prod)._placeholder is cand.buffer._placeholder:
+                        fused = conv_with_second_result(prod, op, pid)
+                        if fused is not None:
+                            result[pos] = None
+                            break
+                    continue
                 steps = _continuation_steps(op.chain, _out(prod))
                 if steps is None:
                     continue
@@ -192,6 +221,9 @@ def fuse_ops(all_ops, bufferpool, outvars):
                         continue
                     extra = _epilogue_steps(steps, geom, op.chain.shape)
                     if extra is None:
+                        continue
+                    tap_at = [k for k, e in enumerate(epilogue) if e.op == K.CONV_TAP]
+                    if tap_at and not K.conv_tap_supported(epilogue[:tap_at[0]], list(epilogue[tap_at[0] + 1:]) + extra):
                         continue
                     fused = Op(_label(prod, op), conv=(op.chain.out, lhs, rhs, geom, list(epilogue) + extra))
                 fused.index = op.index
@@ -430,7 +462,7 @@ def _is_full_contiguous_any_shape(operand: EwOperand, shape) -> bool:
     size = 1
     for d in shape:
         size *= d
-    return operand.offset == 0 and operand.buffer.size == size and tuple(operand.strides) == K.row_major_strides(shape)
+    return operand.offset == 0 and operand.buffer.size == size and _walks_densely(operand.strides, shape)
 
 
 def fuse_stream_chains(ops, bufferpool, outvars):
@@ -545,7 +577,9 @@ def fuse_derived_epilogue_operands(ops, bufferpool, outvars):
 
 
 def _writes(op) -> tp.List:
-    if op.chain is not None or op.conv is not None:
+    if op.conv is not None:
+        return [_out(op)] + [e.operand for e in op.conv[4] if e.op == K.CONV_TAP]
+    if op.chain is not None:
         return [_out(op)]
     if op.meta is not None and op.meta[0] in ('iota', 'concat_part'):
         return [op.meta[1]]

@@ -378,6 +378,21 @@ class ConvEpilogueStep(tp.NamedTuple):
     derived:      tp.Optional[ConvDerivedOperand] = None
 
 
+#A pseudo step: the value as it stands at this point of the epilogue is ALSO stored to `operand`, an array laid
+#out like the result (the centred convolution result a backward pass needs besides the activation)
+CONV_TAP = -1
+
+
+def conv_tap_supported(steps_before: tp.Sequence[ConvEpilogueStep], steps_after: tp.Sequence[ConvEpilogueStep]) -> bool:
+    '''The kernel stores a second result before the first step of its straight-line epilogue, or after that
+    epilogue's `acc - vector` step.'''
+    real = list(steps_before) + list(steps_after)
+    if any(e.op == CONV_TAP for e in real) or not real or len(real) > CONV_MAX_EPI - 1:
+        return False
+    slots = _epilogue_template_slots(real)
+    return slots != 0 and (len(steps_before) == 0 or (len(steps_before) == 1 and bool(slots & 1)))
+
+
 CONV_MAX_DERIVED = 3
 CONV_DERIVED_OPS = ('ADD_F', 'SUB_F', 'MUL_F', 'DIV_F', 'MAX_F', 'MIN_F', 'NEG_F', 'RSQRT_F', 'SQRT_F')
 
@@ -480,6 +495,12 @@ def _magic_division(d: int) -> tp.Tuple[int, int]:
 
 def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: tp.Sequence[ConvEpilogueStep] = (),
               compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0, out_offset: int = 0) -> Launch:
+    taps = [(i, e.operand) for i, e in enumerate(epilogue) if e.op == CONV_TAP]
+    if taps:
+        (tap_position, tap_buffer), = taps
+        epilogue = [e for e in epilogue if e.op != CONV_TAP]
+        if (not conv_tap_supported(epilogue[:tap_position], epilogue[tap_position:]) or out_offset or tap_buffer.size != out.size):
+            raise ValueError('a second result at this point of the epilogue is not supported')
     if len(epilogue) > CONV_MAX_EPI:
         raise ValueError('too many epilogue steps')
     g = _flatten_pointwise(g)
@@ -522,7 +543,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     w_bytes = K * N * 4 if b_fast else (rhs.size - rhs_offset) * 4
     first_full = kinds.index(3) + 1 if 3 in kinds else 0
     flags = (int(c_contig) | int(flat_rows) << 1 | int(needs_masks) << 2 | len(epilogue) << 8 | first_full << 16
-             | slots << 20 | chunk << 25)
+             | slots << 20 | chunk << 25 | ((tap_position + 1) << 12 if taps else 0))
     descs = [0, 0]
     for i, e in enumerate(epilogue):
         assert e.op < 128 and 1 <= e.kind <= 3
@@ -544,9 +565,14 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
                                 *_pad([int(st[2]) for st in d.steps], CONV_MAX_DERIVED))
     params += derived_desc
     buffers = [(out, out_offset * 4), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
-    buffers += _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0)) + derived_ptrs
+    operand_slots = _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
+    if taps:
+        assert operand_slots[-1] == (None, 0)
+        operand_slots[-1] = (tap_buffer, 0)
+    buffers += operand_slots + derived_ptrs
     kernel  = f'conv_gemm_{tag}x{bk}_' + (('ks4' if b_fast else 'ks4g') if ksplit else 'lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
+    nbytes += 4 * tap_buffer.size if taps else 0
     return Launch(kernel, (_cdiv(tiles_m, chunk) * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
                   bytes_moved=nbytes, flops=2 * M * N * K)
 
