@@ -288,13 +288,20 @@ def test_tiled_transposes():
              (lambda x: lax.transpose(x, (0, 3, 1, 2)), [random([3, 17, 19, 24])]),
              (lambda x: lax.transpose(x, (0, 2, 3, 1)), [random([3, 24, 17, 19])]),
              (lambda x: lax.transpose(x[3:, 5:70], (1, 0)), [random([40, 100])]),
-             (lambda x: lax.transpose(x, (1, 0)) * 2.0, [random([300, 200])])]
+             (lambda x: lax.transpose(x, (1, 0)) * 2.0, [random([300, 200])]),
+             #copies of copies are composed into one launch; a reversed leading dimension is a negative stride
+             (lambda x: lax.transpose(lax.rev(x, (0, 1)), (0, 1, 3, 2)), [random([3, 3, 64, 128])]),
+             (lambda x: lax.transpose(lax.rev(x, (0,)), (0, 2, 1)), [random([5, 33, 70])]),
+             (lambda x: lax.transpose(lax.rev(x, (0, 1)), (0, 1, 3, 2)), [random([1, 1, 256, 64])]),
+             (lambda x: lax.transpose(lax.transpose(x, (1, 0, 2)), (0, 2, 1)), [random([6, 5, 40])[:, :, 4:36]])]
     for k, (f, args) in enumerate(cases):
         print(f'case: tiled transpose {k}', flush=True)
         _, _, fn = check_against_oracle(f, args, exact=True)
         kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
-        if k != 9:
+        if k not in (9, 13):
             assert any(name.startswith('transpose_tiled') for name in kernels), kernels
+        if k in (10, 11, 12, 13):
+            assert len(kernels) == 1, kernels
 
 
 def test_nextafter_direction():

@@ -329,14 +329,14 @@ extern "C" __global__ __launch_bounds__(256) void pad_nd_v4(uint32_t* __restrict
 // [B, I, J]. The strided gather of the element-wise kernel touches a new cache line per element on
 // one side; here a 64 x 64 tile goes through LDS, read along i (contiguous in `in`) and written
 // along j (contiguous in `out`). Covers 2-D transposes and NHWC <-> NCHW style permutations.
-struct TransposeParams { uint32_t B, I, J, sb, sj; };
+struct TransposeParams { uint32_t B, I, J; int32_t sb; uint32_t sj; };      // sb may be negative (a reversed leading dimension)
 
 extern "C" __global__ __launch_bounds__(256) void transpose_tiled(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
                                                                   TransposeParams P) {
     __shared__ uint32_t tile[64][65];
     const uint32_t ti = threadIdx.x & 63u, tr = threadIdx.x >> 6;
     const uint32_t j0 = blockIdx.x * 64u, i0 = blockIdx.y * 64u, b = blockIdx.z;
-    const uint32_t* src = in + (uint64_t)b * P.sb;
+    const uint32_t* src = in + (int64_t)b * P.sb;
     uint32_t* dst = out + (uint64_t)b * P.I * P.J;
 #pragma unroll
     for (uint32_t p = 0; p < 16; ++p) {
@@ -359,7 +359,7 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4(uint32_t* _
     __shared__ uint32_t tile[64][65];
     const uint32_t t16 = threadIdx.x & 15u, tr = threadIdx.x >> 4;        // 16 vectors per tile row, 16 rows per pass
     const uint32_t j0 = blockIdx.x * 64u, i0 = blockIdx.y * 64u, b = blockIdx.z;
-    const uint32_t* src = in + (uint64_t)b * P.sb;
+    const uint32_t* src = in + (int64_t)b * P.sb;
     uint32_t* dst = out + (uint64_t)b * P.I * P.J;
 #pragma unroll
     for (uint32_t p = 0; p < 4; ++p) {

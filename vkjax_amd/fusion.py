@@ -68,6 +68,34 @@ def _walks_densely(strides, shape) -> bool:
     return len(strides) == len(shape) and all(n == 1 or s == r for s, r, n in zip(strides, K.row_major_strides(shape), shape))
 
 
+def _through_copy(operand: EwOperand, copy: EwChain, shape) -> tp.Optional[EwOperand]:
+    '''`operand` (of a chain over `shape`) reads the result of `copy`, a chain without steps, i.e. result[c] =
+    source[offset + c . strides] over copy.shape. When every dimension the operand walks is one dimension of the
+    copy's result (a transposition, a slice, a broadcast of it, or the whole of it), the operand that reads the
+    copy's source directly is returned: the two index maps composed. None otherwise.'''
+    src, cshape = copy.first, tuple(copy.shape)
+    if operand.buffer.size != np_prod(cshape) or len(operand.strides) != len(shape):
+        return None
+    dense = K.row_major_strides(cshape)
+    rest, start = operand.offset, []
+    for e in range(len(cshape)):
+        start.append(rest // dense[e])
+        rest -= start[-1] * dense[e]
+    if rest:
+        return None
+    strides, taken = [], set()
+    for n, s in zip(shape, operand.strides):
+        if n == 1 or s == 0:
+            strides.append(0)
+            continue
+        dims = [e for e in range(len(cshape)) if cshape[e] > 1 and dense[e] == s and e not in taken]
+        if len(dims) != 1 or start[dims[0]] + n > cshape[dims[0]]:
+            return None
+        taken.add(dims[0])
+        strides.append(src.strides[dims[0]])
+    return EwOperand(src.buffer, src.offset + sum(a * b for a, b in zip(start, src.strides)), tuple(strides))
+
+
 def _is_full_contiguous(operand: EwOperand, shape) -> bool:
     return operand.offset == 0 and tuple(operand.buffer.shape) == tuple(shape) and _walks_densely(operand.strides, shape)
 
@@ -149,10 +177,11 @@ def fuse_ops(all_ops, bufferpool, outvars):
             pid = id(o.buffer._placeholder)
             pos = producer.get(pid)
             prod = result[pos] if pos is not None else None
-            if (prod is None or prod.chain is None or prod.chain.steps or tuple(prod.chain.shape) != tuple(chain.shape)
-                    or not _is_full_contiguous(o, chain.shape)):
+            if prod is None or prod.chain is None or prod.chain.steps:
                 continue
-            source = prod.chain.first
+            source = _through_copy(o, prod.chain, chain.shape)
+            if source is None:
+                continue
             if k == 0:
                 first = source
             else:

@@ -235,7 +235,7 @@ def _as_tiled_transpose(chain: EwChain, dims, strides) -> tp.Optional[Launch]:
     st = strides[0]
     B, I, J = ([1] + list(dims))[-3:]
     sb = st[0] if len(dims) == 3 else 0
-    if st[-2] != 1 or st[-1] < I or I < 16 or J < 16 or sb < 0 or B > 65535 or _cdiv(I, 64) > 65535:
+    if st[-2] != 1 or st[-1] < I or I < 16 or J < 16 or B > 65535 or _cdiv(I, 64) > 65535:
         return None
     src = chain.first
     if src.buffer.size * 4 >= 2**32:
