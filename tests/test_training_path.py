@@ -351,12 +351,15 @@ def test_scale_relu_backward_and_small_chain_batches_are_planned():
     assert sum(k.startswith('scale_relu_backward') for k in kernels) == 2, kernels       #the two plain layers
     assert sum(k.startswith('scale_backward') for k in kernels) == 1, kernels            #the one whose cotangent the shortcut shares
     assert any(k.startswith('ew_chain_batch') for k in kernels), kernels
+    assert any(k.startswith('reduce_cols_fsum_batch') for k in kernels), kernels        #the second stages of the column sums
+    sums = next(l for l in interp.launches if l.kernel.startswith('reduce_cols_fsum_batch'))
+    assert K.batch_table(sums, lambda b: 0x1000).nbytes == 56 * len(sums.members)
     plain = vkjax_amd.wrap(_scale_shift_relu_step, frontend='minijax', plan_only=True, fuse=False)
     unfused, _ = plain._get_or_create_jaxpr_interpreter(_scale_shift_relu_net())
     assert len(kernels) < len(unfused.launches) - 20
     #the table of a batch launch: one 432-byte entry per member, first workgroups ascending from 0
-    batch = next(l for l in interp.launches if l.members)
-    table = K.ew_batch_table(batch, lambda b: 0x1000)
+    batch = next(l for l in interp.launches if l.members and l.kernel.startswith('ew_chain_batch'))
+    table = K.batch_table(batch, lambda b: 0x1000)
     assert table.nbytes == 432 * len(batch.members)
     firsts = table.reshape(len(batch.members), 108)[:, 0]
     assert firsts[0] == 0 and list(firsts) == list(np.cumsum([0] + [m.grid[0] for m in batch.members[:-1]]))

@@ -150,16 +150,17 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
 // with the same roundings as a separate pass, so that array never exists.
 enum { PRO_NONE = 0, PRO_MUL = 1, PRO_MULV = 2, PRO_NEG = 3 };
 
+// `block`: index of this workgroup in the reduction's own grid
 template <int VEC, int MODE, int PRO = PRO_NONE>
 __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P,
-                                                 const uint32_t* __restrict__ in2 = nullptr) {
+                                                 const uint32_t* __restrict__ in2 = nullptr, const uint32_t block = blockIdx.x) {
     __shared__ uint32_t s_val[256 * VEC];
     __shared__ uint32_t s_idx[256 * VEC];
     const uint32_t TI = P.TI, TR = 256u / TI;
     const uint32_t tid = threadIdx.x, ti = tid % TI, tr = tid / TI;
     // block -> (inner tile, split, outer row)
     const uint32_t tiles_i = (P.inner + TI * VEC - 1u) / (TI * VEC);
-    const uint32_t it = blockIdx.x % tiles_i, rest = blockIdx.x / tiles_i;
+    const uint32_t it = block % tiles_i, rest = block / tiles_i;
     const uint32_t sp = rest % P.nsplit, o = rest / P.nsplit;
     const uint32_t i = (it * TI + ti) * VEC;
     const uint32_t r_lo = sp * P.r_chunk, r_hi = min(P.R, r_lo + P.r_chunk);
@@ -256,6 +257,35 @@ __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, con
 #define REDUCE_COLS_PROLOGUE_KERNELS(tag, PRO)                                                                                 \
     extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v1(uint32_t* out, const uint32_t* in, const uint32_t* in2, ReduceParams P) { reduce_cols_body<1, 0, PRO>(out, in, P, in2); } \
     extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v4(uint32_t* out, const uint32_t* in, const uint32_t* in2, ReduceParams P) { reduce_cols_body<4, 0, PRO>(out, in, P, in2); }
+// Several small, mutually independent float column sums in ONE launch (the second stages of split sums, the
+// per-channel sums of small layers): one table entry per sum, workgroup b belongs to the last entry whose
+// first_block is <= b, as in ew_chain_batch.
+struct ReduceBatchEntry {
+    uint32_t        first_block, pad0;
+    uint32_t*       out;
+    const uint32_t* in;
+    ReduceParams    P;
+};
+static_assert(sizeof(ReduceBatchEntry) == 56, "the host lays the table out with 56-byte entries");
+
+template <int VEC>
+__device__ __forceinline__ void reduce_cols_batch_body(const ReduceBatchEntry* __restrict__ table, uint32_t entries) {
+    uint32_t lo = 0, hi = entries;
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (table[mid].first_block <= blockIdx.x) lo = mid; else hi = mid;
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    const ReduceBatchEntry& e = table[lo];
+    reduce_cols_body<VEC, 0>(e.out, e.in, e.P, nullptr, blockIdx.x - e.first_block);
+}
+extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_batch_v1(const ReduceBatchEntry* __restrict__ table, uint32_t entries) {
+    reduce_cols_batch_body<1>(table, entries);
+}
+extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_batch_v4(const ReduceBatchEntry* __restrict__ table, uint32_t entries) {
+    reduce_cols_batch_body<4>(table, entries);
+}
+
 // the _v4 variants need R % 4 == 0, r_chunk % 4 == 0 (rows) or inner % 4 == 0 (cols) and 16-byte aligned pointers
 REDUCE_COLS_PROLOGUE_KERNELS(mul, PRO_MUL)
 REDUCE_COLS_PROLOGUE_KERNELS(mulv, PRO_MULV)

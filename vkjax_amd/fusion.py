@@ -771,9 +771,19 @@ def fuse_random_streams(ops, bufferpool, outvars):
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed or i in replacement]
 
 
-def _is_small_chain(op) -> bool:
-    return (op.chain is not None and op.launch.kernel in K.EW_BATCH_KERNELS
-            and op.launch.grid[0] <= K.EW_BATCH_MAX_BLOCKS)
+def _is_small(op) -> bool:
+    '''An element-wise chain or a plain float column sum of a few workgroups, of a kind that has a batch kernel.'''
+    if op.chain is None and not (op.conv is None and op.launch.kernel in K.REDUCE_BATCH_KERNELS):
+        return False
+    return op.launch.kernel in K.BATCH_KERNELS and op.launch.grid[0] <= K.BATCH_MAX_BLOCKS
+
+
+def _small_reads(op) -> tp.List:
+    return _reads(op) if op.chain is not None else [b for b, _ in op.launch.buffers[1:]]
+
+
+def _small_out(op):
+    return op.chain.out if op.chain is not None else op.launch.buffers[0][0]
 
 
 def _may_write(op) -> tp.List:
@@ -801,21 +811,21 @@ def batch_small_chains(ops):
        front, and every one whose result nothing but other moved chains reads to the end,
     2. sorts each run of consecutive small chains into dependency levels (read-after-write, write-after-read
        and write-after-write on the buffers) and turns every level's chains of one kernel variant into ONE
-       launch of ew_chain_batch_*, and
+       launch of ew_chain_batch_* / reduce_cols_fsum_batch_*, and
     3. rebuilds the buffers' access positions from the final order, since storage is shared between
        buffers by those positions.
 
     Every chain computes what it computed before; only the order of independent launches changes.'''
     from .ops import Op
     pid = lambda b: id(b._placeholder)
-    small = [_is_small_chain(op) for op in ops]
+    small = [_is_small(op) for op in ops]
     if sum(small) < BATCH_MIN_GAIN + 1:
         return ops
 
     # 1a. to the front
     written, touched, front = set(), set(), set()
     for i, op in enumerate(ops):
-        if small[i] and not any(pid(b) in written for b in _reads(op)) and pid(_out(op)) not in touched:
+        if small[i] and not any(pid(b) in written for b in _small_reads(op)) and pid(_small_out(op)) not in touched:
             front.add(i)
             continue
         written |= {pid(b) for b in _may_write(op)}
@@ -824,7 +834,7 @@ def batch_small_chains(ops):
     written, touched, back = set(), set(), set()
     for i in reversed(range(len(ops))):
         op = ops[i]
-        if i not in front and small[i] and pid(_out(op)) not in touched and not any(pid(b) in written for b in _reads(op)):
+        if i not in front and small[i] and pid(_small_out(op)) not in touched and not any(pid(b) in written for b in _small_reads(op)):
             back.add(i)
             continue
         written |= {pid(b) for b in _may_write(op)}
@@ -836,19 +846,19 @@ def batch_small_chains(ops):
     # 2. runs of small chains -> levels -> batches
     result, saved, i = [], 0, 0
     while i < len(moved):
-        if not _is_small_chain(moved[i]):
+        if not _is_small(moved[i]):
             result.append(moved[i])
             i += 1
             continue
         j = i
-        while j < len(moved) and _is_small_chain(moved[j]):
+        while j < len(moved) and _is_small(moved[j]):
             j += 1
         run, level = moved[i:j], []
         for k, op in enumerate(run):
-            reads, out = {pid(b) for b in _reads(op)}, pid(_out(op))
+            reads, out = {pid(b) for b in _small_reads(op)}, pid(_small_out(op))
             lv = 0
             for q in range(k):
-                q_reads, q_out = {pid(b) for b in _reads(run[q])}, pid(_out(run[q]))
+                q_reads, q_out = {pid(b) for b in _small_reads(run[q])}, pid(_small_out(run[q]))
                 if q_out in reads or q_out == out or out in q_reads:
                     lv = max(lv, level[q] + 1)
             level.append(lv)
@@ -861,7 +871,7 @@ def batch_small_chains(ops):
                 if len(group) == 1:
                     result.append(group[0])
                     continue
-                batch = Op(_label(*group), launch=K.ew_chain_batch([op.launch for op in group]))
+                batch = Op(_label(*group), launch=K.batch_launch([op.launch for op in group]))
                 batch.index = min(op.index for op in group)
                 result.append(batch)
                 saved += len(group) - 1

@@ -77,7 +77,7 @@ class JaxprInterpreter:
         for op, launch in zip(self.all_ops, self.launches):
             if launch.members:
                 #a batch of small launches reads its members' arguments from a table in HBM
-                table = self.mgr.tensor(K.ew_batch_table(launch, lambda b: b.tensor.device_ptr()))
+                table = self.mgr.tensor(K.batch_table(launch, lambda b: b.tensor.device_ptr()))
                 self._batch_tables.append(table)
                 self.sequence.record_launch(launch.kernel, launch.grid, launch.block, [(table, 0)], launch.params, launch.lds)
                 continue

@@ -200,30 +200,37 @@ def lower_ew_chain(chain: EwChain) -> Launch:
 
 
 EW_BATCH_KERNELS     = ('ew_chain_v1_s2', 'ew_chain_v1_s4', 'ew_chain_v4_s2', 'ew_chain_v4_s4')
-EW_BATCH_ENTRY_BYTES = 432
-EW_BATCH_MAX_BLOCKS  = 16          #chains of more workgroups than this keep a launch of their own
+REDUCE_BATCH_KERNELS = ('reduce_cols_fsum_v1', 'reduce_cols_fsum_v4')
+BATCH_KERNELS        = {**{k: k.replace('ew_chain_', 'ew_chain_batch_') for k in EW_BATCH_KERNELS},
+                        **{k: k.replace('fsum_', 'fsum_batch_') for k in REDUCE_BATCH_KERNELS}}
+EW_BATCH_ENTRY_BYTES     = 432
+REDUCE_BATCH_ENTRY_BYTES = 56
+BATCH_MAX_BLOCKS         = 16          #launches of more workgroups than this keep a launch of their own
 
 
-def ew_chain_batch(members: tp.Sequence[Launch]) -> Launch:
-    '''One launch for several small element-wise chains that do not depend on one another and lower
-    to the same kernel variant.'''
+def batch_launch(members: tp.Sequence[Launch]) -> Launch:
+    '''One launch for several small launches of the same kernel (element-wise chains or float column sums)
+    that do not depend on one another.'''
     kernel = members[0].kernel
-    assert kernel in EW_BATCH_KERNELS and all(m.kernel == kernel and not m.members for m in members), [m.kernel for m in members]
-    return Launch(kernel.replace('ew_chain_', 'ew_chain_batch_'), (sum(m.grid[0] for m in members), 1, 1), (BLOCK, 1, 1), [],
+    assert kernel in BATCH_KERNELS and all(m.kernel == kernel and not m.members for m in members), [m.kernel for m in members]
+    return Launch(BATCH_KERNELS[kernel], (sum(m.grid[0] for m in members), 1, 1), (BLOCK, 1, 1), [],
                   _u32(len(members)), bytes_moved=sum(m.bytes_moved for m in members), members=tuple(members))
 
 
-def ew_batch_table(launch: Launch, device_address: tp.Callable[[Buffer], int]) -> np.ndarray:
-    '''The table of a batch launch as uint32 words: per member {first workgroup, 0, address of the result,
-    addresses of the 8 operand slots (0 = none), the member's parameter block, 0}.'''
+def batch_table(launch: Launch, device_address: tp.Callable[[Buffer], int]) -> np.ndarray:
+    '''The table of a batch launch as uint32 words, one entry per member: {first workgroup, 0, the addresses of the
+    member's arrays (0 = none), the member's parameter block}, padded to a multiple of 8 bytes.'''
+    is_chain = launch.members[0].kernel in EW_BATCH_KERNELS
+    entry_bytes, pointers = (EW_BATCH_ENTRY_BYTES, 1 + EW_MAX_STEPS) if is_chain else (REDUCE_BATCH_ENTRY_BYTES, 2)
     rows, first = [], 0
     for m in launch.members:
-        assert len(m.buffers) == 1 + EW_MAX_STEPS and len(m.params) == EW_BATCH_ENTRY_BYTES - 8 - 8 * (1 + EW_MAX_STEPS) - 4
+        assert len(m.buffers) == pointers, (m.kernel, len(m.buffers))
         addresses = [device_address(b) + off if b is not None else 0 for b, off in m.buffers]
-        rows.append(_u32(first, 0) + np.asarray(addresses, dtype=np.uint64).tobytes() + m.params + _u32(0))
+        row = _u32(first, 0) + np.asarray(addresses, dtype=np.uint64).tobytes() + m.params
+        rows.append(row + bytes(entry_bytes - len(row)))
         first += m.grid[0]
     table = b''.join(rows)
-    assert len(table) == EW_BATCH_ENTRY_BYTES * len(launch.members)
+    assert len(table) == entry_bytes * len(launch.members)
     return np.frombuffer(table, dtype=np.uint32).copy()
 
 
