@@ -71,6 +71,11 @@ class JaxprInterpreter:
             return
         self.sequence = self.mgr.sequence(profiling=self.profiling)
         self._input_slots = []
+        #(elements, dtype) of a host array that can be handed to the device as it is
+        self._input_specs = []
+        for var in jaxpr.jaxpr.invars:
+            shape, dtype = core.physical(var.aval)
+            self._input_specs.append((int(np.prod(shape, dtype=np.int64)), dtype if dtype in (np.float32, np.int32, np.uint32) else None))
         for b in self.input_buffers:
             self._input_slots.append(self.sequence.record_upload(b.tensor, b.nbytes()) if b is not None else None)
         self._batch_tables = []
@@ -102,7 +107,7 @@ class JaxprInterpreter:
         for i, x in enumerate(X):
             if i in self.static_argnums:
                 continue
-            these = tree_util.tree_leaves([x])
+            these = [x] if type(x) is np.ndarray else tree_util.tree_leaves([x])
             leaves   += these
             resident += [i in self.resident_argnums] * len(these)
         if len(self.input_buffers) != len(leaves):
@@ -122,7 +127,12 @@ class JaxprInterpreter:
                 if self._resident_leaves.get(k) is x:
                     continue                                    #already in HBM
                 self._resident_leaves[k] = x
-            host[slot] = _device_words_of_argument(x, var.aval)
+            #the common case without the general conversion: an array that already is what the device holds
+            n, dtype = self._input_specs[k]
+            if type(x) is np.ndarray and x.dtype == dtype and x.size == n and x.flags.c_contiguous:
+                host[slot] = x.reshape(-1).view(np.uint32)
+            else:
+                host[slot] = _device_words_of_argument(x, var.aval)
         return host
 
     def _fresh_outputs(self, host) -> tp.List[tp.Optional[np.ndarray]]:
