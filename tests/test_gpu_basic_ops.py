@@ -293,7 +293,11 @@ def test_tiled_transposes():
              (lambda x: lax.transpose(lax.rev(x, (0, 1)), (0, 1, 3, 2)), [random([3, 3, 64, 128])]),
              (lambda x: lax.transpose(lax.rev(x, (0,)), (0, 2, 1)), [random([5, 33, 70])]),
              (lambda x: lax.transpose(lax.rev(x, (0, 1)), (0, 1, 3, 2)), [random([1, 1, 256, 64])]),
-             (lambda x: lax.transpose(lax.transpose(x, (1, 0, 2)), (0, 2, 1)), [random([6, 5, 40])[:, :, 4:36]])]
+             (lambda x: lax.transpose(lax.transpose(x, (1, 0, 2)), (0, 2, 1)), [random([6, 5, 40])[:, :, 4:36]]),
+             #128 x 128 tiles (both sides at least 128 long, multiples of four): ragged edges, a batch, a reversed batch
+             (lambda x: lax.transpose(x, (1, 0)), [random([260, 516])]),
+             (lambda x: lax.transpose(x, (0, 2, 1)), [random([3, 132, 512])]),
+             (lambda x: lax.transpose(lax.rev(x, (0,)), (0, 2, 1)), [random([3, 128, 640])])]
     for k, (f, args) in enumerate(cases):
         print(f'case: tiled transpose {k}', flush=True)
         _, _, fn = check_against_oracle(f, args, exact=True)
@@ -302,6 +306,8 @@ def test_tiled_transposes():
             assert any(name.startswith('transpose_tiled') for name in kernels), kernels
         if k in (10, 11, 12, 13):
             assert len(kernels) == 1, kernels
+        if k >= 14:
+            assert kernels == ['transpose_tiled_v4_t128'], kernels
 
 
 def test_nextafter_direction():

@@ -335,7 +335,9 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled(uint32_t* __re
                                                                   TransposeParams P) {
     __shared__ uint32_t tile[64][65];
     const uint32_t ti = threadIdx.x & 63u, tr = threadIdx.x >> 6;
-    const uint32_t j0 = blockIdx.x * 64u, i0 = blockIdx.y * 64u, b = blockIdx.z;
+    // Tiles are taken along diagonals: with a row pitch that is a large power of two, the tiles of one row or one
+    // column of tiles all start in the same memory channel, and workgroups that run together would queue there.
+    const uint32_t j0 = blockIdx.x * 64u, i0 = ((blockIdx.y + blockIdx.x) % gridDim.y) * 64u, b = blockIdx.z;
     const uint32_t* src = in + (int64_t)b * P.sb;
     uint32_t* dst = out + (uint64_t)b * P.I * P.J;
 #pragma unroll
@@ -358,7 +360,9 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4(uint32_t* _
                                                                      TransposeParams P) {
     __shared__ uint32_t tile[64][65];
     const uint32_t t16 = threadIdx.x & 15u, tr = threadIdx.x >> 4;        // 16 vectors per tile row, 16 rows per pass
-    const uint32_t j0 = blockIdx.x * 64u, i0 = blockIdx.y * 64u, b = blockIdx.z;
+    // Tiles are taken along diagonals: with a row pitch that is a large power of two, the tiles of one row or one
+    // column of tiles all start in the same memory channel, and workgroups that run together would queue there.
+    const uint32_t j0 = blockIdx.x * 64u, i0 = ((blockIdx.y + blockIdx.x) % gridDim.y) * 64u, b = blockIdx.z;
     const uint32_t* src = in + (int64_t)b * P.sb;
     uint32_t* dst = out + (uint64_t)b * P.I * P.J;
 #pragma unroll
@@ -379,6 +383,40 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4(uint32_t* _
             v.x = tile[4u * t16][tr + 16u * p]; v.y = tile[4u * t16 + 1u][tr + 16u * p];
             v.z = tile[4u * t16 + 2u][tr + 16u * p]; v.w = tile[4u * t16 + 3u][tr + 16u * p];
             *reinterpret_cast<u32x4*>(dst + (uint64_t)i * P.J + j) = v;
+        }
+    }
+}
+
+// 128 x 128 tiles for large arrays: runs of 512 contiguous bytes on both sides, sixteen 16-byte loads
+// in flight per thread. Same conditions as transpose_tiled_v4.
+extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4_t128(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                                          TransposeParams P) {
+    __shared__ uint32_t tile[128][129];
+    const uint32_t t32 = threadIdx.x & 31u, tr = threadIdx.x >> 5;        // 32 vectors per tile row, 8 rows per pass
+    const uint32_t j0 = blockIdx.x * 128u, i0 = ((blockIdx.y + blockIdx.x) % gridDim.y) * 128u, b = blockIdx.z;
+    const uint32_t* src = in + (int64_t)b * P.sb;
+    uint32_t* dst = out + (uint64_t)b * P.I * P.J;
+    u32x4 v[16];
+#pragma unroll
+    for (uint32_t p = 0; p < 16; ++p) {
+        const uint32_t j = j0 + tr + 8u * p, i = i0 + 4u * t32;
+        v[p] = u32x4{0u, 0u, 0u, 0u};
+        if (i < P.I && j < P.J) v[p] = *reinterpret_cast<const u32x4*>(src + (uint64_t)j * P.sj + i);
+    }
+#pragma unroll
+    for (uint32_t p = 0; p < 16; ++p) {
+        uint32_t* row = tile[tr + 8u * p] + 4u * t32;
+        row[0] = v[p].x; row[1] = v[p].y; row[2] = v[p].z; row[3] = v[p].w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t p = 0; p < 16; ++p) {
+        const uint32_t i = i0 + tr + 8u * p, j = j0 + 4u * t32;
+        if (i < P.I && j < P.J) {
+            u32x4 w;
+            w.x = tile[4u * t32][tr + 8u * p]; w.y = tile[4u * t32 + 1u][tr + 8u * p];
+            w.z = tile[4u * t32 + 2u][tr + 8u * p]; w.w = tile[4u * t32 + 3u][tr + 8u * p];
+            *reinterpret_cast<u32x4*>(dst + (uint64_t)i * P.J + j) = w;
         }
     }
 }

@@ -234,6 +234,9 @@ def batch_table(launch: Launch, device_address: tp.Callable[[Buffer], int]) -> n
     return np.frombuffer(table, dtype=np.uint32).copy()
 
 
+TRANSPOSE_BIG_TILES = True
+
+
 def _as_tiled_transpose(chain: EwChain, dims, strides) -> tp.Optional[Launch]:
     '''A pure copy whose collapsed form is out[b, i, j] = in[b * sb + j * sj + i] (the two fastest dimensions
     trade places) goes through the LDS-tiled kernel when both of them are at least 16 long.'''
@@ -249,6 +252,9 @@ def _as_tiled_transpose(chain: EwChain, dims, strides) -> tp.Optional[Launch]:
         return None
     n = B * I * J
     vec = all(v % 4 == 0 for v in (I, J, st[-1], sb, src.offset))
+    if vec and I >= 128 and J >= 128 and I * J >= 1 << 16 and TRANSPOSE_BIG_TILES:
+        return Launch('transpose_tiled_v4_t128', (_cdiv(J, 128), _cdiv(I, 128), B), (BLOCK, 1, 1), [(chain.out, 0), (src.buffer, src.offset * 4)],
+                      _u32(B, I, J, sb, st[-1]), lds=0, bytes_moved=8 * n)
     return Launch('transpose_tiled_v4' if vec else 'transpose_tiled', (_cdiv(J, 64), _cdiv(I, 64), B), (BLOCK, 1, 1), [(chain.out, 0), (src.buffer, src.offset * 4)],
                   _u32(B, I, J, sb, st[-1]), bytes_moved=8 * n)
 
