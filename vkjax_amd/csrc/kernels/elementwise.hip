@@ -23,7 +23,8 @@ struct EwParams {
                                        // bit2: the operand's fastest stride is 1 (else 0: one value per vector);
                                        // bits 4-5: how the operand is addressed: 0 through its strides, 1 like the
                                        // output (element = base + linear index), 2 by the fastest dimension only
-                                       // (element = base + coordinate), 3 a single element (base)
+                                       // (element = base + coordinate), 3 a single element (base);
+                                       // bit6: every vector of a thread reads the same elements of the operand
     uint32_t imm[EW_MAX_STEPS];        // immediate (integer_pow exponent)
     int32_t  stride[EW_MAX_STEPS][4];  // operand strides per collapsed dim, in elements
     uint32_t nbytes[EW_MAX_STEPS];     // bytes readable from each operand pointer (0 = no operand)
@@ -113,6 +114,13 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
         };
 #pragma unroll
         for (int k = 0; k < NS; ++k) {
+            if (u > 0 && (flags[k] & 64u)) {
+                // a single value, or a vector over the fastest dimension whose length divides the distance
+                // between a thread's vectors: what the thread's first vector loaded serves the others too
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) vals[k][u * VEC + j] = vals[k][j];
+                continue;
+            }
             const uint32_t idx = operand_index(k);
             const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, (int)nbytes[k], 0x00020000);
             if constexpr (VEC == 4) {

@@ -175,11 +175,14 @@ def lower_ew_chain(chain: EwChain) -> Launch:
             flag |= 1 | (4 if st[-1] == 1 else 0)
             #simple addressing patterns the kernel resolves without multiplications
             if all(s == 0 for s in st):
-                flag |= 3 << 4
+                flag |= 3 << 4 | 64
             elif tuple(st) == row_major_strides(dims):
                 flag |= 1 << 4
             elif st[-1] == 1 and all(s == 0 for s in st[:-1]):
                 flag |= 2 << 4
+                #a thread's vectors are BLOCK * vec elements apart: the same coordinate when the dimension's length divides that
+                if (BLOCK * vec) % dims[-1] == 0:
+                    flag |= 64
             stride_rows.append(_pad(st, 4))
             buffers.append((o.buffer, 0))
         flags.append(flag)
