@@ -42,7 +42,7 @@ int hip_fail(hipError_t e, const char* what) {
 // and transfer overlap instead of running one after the other.
 constexpr size_t STAGE_CHUNK   = 4u << 20;
 constexpr size_t STAGE_MIN     = 8u << 20;     // smaller transfers are copied inline
-constexpr int    STAGE_THREADS = 4;
+constexpr int    STAGE_THREADS = 8;
 
 template <class Issue>
 int staged_upload(char* staging, const char* host, size_t nbytes, Issue&& issue) {
@@ -77,27 +77,37 @@ int staged_upload(char* staging, const char* host, size_t nbytes, Issue&& issue)
     return status;
 }
 
-// Copy out of (or into) pinned memory with a few threads; small sizes are copied inline.
-void parallel_copy(char* dst, const char* src, size_t nbytes) {
-    if (nbytes < STAGE_MIN) { memcpy(dst, src, nbytes); return; }
+// Large downloads, the other way round: the transfer is issued chunk by chunk with an event behind every
+// chunk; the calling thread waits for the events in order and a few threads copy each chunk out of the
+// pinned buffer as soon as it has landed, while the chunks after it are still on their way.
+template <class Wait>
+int staged_copy_out(char* dst, const char* staging, size_t nbytes, Wait&& wait_for_chunk) {
     const size_t nchunks = (nbytes + STAGE_CHUNK - 1) / STAGE_CHUNK;
-    std::atomic<size_t> next{0};
+    std::atomic<size_t> landed{0}, next{0};
     auto worker = [&]() {
         for (;;) {
             const size_t k = next.fetch_add(1, std::memory_order_relaxed);
             if (k >= nchunks) return;
+            while (landed.load(std::memory_order_acquire) <= k) std::this_thread::yield();
             const size_t off = k * STAGE_CHUNK;
-            memcpy(dst + off, src + off, std::min(STAGE_CHUNK, nbytes - off));
+            memcpy(dst + off, staging + off, std::min(STAGE_CHUNK, nbytes - off));
         }
     };
     std::vector<std::thread> threads;
     try {
-        for (int t = 1; t < (int)std::min<size_t>(STAGE_THREADS, nchunks); t++) threads.emplace_back(worker);
+        for (int t = 0; t < (int)std::min<size_t>(STAGE_THREADS, nchunks); t++) threads.emplace_back(worker);
     } catch (...) {
     }
-    worker();
+    int status = 0;
+    for (size_t k = 0; k < nchunks; k++) {
+        if (status == 0) status = wait_for_chunk(k);
+        landed.store(k + 1, std::memory_order_release);      // after a failure too: the helpers must come to an end
+    }
+    if (threads.empty()) worker();
     for (auto& t : threads) t.join();
+    return status;
 }
+
 
 #define HIP_TRY(expr)                                   \
     do {                                                \
@@ -163,6 +173,7 @@ struct Seq {
     bool                  profiling = false;
     std::vector<Transfer> uploads, downloads;
     std::vector<Launch>   launches;
+    std::vector<hipEvent_t> chunk_events;   // one behind every chunk of a large download
     std::vector<hipEvent_t> stamps;   // profiling: 1 + number of steps
     int                   stamps_valid = 0;
     bool                  want_graph = false;     // issue the launches as one captured graph
@@ -480,6 +491,7 @@ int vkj_seq_destroy(vkj_handle sh) {
     }
     for (auto& t : s->downloads) if (t.staging) hipHostFree(t.staging);
     for (auto e : s->stamps) hipEventDestroy(e);
+    for (auto e : s->chunk_events) hipEventDestroy(e);
     drop_graph(s);
     retire(s);
     delete s;
@@ -640,9 +652,23 @@ int vkj_seq_eval_next(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_
     // The downloads are queued after the copies above on purpose: a copy engine works through its
     // queue in order, and a download queued first waits there for the launches, with every upload
     // behind it, even one from the other stream, waiting as well.
+    size_t nchunk_events = 0;
     if (down) for (auto& t : s->downloads) {
         if (!t.nbytes) continue;
-        HIP_TRY(hipMemcpyAsync(t.staging, (char*)t.buf->dptr + t.offset, t.nbytes, hipMemcpyDeviceToHost, c->stream));
+        if (t.nbytes < STAGE_MIN) {
+            HIP_TRY(hipMemcpyAsync(t.staging, (char*)t.buf->dptr + t.offset, t.nbytes, hipMemcpyDeviceToHost, c->stream));
+            continue;
+        }
+        for (size_t off = 0; off < t.nbytes; off += STAGE_CHUNK, nchunk_events++) {
+            if (s->chunk_events.size() <= nchunk_events) {
+                hipEvent_t e;
+                HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+                s->chunk_events.push_back(e);
+            }
+            HIP_TRY(hipMemcpyAsync((char*)t.staging + off, (char*)t.buf->dptr + t.offset + off, std::min(STAGE_CHUNK, t.nbytes - off),
+                                   hipMemcpyDeviceToHost, c->stream));
+            HIP_TRY(hipEventRecord(s->chunk_events[nchunk_events], c->stream));
+        }
     }
     if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[nstamps - 1], c->stream));
     if (landed) {
@@ -652,9 +678,23 @@ int vkj_seq_eval_next(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_
             if (t.nbytes && t.slot < nslots && next_host_ptrs[t.slot])
                 HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.landing, t.nbytes, hipMemcpyDeviceToDevice, c->stream));
     }
+    // large results leave the pinned buffers chunk by chunk as they land; then everything else is waited for
+    if (down) {
+        size_t first_event = 0;
+        for (auto& t : s->downloads) {
+            if (t.nbytes < STAGE_MIN) continue;
+            hipError_t err = hipSuccess;
+            const int r = staged_copy_out((char*)host_ptrs[t.slot], (const char*)t.staging, t.nbytes, [&](size_t k) {
+                err = hipEventSynchronize(s->chunk_events[first_event + k]);
+                return err == hipSuccess ? 0 : 1;
+            });
+            if (r) return hip_fail(err, "hipEventSynchronize (staged download)");
+            first_event += (t.nbytes + STAGE_CHUNK - 1) / STAGE_CHUNK;
+        }
+    }
     HIP_TRY(hipStreamSynchronize(c->stream));
     if (down) for (auto& t : s->downloads)
-        if (t.nbytes) parallel_copy((char*)host_ptrs[t.slot], (const char*)t.staging, t.nbytes);
+        if (t.nbytes && t.nbytes < STAGE_MIN) memcpy(host_ptrs[t.slot], t.staging, t.nbytes);
     if (s->profiling) s->stamps_valid = (int)nstamps;
     return 0;
 }
