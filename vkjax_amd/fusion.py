@@ -399,7 +399,7 @@ def fuse_scale_relu_backward(ops, bufferpool, outvars):
     for i, op in enumerate(ops):
         for b in _reads(op):
             readers.setdefault(pid(b), []).append(i)
-    single = lambda o: o is not None and all(st == 0 for st in o.strides)
+    single = lambda o: o is not None and o.offset == 0 and all(st == 0 for st in o.strides)
     removed, replacement = set(), {}
 
     def column_sum_of(i, buffer):
