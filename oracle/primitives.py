@@ -424,12 +424,25 @@ def reduce_prod(x, axes, **_):
     return x.astype(np.int64).prod(axis=tuple(axes)).astype(x.dtype)
 
 
+def _extreme(dtype, largest: bool):
+    '''XLA's init value of reduce_min (largest) / reduce_max: what a reduction over no elements returns.'''
+    dtype = np.dtype(dtype)
+    if dtype.kind == 'f':
+        return dtype.type(np.inf if largest else -np.inf)
+    if dtype.kind == 'b':
+        return largest
+    info = np.iinfo(dtype)
+    return dtype.type(info.max if largest else info.min)
+
+
 def reduce_max(x, axes, **_):
-    return _canon(x).max(axis=tuple(axes)) if len(axes) else _canon(x)
+    x = _canon(x)
+    return x.max(axis=tuple(axes), initial=_extreme(x.dtype, False)) if len(axes) else x
 
 
 def reduce_min(x, axes, **_):
-    return _canon(x).min(axis=tuple(axes)) if len(axes) else _canon(x)
+    x = _canon(x)
+    return x.min(axis=tuple(axes), initial=_extreme(x.dtype, True)) if len(axes) else x
 
 
 def reduce_or(x, axes, **_):

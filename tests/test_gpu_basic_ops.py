@@ -340,3 +340,29 @@ def test_argmax_ties_and_nan():
     def f(x): return jnp.argmax(x, axis=1), jnp.argmin(x, axis=1)
     (amax, amin), _, _ = check_against_oracle(f, [x], exact=True)
     assert amax.tolist() == [1, 0, 0, 2] and amin.tolist() == [0, 0, 0, 1]
+
+
+def test_arrays_without_elements():
+    '''Shapes with a dimension of size 0: results without elements cost no launch, a reduction or contraction over
+    no elements gives the operation's identity (XLA's init values), and the rest of the program is untouched.'''
+    import vkjax_amd
+    f32 = lambda *shape: np.zeros(shape, np.float32)
+    cases = [('add', lambda x, y: x + y, [f32(0, 5), f32(0, 5)], 0),
+             ('sum over an empty axis', lambda x: jnp.sum(x, axis=0), [f32(0, 5)], 1),
+             ('max over an empty axis', lambda x: lax.reduce_max(x, (1,)), [f32(3, 0)], 1),
+             ('min over an empty axis', lambda x: lax.reduce_min(x, (1,)), [np.zeros((3, 0), np.int32)], 1),
+             ('sum that stays empty', lambda x: jnp.sum(x, axis=1), [f32(0, 5)], 0),
+             ('concatenate with an empty part', lambda x, y: lax.concatenate([x, y], 0), [f32(0, 5), np.ones((2, 5), np.float32)], 1),
+             ('dot over an empty contraction', lambda x, y: jnp.dot(x, y) + 1.0, [f32(4, 0), f32(0, 3)], None),
+             ('dot without rows', lambda x, y: jnp.dot(x, y), [f32(0, 8), np.ones((8, 3), np.float32)], 0),
+             ('gather without indices', lambda t, i: t[i], [np.ones((6, 4), np.float32), np.zeros((0,), np.int32)], 0),
+             ('transpose', lambda x: lax.transpose(x, (1, 0)), [f32(0, 7)], 0),
+             ('empty and not', lambda x, y: (x * 2.0, y + 1.0), [f32(0), np.ones((3,), np.float32)], 1),
+             ('convolution of an empty batch', lambda x, k: lax.conv_general_dilated(x, k, (1, 1), 'SAME', dimension_numbers=('NHWC', 'HWIO', 'NHWC')),
+              [f32(0, 6, 6, 4), np.ones((3, 3, 4, 8), np.float32)], 0)]
+    for name, f, args, launches in cases:
+        print(f'case: {name}', flush=True)
+        _, _, fn = check_against_oracle(f, args, exact=True)
+        n = len(list(fn._jaxpr_interpreters.values())[0].launches)
+        assert launches is None or n == launches, (name, n)
+        check_against_oracle(f, args, exact=True, fuse=False)

@@ -300,3 +300,18 @@ def test_whole_program_identities():
     idx = rng.randint(0, 10, size=(6, 1)).astype(np.int32)
     (t,) = eval_closed_jaxpr(closed, x, idx)
     assert np.array_equal(t, np.take_along_axis(x, idx, axis=-1))
+
+
+def test_reductions_over_no_elements_return_the_init_value():
+    '''XLA reduces with an init value (lax.reduce_max: -inf / the smallest integer, reduce_min: +inf / the largest,
+    reduce_sum: 0), which is what remains when the reduced range is empty.'''
+    from oracle import primitives as P
+    assert np.array_equal(P.reduce_max(np.zeros((3, 0), np.float32), (1,)), np.full(3, -np.inf, np.float32))
+    assert np.array_equal(P.reduce_min(np.zeros((3, 0), np.float32), (1,)), np.full(3, np.inf, np.float32))
+    assert np.array_equal(P.reduce_max(np.zeros((2, 0), np.int32), (1,)), np.full(2, -2**31, np.int32))
+    assert np.array_equal(P.reduce_min(np.zeros((2, 0), np.int32), (1,)), np.full(2, 2**31 - 1, np.int32))
+    assert np.array_equal(P.reduce_sum(np.zeros((0, 4), np.float32), (0,)), np.zeros(4, np.float32))
+    #and nothing changes where there are elements
+    x = np.array([[1.0, -3.0, np.nan], [2.0, 5.0, -1.0]], np.float32)
+    assert np.array_equal(P.reduce_max(x, (1,)), np.array([np.nan, 5.0], np.float32), equal_nan=True)
+    assert np.array_equal(P.reduce_min(x, (0,)), np.array([1.0, -3.0, np.nan], np.float32), equal_nan=True)

@@ -74,6 +74,12 @@ def analyze_jaxpr(bufferpool: BufferPool, jaxpr) -> tp.List[Op]:
     for eq in jaxpr.eqns:
         if all(core.is_dropped(v) for v in eq.outvars):
             continue
+        if all(core.is_dropped(v) or 0 in core.physical(v.aval)[0] for v in eq.outvars):
+            #nothing to compute: results without elements get their (token) storage and no launch
+            for v in eq.outvars:
+                if not core.is_dropped(v):
+                    bufferpool.get_buffer(v)
+            continue
         opname = eq.primitive.name.replace('-', '_')
         method = globals().get(opname, None)
         if method is None or not callable(method) or opname.startswith('_'):
@@ -525,6 +531,8 @@ def dot_general(bufferpool, equation):
     lst, rst = K.row_major_strides(lhs.shape), K.row_major_strides(rhs.shape)
     if outbuf.size == 0:
         return []
+    if Kc == 0:
+        return [Op(equation, launch=K.fill(outbuf, 0))]            #an empty sum for every element
     if tuple(lc) == (0,) and tuple(rc) == (0,) and Kc >= WGRAD_MIN_PIXELS:
         #both operands contracted over their rows (a dense layer's weight gradient): read along the rows
         wg = K.WgradGeometry(images=1, Ho=Kc, Wo=1, H=Kc, W=1, C=M, KH=1, KW=1, N=N)
@@ -567,6 +575,8 @@ def conv_general_dilated(bufferpool, equation):
                           os=(os_[0], os_[2], os_[3], os_[1]))
     if outbuf.size == 0:
         return []
+    if lhs.size == 0 or rhs.size == 0:
+        return [Op(equation, launch=K.fill(outbuf, 0))]            #no input features, or an empty window: sums of nothing
     wg = _as_kernel_gradient(geom)
     if wg is not None:
         return _wgrad_ops(bufferpool, equation, outbuf, lhs, rhs, wg)
@@ -644,6 +654,22 @@ def _as_kernel_gradient(g: 'K.ConvGeometry') -> tp.Optional['K.WgradGeometry']:
 
 # ------------------------------------------------------------------ reductions
 
+def _reduction_identity_word(name: str, dtype, equation) -> int:
+    kind = _kind(dtype)
+    if name == 'reduce_sum':
+        value = 0
+    elif name == 'reduce_prod':
+        value = 1
+    elif name == 'reduce_max':
+        value = {_F: -np.inf, _I: np.iinfo(np.int32).min, _U: 0, _B: 0}[kind]
+    elif name == 'reduce_min':
+        value = {_F: np.inf, _I: np.iinfo(np.int32).max, _U: np.iinfo(np.uint32).max, _B: 1}[kind]
+    else:
+        raise NotImplementedError(f'{name} over an empty range: {equation}')
+    host = np.asarray(value, dtype=np.uint32 if kind == _B else dtype)
+    return int(host.reshape(1).view(np.uint32)[0])
+
+
 def reduce_op(bufferpool, equation):
     axes = tuple(int(a) for a in equation.params['axes'])
     if axes == ():
@@ -661,6 +687,9 @@ def reduce_op(bufferpool, equation):
         raise NotImplementedError(equation)
     if outbuf.size == 0:
         return []
+    if inbuf.size == 0:
+        #a reduction over no elements is the operation's identity (XLA's init value)
+        return [Op(equation, launch=K.fill(outbuf, _reduction_identity_word(name, inbuf.dtype, equation)))]
     shape   = inbuf.shape
     strides = K.row_major_strides(shape)
     #merge neighbouring dims with the same role, drop size-1 dims
