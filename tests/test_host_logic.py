@@ -334,3 +334,23 @@ def test_batch_of_one_fuses_like_any_other():
         interp, _ = fn._get_or_create_jaxpr_interpreter(tuple(W.resnet50_inputs(batch=batch, size=64, num_classes=40, width_scale=0.25)))
         counts.append(len(interp.launches))
     assert counts[0] == counts[1] == 58, counts
+
+
+def test_size_limits_are_reported_when_the_program_is_built():
+    '''Kernels address an array through a 32-bit byte offset: an element-wise operand has to stay below 4 GiB and
+    a convolution operand below 2 GiB. Larger ones are refused with NotImplementedError while the program is
+    planned (nothing is allocated or launched); the largest allowed sizes plan.'''
+    import vkjax_amd
+    from vkjax_amd import minijax as mj
+    def plan(f, *args):
+        fn = vkjax_amd.wrap(f, frontend='minijax', plan_only=True)
+        return fn._get_or_create_jaxpr_interpreter(args)[0]
+    huge = lambda *shape: np.broadcast_to(np.float32(1), shape)            #no memory behind it
+    interp = plan(lambda x: x * 2.0, huge((1 << 30) - 4))
+    assert [l.kernel for l in interp.launches] == ['ew_chain_v4_s2'] and interp.launches[0].grid[0] == (1 << 20)
+    with pytest.raises(NotImplementedError):
+        plan(lambda x: x * 2.0, huge(1 << 30))
+    with pytest.raises(NotImplementedError):
+        plan(lambda x, w: mj.numpy.dot(x, w), huge(1 << 20, 512), huge(512, 8))       #2 GiB lhs
+    interp = plan(lambda x, w: mj.numpy.dot(x, w), huge((1 << 20) - 64, 511), huge(511, 8))
+    assert interp.launches[0].kernel.startswith('conv_gemm')
