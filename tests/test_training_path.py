@@ -8,7 +8,7 @@ import pytest
 
 from oracle import primitives as P
 from oracle.eval_jaxpr import eval_closed_jaxpr
-from tests.common import check_against_oracle, assert_tree_close
+from tests.common import check_against_oracle, assert_tree_close, oracle_outputs
 from vkjax_amd import kernels as K, minijax as mj, workloads as W
 from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
 
@@ -378,3 +378,55 @@ def test_scale_relu_backward_and_small_chain_batches_keep_every_bit():
         unfused = vkjax_amd.wrap(_scale_shift_relu_step, frontend='minijax', fuse=False)(*args)
         assert_tree_close(fused, unfused, exact=True, what=f'fused against unfused {kwargs}')
         check_against_oracle(_scale_shift_relu_step, args, rtol=1e-4, atol=1e-5)
+
+
+def _batch_stat_net_inputs(seed=0, batch=4, size=6, channels=((4, 8), (8, 8))):
+    rng = np.random.default_rng(seed)
+    params = [dict(w=(rng.standard_normal((3, 3, cin, cout)) / np.sqrt(9 * cin)).astype(np.float32),
+                   scale=(1 + 0.1 * rng.standard_normal(cout)).astype(np.float32),
+                   shift=(0.1 * rng.standard_normal(cout)).astype(np.float32)) for cin, cout in channels]
+    return params, rng.standard_normal((batch, size, size, channels[0][0])).astype(np.float32)
+
+
+def _batch_stat_net_loss(params, x):
+    '''Convolution -> batch norm with the BATCH's own mean and variance -> ReLU, twice; mean of squares.'''
+    h = x
+    for p in params:
+        y = mj.lax.conv_general_dilated(h, p['w'], (1, 1), 'SAME', dimension_numbers=('NHWC', 'HWIO', 'NHWC'))
+        mean = mj.numpy.mean(y, axis=(0, 1, 2))
+        var = mj.numpy.mean((y - mean) ** 2, axis=(0, 1, 2))
+        h = mj.nn.relu((y - mean) * mj.lax.rsqrt(var + 1e-5) * p['scale'] + p['shift'])
+    return mj.numpy.sum(h * h) / h.size
+
+
+def _batch_stat_net_step(params, x):
+    return mj.value_and_grad(_batch_stat_net_loss)(params, x)
+
+
+def test_batch_norm_with_batch_statistics_equals_torch_autograd():
+    '''The gradient flows through the batch mean and variance as well (reductions, rsqrt, broadcasts and their
+    transposes); torch's batch_norm in training mode is the independent implementation.'''
+    import torch
+    params, x = _batch_stat_net_inputs()
+    (loss, gradients), _ = oracle_outputs(_batch_stat_net_step, (params, x))
+    grads = mj.tree_util.tree_leaves(gradients)
+    tp = [{k: torch.tensor(v, requires_grad=True) for k, v in p.items()} for p in params]
+    h = torch.tensor(x).permute(0, 3, 1, 2)
+    for p in tp:
+        y = torch.nn.functional.conv2d(h, p['w'].permute(3, 2, 0, 1), padding=1)
+        h = torch.relu(torch.nn.functional.batch_norm(y, None, None, p['scale'], p['shift'], training=True, eps=1e-5))
+    expected = (h * h).sum() / h.numel()
+    expected.backward()
+    assert np.allclose(loss, expected.detach().numpy(), rtol=1e-5)
+    flat = [p[k].grad.numpy() for p in tp for k in sorted(p)]           #tree leaves come in sorted key order
+    assert len(flat) == len(grads)
+    for g, e in zip(grads, flat):
+        assert np.allclose(g, e, rtol=1e-4, atol=1e-6), float(np.abs(g - e).max())
+
+
+@pytest.mark.gpu
+def test_batch_norm_with_batch_statistics_hip():
+    for kwargs in (dict(), dict(seed=5, batch=8, size=12, channels=((4, 16), (16, 12)))):
+        args = _batch_stat_net_inputs(**kwargs)
+        for fuse in (True, False):
+            check_against_oracle(_batch_stat_net_step, args, rtol=1e-4, atol=1e-5, fuse=fuse)

@@ -160,6 +160,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
 
     result: tp.List[tp.Optional[Op]] = []
     producer: tp.Dict[int, int] = {}               #placeholder id -> position in `result` of the op that wrote it
+    last_reader: tp.Dict[int, int] = {}            #placeholder id -> position in `result` of the last op that read it
 
     def extend_lifetimes(op, index):
         for b in _reads(op):
@@ -203,6 +204,9 @@ def fuse_ops(all_ops, bufferpool, outvars):
 
     def conv_with_second_result(prod, op, pid):
         out, lhs, rhs, geom, epilogue = prod.conv
+        #the merged launch stands where the chain stood: nothing in between may have read the convolution's result
+        if last_reader.get(pid, -1) > producer[pid]:
+            return None
         steps = _continuation_steps(op.chain, out)
         if steps is None or tuple(out.shape) != tuple(op.chain.shape) or op.chain.out.size != out.size:
             return None
@@ -263,6 +267,8 @@ def fuse_ops(all_ops, bufferpool, outvars):
                 break
         new = fused if fused is not None else op
         result.append(new)
+        for b in _reads(new):
+            last_reader[id(b._placeholder)] = len(result) - 1
         out = _out(new)
         if out is not None:
             producer[id(out._placeholder)] = len(result) - 1
