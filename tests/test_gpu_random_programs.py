@@ -91,3 +91,77 @@ def test_random_program_hip(seed):
     print(f'case: random program {seed}', flush=True)
     for fuse in (True, False):
         check_against_oracle(f, args, exact=True, fuse=fuse)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Random small networks: convolutions followed by per-channel arithmetic, ReLU, residual additions and channel sums,
+# with intermediate results that are read more than once, forward only or with reverse-mode gradients. These are
+# the shapes the convolution epilogue, second-result, fused backward and batching passes look for; integer-valued
+# data keeps every sum exact, so fused and unfused runs must agree with the oracle bit for bit.
+N_NETWORKS = 60
+
+
+def make_network(seed):
+    rng = np.random.RandomState(5000 + seed)
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    batch, size, cin = int(rng.choice([1, 2, 3])), int(rng.choice([4, 5, 8])), int(rng.choice([4, 8]))
+    x = ints(-3, 4, batch, size, size, cin)
+    params, configs = [], []
+    for _ in range(rng.randint(1, 3)):
+        cout, k = int(rng.choice([4, 8, 12])), int(rng.choice([1, 3]))
+        params.append(dict(w=ints(-2, 3, k, k, cin, cout), mean=ints(-2, 3, cout), scale=ints(1, 3, cout), shift=ints(-3, 4, cout)))
+        configs.append((int(rng.choice([1, 1, 2])), int(rng.randint(0, 5))))
+        cin = cout
+    weights = ints(-2, 3, 1)[0]
+    with_gradients = bool(seed % 2)
+
+    def forward(params, x):
+        h, extras = x, []
+        for p, (stride, mode) in zip(params, configs):
+            y = lax.conv_general_dilated(h, p['w'], (stride, stride), 'SAME', dimension_numbers=('NHWC', 'HWIO', 'NHWC'))
+            if mode == 0:                                   #scale and shift with fixed statistics, ReLU
+                z = mj.nn.relu((y - p['mean']) * p['scale'] + p['shift'])
+            elif mode == 1:                                 #the centred result is read again AFTER the chain
+                centred = y - p['mean']
+                z = mj.nn.relu(centred * p['scale'] + p['shift'])
+                extras.append(jnp.sum(centred, axis=(0, 1, 2)))
+            elif mode == 2:                                 #the plain result is read BEFORE the chain that continues it
+                total = jnp.sum(y, axis=(0, 1, 2))
+                z = mj.nn.relu((y - lax.min(lax.max(total, -2.0), 2.0)) * p['scale'])
+                extras.append(total)
+            elif mode == 3:                                 #no activation
+                z = y * p['scale'] + p['shift']
+            else:                                           #residual connection where the shapes allow it
+                z = (y - p['mean']) * p['scale']
+                z = mj.nn.relu(z + h) if z.shape == h.shape else mj.nn.relu(z)
+            h = lax.min(lax.max(z, -8.0), 8.0)
+        return h, extras
+
+    if not with_gradients:
+        def program(params, x):
+            h, extras = forward(params, x)
+            return (h, *extras)
+    else:
+        def loss(params, x):
+            h, extras = forward(params, x)
+            return jnp.sum(h) * float(weights) + sum(jnp.sum(e) for e in extras)
+        def program(params, x):
+            return mj.value_and_grad(loss)(params, x)
+    return program, (params, x)
+
+
+@pytest.mark.parametrize('seed', range(N_NETWORKS))
+def test_random_network_plans(seed):
+    f, args = make_network(seed)
+    _, closed = oracle_outputs(f, args)
+    for fuse in (True, False):
+        JaxprInterpreter(closed, plan_only=True, fuse=fuse)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('seed', range(N_NETWORKS))
+def test_random_network_hip(seed):
+    f, args = make_network(seed)
+    print(f'case: random network {seed}', flush=True)
+    for fuse in (True, False):
+        check_against_oracle(f, args, exact=True, fuse=fuse)
