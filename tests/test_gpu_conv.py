@@ -244,3 +244,17 @@ def test_convolution_with_a_second_result():
         flags = int(np.frombuffer(launches[0].params, dtype=np.uint32)[21])
         assert (flags >> 12) & 15 in (1, 2), hex(flags)
         check_against_oracle(f, args, exact=True, fuse=False)
+
+
+def test_single_image_with_a_one_column_result():
+    '''Batch 1 and an output one column wide, with stride, padding or taps outside the input: the matrix-product
+    shortcut of the 16-byte loader (output row = input row) must not be taken. Integer-valued, exact.'''
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    cases = [((1, 2, 2, 12), (3, 3, 12, 8), 2, ((0, 1), (0, 1))), ((1, 2, 2, 12), (3, 3, 12, 8), 1, ((0, 1), (0, 1))),
+             ((1, 2, 2, 12), (3, 3, 12, 8), 2, ((1, 0), (1, 0))), ((1, 4, 2, 12), (3, 3, 12, 8), 2, ((0, 1), (0, 1))),
+             ((1, 2, 2, 32), (3, 3, 32, 8), 2, ((0, 1), (0, 1))), ((1, 6, 1, 16), (3, 1, 16, 8), 2, ((0, 0), (0, 0))),
+             ((1, 6, 1, 16), (3, 1, 16, 8), 1, ((0, 0), (0, 0))), ((1, 5, 3, 64), (3, 3, 64, 64), 1, ((1, 1), (0, 0)))]
+    for xs, ks, stride, pad in cases:
+        print(f'case: {xs} {ks} stride {stride} padding {pad}', flush=True)
+        f = lambda x, k: lax.conv_general_dilated(x, k, (stride, stride), pad, dimension_numbers=NHWC)
+        check_against_oracle(f, [ints(-3, 4, *xs), ints(-2, 3, *ks)], exact=True)

@@ -53,8 +53,8 @@ struct ConvParams {
     int32_t SH, SW, PH, PW, DH, DW;
     int32_t xs_b, xs_h, xs_w;       // lhs strides in elements
     int32_t tiles_m, tiles_n;
-    uint32_t flags;                 // bit0: out is row-major [M, N]; bit1: m is the row index itself
-                                    // (batch = Wo = 1: no row decode); bit2: some kernel taps of some
+    uint32_t flags;                 // bit0: out is row-major [M, N]; bit1: m is the input row index itself
+                                    // (batch = Wo = 1, stride 1, no padding: no row decode, no masks); bit2: some kernel taps of some
                                     // rows fall outside the input; bits 8-11: number of epilogue
                                     // steps; bits 12-15: 0, or 1 + t: the value after t template steps
                                     // (t = 0, or t = 1 after `acc - vector`) is ALSO stored, laid out like

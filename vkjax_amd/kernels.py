@@ -543,7 +543,9 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     #the lean kernel variant covers the common case only (see the kernel source)
     lean = (a_fast and b_fast and c_contig and (g.Cin % bk == 0 or g.KH * g.KW == 1)
             and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL)
-    flat_rows = g.batch == 1 and g.Wo == 1
+    #the output row number is the input row number (a matrix product, or a one-column image walked without stride,
+    #padding or taps outside the input): the kernel then skips the row decode and the validity masks
+    flat_rows = g.batch == 1 and g.Wo == 1 and g.SH == 1 and g.PH == 0 and g.PW == 0 and not needs_masks
     #a product with so few 32 x 32 tiles that one wave per tile leaves most MFMA units idle: four waves per
     #tile, each taking a quarter of every (128-long) k step
     ksplit = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
