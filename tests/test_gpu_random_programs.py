@@ -165,3 +165,74 @@ def test_random_network_hip(seed):
     print(f'case: random network {seed}', flush=True)
     for fuse in (True, False):
         check_against_oracle(f, args, exact=True, fuse=fuse)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Random geometry of single primitives: convolutions (batch, image and kernel sizes from 1 up, strides, dilations,
+# uneven padding) and their gradients, matrix products of odd sizes in all three layouts, pooling windows, row
+# gathers and scatter-adds. Integer-valued data: exact results, fused and unfused.
+N_GEOMETRIES = 160
+dn = ('NHWC', 'HWIO', 'NHWC')
+
+
+def make_geometry_case(seed):
+    rng = np.random.RandomState(9000 + seed)
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    kind = ['conv', 'conv', 'conv', 'dot', 'pool', 'gather', 'scatter', 'convgrad'][seed % 8]
+    if kind in ('conv', 'convgrad'):
+        b, h, w = int(rng.choice([1, 1, 2, 3])), int(rng.randint(1, 10)), int(rng.randint(1, 10))
+        cin, cout = int(rng.choice([1, 3, 4, 8, 12, 16, 32])), int(rng.choice([1, 4, 5, 8, 16, 64]))
+        kh, kw = int(rng.choice([1, 2, 3])), int(rng.choice([1, 2, 3]))
+        sh, sw = int(rng.choice([1, 1, 2, 3])), int(rng.choice([1, 1, 2]))
+        dh, dw = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
+        pad = ((int(rng.randint(0, 3)), int(rng.randint(0, 3))), (int(rng.randint(0, 3)), int(rng.randint(0, 3))))
+        eh, ew = (kh - 1) * dh + 1, (kw - 1) * dw + 1
+        if h + sum(pad[0]) < eh or w + sum(pad[1]) < ew:
+            pad = ((eh, eh), (ew, ew))
+        x, k = ints(-3, 4, b, h, w, cin), ints(-2, 3, kh, kw, cin, cout)
+        conv = lambda x, k: lax.conv_general_dilated(x, k, (sh, sw), pad, rhs_dilation=(dh, dw), dimension_numbers=dn)
+        if kind == 'conv':
+            return f'conv x{x.shape} k{k.shape} s{(sh, sw)} d{(dh, dw)} p{pad}', conv, [x, k]
+        return f'convgrad x{x.shape} k{k.shape} s{(sh, sw)} d{(dh, dw)} p{pad}', (lambda x, k: mj.value_and_grad(lambda p: jnp.sum(conv(p[0], p[1]) * 2.0))((x, k))), [x, k]
+    if kind == 'dot':
+        m, n, kk = int(rng.choice([1, 2, 7, 33, 64, 130])), int(rng.choice([1, 3, 4, 10, 64, 72])), int(rng.choice([1, 2, 5, 16, 127, 128, 260]))
+        a, b = ints(-3, 4, m, kk), ints(-2, 3, kk, n)
+        variant = rng.randint(0, 3)
+        if variant == 0: return f'dot {m}x{kk}x{n}', (lambda a, b: jnp.dot(a, b)), [a, b]
+        if variant == 1: return f'dot^T {m}x{kk}x{n}', (lambda a, b: jnp.dot(a, lax.transpose(b, (1, 0)))), [a, np.ascontiguousarray(b.T)]
+        return f'dot T^ {m}x{kk}x{n}', (lambda a, b: jnp.dot(lax.transpose(a, (1, 0)), b)), [np.ascontiguousarray(a.T), b]
+    if kind == 'pool':
+        b, h, w, c = int(rng.choice([1, 2])), int(rng.randint(1, 12)), int(rng.randint(1, 12)), int(rng.choice([1, 3, 4, 8, 64]))
+        wh, ww = int(rng.choice([1, 2, 3])), int(rng.choice([1, 2, 3]))
+        sh, sw = int(rng.choice([1, 2, 3])), int(rng.choice([1, 2]))
+        pad = ((0, 0), (int(rng.randint(0, 2)), int(rng.randint(0, 3))), (int(rng.randint(0, 2)), int(rng.randint(0, 3))), (0, 0))
+        if h + sum(pad[1]) < wh or w + sum(pad[2]) < ww:
+            pad = ((0, 0), (wh, wh), (ww, ww), (0, 0))
+        x = ints(-9, 10, b, h, w, c)
+        if rng.randint(0, 2):
+            return f'maxpool x{x.shape} w{(wh, ww)} s{(sh, sw)} p{pad}', (lambda x: lax.reduce_window(x, -jnp.inf, lax.max, (1, wh, ww, 1), (1, sh, sw, 1), pad)), [x]
+        return f'sumpool x{x.shape} w{(wh, ww)} s{(sh, sw)} p{pad}', (lambda x: lax.reduce_window(x, 0.0, lax.add, (1, wh, ww, 1), (1, sh, sw, 1), pad)), [x]
+    rows, cols = int(rng.choice([1, 5, 64, 300])), int(rng.choice([1, 3, 4, 64, 256]))
+    nidx = int(rng.choice([1, 2, 17, 256, 1000]))
+    table, idx = ints(-9, 10, rows, cols), rng.randint(0, rows, size=(nidx,)).astype(np.int32)
+    if kind == 'gather':
+        return f'gather {rows}x{cols} <- {nidx}', (lambda t, i: t[i]), [table, idx]
+    upd = ints(-3, 4, nidx, cols)
+    return f'scatter-add {rows}x{cols} <- {nidx}', (lambda t, i, u: t.at[i].add(u)), [table, idx, upd]
+
+
+@pytest.mark.parametrize('seed', range(N_GEOMETRIES))
+def test_random_geometry_plans(seed):
+    name, f, args = make_geometry_case(seed)
+    _, closed = oracle_outputs(f, args)
+    for fuse in (True, False):
+        JaxprInterpreter(closed, plan_only=True, fuse=fuse)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('seed', range(N_GEOMETRIES))
+def test_random_geometry_hip(seed):
+    name, f, args = make_geometry_case(seed)
+    print(f'case: random geometry {seed}: {name}', flush=True)
+    for fuse in (True, False):
+        check_against_oracle(f, args, exact=True, fuse=fuse)
