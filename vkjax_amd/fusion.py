@@ -857,7 +857,7 @@ def batch_small_chains(ops):
             i += 1
             continue
         j = i
-        while j < len(moved) and _is_small(moved[j]):
+        while j < len(moved) and j - i < 256 and _is_small(moved[j]):      #(levels are found pair by pair: bounded runs)
             j += 1
         run, level = moved[i:j], []
         for k, op in enumerate(run):
