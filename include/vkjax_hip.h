@@ -5,9 +5,10 @@
  * Python (kp.Manager / kp.Tensor / kp.Sequence / kp.OpAlgoDispatch / kp.OpTensorSync*,
  * package kp==0.7.0): a device context, HBM buffers, gfx950 code objects and a recorded
  * sequence of uploads, kernel launches and downloads that is replayed with ONE call per
- * run. All work of a context is issued on one in-order HIP stream; nothing synchronises
- * with the host except the tail of vkj_seq_eval / vkj_seq_replay, the blocking buffer
- * transfers and vkj_sync.
+ * run. All work of a context is issued on one in-order HIP stream (vkj_seq_eval_next adds
+ * a second one that only carries the following call's uploads); nothing synchronises
+ * with the host except the tail of vkj_seq_eval / vkj_seq_eval_next / vkj_seq_replay, the
+ * blocking buffer transfers and vkj_sync.
  *
  * Conventions: every function returns 0 on success, a positive hipError_t or a negative
  * VKJ_E* code otherwise; vkj_last_error() returns the message of the calling thread's last
