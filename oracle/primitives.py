@@ -388,12 +388,18 @@ def conv_general_dilated(lhs, rhs, window_strides, padding, lhs_dilation, rhs_di
     hd, wdd = ((h - 1) * ld0 + 1 if h else 0), ((wd - 1) * ld1 + 1 if wd else 0)
     xd = np.zeros((n, hd, wdd, c))
     xd[:, ::ld0, ::ld1, :] = x
-    #negative padding crops
+    #negative padding crops; a crop that reaches beyond the array's other end leaves nothing of it, but the
+    #padded size is still m + lo + hi (element i of the padded axis is element i - lo of the array)
     def pad_or_crop(a, axis, lo, hi):
-        if lo < 0: a = np.take(a, range(-lo, a.shape[axis]), axis=axis); lo = 0
-        if hi < 0: a = np.take(a, range(0, a.shape[axis] + hi), axis=axis); hi = 0
-        pads = [(0, 0)] * a.ndim; pads[axis] = (lo, hi)
-        return np.pad(a, pads)
+        m = a.shape[axis]
+        size = builtins_max(m + lo + hi, 0)
+        grown = np.zeros(a.shape[:axis] + (size,) + a.shape[axis + 1:])
+        src_lo, dst_lo = builtins_max(-lo, 0), builtins_max(lo, 0)
+        length = builtins_max(builtins_min(m - src_lo - builtins_max(-hi, 0), size - dst_lo), 0)
+        src, dst = [np.s_[:]] * a.ndim, [np.s_[:]] * a.ndim
+        src[axis], dst[axis] = np.s_[src_lo:src_lo + length], np.s_[dst_lo:dst_lo + length]
+        grown[tuple(dst)] = a[tuple(src)]
+        return grown
     xp = pad_or_crop(pad_or_crop(xd, 1, p0lo, p0hi), 2, p1lo, p1hi)
     keh, kew = (kh - 1) * rd0 + 1, (kw - 1) * rd1 + 1
     ho = (xp.shape[1] - keh) // s0 + 1 if xp.shape[1] >= keh else 0

@@ -258,3 +258,15 @@ def test_single_image_with_a_one_column_result():
         print(f'case: {xs} {ks} stride {stride} padding {pad}', flush=True)
         f = lambda x, k: lax.conv_general_dilated(x, k, (stride, stride), pad, dimension_numbers=NHWC)
         check_against_oracle(f, [ints(-3, 4, *xs), ints(-2, 3, *ks)], exact=True)
+
+
+def test_gradient_of_a_strided_convolution_that_skips_the_whole_input():
+    '''A stride that steps over the only input row: the input gradient is a convolution whose (negative) padding
+    crops more than the cotangent holds. Every tap then lies outside, and the padded size still counts.'''
+    from vkjax_amd import minijax as mj
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    x, k = ints(-3, 4, 2, 1, 5, 12), ints(-2, 3, 1, 2, 12, 16)
+    conv = lambda x, k: lax.conv_general_dilated(x, k, (3, 1), ((2, 0), (2, 2)), rhs_dilation=(2, 1), dimension_numbers=NHWC)
+    f = lambda x, k: mj.value_and_grad(lambda p: jnp.sum(conv(p[0], p[1]) * 2.0))((x, k))
+    for fuse in (True, False):
+        check_against_oracle(f, [x, k], exact=True, fuse=fuse)

@@ -315,3 +315,26 @@ def test_reductions_over_no_elements_return_the_init_value():
     x = np.array([[1.0, -3.0, np.nan], [2.0, 5.0, -1.0]], np.float32)
     assert np.array_equal(P.reduce_max(x, (1,)), np.array([np.nan, 5.0], np.float32), equal_nan=True)
     assert np.array_equal(P.reduce_min(x, (0,)), np.array([1.0, -3.0, np.nan], np.float32), equal_nan=True)
+
+
+def test_convolution_with_a_crop_that_reaches_beyond_the_input():
+    '''Negative padding larger than the input: the padded axis still has in + lo + hi positions, all of them
+    outside the input. Brute force over the definition (element i of the padded axis is element i - lo).'''
+    from oracle import primitives as P
+    rng = np.random.default_rng(3)
+    x, w = rng.standard_normal((2, 1, 5, 3)), rng.standard_normal((1, 2, 3, 4))
+    padding = ((-2, 2), (1, 0))
+    dn = ((0, 3, 1, 2), (3, 2, 0, 1), (0, 3, 1, 2))
+    got = P.conv_general_dilated(x, w, (1, 1), padding, (1, 1), (1, 1), dn)
+    Ho, Wo = 1 - 2 + 2 - 1 + 1, 5 + 1 + 0 - 2 + 1
+    want = np.zeros((2, Ho, Wo, 4))
+    for b in range(2):
+        for ho in range(Ho):
+            for wo in range(Wo):
+                for ky in range(1):
+                    for kx in range(2):
+                        y, xx = ho + ky - padding[0][0], wo + kx - padding[1][0]
+                        if 0 <= y < 1 and 0 <= xx < 5:
+                            want[b, ho, wo] += x[b, y, xx] @ w[ky, kx]
+    assert got.shape == want.shape and np.allclose(got, want, atol=1e-6)
+    assert not np.any(got)                                  #every tap of every position lies outside the input
