@@ -117,6 +117,7 @@ def _bitop(f):
 
 globals()['or']  = _bitop(np.bitwise_or)
 globals()['and'] = _bitop(np.bitwise_and)
+xor = _bitop(np.bitwise_xor)
 bit_or, bit_and = globals()['or'], globals()['and']
 
 

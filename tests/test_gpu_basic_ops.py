@@ -232,6 +232,8 @@ param_matrix += [
     (lax.is_finite, 'is_finite',        [_special]),
     (lax.bitwise_not, 'not bool',       [random([77, 101]) > 0.5]),
     (lax.bitwise_not, 'not int',        [randint(-2**31, 2**31, size=[77, 101])]),
+    (lax.bitwise_xor, 'xor int',        [randint(-2**31, 2**31, size=[77, 101]), randint(-2**31, 2**31, size=[77, 101])]),
+    (lax.bitwise_xor, 'xor bool',       [random([77, 101]) > 0.5, random([77, 101]) > 0.3]),
     (lax.population_count, 'popcount',  [randint(0, 2**32, size=[77, 101], dtype=np.uint64).astype(np.uint32)]),
     (lax.clz, 'clz',                    [np.concatenate([[0, 1, 2**31, 2**32 - 1], 2**randint(0, 32, size=500) - 1]).astype(np.uint32)]),
     (lax.square, 'square float',        [random([77, 101]) * 20 - 10]),

@@ -78,6 +78,7 @@ def eq(x, y): return _binary('eq', x, y, out_dtype=_bool)
 def ne(x, y): return _binary('ne', x, y, out_dtype=_bool)
 def bitwise_or(x, y):  return _binary('or', x, y, allowed=(_i32, _u32, _bool))
 def bitwise_and(x, y): return _binary('and', x, y, allowed=(_i32, _u32, _bool))
+def bitwise_xor(x, y): return _binary('xor', x, y, allowed=(_i32, _u32, _bool))
 def shift_left(x, y):  return _binary('shift_left', x, y, allowed=(_i32, _u32))
 def shift_right_logical(x, y):    return _binary('shift_right_logical', x, y, allowed=(_i32, _u32))
 def shift_right_arithmetic(x, y): return _binary('shift_right_arithmetic', x, y, allowed=(_i32, _u32))
