@@ -17,6 +17,9 @@ _CALLS = {
     'closed_call':           lambda params: params['call_jaxpr'],
     'custom_jvp_call_jaxpr': lambda params: params['fun_jaxpr'],
     'custom_jvp_call':       lambda params: params['call_jaxpr'],
+    'custom_vjp_call':       lambda params: params['call_jaxpr'] if 'call_jaxpr' in params else params['fun_jaxpr'],
+    'custom_vjp_call_jaxpr': lambda params: params['call_jaxpr'] if 'call_jaxpr' in params else params['fun_jaxpr'],
+    'remat':                 lambda params: params['call_jaxpr'],
 }
 
 

@@ -266,6 +266,27 @@ def select(pred, on_true, on_false):
     return np.where(np.asarray(pred, bool), _canon(on_true), _canon(on_false))
 
 
+def select_n(which, *cases):
+    '''select_n of newer jax: case k where `which` is k; for a boolean `which`, case 1 where it is true.'''
+    which = np.asarray(which)
+    if which.dtype == np.bool_:
+        assert len(cases) == 2
+        return np.where(which, _canon(cases[1]), _canon(cases[0]))
+    return np.choose(which, [_canon(c) for c in cases])
+
+
+def copy(x, **_):
+    return _canon(x).copy()
+
+
+copy_p = copy
+
+
+def optimization_barrier(*operands, **_):
+    '''Identity on every operand (a scheduling fence for XLA, nothing to compute).'''
+    return [_canon(x) for x in operands]
+
+
 def convert_element_type(x, new_dtype, **_):
     '''float -> int truncates toward zero and saturates; NaN -> 0 (XLA). bool -> 0/1.
     reference: vkjax/shaders/convert_element_type.comp:9-12.'''

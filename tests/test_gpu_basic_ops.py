@@ -368,3 +368,37 @@ def test_arrays_without_elements():
         n = len(list(fn._jaxpr_interpreters.values())[0].launches)
         assert launches is None or n == launches, (name, n)
         check_against_oracle(f, args, exact=True, fuse=False)
+
+
+def test_call_and_alias_primitives_of_newer_jax():
+    '''The names and parameter layouts newer jax versions put into a jaxpr where the reference's era had xla_call /
+    custom_jvp_call_jaxpr / select: pjit and jit (a closed jaxpr under `jaxpr`), closed_call / core_call / remat
+    (`call_jaxpr`), custom_jvp_call (`call_jaxpr`), custom_vjp_call with either parameter name, copy, copy_p,
+    optimization_barrier on several operands, select_n. The stand-in tracer does not produce them by itself, so the
+    equations are emitted by hand, each around a body with a closed-over constant.'''
+    from vkjax_amd.minijax import tracer, core
+    bias = np.arange(12, dtype=np.float32).reshape(3, 4)
+    body = lambda x, y: (lax.max(x * y + bias, 0.0), x - y)
+
+    def nested(primitive, jaxpr_param, closed, **extra):
+        return lambda x, y: tracer._call_nested(body, primitive, jaxpr_param, extra, closed=closed, args=(x, y))
+    def aliases(x, y):
+        a = tracer.emit('copy', [x], [core.ShapedArray(x.shape, x.dtype)])
+        b = tracer.emit('copy_p', [y], [core.ShapedArray(y.shape, y.dtype)])
+        a, b = tracer.emit('optimization_barrier', [a, b], [core.ShapedArray(x.shape, x.dtype)] * 2, multiple_results=True)
+        pick = tracer.emit('select_n', [lax.gt(a, b), a, b], [core.ShapedArray(x.shape, x.dtype)])       #b where a > b
+        return pick * 2.0, a + b
+    cases = [('pjit', nested('pjit', 'jaxpr', True, name='body', donated_invars=(False, False), inline=False, keep_unused=False)),
+             ('jit', nested('jit', 'jaxpr', True, name='body')),
+             ('closed_call', nested('closed_call', 'call_jaxpr', True)),
+             ('core_call', nested('core_call', 'call_jaxpr', False)),
+             ('remat', nested('remat', 'call_jaxpr', False, prevent_cse=True, differentiated=False)),
+             ('custom_jvp_call', nested('custom_jvp_call', 'call_jaxpr', True, num_consts=0, symbolic_zeros=False, jvp_jaxpr_fun=None)),
+             ('custom_vjp_call', nested('custom_vjp_call', 'call_jaxpr', True, num_consts=0, bwd=None, fwd_jaxpr_thunk=None, out_trees=None, symbolic_zeros=False)),
+             ('custom_vjp_call_jaxpr', nested('custom_vjp_call_jaxpr', 'fun_jaxpr', True, num_consts=0, bwd=None, fwd_jaxpr_thunk=None, out_trees=None)),
+             ('copy, optimization_barrier, select_n', aliases)]
+    x, y = random([3, 4]) - 0.5, random([3, 4]) - 0.5
+    for name, f in cases:
+        print(f'case: {name}', flush=True)
+        check_against_oracle(f, [x, y], rtol=1e-6, atol=1e-7)
+        check_against_oracle(f, [x, y], rtol=1e-6, atol=1e-7, fuse=False)
