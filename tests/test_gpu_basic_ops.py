@@ -232,6 +232,7 @@ param_matrix += [
     (lax.is_finite, 'is_finite',        [_special]),
     (lax.bitwise_not, 'not bool',       [random([77, 101]) > 0.5]),
     (lax.bitwise_not, 'not int',        [randint(-2**31, 2**31, size=[77, 101])]),
+    (lax.sqrt, 'sqrt',                  [np.concatenate([random([500]) * 1e4, [0.0, 1.0, 4.0, np.inf, -1.0, 2.0 ** -140]]).astype(np.float32)]),
     (lax.bitwise_xor, 'xor int',        [randint(-2**31, 2**31, size=[77, 101]), randint(-2**31, 2**31, size=[77, 101])]),
     (lax.bitwise_xor, 'xor bool',       [random([77, 101]) > 0.5, random([77, 101]) > 0.3]),
     (lax.population_count, 'popcount',  [randint(0, 2**32, size=[77, 101], dtype=np.uint64).astype(np.uint32)]),
@@ -387,7 +388,8 @@ def test_call_and_alias_primitives_of_newer_jax():
         b = tracer.emit('copy_p', [y], [core.ShapedArray(y.shape, y.dtype)])
         a, b = tracer.emit('optimization_barrier', [a, b], [core.ShapedArray(x.shape, x.dtype)] * 2, multiple_results=True)
         pick = tracer.emit('select_n', [lax.gt(a, b), a, b], [core.ShapedArray(x.shape, x.dtype)])       #b where a > b
-        return pick * 2.0, a + b
+        wide = tracer.emit('expand_dims', [pick], [core.ShapedArray((1,) + tuple(x.shape) + (1,), x.dtype)], dict(dimensions=(0, 3)))
+        return pick * 2.0, a + b, wide + 1.0
     cases = [('pjit', nested('pjit', 'jaxpr', True, name='body', donated_invars=(False, False), inline=False, keep_unused=False)),
              ('jit', nested('jit', 'jaxpr', True, name='body')),
              ('closed_call', nested('closed_call', 'call_jaxpr', True)),
