@@ -190,9 +190,17 @@ def make_geometry_case(seed):
         if h + sum(pad[0]) < eh or w + sum(pad[1]) < ew:
             pad = ((eh, eh), (ew, ew))
         x, k = ints(-3, 4, b, h, w, cin), ints(-2, 3, kh, kw, cin, cout)
-        conv = lambda x, k: lax.conv_general_dilated(x, k, (sh, sw), pad, rhs_dilation=(dh, dw), dimension_numbers=dn)
+        #the second half of the seeds also draws an input dilation and other dimension numbers
+        ld = [(1, 1), (1, 1), (2, 1), (2, 2), (3, 2)][rng.randint(0, 5)] if seed >= N_GEOMETRIES // 2 else (1, 1)
+        layout = rng.randint(0, 3) if seed >= N_GEOMETRIES // 2 else 0
+        dnums = [('NHWC', 'HWIO', 'NHWC'), ('NCHW', 'OIHW', 'NCHW'), ('NHWC', 'OIHW', 'NCHW')][layout]
+        if layout == 1:
+            x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+        if layout in (1, 2):
+            k = np.ascontiguousarray(k.transpose(3, 2, 0, 1))
+        conv = lambda x, k: lax.conv_general_dilated(x, k, (sh, sw), pad, lhs_dilation=ld, rhs_dilation=(dh, dw), dimension_numbers=dnums)
         if kind == 'conv':
-            return f'conv x{x.shape} k{k.shape} s{(sh, sw)} d{(dh, dw)} p{pad}', conv, [x, k]
+            return f'conv x{x.shape} k{k.shape} s{(sh, sw)} d{(dh, dw)} ld{ld} p{pad} {dnums}', conv, [x, k]
         return f'convgrad x{x.shape} k{k.shape} s{(sh, sw)} d{(dh, dw)} p{pad}', (lambda x, k: mj.value_and_grad(lambda p: jnp.sum(conv(p[0], p[1]) * 2.0))((x, k))), [x, k]
     if kind == 'dot':
         m, n, kk = int(rng.choice([1, 2, 7, 33, 64, 130])), int(rng.choice([1, 3, 4, 10, 64, 72])), int(rng.choice([1, 2, 5, 16, 127, 128, 260]))
