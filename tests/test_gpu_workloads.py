@@ -284,3 +284,16 @@ def test_stream_matches_call_by_call():
     next(it)
     it.close()
     assert_tree_close(fast(*small[0]), plain(*small[0]), exact=True, what='call after an abandoned stream')
+
+    #the same with resident weights: what the helper thread had prepared ahead must not count as uploaded ...
+    it = resident.stream(iter(batches))
+    next(it)
+    it.close()
+    for k in (3, 0, 2):
+        assert_tree_close(resident(*batches[k]), expected[k], exact=True, what=f'resident call {k} after an abandoned stream')
+    #... and other calls of the function while a stream is suspended do not disturb it (nor it them)
+    it = resident.stream(iter(batches))
+    for k in range(len(batches)):
+        assert_tree_close(next(it), expected[k], exact=True, what=f'suspended stream [{k}]')
+        other = (k * 2 + 1) % len(batches)
+        assert_tree_close(resident(*batches[other]), expected[other], exact=True, what=f'call {other} between stream results')

@@ -124,27 +124,35 @@ class Function:
             if entry is None:
                 caught_up.clear()
                 return [None, None, args]
-            return [entry, self._output_shapes[signature], entry._host_inputs(args)]
+            return [entry, self._output_shapes[signature], entry._convert_inputs(args)]
 
         def resolved(item):
             if item is not None and item[0] is None:
                 interpreter, output_shapes = self._get_or_create_jaxpr_interpreter(item[2])
-                item[:] = [interpreter, output_shapes, interpreter._host_inputs(item[2])]
+                item[:] = [interpreter, output_shapes, interpreter._convert_inputs(item[2])]
                 caught_up.set()
             return item
 
         ahead = _Ahead(argument_tuples, prepare, wake=caught_up)
         try:
+            # The helper only converts arguments. Which of them have to be copied (resident ones that changed) is
+            # settled here, immediately before the evaluation that copies them, so that what the interpreter notes as
+            # held in HBM is true at every point where the consumer may stop or call the function in between.
             items   = iter(ahead)
             current = resolved(next(items, None))
+            in_place = False                                     #current's arguments were uploaded by the previous evaluation
             while current is not None:
-                interpreter, output_shapes, host = current
+                interpreter, output_shapes, converted = current
+                if in_place and interpreter._evaluations != stamp:
+                    in_place = False                             #something else used the argument buffers in between
+                host      = [None] * interpreter.sequence.n_slots if in_place else interpreter._select_uploads(converted)
                 following = resolved(next(items, None))
-                next_host = following[2] if following is not None and following[0] is interpreter else None
+                overlap   = following is not None and following[0] is interpreter
+                next_host = interpreter._select_uploads(following[2]) if overlap else None
                 fresh     = interpreter._fresh_outputs(host)
                 interpreter.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT, next_host_arrays=next_host)
-                if next_host is not None:
-                    following[2] = [None] * interpreter.sequence.n_slots      #in place by now
+                interpreter._evaluations += 1
+                stamp, in_place = interpreter._evaluations, overlap
                 yield self._restore_shapes(interpreter._output_values(fresh), output_shapes)
                 current = following
         finally:

@@ -41,6 +41,8 @@ class JaxprInterpreter:
         self.workgroup_size = get_maximum_workgroup_size(self.mgr)
         self.bufferpool     = BufferPool(self.mgr, self.workgroup_size, reuse_buffers)
         self.sequence       = None
+        #counts evaluations: a suspended stream sees from it whether something else has used the argument buffers
+        self._evaluations   = 0
         self.analyze_closed_jaxpr(jaxpr)
 
     def analyze_closed_jaxpr(self, jaxpr):
@@ -114,26 +116,40 @@ class JaxprInterpreter:
             raise TypeError(f'Expected {len(self.input_buffers)} input arguments, received {len(leaves)}')
         return (leaves, resident) if with_residency else leaves
 
-    def _host_inputs(self, X) -> tp.List[tp.Optional[np.ndarray]]:
-        '''One entry per transfer slot: the device words of every argument that has to be copied.'''
+    def _convert_inputs(self, X) -> tp.List[tp.Tuple]:
+        '''(leaf number, transfer slot, the leaf, its device words, whether it is a resident one) for every argument
+        leaf the program reads. Touches no state of the interpreter: it may run ahead of the evaluation it is for.'''
         X, resident = self._flatten_args(X, with_residency=True)
         if self.sequence is None:
             raise RuntimeError('this interpreter was built with plan_only=True and has no device to run on')
-        host = [None] * self.sequence.n_slots
+        converted = []
         for k, (slot, x, var) in enumerate(zip(self._input_slots, X, self.jaxpr.jaxpr.invars)):
             if slot is None:
                 continue
-            if resident[k]:
-                if self._resident_leaves.get(k) is x:
-                    continue                                    #already in HBM
-                self._resident_leaves[k] = x
             #the common case without the general conversion: an array that already is what the device holds
             n, dtype = self._input_specs[k]
             if type(x) is np.ndarray and x.dtype == dtype and x.size == n and x.flags.c_contiguous:
-                host[slot] = x.reshape(-1).view(np.uint32)
+                words = x.reshape(-1).view(np.uint32)
             else:
-                host[slot] = _device_words_of_argument(x, var.aval)
+                words = _device_words_of_argument(x, var.aval)
+            converted.append((k, slot, x, words, resident[k]))
+        return converted
+
+    def _select_uploads(self, converted) -> tp.List[tp.Optional[np.ndarray]]:
+        '''One entry per transfer slot: the device words of every leaf that has to be copied. A resident leaf is
+        copied when the object passed for it is not the one its buffer holds, and is noted as held from here on:
+        to be called only when the evaluation that uploads these arguments follows at once.'''
+        host = [None] * self.sequence.n_slots
+        for k, slot, x, words, is_resident in converted:
+            if is_resident:
+                if self._resident_leaves.get(k) is x:
+                    continue                                    #already in HBM
+                self._resident_leaves[k] = x
+            host[slot] = words
         return host
+
+    def _host_inputs(self, X) -> tp.List[tp.Optional[np.ndarray]]:
+        return self._select_uploads(self._convert_inputs(X))
 
     def _fresh_outputs(self, host) -> tp.List[tp.Optional[np.ndarray]]:
         #every call hands out fresh arrays: the runtime copies the results straight into them
@@ -152,6 +168,7 @@ class JaxprInterpreter:
         host  = self._host_inputs(X)
         fresh = self._fresh_outputs(host)
         self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT if self.resident_argnums else 0)
+        self._evaluations += 1
         output_values = self._output_values(fresh)
         if not return_all:
             return output_values
@@ -169,16 +186,21 @@ class JaxprInterpreter:
         current  = next(iterator, end)
         if current is end:
             return
-        host = self._host_inputs(tuple(current))
+        in_place = False                                         #current's arguments were uploaded by the previous evaluation
         while True:
+            if in_place and self._evaluations != stamp:
+                in_place = False                                 #something else used the argument buffers in between
+            host      = [None] * self.sequence.n_slots if in_place else self._host_inputs(tuple(current))
             following = next(iterator, end)
             next_host = self._host_inputs(tuple(following)) if following is not end else None
             fresh     = self._fresh_outputs(host)
             self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT, next_host_arrays=next_host)
+            self._evaluations += 1
+            stamp, in_place = self._evaluations, following is not end
             yield self._output_values(fresh)
             if following is end:
                 return
-            host = [None] * self.sequence.n_slots                #everything is in place already
+            current = following
 
     def upload_inputs(self, *X):
         '''Copy arguments into their HBM buffers without running (for measurements with resident inputs).'''
