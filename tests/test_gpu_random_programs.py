@@ -244,3 +244,93 @@ def test_random_geometry_hip(seed):
     print(f'case: random geometry {seed}: {name}', flush=True)
     for fuse in (True, False):
         check_against_oracle(f, args, exact=True, fuse=fuse)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Random parameters of the remaining primitives: pad (negative and interior padding), concatenate (empty parts),
+# argmax / argmin (NaNs, ties), products, broadcasts, indexing with negative and repeated indices, scatter-add along
+# the first dimension, take_along_axis, iota, clamp / integer_pow, window reductions over any dimensions of
+# rank-3 and rank-4 arrays. Integer-valued, exact, fused and unfused.
+N_MISC = 120
+
+
+def make_misc_case(seed):
+    rng = np.random.RandomState(64000 + seed)
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    kind = ['pad', 'concat', 'argext', 'prod', 'bcast', 'index1', 'index2', 'scatter_dim', 'take_along', 'iota', 'clamp_pow', 'pool_general'][seed % 12]
+    rank = rng.randint(1, 4)
+    shape = tuple(int(rng.choice([1, 2, 3, 5, 8, 16, 33])) for _ in range(rank))
+    x = ints(-4, 5, *shape)
+    if kind == 'pad':
+        cfg = tuple((int(rng.randint(-2, 4)), int(rng.randint(-2, 4)), int(rng.randint(0, 3))) for _ in shape)
+        for d, (lo, hi, it) in enumerate(cfg):
+            if shape[d] + (shape[d] - 1) * it + lo + hi < 0: cfg = tuple((0, 0, 0) for _ in shape)
+        return f'pad {shape} {cfg}', (lambda x: lax.pad(x, 7.0, cfg)), [x]
+    if kind == 'concat':
+        axis = rng.randint(0, rank); parts = []
+        for _ in range(rng.randint(1, 5)):
+            s = list(shape); s[axis] = int(rng.choice([0, 1, 3, 4, 9])); parts.append(ints(-4, 5, *s))
+        if sum(p.shape[axis] for p in parts) == 0: parts.append(x)
+        return f'concat axis {axis} {[p.shape for p in parts]}', (lambda *ps: lax.concatenate(list(ps), axis)), parts
+    if kind == 'argext':
+        axis = rng.randint(0, rank)
+        xs = x.copy()
+        if rng.randint(0, 3) == 0: xs.flat[rng.randint(0, xs.size)] = np.nan
+        fn = [jnp.argmax, jnp.argmin][rng.randint(0, 2)]
+        return f'{fn.__name__} {shape} axis {axis}', (lambda x: fn(x, axis=axis)), [xs]
+    if kind == 'prod':
+        axis = rng.randint(0, rank)
+        return f'prod {shape} axis {axis}', (lambda x: lax.reduce_prod(lax.min(lax.max(x, -2.0), 2.0), (axis,))), [x]
+    if kind == 'bcast':
+        new = (int(rng.choice([1, 2, 5])),) + shape + (int(rng.choice([1, 3, 4])),)
+        return f'broadcast {shape} -> {new}', (lambda x: lax.broadcast_in_dim(x, new, tuple(range(1, rank + 1))) + 1.0), [x]
+    if kind == 'index1':
+        idx = rng.randint(-shape[0], shape[0], size=(int(rng.choice([1, 4, 17])),)).astype(np.int32)
+        return f'x[idx] {shape} {idx.shape}', (lambda x, i: x[i]), [x, idx]
+    if kind == 'index2':
+        if rank < 2: return f'x[idx] {shape}', (lambda x, i: x[i]), [x, np.zeros((2,), np.int32)]
+        idx = rng.randint(0, shape[1], size=(int(rng.choice([1, 3, 9])),)).astype(np.int32)
+        return f'x[:, idx] {shape} {idx.shape}', (lambda x, i: x[:, i]), [x, idx]
+    if kind == 'scatter_dim':
+        idx = rng.randint(0, shape[0], size=(int(rng.choice([1, 5, 40])),)).astype(np.int32)
+        upd = ints(-3, 4, idx.shape[0], *shape[1:])
+        return f'x.at[idx].add {shape} {idx.shape}', (lambda x, i, u: x.at[i].add(u)), [x, idx, upd]
+    if kind == 'take_along':
+        axis = rng.randint(0, rank)
+        ishape = list(shape); ishape[axis] = int(rng.choice([1, 2, 6]))
+        idx = rng.randint(0, shape[axis], size=ishape).astype(np.int32)
+        return f'take_along_axis {shape} axis {axis}', (lambda x, i: jnp.take_along_axis(x, i, axis=axis)), [x, idx]
+    if kind == 'iota':
+        n = int(rng.choice([1, 7, 64, 1000]))
+        return f'iota {n}', (lambda x: lax.iota(np.int32, n) * 3 + x), [np.asarray(rng.randint(-5, 5), np.int32)]
+    if kind == 'clamp_pow':
+        p = int(rng.choice([0, 1, 2, 3, -1]))
+        base = x if p >= 0 else np.where(x == 0, 1, x).astype(np.float32)
+        return f'clamp+pow {shape} ^{p}', (lambda x: lax.integer_pow(lax.clamp(-3.0, x, 3.0), p) if p >= 0 else lax.clamp(-3.0, x, 3.0) * 2.0), [base]
+    # pool_general: windows over arbitrary dims of a rank-3/4 array
+    r = rng.randint(3, 5)
+    shp = tuple(int(rng.choice([1, 2, 4, 6, 9])) for _ in range(r))
+    win = tuple(int(rng.randint(1, min(3, s) + 1)) for s in shp)
+    strd = tuple(int(rng.randint(1, 3)) for _ in shp)
+    pads = tuple((int(rng.randint(0, 2)), int(rng.randint(0, 2))) for _ in shp)
+    xx = ints(-9, 10, *shp)
+    if rng.randint(0, 2):
+        return f'window max {shp} {win} {strd} {pads}', (lambda x: lax.reduce_window(x, -jnp.inf, lax.max, win, strd, pads)), [xx]
+    return f'window sum {shp} {win} {strd} {pads}', (lambda x: lax.reduce_window(x, 0.0, lax.add, win, strd, pads)), [xx]
+
+
+@pytest.mark.parametrize('seed', range(N_MISC))
+def test_random_misc_plans(seed):
+    name, f, args = make_misc_case(seed)
+    _, closed = oracle_outputs(f, args)
+    for fuse in (True, False):
+        JaxprInterpreter(closed, plan_only=True, fuse=fuse)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('seed', range(N_MISC))
+def test_random_misc_hip(seed):
+    name, f, args = make_misc_case(seed)
+    print(f'case: random primitive {seed}: {name}', flush=True)
+    for fuse in (True, False):
+        check_against_oracle(f, args, exact=True, fuse=fuse)
