@@ -121,36 +121,55 @@ def test_gather_scatter_small_exact_and_full():
     assert np.allclose(acc, expected, rtol=1e-5, atol=1e-6)
 
 
-def test_scatter_add_rows_sorted_and_atomic_paths():
-    '''Row scatter-add through both implementations (bucketed by a counting sort of the indices,
-    and HBM atomics): integer-valued updates make every sum exact; cases cover rows that receive no
-    update, one row that receives more than 64, indices outside the table (dropped), a row length
-    that is not a multiple of 4, integer data and an operand that is not zero.'''
+def test_scatter_add_rows_owner_sorted_and_atomic_paths():
+    '''Row scatter-add through all three implementations (one launch in which every workgroup owns a range of
+    table rows; buckets from a counting sort of the indices; HBM atomics): integer-valued updates make every
+    sum exact. Cases cover rows that receive no update, one row that receives more than 64, more updates for one
+    workgroup's rows than its LDS holds (several rounds), indices outside the table (dropped), row lengths that
+    are not a multiple of 4 or longer than one pass of a wave, integer data, operands that are not zero, and a
+    constant table filled with one value (not read at all).'''
     from vkjax_amd import ops
     rng = np.random.default_rng(7)
 
     def scatter(table, idx, updates):
         return mj.numpy.index_add(table, idx, updates)
 
-    saved = ops.SCATTER_SORT_THRESHOLD
+    def scatter_into_constant(fill):
+        def f(idx, updates):
+            return mj.numpy.index_add(mj.numpy.full((300, 64), fill, np.float32), idx, updates)
+        return f
+
+    saved = ops.SCATTER_SORT_THRESHOLD, ops.SCATTER_OWNER_MAX_IDX
     try:
-        for threshold in (0, 1 << 60):
-            ops.SCATTER_SORT_THRESHOLD = threshold
-            for rows, cols, n, dtype in ((50, 256, 400, np.float32), (9, 10, 37, np.float32), (300, 64, 200, np.int32), (4, 20, 500, np.float32)):
+        for path, threshold, owner_max in (('owner', 0, saved[1]), ('sum', 0, 0), ('atomic', 1 << 60, saved[1])):
+            ops.SCATTER_SORT_THRESHOLD, ops.SCATTER_OWNER_MAX_IDX = threshold, owner_max
+            cases = [(50, 256, 400, np.float32), (9, 10, 37, np.float32), (300, 64, 200, np.int32), (4, 20, 500, np.float32),
+                     (3000, 16, 9000, np.float32), (70, 520, 300, np.float32), (5, 8, 20000, np.int32), (1029, 4, 30000, np.float32),
+                     (300000, 4, 5000, np.float32)]                        #1024 rows per workgroup
+            for rows, cols, n, dtype in cases:
                 table   = rng.integers(-9, 9, size=(rows, cols)).astype(dtype)
                 idx     = rng.integers(0, rows, size=(n,)).astype(np.int32)
                 idx[: n // 3] = idx[0]                                 #one crowded row
                 updates = rng.integers(-5, 6, size=(n, cols)).astype(dtype)
                 _, _, fn = check_against_oracle(scatter, [table, idx, updates], exact=True)
                 kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
-                assert any(k.startswith('scatter_rows_sum') for k in kernels) == (threshold == 0), kernels
+                assert any(k.startswith('scatter_rows_sum') for k in kernels) == (path == 'sum'), kernels
+                assert any(k.startswith('scatter_rows_owner') for k in kernels) == (path == 'owner'), kernels
             #indices beyond the table (jnp's normalisation only wraps negative ones)
             table   = np.zeros((16, 8), np.float32)
             idx     = np.array([3, 99, 16, 15, -1, 3], np.int32)
             updates = rng.integers(-5, 6, size=(6, 8)).astype(np.float32)
             check_against_oracle(scatter, [table, idx, updates], exact=True)
+            #a constant table of one value
+            for fill in (0.0, -3.0):
+                idx     = rng.integers(0, 300, size=(700,)).astype(np.int32)
+                updates = rng.integers(-5, 6, size=(700, 64)).astype(np.float32)
+                _, _, fn = check_against_oracle(scatter_into_constant(fill), [idx, updates], exact=True)
+                if path == 'owner':
+                    launch = [l for l in list(fn._jaxpr_interpreters.values())[0].launches if l.kernel.startswith('scatter_rows_owner')][0]
+                    assert launch.buffers[1][0].size == 1, 'the constant table should have been replaced by its value'
     finally:
-        ops.SCATTER_SORT_THRESHOLD = saved
+        ops.SCATTER_SORT_THRESHOLD, ops.SCATTER_OWNER_MAX_IDX = saved
 
 
 def test_fusion_does_not_change_a_single_bit():
@@ -297,3 +316,25 @@ def test_stream_matches_call_by_call():
         assert_tree_close(next(it), expected[k], exact=True, what=f'suspended stream [{k}]')
         other = (k * 2 + 1) % len(batches)
         assert_tree_close(resident(*batches[other]), expected[other], exact=True, what=f'call {other} between stream results')
+
+
+def test_stream_loader_may_refill_its_batch_array():
+    '''A loader that hands out ONE preallocated batch array and refills it for every tuple: the stream
+    takes its tuples several evaluations ahead, so it has to have copied each batch when it took it.'''
+    rng = np.random.default_rng(11)
+    def scale_shift(x, w):
+        return x * w + 1.0
+    plain  = vkjax_amd.wrap(scale_shift, frontend='minijax')
+    stream = vkjax_amd.wrap(scale_shift, frontend='minijax')
+    for shape in ((33, 17), (1200, 2048)):                    #inline staging, and the chunked path (>= 8 MB)
+        w      = rng.standard_normal(shape[1:]).astype(np.float32)
+        values = [rng.standard_normal(shape).astype(np.float32) for _ in range(9)]
+        batch  = np.empty(shape, np.float32)
+        def loader():
+            for v in values:
+                batch[...] = v
+                yield batch, w
+        got = [np.array(y) for y in stream.stream(loader())]
+        assert len(got) == len(values)
+        for k, (g, v) in enumerate(zip(got, values)):
+            assert_tree_close(g, plain(v, w), exact=True, what=f'{shape} batch {k}')

@@ -354,3 +354,61 @@ def test_size_limits_are_reported_when_the_program_is_built():
         plan(lambda x, w: mj.numpy.dot(x, w), huge(1 << 20, 512), huge(512, 8))       #2 GiB lhs
     interp = plan(lambda x, w: mj.numpy.dot(x, w), huge((1 << 20) - 64, 511), huge(511, 8))
     assert interp.launches[0].kernel.startswith('conv_gemm')
+
+
+# ------------------------------------------------------------------ boundary details
+
+def test_reference_module_path_resolves():
+    '''The reference's own tests import the class as vkjax.kompute_jaxpr_interpreter.JaxprInterpreter
+    (reference: tests/common.py:7, vkjax/function.py:1).'''
+    import vkjax_amd as vkjax
+    assert vkjax.kompute_jaxpr_interpreter.JaxprInterpreter is JaxprInterpreter
+    from vkjax_amd.kompute_jaxpr_interpreter import JaxprInterpreter as by_import
+    assert by_import is JaxprInterpreter
+
+
+def test_no_temporary_shares_storage_with_a_program_output():
+    '''A result that is a view of an intermediate keeps that intermediate's storage to the end of the
+    program, also when launches were fused, moved or batched after the access positions were noted.'''
+    from vkjax_amd import workloads as W
+
+    def views_of_late_intermediates(x, idx, upd):
+        a = jnp.tanh(x) * 2.0
+        table = jnp.index_add(jnp.zeros((64, 8), np.float32), idx, upd)        #several launches for one equation
+        b = (a + 1.0).reshape(16, 4)                                     #output = view of an intermediate
+        c = jnp.sum(table, axis=0)
+        d = (jnp.exp(a) - c.sum()).reshape(4, 16)
+        return b, d, table.reshape(8, 64)
+
+    rng  = np.random.default_rng(0)
+    args = (rng.standard_normal((8, 8)).astype(np.float32), rng.integers(0, 64, (32,)).astype(np.int32),
+            rng.standard_normal((32, 8)).astype(np.float32))
+    programs = [(views_of_late_intermediates, args), (W.mlp_train_step, W.mlp_train_inputs(batch=8)),
+                (W.convnet_train_step, W.convnet_train_inputs(batch=2))]
+    for f, a in programs:
+        for fuse in (True, False):
+            closed = mj.make_jaxpr(f)(*a)
+            interp = JaxprInterpreter(closed, fuse=fuse, plan_only=True)
+            #storage of an output -> position of the first launch that touches it
+            outputs = {id(b.tensor): min(b.accesses) for b in interp.output_buffers if b is not None}
+            out_placeholders = {id(b._placeholder) for b in interp.output_buffers if b is not None}
+            for key, b in interp.bufferpool.buffers.items():
+                if b is None or b.tensor is None or id(b._placeholder) in out_placeholders or id(b.tensor) not in outputs:
+                    continue
+                #only something that is dead before the output is first written may have used its storage
+                assert max(b.accesses) < outputs[id(b.tensor)], f'{f.__name__} fuse={fuse}: {key} shares storage with a live output'
+            for b in interp.output_buffers:
+                assert b is None or max(b.accesses) == np.inf
+
+
+def test_index_modes_that_change_results_are_refused():
+    '''gather clamps and scatter-add drops (XLA); a mode that asks for anything else must not be ignored.'''
+    x, idx = np.zeros((8, 4), np.float32), np.zeros((3, 1), np.int32)
+    dn = lax.GatherDimensionNumbers(offset_dims=(1,), collapsed_slice_dims=(0,), start_index_map=(0,))
+    for mode, ok in (('clip', True), ('promise_in_bounds', True), (None, True), ('fill', False)):
+        closed = mj.make_jaxpr(lambda x, i: lax.gather(x, i, dn, (1, 4), mode=mode))(x, idx)
+        if ok:
+            JaxprInterpreter(closed, plan_only=True)
+        else:
+            with pytest.raises(NotImplementedError, match='mode'):
+                JaxprInterpreter(closed, plan_only=True)

@@ -2,3 +2,4 @@
 executes it through hand-written gfx950 kernels behind a C-ABI HIP runtime.'''
 from .function import Function, wrap
 from . import minijax
+from . import kompute_jaxpr_interpreter

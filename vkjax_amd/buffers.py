@@ -183,8 +183,20 @@ class BufferPool:
     def mark_buffer_as_constant(self, b: Buffer, var, value):
         if b.tensor is None:
             b.tensor = self._create_tensor(var, initial_value=value)
+        if value is not None:
+            b.constant_value = value          #known when the program is built: a lowering may look at it
         #the storage of a constant must never be handed to anything else
         b.accesses += [0, np.inf]
+
+    def scalar_constant(self, value, dtype) -> Buffer:
+        '''A one-element constant that belongs to no jaxpr variable; equal ones share storage.'''
+        dtype = np.dtype(dtype)
+        key   = ('scalar', str(dtype), np.asarray(value, dtype).tobytes())
+        if key not in self.buffers:
+            b = Buffer(self.device.tensor(to_device_words(np.asarray(value, dtype).reshape(1))), dtype, ())
+            b.accesses += [0, np.inf]
+            self.buffers[key] = b
+        return self.buffers[key]
 
     def set_buffer(self, var, b: tp.Optional[Buffer]):
         if b is None:

@@ -305,6 +305,188 @@ SCATTER_SUM_KERNEL(scatter_rows_sum_f_v4, 4, true)
 SCATTER_SUM_KERNEL(scatter_rows_sum_i_v1, 1, false)
 SCATTER_SUM_KERNEL(scatter_rows_sum_i_v4, 4, false)
 
+// ---------------------------------------------------------------------------------------------
+// scatter-add of whole rows in ONE launch, no scratch memory, no atomics on the data ("owner
+// computes"): a workgroup owns `rows_per_group` consecutive table rows. It reads the whole index
+// array once (from L2: the array is a few hundred KB to a few MB and every workgroup reads it),
+// keeps the updates that fall into its rows as keys (row within the group << 22 | update number)
+// in LDS, sorts the keys, and then each wave adds up the updates of one row after the other, in
+// ascending update order, on top of the operand row (or of a single value, when the operand is a
+// constant filled with one value) and writes the result row once. Every update row is read exactly
+// once, the table is written once, and the result does not depend on thread timing.
+// A workgroup whose rows receive more keys than LDS holds works through the index array in
+// several rounds, each taking as many consecutive indices as fit, adding onto what it has written.
+// Needs n_idx <= 2^22 and rows_per_group <= 1024 (the host sees to that).
+struct ScatterOwnerParams { uint32_t n_idx, row_len, n_rows, idx_stride, rows_per_group, operand_is_scalar; };
+
+#define SCATTER_OWNER_CAP     4096u     // keys a workgroup holds in LDS
+#define SCATTER_OWNER_THREADS 1024u
+#define SCATTER_OWNER_INFLIGHT 8        // update rows a wave requests before it adds them
+
+template <int VEC, bool IS_FLOAT>
+__device__ __forceinline__ void scatter_rows_owner_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ operand,
+                                                        const uint32_t* __restrict__ updates, const int32_t* __restrict__ idx,
+                                                        const ScatterOwnerParams& P) {
+    __shared__ uint32_t keys[SCATTER_OWNER_CAP];
+    __shared__ uint32_t start[1024 + 1];
+    __shared__ uint32_t n_keys, n_tile;
+    constexpr uint32_t NT = SCATTER_OWNER_THREADS, NW = NT / 64u, CAP = SCATTER_OWNER_CAP;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t R0 = blockIdx.x * P.rows_per_group;
+    const uint32_t nrows = min(P.rows_per_group, P.n_rows - R0);           // the grid covers n_rows exactly
+    auto add = [](uint32_t a, uint32_t b) -> uint32_t { return IS_FLOAT ? f2u(u2f(a) + u2f(b)) : a + b; };
+    auto take = [&](int32_t r, uint32_t i) {                               // keeps update i if its row is one of ours
+        const uint32_t local = (uint32_t)r - R0;                           // negative and foreign rows wrap to >= nrows
+        if (local < nrows) {
+            const uint32_t p = atomicAdd(&n_keys, 1u);
+            if (p < CAP) keys[p] = local << 22 | i;
+        }
+    };
+
+    // keys[0 .. count) -> sorted; start[j] = first key of row j; then the sums.
+    // first: the rows start from the operand and every row is written; otherwise from what `out` holds, rows with keys only
+    auto process = [&](uint32_t count, bool first) {
+        uint32_t n = 64u;
+        while (n < count) n <<= 1;
+        for (uint32_t p = count + tid; p < n; p += NT) keys[p] = 0xFFFFFFFFu;
+        __syncthreads();
+        for (uint32_t k = 2u; k <= n; k <<= 1) {
+            for (uint32_t j = k >> 1; j > 0u; j >>= 1) {
+                for (uint32_t t = tid; t < (n >> 1); t += NT) {
+                    const uint32_t lo = ((t & ~(j - 1u)) << 1) | (t & (j - 1u)), hi = lo | j;
+                    const uint32_t a = keys[lo], b = keys[hi];
+                    if ((a > b) == ((lo & k) == 0u)) { keys[lo] = b; keys[hi] = a; }
+                }
+                __syncthreads();
+            }
+        }
+        for (uint32_t j = tid; j <= nrows; j += NT) {                      // lower bound of row j's first possible key
+            const uint32_t want = j << 22;
+            uint32_t lo = j < nrows ? 0u : count, hi = count;              // j == nrows: 1024 << 22 does not fit a word
+            while (lo < hi) {
+                const uint32_t mid = (lo + hi) >> 1;
+                if (keys[mid] < want) lo = mid + 1u; else hi = mid;
+            }
+            start[j] = lo;
+        }
+        __syncthreads();
+        for (uint32_t j = wave; j < nrows; j += NW) {
+            const uint32_t s = start[j], e = start[j + 1u];
+            if (!first && s == e) continue;
+            const uint64_t row = (uint64_t)(R0 + j) * P.row_len;
+            for (uint32_t c0 = 0u; c0 < P.row_len; c0 += 64u * VEC) {
+                const uint32_t c = c0 + lane * VEC;
+                if (c >= P.row_len) continue;                              // row_len is a multiple of VEC
+                uint32_t acc[VEC];
+                const uint32_t* base = first ? operand : out;
+                if (first && P.operand_is_scalar) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = operand[0];
+                } else if constexpr (VEC == 4) {
+                    const u32x4 t = *reinterpret_cast<const u32x4*>(base + row + c);
+                    acc[0] = t.x; acc[1] = t.y; acc[2] = t.z; acc[3] = t.w;
+                } else {
+                    acc[0] = base[row + c];
+                }
+                for (uint32_t k = s; k < e; k += SCATTER_OWNER_INFLIGHT) {
+                    uint32_t t[SCATTER_OWNER_INFLIGHT][VEC];
+#pragma unroll
+                    for (uint32_t q = 0; q < SCATTER_OWNER_INFLIGHT; ++q)
+                        if (k + q < e) {
+                            const uint64_t u = (uint64_t)(keys[k + q] & 0x3FFFFFu) * P.row_len + c;
+                            if constexpr (VEC == 4) {
+                                const u32x4 w = *reinterpret_cast<const u32x4*>(updates + u);
+                                t[q][0] = w.x; t[q][1] = w.y; t[q][2] = w.z; t[q][3] = w.w;
+                            } else {
+                                t[q][0] = updates[u];
+                            }
+                        }
+#pragma unroll
+                    for (uint32_t q = 0; q < SCATTER_OWNER_INFLIGHT; ++q)
+                        if (k + q < e) {
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) acc[v] = add(acc[v], t[q][v]);
+                        }
+                }
+                if constexpr (VEC == 4) {
+                    u32x4 t; t.x = acc[0]; t.y = acc[1]; t.z = acc[2]; t.w = acc[3];
+                    *reinterpret_cast<u32x4*>(out + row + c) = t;
+                } else {
+                    out[row + c] = acc[0];
+                }
+            }
+        }
+    };
+
+    if (tid == 0u) n_keys = 0u;
+    __syncthreads();
+    // the whole index array, four 16-byte loads per thread in flight where the indices are dense
+    if (P.idx_stride == 1u && (reinterpret_cast<uintptr_t>(idx) & 15u) == 0u) {
+        const uint32_t nvec = P.n_idx >> 2;
+        const int4* idx4 = reinterpret_cast<const int4*>(idx);
+        for (uint32_t v0 = tid; v0 < nvec; v0 += NT * 4u) {
+            int4 t[4];
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q)
+                if (v0 + q * NT < nvec) t[q] = idx4[v0 + q * NT];
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q)
+                if (v0 + q * NT < nvec) {
+                    const uint32_t i = (v0 + q * NT) << 2;
+                    take(t[q].x, i); take(t[q].y, i + 1u); take(t[q].z, i + 2u); take(t[q].w, i + 3u);
+                }
+        }
+        for (uint32_t i = (nvec << 2) + tid; i < P.n_idx; i += NT) take(idx[i], i);
+    } else {
+        for (uint32_t i = tid; i < P.n_idx; i += NT) take(idx[(uint64_t)i * P.idx_stride], i);
+    }
+    __syncthreads();
+    const uint32_t total = n_keys;
+    if (total <= CAP) {
+        process(total, true);
+        return;
+    }
+    // More keys than LDS holds: rounds over consecutive ranges of the index array. A round takes
+    // tiles of NT indices while their keys still fit (a tile never holds more than NT <= CAP keys,
+    // so every round advances), sums them, and the next round continues behind it.
+    uint32_t pos = 0u;
+    bool first = true;
+    while (pos < P.n_idx) {
+        __syncthreads();
+        if (tid == 0u) n_keys = 0u;
+        __syncthreads();
+        uint32_t count = 0u;
+        while (pos < P.n_idx) {
+            if (tid == 0u) n_tile = 0u;
+            __syncthreads();
+            const uint32_t i = pos + tid;
+            uint32_t local = 0xFFFFFFFFu;
+            if (i < P.n_idx) local = (uint32_t)idx[(uint64_t)i * P.idx_stride] - R0;
+            if (local < nrows) atomicAdd(&n_tile, 1u);
+            __syncthreads();
+            if (count + n_tile > CAP) break;                               // uniform: every thread reads the same two values
+            if (local < nrows) keys[atomicAdd(&n_keys, 1u)] = local << 22 | i;
+            count += n_tile;
+            pos += NT;
+            __syncthreads();                                               // n_tile is reset by the next tile
+        }
+        __syncthreads();
+        process(count, first);
+        first = false;
+    }
+}
+
+#define SCATTER_OWNER_KERNEL(name, VEC, IS_FLOAT)                                                                  \
+    extern "C" __global__ __launch_bounds__(SCATTER_OWNER_THREADS) void name(uint32_t* out, const uint32_t* operand, \
+            const uint32_t* updates, const int32_t* idx, ScatterOwnerParams P) {                                   \
+        scatter_rows_owner_body<VEC, IS_FLOAT>(out, operand, updates, idx, P);                                     \
+    }
+// the _v4 variants require row_len % 4 == 0 and 16-byte aligned data pointers
+SCATTER_OWNER_KERNEL(scatter_rows_owner_f_v1, 1, true)
+SCATTER_OWNER_KERNEL(scatter_rows_owner_f_v4, 4, true)
+SCATTER_OWNER_KERNEL(scatter_rows_owner_i_v1, 1, false)
+SCATTER_OWNER_KERNEL(scatter_rows_owner_i_v4, 4, false)
+
 struct ScatterGeneralParams {
     uint32_t n_upd, upd_rank, op_rank, n_index, is_float;
     uint32_t upd_dims[IDX_MAX_RANK];

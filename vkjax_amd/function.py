@@ -105,6 +105,8 @@ class Function:
         from the iterable and flattens and converts their arguments while the calling thread waits
         for the device; the runtime stages and uploads them during the preceding evaluation.
         A tuple whose signature differs from its predecessor's is uploaded in its own turn.
+        Arrays may be refilled by the caller as soon as the iterable is asked for the next tuple (their
+        contents are copied when a tuple is taken), except those of `resident_argnums`.
         No counterpart in the reference, whose calls copy, run and read back in turn
         (vkjax/kompute_jaxpr_interpreter.py:72-81).'''
         if self._profiling:
@@ -116,6 +118,30 @@ class Function:
         caught_up = threading.Event()
         caught_up.set()
 
+        # A tuple is taken from the iterable up to four evaluations before its arguments are staged, and a
+        # loader may refill the arrays it has handed out (one batch array, or a small ring of them) as soon as
+        # it is asked for the next tuple. Argument leaves that would be passed on as views of the caller's
+        # arrays are therefore copied when the tuple is taken, into one of RING arrays kept per leaf: at most
+        # that many tuples are between the iterable and the end of their upload at any time (one being
+        # prepared, one queued, the following one, the current one). Resident leaves are identified by the
+        # object passed and are not copied: their contract is that the array stays as it is.
+        RING = 4
+        rings: tp.Dict[tp.Tuple[int, int], tp.List] = {}
+
+        def owned(interpreter, converted):
+            result = []
+            for k, slot, x, words, is_resident in converted:
+                if not is_resident and isinstance(x, np.ndarray) and np.may_share_memory(words, x):
+                    ring = rings.setdefault((id(interpreter), k), [0, [None] * RING])
+                    position = ring[0] % RING
+                    ring[0] += 1
+                    if ring[1][position] is None:
+                        ring[1][position] = np.empty_like(words)
+                    np.copyto(ring[1][position], words)
+                    words = ring[1][position]
+                result.append((k, slot, x, words, is_resident))
+            return result
+
         def prepare(args):
             caught_up.wait()
             args      = tuple(args)                  #what __call__ sees as *args
@@ -123,13 +149,18 @@ class Function:
             entry     = self._jaxpr_interpreters.get(signature)
             if entry is None:
                 caught_up.clear()
+                #traced and recorded by the calling thread, later: the arrays are copied now, as above
+                resident = self._interpreter_args[1].get('resident_argnums', ())
+                copy = lambda leaf: np.array(leaf) if isinstance(leaf, np.ndarray) else leaf
+                args = tuple(a if i in resident or i in self._static_argnums else self._tree.tree_map(copy, a)
+                             for i, a in enumerate(args))
                 return [None, None, args]
-            return [entry, self._output_shapes[signature], entry._convert_inputs(args)]
+            return [entry, self._output_shapes[signature], owned(entry, entry._convert_inputs(args))]
 
         def resolved(item):
             if item is not None and item[0] is None:
                 interpreter, output_shapes = self._get_or_create_jaxpr_interpreter(item[2])
-                item[:] = [interpreter, output_shapes, interpreter._convert_inputs(item[2])]
+                item[:] = [interpreter, output_shapes, owned(interpreter, interpreter._convert_inputs(item[2]))]
                 caught_up.set()
             return item
 

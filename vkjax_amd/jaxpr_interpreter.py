@@ -65,6 +65,12 @@ class JaxprInterpreter:
         if self.fuse:
             self.all_ops    = fusion.fuse_ops(self.all_ops, self.bufferpool, jaxpr.jaxpr.outvars)
         self.output_buffers = [self.bufferpool.get_buffer(v) for v in jaxpr.jaxpr.outvars]
+        #A result that is a view of an intermediate (a reshape of the last launch's output) shares that
+        #intermediate's storage, which must stay untouched until the download: pinned to the end of the
+        #program, whatever positions the passes above have given the launches.
+        for b in self.output_buffers:
+            if b is not None:
+                b.accesses.append(np.inf)
         self.bufferpool.create_tensors()
         #lower every op now so that unsupported layouts fail at build time, not at run time
         self.launches = [op.launch for op in self.all_ops]

@@ -832,6 +832,30 @@ def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: 
     ]
 
 
+SCATTER_OWNER_CAP     = 4096          #keys a workgroup of scatter_rows_owner holds in LDS
+SCATTER_OWNER_MAX_IDX = 1 << 22       #update numbers take 22 bits of a key
+SCATTER_OWNER_GROUPS  = 256           #workgroups aimed at: one per compute unit
+
+
+def scatter_add_rows_owner(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_len: int, n_rows: int,
+                           operand_is_scalar: bool = False, idx_stride: int = 1) -> Launch:
+    '''out = operand; out[idx[i], :] += updates[i, :] in one launch: every workgroup owns a range of table rows, picks
+    its updates out of the whole index array and sums them in ascending update order. `operand` is the table, or one
+    word when the table is a constant filled with a single value.'''
+    assert n_idx <= SCATTER_OWNER_MAX_IDX
+    #one workgroup per compute unit where possible (each reads the whole index array), but no more rows per
+    #workgroup than are expected to fill half its key storage, and at most 1024 (10 bits of a key)
+    rows = max(_cdiv(n_rows, SCATTER_OWNER_GROUPS), 1)
+    rows = min(rows, max(n_rows * (SCATTER_OWNER_CAP // 2) // max(n_idx, 1), 1), 1024)
+    vec  = 4 if row_len % 4 == 0 else 1
+    kind = 'f' if out.dtype == np.float32 else 'i'
+    table_passes = 1 if operand_is_scalar else 2
+    return Launch(f'scatter_rows_owner_{kind}_v{vec}', (_cdiv(n_rows, rows), 1, 1), (1024, 1, 1),
+                  [(out, 0), (operand, 0), (updates, 0), (idx, 0)],
+                  _u32(n_idx, row_len, n_rows, idx_stride, rows, int(operand_is_scalar)),
+                  bytes_moved=4 * (n_idx * row_len + n_idx + table_passes * n_rows * row_len))
+
+
 def scatter_add_general(out: Buffer, indices: Buffer, updates: Buffer, update_window_dims, inserted_window_dims,
                         scatter_dims_to_operand_dims) -> Launch:
     upd_rank, op_rank = len(updates.shape), len(out.shape)

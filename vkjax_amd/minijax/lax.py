@@ -491,7 +491,8 @@ def gather(operand, start_indices, dimension_numbers: GatherDimensionNumbers, sl
             raise TypeError(f'slice_sizes {ss} exceed operand shape {ops}')
     return emit('gather', [operand, start_indices], [_aval(out, dtype_of(operand)[0])],
                 dict(dimension_numbers=dn, slice_sizes=ss, indices_are_sorted=indices_are_sorted,
-                     unique_indices=unique_indices))
+                     unique_indices=unique_indices,
+                     **({} if mode is None else dict(mode=mode, fill_value=fill_value))))
 
 
 def scatter_add(operand, scatter_indices, updates, dimension_numbers: ScatterDimensionNumbers,

@@ -128,6 +128,10 @@ def zeros(shape, dtype=np.float32):
     return np.zeros(shape, core.canonicalize_dtype(dtype))
 
 
+def full(shape, fill_value, dtype=np.float32):
+    return np.full(shape, fill_value, core.canonicalize_dtype(dtype))
+
+
 def ones(shape, dtype=np.float32):
     return np.ones(shape, core.canonicalize_dtype(dtype))
 

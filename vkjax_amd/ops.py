@@ -800,8 +800,21 @@ def pad(bufferpool, equation):
     return [Op(equation, launch=K.pad(outbuf, inbuf, value, equation.params['padding_config']))]
 
 
+def _index_mode(params) -> str:
+    '''Name of the equation's GatherScatterMode ('CLIP', 'FILL_OR_DROP', 'PROMISE_IN_BOUNDS'), or '' when the
+    front-end (old jax versions, the reference's era) has no such parameter.'''
+    mode = params.get('mode')
+    if mode is None:
+        return ''
+    return str(getattr(mode, 'name', mode)).upper().rsplit('.', 1)[-1]
+
+
 def gather(bufferpool, equation):
     params = equation.params
+    #start indices are clamped so that the slice stays inside the operand: that is XLA's gather, CLIP, and what
+    #XLA makes of PROMISE_IN_BOUNDS; FILL_OR_DROP would have to return fill_value for such slices instead
+    if _index_mode(params) not in ('', 'CLIP', 'PROMISE_IN_BOUNDS'):
+        raise NotImplementedError(f'gather with mode={params["mode"]}: {equation}')
     dn     = params['dimension_numbers']
     offset_dims, collapsed, start_index_map = (tuple(dn.offset_dims), tuple(dn.collapsed_slice_dims), tuple(dn.start_index_map))
     slice_sizes = tuple(int(s) for s in params['slice_sizes'])
@@ -827,6 +840,10 @@ def gather(bufferpool, equation):
 def scatter_add(bufferpool, equation):
     '''General XLA scatter-add (the reference implements two fixed patterns, vkjax/ops.py:404-433).
     The operand is copied to the output first, then updates are added with HBM atomics.'''
+    #updates whose window does not fit into the operand are dropped: XLA's scatter, FILL_OR_DROP, and what holds
+    #trivially under PROMISE_IN_BOUNDS; CLIP would have to move such windows inside instead
+    if _index_mode(equation.params) not in ('', 'FILL_OR_DROP', 'PROMISE_IN_BOUNDS'):
+        raise NotImplementedError(f'scatter-add with mode={equation.params["mode"]}: {equation}')
     dn = equation.params['dimension_numbers']
     uwd, iwd, sd2od = tuple(dn.update_window_dims), tuple(dn.inserted_window_dims), tuple(dn.scatter_dims_to_operand_dims)
     operand, indices, updates = [bufferpool.get_buffer(v) for v in equation.invars]
@@ -850,6 +867,19 @@ def scatter_add(bufferpool, equation):
         row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
         n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
         n_rows  = operand.shape[0]
+        if n_idx * row_len >= SCATTER_SORT_THRESHOLD and n_idx <= SCATTER_OWNER_MAX_IDX and n_rows < 2**31 - 1:
+            #large: every workgroup owns a range of table rows and sums the updates that fall into it, one launch
+            #(no atomics on the data, no copy of the operand, no scratch arrays)
+            bufferpool.op_counter = counter_before + 1
+            uniform = _uniform_constant(operand)
+            if uniform is not None:
+                #a table that is a constant filled with one value (zeros, usually) is not read at all
+                source = bufferpool.scalar_constant(uniform, operand.dtype)
+                source.accesses.append(counter_before)
+            else:
+                source = operand
+            return [Op(equation, launch=K.scatter_add_rows_owner(outbuf, source, indices, updates, n_idx, row_len, n_rows,
+                                                                 operand_is_scalar=uniform is not None))]
         if n_idx * row_len >= SCATTER_SORT_THRESHOLD and n_idx < 2**30 and n_rows < 2**31 - 1:
             #large: bucket the updates by row and sum each bucket (no atomics on the data, no copy of the operand)
             bufferpool.op_counter = counter_before
@@ -863,8 +893,23 @@ def scatter_add(bufferpool, equation):
     return [copy, Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od))]
 
 
-#scatter-add of rows: from this many update elements on, the sorted (atomic-free) kernels are used
+#scatter-add of rows: from this many update elements on, the atomic-free kernels are used: the single-launch
+#one for up to SCATTER_OWNER_MAX_IDX updates, beyond that the counting sort with its scratch arrays
 SCATTER_SORT_THRESHOLD = 1 << 18
+SCATTER_OWNER_MAX_IDX  = K.SCATTER_OWNER_MAX_IDX
+
+
+def _uniform_constant(b):
+    '''The value of a build-time constant whose elements are all the same, else None.'''
+    value = getattr(b, 'constant_value', None)
+    if value is None:
+        return None
+    value = np.asarray(value)
+    if value.size == 0 or value.size != b.size:
+        return None
+    first = value.reshape(-1)[0]
+    #bit-wise comparison: -0.0 is not 0.0 here, and a NaN-filled table is uniform
+    return first if (value.reshape(-1).view(np.uint8).reshape(value.size, -1) == np.asarray(first).reshape(1).view(np.uint8)).all() else None
 
 
 # ------------------------------------------------------------------ rng
