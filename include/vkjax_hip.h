@@ -71,11 +71,15 @@ int vkj_sync(vkj_handle ctx);
 /* Code objects built ahead of time for gfx950 replace the per-op SPIR-V produced by
  * pyshaderc.compile_into_spirv          reference: vkjax/shaders.py:16-29 */
 int vkj_module_load(vkj_handle ctx, const void* image, size_t nbytes, vkj_handle* module);
+/* Unloading retires the module's function handles with it. A module that recorded launches of
+ * live sequences refer to is not unloaded: VKJ_ESTATE until those sequences are destroyed. */
 int vkj_module_unload(vkj_handle ctx, vkj_handle module);
 int vkj_module_get_function(vkj_handle ctx, vkj_handle module, const char* name, vkj_handle* function);
 
 /* mgr.tensor(array) + OpTensorSyncDevice  reference: vkjax/buffers.py:189-204 */
 int vkj_buf_alloc(vkj_handle ctx, size_t nbytes, vkj_handle* buf);
+/* The handle is retired at once. The memory of a buffer that live sequences have recorded (they hold
+ * its address) is released when the last of those sequences is destroyed. */
 int vkj_buf_free(vkj_handle ctx, vkj_handle buf);
 int vkj_buf_size(vkj_handle ctx, vkj_handle buf, size_t* nbytes);
 int vkj_buf_device_ptr(vkj_handle ctx, vkj_handle buf, uint64_t* device_address);
@@ -105,6 +109,11 @@ int vkj_seq_record_launch(vkj_handle seq, vkj_handle function,
                           const uint64_t* buf_byte_offsets, int nbufs);
 /* seq.record(kp.OpTensorSyncLocal([...]))   reference: vkjax/kompute_jaxpr_interpreter.py:62-63 */
 int vkj_seq_record_download(vkj_handle seq, vkj_handle buf, size_t offset, int slot, size_t nbytes);
+/* There is no vkj_seq_record_memset: an array that has to start at zero inside a sequence (the table
+ * a scatter-add accumulates into) is cleared by a recorded launch of the fill kernel. hipMemsetAsync
+ * nodes inside a captured graph have given wrong results on replays after the first, and
+ * vkj_seq_use_graph captures the launches of a sequence. vkj_buf_memset clears a buffer outside
+ * sequences. */
 int vkj_seq_num_steps(vkj_handle seq, int* uploads, int* launches, int* downloads);
 /* sequence.eval()                     reference: vkjax/kompute_jaxpr_interpreter.py:77
  * All uploads, then all launches, then all downloads, then one stream synchronisation.

@@ -1,0 +1,196 @@
+'''The C-ABI runtime's handle, lifetime and transfer logic on the CPU: vkjax_amd/csrc/shim.cpp is
+compiled against a host-only stand-in of the HIP calls it makes (tests/fake_hip), so contexts,
+modules, buffers and sequences can be created without a GPU. What is checked: objects that live
+sequences refer to cannot be pulled from under them, stale handles are rejected, error paths
+release what they had created, and an evaluation moves the bytes it should.'''
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from vkjax_amd import hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EINVAL, ESTATE = -1, -3
+
+
+@pytest.fixture(scope='module')
+def lib(tmp_path_factory):
+    out  = str(tmp_path_factory.mktemp('fake_shim') / 'libvkjax_fake.so')
+    csrc = os.path.join(ROOT, 'vkjax_amd', 'csrc')
+    fake = os.path.join(ROOT, 'tests', 'fake_hip')
+    subprocess.run(['g++', '-O1', '-g', '-fPIC', '-shared', '-pthread', '-std=c++17', f'-I{fake}', f'-I{csrc}',
+                    f'-I{os.path.join(ROOT, "include")}', os.path.join(csrc, 'shim.cpp'), os.path.join(fake, 'fake_glue.cpp'), '-o', out],
+                   check=True, capture_output=True, text=True)
+    lib = C.CDLL(out)
+    for name, (restype, argtypes) in hip._PROTOTYPES.items():
+        if name == 'vkj_seq_eval_next_static':
+            continue                                   #lives in static_landing.hip (device code), not in this build
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = restype, argtypes
+    lib.fake_hip_live_objects.restype = C.c_long
+    lib.fake_hip_launches.restype = C.c_long
+    lib.fake_hip_fail_after.argtypes = [C.c_long]
+    return lib
+
+
+def H():
+    return C.c_uint64(0)
+
+
+class World:
+    '''A context with one module (two kernels) in the stand-in runtime.'''
+    def __init__(self, lib):
+        self.lib = lib
+        self.ctx, self.mod, self.fn = H(), H(), H()
+        assert lib.vkj_ctx_create(0, C.byref(self.ctx)) == 0
+        image = C.create_string_buffer(b'fake_add_one\nfake_nothing\n')
+        assert lib.vkj_module_load(self.ctx, image, len(image), C.byref(self.mod)) == 0
+        assert lib.vkj_module_get_function(self.ctx, self.mod, b'fake_add_one', C.byref(self.fn)) == 0
+
+    def buf(self, nbytes):
+        b = H()
+        assert self.lib.vkj_buf_alloc(self.ctx, nbytes, C.byref(b)) == 0
+        return b
+
+    def add_one_sequence(self, n):
+        '''upload slot 0 -> src; dst = src + 1; dst -> download slot 1'''
+        lib = self.lib
+        src, dst, seq = self.buf(4 * n), self.buf(4 * n), H()
+        assert lib.vkj_seq_create(self.ctx, 0, C.byref(seq)) == 0
+        assert lib.vkj_seq_record_upload(seq, src, 0, 0, 4 * n) == 0
+        assert self.record_add_one(seq, dst, src, n) == 0
+        assert lib.vkj_seq_record_download(seq, dst, 0, 1, 4 * n) == 0
+        return seq, src, dst
+
+    def record_add_one(self, seq, dst, src, n, fn=None):
+        kernarg = bytes(16) + np.uint32(n).tobytes() + bytes(4)
+        grid = (C.c_uint32 * 3)(1, 1, 1)
+        bufs = (C.c_uint64 * 2)(dst.value, src.value)
+        offs = (C.c_uint32 * 2)(0, 8)
+        return self.lib.vkj_seq_record_launch(seq, fn or self.fn, grid, grid, 0, kernarg, len(kernarg), bufs, offs, None, 2)
+
+    def eval(self, seq, x, nxt=None, flags=0, n=None):
+        y = np.zeros(n or (x.size if x is not None else nxt.size), np.uint32)
+        ptrs = (C.c_void_p * 2)(x.ctypes.data if x is not None else None, y.ctypes.data)
+        if nxt is None:
+            assert self.lib.vkj_seq_eval(seq, ptrs, 2, flags) == 0, self.lib.vkj_last_error()
+        else:
+            nptrs = (C.c_void_p * 2)(nxt.ctypes.data, None)
+            assert self.lib.vkj_seq_eval_next(seq, ptrs, 2, flags, nptrs) == 0, self.lib.vkj_last_error()
+        return y
+
+    def close(self):
+        assert self.lib.vkj_module_unload(self.ctx, self.mod) == 0
+        assert self.lib.vkj_ctx_destroy(self.ctx) == 0
+
+
+def test_eval_moves_the_bytes_and_everything_is_released(lib):
+    before = lib.fake_hip_live_objects()
+    w = World(lib)
+    seq, src, dst = w.add_one_sequence(1000)
+    x = np.arange(1000, dtype=np.uint32)
+    assert np.array_equal(w.eval(seq, x), x + 1)
+    #the following evaluation's arguments ride along; the next call passes NULL for the slot
+    x2 = x * 3
+    assert np.array_equal(w.eval(seq, x, nxt=x2), x + 1)
+    assert np.array_equal(w.eval(seq, None, nxt=x, flags=hip.EVAL_NULL_IS_RESIDENT), x2 + 1)
+    assert np.array_equal(w.eval(seq, None, flags=hip.EVAL_NULL_IS_RESIDENT, n=1000), x + 1)
+    assert lib.vkj_seq_destroy(seq) == 0
+    assert lib.vkj_buf_free(w.ctx, src) == 0 and lib.vkj_buf_free(w.ctx, dst) == 0
+    w.close()
+    assert lib.fake_hip_live_objects() == before
+
+
+def test_module_unload_is_refused_while_a_sequence_uses_it(lib):
+    w = World(lib)
+    seq, src, dst = w.add_one_sequence(8)
+    assert lib.vkj_module_unload(w.ctx, w.mod) == ESTATE
+    assert b'live sequences' in lib.vkj_last_error()
+    x = np.arange(8, dtype=np.uint32)
+    assert np.array_equal(w.eval(seq, x), x + 1)                 #still whole
+    assert lib.vkj_seq_destroy(seq) == 0
+    assert lib.vkj_module_unload(w.ctx, w.mod) == 0
+    #the module's functions went with it: recording one is a bad handle, not a use after free
+    seq2 = H()
+    assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq2)) == 0
+    assert w.record_add_one(seq2, dst, src, 8) == EINVAL
+    f = H()
+    assert lib.vkj_module_get_function(w.ctx, w.mod, b'fake_add_one', C.byref(f)) == EINVAL
+    assert lib.vkj_seq_destroy(seq2) == 0
+    for b in (src, dst):
+        assert lib.vkj_buf_free(w.ctx, b) == 0
+    assert lib.vkj_ctx_destroy(w.ctx) == 0
+
+
+def test_buffer_freed_under_a_live_sequence_outlives_it(lib):
+    before = lib.fake_hip_live_objects()
+    w = World(lib)
+    seq, src, dst = w.add_one_sequence(64)
+    base = lib.fake_hip_live_objects()
+    assert lib.vkj_buf_free(w.ctx, src) == 0                     #handle retired, memory kept
+    assert lib.fake_hip_live_objects() == base
+    n = C.c_size_t(0)
+    assert lib.vkj_buf_size(w.ctx, src, C.byref(n)) == EINVAL    #stale handle
+    assert lib.vkj_buf_free(w.ctx, src) == EINVAL
+    x = np.arange(64, dtype=np.uint32)
+    assert np.array_equal(w.eval(seq, x), x + 1)                 #the sequence still owns valid memory
+    assert lib.vkj_seq_destroy(seq) == 0                         #... and releases it
+    assert lib.fake_hip_live_objects() == base - 1 - 2           #src, and the two pinned staging buffers
+    assert lib.vkj_buf_free(w.ctx, dst) == 0
+    w.close()
+    assert lib.fake_hip_live_objects() == before
+
+
+def test_context_creation_releases_everything_when_a_step_fails(lib):
+    before = lib.fake_hip_live_objects()
+    for successes in range(6):                                   #two streams and four events are created
+        lib.fake_hip_fail_after(successes)
+        ctx = H()
+        assert lib.vkj_ctx_create(0, C.byref(ctx)) != 0
+        assert b'injected' in lib.vkj_last_error()
+        assert lib.fake_hip_live_objects() == before
+    lib.fake_hip_fail_after(6)                                   #nothing left to fail in creation
+    ctx = H()
+    assert lib.vkj_ctx_create(0, C.byref(ctx)) == 0
+    lib.fake_hip_fail_after(-1)
+    assert lib.vkj_ctx_destroy(ctx) == 0
+    assert lib.fake_hip_live_objects() == before
+
+
+def test_landing_allocation_failure_leaves_nothing_behind(lib):
+    w = World(lib)
+    seq, src, dst = w.add_one_sequence(16)
+    x = np.arange(16, dtype=np.uint32)
+    y = np.zeros(16, np.uint32)
+    ptrs, nptrs = (C.c_void_p * 2)(x.ctypes.data, y.ctypes.data), (C.c_void_p * 2)(x.ctypes.data, None)
+    base = lib.fake_hip_live_objects()
+    lib.fake_hip_fail_after(1)                                   #landing buffer succeeds, its pinned staging does not
+    assert lib.vkj_seq_eval_next(seq, ptrs, 2, 0, nptrs) != 0
+    assert lib.fake_hip_live_objects() == base
+    assert np.array_equal(w.eval(seq, x, nxt=x), x + 1)          #and the sequence still works
+    assert lib.fake_hip_live_objects() == base + 2
+    assert lib.vkj_seq_destroy(seq) == 0
+    for b in (src, dst):
+        assert lib.vkj_buf_free(w.ctx, b) == 0
+    w.close()
+
+
+def test_objects_of_another_context_and_bad_ranges_are_rejected(lib):
+    w, w2 = World(lib), World(lib)
+    seq, src, dst = w.add_one_sequence(4)
+    other = w2.buf(16)
+    assert lib.vkj_seq_record_upload(seq, other, 0, 2, 16) == EINVAL
+    assert w.record_add_one(seq, other, src, 4) == EINVAL
+    assert w.record_add_one(seq, dst, src, 4, fn=w2.fn) == EINVAL
+    assert lib.vkj_seq_record_upload(seq, src, 8, 2, 16) == EINVAL       #range beyond the buffer
+    assert lib.vkj_buf_free(w2.ctx, src) == EINVAL
+    ptrs = (C.c_void_p * 2)(None, None)
+    assert lib.vkj_seq_eval(seq, ptrs, 2, 0) == EINVAL                    #no host pointer for the upload
+    assert lib.vkj_seq_destroy(seq) == 0
+    for b in (src, dst):
+        assert lib.vkj_buf_free(w.ctx, b) == 0
+    assert lib.vkj_buf_free(w2.ctx, other) == 0
+    w.close(); w2.close()

@@ -2,9 +2,7 @@
 // gfx950 code objects and recorded sequences, exported through the C ABI declared in
 // include/vkjax_hip.h. Host-only translation unit; kernels live in separate code objects
 // that the caller loads with vkj_module_load.
-#include "vkjax_hip.h"
-
-#include <hip/hip_runtime.h>
+#include "shim_internal.h"
 
 #include <atomic>
 #include <cstdarg>
@@ -18,9 +16,14 @@
 #include <vector>
 #include <algorithm>
 
-namespace {
+namespace vkj {
 
 thread_local std::string g_last_error;
+
+Registry& registry() {
+    static Registry r;
+    return r;
+}
 
 int fail(int code, const char* fmt, ...) {
     char buf[512];
@@ -36,6 +39,12 @@ int hip_fail(hipError_t e, const char* what) {
     g_last_error = std::string(what) + ": " + hipGetErrorString(e);
     return (int)e > 0 ? (int)e : VKJ_EINVAL;
 }
+
+}  // namespace vkj
+
+namespace {
+
+using namespace vkj;
 
 // Large uploads: the copy into the pinned staging buffer is done by a few threads, chunk by chunk,
 // while the calling thread hands every finished chunk to the DMA engine in order, so that staging
@@ -108,111 +117,29 @@ int staged_copy_out(char* dst, const char* staging, size_t nbytes, Wait&& wait_f
     return status;
 }
 
-
-#define HIP_TRY(expr)                                   \
-    do {                                                \
-        hipError_t _e = (expr);                         \
-        if (_e != hipSuccess) return hip_fail(_e, #expr); \
-    } while (0)
-
-constexpr uint32_t MAGIC_CTX = 0x766b4a43, MAGIC_BUF = 0x766b4a42, MAGIC_MOD = 0x766b4a4d,
-                   MAGIC_FN = 0x766b4a46, MAGIC_SEQ = 0x766b4a53;
-
-struct Ctx {
-    uint64_t    handle = 0;
-    uint32_t    magic = MAGIC_CTX;
-    int         device = 0;
-    hipStream_t stream = nullptr;
-    hipEvent_t  ev_begin = nullptr, ev_end = nullptr;
-    hipStream_t copy_stream = nullptr;   // created on first use: uploads that overlap the launches of `stream`
-    hipEvent_t  ev_landed = nullptr;
-};
-
-struct Buf {
-    uint64_t    handle = 0;
-    uint32_t magic = MAGIC_BUF;
-    Ctx*     ctx = nullptr;
-    void*    dptr = nullptr;
-    size_t   nbytes = 0;
-};
-
-struct Mod {
-    uint64_t    handle = 0;
-    uint32_t    magic = MAGIC_MOD;
-    Ctx*        ctx = nullptr;
-    hipModule_t module = nullptr;
-};
-
-struct Fn {
-    uint64_t    handle = 0;
-    uint32_t      magic = MAGIC_FN;
-    Mod*          mod = nullptr;
-    hipFunction_t fn = nullptr;
-    std::string   name;
-};
-
-struct Transfer {
-    Buf*   buf;
-    size_t offset, nbytes;
-    int    slot;
-    void*  staging;    // pinned host memory owned by the sequence
-    void*  next_staging = nullptr;   // pinned host memory and device memory for the arguments of the
-    void*  landing = nullptr;        // following evaluation, allocated when one is first handed in
-};
-
-struct Launch {
-    Fn*                  fn;
-    uint32_t             grid[3], block[3], lds;
-    std::vector<uint8_t> kernarg;
-};
-
-struct Seq {
-    uint64_t    handle = 0;
-    uint32_t              magic = MAGIC_SEQ;
-    Ctx*                  ctx = nullptr;
-    bool                  profiling = false;
-    std::vector<Transfer> uploads, downloads;
-    std::vector<Launch>   launches;
-    std::vector<hipEvent_t> chunk_events;   // one behind every chunk of a large download
-    std::vector<hipEvent_t> stamps;   // profiling: 1 + number of steps
-    int                   stamps_valid = 0;
-    bool                  want_graph = false;     // issue the launches as one captured graph
-    bool                  graph_failed = false;   // capture did not work once: keep to plain launches
-    hipGraphExec_t        graph_exec = nullptr;
-};
-
-// Handles are keys into a process-wide table, never raw addresses, so that a stale or made-up
-// handle is rejected instead of being dereferenced.
-struct Registry {
-    std::mutex mu;
-    std::unordered_map<uint64_t, std::pair<uint32_t, void*>> live;
-    uint64_t next = 0x1000;
-} g_registry;
-
-template <class T>
-T* from_handle(vkj_handle h, uint32_t magic) {
-    std::lock_guard<std::mutex> lock(g_registry.mu);
-    auto it = g_registry.live.find(h);
-    if (it == g_registry.live.end() || it->second.first != magic) return nullptr;
-    return static_cast<T*>(it->second.second);
-}
-template <class T>
-vkj_handle to_handle(T* p) {
-    std::lock_guard<std::mutex> lock(g_registry.mu);
-    const uint64_t h = g_registry.next++;
-    g_registry.live[h] = {p->magic, p};
-    p->handle = h;
-    return h;
-}
-template <class T>
-void retire(T* p) {
-    std::lock_guard<std::mutex> lock(g_registry.mu);
-    g_registry.live.erase(p->handle);
-}
-
 int use(Ctx* c) {
     HIP_TRY(hipSetDevice(c->device));
     return 0;
+}
+
+void destroy_ctx_objects(Ctx* c) {
+    if (c->ev_begin)    hipEventDestroy(c->ev_begin);
+    if (c->ev_end)      hipEventDestroy(c->ev_end);
+    if (c->ev_landed)   hipEventDestroy(c->ev_landed);
+    if (c->ev_uploaded) hipEventDestroy(c->ev_uploaded);
+    if (c->stream)      hipStreamDestroy(c->stream);
+    if (c->copy_stream) hipStreamDestroy(c->copy_stream);
+    c->ev_begin = c->ev_end = c->ev_landed = c->ev_uploaded = nullptr;
+    c->stream = c->copy_stream = nullptr;
+}
+
+// A sequence lets go of a buffer it recorded; the memory of a buffer that vkj_buf_free has
+// already been called on is released with the last such reference.
+void unref_buf(Buf* b) {
+    if (--b->seq_refs == 0 && b->released) {
+        hipFree(b->dptr);
+        delete b;
+    }
 }
 
 int issue_launch(Ctx* c, Launch& l) {
@@ -265,6 +192,154 @@ int issue_all(Ctx* c, Seq* s) {
 
 }  // namespace
 
+int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, void* const* next_host_ptrs,
+                  const LandingRegion* region) {
+    Ctx* c = s->ctx;
+    if (int r = use(c)) return r;
+    const bool up = !(flags & VKJ_EVAL_SKIP_UPLOADS), down = !(flags & VKJ_EVAL_SKIP_DOWNLOADS);
+    auto slot_ok = [&](const Transfer& t) { return t.nbytes == 0 || (host_ptrs && t.slot < nslots && host_ptrs[t.slot]); };
+    const bool null_resident = flags & VKJ_EVAL_NULL_IS_RESIDENT;
+    if (up)   for (auto& t : s->uploads)   if (!slot_ok(t) && !(null_resident && host_ptrs && t.slot < nslots))
+        return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for upload slot %d", t.slot);
+    if (down) for (auto& t : s->downloads) if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for download slot %d", t.slot);
+
+    size_t nstamps = 0;
+    if (s->profiling) {
+        nstamps = 3 + s->launches.size();       // begin, after uploads, after each launch, after downloads
+        while (s->stamps.size() < nstamps) {
+            hipEvent_t e;
+            HIP_TRY(hipEventCreate(&e));
+            s->stamps.push_back(e);
+        }
+        s->stamps_valid = 0;
+        HIP_TRY(hipEventRecord(s->stamps[0], c->stream));
+    }
+    if (up) for (auto& t : s->uploads) {
+        if (!t.nbytes || !host_ptrs[t.slot]) continue;
+        if (t.nbytes >= STAGE_MIN) {
+            hipError_t err = hipSuccess;
+            const int r = staged_upload((char*)t.staging, (const char*)host_ptrs[t.slot], t.nbytes, [&](size_t off, size_t len) {
+                err = hipMemcpyAsync((char*)t.buf->dptr + t.offset + off, (char*)t.staging + off, len, hipMemcpyHostToDevice, c->stream);
+                return err == hipSuccess ? 0 : 1;
+            });
+            if (r) return hip_fail(err, "hipMemcpyAsync (staged upload)");
+            continue;
+        }
+        memcpy(t.staging, host_ptrs[t.slot], t.nbytes);
+        HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
+    }
+    if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[1], c->stream));
+    // With a fixed landing region nothing is allocated: the following arguments are staged in the
+    // upload's own pinned buffer, which must have been emptied by this evaluation's upload first.
+    bool staging_in_use = false;
+    if (region && next_host_ptrs && up)
+        for (auto& t : s->uploads)
+            if (t.nbytes && t.slot < nslots && next_host_ptrs[t.slot] && host_ptrs && host_ptrs[t.slot]) staging_in_use = true;
+    if (staging_in_use) HIP_TRY(hipEventRecord(c->ev_uploaded, c->stream));
+    if (s->profiling) {
+        for (size_t i = 0; i < s->launches.size(); i++) {
+            if (int r = issue_launch(c, s->launches[i])) return r;
+            HIP_TRY(hipEventRecord(s->stamps[2 + i], c->stream));
+        }
+    } else if (int r = issue_all(c, s)) {
+        return r;
+    }
+    bool landed = false;
+    if (next_host_ptrs) {
+        // While the device works through the launches: stage the following evaluation's arguments and
+        // send them, on the second stream, to landing buffers; once the launches are through, move
+        // them on into the argument buffers with device-to-device copies.
+        bool any = false;
+        size_t region_used = 0;
+        if (staging_in_use) HIP_TRY(hipEventSynchronize(c->ev_uploaded));
+        for (auto& t : s->uploads) {
+            if (!t.nbytes || t.slot >= nslots || !next_host_ptrs[t.slot]) continue;
+            char *staging, *landing;
+            if (region) {
+                staging = (char*)t.staging;
+                landing = region->base + region_used;       // the caller has checked that everything fits
+                region_used += (t.nbytes + 255) & ~(size_t)255;
+            } else {
+                if (!t.landing) {
+                    void *device = nullptr, *pinned = nullptr;
+                    HIP_TRY(hipMalloc(&device, t.nbytes));
+                    hipError_t e = hipHostMalloc(&pinned, t.nbytes, hipHostMallocDefault);
+                    if (e != hipSuccess) { hipFree(device); return hip_fail(e, "hipHostMalloc (staging of the next arguments)"); }
+                    t.landing = device;
+                    t.next_staging = pinned;
+                }
+                staging = (char*)t.next_staging;
+                landing = (char*)t.landing;
+            }
+            hipError_t err = hipSuccess;
+            auto send = [&](size_t off, size_t len) {
+                err = hipMemcpyAsync(landing + off, staging + off, len, hipMemcpyHostToDevice, c->copy_stream);
+                return err == hipSuccess ? 0 : 1;
+            };
+            if (t.nbytes >= STAGE_MIN) {
+                if (staged_upload(staging, (const char*)next_host_ptrs[t.slot], t.nbytes, send))
+                    return hip_fail(err, "hipMemcpyAsync (staged upload of the next arguments)");
+            } else {
+                memcpy(staging, next_host_ptrs[t.slot], t.nbytes);
+                if (send(0, t.nbytes)) return hip_fail(err, "hipMemcpyAsync (upload of the next arguments)");
+            }
+            any = true;
+        }
+        landed = any;
+    }
+    // The downloads are queued after the copies above on purpose: a copy engine works through its
+    // queue in order, and a download queued first waits there for the launches, with every upload
+    // behind it, even one from the other stream, waiting as well.
+    size_t nchunk_events = 0;
+    if (down) for (auto& t : s->downloads) {
+        if (!t.nbytes) continue;
+        if (t.nbytes < STAGE_MIN) {
+            HIP_TRY(hipMemcpyAsync(t.staging, (char*)t.buf->dptr + t.offset, t.nbytes, hipMemcpyDeviceToHost, c->stream));
+            continue;
+        }
+        for (size_t off = 0; off < t.nbytes; off += STAGE_CHUNK, nchunk_events++) {
+            HIP_TRY(hipMemcpyAsync((char*)t.staging + off, (char*)t.buf->dptr + t.offset + off, std::min(STAGE_CHUNK, t.nbytes - off),
+                                   hipMemcpyDeviceToHost, c->stream));
+            HIP_TRY(hipEventRecord(s->chunk_events[nchunk_events], c->stream));
+        }
+    }
+    if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[nstamps - 1], c->stream));
+    if (landed) {
+        HIP_TRY(hipEventRecord(c->ev_landed, c->copy_stream));
+        HIP_TRY(hipStreamWaitEvent(c->stream, c->ev_landed, 0));
+        size_t region_used = 0;
+        for (auto& t : s->uploads) {
+            if (!t.nbytes || t.slot >= nslots || !next_host_ptrs[t.slot]) continue;
+            if (region) {
+                if (int r = region->move((char*)t.buf->dptr + t.offset, region->base + region_used, t.nbytes, c->stream)) return r;
+                region_used += (t.nbytes + 255) & ~(size_t)255;
+            } else {
+                HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.landing, t.nbytes, hipMemcpyDeviceToDevice, c->stream));
+            }
+        }
+    }
+    // large results leave the pinned buffers chunk by chunk as they land; then everything else is waited for
+    if (down) {
+        size_t first_event = 0;
+        for (auto& t : s->downloads) {
+            if (t.nbytes < STAGE_MIN) continue;
+            hipError_t err = hipSuccess;
+            const int r = staged_copy_out((char*)host_ptrs[t.slot], (const char*)t.staging, t.nbytes, [&](size_t k) {
+                err = hipEventSynchronize(s->chunk_events[first_event + k]);
+                return err == hipSuccess ? 0 : 1;
+            });
+            if (r) return hip_fail(err, "hipEventSynchronize (staged download)");
+            first_event += (t.nbytes + STAGE_CHUNK - 1) / STAGE_CHUNK;
+        }
+    }
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    if (down) for (auto& t : s->downloads)
+        if (t.nbytes && t.nbytes < STAGE_MIN) memcpy(host_ptrs[t.slot], t.staging, t.nbytes);
+    if (s->profiling) s->stamps_valid = (int)nstamps;
+    return 0;
+}
+
+
 extern "C" {
 
 const char* vkj_last_error(void) { return g_last_error.c_str(); }
@@ -288,10 +363,23 @@ int vkj_ctx_create(int device, vkj_handle* out) {
     Ctx* c = new (std::nothrow) Ctx();
     if (!c) return fail(VKJ_ENOMEM, "vkj_ctx_create: out of host memory");
     c->device = device;
-    HIP_TRY(hipSetDevice(device));
-    HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-    HIP_TRY(hipEventCreate(&c->ev_begin));
-    HIP_TRY(hipEventCreate(&c->ev_end));
+    // everything an evaluation needs besides its own buffers is made here, so that none of the
+    // evaluation entry points has to create a stream or an event
+    int r = [&]() -> int {
+        HIP_TRY(hipSetDevice(device));
+        HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+        HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
+        HIP_TRY(hipEventCreate(&c->ev_begin));
+        HIP_TRY(hipEventCreate(&c->ev_end));
+        HIP_TRY(hipEventCreateWithFlags(&c->ev_landed, hipEventDisableTiming));
+        HIP_TRY(hipEventCreateWithFlags(&c->ev_uploaded, hipEventDisableTiming));
+        return 0;
+    }();
+    if (r) {
+        destroy_ctx_objects(c);
+        delete c;
+        return r;
+    }
     *out = to_handle(c);
     return 0;
 }
@@ -301,11 +389,8 @@ int vkj_ctx_destroy(vkj_handle h) {
     if (!c) return fail(VKJ_EINVAL, "vkj_ctx_destroy: bad context handle");
     if (int r = use(c)) return r;
     hipStreamSynchronize(c->stream);
-    hipEventDestroy(c->ev_begin);
-    hipEventDestroy(c->ev_end);
-    hipStreamDestroy(c->stream);
-    if (c->copy_stream) { hipStreamSynchronize(c->copy_stream); hipStreamDestroy(c->copy_stream); }
-    if (c->ev_landed) hipEventDestroy(c->ev_landed);
+    hipStreamSynchronize(c->copy_stream);
+    destroy_ctx_objects(c);
     retire(c);
     delete c;
     return 0;
@@ -356,9 +441,14 @@ int vkj_module_unload(vkj_handle h, vkj_handle mh) {
     Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
     Mod* m = from_handle<Mod>(mh, MAGIC_MOD);
     if (!c || !m || m->ctx != c) return fail(VKJ_EINVAL, "vkj_module_unload: bad handle");
+    if (m->seq_refs > 0)
+        return fail(VKJ_ESTATE, "vkj_module_unload: %d recorded launch(es) of live sequences use this module; destroy those sequences first",
+                    m->seq_refs);
     if (int r = use(c)) return r;
     HIP_TRY(hipStreamSynchronize(c->stream));
     HIP_TRY(hipModuleUnload(m->module));
+    // the module's function handles go with it: a later use of one is rejected as a bad handle
+    for (Fn* f : m->functions) { retire(f); delete f; }
     retire(m);
     delete m;
     return 0;
@@ -379,7 +469,8 @@ int vkj_module_get_function(vkj_handle h, vkj_handle mh, const char* name, vkj_h
         g_last_error = std::string("kernel '") + name + "' not found in module: " + hipGetErrorString(e);
         return (int)e;
     }
-    *out = to_handle(f);   // lives as long as the process; functions are few and tiny
+    m->functions.push_back(f);   // lives as long as its module
+    *out = to_handle(f);
     return 0;
 }
 
@@ -402,7 +493,15 @@ int vkj_buf_free(vkj_handle h, vkj_handle bh) {
     Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
     if (!c || !b || b->ctx != c) return fail(VKJ_EINVAL, "vkj_buf_free: bad handle");
     if (int r = use(c)) return r;
+    if (b->seq_refs > 0) {
+        // recorded into live sequences, which hold its address: the handle is retired now (any later
+        // use of it is rejected), the memory is released when the last of those sequences is destroyed
+        retire(b);
+        b->released = true;
+        return 0;
+    }
     HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(hipStreamSynchronize(c->copy_stream));
     HIP_TRY(hipFree(b->dptr));
     retire(b);
     delete b;
@@ -483,13 +582,21 @@ int vkj_seq_destroy(vkj_handle sh) {
     if (!s) return fail(VKJ_EINVAL, "vkj_seq_destroy: bad handle");
     if (int r = use(s->ctx)) return r;
     hipStreamSynchronize(s->ctx->stream);
-    if (s->ctx->copy_stream) hipStreamSynchronize(s->ctx->copy_stream);
+    hipStreamSynchronize(s->ctx->copy_stream);
     for (auto& t : s->uploads) {
         if (t.staging) hipHostFree(t.staging);
         if (t.next_staging) hipHostFree(t.next_staging);
         if (t.landing) hipFree(t.landing);
+        unref_buf(t.buf);
     }
-    for (auto& t : s->downloads) if (t.staging) hipHostFree(t.staging);
+    for (auto& t : s->downloads) {
+        if (t.staging) hipHostFree(t.staging);
+        unref_buf(t.buf);
+    }
+    for (auto& l : s->launches) {
+        l.fn->mod->seq_refs--;
+        for (Buf* b : l.bufs) unref_buf(b);
+    }
     for (auto e : s->stamps) hipEventDestroy(e);
     for (auto e : s->chunk_events) hipEventDestroy(e);
     drop_graph(s);
@@ -507,6 +614,7 @@ static int record_transfer(const char* who, std::vector<Transfer>& list, Seq* s,
     Transfer t{b, offset, nbytes, slot, nullptr};
     if (nbytes) HIP_TRY(hipHostMalloc(&t.staging, nbytes, hipHostMallocDefault));
     list.push_back(t);
+    b->seq_refs++;
     return 0;
 }
 
@@ -519,7 +627,16 @@ int vkj_seq_record_upload(vkj_handle sh, vkj_handle bh, size_t offset, int slot,
 int vkj_seq_record_download(vkj_handle sh, vkj_handle bh, size_t offset, int slot, size_t nbytes) {
     Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
     if (!s) return fail(VKJ_EINVAL, "vkj_seq_record_download: bad sequence handle");
-    return record_transfer("vkj_seq_record_download", s->downloads, s, bh, offset, slot, nbytes);
+    if (int r = record_transfer("vkj_seq_record_download", s->downloads, s, bh, offset, slot, nbytes)) return r;
+    // a large result comes back in chunks with an event behind each; the events are made here so
+    // that an evaluation creates nothing
+    if (nbytes >= STAGE_MIN)
+        for (size_t off = 0; off < nbytes; off += STAGE_CHUNK) {
+            hipEvent_t e;
+            HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            s->chunk_events.push_back(e);
+        }
+    return 0;
 }
 
 int vkj_seq_record_launch(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], const uint32_t block[3],
@@ -552,7 +669,10 @@ int vkj_seq_record_launch(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], 
             return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): pointer slot #%d outside the argument block or misaligned", f->name.c_str(), i);
         uint64_t addr = (uint64_t)(uintptr_t)b->dptr + off;
         memcpy(l.kernarg.data() + buf_arg_offsets[i], &addr, 8);
+        l.bufs.push_back(b);
     }
+    for (Buf* b : l.bufs) b->seq_refs++;
+    f->mod->seq_refs++;
     s->launches.push_back(std::move(l));
     drop_graph(s);                                  // a captured graph no longer matches the sequence
     return 0;
@@ -574,129 +694,7 @@ int vkj_seq_eval(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t fla
 int vkj_seq_eval_next(vkj_handle sh, void* const* host_ptrs, int nslots, uint32_t flags, void* const* next_host_ptrs) {
     Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
     if (!s) return fail(VKJ_EINVAL, "vkj_seq_eval: bad handle");
-    Ctx* c = s->ctx;
-    if (int r = use(c)) return r;
-    if (next_host_ptrs && !c->copy_stream) {
-        HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
-        HIP_TRY(hipEventCreateWithFlags(&c->ev_landed, hipEventDisableTiming));
-    }
-    const bool up = !(flags & VKJ_EVAL_SKIP_UPLOADS), down = !(flags & VKJ_EVAL_SKIP_DOWNLOADS);
-    auto slot_ok = [&](const Transfer& t) { return t.nbytes == 0 || (host_ptrs && t.slot < nslots && host_ptrs[t.slot]); };
-    const bool null_resident = flags & VKJ_EVAL_NULL_IS_RESIDENT;
-    if (up)   for (auto& t : s->uploads)   if (!slot_ok(t) && !(null_resident && host_ptrs && t.slot < nslots))
-        return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for upload slot %d", t.slot);
-    if (down) for (auto& t : s->downloads) if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for download slot %d", t.slot);
-
-    size_t nstamps = 0;
-    if (s->profiling) {
-        nstamps = 3 + s->launches.size();       // begin, after uploads, after each launch, after downloads
-        while (s->stamps.size() < nstamps) {
-            hipEvent_t e;
-            HIP_TRY(hipEventCreate(&e));
-            s->stamps.push_back(e);
-        }
-        s->stamps_valid = 0;
-        HIP_TRY(hipEventRecord(s->stamps[0], c->stream));
-    }
-    if (up) for (auto& t : s->uploads) {
-        if (!t.nbytes || !host_ptrs[t.slot]) continue;
-        if (t.nbytes >= STAGE_MIN) {
-            hipError_t err = hipSuccess;
-            const int r = staged_upload((char*)t.staging, (const char*)host_ptrs[t.slot], t.nbytes, [&](size_t off, size_t len) {
-                err = hipMemcpyAsync((char*)t.buf->dptr + t.offset + off, (char*)t.staging + off, len, hipMemcpyHostToDevice, c->stream);
-                return err == hipSuccess ? 0 : 1;
-            });
-            if (r) return hip_fail(err, "hipMemcpyAsync (staged upload)");
-            continue;
-        }
-        memcpy(t.staging, host_ptrs[t.slot], t.nbytes);
-        HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
-    }
-    if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[1], c->stream));
-    if (s->profiling) {
-        for (size_t i = 0; i < s->launches.size(); i++) {
-            if (int r = issue_launch(c, s->launches[i])) return r;
-            HIP_TRY(hipEventRecord(s->stamps[2 + i], c->stream));
-        }
-    } else if (int r = issue_all(c, s)) {
-        return r;
-    }
-    bool landed = false;
-    if (next_host_ptrs) {
-        // While the device works through the launches: stage the following evaluation's arguments and
-        // send them, on the second stream, to landing buffers; once the launches are through, move
-        // them on into the argument buffers with device-to-device copies.
-        bool any = false;
-        for (auto& t : s->uploads) {
-            if (!t.nbytes || t.slot >= nslots || !next_host_ptrs[t.slot]) continue;
-            if (!t.landing) {
-                HIP_TRY(hipHostMalloc(&t.next_staging, t.nbytes, hipHostMallocDefault));
-                HIP_TRY(hipMalloc(&t.landing, t.nbytes));
-            }
-            hipError_t err = hipSuccess;
-            auto send = [&](size_t off, size_t len) {
-                err = hipMemcpyAsync((char*)t.landing + off, (char*)t.next_staging + off, len, hipMemcpyHostToDevice, c->copy_stream);
-                return err == hipSuccess ? 0 : 1;
-            };
-            if (t.nbytes >= STAGE_MIN) {
-                if (staged_upload((char*)t.next_staging, (const char*)next_host_ptrs[t.slot], t.nbytes, send))
-                    return hip_fail(err, "hipMemcpyAsync (staged upload of the next arguments)");
-            } else {
-                memcpy(t.next_staging, next_host_ptrs[t.slot], t.nbytes);
-                if (send(0, t.nbytes)) return hip_fail(err, "hipMemcpyAsync (upload of the next arguments)");
-            }
-            any = true;
-        }
-        landed = any;
-    }
-    // The downloads are queued after the copies above on purpose: a copy engine works through its
-    // queue in order, and a download queued first waits there for the launches, with every upload
-    // behind it, even one from the other stream, waiting as well.
-    size_t nchunk_events = 0;
-    if (down) for (auto& t : s->downloads) {
-        if (!t.nbytes) continue;
-        if (t.nbytes < STAGE_MIN) {
-            HIP_TRY(hipMemcpyAsync(t.staging, (char*)t.buf->dptr + t.offset, t.nbytes, hipMemcpyDeviceToHost, c->stream));
-            continue;
-        }
-        for (size_t off = 0; off < t.nbytes; off += STAGE_CHUNK, nchunk_events++) {
-            if (s->chunk_events.size() <= nchunk_events) {
-                hipEvent_t e;
-                HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-                s->chunk_events.push_back(e);
-            }
-            HIP_TRY(hipMemcpyAsync((char*)t.staging + off, (char*)t.buf->dptr + t.offset + off, std::min(STAGE_CHUNK, t.nbytes - off),
-                                   hipMemcpyDeviceToHost, c->stream));
-            HIP_TRY(hipEventRecord(s->chunk_events[nchunk_events], c->stream));
-        }
-    }
-    if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[nstamps - 1], c->stream));
-    if (landed) {
-        HIP_TRY(hipEventRecord(c->ev_landed, c->copy_stream));
-        HIP_TRY(hipStreamWaitEvent(c->stream, c->ev_landed, 0));
-        for (auto& t : s->uploads)
-            if (t.nbytes && t.slot < nslots && next_host_ptrs[t.slot])
-                HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.landing, t.nbytes, hipMemcpyDeviceToDevice, c->stream));
-    }
-    // large results leave the pinned buffers chunk by chunk as they land; then everything else is waited for
-    if (down) {
-        size_t first_event = 0;
-        for (auto& t : s->downloads) {
-            if (t.nbytes < STAGE_MIN) continue;
-            hipError_t err = hipSuccess;
-            const int r = staged_copy_out((char*)host_ptrs[t.slot], (const char*)t.staging, t.nbytes, [&](size_t k) {
-                err = hipEventSynchronize(s->chunk_events[first_event + k]);
-                return err == hipSuccess ? 0 : 1;
-            });
-            if (r) return hip_fail(err, "hipEventSynchronize (staged download)");
-            first_event += (t.nbytes + STAGE_CHUNK - 1) / STAGE_CHUNK;
-        }
-    }
-    HIP_TRY(hipStreamSynchronize(c->stream));
-    if (down) for (auto& t : s->downloads)
-        if (t.nbytes && t.nbytes < STAGE_MIN) memcpy(host_ptrs[t.slot], t.staging, t.nbytes);
-    if (s->profiling) s->stamps_valid = (int)nstamps;
-    return 0;
+    return seq_eval(s, host_ptrs, nslots, flags, next_host_ptrs, nullptr);
 }
 
 int vkj_seq_replay(vkj_handle sh, int iters, float* ms_total) {
