@@ -128,6 +128,18 @@ int vkj_seq_eval(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t fl
  * turn (vkjax/kompute_jaxpr_interpreter.py:72-77); this is the overlap of the two. */
 int vkj_seq_eval_next(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t flags,
                       void* const* next_host_ptrs);
+/* vkj_seq_eval_next that allocates nothing. No counterpart in the reference; it is for callers that
+ * cannot allocate device or pinned memory where they evaluate (serving loops, harnesses that
+ * forbid hipMalloc): the following evaluation's arguments land in an array of
+ * VKJ_STATIC_LANDING_BYTES that is part of the library's device image (every GPU the library runs
+ * on holds one copy until the process ends), are staged in the pinned buffers the sequence already
+ * owns, and are moved on by a copy kernel. Slots are packed at multiples of 256 bytes; arguments
+ * that do not fit are rejected with VKJ_EINVAL, sequences with timestamps, or with a graph that is
+ * not built yet, with VKJ_ESTATE. All calls on one GPU share the array: calls that overlap in time
+ * on one GPU race. Same arguments and results as vkj_seq_eval_next otherwise. */
+#define VKJ_STATIC_LANDING_BYTES (64u << 20)
+int vkj_seq_eval_next_static(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t flags,
+                             void* const* next_host_ptrs);
 /* Launches only, `iters` times back to back, bracketed by two events on the context's
  * stream; *ms_total receives the elapsed device time of all iterations. Used for
  * measurement with inputs resident in HBM. No counterpart in the reference. */

@@ -47,14 +47,21 @@ def _newer(target, sources):
 
 
 def build_shim(force=True):
-    src = os.path.join(CSRC, 'shim.cpp')
-    hdr = os.path.join(INCLUDE, 'vkjax_hip.h')
+    '''libvkjax_hip.so = shim.cpp (host only) + static_landing.hip (the static landing array, its
+    copy kernel and the entry point that allocates nothing).'''
+    srcs = [os.path.join(CSRC, 'shim.cpp'), os.path.join(CSRC, 'static_landing.hip')]
+    hdrs = [os.path.join(INCLUDE, 'vkjax_hip.h'), os.path.join(CSRC, 'shim_internal.h')]
     out = shim_path()
-    if not force and _newer(out, [src, hdr]):
+    if not force and _newer(out, srcs + hdrs):
         return out
-    _run([HIPCC, '-O2', '-fPIC', '-shared', '-pthread', '-std=c++17', '-x', 'c++', '-D__HIP_PLATFORM_AMD__',
-          f'-I{INCLUDE}', '-I/opt/rocm/include', src, '-o', out, '-L/opt/rocm/lib', '-lamdhip64',
-          '-Wl,-rpath,/opt/rocm/lib'])
+    common = ['-O2', '-fPIC', '-pthread', '-std=c++17', f'-I{INCLUDE}', f'-I{CSRC}', '-I/opt/rocm/include']
+    objs = [os.path.join(LIBDIR, 'shim.o'), os.path.join(LIBDIR, 'static_landing.o')]
+    _run([HIPCC] + common + ['-x', 'c++', '-D__HIP_PLATFORM_AMD__', '-c', srcs[0], '-o', objs[0]])
+    _run([HIPCC] + common + [f'--offload-arch={ARCH}', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+                             '-c', srcs[1], '-o', objs[1]])
+    _run([HIPCC, '-shared', '-pthread'] + objs + ['-o', out, '-L/opt/rocm/lib', '-lamdhip64', '-Wl,-rpath,/opt/rocm/lib'])
+    for o in objs:
+        os.remove(o)
     return out
 
 

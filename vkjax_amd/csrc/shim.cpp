@@ -373,7 +373,7 @@ int vkj_ctx_create(int device, vkj_handle* out) {
         HIP_TRY(hipEventCreate(&c->ev_end));
         HIP_TRY(hipEventCreateWithFlags(&c->ev_landed, hipEventDisableTiming));
         HIP_TRY(hipEventCreateWithFlags(&c->ev_uploaded, hipEventDisableTiming));
-        return 0;
+        return static_landing_init(c);
     }();
     if (r) {
         destroy_ctx_objects(c);

@@ -22,6 +22,7 @@ KERNEL_MODULES = ('elementwise', 'conv_gemm', 'wgrad_gemm', 'reduce', 'index', '
 EVAL_SKIP_UPLOADS   = 1
 EVAL_SKIP_DOWNLOADS = 2
 EVAL_NULL_IS_RESIDENT = 4
+STATIC_LANDING_BYTES  = 64 << 20       #VKJ_STATIC_LANDING_BYTES
 
 
 class Props(C.Structure):
@@ -61,6 +62,7 @@ _PROTOTYPES = {
     'vkj_seq_num_steps':       (C.c_int, [_H, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     'vkj_seq_eval':            (C.c_int, [_H, C.POINTER(C.c_void_p), C.c_int, C.c_uint32]),
     'vkj_seq_eval_next':       (C.c_int, [_H, C.POINTER(C.c_void_p), C.c_int, C.c_uint32, C.POINTER(C.c_void_p)]),
+    'vkj_seq_eval_next_static': (C.c_int, [_H, C.POINTER(C.c_void_p), C.c_int, C.c_uint32, C.POINTER(C.c_void_p)]),
     'vkj_seq_replay':          (C.c_int, [_H, C.c_int, C.POINTER(C.c_float)]),
     'vkj_seq_use_graph':       (C.c_int, [_H, C.c_int]),
     'vkj_seq_timestamps':      (C.c_int, [_H, C.POINTER(C.c_float), C.c_int, C.POINTER(C.c_int)]),
@@ -278,23 +280,26 @@ class Sequence:
         self.n_launches += 1
 
     def eval(self, host_arrays: tp.Sequence[tp.Optional[np.ndarray]], flags: int = 0,
-             next_host_arrays: tp.Optional[tp.Sequence[tp.Optional[np.ndarray]]] = None):
+             next_host_arrays: tp.Optional[tp.Sequence[tp.Optional[np.ndarray]]] = None, static_landing: bool = False):
         '''`next_host_arrays`: the arguments of the following evaluation (None per slot that stays as
         it is); they are uploaded while the device runs this one, and the following call passes None
-        for them with EVAL_NULL_IS_RESIDENT.'''
+        for them with EVAL_NULL_IS_RESIDENT. `static_landing`: through vkj_seq_eval_next_static, which
+        allocates nothing and takes at most STATIC_LANDING_BYTES of following arguments.'''
         def pointers(arrays):
             ptrs = (C.c_void_p * max(len(arrays), 1))()
             for i, a in enumerate(arrays):
                 ptrs[i] = a.ctypes.data if a is not None else None
             return ptrs
         ptrs = pointers(host_arrays)
-        if next_host_arrays is None:
+        if next_host_arrays is None and not static_landing:
             _check(self.device.lib.vkj_seq_eval(self.handle, ptrs, len(host_arrays), flags), 'vkj_seq_eval')
             return
+        if next_host_arrays is None:
+            next_host_arrays = [None] * len(host_arrays)
         if len(next_host_arrays) != len(host_arrays):
             raise ValueError('next_host_arrays must have one entry per slot')
-        _check(self.device.lib.vkj_seq_eval_next(self.handle, ptrs, len(host_arrays), flags, pointers(next_host_arrays)),
-               'vkj_seq_eval_next')
+        name = 'vkj_seq_eval_next_static' if static_landing else 'vkj_seq_eval_next'
+        _check(getattr(self.device.lib, name)(self.handle, ptrs, len(host_arrays), flags, pointers(next_host_arrays)), name)
 
     def replay(self, iters: int = 1) -> float:
         '''Launches only; returns elapsed device milliseconds for all iterations.'''
