@@ -121,13 +121,13 @@ def test_gather_scatter_small_exact_and_full():
     assert np.allclose(acc, expected, rtol=1e-5, atol=1e-6)
 
 
-def test_scatter_add_rows_owner_sorted_and_atomic_paths():
-    '''Row scatter-add through all three implementations (one launch in which every workgroup owns a range of
-    table rows; buckets from a counting sort of the indices; HBM atomics): integer-valued updates make every
-    sum exact. Cases cover rows that receive no update, one row that receives more than 64, more updates for one
-    workgroup's rows than its LDS holds (several rounds), indices outside the table (dropped), row lengths that
-    are not a multiple of 4 or longer than one pass of a wave, integer data, operands that are not zero, and a
-    constant table filled with one value (not read at all).'''
+def test_scatter_add_rows_sorted_and_atomic_paths():
+    '''Row scatter-add through both implementations (buckets from a counting sort of the indices; HBM atomics):
+    integer-valued updates make every sum exact. Cases cover rows that receive no update, rows that receive more
+    than 16 and more than 64, indices outside the table (dropped), row lengths that are not a multiple of 4 or
+    longer than one pass of a wave, integer data, operands that are not zero, more than 256 x 1024 table rows
+    (bucket starts in segments of several tiles), a constant table filled with one value (not read at all), and
+    evaluating twice (the counters go back to zero).'''
     from vkjax_amd import ops
     rng = np.random.default_rng(7)
 
@@ -139,22 +139,28 @@ def test_scatter_add_rows_owner_sorted_and_atomic_paths():
             return mj.numpy.index_add(mj.numpy.full((300, 64), fill, np.float32), idx, updates)
         return f
 
-    saved = ops.SCATTER_SORT_THRESHOLD, ops.SCATTER_OWNER_MAX_IDX
+    saved = ops.SCATTER_SORT_THRESHOLD
     try:
-        for path, threshold, owner_max in (('owner', 0, saved[1]), ('sum', 0, 0), ('atomic', 1 << 60, saved[1])):
-            ops.SCATTER_SORT_THRESHOLD, ops.SCATTER_OWNER_MAX_IDX = threshold, owner_max
+        for path, threshold in (('sum', 0), ('atomic', 1 << 60)):
+            ops.SCATTER_SORT_THRESHOLD = threshold
             cases = [(50, 256, 400, np.float32), (9, 10, 37, np.float32), (300, 64, 200, np.int32), (4, 20, 500, np.float32),
                      (3000, 16, 9000, np.float32), (70, 520, 300, np.float32), (5, 8, 20000, np.int32), (1029, 4, 30000, np.float32),
-                     (300000, 4, 5000, np.float32)]                        #1024 rows per workgroup
+                     (300000, 4, 5000, np.float32), (1025, 4, 3000, np.int32), (1024, 4, 3000, np.int32), (1023, 4, 3000, np.int32)]
             for rows, cols, n, dtype in cases:
                 table   = rng.integers(-9, 9, size=(rows, cols)).astype(dtype)
                 idx     = rng.integers(0, rows, size=(n,)).astype(np.int32)
                 idx[: n // 3] = idx[0]                                 #one crowded row
+                idx[n // 3: n // 3 + 20] = (idx[0] + 1) % rows         #and one with 20 or so
                 updates = rng.integers(-5, 6, size=(n, cols)).astype(dtype)
                 _, _, fn = check_against_oracle(scatter, [table, idx, updates], exact=True)
                 kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
                 assert any(k.startswith('scatter_rows_sum') for k in kernels) == (path == 'sum'), kernels
-                assert any(k.startswith('scatter_rows_owner') for k in kernels) == (path == 'owner'), kernels
+                #again, other values: nothing may be left over from the first evaluation
+                updates2 = rng.integers(-5, 6, size=(n, cols)).astype(dtype)
+                idx2     = rng.permutation(idx)
+                expected = table.copy()
+                np.add.at(expected, idx2, updates2)
+                assert np.array_equal(fn(table, idx2, updates2), expected), (path, rows, cols, n)
             #indices beyond the table (jnp's normalisation only wraps negative ones)
             table   = np.zeros((16, 8), np.float32)
             idx     = np.array([3, 99, 16, 15, -1, 3], np.int32)
@@ -165,11 +171,11 @@ def test_scatter_add_rows_owner_sorted_and_atomic_paths():
                 idx     = rng.integers(0, 300, size=(700,)).astype(np.int32)
                 updates = rng.integers(-5, 6, size=(700, 64)).astype(np.float32)
                 _, _, fn = check_against_oracle(scatter_into_constant(fill), [idx, updates], exact=True)
-                if path == 'owner':
-                    launch = [l for l in list(fn._jaxpr_interpreters.values())[0].launches if l.kernel.startswith('scatter_rows_owner')][0]
+                if path == 'sum':
+                    launch = [l for l in list(fn._jaxpr_interpreters.values())[0].launches if l.kernel.startswith('scatter_rows_sum')][0]
                     assert launch.buffers[1][0].size == 1, 'the constant table should have been replaced by its value'
     finally:
-        ops.SCATTER_SORT_THRESHOLD, ops.SCATTER_OWNER_MAX_IDX = saved
+        ops.SCATTER_SORT_THRESHOLD = saved
 
 
 def test_fusion_does_not_change_a_single_bit():

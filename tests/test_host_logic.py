@@ -95,8 +95,8 @@ def test_kernel_argument_layouts_match_the_structs():
         'GatherRowsParams': K.gather_rows(b(3, 8), b(4, 8), i(3, 1), 3, 8, 4),
         'GatherGeneralParams': K.gather_general(b(3, 8), b(4, 8), i(3, 1), (1,), (0,), (0,), (1, 8)),
         'ScatterRowsParams': K.scatter_add_rows(b(4, 8), i(3, 1), b(3, 8), 3, 8, 4),
-        'ScatterSortParams': K.scatter_add_rows_sorted(b(4, 8), b(4, 8), i(3, 1), b(3, 8), Buffer(None, np.dtype('uint32'), (10,)),
-                                                       Buffer(None, np.dtype('uint32'), (3,)), 3, 8, 4)[1],
+        'ScatterSortParams': K.scatter_add_rows_sorted(b(4, 8), b(4, 8), i(3, 1), b(3, 8), *[Buffer(None, np.dtype('uint32'), (n,)) for n in (4, 5, 3, 3)],
+                                                       3, 8, 4)[0],
         'ScatterGeneralParams': K.scatter_add_general(b(4, 8), i(3, 1), b(3, 8), (1,), (0,), (0,)),
         'ThreefryParams': K.threefry2x32(*[Buffer(None, np.dtype('uint32'), (8,)) for _ in range(6)], key_is_scalar=False),
         'ThreefryStreamParams': K.threefry_stream(Buffer(None, np.dtype('uint32'), (16,)), (Buffer(None, np.dtype('uint32'), (2,)), 0),

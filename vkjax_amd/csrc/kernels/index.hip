@@ -101,85 +101,94 @@ extern "C" __global__ __launch_bounds__(256) void scatter_add_rows(uint32_t* __r
 // ---------------------------------------------------------------------------------------------
 // scatter-add of whole rows without atomics on the data: the update rows are bucketed by target
 // row with a counting sort of their indices (three small launches over the indices), then one
-// wave per table row adds up its updates, in ascending update order, on top of the operand row and
-// writes the result once. Every update row is read exactly once, the table is read once and
-// written once, and the sum does not depend on the order in which threads happen to run (rows
-// that receive more than 64 updates are summed in blocks of 64, each block in ascending order).
-struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride; };
+// wave per table row adds up its updates, in ascending update order, on top of the operand row
+// (or of one value, when the operand is a constant filled with it) and writes the result once.
+// Every update row is read exactly once, the table is written once, and for rows that receive at
+// most 64 updates the sum does not depend on the order in which threads happen to run (rows with
+// more are summed in blocks of 64, each block in ascending order; which updates share a block
+// depends on the order of arrival).
+// Scratch: count (n_rows words, all zero before and after), start (n_rows + 1), rank and order
+// (n_idx each).
+struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride, operand_is_scalar; };
 
-// count[r + 1] += 1 for every in-range index; count has n_rows + 1 words and starts at zero
-extern "C" __global__ __launch_bounds__(256) void scatter_rows_count(uint32_t* __restrict__ count, const int32_t* __restrict__ idx,
-                                                                     ScatterSortParams P) {
+#define SCATTER_DROPPED 0xFFFFFFFFu
+
+// rank[i] = how many updates for the same row arrived before update i (the counter's old value);
+// updates outside the operand are dropped
+extern "C" __global__ __launch_bounds__(256) void scatter_rows_rank(uint32_t* __restrict__ count, uint32_t* __restrict__ rank,
+                                                                    const int32_t* __restrict__ idx, ScatterSortParams P) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= P.n_idx) return;
     const int32_t r = idx[(uint64_t)i * P.idx_stride];
-    if (r < 0 || r >= (int32_t)P.n_rows) return;          // updates outside the operand are dropped
-    atomicAdd(count + r + 1, 1u);
+    uint32_t k = SCATTER_DROPPED;
+    if (r >= 0 && r < (int32_t)P.n_rows) k = atomicAdd(count + r, 1u);
+    rank[i] = k;
 }
 
-// in-place inclusive prefix sum over n words by one block: afterwards word r is the number of
-// updates that go to rows before r, i.e. where row r's bucket starts. The block walks the array
-// in tiles of 1024 x 16 words; a thread scans 16 consecutive words, the 1024 thread totals are
-// scanned with wave shuffles and one exchange through LDS, and a running carry links the tiles.
-extern "C" __global__ __launch_bounds__(1024) void scatter_rows_scan(uint32_t* __restrict__ data, uint32_t n) {
-    __shared__ uint32_t wave_total[16];
+// start[r] = number of updates for rows before r (r = 0 .. n_rows: where row r's bucket begins).
+// Workgroup b produces words [b * seg, (b + 1) * seg) of start, seg a multiple of 1024: it first adds up
+// all counts before its segment itself, so no workgroup waits for another (a fence between
+// workgroups writes back the whole L2 on this GPU, 60 us), then scans its segment in tiles of 1024.
+extern "C" __global__ __launch_bounds__(1024) void scatter_rows_starts(uint32_t* __restrict__ start, const uint32_t* __restrict__ count,
+                                                                       uint32_t n_rows, uint32_t seg) {
+    __shared__ uint32_t wave_total[4], wave_before[16];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    uint32_t carry = 0;
-    for (uint32_t tile = 0; tile < n; tile += 1024u * 16u) {
-        const uint32_t base = tile + threadIdx.x * 16u;
-        uint32_t v[16];
-        if (base + 16u <= n) {                                   // 64 aligned bytes per thread
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const u32x4 t4 = *reinterpret_cast<const u32x4*>(data + base + 4 * q);
-                v[4 * q] = t4.x; v[4 * q + 1] = t4.y; v[4 * q + 2] = t4.z; v[4 * q + 3] = t4.w;
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < 16; ++q) v[q] = base + q < n ? data[base + q] : 0u;
+    const uint32_t first = blockIdx.x * seg;                               // <= n_rows (the grid sees to that)
+    uint32_t before = 0;
+    {
+        const u32x4* c4 = reinterpret_cast<const u32x4*>(count);           // first is a multiple of 1024 words
+        const uint32_t nvec = first >> 2;
+        uint32_t v = threadIdx.x;
+        for (; v + 3072u < nvec; v += 4096u) {
+            const u32x4 a = c4[v], b = c4[v + 1024u], c = c4[v + 2048u], d = c4[v + 3072u];
+            before += (a.x + a.y + a.z + a.w) + (b.x + b.y + b.z + b.w) + (c.x + c.y + c.z + c.w) + (d.x + d.y + d.z + d.w);
         }
+        for (; v < nvec; v += 1024u) { const u32x4 a = c4[v]; before += a.x + a.y + a.z + a.w; }
+    }
+    before = wave_allreduce(before, [](uint32_t a, uint32_t b) { return a + b; });
+    if (lane == 0u) wave_before[wave] = before;
+    __syncthreads();
+    const bool scans = wave < 4u;                                          // the tiles are scanned by the first four waves
+    uint32_t carry = 0;
 #pragma unroll
-        for (int q = 1; q < 16; ++q) v[q] += v[q - 1];
-        // inclusive scan of the thread totals across the wave
-        uint32_t t = v[15];
+    for (int w = 0; w < 16; ++w) carry += wave_before[w];
+    for (uint32_t tile = first; tile < first + seg && tile <= n_rows; tile += 1024u) {
+        const uint32_t base = tile + (threadIdx.x & 255u) * 4u;
+        uint32_t v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = scans && base + q < n_rows ? count[base + q] : 0u;
+        const uint32_t own = v[0] + v[1] + v[2] + v[3];
+        uint32_t t = own;                                                  // inclusive scan over the wave
 #pragma unroll
         for (uint32_t off = 1; off < 64u; off <<= 1) {
             const uint32_t up = __shfl_up(t, off, 64);
             if (lane >= off) t += up;
         }
-        if (lane == 63u) wave_total[wave] = t;
+        if (scans && lane == 63u) wave_total[wave] = t;
         __syncthreads();
-        uint32_t before = carry;                                 // everything before this thread's 16 words
-        for (uint32_t w = 0; w < wave; ++w) before += wave_total[w];
-        before += t - v[15];
-        uint32_t tile_total = 0;
-        for (uint32_t w = 0; w < 16u; ++w) tile_total += wave_total[w];
-        __syncthreads();                                         // wave_total is rewritten by the next tile
-        if (base + 16u <= n) {
+        uint32_t x = carry + t - own;
+        for (uint32_t w = 0; w < (wave & 3u); ++w) x += wave_total[w];
+        const uint32_t tile_total = wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+        __syncthreads();                                                   // wave_total is rewritten by the next tile
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                u32x4 t4;
-                t4.x = v[4 * q] + before; t4.y = v[4 * q + 1] + before; t4.z = v[4 * q + 2] + before; t4.w = v[4 * q + 3] + before;
-                *reinterpret_cast<u32x4*>(data + base + 4 * q) = t4;
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < 16; ++q)
-                if (base + q < n) data[base + q] = v[q] + before;
+        for (int q = 0; q < 4; ++q) {
+            if (scans && base + q <= n_rows) start[base + q] = x;
+            x += v[q];
         }
         carry += tile_total;
     }
 }
 
-// order[start[r] + k] = i for the k-th update (in order of arrival) whose index is r; cursor starts at zero
-extern "C" __global__ __launch_bounds__(256) void scatter_rows_fill(uint32_t* __restrict__ order, uint32_t* __restrict__ cursor,
-                                                                    const uint32_t* __restrict__ start, const int32_t* __restrict__ idx,
-                                                                    ScatterSortParams P) {
+// order[start[idx[i]] + rank[i]] = i, and the counts go back to zero for the next evaluation
+extern "C" __global__ __launch_bounds__(256) void scatter_rows_order(uint32_t* __restrict__ order, uint32_t* __restrict__ count,
+                                                                     const uint32_t* __restrict__ start, const uint32_t* __restrict__ rank,
+                                                                     const int32_t* __restrict__ idx, ScatterSortParams P) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < P.n_rows) count[i] = 0u;
     if (i >= P.n_idx) return;
-    const int32_t r = idx[(uint64_t)i * P.idx_stride];
-    if (r < 0 || r >= (int32_t)P.n_rows) return;
-    order[start[r] + atomicAdd(cursor + r, 1u)] = i;
+    const uint32_t k = rank[i];
+    if (k == SCATTER_DROPPED) return;
+    order[start[idx[(uint64_t)i * P.idx_stride]] + k] = i;
 }
 
 // ascending bitonic sort of one value per lane across the wave
@@ -196,101 +205,75 @@ __device__ __forceinline__ uint32_t wave_sort(uint32_t e, uint32_t lane) {
     return e;
 }
 
-// out[r, :] = operand[r, :] + sum over the updates i in row r's bucket of updates[i, :].
-// One wave takes 4 consecutive rows. Their buckets are adjacent in `order`, so one load fetches
-// them all (up to 64 entries, the usual case); they are sorted together under the key
-// (row, update number), and all the rows' loads of operand and update data are in flight together.
-// A wave whose rows hold more than 64 entries falls back to one row at a time, 64 entries at a time.
-// Update numbers are below 2^30 (the host sees to that).
-#define SCATTER_ROWS_PER_WAVE 4
+// The first n lanes hold distinct values, the others 0xFFFFFFFF: ascending order over the lanes.
+// Few values (the usual bucket): every lane counts the values below its own and sends its value there.
+__device__ __forceinline__ uint32_t wave_sort_first(uint32_t e, uint32_t n, uint32_t lane) {
+    if (n <= 1u) return e;
+    if (n > 16u) return wave_sort(e, lane);
+    uint32_t below = 0;
+    for (uint32_t j = 0; j < n; ++j) below += __builtin_amdgcn_readlane(e, j) < e ? 1u : 0u;
+    if (lane >= n) below = lane;
+    return (uint32_t)__builtin_amdgcn_ds_permute((int)(below << 2), (int)e);
+}
+
+// out[r, :] = operand[r, :] + sum over the updates i in row r's bucket of updates[i, :]; one wave per row.
+// Measured on 262144 updates of 1 KB into 65536 rows: the launch moves its bytes at the same rate whether a
+// wave takes one row or several with all their loads in flight together, i.e. it is not bound by the chain
+// start -> order -> update rows; what helped is to keep the update rows (read once) and the result
+// (not read again here) out of the L2 with nontemporal accesses (65 -> 56 us).
 template <int VEC, bool IS_FLOAT>
 __device__ __forceinline__ void scatter_rows_sum_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ operand,
                                                       const uint32_t* __restrict__ updates, const uint32_t* __restrict__ start,
                                                       const uint32_t* __restrict__ order, const ScatterSortParams& P) {
-    constexpr int ROWS = SCATTER_ROWS_PER_WAVE;
+    constexpr uint32_t INFLIGHT = 4;
+    typedef uint32_t vec_t __attribute__((ext_vector_type(VEC)));
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t r0 = (blockIdx.x * 4u + (threadIdx.x >> 6)) * ROWS;
-    if (r0 >= P.n_rows) return;
-    auto add = [](uint32_t a, uint32_t b) -> uint32_t { return IS_FLOAT ? f2u(u2f(a) + u2f(b)) : a + b; };
-    // bucket boundaries: s[j] .. s[j + 1] for row r0 + j (rows beyond the table get empty buckets)
-    const uint32_t sv = start[min(r0 + lane, P.n_rows)];
-    uint32_t s[ROWS + 1];
+    const uint32_t row = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    if (row >= P.n_rows) return;
+    const uint32_t s = start[row], e = start[row + 1u];
+    auto add = [](vec_t a, vec_t b) -> vec_t {
+        if constexpr (IS_FLOAT) return __builtin_bit_cast(vec_t, __builtin_bit_cast(float __attribute__((ext_vector_type(VEC))), a) +
+                                                                  __builtin_bit_cast(float __attribute__((ext_vector_type(VEC))), b));
+        else return a + b;
+    };
+    // acc += updates[ent(k), c ...] for k < n in ascending k; ent: sorted update numbers, one per lane.
+    // Lanes beyond the row (live == false) ask for column 0 instead, whose values they drop.
+    auto accumulate = [&](uint32_t ent, uint32_t n, uint32_t c, vec_t& acc) {
+        for (uint32_t k = 0; k < n; k += INFLIGHT) {
+            vec_t t[INFLIGHT];
 #pragma unroll
-    for (int j = 0; j <= ROWS; ++j) s[j] = __builtin_amdgcn_readlane(sv, j);
-    const uint32_t total = s[ROWS] - s[0];
-
-    auto load_row = [&](const uint32_t* base, uint32_t row, uint32_t c, uint32_t (&dst)[VEC]) {
-        if constexpr (VEC == 4) {
-            const u32x4 t = *reinterpret_cast<const u32x4*>(base + (uint64_t)row * P.row_len + c);
-            dst[0] = t.x; dst[1] = t.y; dst[2] = t.z; dst[3] = t.w;
+            for (uint32_t q = 0; q < INFLIGHT; ++q) {                      // no branch around a load: the last one is repeated
+                const uint32_t u = __builtin_amdgcn_readlane(ent, min(k + q, n - 1u));
+                t[q] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(updates + (uint64_t)u * P.row_len + c));
+            }
+#pragma unroll
+            for (uint32_t q = 0; q < INFLIGHT; ++q)
+                if (k + q < n) acc = add(acc, t[q]);
+        }
+    };
+    const bool one_block = e - s <= 64u;
+    uint32_t ent = SCATTER_DROPPED;
+    if (one_block) {
+        if (lane < e - s) ent = order[s + lane];
+        ent = wave_sort_first(ent, e - s, lane);
+    }
+    for (uint32_t c0 = 0; c0 < P.row_len; c0 += 64u * VEC) {
+        const bool live = c0 + lane * VEC < P.row_len;                     // row_len is a multiple of VEC
+        const uint32_t c = live ? c0 + lane * VEC : 0u;
+        vec_t acc;
+        if (P.operand_is_scalar) acc = operand[0];
+        else acc = *reinterpret_cast<const vec_t*>(operand + (uint64_t)row * P.row_len + c);
+        if (one_block) {
+            accumulate(ent, e - s, c, acc);
         } else {
-            dst[0] = base[(uint64_t)row * P.row_len + c];
-        }
-    };
-    auto store_row = [&](uint32_t row, uint32_t c, const uint32_t (&src)[VEC]) {
-        if constexpr (VEC == 4) {
-            u32x4 t; t.x = src[0]; t.y = src[1]; t.z = src[2]; t.w = src[3];
-            *reinterpret_cast<u32x4*>(out + (uint64_t)row * P.row_len + c) = t;
-        } else {
-            out[(uint64_t)row * P.row_len + c] = src[0];
-        }
-    };
-    // acc += updates[e(k), c ...] for k in [k0, k1), four rows requested at a time and added in order;
-    // e holds the (sorted) update numbers, one per lane
-    auto accumulate = [&](uint32_t e, uint32_t k0, uint32_t k1, uint32_t c, bool live, uint32_t (&acc)[VEC]) {
-        for (uint32_t k = k0; k < k1; k += 4u) {
-            uint32_t t[4][VEC];
-#pragma unroll
-            for (uint32_t q = 0; q < 4u; ++q)
-                if (k + q < k1 && live) load_row(updates, __builtin_amdgcn_readlane(e, k + q) & 0x3FFFFFFFu, c, t[q]);
-#pragma unroll
-            for (uint32_t q = 0; q < 4u; ++q)
-                if (k + q < k1 && live) {
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) acc[v] = add(acc[v], t[q][v]);
-                }
-        }
-    };
-
-    if (total <= 64u) {
-        uint32_t e = 0xFFFFFFFFu;
-        if (lane < total) {
-            uint32_t row = 0;
-#pragma unroll
-            for (int j = 1; j < ROWS; ++j) row += lane >= s[j] - s[0] ? 1u : 0u;
-            e = order[s[0] + lane] | row << 30;
-        }
-        if (total > 1u) e = wave_sort(e, lane);
-        for (uint32_t c0 = 0; c0 < P.row_len; c0 += 64u * VEC) {
-            const uint32_t c = c0 + lane * VEC;
-            const bool live = c < P.row_len;                   // row_len is a multiple of VEC
-            uint32_t acc[ROWS][VEC];
-#pragma unroll
-            for (int j = 0; j < ROWS; ++j)
-                if (live && r0 + j < P.n_rows) load_row(operand, r0 + j, c, acc[j]);
-#pragma unroll
-            for (int j = 0; j < ROWS; ++j) accumulate(e, s[j] - s[0], s[j + 1] - s[0], c, live, acc[j]);
-#pragma unroll
-            for (int j = 0; j < ROWS; ++j)
-                if (live && r0 + j < P.n_rows) store_row(r0 + j, c, acc[j]);
-        }
-    } else {
-        for (uint32_t j = 0; j < (uint32_t)ROWS && r0 + j < P.n_rows; ++j) {
-            const uint32_t begin = __builtin_amdgcn_readlane(sv, j), end = __builtin_amdgcn_readlane(sv, j + 1);
-            for (uint32_t c0 = 0; c0 < P.row_len; c0 += 64u * VEC) {
-                const uint32_t c = c0 + lane * VEC;
-                const bool live = c < P.row_len;
-                uint32_t acc[VEC];
-                if (live) load_row(operand, r0 + j, c, acc);
-                for (uint32_t b0 = begin; b0 < end; b0 += 64u) {
-                    const uint32_t cnt = min(64u, end - b0);
-                    uint32_t e = lane < cnt ? order[b0 + lane] : 0xFFFFFFFFu;
-                    if (cnt > 1u) e = wave_sort(e, lane);
-                    accumulate(e, 0u, cnt, c, live, acc);
-                }
-                if (live) store_row(r0 + j, c, acc);
+            for (uint32_t b0 = s; b0 < e; b0 += 64u) {
+                const uint32_t n = min(64u, e - b0);
+                uint32_t block = lane < n ? order[b0 + lane] : SCATTER_DROPPED;
+                block = wave_sort_first(block, n, lane);
+                accumulate(block, n, c, acc);
             }
         }
+        if (live) __builtin_nontemporal_store(acc, reinterpret_cast<vec_t*>(out + (uint64_t)row * P.row_len + c));
     }
 }
 
@@ -304,188 +287,6 @@ SCATTER_SUM_KERNEL(scatter_rows_sum_f_v1, 1, true)
 SCATTER_SUM_KERNEL(scatter_rows_sum_f_v4, 4, true)
 SCATTER_SUM_KERNEL(scatter_rows_sum_i_v1, 1, false)
 SCATTER_SUM_KERNEL(scatter_rows_sum_i_v4, 4, false)
-
-// ---------------------------------------------------------------------------------------------
-// scatter-add of whole rows in ONE launch, no scratch memory, no atomics on the data ("owner
-// computes"): a workgroup owns `rows_per_group` consecutive table rows. It reads the whole index
-// array once (from L2: the array is a few hundred KB to a few MB and every workgroup reads it),
-// keeps the updates that fall into its rows as keys (row within the group << 22 | update number)
-// in LDS, sorts the keys, and then each wave adds up the updates of one row after the other, in
-// ascending update order, on top of the operand row (or of a single value, when the operand is a
-// constant filled with one value) and writes the result row once. Every update row is read exactly
-// once, the table is written once, and the result does not depend on thread timing.
-// A workgroup whose rows receive more keys than LDS holds works through the index array in
-// several rounds, each taking as many consecutive indices as fit, adding onto what it has written.
-// Needs n_idx <= 2^22 and rows_per_group <= 1024 (the host sees to that).
-struct ScatterOwnerParams { uint32_t n_idx, row_len, n_rows, idx_stride, rows_per_group, operand_is_scalar; };
-
-#define SCATTER_OWNER_CAP     4096u     // keys a workgroup holds in LDS
-#define SCATTER_OWNER_THREADS 1024u
-#define SCATTER_OWNER_INFLIGHT 8        // update rows a wave requests before it adds them
-
-template <int VEC, bool IS_FLOAT>
-__device__ __forceinline__ void scatter_rows_owner_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ operand,
-                                                        const uint32_t* __restrict__ updates, const int32_t* __restrict__ idx,
-                                                        const ScatterOwnerParams& P) {
-    __shared__ uint32_t keys[SCATTER_OWNER_CAP];
-    __shared__ uint32_t start[1024 + 1];
-    __shared__ uint32_t n_keys, n_tile;
-    constexpr uint32_t NT = SCATTER_OWNER_THREADS, NW = NT / 64u, CAP = SCATTER_OWNER_CAP;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t R0 = blockIdx.x * P.rows_per_group;
-    const uint32_t nrows = min(P.rows_per_group, P.n_rows - R0);           // the grid covers n_rows exactly
-    auto add = [](uint32_t a, uint32_t b) -> uint32_t { return IS_FLOAT ? f2u(u2f(a) + u2f(b)) : a + b; };
-    auto take = [&](int32_t r, uint32_t i) {                               // keeps update i if its row is one of ours
-        const uint32_t local = (uint32_t)r - R0;                           // negative and foreign rows wrap to >= nrows
-        if (local < nrows) {
-            const uint32_t p = atomicAdd(&n_keys, 1u);
-            if (p < CAP) keys[p] = local << 22 | i;
-        }
-    };
-
-    // keys[0 .. count) -> sorted; start[j] = first key of row j; then the sums.
-    // first: the rows start from the operand and every row is written; otherwise from what `out` holds, rows with keys only
-    auto process = [&](uint32_t count, bool first) {
-        uint32_t n = 64u;
-        while (n < count) n <<= 1;
-        for (uint32_t p = count + tid; p < n; p += NT) keys[p] = 0xFFFFFFFFu;
-        __syncthreads();
-        for (uint32_t k = 2u; k <= n; k <<= 1) {
-            for (uint32_t j = k >> 1; j > 0u; j >>= 1) {
-                for (uint32_t t = tid; t < (n >> 1); t += NT) {
-                    const uint32_t lo = ((t & ~(j - 1u)) << 1) | (t & (j - 1u)), hi = lo | j;
-                    const uint32_t a = keys[lo], b = keys[hi];
-                    if ((a > b) == ((lo & k) == 0u)) { keys[lo] = b; keys[hi] = a; }
-                }
-                __syncthreads();
-            }
-        }
-        for (uint32_t j = tid; j <= nrows; j += NT) {                      // lower bound of row j's first possible key
-            const uint32_t want = j << 22;
-            uint32_t lo = j < nrows ? 0u : count, hi = count;              // j == nrows: 1024 << 22 does not fit a word
-            while (lo < hi) {
-                const uint32_t mid = (lo + hi) >> 1;
-                if (keys[mid] < want) lo = mid + 1u; else hi = mid;
-            }
-            start[j] = lo;
-        }
-        __syncthreads();
-        for (uint32_t j = wave; j < nrows; j += NW) {
-            const uint32_t s = start[j], e = start[j + 1u];
-            if (!first && s == e) continue;
-            const uint64_t row = (uint64_t)(R0 + j) * P.row_len;
-            for (uint32_t c0 = 0u; c0 < P.row_len; c0 += 64u * VEC) {
-                const uint32_t c = c0 + lane * VEC;
-                if (c >= P.row_len) continue;                              // row_len is a multiple of VEC
-                uint32_t acc[VEC];
-                const uint32_t* base = first ? operand : out;
-                if (first && P.operand_is_scalar) {
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) acc[v] = operand[0];
-                } else if constexpr (VEC == 4) {
-                    const u32x4 t = *reinterpret_cast<const u32x4*>(base + row + c);
-                    acc[0] = t.x; acc[1] = t.y; acc[2] = t.z; acc[3] = t.w;
-                } else {
-                    acc[0] = base[row + c];
-                }
-                for (uint32_t k = s; k < e; k += SCATTER_OWNER_INFLIGHT) {
-                    uint32_t t[SCATTER_OWNER_INFLIGHT][VEC];
-#pragma unroll
-                    for (uint32_t q = 0; q < SCATTER_OWNER_INFLIGHT; ++q)
-                        if (k + q < e) {
-                            const uint64_t u = (uint64_t)(keys[k + q] & 0x3FFFFFu) * P.row_len + c;
-                            if constexpr (VEC == 4) {
-                                const u32x4 w = *reinterpret_cast<const u32x4*>(updates + u);
-                                t[q][0] = w.x; t[q][1] = w.y; t[q][2] = w.z; t[q][3] = w.w;
-                            } else {
-                                t[q][0] = updates[u];
-                            }
-                        }
-#pragma unroll
-                    for (uint32_t q = 0; q < SCATTER_OWNER_INFLIGHT; ++q)
-                        if (k + q < e) {
-#pragma unroll
-                            for (int v = 0; v < VEC; ++v) acc[v] = add(acc[v], t[q][v]);
-                        }
-                }
-                if constexpr (VEC == 4) {
-                    u32x4 t; t.x = acc[0]; t.y = acc[1]; t.z = acc[2]; t.w = acc[3];
-                    *reinterpret_cast<u32x4*>(out + row + c) = t;
-                } else {
-                    out[row + c] = acc[0];
-                }
-            }
-        }
-    };
-
-    if (tid == 0u) n_keys = 0u;
-    __syncthreads();
-    // the whole index array, four 16-byte loads per thread in flight where the indices are dense
-    if (P.idx_stride == 1u && (reinterpret_cast<uintptr_t>(idx) & 15u) == 0u) {
-        const uint32_t nvec = P.n_idx >> 2;
-        const int4* idx4 = reinterpret_cast<const int4*>(idx);
-        for (uint32_t v0 = tid; v0 < nvec; v0 += NT * 4u) {
-            int4 t[4];
-#pragma unroll
-            for (uint32_t q = 0; q < 4u; ++q)
-                if (v0 + q * NT < nvec) t[q] = idx4[v0 + q * NT];
-#pragma unroll
-            for (uint32_t q = 0; q < 4u; ++q)
-                if (v0 + q * NT < nvec) {
-                    const uint32_t i = (v0 + q * NT) << 2;
-                    take(t[q].x, i); take(t[q].y, i + 1u); take(t[q].z, i + 2u); take(t[q].w, i + 3u);
-                }
-        }
-        for (uint32_t i = (nvec << 2) + tid; i < P.n_idx; i += NT) take(idx[i], i);
-    } else {
-        for (uint32_t i = tid; i < P.n_idx; i += NT) take(idx[(uint64_t)i * P.idx_stride], i);
-    }
-    __syncthreads();
-    const uint32_t total = n_keys;
-    if (total <= CAP) {
-        process(total, true);
-        return;
-    }
-    // More keys than LDS holds: rounds over consecutive ranges of the index array. A round takes
-    // tiles of NT indices while their keys still fit (a tile never holds more than NT <= CAP keys,
-    // so every round advances), sums them, and the next round continues behind it.
-    uint32_t pos = 0u;
-    bool first = true;
-    while (pos < P.n_idx) {
-        __syncthreads();
-        if (tid == 0u) n_keys = 0u;
-        __syncthreads();
-        uint32_t count = 0u;
-        while (pos < P.n_idx) {
-            if (tid == 0u) n_tile = 0u;
-            __syncthreads();
-            const uint32_t i = pos + tid;
-            uint32_t local = 0xFFFFFFFFu;
-            if (i < P.n_idx) local = (uint32_t)idx[(uint64_t)i * P.idx_stride] - R0;
-            if (local < nrows) atomicAdd(&n_tile, 1u);
-            __syncthreads();
-            if (count + n_tile > CAP) break;                               // uniform: every thread reads the same two values
-            if (local < nrows) keys[atomicAdd(&n_keys, 1u)] = local << 22 | i;
-            count += n_tile;
-            pos += NT;
-            __syncthreads();                                               // n_tile is reset by the next tile
-        }
-        __syncthreads();
-        process(count, first);
-        first = false;
-    }
-}
-
-#define SCATTER_OWNER_KERNEL(name, VEC, IS_FLOAT)                                                                  \
-    extern "C" __global__ __launch_bounds__(SCATTER_OWNER_THREADS) void name(uint32_t* out, const uint32_t* operand, \
-            const uint32_t* updates, const int32_t* idx, ScatterOwnerParams P) {                                   \
-        scatter_rows_owner_body<VEC, IS_FLOAT>(out, operand, updates, idx, P);                                     \
-    }
-// the _v4 variants require row_len % 4 == 0 and 16-byte aligned data pointers
-SCATTER_OWNER_KERNEL(scatter_rows_owner_f_v1, 1, true)
-SCATTER_OWNER_KERNEL(scatter_rows_owner_f_v4, 4, true)
-SCATTER_OWNER_KERNEL(scatter_rows_owner_i_v1, 1, false)
-SCATTER_OWNER_KERNEL(scatter_rows_owner_i_v4, 4, false)
 
 struct ScatterGeneralParams {
     uint32_t n_upd, upd_rank, op_rank, n_index, is_float;

@@ -811,49 +811,30 @@ def scatter_add_rows(out: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_
                   bytes_moved=4 * (total + n_idx + out.size))
 
 
-def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, counters: Buffer, order: Buffer,
-                            n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1) -> tp.List[Launch]:
-    '''out = operand; out[idx[i], :] += updates[i, :] without atomics on the data: a counting sort of the
-    indices (`counters`: 2 * (n_rows + 1) words, `order`: n_idx words), then one wave per row sums its bucket.'''
-    assert counters.size == 2 * (n_rows + 1) and order.size == n_idx
-    params = _u32(n_idx, row_len, n_rows, idx_stride)
-    cursor = (n_rows + 1) * 4                       #byte offset of the second half of `counters`
+def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, count: Buffer, start: Buffer, rank: Buffer,
+                            order: Buffer, n_idx: int, row_len: int, n_rows: int, operand_is_scalar: bool = False,
+                            idx_stride: int = 1) -> tp.List[Launch]:
+    '''out = operand; out[idx[i], :] += updates[i, :] without atomics on the data: a counting sort of the indices
+    (`count`: n_rows words that are zero before and after, `start`: n_rows + 1 words, `rank` and `order`: n_idx words
+    each), then one wave per row sums its bucket. `operand` is the table, or one word when the table is a constant
+    filled with a single value.'''
+    assert count.size == n_rows and start.size == n_rows + 1 and rank.size == n_idx and order.size == n_idx
+    params = _u32(n_idx, row_len, n_rows, idx_stride, int(operand_is_scalar))
     vec    = 4 if row_len % 4 == 0 else 1
     kind   = 'f' if out.dtype == np.float32 else 'i'
-    return [
-        fill(counters, 0),
-        Launch('scatter_rows_count', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(counters, 0), (idx, 0)], params, bytes_moved=8 * n_idx),
-        Launch('scatter_rows_scan', (1, 1, 1), (1024, 1, 1), [(counters, 0)], _u32(n_rows + 1), bytes_moved=8 * (n_rows + 1)),
-        Launch('scatter_rows_fill', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(order, 0), (counters, cursor), (counters, 0), (idx, 0)], params,
-               bytes_moved=16 * n_idx),
-        Launch(f'scatter_rows_sum_{kind}_v{vec}', (_cdiv(n_rows, 16), 1, 1), (BLOCK, 1, 1),     #4 waves x 4 rows per block
-               [(out, 0), (operand, 0), (updates, 0), (counters, 0), (order, 0)], params,
-               bytes_moved=4 * (n_idx * row_len + n_idx + 2 * n_rows * row_len)),
-    ]
-
-
-SCATTER_OWNER_CAP     = 4096          #keys a workgroup of scatter_rows_owner holds in LDS
-SCATTER_OWNER_MAX_IDX = 1 << 22       #update numbers take 22 bits of a key
-SCATTER_OWNER_GROUPS  = 256           #workgroups aimed at: one per compute unit
-
-
-def scatter_add_rows_owner(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_len: int, n_rows: int,
-                           operand_is_scalar: bool = False, idx_stride: int = 1) -> Launch:
-    '''out = operand; out[idx[i], :] += updates[i, :] in one launch: every workgroup owns a range of table rows, picks
-    its updates out of the whole index array and sums them in ascending update order. `operand` is the table, or one
-    word when the table is a constant filled with a single value.'''
-    assert n_idx <= SCATTER_OWNER_MAX_IDX
-    #one workgroup per compute unit where possible (each reads the whole index array), but no more rows per
-    #workgroup than are expected to fill half its key storage, and at most 1024 (10 bits of a key)
-    rows = max(_cdiv(n_rows, SCATTER_OWNER_GROUPS), 1)
-    rows = min(rows, max(n_rows * (SCATTER_OWNER_CAP // 2) // max(n_idx, 1), 1), 1024)
-    vec  = 4 if row_len % 4 == 0 else 1
-    kind = 'f' if out.dtype == np.float32 else 'i'
+    #bucket starts: at most 256 workgroups, each scanning a segment of whole 1024-word tiles
+    seg    = 1024 * _cdiv(_cdiv(n_rows + 1, 1024), 256)
     table_passes = 1 if operand_is_scalar else 2
-    return Launch(f'scatter_rows_owner_{kind}_v{vec}', (_cdiv(n_rows, rows), 1, 1), (1024, 1, 1),
-                  [(out, 0), (operand, 0), (updates, 0), (idx, 0)],
-                  _u32(n_idx, row_len, n_rows, idx_stride, rows, int(operand_is_scalar)),
-                  bytes_moved=4 * (n_idx * row_len + n_idx + table_passes * n_rows * row_len))
+    return [
+        Launch('scatter_rows_rank', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(count, 0), (rank, 0), (idx, 0)], params, bytes_moved=12 * n_idx),
+        Launch('scatter_rows_starts', (_cdiv(n_rows + 1, seg), 1, 1), (1024, 1, 1), [(start, 0), (count, 0)], _u32(n_rows, seg),
+               bytes_moved=8 * (n_rows + 1)),
+        Launch('scatter_rows_order', (_cdiv(max(n_idx, n_rows), BLOCK), 1, 1), (BLOCK, 1, 1),
+               [(order, 0), (count, 0), (start, 0), (rank, 0), (idx, 0)], params, bytes_moved=16 * n_idx + 4 * n_rows),
+        Launch(f'scatter_rows_sum_{kind}_v{vec}', (_cdiv(n_rows, 4), 1, 1), (BLOCK, 1, 1),      #one wave per row
+               [(out, 0), (operand, 0), (updates, 0), (start, 0), (order, 0)], params,
+               bytes_moved=4 * (n_idx * row_len + n_idx + table_passes * n_rows * row_len)),
+    ]
 
 
 def scatter_add_general(out: Buffer, indices: Buffer, updates: Buffer, update_window_dims, inserted_window_dims,

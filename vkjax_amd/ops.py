@@ -867,10 +867,14 @@ def scatter_add(bufferpool, equation):
         row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
         n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
         n_rows  = operand.shape[0]
-        if n_idx * row_len >= SCATTER_SORT_THRESHOLD and n_idx <= SCATTER_OWNER_MAX_IDX and n_rows < 2**31 - 1:
-            #large: every workgroup owns a range of table rows and sums the updates that fall into it, one launch
-            #(no atomics on the data, no copy of the operand, no scratch arrays)
-            bufferpool.op_counter = counter_before + 1
+        if n_idx * row_len >= SCATTER_SORT_THRESHOLD and n_idx < 2**31 - 1 and n_rows < 2**31 - 1:
+            #large: bucket the updates by row and sum each bucket (no atomics on the data, no copy of the operand)
+            bufferpool.op_counter = counter_before
+            count = bufferpool.zeroed_scratch(n_rows)          #every evaluation leaves it zero again
+            count.accesses.append(counter_before)
+            start = bufferpool.new_temporary(np.dtype('uint32'), (n_rows + 1,))
+            rank  = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
+            order = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
             uniform = _uniform_constant(operand)
             if uniform is not None:
                 #a table that is a constant filled with one value (zeros, usually) is not read at all
@@ -878,25 +882,17 @@ def scatter_add(bufferpool, equation):
                 source.accesses.append(counter_before)
             else:
                 source = operand
-            return [Op(equation, launch=K.scatter_add_rows_owner(outbuf, source, indices, updates, n_idx, row_len, n_rows,
-                                                                 operand_is_scalar=uniform is not None))]
-        if n_idx * row_len >= SCATTER_SORT_THRESHOLD and n_idx < 2**30 and n_rows < 2**31 - 1:
-            #large: bucket the updates by row and sum each bucket (no atomics on the data, no copy of the operand)
-            bufferpool.op_counter = counter_before
-            counters = bufferpool.new_temporary(np.dtype('uint32'), (2 * (n_rows + 1),))
-            order    = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
             bufferpool.op_counter = counter_before + 1
-            launches = K.scatter_add_rows_sorted(outbuf, operand, indices, updates, counters, order, n_idx, row_len, n_rows)
+            launches = K.scatter_add_rows_sorted(outbuf, source, indices, updates, count, start, rank, order, n_idx, row_len, n_rows,
+                                                 operand_is_scalar=uniform is not None)
             return [Op(equation, launch=l) for l in launches]
         ops = [copy, Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, n_rows))]
         return ops
     return [copy, Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od))]
 
 
-#scatter-add of rows: from this many update elements on, the atomic-free kernels are used: the single-launch
-#one for up to SCATTER_OWNER_MAX_IDX updates, beyond that the counting sort with its scratch arrays
+#scatter-add of rows: from this many update elements on, the sorted (atomic-free) kernels are used
 SCATTER_SORT_THRESHOLD = 1 << 18
-SCATTER_OWNER_MAX_IDX  = K.SCATTER_OWNER_MAX_IDX
 
 
 def _uniform_constant(b):
