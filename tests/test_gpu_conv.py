@@ -210,6 +210,61 @@ def test_four_waves_per_tile_kernel():
         K.FORCE_CONV_KSPLIT = None
 
 
+def test_mixed_tiling_and_two_group_kernels():
+    '''Layers whose 64 x 64 tiles do not divide evenly among the CUs: the first M tiles as 64 x 64 tiles, the rows
+    behind them as 32 x 32 tiles computed by four waves each, in one launch (conv_gemm_64x64x{32,64}_mix); and the
+    64 x 64 tile whose k steps two groups of waves share (conv_gemm_64x64x{64,128}_ks2). Padded 3x3, strided and
+    1x1 convolutions and a plain product, with a batch-norm + residual + ReLU epilogue, bias + ReLU and none; splits
+    that leave one small tile row, several, a last tile that is not full in either direction; integer-valued data,
+    so every result is exact.'''
+    from vkjax_amd import kernels as K
+    from vkjax_amd import minijax as mj
+    lax, nn, jnp = mj.lax, mj.nn, mj.numpy
+    dn = ('NHWC', 'HWIO', 'NHWC')
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+
+    def bn_res_relu(stride):
+        def f(x, k, mean, scale, beta, res):
+            y = lax.conv_general_dilated(x, k, (stride, stride), 'SAME', dimension_numbers=dn)
+            return nn.relu((y - mean) * scale + beta + res)
+        return f
+    def dense(x, w, b): return nn.relu(jnp.dot(x, w) + b)
+
+    def conv_case(batch, h, w, ksize, cin, cout, stride=1):
+        ho, wo = -(-h // stride), -(-w // stride)
+        return (bn_res_relu(stride), [ints(-4, 5, batch, h, w, cin), ints(-3, 4, ksize, ksize, cin, cout), ints(-5, 5, cout), ints(1, 4, cout),
+                                      ints(-9, 9, cout), ints(-50, 50, batch, ho, wo, cout)])
+    cases = [conv_case(3, 13, 11, 3, 64, 72), conv_case(2, 14, 14, 3, 128, 256), conv_case(5, 7, 7, 1, 256, 100),
+             conv_case(3, 14, 14, 3, 64, 64, stride=2), (conv2, [ints(-4, 5, 2, 20, 17, 64), ints(-3, 4, 3, 3, 64, 40)]),
+             (dense, [ints(-4, 5, 300, 328), ints(-3, 4, 328, 136), ints(-9, 9, 136)])]
+    try:
+        for f, args in cases:
+            for bk in (32, 64):
+                K.FORCE_CONV_TILE, K.FORCE_CONV_BK, K.FORCE_CONV_CHUNK, K.FORCE_CONV_KSPLIT = '64x64', bk, 1, False
+                try:
+                    for split in (1, 2, 5):
+                        K.FORCE_CONV_MIX = split
+                        print(f'mixed tiling: {f.__name__} {[a.shape for a in args]} bk {bk}, {split} M tiles of 64 rows', flush=True)
+                        _, _, fn = check_against_oracle(f, args, exact=True)
+                        launches = list(fn._jaxpr_interpreters.values())[0].launches
+                        m = launches[0].flops // (2 * int(np.prod(args[1].shape[:-1])) * args[1].shape[-1])
+                        expected = f'conv_gemm_64x64x{bk}_mix' if split * 64 < m else f'conv_gemm_64x64x{bk}_lean'
+                        assert [l.kernel for l in launches] == [expected], ([l.kernel for l in launches], m)
+                finally:
+                    K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = K.FORCE_CONV_KSPLIT = K.FORCE_CONV_MIX = None
+            for variant in ('64x64x64_ks2', '64x64x128_ks2'):
+                K.FORCE_CONV_KSPLIT = variant
+                print(f'two groups of waves: {f.__name__} {[a.shape for a in args]} {variant}', flush=True)
+                _, _, fn = check_against_oracle(f, args, exact=True)
+                launches = list(fn._jaxpr_interpreters.values())[0].launches
+                bk = int(variant.split('x')[2].split('_')[0])
+                eligible = args[1].shape[-2] % bk == 0 or args[1].ndim == 2 or args[1].shape[0] == 1
+                assert [l.kernel for l in launches] == [f'conv_gemm_{variant}' if eligible else launches[0].kernel], [l.kernel for l in launches]
+                K.FORCE_CONV_KSPLIT = None
+    finally:
+        K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = K.FORCE_CONV_KSPLIT = K.FORCE_CONV_MIX = None
+
+
 def test_convolution_with_a_second_result():
     '''A convolution result that is returned (or read later) AND continued by an element-wise chain: one launch
     stores both, the value before the chain or after its `- vector` step and the chain's result. Integer-valued

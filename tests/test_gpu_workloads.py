@@ -55,16 +55,20 @@ def test_resnet50_batch64_against_its_own_batch_of_two():
     depend on the batch size: an image's logits do not depend on its neighbours, so (1) the first two rows equal
     a batch-of-two evaluation of the same images (which the test above pins to the oracle) within the logits'
     tolerance (the two sizes use different tiles and k splits, so not bit for bit), (2) copies of an image placed
-    elsewhere in the batch give the same bits, and (3) every label is the index of its row's largest logit.'''
+    elsewhere in the batch give the same bits where the same tiling computes them (the last images of the batch
+    fall into the rows that the layers with few tiles compute as 32 x 32 tiles with a four-way k split: the same
+    values within the tolerance of a sum taken in another order), and (3) every label is the index of its row's
+    largest logit.'''
     params, x = W.resnet50_inputs(batch=64, size=224)
     x = x.copy()
-    x[63], x[32] = x[0], x[1]
+    x[63], x[32], x[20] = x[0], x[1], x[0]
     logits, labels = vkjax_amd.wrap(W.resnet50, frontend='minijax')(params, x)
     logits2, labels2 = vkjax_amd.wrap(W.resnet50, frontend='minijax')(params, x[:2].copy())
     assert logits.shape == (64, 1000) and np.all(np.isfinite(logits))
     scale = float(np.abs(logits2).max())
     assert np.allclose(logits[:2], logits2, rtol=1e-3, atol=1e-5 * scale), float(np.abs(logits[:2] - logits2).max())
-    assert np.array_equal(logits[63], logits[0]) and np.array_equal(logits[32], logits[1])
+    assert np.array_equal(logits[20], logits[0]) and np.array_equal(logits[32], logits[1])
+    assert np.allclose(logits[63], logits[0], rtol=1e-4, atol=1e-5 * scale), float(np.abs(logits[63] - logits[0]).max())
     assert np.array_equal(labels, np.argmax(logits, axis=1).astype(labels.dtype))
     assert np.array_equal(labels[:2], labels2)
 

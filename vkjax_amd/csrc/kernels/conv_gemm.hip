@@ -73,7 +73,17 @@ struct ConvParams {
     int32_t LH, LW, xs_c;           // lhs dilation and feature stride
     int32_t ws_r, ws_s, ws_c, ws_n; // rhs strides
     int32_t os_b, os_h, os_w, os_n; // out strides
+    int32_t split_tiles_m;          // mixed kernels only: the first split_tiles_m M tiles (of 64 rows) are computed as 64 x 64
+                                    // tiles, the rows behind them as 32 x 32 tiles by the blocks that follow in the grid
 };
+
+// The part of the output a block's tile number refers to: a grid of tiles_m x tiles_n tiles whose first row is
+// m_base, handed to the blocks from first_block on.
+struct ConvRegion { int first_block, tiles_m, tiles_n, m_base; };
+
+// LDS of one block: A tile, B tile, per-column epilogue operands, row offsets (floats)
+template <int WGM, int WGN, int TM, int TN, int BK>
+constexpr int conv_pool_floats() { return 32 * WGM * TM * (BK + 4) + BK * (32 * WGN * TN + 4) + CONV_MAX_EPI * 32 * WGN * TN + 32 * WGM * TM; }
 
 struct ConvEpiPtrs { const float* p[CONV_MAX_EPI]; };
 
@@ -104,7 +114,7 @@ struct ConvDerived {
 // path, k tiles that never straddle kernel taps, a row-major result, an epilogue that fits the
 // straight-line template.
 template <int WGM, int WGN, int TM, int TN, int BK, bool A_FAST, bool B_FAST, bool LEAN, int KSW = 1>
-__device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const float* __restrict__ x,
+__device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const ConvRegion region, float* __restrict__ out, const float* __restrict__ x,
                                                const float* __restrict__ w, const ConvEpiPtrs& epi,
                                                const ConvDerivedPtrs& Dp, const ConvParams& Pk, const ConvDerived& Dk) {
     // KSW > 1: KSW groups of WGM x WGN waves share one block tile, each taking a 1/KSW slice of every k
@@ -113,10 +123,11 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     static_assert(KSW == 1 || (LEAN && TM == 1 && TN == 1), "k-split blocks exist for the lean single-tile form only");
     constexpr int BM = 32 * WGM * TM, BN = 32 * WGN * TN, NT = 64 * WGM * WGN * KSW;
     constexpr int LDA = BK + 4, LDB = BN + 4;
-    __shared__ __attribute__((aligned(16))) float As[BM * LDA];
-    __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
-    __shared__ float Es[CONV_MAX_EPI * BN];         // per-column operands of the epilogue steps
-    __shared__ int   Rs[BM];                        // row offsets of outputs that are not row-major
+    static_assert((BM * LDA) % 4 == 0 && (BK * LDB) % 4 == 0, "16-byte alignment of the LDS tiles");
+    float* const As = pool;                         // [BM][LDA]
+    float* const Bs = As + BM * LDA;                // [BK][LDB]
+    float* const Es = Bs + BK * LDB;                // [CONV_MAX_EPI][BN]: per-column operands of the epilogue steps
+    int*   const Rs = reinterpret_cast<int*>(Es + CONV_MAX_EPI * BN);   // [BM]: row offsets of outputs that are not row-major
 #ifdef CONV_PHASE_STAMPS
     unsigned long long stamps[16] = {};
 #endif
@@ -154,14 +165,14 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     // Consecutive block ids go to different XCDs (8 of them, each with its own L2). Hand every
     // XCD a contiguous range of work so that the N-tiles of one M-tile share an L2.
     const int chunk = LEAN ? (P.flags >> 25) & 15u : 1;         // the general variants take one tile per block
-    const int chunks_m = (P.tiles_m + chunk - 1) / chunk;
-    int work = blockIdx.x;
+    const int chunks_m = (region.tiles_m + chunk - 1) / chunk;
+    int work = (int)blockIdx.x - region.first_block;
     {
-        const int total = chunks_m * P.tiles_n, per = total / 8;
+        const int total = chunks_m * region.tiles_n, per = total / 8;
         if (per > 0 && work < per * 8) work = (work & 7) * per + (work >> 3);
     }
-    const int chunk_m = work / P.tiles_n, tile_n = work - chunk_m * P.tiles_n;
-    const int tile_m0 = chunk_m * chunk, nsub = LEAN ? min(chunk, P.tiles_m - tile_m0) : 1;
+    const int chunk_m = work / region.tiles_n, tile_n = work - chunk_m * region.tiles_n;
+    const int tile_m0 = chunk_m * chunk, nsub = LEAN ? min(chunk, region.tiles_m - tile_m0) : 1;
     const int n0 = tile_n * BN;
     const int HoWo = P.Ho * P.Wo;
 
@@ -435,7 +446,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
     // K = 0 runs as one k step whose loads are all out of range
     const int ktiles = max(1, (P.K + BK - 1) / BK);
-    setup_rows(tile_m0 * BM);
+    setup_rows(region.m_base + tile_m0 * BM);
     CONV_STAMP(1)
     load_tiles(0);
     if (tid < BN) {
@@ -477,7 +488,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     };
 
     for (int sub = 0; sub < nsub; ++sub) {
-        const int m0 = (tile_m0 + sub) * BM;
+        const int m0 = region.m_base + (tile_m0 + sub) * BM;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -537,8 +548,8 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
 #pragma unroll
                 for (int v = 0; v < 16; ++v) c[i][j][v] = acc[i][j][v];
         if constexpr (KSW > 1) {
-            // the k slices meet in the first group of waves (the A tile's LDS space is free after the last step)
-            static_assert((KSW - 1) * WGM * WGN * 16 * 64 <= BM * LDA, "reduction buffer does not fit the A tile");
+            // the k slices meet in the first group of waves (the LDS space of the A and B tiles is free after the last step)
+            static_assert((KSW - 1) * WGM * WGN * 16 * 64 <= BM * LDA + BK * LDB, "reduction buffer does not fit the A and B tiles (B follows A)");
             float* red = As + ((kw - 1) * WGM * WGN + wm * WGN + wn) * 16 * 64 + lane;
             if (kw > 0) {
 #pragma unroll
@@ -695,7 +706,9 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ out, const fl
     extern "C" __global__ __launch_bounds__(64 * WGM * WGN * (1, ##__VA_ARGS__)) __attribute__((amdgpu_waves_per_eu(2))) void name( \
         float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
         ConvEpiPtrs epi, ConvDerivedPtrs dp, ConvParams P, ConvDerived D) {                                  \
-        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF, LEAN, ##__VA_ARGS__>(out, x, w, epi, dp, P, D);         \
+        __shared__ __attribute__((aligned(16))) float pool[conv_pool_floats<WGM, WGN, TM, TN, BK>()];        \
+        const ConvRegion all{0, P.tiles_m, P.tiles_n, 0};                                                    \
+        conv_gemm_body<WGM, WGN, TM, TN, BK, AF, BF, LEAN, ##__VA_ARGS__>(pool, all, out, x, w, epi, dp, P, D); \
     }
 
 // name = conv_gemm_<BM>x<BN>x<BK>_<a><b>  with a/b = f (16-byte loads) or g (generic strided loads),
@@ -717,3 +730,33 @@ CONV_TILE(32x32x64, 1, 1, 1, 1, 64)
 CONV_KERNEL(conv_gemm_32x32x128_ks4, 1, 1, 1, 1, 128, true, true, true, 4)
 // the same with element-wise loads of the kernel operand (an output width that is no multiple of 4)
 CONV_KERNEL(conv_gemm_32x32x128_ks4g, 1, 1, 1, 1, 128, true, false, true, 4)
+// one 64 x 64 tile per block, every k step shared by two groups of 2 x 2 waves: twice the resident waves for
+// layers whose few hundred tiles leave a CU with three or fewer blocks
+CONV_KERNEL(conv_gemm_64x64x64_ks2, 2, 2, 1, 1, 64, true, true, true, 2)
+CONV_KERNEL(conv_gemm_64x64x128_ks2, 2, 2, 1, 1, 128, true, true, true, 2)
+
+// Mixed tiling for layers whose 64 x 64 tiles do not divide evenly among the CUs (784 tiles on 256 CUs: a CU
+// with four tiles sets the time, the average is 3.06). The first P.split_tiles_m M tiles are computed as 64 x 64
+// tiles, as many as fill every CU equally; the rows behind them as 32 x 32 tiles of a quarter of the work each
+// (four waves sharing every 64-long k step), which spread over the CUs in finer units. Both kinds of block have 256
+// threads and share one LDS pool; with the 64-long step the kernel needs 127 registers, so four blocks fit a CU
+// (the 128-long step of conv_gemm_32x32x128_ks4 takes 149: three blocks, and the small tiles would wait for
+// the large ones). One M tile per block (chunk 1).
+#define CONV_MIX_KERNEL(name, BK)                                                                              \
+    extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void name(            \
+        float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,                   \
+        ConvEpiPtrs epi, ConvDerivedPtrs dp, ConvParams P, ConvDerived D) {                                  \
+        constexpr int big = conv_pool_floats<2, 2, 1, 1, BK>(), small = conv_pool_floats<1, 1, 1, 1, 64>(); \
+        __shared__ __attribute__((aligned(16))) float pool[big > small ? big : small];                       \
+        const int n_big = P.split_tiles_m * P.tiles_n;                                                       \
+        if ((int)blockIdx.x < n_big) {                                                                       \
+            const ConvRegion r{0, P.split_tiles_m, P.tiles_n, 0};                                            \
+            conv_gemm_body<2, 2, 1, 1, BK, true, true, true>(pool, r, out, x, w, epi, dp, P, D);             \
+        } else {                                                                                             \
+            const int m_base = P.split_tiles_m * 64;                                                         \
+            const ConvRegion r{n_big, (P.M - m_base + 31) / 32, (P.N + 31) / 32, m_base};                    \
+            conv_gemm_body<1, 1, 1, 1, 64, true, true, true, 4>(pool, r, out, x, w, epi, dp, P, D);         \
+        }                                                                                                    \
+    }
+CONV_MIX_KERNEL(conv_gemm_64x64x32_mix, 32)
+CONV_MIX_KERNEL(conv_gemm_64x64x64_mix, 64)

@@ -426,6 +426,7 @@ FORCE_CONV_BK:   tp.Optional[int] = None
 FORCE_CONV_CHUNK: tp.Optional[int] = None
 FORCE_CONV_GENERAL = False          #never pick the lean kernel variant
 FORCE_CONV_KSPLIT: tp.Optional[bool] = None    #the four-waves-per-tile kernel: always (where it applies) / never
+FORCE_CONV_MIX = None               #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
 
 
 def choose_conv_tile(M: int, N: int, compute_units: int = 256):
@@ -443,6 +444,18 @@ def choose_conv_tile(M: int, N: int, compute_units: int = 256):
         if best_time is None or time < best_time:
             best, best_time = (tag, bm, bn, nt), time
     return best
+
+
+def choose_conv_split(tiles_m: int, tiles_n: int, compute_units: int = 256) -> int:
+    '''How many M tiles of a layer stay 64 x 64 tiles when the rest is computed as 32 x 32 tiles (0: no split).
+    tiles / CUs = 3.06 means that some CUs work on four tiles while most have three; the whole rounds keep their
+    64 x 64 tiles and the remainder is spread in quarter-size units. Not worth it once a CU has six tiles or more,
+    or when the last round is nearly full anyway.'''
+    rounds = tiles_m * tiles_n / compute_units
+    whole  = int(rounds)
+    if whole < 1 or rounds >= 6 or rounds - whole == 0 or rounds - whole > 0.7:
+        return 0
+    return (whole * compute_units) // tiles_n
 
 
 def choose_conv_chunk(tiles_m: int, tiles_n: int, compute_units: int = 256) -> int:
@@ -550,12 +563,25 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     #tile, each taking a quarter of every (128-long) k step
     ksplit = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
               (_cdiv(M, 32) * _cdiv(N, 32) <= 2 * compute_units and K >= 256 and FORCE_CONV_TILE is None and FORCE_CONV_BK is None))
-    ksplit = bool(ksplit) and a_fast and c_contig and (g.Cin % 128 == 0 or g.KH * g.KW == 1) \
-        and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL
+    ks_variant = ksplit if isinstance(ksplit, str) else '32x32x128_ks4'
+    ks_tag, ks_bk, ks_w = ks_variant.rsplit('x', 1)[0], int(ks_variant.rsplit('x', 1)[1].split('_')[0]), int(ks_variant[-1])
+    ksplit = bool(ksplit) and a_fast and c_contig and (g.Cin % ks_bk == 0 or g.KH * g.KW == 1) \
+        and (b_fast or ks_tag == '32x32') and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL
     if ksplit:
-        tag, bm, bn, nt, bk, lean = '32x32', 32, 32, 256, 128, True
+        side = int(ks_tag.split('x')[0])
+        tag, bm, bn, nt, bk, lean = ks_tag, side, side, (side // 32) ** 2 * 64 * ks_w, ks_bk, True
     tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
     chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean and not ksplit else 1
+    #64 x 64 tiles that do not divide evenly among the CUs: as many M tiles as fill every CU equally stay 64 x 64, the
+    #rows behind them are computed as 32 x 32 tiles with four waves per tile (a quarter of the work each)
+    split_tiles_m = 0
+    mixable = (lean and not ksplit and tag == '64x64' and chunk == 1 and b_fast and (g.Cin % 64 == 0 or g.KH * g.KW == 1) and K >= 256)
+    if mixable and FORCE_CONV_MIX is not None and FORCE_CONV_MIX is not False:
+        split_tiles_m = int(FORCE_CONV_MIX)                      #tests: whatever the other FORCE_ settings are
+    elif mixable and FORCE_CONV_MIX is None and FORCE_CONV_TILE is None and FORCE_CONV_BK is None and FORCE_CONV_CHUNK is None:
+        split_tiles_m = choose_conv_split(tiles_m, tiles_n, compute_units)
+    if split_tiles_m >= tiles_m:
+        split_tiles_m = 0
     kinds = [e.kind for e in epilogue]
     x_bytes = (lhs.size - lhs_offset) * 4
     w_bytes = K * N * 4 if b_fast else (rhs.size - rhs_offset) * 4
@@ -569,7 +595,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW,
                    *g.xs[:3], tiles_m, tiles_n)
               + _u32(flags, *descs, x_bytes, w_bytes, (out.size - out_offset) * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
-              + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os))
+              + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os, split_tiles_m))
     derived_ptrs, derived_desc = [(None, 0)] * (CONV_MAX_DERIVED + 1), _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
     for i, e in enumerate(epilogue):
         if e.derived is not None:
@@ -588,11 +614,14 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
         assert operand_slots[-1] == (None, 0)
         operand_slots[-1] = (tap_buffer, 0)
     buffers += operand_slots + derived_ptrs
-    kernel  = f'conv_gemm_{tag}x{bk}_' + (('ks4' if b_fast else 'ks4g') if ksplit else 'lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
+    kernel  = f'conv_gemm_{tag}x{bk}_' + ((f'ks{ks_w}' if b_fast else f'ks{ks_w}g') if ksplit else 'lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
     nbytes += 4 * tap_buffer.size if taps else 0
-    return Launch(kernel, (_cdiv(tiles_m, chunk) * tiles_n, 1, 1), (nt, 1, 1), buffers, params,
-                  bytes_moved=nbytes, flops=2 * M * N * K)
+    blocks = _cdiv(tiles_m, chunk) * tiles_n
+    if split_tiles_m:
+        kernel = f'conv_gemm_{tag}x{bk}_mix'
+        blocks = split_tiles_m * tiles_n + _cdiv(M - split_tiles_m * 64, 32) * _cdiv(N, 32)
+    return Launch(kernel, (blocks, 1, 1), (nt, 1, 1), buffers, params, bytes_moved=nbytes, flops=2 * M * N * K)
 
 
 # --------------------------------------------------------------------------- reductions
