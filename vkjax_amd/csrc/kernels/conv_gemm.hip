@@ -157,6 +157,20 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kw = wave / (WGM * WGN), wm = (wave % (WGM * WGN)) / WGN, wn = wave % WGN;
     const int l32 = lane & 31, half = lane >> 5;
+    // A single 32 x 32 tile whose k steps are shared by KSW waves: every wave loads, parks in LDS and consumes its
+    // own slice of a k step, so the k loop needs no barrier between the waves; they drift apart and one wave's
+    // MFMAs cover the others' load latencies (a block of these kernels is usually alone on its CU).
+    constexpr bool WAVE_PRIVATE = KSW > 1 && WGM == 1 && WGN == 1 && A_FAST;
+    constexpr int  BKW_ = BK / KSW;
+    // thread -> (row within a pass, 16-byte vector within the row) of the A tile, (k row, vector) of the B tile
+    const int a_r0 = WAVE_PRIVATE ? lane / (BKW_ / 4) : tid / (BK / 4);
+    const int a_kv = WAVE_PRIVATE ? kw * (BKW_ / 4) + lane % (BKW_ / 4) : tid % (BK / 4);
+    const int b_r0 = WAVE_PRIVATE ? kw * BKW_ + lane / (BN / 4) : tid / (BN / 4);
+    const int b_nv = WAVE_PRIVATE ? lane % (BN / 4) : tid % (BN / 4);
+    auto tile_barrier = [&]() {
+        if constexpr (WAVE_PRIVATE) __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // LDS accesses of a wave execute in order
+        else __syncthreads();
+    };
 
     // A block works through up to `chunk` consecutive M tiles of one N tile, one after the other,
     // as one flat sequence of k steps: while a step is computed the loads of the next one are in
@@ -243,7 +257,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     // ---------------- per-thread load assignment ----------------
     // A fast: 16-byte vectors along k. A generic: one row, a run of consecutive k.
     constexpr int A_VPR   = BK / 4;                 // vectors per row
-    constexpr int A_RSTEP = NT / A_VPR;             // rows between a thread's vectors
+    constexpr int A_RSTEP = WAVE_PRIVATE ? 64 / (BKW_ / 4) : NT / A_VPR;   // rows between a thread's vectors
     constexpr int A_NV    = BM / A_RSTEP;           // vectors per thread
     constexpr int A_KG    = NT / BM;                // generic: k groups
     constexpr int A_KPT   = BK / A_KG;              // generic: k per thread
@@ -264,10 +278,10 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     auto setup_rows = [&](int m0) {
 #pragma unroll
         for (int p = 0; p < A_ROWS; ++p) {
-            const int row = A_FAST ? (tid / A_VPR + p * A_RSTEP) : (tid % BM);
+            const int row = A_FAST ? (a_r0 + p * A_RSTEP) : (tid % BM);
             const int m = m0 + row;
             if (A_FAST && flat_rows) {
-                a_voff[p] = m < P.M ? (uint32_t)(m * P.xs_h + (tid % A_VPR) * 4) * 4u : CONV_OOB;
+                a_voff[p] = m < P.M ? (uint32_t)(m * P.xs_h + a_kv * 4) * 4u : CONV_OOB;
                 a_inv[p]  = 0u;
                 continue;
             }
@@ -280,7 +294,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             }
             const int hi0 = ho * P.SH - P.PH, wi0 = wo * P.SW - P.PW;
             if constexpr (A_FAST) {
-                a_voff[p] = m < P.M ? (uint32_t)(b * P.xs_b + ho * P.SH * P.xs_h + wo * P.SW * P.xs_w + (tid % A_VPR) * 4) * 4u : CONV_OOB;
+                a_voff[p] = m < P.M ? (uint32_t)(b * P.xs_b + ho * P.SH * P.xs_h + wo * P.SW * P.xs_w + a_kv * 4) * 4u : CONV_OOB;
                 a_inv[p]  = 0u;
                 if (masked) {
                     uint32_t wbad = 0u;
@@ -297,19 +311,19 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             }
         }
         t_r = 0; t_s = 0; t_c = 0;
-        ak = A_FAST ? (tid % A_VPR) * 4 : (tid / BM) * A_KPT;
+        ak = A_FAST ? a_kv * 4 : (tid / BM) * A_KPT;
         const int rs = ak / P.Cin;
         ac = ak - rs * P.Cin; ar = rs / P.KW; as_ = rs - ar * P.KW;
     };
 
     constexpr int B_VPR   = BN / 4;
-    constexpr int B_RSTEP = NT / B_VPR;
-    constexpr int B_NV    = BK / B_RSTEP;
+    constexpr int B_RSTEP = WAVE_PRIVATE ? 64 / B_VPR : NT / B_VPR;
+    constexpr int B_NV    = (WAVE_PRIVATE ? BKW_ : BK) / B_RSTEP;
     constexpr int B_KG    = NT / BN;                // generic: k groups
     constexpr int B_KPT   = BK / B_KG;
     // B fast: byte offset of this thread's first vector in tile 0, or out of range for columns >= N
-    const int      b_n    = n0 + (tid % B_VPR) * 4;
-    const uint32_t b_voff = b_n < P.N ? (uint32_t)((tid / B_VPR) * P.N + b_n) * 4u : CONV_OOB;
+    const int      b_n    = n0 + b_nv * 4;
+    const uint32_t b_voff = b_n < P.N ? (uint32_t)(b_r0 * P.N + b_n) * 4u : CONV_OOB;
 
     f32x4 a_reg[A_FAST ? A_NV : 1];
     float a_sreg[A_FAST ? 1 : A_KPT];
@@ -329,7 +343,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
                     for (int p = 0; p < A_NV; ++p) a_reg[p] = buffer_load_x4(x_rsrc, a_voff[p], soff);
                 } else {
                     const uint32_t sh   = 31u - (uint32_t)(t_r * P.KW + t_s);
-                    const bool     kbad = tail && k0 + (tid % A_VPR) * 4 >= P.K;
+                    const bool     kbad = tail && k0 + a_kv * 4 >= P.K;
 #pragma unroll
                     for (int p = 0; p < A_NV; ++p) {
                         const uint32_t v = a_voff[p] | ((a_inv[p] << sh) & CONV_OOB);
@@ -337,7 +351,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
                     }
                 }
             } else {
-                const uint32_t koff = (uint32_t)(ar * P.DH * P.xs_h + as_ * P.DW * P.xs_w + ac - (tid % A_VPR) * 4) * 4u;
+                const uint32_t koff = (uint32_t)(ar * P.DH * P.xs_h + as_ * P.DW * P.xs_w + ac - a_kv * 4) * 4u;
                 const uint32_t sh   = 31u - (uint32_t)(ar * P.KW + as_);
                 const bool     kok  = ak < P.K;
 #pragma unroll
@@ -393,7 +407,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         if constexpr (A_FAST) {
 #pragma unroll
             for (int p = 0; p < A_NV; ++p) {
-                const int row = tid / A_VPR + p * A_RSTEP, kv = tid % A_VPR;
+                const int row = a_r0 + p * A_RSTEP, kv = a_kv;
                 *reinterpret_cast<f32x4*>(&As[row * LDA + kv * 4]) = a_reg[p];
             }
         } else {
@@ -404,7 +418,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         if constexpr (B_FAST) {
 #pragma unroll
             for (int p = 0; p < B_NV; ++p) {
-                const int kr = tid / B_VPR + p * B_RSTEP, nv = tid % B_VPR;
+                const int kr = b_r0 + p * B_RSTEP, nv = b_nv;
                 *reinterpret_cast<f32x4*>(&Bs[kr * LDB + nv * 4]) = b_reg[p];
             }
         } else {
@@ -496,18 +510,18 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         // all k steps but the last: the next step's loads are in flight during the MFMAs
         for (int kt = 1; kt < ktiles; ++kt) {
             store_tiles();
-            __syncthreads();
+            tile_barrier();
             load_tiles(kt * BK);
 #ifdef CONV_PHASE_STAMPS
             if (kt == 1 && sub == 0) { CONV_STAMP(2) }
 #endif
             compute();
-            __syncthreads();
+            tile_barrier();
         }
         // last k step: the loads in flight are those of the next M tile's first step and of
         // the residual operand
         store_tiles();
-        __syncthreads();
+        __syncthreads();                 // (also where wave-private tiles publish the epilogue operands parked in LDS)
         if (sub + 1 < nsub) {
             setup_rows(m0 + BM);
             load_tiles(0);
