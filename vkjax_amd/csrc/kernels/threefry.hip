@@ -128,8 +128,18 @@ __device__ __forceinline__ void threefry_stream_steps(uint32_t (&y)[NV], uint32_
 // The chain of jax.random.uniform, known at compile time: the opcode switch folds away and the six
 // single-value operands are fetched before the block function runs instead of one dependent pair
 // of scalar loads per step. (bits >> 9 | 0x3F800000, as float - 1, * (max - min), + min, max(min, .))
+// With the operands of a draw from [0, 1) -- shift 9, exponent bits of 1.0, minus 1.0, times 1.0, plus 0.0,
+// max(0.0, .) -- the first two steps are one funnel shift ((0x7F : bits) >> 9 puts 0x3F800000 above the 23
+// mantissa bits) and the last three change no bit: the value after the subtraction lies in [+0, 1), where
+// x * 1.0, x + 0.0 and max(0.0, x) all return x itself. Two operations per word instead of eight.
 template <int NV>
 __device__ __forceinline__ void threefry_uniform_steps(uint32_t (&y)[NV], const uint32_t (&o)[6]) {
+    const bool unit_interval = o[0] == 9u && o[1] == 0x3F800000u && o[2] == 0x3F800000u && o[3] == 0x3F800000u && o[4] == 0u && o[5] == 0u;
+    if (unit_interval) {                             // the same for every thread of the launch
+#pragma unroll
+        for (int j = 0; j < NV; ++j) y[j] = f2u(u2f(__builtin_amdgcn_alignbit(0x7Fu, y[j], 9u)) - 1.0f);
+        return;
+    }
     constexpr uint32_t ops[6] = {EW_SHR_L, EW_OR_X, EW_SUB_F, EW_MUL_F, EW_ADD_F, EW_MAX_F};
 #pragma unroll
     for (int k = 0; k < 6; ++k) {
