@@ -132,6 +132,22 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
     if (!is_arg) {
         a = red_step<MODE>(P.op, P.type, red_step<MODE>(P.op, P.type, acc[0], acc[1]), red_step<MODE>(P.op, P.type, acc[2], acc[3]));
     }
+    if constexpr (MODE >= 3) {
+        // float argmax / argmin across the lanes as the maximum of one 64-bit key per lane: the value mapped to an
+        // unsigned number that grows with its rank (a NaN above everything), then the complement of the index, so
+        // that of two equal values the earlier one wins. Five operations per butterfly step instead of a dozen.
+        const uint32_t bits = best_v, flipped = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+        const float    x    = u2f(bits);
+        const uint32_t rank = x != x ? 0xFFFFFFFFu : (MODE == 3 ? flipped : ~flipped);
+        uint64_t key = best_i == 0xFFFFFFFFu ? 0ull : ((uint64_t)rank << 32 | (uint32_t)~best_i);   // no rank of a value is 0
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) {
+            const uint64_t other = __shfl_xor(key, s, 64);
+            key = other > key ? other : key;
+        }
+        if (lane == 0) out[unit] = key == 0ull ? 0u : ~(uint32_t)key;
+        return;
+    }
 #pragma unroll
     for (int s = 32; s >= 1; s >>= 1) {
         if (is_arg) {
