@@ -265,6 +265,47 @@ def test_mixed_tiling_and_two_group_kernels():
         K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = K.FORCE_CONV_KSPLIT = K.FORCE_CONV_MIX = None
 
 
+def test_stem_kernel_for_few_input_features():
+    '''conv_gemm_stem_7x22: seven kernel rows whose KW * Cin values (21 or 22) are read from a patch of image rows
+    in LDS. 7 x 7 on 3 features with stride 2 and padding 3 (the ResNet stem), stride 1, a 7 x 11 kernel on 2
+    features, fewer than 64 output features, images that are not square, several tiles per block (more tiles than
+    the grid has blocks), with a batch-norm + ReLU epilogue, bias + ReLU and none; integer-valued data, so every
+    result is exact.'''
+    from vkjax_amd import kernels as K
+    from vkjax_amd import minijax as mj
+    lax, nn = mj.lax, mj.nn
+    dn = ('NHWC', 'HWIO', 'NHWC')
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    vec = lambda lo, hi, n: rng.randint(lo, hi, size=[n]).astype(np.float32)
+
+    def conv(stride, padding):
+        return lambda x, k: lax.conv_general_dilated(x, k, (stride, stride), padding, dimension_numbers=dn)
+    def bn_relu(stride, padding):
+        def f(x, k, mean, var, scale, beta):
+            y = lax.conv_general_dilated(x, k, (stride, stride), padding, dimension_numbers=dn)
+            return nn.relu((y - mean) * (scale * lax.rsqrt(var + 3.0)) + beta)       #var + 3 = 4: an exact rsqrt
+        return f
+    def bias_relu(stride, padding):
+        return lambda x, k, b: nn.relu(lax.conv_general_dilated(x, k, (stride, stride), padding, dimension_numbers=dn) + b)
+
+    p3 = ((3, 3), (3, 3))
+    cases = [(bn_relu(2, p3), [ints(-4, 5, 2, 128, 128, 3), ints(-3, 4, 7, 7, 3, 64), vec(-5, 5, 64), np.ones(64, np.float32), vec(1, 4, 64) * 2, vec(-9, 9, 64)]),
+             (conv(2, p3), [ints(-4, 5, 3, 20, 192, 3), ints(-3, 4, 7, 7, 3, 40)]),
+             (bias_relu(1, p3), [ints(-4, 5, 1, 12, 64, 3), ints(-3, 4, 7, 7, 3, 64), vec(-9, 9, 64)]),
+             (conv(2, ((3, 3), (5, 5))), [ints(-4, 5, 2, 16, 128, 2), ints(-3, 4, 7, 11, 2, 24)]),
+             (conv(2, ((0, 2), (3, 4))), [ints(-4, 5, 1, 132, 128, 3), ints(-3, 4, 7, 7, 3, 64)]),
+             (bn_relu(2, p3), [ints(-4, 5, 18, 128, 128, 3), ints(-3, 4, 7, 7, 3, 64), vec(-5, 5, 64), np.ones(64, np.float32), vec(1, 4, 64) * 2, vec(-9, 9, 64)])]
+    for f, args in cases:
+        print(f'stem kernel: {[a.shape for a in args]}', flush=True)
+        for fuse in (True, False):
+            _, _, fn = check_against_oracle(f, args, exact=True, fuse=fuse)
+            kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches if l.kernel.startswith('conv_gemm')]
+            assert kernels == ['conv_gemm_stem_7x22'], kernels
+    #a shape it does not take falls back to the general kernel
+    _, _, fn = check_against_oracle(conv(2, p3), [ints(-4, 5, 2, 30, 26, 3), ints(-3, 4, 7, 7, 3, 64)], exact=True)
+    assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['conv_gemm_64x64x32_gf']
+
+
 def test_convolution_with_a_second_result():
     '''A convolution result that is returned (or read later) AND continued by an element-wise chain: one launch
     stores both, the value before the chain or after its `- vector` step and the chain's result. Integer-valued

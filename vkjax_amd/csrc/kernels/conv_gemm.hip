@@ -774,3 +774,203 @@ CONV_KERNEL(conv_gemm_64x64x128_ks2, 2, 2, 1, 1, 128, true, true, true, 2)
     }
 CONV_MIX_KERNEL(conv_gemm_64x64x32_mix, 32)
 CONV_MIX_KERNEL(conv_gemm_64x64x64_mix, 64)
+
+// ---------------------------------------------------------------------------------------------
+// Convolutions of dense images with very few features (an RGB stem: 7 x 7 x 3, stride 2). The general kernel
+// above assembles the A tile element by element for them: 1650 vector instructions per 64 x 64 tile against
+// 80 MFMAs, and the two share the SIMDs' issue slots (counters: the vector ALUs busy 56 % of the kernel's time).
+// Here a block copies the image rows its 64 output positions touch into LDS once (16-byte loads of whole
+// rows, zero borders written beside them) and the MFMA operands are read straight from that patch: the
+// KW * Cin values one kernel row reads for an output position are contiguous there, so the address of A(m, k)
+// is a per-lane base plus a compile-time offset. The whole kernel (KH * RLP rows, RLP = KW * Cin rounded up to
+// even, the extra row zero) sits in LDS for the block's lifetime; a block walks the tiles in steps of the grid.
+//   KH: kernel rows; RLP: padded run length; PR: image rows of a patch (>= KH + SH, a tile spans two output rows
+//   at most); NVEC: 16-byte vectors a thread fetches per patch.
+// Requirements (the host checks them): pixels dense ([B, H, W, Cin], W * Cin % 4 == 0), no dilation, M % 64 == 0,
+// Ho * Wo % 64 == 0 (a tile lies in one image), Wo >= 64, N <= 64, row-major result, template epilogue without a
+// full-size operand, KW * Cin in (RLP - 2, RLP], KH + SH <= PR, PR * W * Cin / 4 <= 256 * NVEC.
+struct ConvStemParams {
+    int32_t M, N, K;
+    int32_t Ho, Wo, H, W, Cin, KH, KW, SH, SW, PH, PW;
+    int32_t pitch;                  // floats per patch row: left border, W * Cin values, right border (a multiple of 4)
+    int32_t left;                   // floats of left border (>= PW * Cin, a multiple of 4)
+    uint32_t flags;                 // bits 20-24: template epilogue steps as in ConvParams.flags (bit 23 never)
+    uint32_t x_bytes, w_bytes, out_bytes;
+    uint32_t howo_magic, howo_shift, wo_magic, wo_shift;
+};
+
+template <int KH, int RLP, int PR, int NVEC>
+__device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+                                               const ConvEpiPtrs& epi, const ConvDerivedPtrs& Dp, const ConvStemParams& P,
+                                               const ConvDerived& Dk, float* __restrict__ Ws, float* __restrict__ Ps, float* __restrict__ Es) {
+    constexpr int BN = 64, LDB = BN + 4, G = RLP / 2;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int RL = P.KW * P.Cin, WC = P.W * P.Cin, vecs_per_row = WC >> 2, HoWo = P.Ho * P.Wo;
+    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, P.x_bytes), w_rsrc = make_rsrc(w, P.w_bytes), o_rsrc = make_rsrc(out, P.out_bytes);
+
+    // the kernel: Ws[ky * RLP + j][n] = w[ky, j, n] for j < KW * Cin, zero behind
+    for (int e = tid; e < KH * RLP * (BN / 4); e += 256) {
+        const int row = e / (BN / 4), n4 = (e - row * (BN / 4)) * 4, ky = row / RLP, j = row - ky * RLP;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (j < RL) {
+            const uint32_t off = (uint32_t)((ky * RL + j) * P.N + n4) * 4u;
+            if (n4 + 3 < P.N) v = buffer_load_x4(w_rsrc, off);
+            else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[q] = n4 + q < P.N ? buffer_load_x1(w_rsrc, off + 4u * q) : 0.f;
+            }
+        }
+        *reinterpret_cast<f32x4*>(&Ws[row * LDB + n4]) = v;
+    }
+    // the borders of the patch rows stay zero
+    for (int e = tid; e < PR * P.pitch; e += 256) {
+        const int c = e % P.pitch;
+        if (c < P.left || c >= P.left + WC) Ps[e] = 0.f;
+    }
+    // per-column epilogue operands (see conv_gemm_body)
+    const int nepi = __builtin_popcount((P.flags >> 20) & 31u);
+    if (tid < BN) {
+        float e_reg[CONV_MAX_EPI];
+#pragma unroll
+        for (int e = 0; e < CONV_MAX_EPI; ++e) {
+            e_reg[e] = 0.f;
+            if (e < nepi) {
+                const uint32_t present = epi.p[e] != nullptr ? 1u : 0u;
+                // template steps in order: vector, vector, vector, (full tensor: never here), scalar
+                const bool scalar = e == nepi - 1 && ((P.flags >> 24) & 1u);
+                e_reg[e] = scalar ? buffer_load_x1(make_rsrc(epi.p[e], 4u * present), 0u)
+                                  : buffer_load_x1(make_rsrc(epi.p[e], (uint32_t)P.N * 4u * present), (uint32_t)tid * 4u);
+            }
+        }
+        if (Dk.nsteps) {
+            float in[CONV_MAX_DERIVED + 1];
+#pragma unroll
+            for (int k = 0; k <= CONV_MAX_DERIVED; ++k) {
+                const bool vec = (Dk.vector_mask >> k) & 1u;
+                in[k] = buffer_load_x1(make_rsrc(Dp.p[k], Dp.p[k] == nullptr ? 0u : vec ? (uint32_t)P.N * 4u : 4u), vec ? (uint32_t)tid * 4u : 0u);
+            }
+            float v = in[0];
+#pragma unroll
+            for (int k = 0; k < CONV_MAX_DERIVED; ++k) {
+                if (k < (int)Dk.nsteps) {
+                    const float a = Dk.left[k] ? in[k + 1] : v, b = Dk.left[k] ? v : in[k + 1];
+                    switch (Dk.op[k]) {
+                        case CEW_ADD_F:   v = a + b; break;
+                        case CEW_SUB_F:   v = a - b; break;
+                        case CEW_MUL_F:   v = a * b; break;
+                        case CEW_DIV_F:   v = a / b; break;
+                        case CEW_MAX_F:   v = (a > b || a != a) ? a : b; break;
+                        case CEW_MIN_F:   v = (a < b || a != a) ? a : b; break;
+                        case CEW_NEG_F:   v = -v; break;
+                        case CEW_RSQRT_F: v = 1.0f / sqrtf(v); break;
+                        case CEW_SQRT_F:  v = sqrtf(v); break;
+                        default: break;
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < CONV_MAX_EPI; ++e)
+                if (e == (int)Dk.step) e_reg[e] = v;
+        }
+#pragma unroll
+        for (int e = 0; e < CONV_MAX_EPI; ++e)
+            if (e < nepi) Es[e * BN + tid] = e_reg[e];
+    }
+
+    const int tiles = P.M / 64;
+    // the image rows of the patch of tile t: requested into registers, written to LDS later
+    f32x4 pv[NVEC];
+    auto patch_geometry = [&](int t, int& b, int& ho0, int& hi0) {
+        const int m0 = t * 64;
+        b = magic_div(m0, P.howo_magic, P.howo_shift);
+        ho0 = magic_div(m0 - b * HoWo, P.wo_magic, P.wo_shift);
+        hi0 = ho0 * P.SH - P.PH;
+    };
+    auto request_patch = [&](int t) {
+        int b, ho0, hi0;
+        patch_geometry(t, b, ho0, hi0);
+#pragma unroll
+        for (int q = 0; q < NVEC; ++q) {
+            const int v = tid + q * 256, r = v / vecs_per_row, c4 = v - r * vecs_per_row, hi = hi0 + r;
+            const bool ok = r < PR && (uint32_t)hi < (uint32_t)P.H;
+            pv[q] = buffer_load_x4(x_rsrc, ok ? (uint32_t)(((b * P.H + hi) * P.W) * P.Cin + c4 * 4) * 4u : CONV_OOB);   // zeros outside the image
+        }
+    };
+    auto park_patch = [&]() {
+#pragma unroll
+        for (int q = 0; q < NVEC; ++q) {
+            const int v = tid + q * 256, r = v / vecs_per_row, c4 = v - r * vecs_per_row;
+            if (r < PR) *reinterpret_cast<f32x4*>(&Ps[r * P.pitch + P.left + c4 * 4]) = pv[q];
+        }
+    };
+
+    int t = blockIdx.x;
+    if (t < tiles) request_patch(t);
+    for (; t < tiles; t += gridDim.x) {
+        __syncthreads();                              // the previous tile's reads of the patch are over (first pass: the fills above)
+        park_patch();
+        __syncthreads();
+        if (t + (int)gridDim.x < tiles) request_patch(t + gridDim.x);   // in flight during this tile's MFMAs
+        int b, ho0, hi0;
+        patch_geometry(t, b, ho0, hi0);
+        // this lane's output position and where its kernel row 0 starts in the patch
+        const int m  = t * 64 + wm * 32 + l32;
+        const int r2 = m - b * HoWo, ho = magic_div(r2, P.wo_magic, P.wo_shift), wo = r2 - ho * P.Wo;
+        const float* a_base = Ps + (ho - ho0) * P.SH * P.pitch + P.left + (wo * P.SW - P.PW) * P.Cin + half;
+        const float* b_base = Ws + half * LDB + wn * 32 + l32;
+        f32x16 acc = {};
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky) {
+            const float* a_row = a_base + ky * P.pitch;
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float a = a_row[2 * g];
+                // the padding position behind an odd run is a neighbouring pixel, not a zero: 0 * Inf would be NaN
+                if (g == G - 1 && 2 * g + half >= RL) a = 0.f;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b_base[(ky * RLP + 2 * g) * LDB], acc, 0, 0, 0);
+            }
+        }
+        // epilogue: (acc - vector) * vector + vector, max(., scalar), each optional, then the store
+        float y[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = acc[v];
+        const uint32_t slots = (P.flags >> 20) & 31u;
+        const int col = wn * 32 + l32;
+        const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u), e_max = __builtin_popcount(slots & 15u);
+        if (slots & 1u) {
+            const float o = Es[col];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) y[v] = y[v] - o;
+        }
+        if (slots & 2u) {
+            const float o = Es[e_mul * BN + col];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) y[v] = y[v] * o;
+        }
+        if (slots & 4u) {
+            const float o = Es[e_add * BN + col];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) y[v] = y[v] + o;
+        }
+        if (slots & 16u) {
+            const float o = Es[e_max * BN + col];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) y[v] = (y[v] > o || y[v] != y[v]) ? y[v] : o;
+        }
+        const uint32_t base = col < P.N ? (uint32_t)((t * 64 + wm * 32 + 4 * half) * P.N + col) * 4u : CONV_OOB;
+        const uint32_t rowb = (uint32_t)P.N * 4u;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) buffer_store_x1(y[v], o_rsrc, base, (uint32_t)(8 * (v / 4) + (v % 4)) * rowb);
+    }
+}
+
+#define CONV_STEM_PATCH_FLOATS 6272          // PR rows of at most 696 floats (W * Cin = 672 with borders), + slack
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void conv_gemm_stem_7x22(
+        float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+        ConvEpiPtrs epi, ConvDerivedPtrs dp, ConvStemParams P, ConvDerived D) {
+    __shared__ __attribute__((aligned(16))) float Ws[7 * 22 * 68];
+    __shared__ __attribute__((aligned(16))) float Ps[CONV_STEM_PATCH_FLOATS];
+    __shared__ float Es[CONV_MAX_EPI * 64];
+    conv_stem_body<7, 22, 9, 6>(out, x, w, epi, dp, P, D, Ws, Ps, Es);
+}

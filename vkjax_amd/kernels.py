@@ -522,6 +522,57 @@ def _magic_division(d: int) -> tp.Tuple[int, int]:
     return magic, l - 1
 
 
+STEM_PATCH_FLOATS, STEM_PATCH_ROWS, STEM_VECTORS_PER_THREAD = 6272, 9, 6      #conv_gemm_stem_7x22's LDS patch
+FORCE_CONV_STEM: tp.Optional[bool] = None       #the patch kernel for few input features: never (False); None / True: where it applies
+
+
+def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_units, lhs_offset, rhs_offset, out_offset) -> tp.Optional[Launch]:
+    '''conv_gemm_stem_7x22 where it applies: dense images with so few features that KW * Cin is 21 or 22 (7 x 7 x 3),
+    seven kernel rows, a template epilogue; see the conditions listed at the kernel.'''
+    if FORCE_CONV_STEM is False or FORCE_CONV_TILE is not None or FORCE_CONV_GENERAL or taps or lhs_offset or rhs_offset or out_offset:
+        return None
+    M, N, K = g.M, g.N, g.K
+    RL, WC = g.KW * g.Cin, g.W * g.Cin
+    dense_in  = g.xs == (g.H * WC, WC, g.Cin, 1)
+    dense_w   = g.ws == (g.KW * g.Cin * N, g.Cin * N, N, 1)
+    dense_out = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
+    slots = _epilogue_template_slots(epilogue)
+    left  = _cdiv(g.PW * g.Cin, 4) * 4
+    right = max(0, (g.Wo - 1) * g.SW - g.PW + g.KW - g.W)          #pixels the last window reaches beyond the row
+    pitch = _cdiv(left + (g.W + right) * g.Cin + 1, 4) * 4
+    ok = (g.KH == 7 and RL in (21, 22) and dense_in and dense_w and dense_out and g.DH == g.DW == g.LH == g.LW == 1
+          and g.PH >= 0 and g.PW >= 0 and WC % 4 == 0 and M % 64 == 0 and (g.Ho * g.Wo) % 64 == 0 and g.Wo >= 64 and N <= 64
+          and (not epilogue or (slots != 0 and not slots & 8)) and g.KH + g.SH <= STEM_PATCH_ROWS
+          and STEM_PATCH_ROWS * pitch <= STEM_PATCH_FLOATS and STEM_PATCH_ROWS * (WC // 4) <= 256 * STEM_VECTORS_PER_THREAD)
+    if not ok:
+        return None
+    flags  = slots << 20
+    params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, pitch, left)
+              + _u32(flags, lhs.size * 4, rhs.size * 4, out.size * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo)))
+    derived_ptrs, derived_desc = _conv_derived(epilogue, N)
+    params += derived_desc
+    buffers = [(out, 0), (lhs, 0), (rhs, 0)] + _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0)) + derived_ptrs
+    nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
+    return Launch('conv_gemm_stem_7x22', (min(M // 64, 2 * compute_units), 1, 1), (256, 1, 1), buffers, params,
+                  bytes_moved=nbytes, flops=2 * M * N * K)
+
+
+def _conv_derived(epilogue, N):
+    '''(pointer slots, descriptor words) of the one per-feature epilogue operand that the kernel computes itself.'''
+    derived_ptrs, derived_desc = [(None, 0)] * (CONV_MAX_DERIVED + 1), _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
+    for i, e in enumerate(epilogue):
+        if e.derived is not None:
+            d = e.derived
+            assert e.kind == 2 and len(d.steps) <= CONV_MAX_DERIVED and derived_desc == _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
+            arrays = [d.first] + [st[1] for st in d.steps]
+            assert all(a is None or a.size in (1, N) for a in arrays)
+            derived_ptrs = _pad([(a, 0) for a in arrays], CONV_MAX_DERIVED + 1, (None, 0))
+            mask = sum(1 << k for k, a in enumerate(arrays) if a is not None and a.size == N and N != 1)
+            derived_desc = _u32(i, len(d.steps), mask, *_pad([st[0] for st in d.steps], CONV_MAX_DERIVED),
+                                *_pad([int(st[2]) for st in d.steps], CONV_MAX_DERIVED))
+    return derived_ptrs, derived_desc
+
+
 def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: tp.Sequence[ConvEpilogueStep] = (),
               compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0, out_offset: int = 0) -> Launch:
     taps = [(i, e.operand) for i, e in enumerate(epilogue) if e.op == CONV_TAP]
@@ -537,6 +588,9 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     for name, extent in (('lhs', lhs.size), ('rhs', rhs.size), ('out', out.size)):
         if extent * 4 >= 2**31:
             raise NotImplementedError(f'conv/dot {name} operand of {extent * 4} bytes exceeds the 2 GiB the kernel addresses')
+    stem = _conv_stem_launch(out, lhs, rhs, g, epilogue, taps, compute_units, lhs_offset, rhs_offset, out_offset)
+    if stem is not None:
+        return stem
     tag, bm, bn, nt = choose_conv_tile(M, N, compute_units)
     bk = choose_conv_bk(tag, g)
     #some kernel tap of some output position falls outside the input (padding, or a window that overhangs)
@@ -596,17 +650,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
                    *g.xs[:3], tiles_m, tiles_n)
               + _u32(flags, *descs, x_bytes, w_bytes, (out.size - out_offset) * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
               + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os, split_tiles_m))
-    derived_ptrs, derived_desc = [(None, 0)] * (CONV_MAX_DERIVED + 1), _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
-    for i, e in enumerate(epilogue):
-        if e.derived is not None:
-            d = e.derived
-            assert e.kind == 2 and len(d.steps) <= CONV_MAX_DERIVED and derived_desc == _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
-            arrays = [d.first] + [st[1] for st in d.steps]
-            assert all(a is None or a.size in (1, N) for a in arrays)
-            derived_ptrs = _pad([(a, 0) for a in arrays], CONV_MAX_DERIVED + 1, (None, 0))
-            mask = sum(1 << k for k, a in enumerate(arrays) if a is not None and a.size == N and N != 1)
-            derived_desc = _u32(i, len(d.steps), mask, *_pad([st[0] for st in d.steps], CONV_MAX_DERIVED),
-                                *_pad([int(st[2]) for st in d.steps], CONV_MAX_DERIVED))
+    derived_ptrs, derived_desc = _conv_derived(epilogue, N)
     params += derived_desc
     buffers = [(out, out_offset * 4), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
     operand_slots = _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
