@@ -85,6 +85,9 @@ def test_kernel_argument_layouts_match_the_structs():
     launches = {
         'EwParams': K.lower_ew_chain(chain), 'IotaParams': K.iota(i(8), 0), 'FillParams': K.fill(b(8), 0),
         'ConcatParams': K.concat_part(b(4, 8), b(4, 3), 1, 0), 'ConvParams': K.conv_gemm(b(1, 4, 4, 8), b(1, 4, 4, 4), b(1, 1, 4, 8), geom),
+        'ConvStemParams': K.conv_gemm(b(1, 64, 64, 8), b(1, 128, 128, 3), b(7, 7, 3, 8),
+                                      K.ConvGeometry(batch=1, Ho=64, Wo=64, N=8, H=128, W=128, Cin=3, KH=7, KW=7, SH=2, SW=2, PH=3, PW=3,
+                                                     xs=(128 * 384, 384, 3, 1), ws=(168, 24, 8, 1), os=(64 * 512, 512, 8, 1))),
         'ReduceParams': K.reduce(b(4), b(4, 8), 4, 8, 1, 'reduce_sum')[0],
         'ReduceGeneralParams': K.reduce_general(b(4), b(4, 8), [(4, 8)], [(8, 1)], 'reduce_sum'),
         'PoolParams': K.pool(b(1, 2, 2, 4), b(1, 4, 4, 4), 'reduce_max', (1, 2, 2, 1), (1, 2, 2, 1), (0, 0, 0, 0), (1, 1, 1, 1)),
@@ -104,6 +107,8 @@ def test_kernel_argument_layouts_match_the_structs():
     }
     #the convolution kernel takes two parameter structs, one after the other
     sizes['ConvParams'] += sizes['ConvDerived']
+    sizes['ConvStemParams'] += sizes['ConvDerived']
+    assert launches['ConvStemParams'].kernel == 'conv_gemm_stem_7x22'
     for struct, launch in launches.items():
         assert len(launch.params) == sizes[struct], (struct, len(launch.params), sizes[struct])
     assert sizes['ConvEpiPtrs'] == 8 * K.CONV_MAX_EPI and sizes['ThreefryStreamPtrs'] == 8 * K.TF_MAX_STEPS

@@ -617,13 +617,10 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     #tile, each taking a quarter of every (128-long) k step
     ksplit = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
               (_cdiv(M, 32) * _cdiv(N, 32) <= 2 * compute_units and K >= 256 and FORCE_CONV_TILE is None and FORCE_CONV_BK is None))
-    ks_variant = ksplit if isinstance(ksplit, str) else '32x32x128_ks4'
-    ks_tag, ks_bk, ks_w = ks_variant.rsplit('x', 1)[0], int(ks_variant.rsplit('x', 1)[1].split('_')[0]), int(ks_variant[-1])
-    ksplit = bool(ksplit) and a_fast and c_contig and (g.Cin % ks_bk == 0 or g.KH * g.KW == 1) \
-        and (b_fast or ks_tag == '32x32') and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL
+    ksplit = bool(ksplit) and a_fast and c_contig and (g.Cin % 128 == 0 or g.KH * g.KW == 1) \
+        and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL
     if ksplit:
-        side = int(ks_tag.split('x')[0])
-        tag, bm, bn, nt, bk, lean = ks_tag, side, side, (side // 32) ** 2 * 64 * ks_w, ks_bk, True
+        tag, bm, bn, nt, bk, lean = '32x32', 32, 32, 256, 128, True
     tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
     chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean and not ksplit else 1
     #64 x 64 tiles that do not divide evenly among the CUs: as many M tiles as fill every CU equally stay 64 x 64, the
@@ -658,7 +655,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
         assert operand_slots[-1] == (None, 0)
         operand_slots[-1] = (tap_buffer, 0)
     buffers += operand_slots + derived_ptrs
-    kernel  = f'conv_gemm_{tag}x{bk}_' + ((f'ks{ks_w}' if b_fast else f'ks{ks_w}g') if ksplit else 'lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
+    kernel  = f'conv_gemm_{tag}x{bk}_' + (('ks4' if b_fast else 'ks4g') if ksplit else 'lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
     nbytes += 4 * tap_buffer.size if taps else 0
     blocks = _cdiv(tiles_m, chunk) * tiles_n
