@@ -35,6 +35,10 @@ __device__ __forceinline__ float buffer_load_x1(__amdgpu_buffer_rsrc_t r, uint32
 __device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, voff, soff, 0);
 }
+// the same for data that is touched once (nontemporal: not kept in the caches at the expense of what is reused)
+__device__ __forceinline__ float buffer_load_x1_nt(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 2));
+}
 __device__ __forceinline__ int magic_div(int n, uint32_t magic, uint32_t shift) {
     return magic ? (int)(__umulhi((uint32_t)n, magic) >> shift) : n;
 }

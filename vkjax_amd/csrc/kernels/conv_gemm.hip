@@ -599,7 +599,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
                     // after the per-feature steps
                     float ov[16];
                     if ((slots & 8u) && !(PREFETCH_FULL && first_full >= 0))
-                        sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1(f_rsrc, vo, so); });
+                        sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) { ov[v] = buffer_load_x1_nt(f_rsrc, vo, so); });   // read once: kept out of the caches (-0.8 % on ResNet-50's step)
                     // a second result: the value as it stands before or after the first step
 #define CONV_TAP_STORE() sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) {                                   \
                             buffer_store_x1(y[v], make_rsrc(epi.p[CONV_MAX_EPI - 1], P.out_bytes), vo, so); })
