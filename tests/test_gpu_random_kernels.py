@@ -1,0 +1,93 @@
+'''Seeded random geometry through three kernels whose applicability depends on the shape: the mixed 64 x 64 /
+32 x 32 tiling (split point, k step and epilogue drawn at random), the stem kernel (kernel width x features of 21
+or 22 in several factorisations, strides, paddings on all four sides, image sizes around its limits; shapes it does
+not take fall back to the general kernel and are checked all the same) and the sorted scatter-add (table and index
+sizes around the segment and block limits, crowded rows, indices outside the table). Integer-valued data: every
+result equals the oracle's bit for bit.'''
+import numpy as np
+import pytest
+
+from vkjax_amd import kernels as K, minijax as mj, ops
+from tests.common import check_against_oracle
+
+pytestmark = pytest.mark.gpu
+lax, jnp, nn = mj.lax, mj.numpy, mj.nn
+DN = ('NHWC', 'HWIO', 'NHWC')
+
+
+def _mixed_tiling_case(rng, ints):
+    b, h, w = int(rng.choice([1, 2, 3])), int(rng.randint(3, 20)), int(rng.randint(3, 20))
+    ks, stride = int(rng.choice([1, 3])), int(rng.choice([1, 1, 2]))
+    cin  = int(rng.choice([64, 68, 100, 128, 260])) if ks == 1 else int(rng.choice([64, 128, 192]))
+    cout = int(rng.choice([8, 40, 64, 72, 130]))
+    ho, wo = -(-h // stride), -(-w // stride)
+    m = b * ho * wo
+    if m < 70 or cin * ks * ks < 256:
+        return None
+    x, k = ints(-3, 4, b, h, w, cin), ints(-2, 3, ks, ks, cin, cout)
+    conv = lambda x, k: lax.conv_general_dilated(x, k, (stride, stride), 'SAME', dimension_numbers=DN)
+    epilogue = rng.randint(0, 3)
+    if epilogue == 0:
+        f, args = conv, [x, k]
+    elif epilogue == 1:
+        f, args = (lambda x, k, bias: nn.relu(conv(x, k) + bias)), [x, k, ints(-9, 9, cout)]
+    else:
+        f = lambda x, k, mean, scale, shift, res: nn.relu((conv(x, k) - mean) * scale + shift + res)
+        args = [x, k, ints(-5, 5, cout), ints(1, 4, cout), ints(-9, 9, cout), ints(-50, 50, b, ho, wo, cout)]
+    forced = dict(FORCE_CONV_TILE='64x64', FORCE_CONV_BK=int(rng.choice([32, 64])), FORCE_CONV_CHUNK=1, FORCE_CONV_KSPLIT=False,
+                  FORCE_CONV_MIX=int(rng.randint(1, max(2, m // 64 + 1))))
+    #(an output width that is no multiple of 4 takes the element-wise kernel loader and with it the general kernel)
+    return f, args, forced, 'conv_gemm' if cout % 4 else '_mix' if forced['FORCE_CONV_MIX'] * 64 < m else '_lean'
+
+
+def _stem_case(rng, ints):
+    cin, kw = [(3, 7), (3, 7), (2, 11), (1, 21), (1, 22), (11, 2), (7, 3)][rng.randint(0, 7)]
+    stride = int(rng.choice([1, 2, 2]))
+    pw, ph = (int(rng.randint(0, kw)), int(rng.randint(0, kw))), (int(rng.randint(0, 5)), int(rng.randint(0, 5)))
+    w = (int(rng.choice([64, 64, 96, 128])) - 1) * stride + kw - sum(pw) + int(rng.randint(0, stride))
+    while w < 1 or (w * cin) % 4:
+        w += 1
+    wo = (w + sum(pw) - kw) // stride + 1
+    ho = int(rng.choice([1, 2, 3, 5, 8]))
+    while (ho * wo) % 64:
+        ho += 1
+    h = (ho - 1) * stride + 7 - sum(ph) + int(rng.randint(0, stride))
+    if wo < 64 or h < 1:
+        return None
+    cout = int(rng.choice([8, 24, 40, 64]))
+    x, k = ints(-3, 4, int(rng.choice([1, 2, 3])), h, w, cin), ints(-2, 3, 7, kw, cin, cout)
+    f = lambda x, k, bias: nn.relu(lax.conv_general_dilated(x, k, (stride, stride), (ph, pw), dimension_numbers=DN) + bias)
+    return f, [x, k, ints(-9, 9, cout)], {}, ''
+
+
+def _scatter_case(rng, ints):
+    rows, cols = int(rng.choice([1, 5, 64, 300, 1024, 1025, 5000, 70000])), int(rng.choice([1, 3, 4, 64, 256, 260]))
+    n = int(rng.choice([1, 2, 17, 65, 256, 1000, 5000]))
+    idx = rng.randint(-2, rows + 2, size=(n,)).astype(np.int32)
+    if rng.randint(0, 2):
+        idx[: n // 2] = idx[0]
+    return (lambda t, i, u: jnp.index_add(t, i, u)), [ints(-9, 10, rows, cols), idx, ints(-3, 4, n, cols)], {}, 'scatter_rows_sum'
+
+
+@pytest.mark.parametrize('seed', range(90))
+def test_random_geometry(seed):
+    rng  = np.random.RandomState(777 + seed)
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    case = (_mixed_tiling_case, _stem_case, _scatter_case)[seed % 3](rng, ints)
+    if case is None:
+        pytest.skip('the draw gave a shape outside the kernels\' range')
+    f, args, forced, expected = case
+    saved_threshold = ops.SCATTER_SORT_THRESHOLD
+    try:
+        for name, value in forced.items():
+            setattr(K, name, value)
+        if seed % 3 == 2:
+            ops.SCATTER_SORT_THRESHOLD = 0
+        print(f'seed {seed}: {[a.shape for a in args]} {forced}', flush=True)
+        _, _, fn = check_against_oracle(f, args, exact=True)
+        kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+        assert any(expected in k for k in kernels), kernels
+    finally:
+        for name in forced:
+            setattr(K, name, None)
+        ops.SCATTER_SORT_THRESHOLD = saved_threshold
