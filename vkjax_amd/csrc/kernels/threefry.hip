@@ -36,7 +36,9 @@ __device__ __forceinline__ void threefry_body(uint32_t* __restrict__ out0, uint3
     if (e >= P.n) return;
     uint32_t a[VEC], b[VEC], ka[VEC], kb[VEC];
     if constexpr (VEC == 4) {
-        const u32x4 va = *reinterpret_cast<const u32x4*>(in0 + e), vb = *reinterpret_cast<const u32x4*>(in1 + e);
+        // counters in, random words out: every byte is touched once (nontemporal accesses)
+        const u32x4 va = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in0 + e)),
+                    vb = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in1 + e));
         a[0] = va.x; a[1] = va.y; a[2] = va.z; a[3] = va.w;
         b[0] = vb.x; b[1] = vb.y; b[2] = vb.z; b[3] = vb.w;
     } else {
@@ -56,8 +58,8 @@ __device__ __forceinline__ void threefry_body(uint32_t* __restrict__ out0, uint3
         u32x4 va, vb;
         va.x = a[0]; va.y = a[1]; va.z = a[2]; va.w = a[3];
         vb.x = b[0]; vb.y = b[1]; vb.z = b[2]; vb.w = b[3];
-        *reinterpret_cast<u32x4*>(out0 + e) = va;
-        *reinterpret_cast<u32x4*>(out1 + e) = vb;
+        __builtin_nontemporal_store(va, reinterpret_cast<u32x4*>(out0 + e));
+        __builtin_nontemporal_store(vb, reinterpret_cast<u32x4*>(out1 + e));
     } else {
         out0[e] = a[0]; out1[e] = b[0];
     }
