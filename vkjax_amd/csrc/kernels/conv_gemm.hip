@@ -325,12 +325,17 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     const int      b_n    = n0 + b_nv * 4;
     const uint32_t b_voff = b_n < P.N ? (uint32_t)(b_r0 * P.N + b_n) * 4u : CONV_OOB;
 
-    f32x4 a_reg[A_FAST ? A_NV : 1];
+    // what a thread has requested of the coming k step(s): one step ahead, two for the wave-private tiles, whose
+    // single block per CU has nothing else to cover a load's latency with
+    // (not for the small tiles of the mixed kernels, k step 64: their registers decide how many blocks share a CU;
+    // nor with element-wise loads of B, whose 16 values per step and stage would spill)
+    constexpr int STAGES = WAVE_PRIVATE && BK >= 128 && B_FAST ? 2 : 1;
+    f32x4 a_reg[STAGES][A_FAST ? A_NV : 1];
     float a_sreg[A_FAST ? 1 : A_KPT];
-    f32x4 b_reg[B_FAST ? B_NV : 1];
-    float b_sreg[B_FAST ? 1 : B_KPT];
+    f32x4 b_reg[STAGES][B_FAST ? B_NV : 1];
+    float b_sreg[STAGES][B_FAST ? 1 : B_KPT];
 
-    auto load_tiles = [&](int k0) {
+    auto load_tiles = [&](int k0, int st = 0) {
         // ---- A ----
         if constexpr (A_FAST) {
             if (uniform_taps) {
@@ -340,14 +345,14 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
                 if (!masked && !tail) {
                     // the common case issues the loads with no vector arithmetic at all
 #pragma unroll
-                    for (int p = 0; p < A_NV; ++p) a_reg[p] = buffer_load_x4(x_rsrc, a_voff[p], soff);
+                    for (int p = 0; p < A_NV; ++p) a_reg[st][p] = buffer_load_x4(x_rsrc, a_voff[p], soff);
                 } else {
                     const uint32_t sh   = 31u - (uint32_t)(t_r * P.KW + t_s);
                     const bool     kbad = tail && k0 + a_kv * 4 >= P.K;
 #pragma unroll
                     for (int p = 0; p < A_NV; ++p) {
                         const uint32_t v = a_voff[p] | ((a_inv[p] << sh) & CONV_OOB);
-                        a_reg[p] = buffer_load_x4(x_rsrc, kbad ? CONV_OOB : v, soff);
+                        a_reg[st][p] = buffer_load_x4(x_rsrc, kbad ? CONV_OOB : v, soff);
                     }
                 }
             } else {
@@ -358,7 +363,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
                 for (int p = 0; p < A_NV; ++p) {
                     uint32_t v = (a_voff[p] + koff) | (a_voff[p] & CONV_OOB);
                     if (masked) v |= (a_inv[p] << sh) & CONV_OOB;
-                    a_reg[p] = buffer_load_x4(x_rsrc, kok ? v : CONV_OOB);
+                    a_reg[st][p] = buffer_load_x4(x_rsrc, kok ? v : CONV_OOB);
                 }
             }
         } else {
@@ -380,7 +385,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             // rows k >= K fall beyond the descriptor and read as zeros
 #pragma unroll
             for (int p = 0; p < B_NV; ++p)
-                b_reg[p] = buffer_load_x4(w_rsrc, b_voff, (uint32_t)(k0 + p * B_RSTEP) * (uint32_t)P.N * 4u);
+                b_reg[st][p] = buffer_load_x4(w_rsrc, b_voff, (uint32_t)(k0 + p * B_RSTEP) * (uint32_t)P.N * 4u);
         } else {
             const int n = n0 + tid % BN;
             int k = k0 + (tid / BN) * B_KPT;
@@ -388,7 +393,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             int c = k - rs * P.Cin, r = rs / P.KW, s = rs - r * P.KW;
 #pragma unroll
             for (int j = 0; j < B_KPT; ++j) {
-                b_sreg[j] = (k < P.K && n < P.N) ? w[r * Pk.ws_r + s * Pk.ws_s + c * Pk.ws_c + n * Pk.ws_n] : 0.f;
+                b_sreg[st][j] = (k < P.K && n < P.N) ? w[r * Pk.ws_r + s * Pk.ws_s + c * Pk.ws_c + n * Pk.ws_n] : 0.f;
                 ++k; ++c;
                 if (c == P.Cin) { c = 0; ++s; if (s == P.KW) { s = 0; ++r; } }
             }
@@ -403,12 +408,12 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         }
     };
 
-    auto store_tiles = [&]() {
+    auto store_tiles = [&](int st = 0) {
         if constexpr (A_FAST) {
 #pragma unroll
             for (int p = 0; p < A_NV; ++p) {
                 const int row = a_r0 + p * A_RSTEP, kv = a_kv;
-                *reinterpret_cast<f32x4*>(&As[row * LDA + kv * 4]) = a_reg[p];
+                *reinterpret_cast<f32x4*>(&As[row * LDA + kv * 4]) = a_reg[st][p];
             }
         } else {
             const int row = tid % BM, kb = (tid / BM) * A_KPT;
@@ -419,12 +424,12 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
 #pragma unroll
             for (int p = 0; p < B_NV; ++p) {
                 const int kr = b_r0 + p * B_RSTEP, nv = b_nv;
-                *reinterpret_cast<f32x4*>(&Bs[kr * LDB + nv * 4]) = b_reg[p];
+                *reinterpret_cast<f32x4*>(&Bs[kr * LDB + nv * 4]) = b_reg[st][p];
             }
         } else {
             const int n = tid % BN, kb = (tid / BN) * B_KPT;
 #pragma unroll
-            for (int j = 0; j < B_KPT; ++j) Bs[(kb + j) * LDB + n] = b_sreg[j];
+            for (int j = 0; j < B_KPT; ++j) Bs[(kb + j) * LDB + n] = b_sreg[st][j];
         }
     };
 
@@ -507,36 +512,58 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = f32x16{};
-        // all k steps but the last: the next step's loads are in flight during the MFMAs
-        for (int kt = 1; kt < ktiles; ++kt) {
-            store_tiles();
-            tile_barrier();
-            load_tiles(kt * BK);
+        if constexpr (STAGES == 2) {
+            // Two k steps of loads in flight per wave, the stages alternating (written out twice: the stage is a
+            // compile-time index into the registers). The waves meet once, behind the first store, which also
+            // publishes the epilogue operands parked in LDS, and again before the reduction reuses the tiles.
+            if (ktiles > 1) load_tiles(BK, 1);
+            for (int kt = 0; kt < ktiles; kt += 2) {
+                store_tiles(0);
+                if (kt == 0) __syncthreads(); else tile_barrier();
+                if (kt + 2 < ktiles) load_tiles((kt + 2) * BK, 0);
+                compute();
+                tile_barrier();
+                if (kt + 1 < ktiles) {
+                    store_tiles(1);
+                    tile_barrier();
+                    if (kt + 3 < ktiles) load_tiles((kt + 3) * BK, 1);
+                    compute();
+                    tile_barrier();
+                }
+            }
+            __syncthreads();
+        } else {
+            // all k steps but the last: the next step's loads are in flight during the MFMAs
+            for (int kt = 1; kt < ktiles; ++kt) {
+                store_tiles();
+                tile_barrier();
+                load_tiles(kt * BK);
 #ifdef CONV_PHASE_STAMPS
-            if (kt == 1 && sub == 0) { CONV_STAMP(2) }
+                if (kt == 1 && sub == 0) { CONV_STAMP(2) }
 #endif
+                compute();
+                tile_barrier();
+            }
+            // last k step: the loads in flight are those of the next M tile's first step and of
+            // the residual operand
+            store_tiles();
+            __syncthreads();                 // (also where wave-private tiles publish the epilogue operands parked in LDS)
+            if (sub + 1 < nsub) {
+                setup_rows(m0 + BM);
+                load_tiles(0);
+            }
+            if (first_full >= 0) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) {
+                            full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, vo, so);
+                        });
+            }
             compute();
-            tile_barrier();
+            __syncthreads();
         }
-        // last k step: the loads in flight are those of the next M tile's first step and of
-        // the residual operand
-        store_tiles();
-        __syncthreads();                 // (also where wave-private tiles publish the epilogue operands parked in LDS)
-        if (sub + 1 < nsub) {
-            setup_rows(m0 + BM);
-            load_tiles(0);
-        }
-        if (first_full >= 0) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) {
-                        full[PREFETCH_FULL ? i : 0][PREFETCH_FULL ? j : 0][v] = buffer_load_x1(f_rsrc, vo, so);
-                    });
-        }
-        compute();
-        __syncthreads();
 #ifdef CONV_PHASE_STAMPS
         if (sub == 0) { CONV_STAMP(3) }
 #endif
