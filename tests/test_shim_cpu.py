@@ -104,6 +104,35 @@ def test_eval_moves_the_bytes_and_everything_is_released(lib):
     assert lib.fake_hip_live_objects() == before
 
 
+def test_many_arguments_are_staged_together(lib):
+    '''From 8 MB of arguments on, all uploads of an evaluation are staged as one stream of 4 MB chunks by helper
+    threads: many arrays of different sizes (some smaller than a chunk, one of several chunks, one empty slot
+    passed as resident) have to arrive intact, in their own buffers.'''
+    w = World(lib)
+    sizes = [3, 1 << 20, 70001, (5 << 20) + 13, 1 << 18, 17]            #elements; 26 MB together
+    seq = H()
+    assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq)) == 0
+    bufs = [w.buf(4 * n) for n in sizes]
+    for slot, (b, n) in enumerate(zip(bufs, sizes)):
+        assert lib.vkj_seq_record_upload(seq, b, 0, slot, 4 * n) == 0
+    for slot, (b, n) in enumerate(zip(bufs, sizes)):
+        assert lib.vkj_seq_record_download(seq, b, 0, len(sizes) + slot, 4 * n) == 0
+    rng = np.random.default_rng(3)
+    for resident in (None, 2):
+        xs = [rng.integers(0, 1 << 32, size=n, dtype=np.uint64).astype(np.uint32) for n in sizes]
+        ys = [np.zeros(n, np.uint32) for n in sizes]
+        ptrs = (C.c_void_p * (2 * len(sizes)))(*[None if k == resident else x.ctypes.data for k, x in enumerate(xs)], *[y.ctypes.data for y in ys])
+        assert lib.vkj_seq_eval(seq, ptrs, 2 * len(sizes), hip.EVAL_NULL_IS_RESIDENT) == 0, lib.vkj_last_error()
+        for k, (x, y) in enumerate(zip(xs, ys)):
+            if k == resident:
+                assert np.array_equal(y, previous[k]), k            #untouched: still what the first evaluation uploaded
+            else:
+                assert np.array_equal(y, x), k
+        previous = xs
+    assert lib.vkj_seq_destroy(seq) == 0
+    w.close()
+
+
 def test_module_unload_is_refused_while_a_sequence_uses_it(lib):
     w = World(lib)
     seq, src, dst = w.add_one_sequence(8)

@@ -86,6 +86,48 @@ int staged_upload(char* staging, const char* host, size_t nbytes, Issue&& issue)
     return status;
 }
 
+// The same for all arguments of an evaluation together (a network's weights: hundreds of arrays of a few MB each,
+// which one thread would stage one after the other at the speed of a single core's memcpy).
+struct UploadPiece { char* staging; const char* host; char* device; size_t nbytes; };
+
+template <class Issue>
+int staged_upload_pieces(const std::vector<UploadPiece>& pieces, Issue&& issue) {
+    struct Chunk { size_t piece, off, len; };
+    std::vector<Chunk> chunks;
+    for (size_t p = 0; p < pieces.size(); p++)
+        for (size_t off = 0; off < pieces[p].nbytes; off += STAGE_CHUNK)
+            chunks.push_back({p, off, std::min(STAGE_CHUNK, pieces[p].nbytes - off)});
+    const size_t nchunks = chunks.size();
+    std::vector<std::atomic<int>> done(nchunks);
+    for (auto& d : done) d.store(0, std::memory_order_relaxed);
+    std::atomic<size_t> next{0};
+    auto worker = [&]() {
+        for (;;) {
+            const size_t k = next.fetch_add(1, std::memory_order_relaxed);
+            if (k >= nchunks) return;
+            const Chunk& ch = chunks[k];
+            memcpy(pieces[ch.piece].staging + ch.off, pieces[ch.piece].host + ch.off, ch.len);
+            done[k].store(1, std::memory_order_release);
+        }
+    };
+    std::vector<std::thread> threads;
+    const int nthreads = (int)std::min<size_t>(STAGE_THREADS, nchunks);
+    try {
+        for (int t = 0; t < nthreads; t++) threads.emplace_back(worker);
+    } catch (...) {
+        // no (more) threads to be had: the calling thread copies whatever is left
+    }
+    if ((int)threads.size() < nthreads) worker();
+    int status = 0;
+    for (size_t k = 0; k < nchunks; k++) {
+        while (!done[k].load(std::memory_order_acquire)) std::this_thread::yield();
+        const Chunk& ch = chunks[k];
+        if (status == 0) status = issue(pieces[ch.piece].device + ch.off, pieces[ch.piece].staging + ch.off, ch.len);
+    }
+    for (auto& t : threads) t.join();
+    return status;
+}
+
 // Large downloads, the other way round: the transfer is issued chunk by chunk with an event behind every
 // chunk; the calling thread waits for the events in order and a few threads copy each chunk out of the
 // pinned buffer as soon as it has landed, while the chunks after it are still on their way.
@@ -214,19 +256,29 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
         s->stamps_valid = 0;
         HIP_TRY(hipEventRecord(s->stamps[0], c->stream));
     }
-    if (up) for (auto& t : s->uploads) {
-        if (!t.nbytes || !host_ptrs[t.slot]) continue;
-        if (t.nbytes >= STAGE_MIN) {
+    if (up) {
+        size_t total = 0;
+        for (auto& t : s->uploads) if (t.nbytes && host_ptrs[t.slot]) total += t.nbytes;
+        if (total >= STAGE_MIN) {
+            // all arguments as one stream of chunks: a few threads stage them, this one hands each chunk to the
+            // DMA engine as soon as it is staged
+            std::vector<UploadPiece> pieces;
+            for (auto& t : s->uploads)
+                if (t.nbytes && host_ptrs[t.slot])
+                    pieces.push_back({(char*)t.staging, (const char*)host_ptrs[t.slot], (char*)t.buf->dptr + t.offset, t.nbytes});
             hipError_t err = hipSuccess;
-            const int r = staged_upload((char*)t.staging, (const char*)host_ptrs[t.slot], t.nbytes, [&](size_t off, size_t len) {
-                err = hipMemcpyAsync((char*)t.buf->dptr + t.offset + off, (char*)t.staging + off, len, hipMemcpyHostToDevice, c->stream);
+            const int r = staged_upload_pieces(pieces, [&](char* device, const char* staging, size_t len) {
+                err = hipMemcpyAsync(device, staging, len, hipMemcpyHostToDevice, c->stream);
                 return err == hipSuccess ? 0 : 1;
             });
             if (r) return hip_fail(err, "hipMemcpyAsync (staged upload)");
-            continue;
+        } else {
+            for (auto& t : s->uploads) {
+                if (!t.nbytes || !host_ptrs[t.slot]) continue;
+                memcpy(t.staging, host_ptrs[t.slot], t.nbytes);
+                HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
+            }
         }
-        memcpy(t.staging, host_ptrs[t.slot], t.nbytes);
-        HIP_TRY(hipMemcpyAsync((char*)t.buf->dptr + t.offset, t.staging, t.nbytes, hipMemcpyHostToDevice, c->stream));
     }
     if (s->profiling) HIP_TRY(hipEventRecord(s->stamps[1], c->stream));
     // With a fixed landing region nothing is allocated: the following arguments are staged in the
