@@ -127,6 +127,7 @@ def test_every_tile_and_loader_variant(tile, bk):
         for variant, (xs, ks) in cases.items():
             for general in (True, False):
                 K.FORCE_CONV_GENERAL = general
+                K.FORCE_CONV_B_GENERAL = variant[1] == 'g'           #(a dense kernel operand takes 16-byte loads whatever its width)
                 expected = variant[:2] if general or variant not in ('ff2', 'ff3') else 'lean'
                 print(f'tile {tile} bk {bk} loaders {variant} -> {expected}', flush=True)
                 x = rng.randint(-4, 5, size=xs).astype(np.float32)
@@ -136,7 +137,7 @@ def test_every_tile_and_loader_variant(tile, bk):
                 assert kernel == f'conv_gemm_{tile}x{bk}_{expected}', kernel
     finally:
         K.FORCE_CONV_TILE = K.FORCE_CONV_BK = None
-        K.FORCE_CONV_GENERAL = False
+        K.FORCE_CONV_GENERAL = K.FORCE_CONV_B_GENERAL = False
 
 
 @pytest.mark.parametrize('tile,bk', TILES)
@@ -202,12 +203,15 @@ def test_four_waves_per_tile_kernel():
     K.FORCE_CONV_KSPLIT = True
     try:
         for f, args in cases:
-            print(f'four waves per tile: {f.__name__} {[a.shape for a in args]}', flush=True)
-            _, _, fn = check_against_oracle(f, args, exact=True)
-            launches = list(fn._jaxpr_interpreters.values())[0].launches
-            assert [l.kernel for l in launches] in (['conv_gemm_32x32x128_ks4'], ['conv_gemm_32x32x128_ks4g']), [l.kernel for l in launches]
+            for b_general in (False, True):
+                K.FORCE_CONV_B_GENERAL = b_general
+                print(f'four waves per tile: {f.__name__} {[a.shape for a in args]} element-wise kernel loads {b_general}', flush=True)
+                _, _, fn = check_against_oracle(f, args, exact=True)
+                launches = list(fn._jaxpr_interpreters.values())[0].launches
+                assert [l.kernel for l in launches] == ['conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4'], [l.kernel for l in launches]
     finally:
         K.FORCE_CONV_KSPLIT = None
+        K.FORCE_CONV_B_GENERAL = False
 
 
 def test_mixed_tiling():

@@ -36,8 +36,7 @@ def _mixed_tiling_case(rng, ints):
         args = [x, k, ints(-5, 5, cout), ints(1, 4, cout), ints(-9, 9, cout), ints(-50, 50, b, ho, wo, cout)]
     forced = dict(FORCE_CONV_TILE='64x64', FORCE_CONV_BK=int(rng.choice([32, 64])), FORCE_CONV_CHUNK=1, FORCE_CONV_KSPLIT=False,
                   FORCE_CONV_MIX=int(rng.randint(1, max(2, m // 64 + 1))))
-    #(an output width that is no multiple of 4 takes the element-wise kernel loader and with it the general kernel)
-    return f, args, forced, 'conv_gemm' if cout % 4 else '_mix' if forced['FORCE_CONV_MIX'] * 64 < m else '_lean'
+    return f, args, forced, '_mix' if forced['FORCE_CONV_MIX'] * 64 < m else '_lean'
 
 
 def _stem_case(rng, ints):

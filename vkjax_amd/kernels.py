@@ -425,6 +425,7 @@ FORCE_CONV_TILE: tp.Optional[str] = None
 FORCE_CONV_BK:   tp.Optional[int] = None
 FORCE_CONV_CHUNK: tp.Optional[int] = None
 FORCE_CONV_GENERAL = False          #never pick the lean kernel variant
+FORCE_CONV_B_GENERAL = False        #element-wise loads of the kernel operand also where 16-byte loads would do
 FORCE_CONV_KSPLIT: tp.Optional[bool] = None    #the four-waves-per-tile kernel: always (where it applies) / never
 FORCE_CONV_MIX = None               #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
 
@@ -603,7 +604,10 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0 and g.PH >= 0 and g.PW >= 0
               and all(s % 4 == 0 and s >= 0 for s in g.xs[:3]) and (not needs_masks or g.KH * g.KW <= 32)
               and (lhs.size - lhs_offset) * 4 + x_bias <= 2**31)
-    b_fast = (g.ws[3] == 1 and N % 4 == 0 and rhs_offset % 4 == 0
+    #16-byte loads of the kernel operand need a dense [ky, kx, in, out] array, not an output width that is a multiple of 4:
+    #a buffer load of four words only has to start at a word (verified on gfx950 with integer-exact products of odd
+    #widths); the words a vector reads beyond its row belong to columns >= N, which are never stored
+    b_fast = (g.ws[3] == 1 and rhs_offset % 4 == 0 and not FORCE_CONV_B_GENERAL
               and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
     c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
     slots = _epilogue_template_slots(epilogue)
