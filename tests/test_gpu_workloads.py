@@ -199,6 +199,36 @@ def test_fusion_does_not_change_a_single_bit():
         assert_tree_close(a, b, exact=True, what=getattr(f, '__name__', 'f'))
 
 
+def test_softmax_with_its_argmax_in_one_launch():
+    '''softmax over rows followed by the arg-max of the probabilities becomes one launch; probabilities and labels
+    equal the unfused program's bit for bit, with ties (first occurrence), NaN rows (the first NaN), rows of equal
+    values, -inf entries, row lengths below and above one pass of a wave, and labels that are also a result when the
+    probabilities are not.'''
+    rng = np.random.default_rng(5)
+    def probabilities_and_labels(x):
+        p = mj.nn.softmax(x, axis=-1)
+        return p, mj.numpy.argmax(p, axis=1)
+    def labels_only(x):
+        return mj.numpy.argmax(mj.nn.softmax(x, axis=-1), axis=1)
+    for rows, cols in ((256, 10), (7, 1), (33, 64), (5, 200), (4, 1000)):
+        x = rng.standard_normal((rows, cols)).astype(np.float32)
+        x[0, :] = 0.5                                             #all equal: label 0
+        if cols > 3:
+            x[1, 2], x[1, cols - 1] = 9.0, 9.0                    #a tie: the first
+            x[2, cols // 2] = np.nan                              #NaN probabilities in the whole row: label 0
+            x[3 % rows, 0] = -np.inf
+        for f in (probabilities_and_labels, labels_only):
+            fused   = vkjax_amd.wrap(f, frontend='minijax', fuse=True)
+            unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)
+            a, b = fused(x), unfused(x)
+            kernels = [l.kernel for l in list(fused._jaxpr_interpreters.values())[0].launches]
+            #rows of one value have nothing to reduce: no softmax kernel is involved there
+            assert cols == 1 or (len(kernels) == 1 and kernels[0].startswith('softmax_rows')), (kernels, rows, cols)
+            assert_tree_close(a, b, exact=True, what=f'{f.__name__} {rows}x{cols}')
+            labels = a[1] if isinstance(a, tuple) else a
+            assert labels[0] == 0 and (cols <= 3 or labels[1] == 2)
+
+
 def test_return_all_and_profiling():
     '''The debugging surface of the reference: run(..., return_all=True) returns every variable
     (reference: vkjax/kompute_jaxpr_interpreter.py:85-89) and profiling=True returns per-op timings

@@ -361,6 +361,28 @@ def test_size_limits_are_reported_when_the_program_is_built():
     assert interp.launches[0].kernel.startswith('conv_gemm')
 
 
+def test_softmax_plan_keeps_every_result_of_the_fused_launch():
+    '''softmax over rows with the arg-max of the probabilities plans as ONE launch with three buffers (probabilities,
+    input, labels), also when only the labels are returned: the launch is alive through its second result.'''
+    from vkjax_amd import minijax as mj
+    from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
+    def both(x):
+        p = mj.nn.softmax(x, axis=-1)
+        return p, mj.numpy.argmax(p, axis=1)
+    def labels_only(x):
+        return mj.numpy.argmax(mj.nn.softmax(x, axis=-1), axis=1)
+    x = np.zeros((33, 64), np.float32)
+    for f in (both, labels_only):
+        interp = JaxprInterpreter(mj.make_jaxpr(f)(x), plan_only=True)
+        assert [l.kernel for l in interp.launches] == ['softmax_rows_v4']
+        buffers = [b for b, _ in interp.launches[0].buffers]
+        assert len(buffers) == 3 and all(b is not None and b.tensor is not None for b in buffers)
+        assert buffers[2] is interp.output_buffers[-1] and buffers[2].dtype == 'int32'
+    #softmax alone: the labels argument is absent
+    interp = JaxprInterpreter(mj.make_jaxpr(lambda v: mj.nn.softmax(v, axis=-1))(x), plan_only=True)
+    assert [l.kernel for l in interp.launches] == ['softmax_rows_v4'] and interp.launches[0].buffers[2][0] is None
+
+
 # ------------------------------------------------------------------ boundary details
 
 def test_reference_module_path_resolves():

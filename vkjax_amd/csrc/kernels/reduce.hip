@@ -457,8 +457,11 @@ __device__ __forceinline__ float row_sum_as_reduce_rows(F value_at, uint32_t R, 
     return a;
 }
 
+// `arg_out` (may be null): the index of each result row's largest value as reduce_rows_fargmax would report it
+// (first occurrence, a NaN wins), for programs that take the arg-max of the probabilities right away.
 template <int VEC>
-__device__ __forceinline__ void softmax_rows_body(float* __restrict__ out, const float* __restrict__ in, const SoftmaxParams& P) {
+__device__ __forceinline__ void softmax_rows_body(float* __restrict__ out, const float* __restrict__ in, uint32_t* __restrict__ arg_out,
+                                                  const SoftmaxParams& P) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (row >= P.outer) return;                                       // whole wave leaves together
@@ -469,15 +472,37 @@ __device__ __forceinline__ void softmax_rows_body(float* __restrict__ out, const
 #pragma unroll
     for (int s = 32; s >= 1; s >>= 1) { const float o = __shfl_xor(m, s, 64); m = (m > o || m != m) ? m : o; }
     const float total = row_sum_as_reduce_rows<VEC>([&](uint32_t r) { return expf(x[r] - m); }, P.R, lane);
-    for (uint32_t r = lane; r < P.R; r += 64u) y[r] = expf(x[r] - m) / total;
+    uint32_t best_v = 0, best_i = 0xFFFFFFFFu;
+    for (uint32_t r = lane; r < P.R; r += 64u) {
+        const float p = expf(x[r] - m) / total;
+        y[r] = p;
+        // a lane meets its elements in ascending order: on a tie the earlier one stays; a NaN replaces any number
+        const float q = u2f(best_v);
+        const bool better = p > q || (p != p && q == q) || best_i == 0xFFFFFFFFu;
+        best_v = better ? f2u(p) : best_v;
+        best_i = better ? r : best_i;
+    }
+    if (arg_out == nullptr) return;
+    // across the lanes as in reduce_rows: the maximum of (rank of the value, complement of the index)
+    const uint32_t flipped = best_v ^ ((best_v >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+    const float    bv      = u2f(best_v);
+    uint64_t key = best_i == 0xFFFFFFFFu ? 0ull : ((uint64_t)(bv != bv ? 0xFFFFFFFFu : flipped) << 32 | (uint32_t)~best_i);
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        const uint64_t other = __shfl_xor(key, s, 64);
+        key = other > key ? other : key;
+    }
+    if (lane == 0) arg_out[row] = key == 0ull ? 0u : ~(uint32_t)key;
 }
 
-extern "C" __global__ __launch_bounds__(256) void softmax_rows_v1(float* __restrict__ out, const float* __restrict__ in, SoftmaxParams P) {
-    softmax_rows_body<1>(out, in, P);
+extern "C" __global__ __launch_bounds__(256) void softmax_rows_v1(float* __restrict__ out, const float* __restrict__ in, uint32_t* __restrict__ arg_out,
+                                                                  SoftmaxParams P) {
+    softmax_rows_body<1>(out, in, arg_out, P);
 }
 // R % 4 == 0: the summation order of the 16-byte reduce_rows kernel
-extern "C" __global__ __launch_bounds__(256) void softmax_rows_v4(float* __restrict__ out, const float* __restrict__ in, SoftmaxParams P) {
-    softmax_rows_body<4>(out, in, P);
+extern "C" __global__ __launch_bounds__(256) void softmax_rows_v4(float* __restrict__ out, const float* __restrict__ in, uint32_t* __restrict__ arg_out,
+                                                                  SoftmaxParams P) {
+    softmax_rows_body<4>(out, in, arg_out, P);
 }
 
 struct ReduceGeneralParams {

@@ -52,6 +52,8 @@ def _reads(op) -> tp.List:
             return list(op.meta[2])
         if op.meta[0] in ('random_stream', 'reduce'):
             return [b for b, _ in op.launch.buffers[1:] if b is not None]
+        if op.meta[0] == 'softmax':
+            return [op.meta[2]]
     return [b for b, _ in op.launch.buffers if b is not None]
 
 
@@ -320,13 +322,23 @@ def fuse_softmax(ops, bufferpool, outvars):
                 or c2.steps[0].operand.buffer._placeholder is not s._placeholder or not per_row(c2.steps[0].operand, c2.shape)
                 or uses[pid(m)] != 1 or uses[pid(c1.out)] != 2 or uses[pid(s)] != 1):
             continue
-        fused = Op(_label(R1, C1, R2, C2), launch=K.softmax_rows(c2.out, x, outer, rows))
-        fused.index = C2.index
-        x.accesses.append(C2.index)
+        members, last, arg_out = (R1, C1, R2, C2), C2, None
+        #the arg-max over the same rows of the probabilities, right behind them: one more result of the same launch
+        A = ops[i + 4] if i + 4 < len(ops) else None
+        if (A is not None and A.meta is not None and A.meta[0] == 'reduce' and A.meta[6] == 'argmax' and A.meta[8] == 1
+                and A.meta[2]._placeholder is c2.out._placeholder and tuple(A.meta[3:6]) == (outer, rows, 1) and A.meta[1].dtype == 'int32'):
+            members, last, arg_out = (R1, C1, R2, C2, A), A, A.meta[1]
+            removed.add(i + 3)
+        fused = Op(_label(*members), launch=K.softmax_rows(c2.out, x, outer, rows, arg_out),
+                   meta=('softmax', [c2.out] + ([arg_out] if arg_out is not None else []), x))
+        fused.index = last.index
+        x.accesses.append(last.index)
+        if arg_out is not None:
+            c2.out.accesses.append(last.index)
         for b in (m, c1.out, s):
             b._placeholder.elided = True
         removed |= {i, i + 1, i + 2}
-        replacement[i + 3] = fused
+        replacement[i + 3 + (arg_out is not None)] = fused
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
 
 
@@ -618,7 +630,7 @@ def _writes(op) -> tp.List:
         return [_out(op)]
     if op.meta is not None and op.meta[0] in ('iota', 'concat_part'):
         return [op.meta[1]]
-    if op.meta is not None and op.meta[0] == 'threefry':
+    if op.meta is not None and op.meta[0] in ('threefry', 'softmax'):
         return list(op.meta[1])
     return [b for b, _ in op.launch.buffers[:1] if b is not None]      #kernels write their first argument
 
@@ -794,7 +806,7 @@ def _small_out(op):
 
 def _may_write(op) -> tp.List:
     '''Buffers an op may change: its result where the op's structure is known, else everything it touches.'''
-    if op.chain is not None or op.conv is not None or (op.meta is not None and op.meta[0] in ('iota', 'concat_part', 'threefry', 'reduce')):
+    if op.chain is not None or op.conv is not None or (op.meta is not None and op.meta[0] in ('iota', 'concat_part', 'threefry', 'reduce', 'softmax')):
         return _writes(op)
     return [b for b, _ in op.launch.buffers if b is not None]
 

@@ -762,12 +762,13 @@ def scale_relu_backward(column_sum: Launch, dx: Buffer, sum_m: Buffer, sum_mx: B
 SOFTMAX_MAX_ROW = 4096      #rows this short run unsplit in reduce_rows, whose summation order softmax_rows repeats
 
 
-def softmax_rows(out: Buffer, inp: Buffer, outer: int, R: int) -> Launch:
-    '''exp(x - max) / sum(exp(x - max)) over the rows of [outer, R]; see softmax_rows_body in reduce.hip.'''
-    assert 0 < R < SOFTMAX_MAX_ROW and inp.size == out.size == outer * R
+def softmax_rows(out: Buffer, inp: Buffer, outer: int, R: int, arg_out: tp.Optional[Buffer] = None) -> Launch:
+    '''exp(x - max) / sum(exp(x - max)) over the rows of [outer, R]; see softmax_rows_body in reduce.hip.
+    `arg_out`: also the arg-max of every result row (int32 [outer]).'''
+    assert 0 < R < SOFTMAX_MAX_ROW and inp.size == out.size == outer * R and (arg_out is None or arg_out.size == outer)
     vec = 4 if R % 4 == 0 else 1
-    return Launch(f'softmax_rows_v{vec}', (_cdiv(outer, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], _u32(outer, R),
-                  bytes_moved=8 * outer * R)
+    return Launch(f'softmax_rows_v{vec}', (_cdiv(outer, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0), (arg_out, 0)], _u32(outer, R),
+                  bytes_moved=8 * outer * R + (4 * outer if arg_out is not None else 0))
 
 
 def reduce_general(out: Buffer, inp: Buffer, kept, reduced, op: str) -> Launch:
