@@ -200,7 +200,7 @@ def test_four_waves_per_tile_kernel():
              (plain, [ints(-4, 5, 40, 388), ints(-2, 3, 388, 7)]),
              (bn_res_relu, [ints(-4, 5, 2, 9, 7, 128), ints(-3, 4, 1, 1, 128, 72), ints(-5, 5, 72), ints(1, 4, 72), ints(-9, 9, 72), ints(-50, 50, 2, 9, 7, 72)]),
              (bn_res_relu, [ints(-4, 5, 2, 9, 7, 256), ints(-3, 4, 3, 3, 256, 40), ints(-5, 5, 40), ints(1, 4, 40), ints(-9, 9, 40), ints(-50, 50, 2, 9, 7, 40)])]
-    K.FORCE_CONV_KSPLIT = True
+    K.FORCE_CONV_KSPLIT, K.FORCE_CONV_K_SPLITS = True, 1
     try:
         for f, args in cases:
             for b_general in (False, True):
@@ -210,8 +210,54 @@ def test_four_waves_per_tile_kernel():
                 launches = list(fn._jaxpr_interpreters.values())[0].launches
                 assert [l.kernel for l in launches] == ['conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4'], [l.kernel for l in launches]
     finally:
-        K.FORCE_CONV_KSPLIT = None
+        K.FORCE_CONV_KSPLIT = K.FORCE_CONV_K_SPLITS = None
         K.FORCE_CONV_B_GENERAL = False
+
+
+def test_sliced_contractions():
+    '''Products with few tiles and a long contraction: blocks of their own sum slices of the contraction (2, 3, 4 and
+    7 slices, also slices of unequal length and a last k step that is not full) into one matrix per slice, and an
+    element-wise launch adds the slices and applies what follows the product. Dense layers, a 1x1 and padded 3x3
+    convolutions whose later slices start at another kernel tap, with bias + ReLU, a batch-norm + residual + ReLU
+    chain and nothing behind them; row counts that do not fill the last tile; both loaders of the kernel operand;
+    integer-valued data, so every result is exact. The heuristic slices the layers it is meant for.'''
+    from vkjax_amd import kernels as K
+    from vkjax_amd import minijax as mj
+    lax, nn, jnp = mj.lax, mj.nn, mj.numpy
+    dn = ('NHWC', 'HWIO', 'NHWC')
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+
+    def dense(x, w, b): return nn.relu(jnp.dot(x, w) + b)
+    def plain(x, w): return jnp.dot(x, w)
+    def bn_res_relu(x, k, mean, scale, beta, res):
+        y = lax.conv_general_dilated(x, k, (1, 1), 'SAME', dimension_numbers=dn)
+        return nn.relu((y - mean) * scale + beta + res)
+
+    cases = [(dense, [ints(-4, 5, 49, 1024), ints(-3, 4, 1024, 96), ints(-9, 9, 96)]),
+             (plain, [ints(-4, 5, 70, 900), ints(-2, 3, 900, 36)]),
+             (plain, [ints(-4, 5, 33, 1300), ints(-2, 3, 1300, 7)]),
+             (bn_res_relu, [ints(-4, 5, 1, 7, 7, 512), ints(-3, 4, 1, 1, 512, 72), ints(-5, 5, 72), ints(1, 4, 72), ints(-9, 9, 72), ints(-50, 50, 1, 7, 7, 72)]),
+             (bn_res_relu, [ints(-4, 5, 1, 7, 7, 128), ints(-3, 4, 3, 3, 128, 40), ints(-5, 5, 40), ints(1, 4, 40), ints(-9, 9, 40), ints(-50, 50, 1, 7, 7, 40)]),
+             (bn_res_relu, [ints(-4, 5, 2, 5, 6, 256), ints(-3, 4, 3, 3, 256, 33), ints(-5, 5, 33), ints(1, 4, 33), ints(-9, 9, 33), ints(-50, 50, 2, 5, 6, 33)])]
+    K.FORCE_CONV_KSPLIT = True
+    try:
+        for f, args in cases:
+            for slices in (2, 3, 4, 7):
+                for b_general in (False, True):
+                    K.FORCE_CONV_K_SPLITS, K.FORCE_CONV_B_GENERAL = slices, b_general
+                    print(f'sliced contraction: {f.__name__} {[a.shape for a in args]} {slices} slices, element-wise kernel loads {b_general}', flush=True)
+                    _, _, fn = check_against_oracle(f, args, exact=True)
+                    launches = list(fn._jaxpr_interpreters.values())[0].launches
+                    assert launches[0].kernel == ('conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4')
+                    assert launches[0].buffers[0][0].shape[0] > 1 and all(l.kernel.startswith('ew_chain') for l in launches[1:]), [l.kernel for l in launches]
+    finally:
+        K.FORCE_CONV_KSPLIT = K.FORCE_CONV_K_SPLITS = None
+        K.FORCE_CONV_B_GENERAL = False
+    #by the heuristic: a 3x3 layer of a network's last stage on one image (32 tiles, 36 k steps), against float data
+    x, k = rng.randn(1, 7, 7, 512).astype(np.float32), (rng.randn(3, 3, 512, 512) / 68).astype(np.float32)
+    _, _, fn = check_against_oracle(lambda a, b: nn.relu(lax.conv_general_dilated(a, b, (1, 1), 'SAME', dimension_numbers=dn)), [x, k], rtol=1e-4, atol=1e-5)
+    launches = list(fn._jaxpr_interpreters.values())[0].launches
+    assert [l.kernel for l in launches][0] == 'conv_gemm_32x32x128_ks4' and launches[0].grid == (128, 1, 1) and len(launches) == 2
 
 
 def test_mixed_tiling():

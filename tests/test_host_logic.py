@@ -333,12 +333,48 @@ def test_batch_of_one_fuses_like_any_other():
     chains from joining each other or a convolution's epilogue.'''
     import vkjax_amd
     from vkjax_amd import workloads as W
+    from vkjax_amd import kernels as K
     counts = []
-    for batch in (1, 2):
-        fn = vkjax_amd.wrap(W.resnet50, frontend='minijax', plan_only=True)
-        interp, _ = fn._get_or_create_jaxpr_interpreter(tuple(W.resnet50_inputs(batch=batch, size=64, num_classes=40, width_scale=0.25)))
-        counts.append(len(interp.launches))
+    K.FORCE_CONV_K_SPLITS = 1                  #(a sliced contraction would add a launch of its own)
+    try:
+        for batch in (1, 2):
+            fn = vkjax_amd.wrap(W.resnet50, frontend='minijax', plan_only=True)
+            interp, _ = fn._get_or_create_jaxpr_interpreter(tuple(W.resnet50_inputs(batch=batch, size=64, num_classes=40, width_scale=0.25)))
+            counts.append(len(interp.launches))
+    finally:
+        K.FORCE_CONV_K_SPLITS = None
     assert counts[0] == counts[1] == 58, counts
+
+
+def test_long_contractions_of_few_tiles_are_sliced():
+    '''A product with few 32 x 32 tiles and a long contraction is planned as a launch that sums up to four slices of
+    the contraction into a temporary (one [M, N] matrix per slice, blocks = tiles x slices) followed by an element-wise
+    launch that adds the slices in order and takes over the equations behind the product. Products with many tiles or
+    short contractions are planned as before.'''
+    import vkjax_amd
+    from vkjax_amd import minijax as mj, kernels as K
+    from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
+    def layer(x, w, b):
+        return mj.nn.relu(mj.numpy.dot(x, w) + b)
+    def plan(m, k, n, **kw):
+        args = (np.zeros((m, k), np.float32), np.zeros((k, n), np.float32), np.zeros((n,), np.float32))
+        return JaxprInterpreter(mj.make_jaxpr(layer)(*args), plan_only=True, **kw)
+    interp = plan(49, 4608, 512)                                   #2 x 16 tiles, 36 k steps
+    assert [l.kernel for l in interp.launches] == ['conv_gemm_32x32x128_ks4', 'ew_chain_v4_s6']
+    first, second = interp.launches
+    assert first.grid == (32 * 4, 1, 1) and first.buffers[0][0].shape == (4, 49 * 512)
+    assert np.frombuffer(first.params, np.int32)[-1 - 9] == 9      #k steps per slice: the last word before the 9 of ConvDerived
+    assert second.buffers[0][0] is interp.output_buffers[0]
+    assert len(plan(49, 4608, 512, fuse=False).launches) == 4      #slices, their sum, add, max
+    assert [l.kernel for l in plan(49, 640, 512).launches] == ['conv_gemm_32x32x128_ks4']        #5 k steps: too short to slice
+    assert [l.kernel for l in plan(49, 1024, 512).launches][0] == 'conv_gemm_32x32x128_ks4' and plan(49, 1024, 512).launches[0].grid == (64, 1, 1)
+    assert len(plan(2048, 4608, 512).launches) == 1                #1024 tiles
+    K.FORCE_CONV_K_SPLITS = 3
+    try:
+        forced = plan(40, 1000, 24)                                #8 k steps in 3 slices of 3, 3 and 2
+        assert forced.launches[0].grid == (2 * 3, 1, 1) and forced.launches[0].buffers[0][0].shape == (3, 40 * 24)
+    finally:
+        K.FORCE_CONV_K_SPLITS = None
 
 
 def test_size_limits_are_reported_when_the_program_is_built():

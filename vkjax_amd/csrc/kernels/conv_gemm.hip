@@ -75,6 +75,9 @@ struct ConvParams {
     int32_t os_b, os_h, os_w, os_n; // out strides
     int32_t split_tiles_m;          // mixed kernels only: the first split_tiles_m M tiles (of 64 rows) are computed as 64 x 64
                                     // tiles, the rows behind them as 32 x 32 tiles by the blocks that follow in the grid
+    int32_t k_split_steps;          // four-waves-per-tile kernels only: 0, or the k steps (of 128) one block sums. The grid then holds
+                                    // ceil(k steps / k_split_steps) blocks per tile; those of slice s store their sums, without an
+                                    // epilogue, to the s-th [M, N] matrix behind out, and a later launch adds the slices
 };
 
 // The part of the output a block's tile number refers to: a grid of tiles_m x tiles_n tiles whose first row is
@@ -181,6 +184,20 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     const int chunk = LEAN ? (P.flags >> 25) & 15u : 1;         // the general variants take one tile per block
     const int chunks_m = (region.tiles_m + chunk - 1) / chunk;
     int work = (int)blockIdx.x - region.first_block;
+    // K_SPLIT kernels can share a tile's contraction among several blocks (for products with so few tiles that most
+    // CUs would stay idle while a few fetch all the weights): slice s sums k steps [kbase, kbase + ktiles)
+    constexpr bool K_SPLIT = KSW > 1 && BK == 128;
+    int kbase = 0, ktiles = max(1, (P.K + BK - 1) / BK);       // K = 0 runs as one k step whose loads are all out of range
+    if constexpr (K_SPLIT) {
+        const int per = Pk.k_split_steps;
+        if (per > 0) {
+            const int tiles = chunks_m * region.tiles_n, slice = work / tiles;
+            work -= slice * tiles;
+            kbase = slice * per;
+            ktiles = min(per, ktiles - kbase);
+            out += (size_t)slice * (size_t)P.M * (size_t)P.N;
+        }
+    }
     {
         const int total = chunks_m * region.tiles_n, per = total / 8;
         if (per > 0 && work < per * 8) work = (work & 7) * per + (work >> 3);
@@ -311,6 +328,12 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             }
         }
         t_r = 0; t_s = 0; t_c = 0;
+        if constexpr (K_SPLIT) {
+            if (kbase > 0) {                          // a later slice of the contraction starts at its own tap and feature
+                const int k0 = kbase * BK, rs = k0 / P.Cin;
+                t_c = k0 - rs * P.Cin; t_r = rs / P.KW; t_s = rs - t_r * P.KW;
+            }
+        }
         ak = A_FAST ? a_kv * 4 : (tid / BM) * A_KPT;
         const int rs = ak / P.Cin;
         ac = ak - rs * P.Cin; ar = rs / P.KW; as_ = rs - ar * P.KW;
@@ -463,11 +486,9 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     };
 
     float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
-    // K = 0 runs as one k step whose loads are all out of range
-    const int ktiles = max(1, (P.K + BK - 1) / BK);
     setup_rows(region.m_base + tile_m0 * BM);
     CONV_STAMP(1)
-    load_tiles(0);
+    load_tiles(kbase * BK);
     if (tid < BN) {
 #pragma unroll
         for (int e = 0; e < CONV_MAX_EPI; ++e)
@@ -516,17 +537,17 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             // Two k steps of loads in flight per wave, the stages alternating (written out twice: the stage is a
             // compile-time index into the registers). The waves meet once, behind the first store, which also
             // publishes the epilogue operands parked in LDS, and again before the reduction reuses the tiles.
-            if (ktiles > 1) load_tiles(BK, 1);
+            if (ktiles > 1) load_tiles((kbase + 1) * BK, 1);
             for (int kt = 0; kt < ktiles; kt += 2) {
                 store_tiles(0);
                 if (kt == 0) __syncthreads(); else tile_barrier();
-                if (kt + 2 < ktiles) load_tiles((kt + 2) * BK, 0);
+                if (kt + 2 < ktiles) load_tiles((kbase + kt + 2) * BK, 0);
                 compute();
                 tile_barrier();
                 if (kt + 1 < ktiles) {
                     store_tiles(1);
                     tile_barrier();
-                    if (kt + 3 < ktiles) load_tiles((kt + 3) * BK, 1);
+                    if (kt + 3 < ktiles) load_tiles((kbase + kt + 3) * BK, 1);
                     compute();
                     tile_barrier();
                 }
@@ -537,7 +558,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             for (int kt = 1; kt < ktiles; ++kt) {
                 store_tiles();
                 tile_barrier();
-                load_tiles(kt * BK);
+                load_tiles((kbase + kt) * BK);
 #ifdef CONV_PHASE_STAMPS
                 if (kt == 1 && sub == 0) { CONV_STAMP(2) }
 #endif
@@ -550,7 +571,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             __syncthreads();                 // (also where wave-private tiles publish the epilogue operands parked in LDS)
             if (sub + 1 < nsub) {
                 setup_rows(m0 + BM);
-                load_tiles(0);
+                load_tiles(kbase * BK);
             }
             if (first_full >= 0) {
 #pragma unroll

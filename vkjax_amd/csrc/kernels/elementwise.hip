@@ -43,24 +43,32 @@ struct EwParams {
 template <int VEC, int NS, bool PIN = true>
 __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const uint32_t* const (&in)[EW_MAX_STEPS],
                                               const EwParams& P, const uint32_t block) {
+    // All fields are read first and pinned afterwards: an inline-asm statement is a boundary for the instruction
+    // scheduler, and loads issued behind the first pin would wait for a second round trip to the argument block.
     uint32_t n = P.n, ndim = P.ndim, nsteps = P.nsteps;
     uint32_t dims[4], op[NS], flags[NS], imm[NS], nbytes[NS], base[NS];
     int32_t  stride[NS][4];
-    EW_PIN(n); EW_PIN(ndim); EW_PIN(nsteps);
     uint32_t dim_magic[4], dim_shift[4];
 #pragma unroll
+    for (int d = 0; d < 4; ++d) { dims[d] = P.dims[d]; dim_magic[d] = P.dim_magic[d]; dim_shift[d] = P.dim_shift[d]; }
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+        flags[k] = P.flags[k]; nbytes[k] = P.nbytes[k]; base[k] = P.base[k];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) stride[k][d] = P.stride[k][d];
+    }
+    EW_PIN(n); EW_PIN(ndim); EW_PIN(nsteps);
+#pragma unroll
     for (int d = 0; d < 4; ++d) {
-        dims[d] = P.dims[d]; dim_magic[d] = P.dim_magic[d]; dim_shift[d] = P.dim_shift[d];
         EW_PIN(dims[d]);
         if (d >= 1) { EW_PIN(dim_magic[d]); EW_PIN(dim_shift[d]); }
     }
 #pragma unroll
     for (int k = 0; k < NS; ++k) {
-        flags[k] = P.flags[k]; nbytes[k] = P.nbytes[k]; base[k] = P.base[k];
         EW_PIN(flags[k]); EW_PIN(nbytes[k]); EW_PIN(base[k]);
         if constexpr (PIN && NS <= 6) asm volatile("" :: "s"(in[k]));
 #pragma unroll
-        for (int d = 0; d < 4; ++d) { stride[k][d] = P.stride[k][d]; EW_PIN(stride[k][d]); }
+        for (int d = 0; d < 4; ++d) EW_PIN(stride[k][d]);
     }
 
     // A thread works on U vectors, 256 vectors apart (so that a wave's loads stay contiguous). All
@@ -74,7 +82,9 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     // Every operand is read through a buffer descriptor with one branch-free load per slot: 16 bytes
     // (of which only the first dword is used where the operand is constant along the vector), or
     // nothing at all for an empty slot, whose descriptor has size 0.
-    uint32_t vals[NS][W];
+    // (what a load returns is looked at only after all loads of all vectors have been requested: a use in between
+    // would wait for the load in flight and serialise all that follow)
+    u32x4 raw[NS][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint32_t i0 = first + u * 256u * VEC;
@@ -114,25 +124,10 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
         };
 #pragma unroll
         for (int k = 0; k < NS; ++k) {
-            if (u > 0 && (flags[k] & 64u)) {
-                // a single value, or a vector over the fastest dimension whose length divides the distance
-                // between a thread's vectors: what the thread's first vector loaded serves the others too
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) vals[k][u * VEC + j] = vals[k][j];
-                continue;
-            }
             const uint32_t idx = operand_index(k);
             const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, (int)nbytes[k], 0x00020000);
-            if constexpr (VEC == 4) {
-                const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 4u, 0, 0);
-                const bool is_vec = (flags[k] & 4u) != 0;
-                vals[k][u * 4 + 0] = t.x;
-                vals[k][u * 4 + 1] = is_vec ? t.y : t.x;
-                vals[k][u * 4 + 2] = is_vec ? t.z : t.x;
-                vals[k][u * 4 + 3] = is_vec ? t.w : t.x;
-            } else {
-                vals[k][u] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, idx * 4u, 0, 0);
-            }
+            if constexpr (VEC == 4) raw[k][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 4u, 0, 0);
+            else                    raw[k][u].x = __builtin_amdgcn_raw_buffer_load_b32(rsrc, idx * 4u, 0, 0);
         }
     }
 
@@ -140,6 +135,23 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
 #pragma unroll
     for (int k = 0; k < NS; ++k) { op[k] = P.op[k]; imm[k] = P.imm[k]; EW_PIN(op[k]); EW_PIN(imm[k]); }
 
+    uint32_t vals[NS][W];
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+        const bool is_vec = (flags[k] & 4u) != 0;          // else one value per vector: its first word
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const u32x4 t = raw[k][u];
+            if constexpr (VEC == 4) {
+                vals[k][u * 4 + 0] = t.x;
+                vals[k][u * 4 + 1] = is_vec ? t.y : t.x;
+                vals[k][u * 4 + 2] = is_vec ? t.z : t.x;
+                vals[k][u * 4 + 3] = is_vec ? t.w : t.x;
+            } else {
+                vals[k][u] = t.x;
+            }
+        }
+    }
     uint32_t acc[W];
 #pragma unroll
     for (int j = 0; j < W; ++j) acc[j] = vals[0][j];
@@ -177,12 +189,29 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     }
 }
 
+// Requests one word of every 64-byte line of the argument block at the very start of a kernel and waits for all of
+// them at once. The fields are fetched where the compiler needs them, in several dependent groups; a group that
+// touches a line for the first time waits for a round trip to memory (about 1600 cycles), later ones find their
+// line in the scalar cache. For a launch of a few waves those round trips are most of its duration.
+template <int BYTES>
+__device__ __forceinline__ void ew_touch_arguments() {
+    static_assert(BYTES > 384 && BYTES <= 448, "seven lines");
+    const char* args = reinterpret_cast<const char*>(__builtin_amdgcn_kernarg_segment_ptr());
+    uint32_t w0, w1, w2, w3, w4, w5, w6;
+    // one statement: the requests, then the wait (the compiler does not track loads issued by inline assembly)
+    asm volatile("s_load_dword %0, %7, 0x0\n\ts_load_dword %1, %7, 0x40\n\ts_load_dword %2, %7, 0x80\n\t"
+                 "s_load_dword %3, %7, 0xc0\n\ts_load_dword %4, %7, 0x100\n\ts_load_dword %5, %7, 0x140\n\t"
+                 "s_load_dword %6, %7, 0x180\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(w0), "=&s"(w1), "=&s"(w2), "=&s"(w3), "=&s"(w4), "=&s"(w5), "=&s"(w6) : "s"(args) : "memory");
+}
+
 #define EW_KERNEL(name, VEC, NS)                                                                      \
     extern "C" __global__ __launch_bounds__(256) void name(                                            \
         uint32_t* __restrict__ out, const uint32_t* in0, const uint32_t* in1, const uint32_t* in2,      \
         const uint32_t* in3, const uint32_t* in4, const uint32_t* in5, const uint32_t* in6,             \
         const uint32_t* in7, EwParams P) {                                                              \
         const uint32_t* const in[EW_MAX_STEPS] = {in0, in1, in2, in3, in4, in5, in6, in7};              \
+        ew_touch_arguments<sizeof(EwParams) + 9 * sizeof(void*)>();                                     \
         ew_chain_body<VEC, NS>(out, in, P, blockIdx.x);                                                 \
     }
 

@@ -236,7 +236,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
                 if uses[pid] != 1:
                     #a convolution whose result something else reads as well can still take the chain over,
                     #by storing both: its result as it was, and the chain's
-                    if prod.conv is not None and _out(prod)._placeholder is cand.buffer._placeholder:
+                    if prod.conv is not None and prod.conv[3].k_splits == 1 and _out(prod)._placeholder is cand.buffer._placeholder:
                         fused = conv_with_second_result(prod, op, pid)
                         if fused is not None:
                             result[pos] = None
@@ -252,7 +252,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
                     fused = Op(_label(prod, op), chain=chain)
                 else:
                     out, lhs, rhs, geom, epilogue = prod.conv
-                    if tuple(out.shape) != tuple(op.chain.shape) or len(epilogue) + len(steps) > K.CONV_MAX_EPI:
+                    if geom.k_splits > 1 or tuple(out.shape) != tuple(op.chain.shape) or len(epilogue) + len(steps) > K.CONV_MAX_EPI:
                         continue
                     extra = _epilogue_steps(steps, geom, op.chain.shape)
                     if extra is None:

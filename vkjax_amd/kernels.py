@@ -335,6 +335,9 @@ class ConvGeometry(tp.NamedTuple):
     xs: tp.Tuple[int, int, int, int] = (0, 0, 0, 1)      #lhs strides: batch, y, x, feature
     ws: tp.Tuple[int, int, int, int] = (0, 0, 0, 1)      #rhs strides: ky, kx, in feature, out feature
     os: tp.Tuple[int, int, int, int] = (0, 0, 0, 1)      #out strides: batch, y, x, feature
+    #> 1: the contraction is cut into this many slices, each summed by blocks of its own into its own [M, N] matrix of
+    #the result array (no epilogue); another launch adds the slices
+    k_splits: int = 1
 
     @property
     def M(self): return self.batch * self.Ho * self.Wo
@@ -574,6 +577,63 @@ def _conv_derived(epilogue, N):
     return derived_ptrs, derived_desc
 
 
+def _conv_fast_paths(lhs: Buffer, rhs: Buffer, g: ConvGeometry, lhs_offset: int = 0, rhs_offset: int = 0):
+    '''(needs_masks, x_bias, a_fast, b_fast, c_contig) of a flattened geometry: which loaders and stores apply.'''
+    N = g.N
+    #some kernel tap of some output position falls outside the input (padding, or a window that overhangs)
+    needs_masks = (g.PH > 0 or g.PW > 0 or (g.Ho - 1) * g.SH - g.PH + (g.KH - 1) * g.DH >= g.H
+                   or (g.Wo - 1) * g.SW - g.PW + (g.KW - 1) * g.DW >= g.W)
+    #the 16-byte A path keeps the validity of a row's taps in one 32-bit mask and addresses the
+    #input from (PH, PW) positions before its start
+    x_bias = (g.PH * g.xs[1] + g.PW * g.xs[2]) * 4
+    #(negative padding, i.e. cropping, goes through the generic loader's coordinate checks)
+    a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0 and g.PH >= 0 and g.PW >= 0
+              and all(s % 4 == 0 and s >= 0 for s in g.xs[:3]) and (not needs_masks or g.KH * g.KW <= 32)
+              and (lhs.size - lhs_offset) * 4 + x_bias <= 2**31)
+    #16-byte loads of the kernel operand need a dense [ky, kx, in, out] array, not an output width that is a multiple of 4:
+    #a buffer load of four words only has to start at a word (verified on gfx950 with integer-exact products of odd
+    #widths); the words a vector reads beyond its row belong to columns >= N, which are never stored
+    b_fast = (g.ws[3] == 1 and rhs_offset % 4 == 0 and not FORCE_CONV_B_GENERAL
+              and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
+    c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
+    return needs_masks, x_bias, a_fast, b_fast, c_contig
+
+
+def _four_waves_per_tile(g: ConvGeometry, a_fast: bool, c_contig: bool, compute_units: int) -> bool:
+    '''A product with so few 32 x 32 tiles that one wave per tile leaves most MFMA units idle: four waves per tile,
+    each taking a quarter of every (128-long) k step.'''
+    want = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
+            (_cdiv(g.M, 32) * _cdiv(g.N, 32) <= 2 * compute_units and g.K >= 256 and FORCE_CONV_TILE is None and FORCE_CONV_BK is None))
+    return bool(want) and a_fast and c_contig and (g.Cin % 128 == 0 or g.KH * g.KW == 1) and not FORCE_CONV_GENERAL
+
+
+#tests: the number of slices a contraction is cut into where that applies (None: by the heuristic, 1: never)
+FORCE_CONV_K_SPLITS: tp.Optional[int] = None
+
+
+def conv_k_splits(lhs: Buffer, rhs: Buffer, g: ConvGeometry, compute_units: int = 256) -> int:
+    '''Into how many slices the contraction of a product with very few tiles is cut (1: not at all). With 32 blocks on
+    256 CUs, a layer whose kernel operand is megabytes long (the 3 x 3 layers of a network's last stages at batch 1)
+    is bound by the rate at which those few CUs fetch it; slices spread the fetch over the chip. Every slice keeps at
+    least four k steps, at most four slices (the launch that adds them is an element-wise chain with room for a
+    following scale, shift and ReLU), and never more blocks than CUs.'''
+    g = _flatten_pointwise(g)
+    if g.K * g.N * 4 >= 2**31 or lhs.size * 4 >= 2**31 or g.M * g.N == 0:
+        return 1
+    _, _, a_fast, _, c_contig = _conv_fast_paths(lhs, rhs, g)
+    if not _four_waves_per_tile(g, a_fast, c_contig, compute_units):
+        return 1
+    tiles, ksteps = _cdiv(g.M, 32) * _cdiv(g.N, 32), _cdiv(g.K, 128)
+    if FORCE_CONV_K_SPLITS is not None:
+        want = FORCE_CONV_K_SPLITS
+    else:
+        want = min(4, compute_units // tiles, ksteps // 4)
+    if want <= 1 or ksteps < 2:
+        return 1
+    per = _cdiv(ksteps, min(want, ksteps))
+    return _cdiv(ksteps, per)
+
+
 def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: tp.Sequence[ConvEpilogueStep] = (),
               compute_units: int = 256, lhs_offset: int = 0, rhs_offset: int = 0, out_offset: int = 0) -> Launch:
     taps = [(i, e.operand) for i, e in enumerate(epilogue) if e.op == CONV_TAP]
@@ -594,22 +654,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
         return stem
     tag, bm, bn, nt = choose_conv_tile(M, N, compute_units)
     bk = choose_conv_bk(tag, g)
-    #some kernel tap of some output position falls outside the input (padding, or a window that overhangs)
-    needs_masks = (g.PH > 0 or g.PW > 0 or (g.Ho - 1) * g.SH - g.PH + (g.KH - 1) * g.DH >= g.H
-                   or (g.Wo - 1) * g.SW - g.PW + (g.KW - 1) * g.DW >= g.W)
-    #the 16-byte A path keeps the validity of a row's taps in one 32-bit mask and addresses the
-    #input from (PH, PW) positions before its start
-    x_bias = (g.PH * g.xs[1] + g.PW * g.xs[2]) * 4
-    #(negative padding, i.e. cropping, goes through the generic loader's coordinate checks)
-    a_fast = (g.xs[3] == 1 and g.Cin % 4 == 0 and g.LH == 1 and g.LW == 1 and lhs_offset % 4 == 0 and g.PH >= 0 and g.PW >= 0
-              and all(s % 4 == 0 and s >= 0 for s in g.xs[:3]) and (not needs_masks or g.KH * g.KW <= 32)
-              and (lhs.size - lhs_offset) * 4 + x_bias <= 2**31)
-    #16-byte loads of the kernel operand need a dense [ky, kx, in, out] array, not an output width that is a multiple of 4:
-    #a buffer load of four words only has to start at a word (verified on gfx950 with integer-exact products of odd
-    #widths); the words a vector reads beyond its row belong to columns >= N, which are never stored
-    b_fast = (g.ws[3] == 1 and rhs_offset % 4 == 0 and not FORCE_CONV_B_GENERAL
-              and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
-    c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
+    needs_masks, x_bias, a_fast, b_fast, c_contig = _conv_fast_paths(lhs, rhs, g, lhs_offset, rhs_offset)
     slots = _epilogue_template_slots(epilogue)
     #the lean kernel variant covers the common case only (see the kernel source)
     lean = (a_fast and b_fast and c_contig and (g.Cin % bk == 0 or g.KH * g.KW == 1)
@@ -619,13 +664,16 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     flat_rows = g.batch == 1 and g.Wo == 1 and g.SH == 1 and g.PH == 0 and g.PW == 0 and not needs_masks
     #a product with so few 32 x 32 tiles that one wave per tile leaves most MFMA units idle: four waves per
     #tile, each taking a quarter of every (128-long) k step
-    ksplit = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
-              (_cdiv(M, 32) * _cdiv(N, 32) <= 2 * compute_units and K >= 256 and FORCE_CONV_TILE is None and FORCE_CONV_BK is None))
-    ksplit = bool(ksplit) and a_fast and c_contig and (g.Cin % 128 == 0 or g.KH * g.KW == 1) \
-        and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL
+    ksplit = _four_waves_per_tile(g, a_fast, c_contig, compute_units) and (not epilogue or slots != 0)
     if ksplit:
         tag, bm, bn, nt, bk, lean = '32x32', 32, 32, 256, 128, True
     tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
+    k_split_steps = 0
+    if g.k_splits > 1:
+        k_split_steps = _cdiv(_cdiv(K, 128), g.k_splits)
+        if (not ksplit or epilogue or taps or out_offset or out.size != g.k_splits * M * N
+                or _cdiv(_cdiv(K, 128), k_split_steps) != g.k_splits):
+            raise ValueError('a sliced contraction needs the four-waves-per-tile kernel, no epilogue and one [M, N] matrix per non-empty slice')
     chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean and not ksplit else 1
     #64 x 64 tiles that do not divide evenly among the CUs: as many M tiles as fill every CU equally stay 64 x 64, the
     #rows behind them are computed as 32 x 32 tiles with four waves per tile (a quarter of the work each)
@@ -649,8 +697,10 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
         descs[i // 3] |= ((e.op * 2 + int(e.operand_left)) | e.kind << 8) << (10 * (i % 3))
     params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, g.DH, g.DW,
                    *g.xs[:3], tiles_m, tiles_n)
-              + _u32(flags, *descs, x_bytes, w_bytes, (out.size - out_offset) * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
-              + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os, split_tiles_m))
+              #(rows beyond M are dropped by the descriptor's size: with slices, that of one slice's matrix)
+              + _u32(flags, *descs, x_bytes, w_bytes, M * N * 4 if k_split_steps else (out.size - out_offset) * 4,
+                     *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
+              + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os, split_tiles_m, k_split_steps))
     derived_ptrs, derived_desc = _conv_derived(epilogue, N)
     params += derived_desc
     buffers = [(out, out_offset * 4), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
@@ -662,7 +712,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     kernel  = f'conv_gemm_{tag}x{bk}_' + (('ks4' if b_fast else 'ks4g') if ksplit else 'lean' if lean else ('f' if a_fast else 'g') + ('f' if b_fast else 'g'))
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
     nbytes += 4 * tap_buffer.size if taps else 0
-    blocks = _cdiv(tiles_m, chunk) * tiles_n
+    blocks = _cdiv(tiles_m, chunk) * tiles_n * max(1, g.k_splits)
     if split_tiles_m:
         kernel = f'conv_gemm_{tag}x{bk}_mix'
         blocks = split_tiles_m * tiles_n + _cdiv(M - split_tiles_m * 64, 32) * _cdiv(N, 32)

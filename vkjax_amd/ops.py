@@ -522,6 +522,23 @@ def _wgrad_ops(bufferpool, equation, outbuf, x, cot, wg: 'K.WgradGeometry'):
     return [Op(equation, launch=l) for l in launches]
 
 
+def _product_ops(bufferpool, equation, outbuf, lhs, rhs, geom: 'K.ConvGeometry'):
+    '''The implicit-GEMM launch of a convolution or matrix product; for a product with very few output tiles and a
+    long contraction, a launch that sums slices of the contraction into a temporary and an element-wise launch that
+    adds the slices in order (which later takes over the element-wise equations that follow).'''
+    splits = K.conv_k_splits(lhs, rhs, geom)
+    if splits <= 1:
+        return [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+    position = bufferpool.op_counter
+    bufferpool.op_counter -= 1                  #the temporary lives at the equation's own position
+    partial = bufferpool.new_temporary(np.float32, (splits, outbuf.size))
+    bufferpool.op_counter = position
+    strides = K.row_major_strides(outbuf.shape)
+    slices  = [K.EwOperand(partial, s * outbuf.size, strides) for s in range(splits)]
+    total   = K.EwChain(outbuf, outbuf.shape, slices[0], [K.EwStep(K.EW['ADD_F'], o) for o in slices[1:]])
+    return [Op(equation, conv=(partial, lhs, rhs, geom._replace(k_splits=splits), [])), Op(equation, chain=total)]
+
+
 def dot_general(bufferpool, equation):
     '''2-D x 2-D, one contracting dimension per side, no batch dimensions, float32
     (reference: vkjax/ops.py:277-297). Lowered onto the implicit-GEMM kernel with a 1x1 window.'''
@@ -552,7 +569,7 @@ def dot_general(bufferpool, equation):
                           ws=(rst[rc[0]] * Kc, rst[rc[0]] * Kc, rst[rc[0]], rst[1 - rc[0]]),
                           os=(M * N, N, N, 1))
     ops, rhs, geom, _ = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
-    return ops + [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+    return ops + _product_ops(bufferpool, equation, outbuf, lhs, rhs, geom)
 
 
 def conv_general_dilated(bufferpool, equation):
@@ -593,7 +610,7 @@ def conv_general_dilated(bufferpool, equation):
     if (geom.LH > 1 or geom.LW > 1) and geom.SH == geom.SW == 1 and geom.DH == geom.DW == 1:
         return _dilated_input_convolution(bufferpool, equation, outbuf, lhs, rhs, geom)
     ops, rhs, geom, _ = _with_dense_kernel(bufferpool, equation, rhs, geom, lhs, outbuf)
-    return ops + [Op(equation, conv=(outbuf, lhs, rhs, geom, []))]
+    return ops + _product_ops(bufferpool, equation, outbuf, lhs, rhs, geom)
 
 
 def _with_dense_kernel(bufferpool, equation, rhs: Buffer, geom: 'K.ConvGeometry', lhs: Buffer, outbuf: Buffer, rhs_offset: int = 0):
