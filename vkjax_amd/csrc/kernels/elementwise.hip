@@ -125,7 +125,11 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
 #pragma unroll
         for (int k = 0; k < NS; ++k) {
             const uint32_t idx = operand_index(k);
-            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, (int)nbytes[k], 0x00020000);
+            // a single value, or a vector over the fastest dimension whose length divides the distance between a thread's
+            // vectors: what the thread's first vector loads serves the others too. Their loads go through a descriptor
+            // of size 0, which returns zeros without touching memory, so that every vector issues the same instructions.
+            const int readable = (u > 0 && (flags[k] & 64u)) ? 0 : (int)nbytes[k];
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, readable, 0x00020000);
             if constexpr (VEC == 4) raw[k][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 4u, 0, 0);
             else                    raw[k][u].x = __builtin_amdgcn_raw_buffer_load_b32(rsrc, idx * 4u, 0, 0);
         }
@@ -139,9 +143,14 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
 #pragma unroll
     for (int k = 0; k < NS; ++k) {
         const bool is_vec = (flags[k] & 4u) != 0;          // else one value per vector: its first word
+        const bool shared = (flags[k] & 64u) != 0;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const u32x4 t = raw[k][u];
+            u32x4 t = raw[k][u];
+            if (u > 0) {
+                t.x = shared ? raw[k][0].x : t.x; t.y = shared ? raw[k][0].y : t.y;
+                t.z = shared ? raw[k][0].z : t.z; t.w = shared ? raw[k][0].w : t.w;
+            }
             if constexpr (VEC == 4) {
                 vals[k][u * 4 + 0] = t.x;
                 vals[k][u * 4 + 1] = is_vec ? t.y : t.x;
