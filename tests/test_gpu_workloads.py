@@ -229,6 +229,64 @@ def test_softmax_with_its_argmax_in_one_launch():
             assert labels[0] == 0 and (cols <= 3 or labels[1] == 2)
 
 
+def test_products_with_few_output_features():
+    '''dense_rows_n16: one wave per row on the vector ALUs for products with at most 16 output features. Every width
+    from 1 to 16, contractions of one vector, several passes and a last pass that is not full, one row and row counts
+    that do not fill a workgroup; bias, bias + ReLU, scale and shift, nothing; integer-valued data, so every result is
+    exact against the oracle. Followed by softmax (and the arg-max of the probabilities) the whole layer is ONE
+    launch whose probabilities and labels equal the unfused program's bit for bit: ties, NaN and infinite logits, a
+    single class. 17 features go to the matrix-core kernels.'''
+    rng = np.random.default_rng(12)
+    ints = lambda lo, hi, *shape: rng.integers(lo, hi, size=shape).astype(np.float32)
+    def plain(x, w): return mj.numpy.dot(x, w)
+    def bias(x, w, b): return mj.numpy.dot(x, w) + b
+    def bias_relu(x, w, b): return mj.nn.relu(mj.numpy.dot(x, w) + b)
+    def scale_shift(x, w, m, s, b): return (mj.numpy.dot(x, w) - m) * s + b
+    shapes = [(256, 512, 10), (1, 4, 1), (3, 8, 2), (5, 252, 3), (4, 256, 4), (7, 260, 5), (33, 516, 6), (2, 784, 7), (65, 1028, 8),
+              (9, 64, 9), (130, 300, 11), (6, 1024, 12), (17, 2052, 13), (40, 128, 14), (3, 388, 15), (100, 768, 16)]
+    for rows, k, n in shapes:
+        x, w = ints(-4, 5, rows, k), ints(-3, 4, k, n)
+        for f, extra in ((plain, []), (bias, [ints(-9, 9, n)]), (bias_relu, [ints(-9, 9, n)]),
+                         (scale_shift, [ints(-5, 5, n), ints(1, 4, n), ints(-9, 9, n)])):
+            _, _, fn = check_against_oracle(f, [x, w] + extra, exact=True)
+            kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+            #(with one output feature a per-feature vector is a single value, which the general epilogue handles)
+            assert kernels == ['dense_rows_n16'] or (n == 1 and f is not plain), (kernels, f.__name__, rows, k, n)
+    _, _, fn = check_against_oracle(plain, [ints(-4, 5, 40, 256), ints(-3, 4, 256, 17)], exact=True)
+    assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] != ['dense_rows_n16']
+
+    def head(x, w, b):
+        p = mj.nn.softmax(mj.numpy.dot(x, w) + b, axis=-1)
+        return p, mj.numpy.argmax(p, axis=1)
+    def head_probabilities(x, w, b):
+        return mj.nn.softmax(mj.numpy.dot(x, w) + b, axis=-1)
+    def head_relu_labels(x, w, b):
+        return mj.numpy.argmax(mj.nn.softmax(mj.nn.relu(mj.numpy.dot(x, w) + b), axis=-1), axis=1)
+    for rows, k, classes in [(256, 512, 10), (7, 256, 12)] + [(9, 64, c) for c in range(1, 17)] + [(40, 256, 17)]:
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        w = (rng.standard_normal((k, classes)) / np.sqrt(k)).astype(np.float32)
+        b = rng.standard_normal(classes).astype(np.float32)
+        x[0, :] = 0.0                                             #logits = bias
+        if classes > 1:
+            w[:, 1] = w[:, 0]; b[1] = b[0]                        #classes 0 and 1 tie in every row
+        x[2, 5] = np.nan                                          #a row of NaN logits
+        x[3, 7] = np.inf                                          #logits +-inf (or NaN) in row 3
+        for f in (head, head_probabilities, head_relu_labels):
+            fused   = vkjax_amd.wrap(f, frontend='minijax', fuse=True)
+            unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)
+            a, c = fused(x, w, b), unfused(x, w, b)
+            kernels = [l.kernel for l in list(fused._jaxpr_interpreters.values())[0].launches]
+            if 1 < classes <= 16:
+                assert kernels == ['dense_rows_n16'], (kernels, rows, k, classes)
+            elif classes > 16:
+                assert len(kernels) == 2 and kernels[1].startswith('softmax_rows'), kernels
+            assert_tree_close(a, c, exact=True, what=f'{f.__name__} {rows}x{k}x{classes}')
+    #against the oracle
+    check_against_oracle(head, [rng.standard_normal((256, 512)).astype(np.float32),
+                                (rng.standard_normal((512, 10)) / 23).astype(np.float32), rng.standard_normal(10).astype(np.float32)],
+                         rtol=1e-4, atol=1e-6)
+
+
 def test_return_all_and_profiling():
     '''The debugging surface of the reference: run(..., return_all=True) returns every variable
     (reference: vkjax/kompute_jaxpr_interpreter.py:85-89) and profiling=True returns per-op timings

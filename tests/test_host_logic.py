@@ -80,11 +80,13 @@ def test_kernel_argument_layouts_match_the_structs():
     b = lambda *shape: Buffer(None, f32, shape)
     i = lambda *shape: Buffer(None, np.dtype('int32'), shape)
     chain = K.EwChain(b(4, 8), (4, 8), K.broadcast_operand(b(4, 8), (4, 8)), [K.EwStep(K.EW['ADD_F'], K.broadcast_operand(b(8), (4, 8)))])
-    geom  = K.ConvGeometry(batch=1, Ho=4, Wo=4, N=8, H=4, W=4, Cin=4, KH=1, KW=1, xs=(64, 16, 4, 1), ws=(32, 32, 8, 1), os=(128, 32, 8, 1))
+    geom  = K.ConvGeometry(batch=1, Ho=4, Wo=4, N=24, H=4, W=4, Cin=4, KH=1, KW=1, xs=(64, 16, 4, 1), ws=(96, 96, 24, 1), os=(384, 96, 24, 1))
+    few   = K.ConvGeometry(batch=1, Ho=16, Wo=1, N=8, H=16, W=1, Cin=4, KH=1, KW=1, xs=(0, 4, 0, 1), ws=(32, 32, 8, 1), os=(128, 8, 8, 1))
     G, S = core.GatherDimensionNumbers, core.ScatterDimensionNumbers
     launches = {
         'EwParams': K.lower_ew_chain(chain), 'IotaParams': K.iota(i(8), 0), 'FillParams': K.fill(b(8), 0),
-        'ConcatParams': K.concat_part(b(4, 8), b(4, 3), 1, 0), 'ConvParams': K.conv_gemm(b(1, 4, 4, 8), b(1, 4, 4, 4), b(1, 1, 4, 8), geom),
+        'ConcatParams': K.concat_part(b(4, 8), b(4, 3), 1, 0), 'ConvParams': K.conv_gemm(b(1, 4, 4, 24), b(1, 4, 4, 4), b(1, 1, 4, 24), geom),
+        'DenseRowsParams': K.conv_gemm(b(16, 8), b(16, 4), b(4, 8), few),
         'ConvStemParams': K.conv_gemm(b(1, 64, 64, 8), b(1, 128, 128, 3), b(7, 7, 3, 8),
                                       K.ConvGeometry(batch=1, Ho=64, Wo=64, N=8, H=128, W=128, Cin=3, KH=7, KW=7, SH=2, SW=2, PH=3, PW=3,
                                                      xs=(128 * 384, 384, 3, 1), ws=(168, 24, 8, 1), os=(64 * 512, 512, 8, 1))),
@@ -108,7 +110,8 @@ def test_kernel_argument_layouts_match_the_structs():
     #the convolution kernel takes two parameter structs, one after the other
     sizes['ConvParams'] += sizes['ConvDerived']
     sizes['ConvStemParams'] += sizes['ConvDerived']
-    assert launches['ConvStemParams'].kernel == 'conv_gemm_stem_7x22'
+    assert launches['ConvStemParams'].kernel == 'conv_gemm_stem_7x22' and launches['DenseRowsParams'].kernel == 'dense_rows_n16'
+    assert len(launches['DenseRowsParams'].buffers) == 3 + K.CONV_MAX_EPI
     for struct, launch in launches.items():
         assert len(launch.params) == sizes[struct], (struct, len(launch.params), sizes[struct])
     assert sizes['ConvEpiPtrs'] == 8 * K.CONV_MAX_EPI and sizes['ThreefryStreamPtrs'] == 8 * K.TF_MAX_STEPS

@@ -1017,3 +1017,138 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     __shared__ float Es[CONV_MAX_EPI * 64];
     conv_stem_body<7, 22, 9, 6>(out, x, w, epi, dp, P, D, Ws, Ps, Es);
 }
+
+// ---------------------------------------------------------------------------------------------
+// Products with at most 16 output features (a classifier's last layer): out = x [M, K] . w [K, N], one wave per
+// row of x, on the vector ALUs. A 32-column MFMA tile would be mostly padding, and for the few rows of a small
+// batch the launch is all latency: this kernel runs a few hundred instructions per wave, all its loads are in
+// flight together, and the softmax (and arg-max) that usually follows can run on the row before it is stored.
+//
+// Lane l multiplies x[row][k] for k = 4l .. 4l+3 (+ 256, + 512, ...) with the rows k of w, which are 4N consecutive
+// floats, into N running sums with fused multiply-adds, in ascending k; the lanes' sums are then added by a
+// butterfly (xor 32, 16, ..., 1), so that every lane holds all N results. Epilogue: the steps of the straight-line
+// epilogue of conv_gemm_body that take a per-feature vector or a single value; then, with bit 29 of the flags, the
+// softmax of the row exactly as softmax_rows_v1 / _v4 computes it for a row of N values (the maximum, exp(x - max)
+// added in the order of the row-sum kernel, one division per value), and, if the last pointer slot is not null,
+// the arg-max of the probabilities (first occurrence; a NaN wins).
+// Needs K % 4 == 0, rows of x that start at multiples of 4 floats, dense w and out; the host checks.
+struct DenseRowsParams {
+    int32_t M, N, K;
+    int32_t x_pitch;                // floats between two rows of x
+    uint32_t flags;                 // bits 20-22 and 24: template epilogue steps as in ConvParams.flags; bit 29: softmax
+    uint32_t x_bytes, w_bytes, out_bytes;
+};
+
+template <int N>
+__device__ __forceinline__ void dense_rows_body(float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+                                                const ConvEpiPtrs& epi, const DenseRowsParams& P) {
+    const int lane = threadIdx.x & 63, row = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+    if (row >= P.M) return;                                            // whole wave leaves together
+    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, P.x_bytes), w_rsrc = make_rsrc(w, P.w_bytes), o_rsrc = make_rsrc(out, P.out_bytes);
+    const uint32_t slots = (P.flags >> 20) & 31u;
+    const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u), e_max = __builtin_popcount(slots & 15u);
+    // epilogue operands: requested before the products, used after them
+    float o_sub[N], o_mul[N], o_add[N], o_max = 0.f;
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+        o_sub[n] = buffer_load_x1(make_rsrc(epi.p[0], (slots & 1u) ? (uint32_t)N * 4u : 0u), (uint32_t)n * 4u);
+        o_mul[n] = buffer_load_x1(make_rsrc(epi.p[e_mul], (slots & 2u) ? (uint32_t)N * 4u : 0u), (uint32_t)n * 4u);
+        o_add[n] = buffer_load_x1(make_rsrc(epi.p[e_add], (slots & 4u) ? (uint32_t)N * 4u : 0u), (uint32_t)n * 4u);
+    }
+    if (slots & 16u) o_max = buffer_load_x1(make_rsrc(epi.p[e_max], 4u), 0u);
+
+    float acc[N];
+#pragma unroll
+    for (int n = 0; n < N; ++n) acc[n] = 0.f;
+    const uint32_t xrow = (uint32_t)row * (uint32_t)P.x_pitch * 4u;
+    for (int k0 = 0; k0 < P.K; k0 += 512) {
+        f32x4 xv[2], wv[2][N];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int  k4 = k0 + u * 256 + lane * 4;
+            const bool in = k4 < P.K;                                  // beyond K: zeros, which leave the sums as they are
+            xv[u] = buffer_load_x4(x_rsrc, in ? xrow + (uint32_t)k4 * 4u : CONV_OOB);
+#pragma unroll
+            for (int j = 0; j < N; ++j) wv[u][j] = buffer_load_x4(w_rsrc, in ? (uint32_t)(k4 * N + 4 * j) * 4u : CONV_OOB);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int n = 0; n < N; ++n) acc[n] = __builtin_fmaf(xv[u][q], wv[u][(q * N + n) / 4][(q * N + n) % 4], acc[n]);
+    }
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        float o[N];
+#pragma unroll
+        for (int n = 0; n < N; ++n) o[n] = __shfl_xor(acc[n], s, 64);
+#pragma unroll
+        for (int n = 0; n < N; ++n) acc[n] = acc[n] + o[n];
+    }
+    float y[N];
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+        float v = acc[n];
+        if (slots & 1u) v = v - o_sub[n];
+        if (slots & 2u) v = v * o_mul[n];
+        if (slots & 4u) v = v + o_add[n];
+        if (slots & 16u) v = (v > o_max || v != v) ? v : o_max;
+        y[n] = v;
+    }
+    if (P.flags & (1u << 29)) {
+        float m = -INFINITY;                                           // a NaN wins
+#pragma unroll
+        for (int n = 0; n < N; ++n) m = (y[n] > m || y[n] != y[n]) ? y[n] : m;
+        float e[16];
+#pragma unroll
+        for (int n = 0; n < 16; ++n) e[n] = n < N ? expf(y[n < N ? n : 0] - m) : 0.f;
+        float total;
+        if constexpr (N % 4 == 0) {
+            // the 16-byte row-sum kernel: lane l holds (e[4l] + e[4l+1]) + (e[4l+2] + e[4l+3]), then lanes xor 2, xor 1
+            float a[4];
+#pragma unroll
+            for (int l = 0; l < 4; ++l) a[l] = (e[4 * l] + e[4 * l + 1]) + (e[4 * l + 2] + e[4 * l + 3]);
+            total = (a[0] + a[2]) + (a[1] + a[3]);
+        } else {
+            // the 4-byte row-sum kernel: lane l holds e[l], then lanes xor 8, 4, 2, 1 (xor 32 and 16 add zeros)
+            float a[16];
+#pragma unroll
+            for (int l = 0; l < 16; ++l) a[l] = e[l];
+#pragma unroll
+            for (int s = 8; s >= 1; s >>= 1)
+#pragma unroll
+                for (int l = 0; l < s; ++l) a[l] = a[l] + a[l + s];
+            total = a[0];
+        }
+#pragma unroll
+        for (int n = 0; n < N; ++n) y[n] = e[n] / total;
+        // arg-max: the first occurrence of the maximum; a NaN replaces any number and is never replaced
+        uint32_t best = 0;
+        float bv = y[0];
+#pragma unroll
+        for (int n = 1; n < N; ++n) {
+            const bool better = y[n] > bv || (y[n] != y[n] && bv == bv);
+            bv = better ? y[n] : bv;
+            best = better ? (uint32_t)n : best;
+        }
+        uint32_t* const arg_out = reinterpret_cast<uint32_t*>(const_cast<float*>(epi.p[CONV_MAX_EPI - 1]));
+        if (arg_out != nullptr && lane == 0) arg_out[row] = best;
+    }
+    float mine = 0.f;
+#pragma unroll
+    for (int n = 0; n < N; ++n) mine = lane == n ? y[n] : mine;
+    buffer_store_x1(mine, o_rsrc, lane < N ? (uint32_t)(row * N + lane) * 4u : CONV_OOB);
+}
+
+extern "C" __global__ __launch_bounds__(256) void dense_rows_n16(float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+                                                                ConvEpiPtrs epi, DenseRowsParams P) {
+    switch (P.N) {
+#define DENSE_ROWS_CASE(n) case n: dense_rows_body<n>(out, x, w, epi, P); break;
+        DENSE_ROWS_CASE(1) DENSE_ROWS_CASE(2) DENSE_ROWS_CASE(3) DENSE_ROWS_CASE(4) DENSE_ROWS_CASE(5) DENSE_ROWS_CASE(6)
+        DENSE_ROWS_CASE(7) DENSE_ROWS_CASE(8) DENSE_ROWS_CASE(9) DENSE_ROWS_CASE(10) DENSE_ROWS_CASE(11) DENSE_ROWS_CASE(12)
+        DENSE_ROWS_CASE(13) DENSE_ROWS_CASE(14) DENSE_ROWS_CASE(15) DENSE_ROWS_CASE(16)
+#undef DENSE_ROWS_CASE
+        default: break;
+    }
+}

@@ -38,7 +38,7 @@ def _reads(op) -> tp.List:
         return [o.buffer for o in op.chain.operands() if o is not None]
     if op.conv is not None:
         out, lhs, rhs, geom, epilogue = op.conv
-        reads = [lhs, rhs] + [e.operand for e in epilogue if e.operand is not None and e.op != K.CONV_TAP]
+        reads = [lhs, rhs] + [e.operand for e in epilogue if e.operand is not None and e.op not in (K.CONV_TAP, K.CONV_SOFTMAX)]
         for e in epilogue:
             if e.derived is not None:
                 reads += [e.derived.first] + [st[1] for st in e.derived.steps if st[1] is not None]
@@ -213,7 +213,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
         if steps is None or tuple(out.shape) != tuple(op.chain.shape) or op.chain.out.size != out.size:
             return None
         extra = _epilogue_steps(steps, geom, op.chain.shape)
-        if extra is None or not K.conv_tap_supported(epilogue, extra):
+        if extra is None or not K.conv_tap_supported(epilogue, extra) or K.conv_is_dense_rows(lhs, geom):
             return None
         tap = K.ConvEpilogueStep(K.CONV_TAP, 3, out)
         fused = Op(_label(prod, op), conv=(op.chain.out, lhs, rhs, geom, list(epilogue) + [tap] + extra))
@@ -257,6 +257,8 @@ def fuse_ops(all_ops, bufferpool, outvars):
                     extra = _epilogue_steps(steps, geom, op.chain.shape)
                     if extra is None:
                         continue
+                    if K.conv_is_dense_rows(lhs, geom) and not K.dense_rows_epilogue_supported(list(epilogue) + extra):
+                        continue                                  #the chain stays a launch of its own
                     tap_at = [k for k, e in enumerate(epilogue) if e.op == K.CONV_TAP]
                     if tap_at and not K.conv_tap_supported(epilogue[:tap_at[0]], list(epilogue[tap_at[0] + 1:]) + extra):
                         continue
@@ -280,6 +282,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
     ops = fuse_scale_relu_backward(ops, bufferpool, outvars)
     ops = fuse_reduce_prologues(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
+    ops = fuse_dense_softmax(ops, bufferpool, outvars)
     ops = remove_dead_ops(ops, bufferpool, outvars)
     return batch_small_chains(ops)
 
@@ -330,7 +333,7 @@ def fuse_softmax(ops, bufferpool, outvars):
             members, last, arg_out = (R1, C1, R2, C2, A), A, A.meta[1]
             removed.add(i + 3)
         fused = Op(_label(*members), launch=K.softmax_rows(c2.out, x, outer, rows, arg_out),
-                   meta=('softmax', [c2.out] + ([arg_out] if arg_out is not None else []), x))
+                   meta=('softmax', [c2.out] + ([arg_out] if arg_out is not None else []), x, outer, rows))
         fused.index = last.index
         x.accesses.append(last.index)
         if arg_out is not None:
@@ -339,6 +342,36 @@ def fuse_softmax(ops, bufferpool, outvars):
             b._placeholder.elided = True
         removed |= {i, i + 1, i + 2}
         replacement[i + 3 + (arg_out is not None)] = fused
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
+
+
+def fuse_dense_softmax(ops, bufferpool, outvars):
+    '''A classifier's last layer: a product with at most 16 output features, read by nothing but the softmax launch
+    right behind it, computes the softmax (and the arg-max that launch carries) on the row before it is stored
+    (dense_rows_n16). The exponentials are added in the order of the separate launch: same values, bit for bit.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    removed, replacement = set(), {}
+    for i, (D, S) in enumerate(zip(ops, ops[1:])):
+        if D.conv is None or S.meta is None or S.meta[0] != 'softmax':
+            continue
+        out, lhs, rhs, geom, epilogue = D.conv
+        _, results, x, outer, rows = S.meta
+        if (x._placeholder is not out._placeholder or uses[id(out._placeholder)] != 1 or (geom.M, geom.N) != (outer, rows)
+                or any(e.op in (K.CONV_TAP, K.CONV_SOFTMAX) for e in epilogue)):
+            continue
+        steps = list(epilogue) + [K.ConvEpilogueStep(K.CONV_SOFTMAX, 0, results[1] if len(results) > 1 else None)]
+        try:
+            K.conv_gemm(results[0], lhs, rhs, geom, steps)
+        except ValueError:
+            continue                                   #another kernel serves this product
+        fused = Op(_label(D, S), conv=(results[0], lhs, rhs, geom, steps))
+        fused.index = S.index
+        for b in _reads(D):
+            b.accesses.append(S.index)
+        out._placeholder.elided = True
+        removed.add(i)
+        replacement[i + 1] = fused
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
 
 
@@ -568,6 +601,8 @@ def fuse_derived_epilogue_operands(ops, bufferpool, outvars):
             continue
         out, lhs, rhs, geom, epilogue = op.conv
         N = geom.N
+        if K.conv_is_dense_rows(lhs, geom):
+            continue                                              #that kernel reads its epilogue operands as they are
         for ei, e in enumerate(epilogue):
             if e.kind != 2 or e.derived is not None or e.operand is None:
                 continue
@@ -625,7 +660,7 @@ def fuse_derived_epilogue_operands(ops, bufferpool, outvars):
 
 def _writes(op) -> tp.List:
     if op.conv is not None:
-        return [_out(op)] + [e.operand for e in op.conv[4] if e.op == K.CONV_TAP]
+        return [_out(op)] + [e.operand for e in op.conv[4] if e.op in (K.CONV_TAP, K.CONV_SOFTMAX) and e.operand is not None]
     if op.chain is not None:
         return [_out(op)]
     if op.meta is not None and op.meta[0] in ('iota', 'concat_part'):

@@ -400,6 +400,10 @@ class ConvEpilogueStep(tp.NamedTuple):
 #A pseudo step: the value as it stands at this point of the epilogue is ALSO stored to `operand`, an array laid
 #out like the result (the centred convolution result a backward pass needs besides the activation)
 CONV_TAP = -1
+#A pseudo step, the last of an epilogue: the rows of the result are replaced by their softmax before the store;
+#`operand`, if not None, is an int32 array [M] that receives each row's arg-max. Only the kernel for products with at
+#most 16 output features (dense_rows_n16) can do this.
+CONV_SOFTMAX = -2
 
 
 def conv_tap_supported(steps_before: tp.Sequence[ConvEpilogueStep], steps_after: tp.Sequence[ConvEpilogueStep]) -> bool:
@@ -430,6 +434,7 @@ FORCE_CONV_CHUNK: tp.Optional[int] = None
 FORCE_CONV_GENERAL = False          #never pick the lean kernel variant
 FORCE_CONV_B_GENERAL = False        #element-wise loads of the kernel operand also where 16-byte loads would do
 FORCE_CONV_KSPLIT: tp.Optional[bool] = None    #the four-waves-per-tile kernel: always (where it applies) / never
+FORCE_CONV_DENSE_ROWS = None        #the kernel for at most 16 output features: None = where it applies, False = never
 FORCE_CONV_MIX = None               #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
 
 
@@ -561,6 +566,56 @@ def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_
                   bytes_moved=nbytes, flops=2 * M * N * K)
 
 
+DENSE_ROWS_MAX_N = 16
+
+
+def _dense_rows_shape(lhs: Buffer, g: 'ConvGeometry') -> bool:
+    '''The operands of a product suit dense_rows_n16. `g` as the caller gave it: a matrix product, not a 1 x 1
+    convolution over a feature map (those keep the kernels whose epilogue takes a residual operand).'''
+    if (FORCE_CONV_DENSE_ROWS is False or FORCE_CONV_TILE is not None or FORCE_CONV_BK is not None or FORCE_CONV_GENERAL
+            or FORCE_CONV_KSPLIT is not None):
+        return False
+    M, N, K = g.M, g.N, g.K
+    flat = (g.batch == 1 and g.Wo == 1 and g.KH == g.KW == 1 and g.SH == 1 and g.PH == g.PW == 0 and g.LH == 1 and g.H == g.Ho
+            and g.xs[3] == 1 and g.xs[1] % 4 == 0 and g.xs[1] >= K)
+    return (flat and 1 <= N <= DENSE_ROWS_MAX_N and K % 4 == 0 and K > 0 and tuple(g.ws[2:]) == (N, 1) and tuple(g.os[1:]) == (N, N, 1)
+            and lhs.size * 4 < 2**31 and M * N * 4 < 2**31)
+
+
+def conv_is_dense_rows(lhs: Buffer, g: 'ConvGeometry') -> bool:
+    '''This product is computed by dense_rows_n16 whatever its epilogue: a fusion pass must not hand it an epilogue that
+    kernel cannot apply (another kernel would add the products in another order than in the unfused program).'''
+    return g.k_splits == 1 and _dense_rows_shape(lhs, g)
+
+
+def dense_rows_epilogue_supported(epilogue: tp.Sequence[ConvEpilogueStep]) -> bool:
+    real  = [e for e in epilogue if e.op != CONV_SOFTMAX]
+    slots = _epilogue_template_slots(real)
+    return (all(e.op != CONV_TAP and e.derived is None for e in real) and (not real or (slots != 0 and not slots & 8))
+            and all(e.op != CONV_SOFTMAX for e in epilogue[:-1]))
+
+
+def _dense_rows_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, lhs_offset, rhs_offset, out_offset,
+                       softmax: bool, arg_out: tp.Optional[Buffer]) -> tp.Optional[Launch]:
+    '''dense_rows_n16 where it applies: a matrix product (or 1x1 convolution over a dense array) with at most 16 output
+    features, a contraction that is a multiple of 4, dense operands, and an epilogue of per-feature and single-value
+    template steps; see the kernel.'''
+    if taps or lhs_offset or rhs_offset or out_offset or g.k_splits > 1:
+        return None
+    M, N, K = g.M, g.N, g.K
+    slots = _epilogue_template_slots(epilogue)
+    if not (_dense_rows_shape(lhs, g) and dense_rows_epilogue_supported(epilogue)):
+        return None
+    params  = _i32(M, N, K, g.xs[1]) + _u32(slots << 20 | int(softmax) << 29, lhs.size * 4, K * N * 4, M * N * 4)
+    slots_p = _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
+    if softmax:
+        slots_p[-1] = (arg_out, 0)
+    nbytes  = (4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
+               + (4 * arg_out.size if arg_out is not None else 0))
+    return Launch('dense_rows_n16', (_cdiv(M, 4), 1, 1), (256, 1, 1), [(out, 0), (lhs, 0), (rhs, 0)] + slots_p, params,
+                  bytes_moved=nbytes, flops=2 * M * N * K)
+
+
 def _conv_derived(epilogue, N):
     '''(pointer slots, descriptor words) of the one per-feature epilogue operand that the kernel computes itself.'''
     derived_ptrs, derived_desc = [(None, 0)] * (CONV_MAX_DERIVED + 1), _u32(*[0] * (3 + 2 * CONV_MAX_DERIVED))
@@ -617,6 +672,8 @@ def conv_k_splits(lhs: Buffer, rhs: Buffer, g: ConvGeometry, compute_units: int 
     is bound by the rate at which those few CUs fetch it; slices spread the fetch over the chip. Every slice keeps at
     least four k steps, at most four slices (the launch that adds them is an element-wise chain with room for a
     following scale, shift and ReLU), and never more blocks than CUs.'''
+    if _dense_rows_shape(lhs, g):
+        return 1
     g = _flatten_pointwise(g)
     if g.K * g.N * 4 >= 2**31 or lhs.size * 4 >= 2**31 or g.M * g.N == 0:
         return 1
@@ -642,13 +699,26 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
         epilogue = [e for e in epilogue if e.op != CONV_TAP]
         if (not conv_tap_supported(epilogue[:tap_position], epilogue[tap_position:]) or out_offset or tap_buffer.size != out.size):
             raise ValueError('a second result at this point of the epilogue is not supported')
+    softmax, arg_out = False, None
+    if epilogue and epilogue[-1].op == CONV_SOFTMAX:
+        softmax, arg_out = True, epilogue[-1].operand
+        epilogue = list(epilogue[:-1])
+        if len(epilogue) > CONV_MAX_EPI - 1 or (arg_out is not None and arg_out.size != g.M):
+            raise ValueError('softmax epilogue: too many steps, or labels of another size')
+    if any(e.op == CONV_SOFTMAX for e in epilogue):
+        raise ValueError('softmax can only be the last step of an epilogue')
     if len(epilogue) > CONV_MAX_EPI:
         raise ValueError('too many epilogue steps')
-    g = _flatten_pointwise(g)
+    g_given, g = g, _flatten_pointwise(g)
     M, N, K = g.M, g.N, g.K
     for name, extent in (('lhs', lhs.size), ('rhs', rhs.size), ('out', out.size)):
         if extent * 4 >= 2**31:
             raise NotImplementedError(f'conv/dot {name} operand of {extent * 4} bytes exceeds the 2 GiB the kernel addresses')
+    rows = _dense_rows_launch(out, lhs, rhs, g_given, epilogue, taps, lhs_offset, rhs_offset, out_offset, softmax, arg_out)
+    if rows is not None:
+        return rows
+    if softmax:
+        raise ValueError('softmax epilogue: only in the kernel for at most 16 output features')
     stem = _conv_stem_launch(out, lhs, rhs, g, epilogue, taps, compute_units, lhs_offset, rhs_offset, out_offset)
     if stem is not None:
         return stem
