@@ -249,7 +249,7 @@ def test_sliced_contractions():
                     _, _, fn = check_against_oracle(f, args, exact=True)
                     launches = list(fn._jaxpr_interpreters.values())[0].launches
                     assert launches[0].kernel == ('conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4')
-                    assert launches[0].buffers[0][0].shape[0] > 1 and all(l.kernel.startswith('ew_chain') for l in launches[1:]), [l.kernel for l in launches]
+                    assert launches[0].buffers[0][0].shape[0] > 1 and all(l.kernel.startswith(('ew_chain', 'ew_affine')) for l in launches[1:]), [l.kernel for l in launches]
     finally:
         K.FORCE_CONV_KSPLIT = K.FORCE_CONV_K_SPLITS = None
         K.FORCE_CONV_B_GENERAL = False

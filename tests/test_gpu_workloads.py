@@ -287,6 +287,57 @@ def test_products_with_few_output_features():
                          rtol=1e-4, atol=1e-6)
 
 
+def test_affine_chains_in_straight_line_code():
+    '''ew_affine_v4 evaluates ((first + s1 + s2 + s3) - vsub) * vmul + vadd + full, max(., floor) without the opcode
+    interpreter. Every subset of those parts, on 2-D, 4-D and (without vectors) 1-D arrays, gives the bits of the
+    general chain kernel, NaN and infinite values included, and agrees with the oracle.'''
+    import itertools
+    from vkjax_amd import kernels as K
+    rng = np.random.default_rng(21)
+    r = lambda *shape: rng.standard_normal(shape).astype(np.float32)
+    for shape in ((37, 24), (2, 5, 7, 64), (4100,)):
+        c = shape[-1]
+        first, s1, s2, s3, full = (r(*shape) for _ in range(5))
+        first.reshape(-1)[3] = np.nan; first.reshape(-1)[5] = np.inf; full.reshape(-1)[9] = -np.inf
+        vsub, vmul, vadd = r(c), r(c), r(c)
+        for nsum, parts in itertools.product(range(4), itertools.product((0, 1), repeat=5)):
+            if len(shape) == 1 and any(parts[:3]):
+                continue
+            if nsum == 0 and not any(parts):
+                continue
+            def f(first, s1, s2, s3, vsub, vmul, vadd, full):
+                v = first
+                for s in (s1, s2, s3)[:nsum]:
+                    v = v + s
+                if parts[0]: v = v - vsub
+                if parts[1]: v = v * vmul
+                if parts[2]: v = v + vadd
+                if parts[3]: v = v + full
+                if parts[4]: v = mj.nn.relu(v)
+                return v
+            args = [first, s1, s2, s3, vsub, vmul, vadd, full]
+            results = []
+            for forced in (True, False):
+                K.FORCE_EW_AFFINE = forced
+                try:
+                    fn = vkjax_amd.wrap(f, frontend='minijax')
+                    results.append(fn(*args))
+                    kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+                finally:
+                    K.FORCE_EW_AFFINE = None
+                #(nine operands are two launches: a chain holds eight)
+                assert all((k == 'ew_affine_v4') == forced for k in kernels) and len(kernels) <= 2, (kernels, forced, shape, nsum, parts)
+            assert_tree_close(results[0], results[1], exact=True, what=f'{shape} {nsum} {parts}')
+        check_against_oracle(lambda a, b, m, s, t, q: mj.nn.relu((a + b - m) * s + t + q), [first, s1, vsub, vmul, vadd, full][:6] if len(shape) > 1
+                             else [first, s1, np.float32(0.5), np.float32(2.0), np.float32(-1.0), full], rtol=1e-5, atol=1e-6)
+    #by itself: chains of more than four operands on arrays that are not large
+    x, m, k, t = r(64, 7, 7, 64), r(64), r(64), r(64)
+    _, _, fn = check_against_oracle(lambda x, m, k, t: mj.nn.relu((x - m) * k + t), [x, m, k, t], rtol=1e-5, atol=1e-6)
+    assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['ew_affine_v4']
+    _, _, fn = check_against_oracle(lambda x, m: mj.nn.relu(x - m), [x, m], rtol=1e-6)
+    assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['ew_chain_v4_s4']
+
+
 def test_return_all_and_profiling():
     '''The debugging surface of the reference: run(..., return_all=True) returns every variable
     (reference: vkjax/kompute_jaxpr_interpreter.py:85-89) and profiling=True returns per-op timings

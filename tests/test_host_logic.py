@@ -84,7 +84,8 @@ def test_kernel_argument_layouts_match_the_structs():
     few   = K.ConvGeometry(batch=1, Ho=16, Wo=1, N=8, H=16, W=1, Cin=4, KH=1, KW=1, xs=(0, 4, 0, 1), ws=(32, 32, 8, 1), os=(128, 8, 8, 1))
     G, S = core.GatherDimensionNumbers, core.ScatterDimensionNumbers
     launches = {
-        'EwParams': K.lower_ew_chain(chain), 'IotaParams': K.iota(i(8), 0), 'FillParams': K.fill(b(8), 0),
+        'EwParams': K.lower_ew_chain(chain), 'EwAffineParams': K.lower_ew_chain(K.EwChain(b(64, 8), (64, 8), K.broadcast_operand(b(64, 8), (64, 8)), [K.EwStep(K.EW[o], K.broadcast_operand(b(*sh), (64, 8))) for o, sh in (('ADD_F', (64, 8)), ('SUB_F', (8,)), ('MUL_F', (8,)), ('ADD_F', (8,)))])),
+        'IotaParams': K.iota(i(8), 0), 'FillParams': K.fill(b(8), 0),
         'ConcatParams': K.concat_part(b(4, 8), b(4, 3), 1, 0), 'ConvParams': K.conv_gemm(b(1, 4, 4, 24), b(1, 4, 4, 4), b(1, 1, 4, 24), geom),
         'DenseRowsParams': K.conv_gemm(b(16, 8), b(16, 4), b(4, 8), few),
         'ConvStemParams': K.conv_gemm(b(1, 64, 64, 8), b(1, 128, 128, 3), b(7, 7, 3, 8),
@@ -110,6 +111,7 @@ def test_kernel_argument_layouts_match_the_structs():
     #the convolution kernel takes two parameter structs, one after the other
     sizes['ConvParams'] += sizes['ConvDerived']
     sizes['ConvStemParams'] += sizes['ConvDerived']
+    assert launches['EwAffineParams'].kernel == 'ew_affine_v4' and len(launches['EwAffineParams'].buffers) == 10
     assert launches['ConvStemParams'].kernel == 'conv_gemm_stem_7x22' and launches['DenseRowsParams'].kernel == 'dense_rows_n16'
     assert len(launches['DenseRowsParams'].buffers) == 3 + K.CONV_MAX_EPI
     for struct, launch in launches.items():
@@ -363,7 +365,7 @@ def test_long_contractions_of_few_tiles_are_sliced():
         args = (np.zeros((m, k), np.float32), np.zeros((k, n), np.float32), np.zeros((n,), np.float32))
         return JaxprInterpreter(mj.make_jaxpr(layer)(*args), plan_only=True, **kw)
     interp = plan(49, 4608, 512)                                   #2 x 16 tiles, 36 k steps
-    assert [l.kernel for l in interp.launches] == ['conv_gemm_32x32x128_ks4', 'ew_chain_v4_s6']
+    assert [l.kernel for l in interp.launches] == ['conv_gemm_32x32x128_ks4', 'ew_affine_v4']       #sum of four slices + bias, ReLU
     first, second = interp.launches
     assert first.grid == (32 * 4, 1, 1) and first.buffers[0][0].shape == (4, 49 * 512)
     assert np.frombuffer(first.params, np.int32)[-1 - 9] == 9      #k steps per slice: the last word before the 9 of ConvDerived

@@ -198,6 +198,65 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     }
 }
 
+// The chains that a convolution's epilogue would otherwise hold, as a launch of their own (a batch norm over an array
+// that no convolution has just produced, the sum of the slices of a sliced contraction followed by scale, shift,
+// residual and ReLU): on contiguous float arrays of n elements whose fastest dimension has C elements,
+//     v = first + s1 + s2 + s3            (the first nsum of them, in this order)
+//     v = v - vsub[c]; v = v * vmul[c]; v = v + vadd[c]; v = v + full; v = max(v, floor)      (each optional, in this order)
+// Straight-line code: every load is issued through a buffer descriptor whose size is 0 for an absent operand (such a
+// load returns zeros without touching memory), every step is a select on a flag. The opcode interpreter of ew_chain
+// spends 750 instructions and 170 branches per wave on such a chain, which is most of a small launch's duration and
+// a quarter of the bandwidth of a large one. n and C are multiples of 4; two 16-byte vectors per thread.
+struct EwAffineParams {
+    uint32_t n, cq;                 // elements; C / 4
+    uint32_t cq_magic, cq_shift;    // v / cq = mulhi(v, magic) >> shift for v < 2^31 (magic 0: cq == 1)
+    uint32_t nsum;                  // 0..3
+    uint32_t flags;                 // bit0 - vsub, bit1 * vmul, bit2 + vadd, bit3 + full, bit4 max(., floor)
+};
+
+extern "C" __global__ __launch_bounds__(256) void ew_affine_v4(
+        float* __restrict__ out, const float* first, const float* s1, const float* s2, const float* s3,
+        const float* vsub, const float* vmul, const float* vadd, const float* full, const float* floor_, EwAffineParams P) {
+    constexpr int U = 2;
+    const uint32_t nb = P.n * 4u, cb = P.cq * 16u, fl = P.flags;
+    const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out, nb), r_first = make_rsrc(first, nb),
+        r_s1 = make_rsrc(s1, P.nsum >= 1u ? nb : 0u), r_s2 = make_rsrc(s2, P.nsum >= 2u ? nb : 0u), r_s3 = make_rsrc(s3, P.nsum >= 3u ? nb : 0u),
+        r_sub = make_rsrc(vsub, (fl & 1u) ? cb : 0u), r_mul = make_rsrc(vmul, (fl & 2u) ? cb : 0u), r_add = make_rsrc(vadd, (fl & 4u) ? cb : 0u),
+        r_full = make_rsrc(full, (fl & 8u) ? nb : 0u), r_floor = make_rsrc(floor_, (fl & 16u) ? 4u : 0u);
+    f32x4 a[U], b1[U], b2[U], b3[U], fu[U], vs[U], vm[U], va[U];
+    uint32_t off[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = (blockIdx.x * U + u) * 256u + threadIdx.x;          // vector index; beyond n / 4: every access is out of range
+        const uint32_t q = P.cq_magic ? __umulhi(v, P.cq_magic) >> P.cq_shift : v;
+        const uint32_t c = (P.cq == 1u ? 0u : v - q * P.cq) * 16u;
+        off[u] = v * 16u;
+        a[u]  = buffer_load_x4(r_first, off[u]);
+        b1[u] = buffer_load_x4(r_s1, off[u]); b2[u] = buffer_load_x4(r_s2, off[u]); b3[u] = buffer_load_x4(r_s3, off[u]);
+        fu[u] = buffer_load_x4(r_full, off[u]);
+        vs[u] = buffer_load_x4(r_sub, c); vm[u] = buffer_load_x4(r_mul, c); va[u] = buffer_load_x4(r_add, c);
+    }
+    const float lo = buffer_load_x1(r_floor, 0u);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        f32x4 y;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float v = a[u][j];
+            v = P.nsum >= 1u ? v + b1[u][j] : v;
+            v = P.nsum >= 2u ? v + b2[u][j] : v;
+            v = P.nsum >= 3u ? v + b3[u][j] : v;
+            v = (fl & 1u) ? v - vs[u][j] : v;
+            v = (fl & 2u) ? v * vm[u][j] : v;
+            v = (fl & 4u) ? v + va[u][j] : v;
+            v = (fl & 8u) ? v + fu[u][j] : v;
+            v = (fl & 16u) ? ((v > lo || v != v) ? v : lo) : v;               // a NaN stays
+            y[j] = v;
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 0);
+    }
+}
+
 // Requests one word of every 64-byte line of the argument block at the very start of a kernel and waits for all of
 // them at once. The fields are fetched where the compiler needs them, in several dependent groups; a group that
 // touches a line for the first time waits for a round trip to memory (about 1600 cycles), later ones find their

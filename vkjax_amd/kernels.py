@@ -145,6 +145,9 @@ def lower_ew_chain(chain: EwChain) -> Launch:
     transposed = _as_tiled_transpose(chain, dims, strides)
     if transposed is not None:
         return transposed
+    affine = _as_affine_chain(chain, n, dims, strides)
+    if affine is not None:
+        return affine
     vec = 4
     if n % 4 or dims[-1] % 4:
         vec = 1
@@ -200,6 +203,59 @@ def lower_ew_chain(chain: EwChain) -> Launch:
     per_thread = {2: 1, 4: 2, 6: 2, 8: 1}[slots]               #vectors a thread works on (the kernel's U)
     return Launch(f'ew_chain_v{vec}_s{slots}', (_cdiv(_cdiv(n, vec), BLOCK * per_thread), 1, 1), (BLOCK, 1, 1),
                   [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
+
+
+#tests: None = where it applies, False = never
+FORCE_EW_AFFINE: tp.Optional[bool] = None
+EW_AFFINE_MAX_ELEMENTS = 1 << 22
+
+
+def _as_affine_chain(chain: EwChain, n: int, dims, strides) -> tp.Optional[Launch]:
+    '''ew_affine_v4 for float chains of the form ((first + s1 + s2 + s3) - vsub) * vmul + vadd + full, max(., floor)
+    (every part optional, in this order; s and full arrays of the output's shape, v vectors over the fastest
+    dimension, floor one value), for chains of more than four operands on arrays of at most 16 MB, where the launch
+    is mostly the interpreter's latency. Shorter chains keep the general kernel (small ones are batched with their
+    neighbours), and so do large arrays: there the ten loads per vector, most of them through empty descriptors,
+    cost more than the interpreter (relu on 64 M elements 4.4 TB/s against 5.7).'''
+    operands = chain.operands()
+    if (FORCE_EW_AFFINE is False or not chain.steps or any(o is None for o in operands) or n % 4 or dims[-1] % 4 or n * 4 >= 2**32 - 2**16
+            or len(dims) > 2 or (FORCE_EW_AFFINE is None and (len(operands) <= 4 or n > EW_AFFINE_MAX_ELEMENTS))
+            or any(np.dtype(b.dtype) != np.float32 for b in [chain.out] + [o.buffer for o in operands])):
+        return None
+    dense = row_major_strides(dims)
+    kind  = lambda st: ('full' if tuple(st) == dense else 'vec' if len(dims) == 2 and tuple(st) == (0, 1)
+                        else 'one' if all(s == 0 for s in st) else None)
+    kinds = [kind(st) for st in strides]
+    if kinds[0] != 'full' or (len(dims) == 1 and 'vec' in kinds):
+        return None
+    steps, k = list(zip(chain.steps, operands[1:], kinds[1:])), 0
+    sums, slot = [], {}
+    while k < len(steps) and len(sums) < 3 and steps[k][0].op == EW['ADD_F'] and steps[k][2] == 'full':
+        sums.append(steps[k][1]); k += 1
+    template = ((0, EW['SUB_F'], 'vec', False), (1, EW['MUL_F'], 'vec', None), (2, EW['ADD_F'], 'vec', None),
+                (3, EW['ADD_F'], 'full', None), (4, EW['MAX_F'], 'one', False))
+    t = 0
+    while k < len(steps):
+        step, operand, what = steps[k]
+        while t < len(template) and not (step.op == template[t][1] and what == template[t][2]
+                                         and (template[t][3] is None or bool(step.operand_left) == template[t][3])):
+            t += 1
+        if t == len(template):
+            return None
+        slot[template[t][0]] = operand
+        t += 1; k += 1
+    if not sums and not slot:
+        return None
+    C = dims[-1] if len(dims) == 2 else 4
+    if any(o.buffer.size != C for b, o in slot.items() if b in (0, 1, 2)):
+        return None
+    magic, shift = _magic_division(C // 4)
+    at = lambda o: (o.buffer, o.offset * 4) if o is not None else (None, 0)
+    buffers = ([(chain.out, 0), at(operands[0])] + [at(o) for o in _pad(sums, 3, None)]
+               + [at(slot.get(b)) for b in range(5)])
+    params  = _u32(n, C // 4, magic, shift, len(sums), sum(1 << b for b in slot))
+    nbytes  = 4 * n + sum(4 * min(n, o.buffer.size) for o in operands)
+    return Launch('ew_affine_v4', (_cdiv(n // 4, 2 * BLOCK), 1, 1), (BLOCK, 1, 1), buffers, params, bytes_moved=nbytes)
 
 
 EW_BATCH_KERNELS     = ('ew_chain_v1_s2', 'ew_chain_v1_s4', 'ew_chain_v4_s2', 'ew_chain_v4_s4')
