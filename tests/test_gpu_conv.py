@@ -199,16 +199,23 @@ def test_four_waves_per_tile_kernel():
              (dense, [ints(-4, 5, 256, 512), ints(-3, 4, 512, 10), ints(-9, 9, 10)]),
              (plain, [ints(-4, 5, 40, 388), ints(-2, 3, 388, 7)]),
              (bn_res_relu, [ints(-4, 5, 2, 9, 7, 128), ints(-3, 4, 1, 1, 128, 72), ints(-5, 5, 72), ints(1, 4, 72), ints(-9, 9, 72), ints(-50, 50, 2, 9, 7, 72)]),
-             (bn_res_relu, [ints(-4, 5, 2, 9, 7, 256), ints(-3, 4, 3, 3, 256, 40), ints(-5, 5, 40), ints(1, 4, 40), ints(-9, 9, 40), ints(-50, 50, 2, 9, 7, 40)])]
+             (bn_res_relu, [ints(-4, 5, 2, 9, 7, 256), ints(-3, 4, 3, 3, 256, 40), ints(-5, 5, 40), ints(1, 4, 40), ints(-9, 9, 40), ints(-50, 50, 2, 9, 7, 40)]),
+             #windows over 64 and 192 features: the 64-long k step
+             (bn_res_relu, [ints(-4, 5, 1, 14, 9, 64), ints(-3, 4, 3, 3, 64, 64), ints(-5, 5, 64), ints(1, 4, 64), ints(-9, 9, 64), ints(-50, 50, 1, 14, 9, 64)]),
+             (bn_res_relu, [ints(-4, 5, 2, 5, 6, 192), ints(-3, 4, 3, 3, 192, 33), ints(-5, 5, 33), ints(1, 4, 33), ints(-9, 9, 33), ints(-50, 50, 2, 5, 6, 33)])]
     K.FORCE_CONV_KSPLIT, K.FORCE_CONV_K_SPLITS = True, 1
     try:
         for f, args in cases:
+            short = f is bn_res_relu and args[1].shape[0] == 3 and args[1].shape[2] % 128 != 0
             for b_general in (False, True):
                 K.FORCE_CONV_B_GENERAL = b_general
                 print(f'four waves per tile: {f.__name__} {[a.shape for a in args]} element-wise kernel loads {b_general}', flush=True)
                 _, _, fn = check_against_oracle(f, args, exact=True)
                 launches = list(fn._jaxpr_interpreters.values())[0].launches
-                assert [l.kernel for l in launches] == ['conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4'], [l.kernel for l in launches]
+                if short:                                     #(this variant exists with 16-byte loads of the kernel operand only)
+                    assert ([l.kernel for l in launches] == ['conv_gemm_32x32x64_ks4']) == (not b_general), [l.kernel for l in launches]
+                else:
+                    assert [l.kernel for l in launches] == ['conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4'], [l.kernel for l in launches]
     finally:
         K.FORCE_CONV_KSPLIT = K.FORCE_CONV_K_SPLITS = None
         K.FORCE_CONV_B_GENERAL = False

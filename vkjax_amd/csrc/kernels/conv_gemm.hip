@@ -792,6 +792,8 @@ CONV_TILE(32x32x64, 1, 1, 1, 1, 64)
 CONV_KERNEL(conv_gemm_32x32x128_ks4, 1, 1, 1, 1, 128, true, true, true, 4)
 // the same with element-wise loads of the kernel operand (an output width that is no multiple of 4)
 CONV_KERNEL(conv_gemm_32x32x128_ks4g, 1, 1, 1, 1, 128, true, false, true, 4)
+// the same with a 64-long k step, for windows over 64 (or 192, ...) input features, whose taps a 128-long step would straddle
+CONV_KERNEL(conv_gemm_32x32x64_ks4, 1, 1, 1, 1, 64, true, true, true, 4)
 // Mixed tiling for layers whose 64 x 64 tiles do not divide evenly among the CUs (784 tiles on 256 CUs: a CU
 // with four tiles sets the time, the average is 3.06). The first P.split_tiles_m M tiles are computed as 64 x 64
 // tiles, as many as fill every CU equally; the rows behind them as 32 x 32 tiles of a quarter of the work each

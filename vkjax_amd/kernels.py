@@ -715,7 +715,7 @@ def _four_waves_per_tile(g: ConvGeometry, a_fast: bool, c_contig: bool, compute_
     each taking a quarter of every (128-long) k step.'''
     want = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
             (_cdiv(g.M, 32) * _cdiv(g.N, 32) <= 2 * compute_units and g.K >= 256 and FORCE_CONV_TILE is None and FORCE_CONV_BK is None))
-    return bool(want) and a_fast and c_contig and (g.Cin % 128 == 0 or g.KH * g.KW == 1) and not FORCE_CONV_GENERAL
+    return bool(want) and a_fast and c_contig and (g.Cin % 64 == 0 or g.KH * g.KW == 1) and not FORCE_CONV_GENERAL
 
 
 #tests: the number of slices a contraction is cut into where that applies (None: by the heuristic, 1: never)
@@ -734,7 +734,7 @@ def conv_k_splits(lhs: Buffer, rhs: Buffer, g: ConvGeometry, compute_units: int 
     if g.K * g.N * 4 >= 2**31 or lhs.size * 4 >= 2**31 or g.M * g.N == 0:
         return 1
     _, _, a_fast, _, c_contig = _conv_fast_paths(lhs, rhs, g)
-    if not _four_waves_per_tile(g, a_fast, c_contig, compute_units):
+    if not _four_waves_per_tile(g, a_fast, c_contig, compute_units) or (g.Cin % 128 != 0 and g.KH * g.KW != 1):
         return 1
     tiles, ksteps = _cdiv(g.M, 32) * _cdiv(g.N, 32), _cdiv(g.K, 128)
     if FORCE_CONV_K_SPLITS is not None:
@@ -791,13 +791,17 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     #a product with so few 32 x 32 tiles that one wave per tile leaves most MFMA units idle: four waves per
     #tile, each taking a quarter of every (128-long) k step
     ksplit = _four_waves_per_tile(g, a_fast, c_contig, compute_units) and (not epilogue or slots != 0)
+    #(windows over 64 input features take a 64-long k step, with 16-byte loads of the kernel operand only)
+    short_step = ksplit and g.Cin % 128 != 0 and g.KH * g.KW != 1
+    if short_step and not b_fast:
+        ksplit = False
     if ksplit:
-        tag, bm, bn, nt, bk, lean = '32x32', 32, 32, 256, 128, True
+        tag, bm, bn, nt, bk, lean = '32x32', 32, 32, 256, 64 if short_step else 128, True
     tiles_m, tiles_n = _cdiv(M, bm), _cdiv(N, bn)
     k_split_steps = 0
     if g.k_splits > 1:
         k_split_steps = _cdiv(_cdiv(K, 128), g.k_splits)
-        if (not ksplit or epilogue or taps or out_offset or out.size != g.k_splits * M * N
+        if (not ksplit or short_step or epilogue or taps or out_offset or out.size != g.k_splits * M * N
                 or _cdiv(_cdiv(K, 128), k_split_steps) != g.k_splits):
             raise ValueError('a sliced contraction needs the four-waves-per-tile kernel, no epilogue and one [M, N] matrix per non-empty slice')
     chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean and not ksplit else 1
