@@ -48,7 +48,7 @@ OTHER_CONFIGS = ('affine', 'mlp', 'conv_block', 'rng_uniform', 'gather_scatter')
 
 
 def kernel_family(name: str) -> str:
-    for prefix in ('conv_gemm', 'wgrad_gemm', 'softmax_rows', 'ew_chain', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows',
+    for prefix in ('conv_gemm', 'wgrad_gemm', 'dense_rows', 'softmax_rows', 'ew_chain', 'ew_affine', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows',
                    'select_window', 'scatter_selected', 'pad_nd', 'scale_relu_backward', 'scale_backward', 'transpose_tiled'):
         if name.startswith(prefix):
             return prefix
@@ -151,7 +151,8 @@ def measure(workload, steps, warmup, batch=None, fuse=True, graph=False, profile
             kernels[name] = entry
         dominant = max(fam, key=lambda k: fam[k]['stamped_ms'])
         d, ms = fam[dominant], fam[dominant]['stamped_ms'] * scale
-        if d['flops']:
+        #(dense_rows_n16 multiplies on the vector ALUs: a few rows of a small batch, priced by the bytes it moves)
+        if d['flops'] and dominant != 'dense_rows':
             achieved = d['flops'] / ms / 1e9
             roofline = dict(bound='mfma', kernel=dominant, achieved=round(achieved, 3), peak=PEAK_FP32_MFMA_TFLOPS, unit='TFLOP/s',
                             frac=round(achieved / PEAK_FP32_MFMA_TFLOPS, 4))
