@@ -613,7 +613,9 @@ __device__ __forceinline__ void pool_body(uint32_t* __restrict__ out, const uint
 // taps of a thread's four channels are requested before the first is used (the general kernel
 // above walks the window with one load in flight), with 32-bit index arithmetic. Needs channels % 4 == 0
 // and fewer than 2^32 bytes on either side; the host checks.
-template <int KH, int KW>
+// MODE as for the reductions (0 float sum, 1 float max, 2 whatever op and type say): with the combine chosen at run
+// time every one of a thread's 32 combines went through the branches of red_combine, 336 branches per wave.
+template <int KH, int KW, int MODE>
 __device__ __forceinline__ void pool2d_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const PoolParams& P) {
     const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u;
     if (e0 >= P.n_out) return;
@@ -623,7 +625,7 @@ __device__ __forceinline__ void pool2d_body(uint32_t* __restrict__ out, const ui
     const uint32_t wo = r % Wo; r /= Wo;
     const uint32_t ho = r % Ho, b = r / Ho;
     const int32_t y0 = (int32_t)(ho * P.stride[1]) - P.pad_low[1], x0 = (int32_t)(wo * P.stride[2]) - P.pad_low[2];
-    const uint32_t ident = red_identity(P.op, P.type);
+    const uint32_t ident = MODE == 0 ? 0u : MODE == 1 ? 0xFF800000u : red_identity(P.op, P.type);
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in), 0,
         (int)(P.in_dims[0] * P.in_dims[1] * P.in_dims[2] * P.in_dims[3] * 4u), 0x00020000);
     u32x4 v[KH][KW];
@@ -643,18 +645,24 @@ __device__ __forceinline__ void pool2d_body(uint32_t* __restrict__ out, const ui
 #pragma unroll
         for (int kx = 0; kx < KW; ++kx) {
             if (ky == 0 && kx == 0) continue;
-            acc.x = red_combine(P.op, P.type, acc.x, v[ky][kx].x);
-            acc.y = red_combine(P.op, P.type, acc.y, v[ky][kx].y);
-            acc.z = red_combine(P.op, P.type, acc.z, v[ky][kx].z);
-            acc.w = red_combine(P.op, P.type, acc.w, v[ky][kx].w);
+            acc.x = red_step<MODE>(P.op, P.type, acc.x, v[ky][kx].x);
+            acc.y = red_step<MODE>(P.op, P.type, acc.y, v[ky][kx].y);
+            acc.z = red_step<MODE>(P.op, P.type, acc.z, v[ky][kx].z);
+            acc.w = red_step<MODE>(P.op, P.type, acc.w, v[ky][kx].w);
         }
     *reinterpret_cast<u32x4*>(out + e0) = acc;
 }
+template <int KH, int KW>
+__device__ __forceinline__ void pool2d_dispatch(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const PoolParams& P) {
+    if (P.type == RT_F32 && P.op == RED_MAX) pool2d_body<KH, KW, 1>(out, in, P);
+    else if (P.type == RT_F32 && P.op == RED_SUM) pool2d_body<KH, KW, 0>(out, in, P);
+    else pool2d_body<KH, KW, 2>(out, in, P);
+}
 extern "C" __global__ __launch_bounds__(256) void pool2d_3x3_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, PoolParams P) {
-    pool2d_body<3, 3>(out, in, P);
+    pool2d_dispatch<3, 3>(out, in, P);
 }
 extern "C" __global__ __launch_bounds__(256) void pool2d_2x2_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, PoolParams P) {
-    pool2d_body<2, 2>(out, in, P);
+    pool2d_dispatch<2, 2>(out, in, P);
 }
 
 extern "C" __global__ __launch_bounds__(256) void pool_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, PoolParams P) {
