@@ -18,11 +18,18 @@ import numpy as np
 from .minijax import core
 
 
-class TensorPlaceholder:
+class StorageCell:
+    '''The device allocation that one or several buffers (views of one another) stand on. It is filled in when
+    storage is assigned, after the whole program is known, so all views see the allocation at once.'''
+    __slots__ = ('t', 'elided')
+
     def __init__(self, t=None):
         self.t = t
         #set when fusion keeps the value in registers: the variable never gets storage
         self.elided = False
+
+
+TensorPlaceholder = StorageCell          #the reference's name for it (vkjax/buffers.py:13-15)
 
 
 class PlannedTensor:
@@ -54,25 +61,29 @@ class PlanOnlyDevice:
 
 
 class Buffer:
+    '''dtype, shape and liveness (`accesses`: positions of the ops that touch it) of one array in HBM. `tensor` is the
+    device allocation of the storage cell the buffer stands on; views made by `view` share cell and access list, as in
+    the reference (vkjax/buffers.py:17-51), where the sharing is done by intercepting attribute access.'''
+    __slots__ = ('_cell', 'dtype', 'shape', 'accesses', 'constant_value')
+
     def __init__(self, tensor, dtype: np.dtype, shape: tp.Tuple[int, ...]):
-        if isinstance(tensor, TensorPlaceholder):
-            super().__setattr__('tensor', tensor)
-        else:
-            super().__setattr__('tensor', TensorPlaceholder(tensor))
+        self._cell = tensor if isinstance(tensor, StorageCell) else StorageCell(tensor)
         self.dtype = np.dtype(dtype)
         self.shape = tuple(int(s) for s in shape)
         self.accesses: tp.List[float] = []
+        self.constant_value = None
 
-    def __getattribute__(self, name):
-        if name == 'tensor':
-            return super().__getattribute__(name).t
-        return super().__getattribute__(name)
+    @property
+    def tensor(self):
+        return self._cell.t
 
-    def __setattr__(self, name, value):
-        if name == 'tensor':
-            super().__getattribute__(name).t = value
-        else:
-            super().__setattr__(name, value)
+    @tensor.setter
+    def tensor(self, allocation):
+        self._cell.t = allocation
+
+    @property
+    def _placeholder(self) -> StorageCell:
+        return self._cell
 
     @property
     def size(self) -> int:
@@ -86,16 +97,12 @@ class Buffer:
 
     def view(self, new_dtype, new_shape) -> 'Buffer':
         '''Another dtype/shape on the same storage; shares the access list (reference: vkjax/buffers.py:48-51).'''
-        new_b          = Buffer(super().__getattribute__('tensor'), new_dtype, new_shape)
-        new_b.accesses = self.accesses
-        return new_b
+        other = Buffer(self._cell, new_dtype, new_shape)
+        other.accesses = self.accesses
+        return other
 
     def same_storage(self, other: 'Buffer') -> bool:
-        return self._placeholder is other._placeholder
-
-    @property
-    def _placeholder(self):
-        return super().__getattribute__('tensor')
+        return self._cell is other._cell
 
     def numpy(self) -> np.ndarray:
         '''Blocking read of the device contents as an array of this buffer's dtype and shape.'''
