@@ -1,8 +1,10 @@
-'''Seeded random geometry through three kernels whose applicability depends on the shape: the mixed 64 x 64 /
+'''Seeded random geometry through the kernels whose applicability depends on the shape: the mixed 64 x 64 /
 32 x 32 tiling (split point, k step and epilogue drawn at random), the stem kernel (kernel width x features of 21
 or 22 in several factorisations, strides, paddings on all four sides, image sizes around its limits; shapes it does
 not take fall back to the general kernel and are checked all the same) and the sorted scatter-add (table and index
-sizes around the segment and block limits, crowded rows, indices outside the table). Integer-valued data: every
+sizes around the segment and block limits, crowded rows, indices outside the table), sliced contractions (number of
+slices, 1x1 and 3x3 windows, k steps that are not full), the kernel for at most 16 output features, and the
+straight-line kernel for sums of arrays followed by scale, shift, residual and ReLU. Integer-valued data: every
 result equals the oracle's bit for bit.'''
 import numpy as np
 import pytest
@@ -68,11 +70,66 @@ def _scatter_case(rng, ints):
     return (lambda t, i, u: jnp.index_add(t, i, u)), [ints(-9, 10, rows, cols), idx, ints(-3, 4, n, cols)], {}, 'scatter_rows_sum'
 
 
-@pytest.mark.parametrize('seed', range(90))
+def _sliced_case(rng, ints):
+    ks = int(rng.choice([1, 1, 3]))
+    if ks == 1:
+        m, kdim, n = int(rng.randint(1, 130)), int(rng.choice([256, 388, 512, 900, 1300, 2048])), int(rng.choice([17, 24, 40, 72, 96]))
+        x, w = ints(-3, 4, m, kdim), ints(-2, 3, kdim, n)
+        product, out_shape = (lambda x, w: jnp.dot(x, w)), (m, n)
+    else:
+        b, h, wd, cin, n = int(rng.choice([1, 2])), int(rng.randint(3, 9)), int(rng.randint(3, 9)), int(rng.choice([128, 256])), int(rng.choice([24, 40, 72]))
+        x, w = ints(-3, 4, b, h, wd, cin), ints(-2, 3, 3, 3, cin, n)
+        product, out_shape = (lambda x, w: lax.conv_general_dilated(x, w, (1, 1), 'SAME', dimension_numbers=DN)), (b, h, wd, n)
+    epilogue = rng.randint(0, 3)
+    if epilogue == 0:
+        f, args = product, [x, w]
+    elif epilogue == 1:
+        f, args = (lambda x, w, bias: nn.relu(product(x, w) + bias)), [x, w, ints(-9, 9, n)]
+    else:
+        f = lambda x, w, mean, scale, shift, res: nn.relu((product(x, w) - mean) * scale + shift + res)
+        args = [x, w, ints(-5, 5, n), ints(1, 4, n), ints(-9, 9, n), ints(-50, 50, *out_shape)]
+    return f, args, dict(FORCE_CONV_KSPLIT=True, FORCE_CONV_K_SPLITS=int(rng.randint(2, 6))), 'ks4'
+
+
+def _few_features_case(rng, ints):
+    m, kdim, n = int(rng.randint(1, 300)), 4 * int(rng.randint(1, 300)), int(rng.randint(1, 17))
+    x, w = ints(-3, 4, m, kdim), ints(-2, 3, kdim, n)
+    epilogue = rng.randint(0, 3)
+    if epilogue == 0:
+        return (lambda x, w: jnp.dot(x, w)), [x, w], {}, 'dense_rows_n16'
+    if epilogue == 1 and n > 1:
+        return (lambda x, w, bias: nn.relu(jnp.dot(x, w) + bias)), [x, w, ints(-9, 9, n)], {}, 'dense_rows_n16'
+    if n > 1:
+        return (lambda x, w, mean, scale, shift: (jnp.dot(x, w) - mean) * scale + shift), [x, w, ints(-5, 5, n), ints(1, 4, n), ints(-9, 9, n)], {}, 'dense_rows_n16'
+    return None
+
+
+def _affine_chain_case(rng, ints):
+    shape = [(int(rng.randint(2, 70)), 4 * int(rng.randint(1, 40))), (2, int(rng.randint(1, 9)), int(rng.randint(1, 9)), 4 * int(rng.randint(1, 20)))][rng.randint(0, 2)]
+    c, nsum = shape[-1], int(rng.randint(0, 4))
+    parts = [int(rng.randint(0, 2)) for _ in range(5)]
+    if nsum + sum(parts) == 0:
+        return None
+    arrays, vectors = [ints(-9, 10, *shape) for _ in range(5)], [ints(-5, 5, c), ints(-3, 4, c), ints(-9, 9, c)]
+    def f(first, s1, s2, s3, full, vsub, vmul, vadd):
+        v = first
+        for a in (s1, s2, s3)[:nsum]:
+            v = v + a
+        if parts[0]: v = v - vsub
+        if parts[1]: v = v * vmul
+        if parts[2]: v = v + vadd
+        if parts[3]: v = v + full
+        if parts[4]: v = nn.relu(v)
+        return v
+    return f, arrays + vectors, dict(FORCE_EW_AFFINE=True), 'ew_affine_v4'
+
+
+@pytest.mark.parametrize('seed', range(180))
 def test_random_geometry(seed):
     rng  = np.random.RandomState(777 + seed)
     ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
-    case = (_mixed_tiling_case, _stem_case, _scatter_case)[seed % 3](rng, ints)
+    cases = (_mixed_tiling_case, _stem_case, _scatter_case, _sliced_case, _few_features_case, _affine_chain_case)
+    case = cases[seed % 3 if seed < 90 else 3 + seed % 3](rng, ints)          #(the first 90 seeds keep the cases they always had)
     if case is None:
         pytest.skip('the draw gave a shape outside the kernels\' range')
     f, args, forced, expected = case
@@ -80,7 +137,7 @@ def test_random_geometry(seed):
     try:
         for name, value in forced.items():
             setattr(K, name, value)
-        if seed % 3 == 2:
+        if seed < 90 and seed % 3 == 2:
             ops.SCATTER_SORT_THRESHOLD = 0
         print(f'seed {seed}: {[a.shape for a in args]} {forced}', flush=True)
         _, _, fn = check_against_oracle(f, args, exact=True)
