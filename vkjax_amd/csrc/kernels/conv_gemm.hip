@@ -217,7 +217,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     // Scalar and per-feature epilogue operands are fetched once per block, at its very start, and
     // parked in LDS behind the first k tile's loads, so that the epilogue never waits on global
     // memory for them. Thread t fetches column t of every step.
-    float e_reg[CONV_MAX_EPI];
+    float e_reg[CONV_MAX_EPI], d_in[CONV_MAX_DERIVED + 1];
     if (tid < BN) {
 #pragma unroll
         for (int e = 0; e < CONV_MAX_EPI; ++e) {
@@ -229,36 +229,15 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             else if (kind == 2) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], (uint32_t)P.N * 4u * present), (uint32_t)(n0 + tid) * 4u);
         }
         if (Dk.nsteps) {
-            // the derived operand: same arithmetic, operation by operation, as the element-wise kernel
-            float in[CONV_MAX_DERIVED + 1];
+            // the arrays of the derived operand: requested here, combined once the first k tile's loads are on their
+            // way (combining them here would hold the wave, and with it the block's first barrier, for a round trip
+            // to memory before any tile load is issued)
 #pragma unroll
             for (int k = 0; k <= CONV_MAX_DERIVED; ++k) {
                 const bool vec = (Dk.vector_mask >> k) & 1u;
-                in[k] = buffer_load_x1(make_rsrc(Dp.p[k], Dp.p[k] == nullptr ? 0u : vec ? (uint32_t)P.N * 4u : 4u),
-                                       vec ? (uint32_t)(n0 + tid) * 4u : 0u);
+                d_in[k] = buffer_load_x1(make_rsrc(Dp.p[k], Dp.p[k] == nullptr ? 0u : vec ? (uint32_t)P.N * 4u : 4u),
+                                         vec ? (uint32_t)(n0 + tid) * 4u : 0u);
             }
-            float v = in[0];
-#pragma unroll
-            for (int k = 0; k < CONV_MAX_DERIVED; ++k) {
-                if (k < (int)Dk.nsteps) {
-                    const float a = Dk.left[k] ? in[k + 1] : v, b = Dk.left[k] ? v : in[k + 1];
-                    switch (Dk.op[k]) {
-                        case CEW_ADD_F:   v = a + b; break;
-                        case CEW_SUB_F:   v = a - b; break;
-                        case CEW_MUL_F:   v = a * b; break;
-                        case CEW_DIV_F:   v = a / b; break;
-                        case CEW_MAX_F:   v = (a > b || a != a) ? a : b; break;
-                        case CEW_MIN_F:   v = (a < b || a != a) ? a : b; break;
-                        case CEW_NEG_F:   v = -v; break;
-                        case CEW_RSQRT_F: v = 1.0f / sqrtf(v); break;
-                        case CEW_SQRT_F:  v = sqrtf(v); break;
-                        default: break;
-                    }
-                }
-            }
-#pragma unroll
-            for (int e = 0; e < CONV_MAX_EPI; ++e)
-                if (e == (int)Dk.step) e_reg[e] = v;
         }
     }
     // the first full-size operand (a residual input) is fetched for a whole tile at once, while
@@ -490,6 +469,31 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     CONV_STAMP(1)
     load_tiles(kbase * BK);
     if (tid < BN) {
+        if (Dk.nsteps) {
+            // the derived operand: same arithmetic, operation by operation, as the element-wise kernel
+            float v = d_in[0];
+#pragma unroll
+            for (int k = 0; k < CONV_MAX_DERIVED; ++k) {
+                if (k < (int)Dk.nsteps) {
+                    const float a = Dk.left[k] ? d_in[k + 1] : v, b = Dk.left[k] ? v : d_in[k + 1];
+                    switch (Dk.op[k]) {
+                        case CEW_ADD_F:   v = a + b; break;
+                        case CEW_SUB_F:   v = a - b; break;
+                        case CEW_MUL_F:   v = a * b; break;
+                        case CEW_DIV_F:   v = a / b; break;
+                        case CEW_MAX_F:   v = (a > b || a != a) ? a : b; break;
+                        case CEW_MIN_F:   v = (a < b || a != a) ? a : b; break;
+                        case CEW_NEG_F:   v = -v; break;
+                        case CEW_RSQRT_F: v = 1.0f / sqrtf(v); break;
+                        case CEW_SQRT_F:  v = sqrtf(v); break;
+                        default: break;
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < CONV_MAX_EPI; ++e)
+                if (e == (int)Dk.step) e_reg[e] = v;
+        }
 #pragma unroll
         for (int e = 0; e < CONV_MAX_EPI; ++e)
             if (e < nepi) Es[e * BN + tid] = e_reg[e];           // published by the barriers of the first k step
@@ -541,6 +545,9 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             for (int kt = 0; kt < ktiles; kt += 2) {
                 store_tiles(0);
                 if (kt == 0) __syncthreads(); else tile_barrier();
+#ifdef CONV_PHASE_STAMPS
+                if (kt == 0 && sub == 0) { CONV_STAMP(2) }
+#endif
                 if (kt + 2 < ktiles) load_tiles((kbase + kt + 2) * BK, 0);
                 compute();
                 tile_barrier();
