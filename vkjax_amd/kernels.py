@@ -891,6 +891,10 @@ def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op:
                       bytes_moved=4 * (outer * R + outer * nsplit)), nsplit
     vec = 4 if inner % 4 == 0 else 1
     TI  = min(64, _pow2_at_least(_cdiv(inner, vec)))
+    #few blocks with many rows each (the second stage of a split sum): narrower blocks, more of them, more thread rows
+    #walking the rows side by side
+    while TI > 8 and _cdiv(inner, TI * vec) * nsplit * outer < 64 and _cdiv(R, nsplit) * TI >= 256 * 8:
+        TI //= 2
     params = _u32(outer, R, inner, RED[op], ty, r_chunk, nsplit, TI)
     blocks = _cdiv(inner, TI * vec) * nsplit * outer
     if blocks >= 2**31:
