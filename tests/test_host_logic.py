@@ -424,6 +424,32 @@ def test_softmax_plan_keeps_every_result_of_the_fused_launch():
     assert [l.kernel for l in interp.launches] == ['softmax_rows_v4'] and interp.launches[0].buffers[2][0] is None
 
 
+def test_repeated_equations_are_evaluated_once():
+    '''An element-wise or shape equation with the primitive, parameters and operands of an earlier one is bound to that
+    equation's buffer: indexing and scatter-add through the same index array normalise it once (two launches less),
+    literals of different value or dtype are told apart, and results of the program keep equations of their own.'''
+    import vkjax_amd
+    from vkjax_amd import minijax as mj, ops, workloads as W
+    from vkjax_amd.jaxpr_interpreter import JaxprInterpreter
+    fn, make = W.WORKLOADS['gather_scatter']
+    closed = mj.make_jaxpr(fn)(*make())
+    kernels = lambda **kw: [l.kernel for l in JaxprInterpreter(closed, plan_only=True, **kw).launches]
+    assert len(kernels()) == 7 and len(kernels(fuse=False)) == 8
+    ops.REUSE_EQUAL_EQUATIONS = False
+    try:
+        assert len(kernels()) == 9 and len(kernels(fuse=False)) == 11
+    finally:
+        ops.REUSE_EQUAL_EQUATIONS = True
+    def f(x):
+        a = (x + 1.0) * (x + 1.0)          #x + 1 once
+        b = (x + 2.0) * (x + np.float32(1.0))
+        return a + b, x + 1.0              #the result x + 1 is an equation of its own
+    x = np.zeros((8, 4), np.float32)
+    interp = JaxprInterpreter(mj.make_jaxpr(f)(x), plan_only=True, fuse=False)
+    names = [str(op.equation.primitive) for op in interp.all_ops]
+    assert names.count('add') == 4 and names.count('mul') == 2, names          #x+1, x+2, a+b, the result x+1
+
+
 # ------------------------------------------------------------------ boundary details
 
 def test_reference_module_path_resolves():

@@ -84,6 +84,8 @@ def analyze_jaxpr(bufferpool: BufferPool, jaxpr) -> tp.List[Op]:
         method = globals().get(opname, None)
         if method is None or not callable(method) or opname.startswith('_'):
             raise NotImplementedError(eq)
+        if _reuse_equal_equation(bufferpool, eq):
+            continue
         position   = bufferpool.op_counter
         method_ops = method(bufferpool, eq)
         for op in method_ops:
@@ -91,6 +93,47 @@ def analyze_jaxpr(bufferpool: BufferPool, jaxpr) -> tp.List[Op]:
                 op.index = position
         all_ops += method_ops
     return all_ops
+
+
+#Set to False to evaluate every equation, also one that repeats an earlier one.
+REUSE_EQUAL_EQUATIONS = True
+
+
+def _reuse_equal_equation(bufferpool: BufferPool, eq) -> bool:
+    '''An element-wise or shape equation with the primitive, parameters and operands of an earlier one computes the same
+    array: its result variable is bound to that equation's buffer and nothing is launched. (Tracing `x[i]` and
+    `x.at[i].add(u)` normalises the same index array twice, three equations each time.) Results of the program keep
+    their own storage and equation.'''
+    from .buffers import hashable
+    name = eq.primitive.name
+    if not REUSE_EQUAL_EQUATIONS or len(eq.outvars) != 1 or not (name in _BINARY or name in _UNARY or name in _REUSABLE_OTHERS):
+        return False
+    outvar = eq.outvars[0]
+    if hashable(outvar) in bufferpool.buffers:
+        return False                                       #a result of the program
+    operands = []
+    for v in eq.invars:
+        if core.is_literal(v):
+            value = np.asarray(v.val)
+            operands.append(('literal', str(value.dtype), value.shape, value.tobytes()))
+        else:
+            b = bufferpool.buffers.get(hashable(v))
+            if b is None:
+                return False
+            operands.append((id(b._placeholder), str(b.dtype), b.shape))
+    params = _params_without_jax_bookkeeping(eq.params)
+    key = (name, repr(sorted(params.items())), tuple(operands), str(outvar.aval.dtype), tuple(outvar.aval.shape))
+    seen = bufferpool.__dict__.setdefault('_equal_equations', {})
+    earlier = seen.get(key)
+    if earlier is None:
+        seen[key] = outvar
+        return False
+    bufferpool.set_buffer(outvar, bufferpool.get_buffer(earlier))
+    return True
+
+
+_REUSABLE_OTHERS = {'select', 'select_n', 'convert_element_type', 'integer_pow', 'square', 'reshape', 'broadcast_in_dim',
+                    'squeeze', 'expand_dims'}
 
 
 # ------------------------------------------------------------------ dtype helpers
