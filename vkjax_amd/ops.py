@@ -893,6 +893,13 @@ def gather(bufferpool, equation):
     if is_rows:
         row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
         n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
+        known   = getattr(indices, 'constant_value', None)
+        if n_idx == 1 and known is not None and operand.shape[0] > 0:
+            #one row whose number is known when the program is built (`keys[1]` of a split key, a static `x[3]`, which
+            #old jax versions trace as a gather with a constant index): a copy of that row, which the consumer's
+            #fusion can read in place. Clamped like any gather.
+            row = builtins_min(builtins_max(int(np.asarray(known).reshape(-1)[0]), 0), operand.shape[0] - 1)
+            return [_copy_op(equation, outbuf, EwOperand(operand, row * row_len, K.row_major_strides(outbuf.shape)))]
         return [Op(equation, launch=K.gather_rows(outbuf, operand, indices, n_idx, row_len, operand.shape[0]))]
     return [Op(equation, launch=K.gather_general(outbuf, operand, indices, offset_dims, collapsed, start_index_map, slice_sizes))]
 
