@@ -338,6 +338,26 @@ def test_affine_chains_in_straight_line_code():
     assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['ew_chain_v4_s4']
 
 
+def test_indices_that_count_from_the_end():
+    '''`x[i]` and `x.at[i].add(u)` with negative entries in i: tracing normalises the index as select(i < 0, i + n, i),
+    which runs as one launch (opcode WRAP_I) whose result both the gather and the scatter-add read. Bit-exact against
+    the oracle; the normalised index is also correct as a result of its own.'''
+    rng = np.random.default_rng(31)
+    table = rng.integers(-9, 10, size=(50, 12)).astype(np.float32)
+    idx = rng.integers(-50, 50, size=(7, 9)).astype(np.int32)
+    updates = rng.integers(-3, 4, size=(7, 9, 12)).astype(np.float32)
+    def f(t, i, u):
+        return t[i], mj.numpy.index_add(t, i, u)
+    _, _, fn = check_against_oracle(f, [table, idx, updates], exact=True)
+    ops_ = list(fn._jaxpr_interpreters.values())[0].all_ops
+    labels = [repr(op.equation) for op in ops_]
+    assert sum('add ; lt ; select' in l for l in labels) == 1, labels
+    def normalised(i):
+        return mj.lax.select(i < 0, i + 50, i)
+    check_against_oracle(normalised, [idx], exact=True)
+    check_against_oracle(lambda i: mj.lax.select(i < 0, i + 50, i) * 2, [np.array([-50, -1, 0, 49, -2147483648, 2147483647], np.int32)], exact=True)
+
+
 def test_return_all_and_profiling():
     '''The debugging surface of the reference: run(..., return_all=True) returns every variable
     (reference: vkjax/kompute_jaxpr_interpreter.py:85-89) and profiling=True returns per-op timings

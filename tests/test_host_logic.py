@@ -434,10 +434,10 @@ def test_repeated_equations_are_evaluated_once():
     fn, make = W.WORKLOADS['gather_scatter']
     closed = mj.make_jaxpr(fn)(*make())
     kernels = lambda **kw: [l.kernel for l in JaxprInterpreter(closed, plan_only=True, **kw).launches]
-    assert len(kernels()) == 7 and len(kernels(fuse=False)) == 8
+    assert len(kernels()) == 6 and len(kernels(fuse=False)) == 8          #(fused: x + n, x < 0 and the select in one pass)
     ops.REUSE_EQUAL_EQUATIONS = False
     try:
-        assert len(kernels()) == 9 and len(kernels(fuse=False)) == 11
+        assert len(kernels()) == 7 and len(kernels(fuse=False)) == 11
     finally:
         ops.REUSE_EQUAL_EQUATIONS = True
     def f(x):

@@ -139,6 +139,7 @@ __device__ __forceinline__ void ew_apply_vec(uint32_t op, uint32_t (&acc)[VEC], 
         EW_CASE(EW_CVT_U2F, f2u((float)a))
         EW_CASE(EW_CVT_F2B, x != 0.f)
         EW_CASE(EW_CVT_X2B, a != 0u)
+        EW_CASE(EW_WRAP_I,  p < 0 ? a + b : a)
         default:
 #pragma unroll
             for (int j = 0; j < VEC; ++j)

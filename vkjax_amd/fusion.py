@@ -282,6 +282,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
     ops = fuse_scale_relu_backward(ops, bufferpool, outvars)
     ops = fuse_reduce_prologues(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
+    ops = fuse_index_wrap(ops, bufferpool, outvars)
     ops = fuse_dense_softmax(ops, bufferpool, outvars)
     ops = remove_dead_ops(ops, bufferpool, outvars)
     return batch_small_chains(ops)
@@ -342,6 +343,42 @@ def fuse_softmax(ops, bufferpool, outvars):
             b._placeholder.elided = True
         removed |= {i, i + 1, i + 2}
         replacement[i + 3 + (arg_out is not None)] = fused
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
+
+
+def fuse_index_wrap(ops, bufferpool, outvars):
+    '''`select(x < 0, x + n, x)` on int32, the way tracing normalises an index that may count from the end, is two
+    launches after chain fusion (x + n, and the comparison with the select, which needs x + n as a second full-size
+    value). One opcode does it in one pass over x.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    writer = {pid(op.chain.out): i for i, op in enumerate(ops) if op.chain is not None}
+    same   = lambda a, b: a.buffer._placeholder is b.buffer._placeholder and a.offset == b.offset and tuple(a.strides) == tuple(b.strides)
+    single = lambda o: o is not None and all(s == 0 for s in o.strides)
+    removed, replacement = set(), {}
+    for i, B in enumerate(ops):
+        ch = B.chain
+        if ch is None or [st.op for st in ch.steps] != [EW['LT_I'], EW['SEL_P'], EW['NOP']]:
+            continue
+        less, pick, carrier = ch.steps
+        zero = getattr(less.operand.buffer, 'constant_value', None) if single(less.operand) else None
+        if (less.operand_left or zero is None or np_prod(zero.shape) != 1 or int(zero.reshape(-1)[0]) != 0
+                or not same(carrier.operand, ch.first) or not _is_full_contiguous_any_shape(pick.operand, ch.shape)):
+            continue
+        a = writer.get(pid(pick.operand.buffer))
+        if a is None or a >= i or a in removed or uses[pid(pick.operand.buffer)] != 1:
+            continue
+        A = ops[a].chain
+        if (tuple(A.shape) != tuple(ch.shape) or len(A.steps) != 1 or A.steps[0].op != EW['ADD_I'] or not single(A.steps[0].operand)
+                or not same(A.first, ch.first) or A.out.dtype != ch.first.buffer.dtype):
+            continue
+        fused = Op(_label(ops[a], B), chain=EwChain(ch.out, ch.shape, ch.first, [EwStep(EW['WRAP_I'], A.steps[0].operand)]))
+        fused.index = B.index
+        A.steps[0].operand.buffer.accesses.append(B.index)
+        pick.operand.buffer._placeholder.elided = True
+        removed.add(a)
+        replacement[i] = fused
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
 
 
