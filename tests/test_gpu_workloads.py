@@ -330,6 +330,23 @@ def test_affine_chains_in_straight_line_code():
             assert_tree_close(results[0], results[1], exact=True, what=f'{shape} {nsum} {parts}')
         check_against_oracle(lambda a, b, m, s, t, q: mj.nn.relu((a + b - m) * s + t + q), [first, s1, vsub, vmul, vadd, full][:6] if len(shape) > 1
                              else [first, s1, np.float32(0.5), np.float32(2.0), np.float32(-1.0), full], rtol=1e-5, atol=1e-6)
+    #arrays of more than 4 M elements: the variant that skips absent operands, same bits as the general kernel
+    big, res, m, k, t = r(1 << 16, 72), r(1 << 16, 72), r(72), r(72), r(72)
+    big[5, 7] = np.nan
+    for f, args in ((lambda x, m, k, t: mj.nn.relu((x - m) * k + t), [big, m, k, t]),
+                    (lambda x, y, m, k, t: mj.nn.relu((x - m) * k + t + y), [big, res, m, k, t]),
+                    (lambda x, y, z, w, t: x + y + z + w + t, [big, res, big[::-1].copy(), res[::-1].copy(), t])):
+        results = []
+        for forced in (None, False):
+            K.FORCE_EW_AFFINE = forced
+            try:
+                fn = vkjax_amd.wrap(f, frontend='minijax')
+                results.append(fn(*args))
+                kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+            finally:
+                K.FORCE_EW_AFFINE = None
+            assert kernels == (['ew_affine_big_v4'] if forced is None else [kernels[0]]) and (forced is None or kernels[0].startswith('ew_chain')), kernels
+        assert_tree_close(results[0], results[1], exact=True, what='large affine chain')
     #by itself: chains of more than four operands on arrays that are not large
     x, m, k, t = r(64, 7, 7, 64), r(64), r(64), r(64)
     _, _, fn = check_against_oracle(lambda x, m, k, t: mj.nn.relu((x - m) * k + t), [x, m, k, t], rtol=1e-5, atol=1e-6)

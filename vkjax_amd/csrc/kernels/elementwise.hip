@@ -203,8 +203,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
 // residual and ReLU): on contiguous float arrays of n elements whose fastest dimension has C elements,
 //     v = first + s1 + s2 + s3            (the first nsum of them, in this order)
 //     v = v - vsub[c]; v = v * vmul[c]; v = v + vadd[c]; v = v + full; v = max(v, floor)      (each optional, in this order)
-// Straight-line code: every load is issued through a buffer descriptor whose size is 0 for an absent operand (such a
-// load returns zeros without touching memory), every step is a select on a flag. The opcode interpreter of ew_chain
+// No interpreter: the operands that are present are told by flags. The opcode interpreter of ew_chain
 // spends 750 instructions and 170 branches per wave on such a chain, which is most of a small launch's duration and
 // a quarter of the bandwidth of a large one. n and C are multiples of 4; two 16-byte vectors per thread.
 struct EwAffineParams {
@@ -214,9 +213,14 @@ struct EwAffineParams {
     uint32_t flags;                 // bit0 - vsub, bit1 * vmul, bit2 + vadd, bit3 + full, bit4 max(., floor)
 };
 
-extern "C" __global__ __launch_bounds__(256) void ew_affine_v4(
-        float* __restrict__ out, const float* first, const float* s1, const float* s2, const float* s3,
-        const float* vsub, const float* vmul, const float* vadd, const float* full, const float* floor_, EwAffineParams P) {
+// SKIP = false: every load is issued, through a descriptor of size 0 for an absent operand (such a load returns zeros
+// without touching memory), and every step is a select on its flag: no taken branch, which is what a launch of a few
+// waves wants. SKIP = true: absent operands are skipped by uniform branches, which is what a large array wants (ten
+// loads per vector, most of them empty, cost it a quarter of its bandwidth).
+template <bool SKIP>
+__device__ __forceinline__ void ew_affine_body(float* __restrict__ out, const float* first, const float* s1, const float* s2, const float* s3,
+                                               const float* vsub, const float* vmul, const float* vadd, const float* full, const float* floor_,
+                                               const EwAffineParams& P) {
     constexpr int U = 2;
     const uint32_t nb = P.n * 4u, cb = P.cq * 16u, fl = P.flags;
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out, nb), r_first = make_rsrc(first, nb),
@@ -225,36 +229,67 @@ extern "C" __global__ __launch_bounds__(256) void ew_affine_v4(
         r_full = make_rsrc(full, (fl & 8u) ? nb : 0u), r_floor = make_rsrc(floor_, (fl & 16u) ? 4u : 0u);
     f32x4 a[U], b1[U], b2[U], b3[U], fu[U], vs[U], vm[U], va[U];
     uint32_t off[U];
+    float lo = 0.f;
+    // every load of both vectors is requested before anything is used
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint32_t v = (blockIdx.x * U + u) * 256u + threadIdx.x;          // vector index; beyond n / 4: every access is out of range
         const uint32_t q = P.cq_magic ? __umulhi(v, P.cq_magic) >> P.cq_shift : v;
         const uint32_t c = (P.cq == 1u ? 0u : v - q * P.cq) * 16u;
         off[u] = v * 16u;
-        a[u]  = buffer_load_x4(r_first, off[u]);
-        b1[u] = buffer_load_x4(r_s1, off[u]); b2[u] = buffer_load_x4(r_s2, off[u]); b3[u] = buffer_load_x4(r_s3, off[u]);
-        fu[u] = buffer_load_x4(r_full, off[u]);
-        vs[u] = buffer_load_x4(r_sub, c); vm[u] = buffer_load_x4(r_mul, c); va[u] = buffer_load_x4(r_add, c);
+        a[u] = buffer_load_x4(r_first, off[u]);
+        if (!SKIP || P.nsum >= 1u) b1[u] = buffer_load_x4(r_s1, off[u]);
+        if (!SKIP || P.nsum >= 2u) b2[u] = buffer_load_x4(r_s2, off[u]);
+        if (!SKIP || P.nsum >= 3u) b3[u] = buffer_load_x4(r_s3, off[u]);
+        if (!SKIP || (fl & 8u)) fu[u] = buffer_load_x4(r_full, off[u]);
+        if (!SKIP || (fl & 1u)) vs[u] = buffer_load_x4(r_sub, c);
+        if (!SKIP || (fl & 2u)) vm[u] = buffer_load_x4(r_mul, c);
+        if (!SKIP || (fl & 4u)) va[u] = buffer_load_x4(r_add, c);
     }
-    const float lo = buffer_load_x1(r_floor, 0u);
+    if (!SKIP || (fl & 16u)) lo = buffer_load_x1(r_floor, 0u);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        f32x4 y;
+        f32x4 y = a[u];
+        if constexpr (SKIP) {
+            if (P.nsum >= 1u) y = y + b1[u];
+            if (P.nsum >= 2u) y = y + b2[u];
+            if (P.nsum >= 3u) y = y + b3[u];
+            if (fl & 1u) y = y - vs[u];
+            if (fl & 2u) y = y * vm[u];
+            if (fl & 4u) y = y + va[u];
+            if (fl & 8u) y = y + fu[u];
+            if (fl & 16u) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float v = a[u][j];
-            v = P.nsum >= 1u ? v + b1[u][j] : v;
-            v = P.nsum >= 2u ? v + b2[u][j] : v;
-            v = P.nsum >= 3u ? v + b3[u][j] : v;
-            v = (fl & 1u) ? v - vs[u][j] : v;
-            v = (fl & 2u) ? v * vm[u][j] : v;
-            v = (fl & 4u) ? v + va[u][j] : v;
-            v = (fl & 8u) ? v + fu[u][j] : v;
-            v = (fl & 16u) ? ((v > lo || v != v) ? v : lo) : v;               // a NaN stays
-            y[j] = v;
+                for (int j = 0; j < 4; ++j) y[j] = (y[j] > lo || y[j] != y[j]) ? y[j] : lo;       // a NaN stays
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v = y[j];
+                v = P.nsum >= 1u ? v + b1[u][j] : v;
+                v = P.nsum >= 2u ? v + b2[u][j] : v;
+                v = P.nsum >= 3u ? v + b3[u][j] : v;
+                v = (fl & 1u) ? v - vs[u][j] : v;
+                v = (fl & 2u) ? v * vm[u][j] : v;
+                v = (fl & 4u) ? v + va[u][j] : v;
+                v = (fl & 8u) ? v + fu[u][j] : v;
+                v = (fl & 16u) ? ((v > lo || v != v) ? v : lo) : v;               // a NaN stays
+                y[j] = v;
+            }
         }
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 0);
     }
+}
+
+extern "C" __global__ __launch_bounds__(256) void ew_affine_v4(
+        float* __restrict__ out, const float* first, const float* s1, const float* s2, const float* s3,
+        const float* vsub, const float* vmul, const float* vadd, const float* full, const float* floor_, EwAffineParams P) {
+    ew_affine_body<false>(out, first, s1, s2, s3, vsub, vmul, vadd, full, floor_, P);
+}
+extern "C" __global__ __launch_bounds__(256) void ew_affine_big_v4(
+        float* __restrict__ out, const float* first, const float* s1, const float* s2, const float* s3,
+        const float* vsub, const float* vmul, const float* vadd, const float* full, const float* floor_, EwAffineParams P) {
+    ew_affine_body<true>(out, first, s1, s2, s3, vsub, vmul, vadd, full, floor_, P);
 }
 
 // Requests one word of every 64-byte line of the argument block at the very start of a kernel and waits for all of

@@ -207,19 +207,19 @@ def lower_ew_chain(chain: EwChain) -> Launch:
 
 #tests: None = where it applies, False = never
 FORCE_EW_AFFINE: tp.Optional[bool] = None
-EW_AFFINE_MAX_ELEMENTS = 1 << 22
+EW_AFFINE_BIG_ELEMENTS = 1 << 22
 
 
 def _as_affine_chain(chain: EwChain, n: int, dims, strides) -> tp.Optional[Launch]:
     '''ew_affine_v4 for float chains of the form ((first + s1 + s2 + s3) - vsub) * vmul + vadd + full, max(., floor)
     (every part optional, in this order; s and full arrays of the output's shape, v vectors over the fastest
-    dimension, floor one value), for chains of more than four operands on arrays of at most 16 MB, where the launch
-    is mostly the interpreter's latency. Shorter chains keep the general kernel (small ones are batched with their
-    neighbours), and so do large arrays: there the ten loads per vector, most of them through empty descriptors,
-    cost more than the interpreter (relu on 64 M elements 4.4 TB/s against 5.7).'''
+    dimension, floor one value), for chains of more than four operands: a small launch is mostly the interpreter's
+    latency, and on large arrays the interpreter's instructions cost a fifth of the bandwidth (batch norm + ReLU on
+    51 M elements 4.5 TB/s, here 5.7). Shorter chains keep the general kernel, which is as fast for them and whose
+    small launches are batched with their neighbours.'''
     operands = chain.operands()
     if (FORCE_EW_AFFINE is False or not chain.steps or any(o is None for o in operands) or n % 4 or dims[-1] % 4 or n * 4 >= 2**32 - 2**16
-            or len(dims) > 2 or (FORCE_EW_AFFINE is None and (len(operands) <= 4 or n > EW_AFFINE_MAX_ELEMENTS))
+            or len(dims) > 2 or (FORCE_EW_AFFINE is None and len(operands) <= 4)
             or any(np.dtype(b.dtype) != np.float32 for b in [chain.out] + [o.buffer for o in operands])):
         return None
     dense = row_major_strides(dims)
@@ -255,7 +255,9 @@ def _as_affine_chain(chain: EwChain, n: int, dims, strides) -> tp.Optional[Launc
                + [at(slot.get(b)) for b in range(5)])
     params  = _u32(n, C // 4, magic, shift, len(sums), sum(1 << b for b in slot))
     nbytes  = 4 * n + sum(4 * min(n, o.buffer.size) for o in operands)
-    return Launch('ew_affine_v4', (_cdiv(n // 4, 2 * BLOCK), 1, 1), (BLOCK, 1, 1), buffers, params, bytes_moved=nbytes)
+    #(arrays of more than 16 MB: the variant that skips absent operands instead of loading through empty descriptors)
+    kernel = 'ew_affine_big_v4' if n > EW_AFFINE_BIG_ELEMENTS else 'ew_affine_v4'
+    return Launch(kernel, (_cdiv(n // 4, 2 * BLOCK), 1, 1), (BLOCK, 1, 1), buffers, params, bytes_moved=nbytes)
 
 
 EW_BATCH_KERNELS     = ('ew_chain_v1_s2', 'ew_chain_v1_s4', 'ew_chain_v4_s2', 'ew_chain_v4_s4')
