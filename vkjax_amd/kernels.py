@@ -895,7 +895,8 @@ def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op:
     TI  = min(64, _pow2_at_least(_cdiv(inner, vec)))
     #few blocks with many rows each (the second stage of a split sum): narrower blocks, more of them, more thread rows
     #walking the rows side by side
-    while TI > 8 and _cdiv(inner, TI * vec) * nsplit * outer < 64 and _cdiv(R, nsplit) * TI >= 256 * 8:
+    #(up to the number of blocks below which small sums are batched with their neighbours into one launch)
+    while TI > 8 and 2 * _cdiv(inner, TI * vec) * nsplit * outer <= BATCH_MAX_BLOCKS and _cdiv(R, nsplit) >= 128:
         TI //= 2
     params = _u32(outer, R, inner, RED[op], ty, r_chunk, nsplit, TI)
     blocks = _cdiv(inner, TI * vec) * nsplit * outer
