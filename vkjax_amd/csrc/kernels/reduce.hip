@@ -87,24 +87,28 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
     const bool is_arg = MODE >= 3 || (MODE == 2 && P.op >= RED_ARGMAX), is_max = MODE == 3 || (MODE == 2 && P.op == RED_ARGMAX);
     const uint32_t ident = MODE == 0 ? 0u : MODE == 1 ? 0xFF800000u : red_identity(P.op, P.type);
     uint32_t acc[4] = {ident, ident, ident, ident}, best_i = 0xFFFFFFFFu, best_v = 0;
-    auto take = [&](uint32_t v, uint32_t r, int slot) {
+    // `ok` false: position r lies beyond the row's range and v holds the identity
+    auto take = [&](uint32_t v, uint32_t r, int slot, bool ok = true) {
         if constexpr (MODE >= 3) {
             // float argmax / argmin: a lane meets its elements in ascending index order, so on a tie the
             // earlier one stays; a NaN replaces any number and is never replaced
             const float x = u2f(v), y = u2f(best_v);
-            const bool better = (MODE == 3 ? x > y : x < y) || (x != x && y == y) || best_i == 0xFFFFFFFFu;
+            const bool better = ok && ((MODE == 3 ? x > y : x < y) || (x != x && y == y) || best_i == 0xFFFFFFFFu);
             best_v = better ? v : best_v;
             best_i = better ? r : best_i;
         } else if (is_arg) {
-            if (best_i == 0xFFFFFFFFu || arg_better(is_max, P.type, v, r, best_v, best_i)) { best_v = v; best_i = r; }
+            if (ok && (best_i == 0xFFFFFFFFu || arg_better(is_max, P.type, v, r, best_v, best_i))) { best_v = v; best_i = r; }
         } else {
-            acc[slot] = red_step<MODE>(P.op, P.type, acc[slot], v);
+            acc[slot] = red_step<MODE>(P.op, P.type, acc[slot], v);   // combining with the identity changes nothing
         }
     };
+    // Every lane of the wave takes the same number of steps, four loads in flight in each; in the last step
+    // the positions beyond the range are not loaded and count as the identity. (Lanes that left the
+    // four-load loop one by one would each wait for their remaining loads in turn.)
     if constexpr (VEC == 4) {
-        // r_lo, R and the row starts are multiples of 4 (the host checks); four loads in flight per lane
-        uint32_t r = r_lo + lane * 4u;
-        for (; r + 3u * 256u < r_hi; r += 4u * 256u) {
+        // r_lo, R and the row starts are multiples of 4 (the host checks)
+        uint32_t r = r_lo + lane * 4u, base = r_lo;
+        for (; base + 4u * 256u <= r_hi; base += 4u * 256u, r += 4u * 256u) {
             u32x4 v[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) v[q] = *reinterpret_cast<const u32x4*>(row + r + q * 256u);
@@ -113,20 +117,42 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
                 take(v[q].x, r + q * 256u, 0); take(v[q].y, r + q * 256u + 1u, 1); take(v[q].z, r + q * 256u + 2u, 2); take(v[q].w, r + q * 256u + 3u, 3);
             }
         }
-        for (; r < r_hi; r += 256u) {                                    // r_hi - r_lo is a multiple of 4 too
-            const u32x4 v = *reinterpret_cast<const u32x4*>(row + r);
-            take(v.x, r, 0); take(v.y, r + 1u, 1); take(v.z, r + 2u, 2); take(v.w, r + 3u, 3);
+        if (base < r_hi) {                                               // r_hi - r_lo is a multiple of 4 too
+            u32x4 v[4];
+            bool ok[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                ok[q] = r + q * 256u < r_hi;
+                v[q] = u32x4{ident, ident, ident, ident};
+                if (ok[q]) v[q] = *reinterpret_cast<const u32x4*>(row + r + q * 256u);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                take(v[q].x, r + q * 256u, 0, ok[q]); take(v[q].y, r + q * 256u + 1u, 1, ok[q]);
+                take(v[q].z, r + q * 256u + 2u, 2, ok[q]); take(v[q].w, r + q * 256u + 3u, 3, ok[q]);
+            }
         }
     } else {
-        uint32_t r = r_lo + lane;
-        for (; r + 3u * 64u < r_hi; r += 4u * 64u) {
+        uint32_t r = r_lo + lane, base = r_lo;
+        for (; base + 4u * 64u <= r_hi; base += 4u * 64u, r += 4u * 64u) {
             uint32_t v[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) v[q] = row[r + q * 64u];
 #pragma unroll
             for (int q = 0; q < 4; ++q) take(v[q], r + q * 64u, q);
         }
-        for (; r < r_hi; r += 64u) take(row[r], r, 0);
+        if (base < r_hi) {
+            uint32_t v[4];
+            bool ok[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                ok[q] = r + q * 64u < r_hi;
+                v[q] = ident;
+                if (ok[q]) v[q] = row[r + q * 64u];
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) take(v[q], r + q * 64u, q, ok[q]);
+        }
     }
     uint32_t a = acc[0];
     if (!is_arg) {
@@ -221,8 +247,10 @@ __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, con
                 if constexpr (PRO == PRO_NEG)  v[j] ^= 0x80000000u;
             }
         };
-        uint32_t r = r_lo + tr;
-        for (; r + 3u * TR < r_hi; r += 4u * TR) {                    // four loads in flight per thread
+        // all thread rows take the same number of steps, four loads in flight per thread in each; the last
+        // step leaves out the rows beyond the range
+        uint32_t r = r_lo + tr, first = r_lo;
+        for (; first + 4u * TR <= r_hi; first += 4u * TR, r += 4u * TR) {
             uint32_t v[4][VEC];
 #pragma unroll
             for (int q = 0; q < 4; ++q) fetch(r + q * TR, v[q]);
@@ -231,11 +259,16 @@ __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, con
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) take(v[q][j], r + q * TR, j);
         }
-        for (; r < r_hi; r += TR) {
-            uint32_t v[VEC];
-            fetch(r, v);
+        if (first < r_hi) {
+            uint32_t v[4][VEC];
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) take(v[j], r, j);
+            for (int q = 0; q < 4; ++q) if (r + q * TR < r_hi) fetch(r + q * TR, v[q]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (r + q * TR < r_hi) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) take(v[q][j], r + q * TR, j);
+                }
         }
     }
 #pragma unroll
@@ -393,18 +426,22 @@ __device__ __forceinline__ void scale_relu_backward_body(float* __restrict__ dx,
             if constexpr (VEC == 4) *reinterpret_cast<f32x4*>(dx + off) = f32x4{d[0], d[1], d[2], d[3]};
             else dx[off] = d[0];
         };
-        uint32_t r = r_lo + tr;
-        for (; r + 3u * TR < r_hi; r += 4u * TR) {                    // four rows in flight per thread
+        // all thread rows take the same number of steps, four rows in flight per thread in each; the last
+        // step leaves out the rows beyond the range
+        uint32_t r = r_lo + tr, first = r_lo;
+        for (; first + 4u * TR <= r_hi; first += 4u * TR, r += 4u * TR) {
             float a[4][VEC], c[4][VEC], v[4][VEC];
 #pragma unroll
             for (int q = 0; q < 4; ++q) fetch(r + q * TR, a[q], c[q], v[q]);
 #pragma unroll
             for (int q = 0; q < 4; ++q) take(r + q * TR, a[q], c[q], v[q]);
         }
-        for (; r < r_hi; r += TR) {
-            float a[VEC], c[VEC], v[VEC];
-            fetch(r, a, c, v);
-            take(r, a, c, v);
+        if (first < r_hi) {
+            float a[4][VEC], c[4][VEC], v[4][VEC];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) if (r + q * TR < r_hi) fetch(r + q * TR, a[q], c[q], v[q]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) if (r + q * TR < r_hi) take(r + q * TR, a[q], c[q], v[q]);
         }
     }
 #pragma unroll
@@ -452,21 +489,16 @@ template <int VEC, class F>
 __device__ __forceinline__ float row_sum_as_reduce_rows(F value_at, uint32_t R, uint32_t lane) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if constexpr (VEC == 4) {
-        uint32_t r = lane * 4u;
-        for (; r + 3u * 256u < R; r += 4u * 256u)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] += value_at(r + q * 256u + j);
-        for (; r < R; r += 256u)
+        for (uint32_t r = lane * 4u; r < R; r += 256u)
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[j] += value_at(r + j);
     } else {
         uint32_t r = lane;
-        for (; r + 3u * 64u < R; r += 4u * 64u)
+        for (int q = 0; r < R; r += 64u, q = (q + 1) & 3) {
+            const float v = value_at(r);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) acc[q] += value_at(r + q * 64u);
-        for (; r < R; r += 64u) acc[0] += value_at(r);
+            for (int j = 0; j < 4; ++j) acc[j] += j == q ? v : 0.f;     // the sums are never -0, so adding 0 keeps them
+        }
     }
     float a = (acc[0] + acc[1]) + (acc[2] + acc[3]);
 #pragma unroll
