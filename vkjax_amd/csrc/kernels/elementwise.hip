@@ -430,21 +430,27 @@ struct PadParams {
     uint32_t step[PAD_MAX_RANK];          // interior + 1
 };
 
+// 32-bit index arithmetic (the host keeps both arrays below 2^32 - 2^12 elements); dimensions of extent 1 and
+// steps of 1 cost no division: those branches are the same for the whole launch.
 template <int VEC>
 __device__ __forceinline__ void pad_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
                                          const uint32_t* __restrict__ value, const PadParams& P) {
-    const uint64_t e0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * VEC;
+    const uint32_t e0 = (blockIdx.x * 256u + threadIdx.x) * VEC;
     if (e0 >= P.n) return;
-    uint64_t r = e0, off = 0, mul = 1;
+    uint32_t r = e0, off = 0, mul = 1;
     bool inside = true;
 #pragma unroll
     for (int d = PAD_MAX_RANK - 1; d >= 0; --d) {
-        const uint64_t q = r / P.out_dims[d];
-        const int64_t  p = (int64_t)(r - q * P.out_dims[d]) - P.low[d];
-        r = q;
-        const int64_t i = p / (int64_t)P.step[d];
-        inside = inside && p >= 0 && i * (int64_t)P.step[d] == p && i < (int64_t)P.in_dims[d];
-        off += (uint64_t)i * mul;
+        const uint32_t od = P.out_dims[d], step = P.step[d];
+        if (od == 1u && P.low[d] == 0 && P.in_dims[d] == 1u) continue;
+        uint32_t c = r;
+        if (d > 0) { const uint32_t q = r / od; c = r - q * od; r = q; }   // the slowest dimension needs no split
+        const int32_t p = (int32_t)c - P.low[d];
+        uint32_t i = (uint32_t)p;
+        bool on_grid = true;
+        if (step != 1u) { i = (uint32_t)p / step; on_grid = i * step == (uint32_t)p; }
+        inside = inside && p >= 0 && on_grid && i < P.in_dims[d];
+        off += i * mul;
         mul *= P.in_dims[d];
     }
     const uint32_t v = value[0];

@@ -1024,18 +1024,34 @@ def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, selected: B
 PAD_MAX_RANK = 6
 
 
+def _merged_pad_dims(out_shape, in_shape, padding_config):
+    '''(out extent, in extent, low, step) per dimension after folding every dimension the padding leaves alone into
+    the one before it when that one has no interior padding: (w, c) -> w * C + c turns `low` into low * C.'''
+    dims = [(int(o), int(i), int(c[0]), int(c[2]) + 1) for o, i, c in zip(out_shape, in_shape, padding_config)]
+    merged: tp.List[tp.Tuple[int, int, int, int]] = []
+    for o, i, low, step in reversed(dims):
+        if merged:
+            o2, i2, low2, step2 = merged[-1]
+            if low2 == 0 and step2 == 1 and o2 == i2 and step == 1:
+                merged[-1] = (o * o2, i * o2, low * o2, 1)
+                continue
+        merged.append((o, i, low, step))
+    return merged[::-1]
+
+
 def pad(out: Buffer, inp: Buffer, value: Buffer, padding_config) -> Launch:
-    rank = len(inp.shape)
-    if rank > PAD_MAX_RANK:
+    dims = _merged_pad_dims(out.shape, inp.shape, padding_config)
+    if len(dims) > PAD_MAX_RANK:
         raise NotImplementedError('pad with rank > 6')
-    lead = PAD_MAX_RANK - rank
-    config   = [(0, 0, 0)] * lead + [tuple(int(v) for v in c) for c in padding_config]
-    in_dims  = [1] * lead + list(inp.shape)
-    out_dims = [1] * lead + list(out.shape)
-    #an empty operand contributes nothing: give the kernel a dimension no index can fall into
-    in_dims  = [max(d, 0) for d in in_dims]
-    vec = 4 if (config[-1] == (0, 0, 0) and out_dims[-1] % 4 == 0) else 1
-    params = _u32(out.size, *out_dims, *in_dims) + _i32(*[c[0] for c in config]) + _u32(*[c[2] + 1 for c in config])
+    if max(out.size, inp.size) >= 2**32 - 2**12 or any(abs(d[2]) >= 2**31 for d in dims):
+        raise NotImplementedError('pad of arrays with 2^32 elements or more')
+    #the dimensions fill the front of the tables (the kernel does not split its index for dimension 0) and the unused
+    #ones behind them have extent 1; an empty operand keeps an extent of 0 no index can fall into
+    dims = dims + [(1, 1, 0, 1)] * (PAD_MAX_RANK - len(dims))
+    last = max((d for d in range(PAD_MAX_RANK) if dims[d][:3] != (1, 1, 0)), default=0)
+    o, i, low, step = dims[last]
+    vec = 4 if (step == 1 and low % 4 == 0 and o % 4 == 0 and i % 4 == 0) else 1
+    params = _u32(out.size, *[d[0] for d in dims], *[d[1] for d in dims]) + _i32(*[d[2] for d in dims]) + _u32(*[d[3] for d in dims])
     return Launch(f'pad_nd_v{vec}', (_cdiv(_cdiv(out.size, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                   [(out, 0), (inp, 0), (value, 0)], params, bytes_moved=4 * (inp.size + out.size))
 
