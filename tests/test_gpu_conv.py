@@ -335,8 +335,17 @@ def test_stem_kernel_for_few_input_features():
     def bias_relu(stride, padding):
         return lambda x, k, b: nn.relu(lax.conv_general_dilated(x, k, (stride, stride), padding, dimension_numbers=dn) + b)
 
+    def centred_and_activated(x, k, mean, scale, beta):           #a second result after the `- vector` step (what a training step keeps)
+        y = lax.conv_general_dilated(x, k, (2, 2), ((3, 3), (3, 3)), dimension_numbers=dn) - mean
+        return y, nn.relu(y * scale + beta)
+    def raw_and_activated(x, k, scale, beta):                      #a second result before the first step
+        y = lax.conv_general_dilated(x, k, (2, 2), ((3, 3), (3, 3)), dimension_numbers=dn)
+        return y, nn.relu(y * scale + beta)
+
     p3 = ((3, 3), (3, 3))
-    cases = [(bn_relu(2, p3), [ints(-4, 5, 2, 128, 128, 3), ints(-3, 4, 7, 7, 3, 64), vec(-5, 5, 64), np.ones(64, np.float32), vec(1, 4, 64) * 2, vec(-9, 9, 64)]),
+    cases = [(centred_and_activated, [ints(-4, 5, 2, 128, 128, 3), ints(-3, 4, 7, 7, 3, 64), vec(-5, 5, 64), vec(1, 4, 64), vec(-9, 9, 64)]),
+             (raw_and_activated, [ints(-4, 5, 3, 128, 192, 3), ints(-3, 4, 7, 7, 3, 48), vec(1, 4, 48), vec(-9, 9, 48)]),
+             (bn_relu(2, p3), [ints(-4, 5, 2, 128, 128, 3), ints(-3, 4, 7, 7, 3, 64), vec(-5, 5, 64), np.ones(64, np.float32), vec(1, 4, 64) * 2, vec(-9, 9, 64)]),
              (conv(2, p3), [ints(-4, 5, 3, 20, 192, 3), ints(-3, 4, 7, 7, 3, 40)]),
              (bias_relu(1, p3), [ints(-4, 5, 1, 12, 64, 3), ints(-3, 4, 7, 7, 3, 64), vec(-9, 9, 64)]),
              (conv(2, ((3, 3), (5, 5))), [ints(-4, 5, 2, 16, 128, 2), ints(-3, 4, 7, 11, 2, 24)]),
@@ -346,8 +355,11 @@ def test_stem_kernel_for_few_input_features():
         print(f'stem kernel: {[a.shape for a in args]}', flush=True)
         for fuse in (True, False):
             _, _, fn = check_against_oracle(f, args, exact=True, fuse=fuse)
-            kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches if l.kernel.startswith('conv_gemm')]
+            launches = list(fn._jaxpr_interpreters.values())[0].launches
+            kernels = [l.kernel for l in launches if l.kernel.startswith('conv_gemm')]
             assert kernels == ['conv_gemm_stem_7x22'], kernels
+            if fuse and 'and_activated' in f.__name__:
+                assert len(launches) == 1, [l.kernel for l in launches]       #both results from the one launch
     #a shape it does not take falls back to the general kernel
     _, _, fn = check_against_oracle(conv(2, p3), [ints(-4, 5, 2, 30, 26, 3), ints(-3, 4, 7, 7, 3, 64)], exact=True)
     assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['conv_gemm_64x64x32_gf']

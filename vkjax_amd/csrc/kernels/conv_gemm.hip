@@ -990,10 +990,21 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
         const uint32_t slots = (P.flags >> 20) & 31u;
         const int col = wn * 32 + l32;
         const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u), e_max = __builtin_popcount(slots & 15u);
+        const uint32_t base = col < P.N ? (uint32_t)((t * 64 + wm * 32 + 4 * half) * P.N + col) * 4u : CONV_OOB;
+        const uint32_t rowb = (uint32_t)P.N * 4u;
+        // a second result (bits 12-15 of the flags, as in conv_gemm_body): the value as it stands before (1) or after (2) the first step
+        const int tap = (int)((P.flags >> 12) & 15u) - 1;
+        const auto tap_store = [&]() {
+            const auto t_rsrc = make_rsrc(epi.p[CONV_MAX_EPI - 1], P.out_bytes);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) buffer_store_x1(y[v], t_rsrc, base, (uint32_t)(8 * (v / 4) + (v % 4)) * rowb);
+        };
+        if (tap == 0) tap_store();
         if (slots & 1u) {
             const float o = Es[col];
 #pragma unroll
             for (int v = 0; v < 16; ++v) y[v] = y[v] - o;
+            if (tap == 1) tap_store();
         }
         if (slots & 2u) {
             const float o = Es[e_mul * BN + col];
@@ -1010,8 +1021,6 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
 #pragma unroll
             for (int v = 0; v < 16; ++v) y[v] = (y[v] > o || y[v] != y[v]) ? y[v] : o;
         }
-        const uint32_t base = col < P.N ? (uint32_t)((t * 64 + wm * 32 + 4 * half) * P.N + col) * 4u : CONV_OOB;
-        const uint32_t rowb = (uint32_t)P.N * 4u;
 #pragma unroll
         for (int v = 0; v < 16; ++v) buffer_store_x1(y[v], o_rsrc, base, (uint32_t)(8 * (v / 4) + (v % 4)) * rowb);
     }

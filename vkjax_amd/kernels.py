@@ -596,7 +596,7 @@ FORCE_CONV_STEM: tp.Optional[bool] = None       #the patch kernel for few input 
 def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_units, lhs_offset, rhs_offset, out_offset) -> tp.Optional[Launch]:
     '''conv_gemm_stem_7x22 where it applies: dense images with so few features that KW * Cin is 21 or 22 (7 x 7 x 3),
     seven kernel rows, a template epilogue; see the conditions listed at the kernel.'''
-    if FORCE_CONV_STEM is False or FORCE_CONV_TILE is not None or FORCE_CONV_GENERAL or taps or lhs_offset or rhs_offset or out_offset:
+    if FORCE_CONV_STEM is False or FORCE_CONV_TILE is not None or FORCE_CONV_GENERAL or lhs_offset or rhs_offset or out_offset:
         return None
     M, N, K = g.M, g.N, g.K
     RL, WC = g.KW * g.Cin, g.W * g.Cin
@@ -613,13 +613,19 @@ def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_
           and STEM_PATCH_ROWS * pitch <= STEM_PATCH_FLOATS and STEM_PATCH_ROWS * (WC // 4) <= 256 * STEM_VECTORS_PER_THREAD)
     if not ok:
         return None
-    flags  = slots << 20
+    #a second result (the value before or after the first epilogue step) goes to the last operand slot, as in conv_gemm_body
+    flags  = slots << 20 | ((taps[0][0] + 1) << 12 if taps else 0)
     params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, pitch, left)
               + _u32(flags, lhs.size * 4, rhs.size * 4, out.size * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo)))
     derived_ptrs, derived_desc = _conv_derived(epilogue, N)
     params += derived_desc
-    buffers = [(out, 0), (lhs, 0), (rhs, 0)] + _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0)) + derived_ptrs
+    operand_slots = _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
+    if taps:
+        assert operand_slots[-1] == (None, 0)
+        operand_slots[-1] = (taps[0][1], 0)
+    buffers = [(out, 0), (lhs, 0), (rhs, 0)] + operand_slots + derived_ptrs
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
+    nbytes += 4 * taps[0][1].size if taps else 0
     return Launch('conv_gemm_stem_7x22', (min(M // 64, 2 * compute_units), 1, 1), (256, 1, 1), buffers, params,
                   bytes_moved=nbytes, flops=2 * M * N * K)
 
