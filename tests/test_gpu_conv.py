@@ -158,6 +158,7 @@ def test_lean_kernel_tile_chunks_with_epilogue(tile, bk):
         return nn.relu(lax.conv_general_dilated(x, k, (2, 2), 'VALID', dimension_numbers=dn) + bias)
 
     K.FORCE_CONV_TILE, K.FORCE_CONV_BK = tile, bk
+    blocks_per_cu, min_tiles = K.CONV_BLOCKS_PER_CU, K.CONV_EVEN_SPLIT_MIN_TILES
     try:
         for chunk in (1, 2, 3, 5):
             K.FORCE_CONV_CHUNK = chunk
@@ -172,8 +173,27 @@ def test_lean_kernel_tile_chunks_with_epilogue(tile, bk):
                     _, _, fn = check_against_oracle(f, args, exact=True)
                     launches = list(fn._jaxpr_interpreters.values())[0].launches
                     assert [l.kernel for l in launches] == [f'conv_gemm_{tile}x{bk}_lean'], [l.kernel for l in launches]
+        # a grid of a fixed number of blocks that share the M tiles of every N tile evenly (here 1, 2, 3 or 5 blocks
+        # per N tile: runs of unequal length, blocks with a single tile, one block with all of them)
+        K.FORCE_CONV_CHUNK, K.CONV_EVEN_SPLIT_MIN_TILES = None, 0.0
+        for per_n_tile in (1, 2, 3, 5):
+            for ksize, cin, cout in ((3, 64, 40), (1, 128, 72)):
+                tiles_n = -(-cout // int(tile.split('x')[1]))
+                K.CONV_BLOCKS_PER_CU = (per_n_tile * tiles_n + 0.5) / 256
+                print(f'tile {tile} bk {bk} {per_n_tile} blocks per N tile, kernel {ksize}x{ksize} {cin}->{cout}', flush=True)
+                x = rng.randint(-4, 5, size=[3, 13, 11, cin]).astype(np.float32)
+                k = rng.randint(-3, 4, size=[ksize, ksize, cin, cout]).astype(np.float32)
+                vec = lambda lo, hi: rng.randint(lo, hi, size=[cout]).astype(np.float32)
+                res = rng.randint(-50, 50, size=[3, 13, 11, cout]).astype(np.float32)
+                for f, args in ((bn_res_relu, [x, k, vec(-5, 5), vec(1, 4), vec(-9, 9), res]), (bias_relu, [x, k, vec(-9, 9)])):
+                    _, _, fn = check_against_oracle(f, args, exact=True)
+                    launches = list(fn._jaxpr_interpreters.values())[0].launches
+                    assert [l.kernel for l in launches] == [f'conv_gemm_{tile}x{bk}_lean'], [l.kernel for l in launches]
+                    tiles_m = -(-launches[0].buffers[0][0].size // cout // int(tile.split('x')[0]))
+                    assert launches[0].grid[0] == min(per_n_tile, tiles_m) * tiles_n, (launches[0].grid, tiles_m, tiles_n)
     finally:
         K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = None
+        K.CONV_BLOCKS_PER_CU, K.CONV_EVEN_SPLIT_MIN_TILES = blocks_per_cu, min_tiles
 
 
 def test_four_waves_per_tile_kernel():

@@ -368,7 +368,7 @@ def test_long_contractions_of_few_tiles_are_sliced():
     assert [l.kernel for l in interp.launches] == ['conv_gemm_32x32x128_ks4', 'ew_affine_v4']       #sum of four slices + bias, ReLU
     first, second = interp.launches
     assert first.grid == (32 * 4, 1, 1) and first.buffers[0][0].shape == (4, 49 * 512)
-    assert np.frombuffer(first.params, np.int32)[-1 - 9] == 9      #k steps per slice: the last word before the 9 of ConvDerived
+    assert np.frombuffer(first.params, np.int32)[-2 - 9] == 9      #k steps per slice: the last word but one before the 9 of ConvDerived
     assert second.buffers[0][0] is interp.output_buffers[0]
     assert len(plan(49, 4608, 512, fuse=False).launches) == 4      #slices, their sum, add, max
     assert [l.kernel for l in plan(49, 640, 512).launches] == ['conv_gemm_32x32x128_ks4']        #5 k steps: too short to slice
@@ -506,3 +506,19 @@ def test_index_modes_that_change_results_are_refused():
         else:
             with pytest.raises(NotImplementedError, match='mode'):
                 JaxprInterpreter(closed, plan_only=True)
+
+
+def test_evenly_split_conv_grids():
+    '''Layers with at least 4.5 tiles per resident block get a grid of exactly 5 blocks per CU whose blocks share the
+    M tiles of every N tile evenly; smaller ones keep one block per run of `chunk` tiles.'''
+    from vkjax_amd import kernels as K
+    assert K.choose_conv_m_blocks(784, 8) == 160            #ResNet-50 bs64, 28 x 28 x 512 outputs: 6272 tiles, 4.9 per block
+    assert K.choose_conv_m_blocks(3136, 2) == 640
+    assert K.choose_conv_m_blocks(3136, 1) == 0             #2.45 tiles per block: one more or less would unbalance the CUs
+    assert K.choose_conv_m_blocks(10, 1) == 0
+    assert K.choose_conv_m_blocks(100000, 1) == 1280 and K.choose_conv_m_blocks(4, 4000) == 1
+    geom = K.ConvGeometry(batch=64, Ho=28, Wo=28, N=512, H=28, W=28, Cin=128, KH=1, KW=1, xs=(100352, 3584, 128, 1), ws=(65536, 65536, 512, 1), os=(401408, 14336, 512, 1))
+    b = lambda *shape: Buffer(None, np.float32, shape)
+    launch = K.conv_gemm(b(64, 28, 28, 512), b(64, 28, 28, 128), b(1, 1, 128, 512), geom)
+    assert launch.kernel == 'conv_gemm_64x64x32_lean' and launch.grid[0] == 1280
+    assert np.frombuffer(launch.params, np.int32)[-1 - 9] == 160   #the last word of ConvParams, before the 9 of ConvDerived
