@@ -222,32 +222,40 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(reinterpret_cast<const char*>(x) - x_bias, P.x_bytes + x_bias),
                                  w_rsrc = make_rsrc(w, P.w_bytes), o_rsrc = make_rsrc(out, P.out_bytes);
 
-    // Scalar and per-feature epilogue operands are fetched once per block, at its very start, and
-    // parked in LDS behind the first k tile's loads, so that the epilogue never waits on global
-    // memory for them. Thread t fetches column t of every step.
+    // Scalar and per-feature epilogue operands are fetched once per block and parked in LDS, so that the epilogue
+    // never waits on global memory for them. Thread t fetches column t of every step. Every step issues one load,
+    // whatever its kind, so that none waits for the one before: an absent operand, one that is derived below, or a
+    // full tensor (read in the epilogue) has a descriptor of size 0, which reads nothing and returns 0.
+    // Where a block is alone on its CU (the four-waves-per-tile kernels) they are requested right behind the first
+    // k tile's loads: one round trip to memory for both. Elsewhere they go first, and the other blocks' work covers them.
+    constexpr bool EPI_BEHIND_TILES = KSW > 1;
     float e_reg[CONV_MAX_EPI], d_in[CONV_MAX_DERIVED + 1];
-    if (tid < BN) {
+    uint32_t e_bytes[CONV_MAX_EPI], e_scale[CONV_MAX_EPI];       // (the same in every lane: worked out before the lanes part)
 #pragma unroll
-        for (int e = 0; e < CONV_MAX_EPI; ++e) {
-            const uint32_t kind = step_desc(e) >> 8;             // 0 beyond the last step
-            e_reg[e] = 0.f;
-            // (a step whose operand is derived below has no array: a descriptor of size 0 reads nothing)
-            const uint32_t present = epi.p[e] != nullptr ? 1u : 0u;
-            if (kind == 1) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], 4u * present), 0u);
-            else if (kind == 2) e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], (uint32_t)P.N * 4u * present), (uint32_t)(n0 + tid) * 4u);
-        }
-        if (Dk.nsteps) {
-            // the arrays of the derived operand: requested here, combined once the first k tile's loads are on their
-            // way (combining them here would hold the wave, and with it the block's first barrier, for a round trip
-            // to memory before any tile load is issued)
+    for (int e = 0; e < CONV_MAX_EPI; ++e) {
+        const uint32_t kind = step_desc(e) >> 8;                 // 0 beyond the last step
+        const uint32_t present = epi.p[e] != nullptr ? 1u : 0u;
+        e_bytes[e] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(kind == 1 ? 4u * present : kind == 2 ? (uint32_t)P.N * 4u * present : 0u));
+        e_scale[e] = kind == 2 ? 4u : 0u;
+    }
+    auto request_epilogue_operands = [&]() {
+        if (tid < BN) {
 #pragma unroll
-            for (int k = 0; k <= CONV_MAX_DERIVED; ++k) {
-                const bool vec = (Dk.vector_mask >> k) & 1u;
-                d_in[k] = buffer_load_x1(make_rsrc(Dp.p[k], Dp.p[k] == nullptr ? 0u : vec ? (uint32_t)P.N * 4u : 4u),
-                                         vec ? (uint32_t)(n0 + tid) * 4u : 0u);
+            for (int e = 0; e < CONV_MAX_EPI; ++e)
+                e_reg[e] = buffer_load_x1(make_rsrc(epi.p[e], e_bytes[e]), (uint32_t)(n0 + tid) * e_scale[e]);
+            if (Dk.nsteps) {
+                // the arrays of the derived operand: combined once the first k tile's loads are on their way (combining
+                // them at once would hold the wave, and with it the block's first barrier, for a round trip to memory)
+#pragma unroll
+                for (int k = 0; k <= CONV_MAX_DERIVED; ++k) {
+                    const bool vec = (Dk.vector_mask >> k) & 1u;
+                    d_in[k] = buffer_load_x1(make_rsrc(Dp.p[k], Dp.p[k] == nullptr ? 0u : vec ? (uint32_t)P.N * 4u : 4u),
+                                             vec ? (uint32_t)(n0 + tid) * 4u : 0u);
+                }
             }
         }
-    }
+    };
+    if constexpr (!EPI_BEHIND_TILES) request_epilogue_operands();
     // the first full-size operand (a residual input) is fetched for a whole tile at once, while
     // the tile's last k step is computed (for the largest tile that would not fit the register
     // file: it loads sub-tile by sub-tile in the epilogue)
@@ -476,6 +484,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     setup_rows(region.m_base + tile_m0 * BM);
     CONV_STAMP(1)
     load_tiles(kbase * BK);
+    if constexpr (EPI_BEHIND_TILES) request_epilogue_operands();
     if (tid < BN) {
         if (Dk.nsteps) {
             // the derived operand: same arithmetic, operation by operation, as the element-wise kernel
