@@ -580,14 +580,31 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         } else {
             // all k steps but the last: the next step's loads are in flight during the MFMAs
             for (int kt = 1; kt < ktiles; ++kt) {
+#ifdef CONV_PHASE_STAMPS
+                const unsigned long long c0 = clock64();
+#endif
                 store_tiles();
+#ifdef CONV_PHASE_STAMPS
+                __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0): the LDS writes have landed
+                const unsigned long long c1 = clock64();
+#endif
                 tile_barrier();
+#ifdef CONV_PHASE_STAMPS
+                const unsigned long long c2 = clock64();
+#endif
                 load_tiles((kbase + kt) * BK);
 #ifdef CONV_PHASE_STAMPS
                 if (kt == 1 && sub == 0) { CONV_STAMP(2) }
 #endif
                 compute();
+#ifdef CONV_PHASE_STAMPS
+                const unsigned long long c3 = clock64();
+#endif
                 tile_barrier();
+#ifdef CONV_PHASE_STAMPS
+                const unsigned long long c4 = clock64();
+                stamps[8] += c1 - c0; stamps[9] += c2 - c1; stamps[10] += c3 - c2; stamps[11] += c4 - c3; stamps[12] += 1;
+#endif
             }
             // last k step: the loads in flight are those of the next M tile's first step and of
             // the residual operand
