@@ -368,7 +368,7 @@ def test_long_contractions_of_few_tiles_are_sliced():
     assert [l.kernel for l in interp.launches] == ['conv_gemm_32x32x128_ks4', 'ew_affine_v4']       #sum of four slices + bias, ReLU
     first, second = interp.launches
     assert first.grid == (32 * 4, 1, 1) and first.buffers[0][0].shape == (4, 49 * 512)
-    assert np.frombuffer(first.params, np.int32)[-2 - 9] == 9      #k steps per slice: the last word but one before the 9 of ConvDerived
+    assert np.frombuffer(first.params, np.int32)[-4 - 9] == 9      #k steps per slice: the fourth word from the end of ConvParams, which the 9 of ConvDerived follow
     assert second.buffers[0][0] is interp.output_buffers[0]
     assert len(plan(49, 4608, 512, fuse=False).launches) == 4      #slices, their sum, add, max
     assert [l.kernel for l in plan(49, 640, 512).launches] == ['conv_gemm_32x32x128_ks4']        #5 k steps: too short to slice
@@ -521,4 +521,4 @@ def test_evenly_split_conv_grids():
     b = lambda *shape: Buffer(None, np.float32, shape)
     launch = K.conv_gemm(b(64, 28, 28, 512), b(64, 28, 28, 128), b(1, 1, 128, 512), geom)
     assert launch.kernel == 'conv_gemm_64x64x32_lean' and launch.grid[0] == 1280
-    assert np.frombuffer(launch.params, np.int32)[-1 - 9] == 160   #the last word of ConvParams, before the 9 of ConvDerived
+    assert np.frombuffer(launch.params, np.int32)[-3 - 9:-9].tolist() == [160, 4, 144]   #blocks per N tile, tiles each, blocks with one more: the end of ConvParams, before the 9 of ConvDerived

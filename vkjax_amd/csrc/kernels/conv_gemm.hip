@@ -79,8 +79,10 @@ struct ConvParams {
                                     // ceil(k steps / k_split_steps) blocks per tile; those of slice s store their sums, without an
                                     // epilogue, to the s-th [M, N] matrix behind out, and a later launch adds the slices
     int32_t m_blocks;               // lean kernels: 0, or the number of blocks that share the M tiles of one N tile as evenly as whole
-                                    // tiles allow (block b takes tiles [b * tiles_m / m_blocks, (b + 1) * tiles_m / m_blocks)); the
-                                    // M tiles per block in the flags are then ignored. For grids sized to what the GPU holds at once.
+                                    // tiles allow: every block takes m_each = tiles_m / m_blocks consecutive tiles, the first
+                                    // m_extra = tiles_m % m_blocks blocks one more; the M tiles per block in the flags are then
+                                    // ignored. For grids sized to what the GPU holds at once.
+    int32_t m_each, m_extra;
 };
 
 // The part of the output a block's tile number refers to: a grid of tiles_m x tiles_n tiles whose first row is
@@ -143,7 +145,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     // to itself the compiler fetches each field right before its first use; under load every such
     // fetch costs about a microsecond, and the prologue and the epilogue would each chain several.
     struct {
-        int32_t M, N, K, Ho, Wo, H, W, Cin, KH, KW, SH, SW, PH, PW, DH, DW, xs_b, xs_h, xs_w, tiles_m, tiles_n, m_blocks;
+        int32_t M, N, K, Ho, Wo, H, W, Cin, KH, KW, SH, SW, PH, PW, DH, DW, xs_b, xs_h, xs_w, tiles_m, tiles_n, m_blocks, m_each, m_extra;
         uint32_t flags, epi_desc[2], x_bytes, w_bytes, out_bytes, howo_magic, howo_shift, wo_magic, wo_shift;
     } P;
 #define CONV_PIN(f) P.f = Pk.f; asm volatile("" : "+s"(P.f));
@@ -154,7 +156,7 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     CONV_PIN(KH) CONV_PIN(KW) CONV_PIN(SH) CONV_PIN(SW) CONV_PIN(PH) CONV_PIN(PW) CONV_PIN(DH) CONV_PIN(DW)
     CONV_PIN(xs_b) CONV_PIN(xs_h) CONV_PIN(xs_w) CONV_PIN(tiles_m) CONV_PIN(tiles_n) CONV_PIN(flags)
     CONV_PIN(epi_desc[0]) CONV_PIN(epi_desc[1]) CONV_PIN(x_bytes) CONV_PIN(w_bytes) CONV_PIN(out_bytes)
-    CONV_PIN(howo_magic) CONV_PIN(howo_shift) CONV_PIN(wo_magic) CONV_PIN(wo_shift) CONV_PIN(m_blocks)
+    CONV_PIN(howo_magic) CONV_PIN(howo_shift) CONV_PIN(wo_magic) CONV_PIN(wo_shift) CONV_PIN(m_blocks) CONV_PIN(m_each) CONV_PIN(m_extra)
 #undef CONV_PIN
     static_assert(CONV_MAX_EPI == 6, "descriptor packing");
     auto step_desc = [&](int e) -> uint32_t { return ((e < 3 ? P.epi_desc[0] : P.epi_desc[1]) >> (10 * (e < 3 ? e : e - 3))) & 1023u; };
@@ -186,7 +188,10 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     // XCD a contiguous range of work so that the N-tiles of one M-tile share an L2.
     const int chunk = LEAN ? (P.flags >> 25) & 15u : 1;         // the general variants take one tile per block
     const int m_blocks = LEAN && KSW == 1 ? P.m_blocks : 0;
-    const int chunks_m = m_blocks > 0 ? m_blocks : (region.tiles_m + chunk - 1) / chunk;
+    // (every wave runs this once per block on the CU's one scalar unit: divisors that are powers of two, the usual
+    // case for the M tiles per block and the number of N tiles, cost a shift instead of the long division sequence)
+    auto div_small = [](int n, int d) { return (d & (d - 1)) == 0 ? n >> __builtin_ctz((unsigned)d) : n / d; };
+    const int chunks_m = m_blocks > 0 ? m_blocks : div_small(region.tiles_m + chunk - 1, chunk);
     int work = (int)blockIdx.x - region.first_block;
     // K_SPLIT kernels can share a tile's contraction among several blocks (for products with so few tiles that most
     // CUs would stay idle while a few fetch all the weights): slice s sums k steps [kbase, kbase + ktiles)
@@ -206,11 +211,11 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         const int total = chunks_m * region.tiles_n, per = total / 8;
         if (per > 0 && work < per * 8) work = (work & 7) * per + (work >> 3);
     }
-    const int chunk_m = work / region.tiles_n, tile_n = work - chunk_m * region.tiles_n;
+    const int chunk_m = div_small(work, region.tiles_n), tile_n = work - chunk_m * region.tiles_n;
     int tile_m0 = chunk_m * chunk, nsub = LEAN ? min(chunk, region.tiles_m - tile_m0) : 1;
     if (m_blocks > 0) {
-        tile_m0 = (int)((uint64_t)(uint32_t)chunk_m * (uint32_t)region.tiles_m / (uint32_t)m_blocks);
-        nsub    = (int)((uint64_t)(uint32_t)(chunk_m + 1) * (uint32_t)region.tiles_m / (uint32_t)m_blocks) - tile_m0;
+        tile_m0 = chunk_m * P.m_each + min(chunk_m, P.m_extra);
+        nsub    = P.m_each + (chunk_m < P.m_extra ? 1 : 0);
     }
     const int n0 = tile_n * BN;
     const int HoWo = P.Ho * P.Wo;

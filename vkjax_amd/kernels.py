@@ -857,7 +857,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
               #(rows beyond M are dropped by the descriptor's size: with slices, that of one slice's matrix)
               + _u32(flags, *descs, x_bytes, w_bytes, M * N * 4 if k_split_steps else (out.size - out_offset) * 4,
                      *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo))
-              + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os, split_tiles_m, k_split_steps, m_blocks))
+              + _i32(g.LH, g.LW, g.xs[3], *g.ws, *g.os, split_tiles_m, k_split_steps, m_blocks, tiles_m // m_blocks if m_blocks else 0, tiles_m % m_blocks if m_blocks else 0))
     derived_ptrs, derived_desc = _conv_derived(epilogue, N)
     params += derived_desc
     buffers = [(out, out_offset * 4), (lhs, lhs_offset * 4), (rhs, rhs_offset * 4)]
