@@ -162,6 +162,16 @@ def measure(workload, steps, warmup, batch=None, fuse=True, graph=False, profile
                             frac=round(achieved / PEAK_HBM_GBS, 4))
         roofline.update(traffic=measured_hbm_traffic(workload, dominant), launches_per_step=d['launches'],
                         avg_launch_ms=round(ms / d['launches'], 5), stamped_avg_launch_ms=round(d['stamped_ms'] / d['launches'], 5))
+        if dominant == 'threefry2x32':
+            #the draw is bound by the integer ALUs, not by its stores: 68 vector instructions per Threefry block of two
+            #words (20 rounds of add / rotate / xor, five key injections, counters, the uniform chain), 16 lanes per
+            #SIMD and clock; the time below is that floor at the device's nominal clock
+            props   = hip.Device.get().get_device_properties()
+            blocks  = sum(l.bytes_moved for l in prof.launches if kernel_family(l.kernel) == dominant) / 8
+            floor   = blocks * 68 / (props['compute_units'] * 4 * 16 * props['clock_khz'] * 1e3) * 1e3
+            longest = max(m for l, m in zip(prof.launches, stamped * scale) if kernel_family(l.kernel) == dominant)
+            roofline.update(valu_floor_ms=round(floor, 5), longest_launch_ms=round(float(longest), 5),
+                            frac_of_valu_floor=round(floor / float(longest), 4))
         result.update(roofline=roofline, kernels=kernels)
 
     if end_to_end:

@@ -80,6 +80,22 @@ def test_rng_small_and_full_bit_exact():
     assert 0.0 <= y.min() and y.max() < 1.0 and abs(y.mean() - 0.5) < 1e-3
 
 
+def test_randint_bit_exact():
+    '''jax.random.randint as the reference tests it (reference: tests/test_random.py:45-60: seed 0 and 50 random
+    seeds, shape [1], bounds 0 and 9999), then larger draws, negative and reversed bounds, a span over 2**16 (whose
+    products wrap in 32 bits, as they do in jax) and an upper bound beyond int32.'''
+    r = mj.random
+    fn = lambda k: r.randint(k, [1], 0, 9999)
+    wrapped = vkjax_amd.wrap(fn, frontend='minijax')
+    for seed in [0] + list(np.random.RandomState(3).randint(10000, size=50)):
+        key = r.PRNGKey(int(seed))
+        assert np.array_equal(wrapped(key), oracle_outputs(fn, [key])[0]), seed
+    for shape, lo, hi in (((257, 33), -5, 17), ((1000,), 0, 2**31 - 1), ((64, 64), 0, 2**31), ((5,), 7, 7), ((5,), 9, -9), ((4096,), 0, 100000)):
+        print(f'randint {shape} [{lo}, {hi})', flush=True)
+        y, _, _ = check_against_oracle(lambda k: r.randint(k, shape, lo, hi), [r.PRNGKey(11)], exact=True)
+        assert y.dtype == np.int32 and (y >= lo).all() and (y.astype(np.int64) < max(hi, lo + 1)).all()
+
+
 def test_random_stream_fusion_variants_bit_exact():
     '''The fused counter + block function + concatenate + chain launch against the oracle's
     one-primitive-at-a-time evaluation: lengths that are and are not multiples of 8 (16-byte and

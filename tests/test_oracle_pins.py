@@ -77,6 +77,24 @@ def test_random_bits_odd_sizes_pad_and_trim():
         assert np.array_equal(bits, np.concatenate([a, b])[:n])
 
 
+def test_randint_is_the_remainder_of_a_64_bit_draw():
+    '''randint composes a key split, two draws and 32-bit remainder arithmetic that stands for
+    (hi * 2**32 + lo) % span; with spans below 2**16 no product overflows, so the oracle's result must equal that
+    remainder computed with Python's integers from the (pinned) draws of the two half keys. Bounds the wrong way
+    round return minval.'''
+    r = mj.random
+    for seed, shape, lo, hi in ((0, (1,), 0, 9999), (17, (6, 5), -77, 1234), (5, (33,), 10, 11), (9, (4,), -3, 65000), (1, (3,), 8, 8), (2, (3,), 9, -9)):
+        key = r.PRNGKey(seed)
+        (got,) = eval_closed_jaxpr(mj.make_jaxpr(lambda k: r.randint(k, shape, lo, hi))(key), key)
+        (keys,) = eval_closed_jaxpr(mj.make_jaxpr(lambda k: r.split(k))(key), key)
+        (high,) = eval_closed_jaxpr(mj.make_jaxpr(lambda k: r.random_bits(k, shape))(keys[0]), keys[0])
+        (low,)  = eval_closed_jaxpr(mj.make_jaxpr(lambda k: r.random_bits(k, shape))(keys[1]), keys[1])
+        span = max(hi - lo, 1)
+        want = [(int(h) * 2**32 + int(l)) % span + lo for h, l in zip(high.ravel(), low.ravel())]
+        assert got.dtype == np.int32 and got.shape == shape and got.ravel().tolist() == want, (seed, shape, lo, hi)
+        assert (got >= lo).all() and (got < max(hi, lo + 1)).all()
+
+
 # ------------------------------------------------------------------ dot / conv
 
 def test_dot_general_exact_integers_and_einsum_layouts():

@@ -119,3 +119,30 @@ def normal(key, shape=(), dtype=np.float32):
     lo = np.nextafter(np.float32(-1.0), np.float32(0.0))
     u  = uniform(key, shape, dtype, minval=lo, maxval=1.0)
     return lax.mul(np.float32(np.sqrt(2)), lax.erf_inv(u))
+
+
+def randint(key, shape, minval, maxval, dtype=np.int32):
+    '''Integers in [minval, maxval) the way jax.random.randint draws them (int32, Python-integer bounds): two
+    32-bit draws from the halves of a split key stand for one 64-bit number, whose remainder by the span is
+    taken in 32-bit arithmetic as ((hi % span) * (2**32 % span) + lo % span) % span.
+    (The reference runs this composition in tests/test_random.py:45-60.)'''
+    if np.dtype(dtype) != np.int32:
+        raise NotImplementedError('randint: int32 only')
+    minval, maxval = int(minval), int(maxval)
+    info = np.iinfo(np.int32)
+    maxval_out_of_range = maxval > info.max
+    minval, maxval = max(info.min, min(info.max, minval)), max(info.min, min(info.max, maxval))
+    shape = tuple(shape)
+    keys  = split(key)
+    k1    = mnp.reshape(lax.slice(keys, (0, 0), (1, 2)), (2,))
+    k2    = mnp.reshape(lax.slice(keys, (1, 0), (2, 2)), (2,))
+    higher_bits, lower_bits = random_bits(k1, shape), random_bits(k2, shape)
+    span = maxval - minval if maxval > minval else 1
+    if maxval_out_of_range and maxval > minval:
+        span += 1
+    span = np.uint32(span)
+    multiplier = np.uint32(2 ** 16) % span
+    multiplier = np.uint32((int(multiplier) * int(multiplier)) & 0xFFFFFFFF) % span
+    offset = lax.add(lax.mul(lax.rem(higher_bits, span), multiplier), lax.rem(lower_bits, span))
+    offset = lax.rem(offset, span)
+    return lax.add(np.int32(minval), lax.convert_element_type(offset, np.int32))
