@@ -587,12 +587,34 @@ def pad(x, padding_value, padding_config, **_):
 
 # ------------------------------------------------------------------ indexing
 
-def gather(operand, start_indices, dimension_numbers, slice_sizes, **_):
+def _index_mode_name(mode) -> str:
+    name = '' if mode is None else str(getattr(mode, 'name', mode)).upper().rsplit('.', 1)[-1]
+    return {'FILL': 'FILL_OR_DROP', 'DROP': 'FILL_OR_DROP'}.get(name, name)      #the strings jax accepts for the enum
+
+
+def gather(operand, start_indices, dimension_numbers, slice_sizes, mode=None, fill_value=None, **_):
     '''XLA gather. Output dims listed in offset_dims enumerate the positions inside a slice
     (slice dims that are not collapsed, in order); the remaining output dims are the batch
     dims of start_indices (all but its last). Each batch position holds one start vector,
     scattered into operand coordinates through start_index_map and clamped so the slice
-    fits. reference: vkjax/ops.py:372-401, vkjax/shaders/gather.comp:62-103 (no clamping there).'''
+    fits. With mode FILL_OR_DROP (newer jax versions) a slice that does not fit is not moved inside:
+    its positions read as fill_value (default: NaN, the most negative signed integer, the largest
+    unsigned one, True). reference: vkjax/ops.py:372-401, vkjax/shaders/gather.comp:62-103 (no clamping there).'''
+    if _index_mode_name(mode) == 'FILL_OR_DROP':
+        clamped = gather(operand, start_indices, dimension_numbers, slice_sizes)
+        op, idx = _canon(operand), _canon(start_indices).astype(np.int64)
+        outside = np.zeros(idx.shape[:-1], dtype=bool)
+        for k, d in enumerate(dimension_numbers[2]):
+            outside |= (idx[..., k] < 0) | (idx[..., k] > op.shape[d] - slice_sizes[d])
+        if fill_value is None:
+            kind = op.dtype.kind
+            fill_value = np.nan if kind == 'f' else np.iinfo(op.dtype).min if kind == 'i' else np.iinfo(op.dtype).max if kind == 'u' else True
+        #the batch dims of the result are those not listed in offset_dims, in order
+        batch_dims = [d for d in range(clamped.ndim) if d not in dimension_numbers[0]]
+        shape = [1] * clamped.ndim
+        for d, n in zip(batch_dims, outside.shape):
+            shape[d] = n
+        return np.where(outside.reshape(shape), np.asarray(fill_value, op.dtype), clamped).astype(op.dtype)
     offset_dims, collapsed, start_index_map = dimension_numbers
     operand, idx = _canon(operand), _canon(start_indices).astype(np.int64)
     batch_shape  = idx.shape[:-1]
@@ -620,14 +642,22 @@ def gather(operand, start_indices, dimension_numbers, slice_sizes, **_):
     return np.transpose(vals, np.argsort(src_order)).copy() if vals.ndim else vals
 
 
-def scatter_add(operand, scatter_indices, updates, dimension_numbers, **_):
+def scatter_add(operand, scatter_indices, updates, dimension_numbers, mode=None, **_):
     '''XLA scatter with addition. update_window_dims are the dims of `updates` that run
     inside a window; the window spans the operand dims not in inserted_window_dims; the
     other update dims are the batch dims of scatter_indices. A window that does not fit
-    entirely inside the operand is dropped. Float sums accumulate in float64.
+    entirely inside the operand is dropped; with mode CLIP (newer jax versions) it is moved inside
+    instead. Float sums accumulate in float64.
     reference: vkjax/ops.py:404-433 (two fixed patterns), vkjax/shaders/scatter0.comp, scatter1.comp.'''
     uwd, iwd, sd2od = dimension_numbers
     operand, idx, updates = _canon(operand), _canon(scatter_indices).astype(np.int64), _canon(updates)
+    if _index_mode_name(mode) == 'CLIP' and operand.size:
+        sizes = [updates.shape[d] for d in uwd]
+        window = iter(sizes)
+        per_dim = [1 if d in iwd else next(window) for d in range(operand.ndim)]
+        idx = idx.copy()
+        for k, d in enumerate(sd2od):
+            idx[..., k] = np.clip(idx[..., k], 0, operand.shape[d] - per_dim[d])
     acc = operand.astype(np.float64) if operand.dtype.kind == 'f' else operand.astype(np.int64)
     window_op_dims = [d for d in range(operand.ndim) if d not in iwd]
     scatter_dims   = [d for d in range(updates.ndim) if d not in uwd]

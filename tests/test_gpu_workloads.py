@@ -371,6 +371,49 @@ def test_affine_chains_in_straight_line_code():
     assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['ew_chain_v4_s4']
 
 
+def test_gather_fill_and_scatter_clip_modes():
+    '''jax's indexing modes on the GPU against the oracle, bit for bit: FILL_OR_DROP gathers (rows of 5 and of 8
+    words, a default and a given fill value, floats and integers, windows, a build-time index outside the table) and
+    CLIP scatter-adds (atomic rows, the sorted kernels, windows). Integer-valued updates: every sum is exact.'''
+    from vkjax_amd.minijax import core
+    from vkjax_amd import ops
+    lax = mj.lax
+    G, S = core.GatherDimensionNumbers, core.ScatterDimensionNumbers
+    rng = np.random.default_rng(12)
+    rows_dn, rows_sd = G((1,), (0,), (0,)), S((1,), (0,), (0,))
+    for width in (5, 8):
+        table = rng.integers(-50, 50, size=(37, width)).astype(np.float32)
+        idx   = rng.integers(-20, 60, size=(300, 1)).astype(np.int32)
+        upd   = rng.integers(-9, 9, size=(300, width)).astype(np.float32)
+        print(f'rows of {width}', flush=True)
+        y, _, _ = check_against_oracle(lambda t, i: lax.gather(t, i, rows_dn, (1, width), mode='fill'), [table, idx], exact=True)
+        assert np.isnan(y[(idx[:, 0] < 0) | (idx[:, 0] >= 37)]).all() and not np.isnan(y[(idx[:, 0] >= 0) & (idx[:, 0] < 37)]).any()
+        check_against_oracle(lambda t, i: lax.gather(t, i, rows_dn, (1, width), mode='fill', fill_value=-1.5), [table, idx], exact=True)
+        check_against_oracle(lambda t, i: lax.gather(t, i, rows_dn, (1, width), mode='FILL_OR_DROP'), [table.astype(np.int32), idx], exact=True)
+        check_against_oracle(lambda t, i: lax.gather(t, i, rows_dn, (1, width), mode='clip'), [table, idx], exact=True)
+        for fuse in (True, False):
+            check_against_oracle(lambda t, i, u: lax.scatter_add(t, i, u, rows_sd, mode='clip'), [table, idx, upd], exact=True, fuse=fuse)
+            check_against_oracle(lambda t, i, u: lax.scatter_add(t, i, u, rows_sd, mode='drop'), [table, idx, upd], exact=True, fuse=fuse)
+    #a single index known when the program is built: inside it is a copy, outside the fill value
+    table = rng.integers(-50, 50, size=(6, 4)).astype(np.float32)
+    for row in (2, 9, -1):
+        check_against_oracle(lambda t: lax.gather(t, np.array([[row]], np.int32), rows_dn, (1, 4), mode='fill'), [table], exact=True)
+    #windows of 2 x 3 in a 7 x 5 table
+    table  = rng.integers(-50, 50, size=(7, 5)).astype(np.float32)
+    starts = rng.integers(-3, 8, size=(40, 2)).astype(np.int32)
+    win    = rng.integers(-9, 9, size=(40, 2, 3)).astype(np.float32)
+    check_against_oracle(lambda t, i: lax.gather(t, i, G((1, 2), (), (0, 1)), (2, 3), mode='fill'), [table, starts], exact=True)
+    check_against_oracle(lambda t, i, u: lax.scatter_add(t, i, u, S((1, 2), (), (0, 1)), mode='clip'), [table, starts, win], exact=True)
+    #the sorted (atomic-free) kernels
+    table = rng.integers(-50, 50, size=(500, 64)).astype(np.float32)
+    idx   = rng.integers(-100, 600, size=(ops.SCATTER_SORT_THRESHOLD // 64 + 7, 1)).astype(np.int32)
+    upd   = rng.integers(-9, 9, size=(idx.shape[0], 64)).astype(np.float32)
+    for mode in ('clip', None):
+        _, _, fn = check_against_oracle(lambda t, i, u: lax.scatter_add(t, i, u, rows_sd, mode=mode), [table, idx, upd], exact=True)
+        kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+        assert 'scatter_rows_rank' in kernels, kernels
+
+
 def test_indices_that_count_from_the_end():
     '''`x[i]` and `x.at[i].add(u)` with negative entries in i: tracing normalises the index as select(i < 0, i + n, i),
     which runs as one launch (opcode WRAP_I) whose result both the gather and the scatter-add read. Bit-exact against

@@ -495,17 +495,26 @@ def test_no_temporary_shares_storage_with_a_program_output():
                 assert b is None or max(b.accesses) == np.inf
 
 
-def test_index_modes_that_change_results_are_refused():
-    '''gather clamps and scatter-add drops (XLA); a mode that asks for anything else must not be ignored.'''
-    x, idx = np.zeros((8, 4), np.float32), np.zeros((3, 1), np.int32)
+def test_index_modes():
+    '''gather clamps and scatter-add drops by default (XLA); jax's other modes are planned with the matching kernel
+    flag (a fill word for gather, clipping for scatter-add), and a mode nobody knows must not be ignored.'''
+    x, idx, upd = np.zeros((8, 4), np.float32), np.zeros((3, 1), np.int32), np.zeros((3, 4), np.float32)
     dn = lax.GatherDimensionNumbers(offset_dims=(1,), collapsed_slice_dims=(0,), start_index_map=(0,))
-    for mode, ok in (('clip', True), ('promise_in_bounds', True), (None, True), ('fill', False)):
+    for mode, fill in (('clip', None), ('promise_in_bounds', None), (None, None), ('fill', 0x7FC00000), ('FILL_OR_DROP', 0x7FC00000)):
         closed = mj.make_jaxpr(lambda x, i: lax.gather(x, i, dn, (1, 4), mode=mode))(x, idx)
-        if ok:
-            JaxprInterpreter(closed, plan_only=True)
-        else:
-            with pytest.raises(NotImplementedError, match='mode'):
-                JaxprInterpreter(closed, plan_only=True)
+        (launch,) = JaxprInterpreter(closed, plan_only=True).launches
+        assert np.frombuffer(launch.params, np.uint32)[-2:].tolist() == [int(fill is not None), fill or 0], mode
+    closed = mj.make_jaxpr(lambda x, i: lax.gather(x.astype(np.int32), i, dn, (1, 4), mode='fill', fill_value=-7))(x, idx)
+    assert np.frombuffer(JaxprInterpreter(closed, plan_only=True).launches[-1].params, np.int32)[-2:].tolist() == [1, -7]
+    sd = lax.ScatterDimensionNumbers(update_window_dims=(1,), inserted_window_dims=(0,), scatter_dims_to_operand_dims=(0,))
+    for mode, clip in (('clip', 1), ('drop', 0), (None, 0), ('promise_in_bounds', 0)):
+        closed = mj.make_jaxpr(lambda x, i, u: lax.scatter_add(x, i, u, sd, mode=mode))(x, idx, upd)
+        launch = JaxprInterpreter(closed, plan_only=True, fuse=False).launches[-1]
+        assert launch.kernel == 'scatter_add_rows' and np.frombuffer(launch.params, np.uint32)[-1] == clip, mode
+    for f, args in ((lambda x, i: lax.gather(x, i, dn, (1, 4), mode='one_hot'), (x, idx)),
+                    (lambda x, i, u: lax.scatter_add(x, i, u, sd, mode='wrap'), (x, idx, upd))):
+        with pytest.raises(NotImplementedError, match='mode'):
+            JaxprInterpreter(mj.make_jaxpr(f)(*args), plan_only=True)
 
 
 def test_evenly_split_conv_grids():

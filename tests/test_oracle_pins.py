@@ -270,6 +270,44 @@ def test_scatter_add_forms_against_add_at():
 
 # ------------------------------------------------------------------ reductions / element-wise
 
+def test_gather_fill_and_scatter_clip_modes():
+    '''The modes newer jax versions attach to indexing: a FILL_OR_DROP gather returns fill_value where the slice does
+    not fit (instead of moving it inside), a CLIP scatter-add moves windows inside (instead of dropping them).
+    Against plain numpy indexing.'''
+    G, S = core.GatherDimensionNumbers, core.ScatterDimensionNumbers
+    table = rng.random_sample((7, 5)).astype(np.float32)
+    rows  = np.array([3, -1, 7, 0, 6, 100, -2**31], np.int64)
+    inside = (rows >= 0) & (rows < 7)
+    got = P.gather(table, rows[:, None].astype(np.int32), (G((1,), (0,), (0,))), (1, 5), mode='fill')
+    assert np.array_equal(got[inside], table[rows[inside]]) and np.isnan(got[~inside]).all()
+    got = P.gather(table.astype(np.int32) + 3, rows[:, None].astype(np.int32), (G((1,), (0,), (0,))), (1, 5), mode='FILL_OR_DROP')
+    assert (got[~inside] == np.iinfo(np.int32).min).all() and np.array_equal(got[inside], (table.astype(np.int32) + 3)[rows[inside]])
+    got = P.gather(table, rows[:, None].astype(np.int32), (G((1,), (0,), (0,))), (1, 5), mode='fill', fill_value=-2.5)
+    assert (got[~inside] == -2.5).all()
+    #windows of 2 x 3 at (r, c): they fit for r <= 5 and c <= 2
+    starts = np.array([[0, 0], [5, 2], [6, 0], [2, 3], [-1, 1]], np.int32)
+    got = P.gather(table, starts, G((1, 2), (), (0, 1)), (2, 3), mode='fill')
+    for k, (r, c) in enumerate(starts):
+        want = table[r:r + 2, c:c + 3] if 0 <= r <= 5 and 0 <= c <= 2 else np.full((2, 3), np.nan, np.float32)
+        assert np.array_equal(got[k], want, equal_nan=True), k
+    #the default mode moves the same windows inside
+    assert np.array_equal(P.gather(table, starts, G((1, 2), (), (0, 1)), (2, 3))[2], table[5:7, 0:3])
+    upd = rng.random_sample((7, 5)).astype(np.float32)
+    want = table.astype(np.float64)
+    np.add.at(want, np.clip(rows, 0, 6), upd)
+    got = P.scatter_add(table, rows[:, None].astype(np.int32), upd, S((1,), (0,), (0,)), mode='clip')
+    assert np.allclose(got, want, rtol=1e-6)
+    dropped = table.astype(np.float64)
+    np.add.at(dropped, rows[inside], upd[inside])
+    assert np.allclose(P.scatter_add(table, rows[:, None].astype(np.int32), upd, S((1,), (0,), (0,))), dropped, rtol=1e-6)
+    win = rng.random_sample((5, 2, 3)).astype(np.float32)
+    want = table.astype(np.float64)
+    for k, (r, c) in enumerate(starts):
+        r, c = min(max(r, 0), 5), min(max(c, 0), 2)
+        want[r:r + 2, c:c + 3] += win[k]
+    assert np.allclose(P.scatter_add(table, starts, win, S((1, 2), (), (0, 1)), mode='clip'), want, rtol=1e-6)
+
+
 def test_reductions_and_argmax_rules():
     x = rng.rand(5, 6, 7).astype(np.float32)
     assert np.allclose(P.reduce_sum(x, (0, 2)), x.astype(np.float64).sum(axis=(0, 2)), rtol=1e-6)

@@ -12,9 +12,10 @@
 
 #define IDX_MAX_RANK 6
 
-struct GatherRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride; };
+struct GatherRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride, fill_mode, fill_bits; };
 
-// out[i, :] = table[clamp(idx[i*idx_stride]), :]
+// out[i, :] = table[clamp(idx[i*idx_stride]), :]; with fill_mode, rows outside the table read as fill_bits instead
+// (jax's GatherScatterMode.FILL_OR_DROP)
 template <int VEC>
 __device__ __forceinline__ void gather_rows_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ table,
                                                  const int32_t* __restrict__ idx, const GatherRowsParams& P) {
@@ -23,9 +24,14 @@ __device__ __forceinline__ void gather_rows_body(uint32_t* __restrict__ out, con
     if (q >= (uint64_t)P.n_idx * vpr) return;
     const uint32_t i = (uint32_t)(q / vpr), c = (uint32_t)(q - (uint64_t)i * vpr) * VEC;
     int32_t r = idx[(uint64_t)i * P.idx_stride];
+    uint32_t* dst = out + (uint64_t)i * P.row_len + c;
+    if (P.fill_mode && (r < 0 || r >= (int32_t)P.n_rows)) {
+        if constexpr (VEC == 4) *reinterpret_cast<u32x4*>(dst) = u32x4{P.fill_bits, P.fill_bits, P.fill_bits, P.fill_bits};
+        else *dst = P.fill_bits;
+        return;
+    }
     r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
     const uint32_t* src = table + (uint64_t)r * P.row_len + c;
-    uint32_t* dst = out + (uint64_t)i * P.row_len + c;
     if constexpr (VEC == 4) *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
     else *dst = *src;
 }
@@ -48,6 +54,7 @@ struct GatherGeneralParams {
     uint32_t start_index_map[IDX_MAX_RANK];           // indices component k -> operand dim
     uint32_t batch_dims[IDX_MAX_RANK];                // sizes of indices.shape[:-1] (row-major), padded with 1
     uint32_t n_batch_dims;
+    uint32_t fill_mode, fill_bits;                    // fill_mode: slices that do not fit read as fill_bits instead of being moved inside
 };
 
 extern "C" __global__ __launch_bounds__(256) void gather_general(uint32_t* __restrict__ out, const uint32_t* __restrict__ operand,
@@ -66,13 +73,16 @@ extern "C" __global__ __launch_bounds__(256) void gather_general(uint32_t* __res
         else { batch = batch * P.batch_dims[b] + oc[d]; ++b; }
     }
     int32_t start[IDX_MAX_RANK];
+    bool outside = false;
     for (uint32_t d = 0; d < P.op_rank; ++d) start[d] = 0;
     for (uint32_t k = 0; k < P.n_index; ++k) {
         const uint32_t d = P.start_index_map[k];
         int32_t s = indices[(uint64_t)batch * P.n_index + k];
         const int32_t hi = (int32_t)P.op_dims[d] - (int32_t)P.slice_sizes[d];
+        outside = outside || s < 0 || s > hi;
         start[d] = s < 0 ? 0 : (s > hi ? hi : s);
     }
+    if (P.fill_mode && outside) { out[e] = P.fill_bits; return; }
     uint64_t off = 0;
     for (uint32_t d = 0, j = 0; d < P.op_rank; ++d) {
         uint32_t c = (uint32_t)start[d];
@@ -82,7 +92,7 @@ extern "C" __global__ __launch_bounds__(256) void gather_general(uint32_t* __res
     out[e] = operand[off];
 }
 
-struct ScatterRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride, is_float; };
+struct ScatterRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride, is_float, clip; };   // clip: rows outside the table go to its first / last row instead of being dropped
 
 // out[idx[i], :] += updates[i, :]   (out already holds the operand)
 extern "C" __global__ __launch_bounds__(256) void scatter_add_rows(uint32_t* __restrict__ out, const int32_t* __restrict__ idx,
@@ -90,7 +100,8 @@ extern "C" __global__ __launch_bounds__(256) void scatter_add_rows(uint32_t* __r
     const uint64_t q = (uint64_t)blockIdx.x * 256u + threadIdx.x;
     if (q >= (uint64_t)P.n_idx * P.row_len) return;
     const uint32_t i = (uint32_t)(q / P.row_len), c = (uint32_t)(q - (uint64_t)i * P.row_len);
-    const int32_t r = idx[(uint64_t)i * P.idx_stride];
+    int32_t r = idx[(uint64_t)i * P.idx_stride];
+    if (P.clip) r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
     if (r < 0 || r >= (int32_t)P.n_rows) return;
     const uint32_t u = updates[q];
     uint32_t* dst = out + (uint64_t)r * P.row_len + c;
@@ -109,7 +120,7 @@ extern "C" __global__ __launch_bounds__(256) void scatter_add_rows(uint32_t* __r
 // depends on the order of arrival).
 // Scratch: count (n_rows words, all zero before and after), start (n_rows + 1), rank and order
 // (n_idx each).
-struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride, operand_is_scalar; };
+struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride, operand_is_scalar, clip; };   // clip: as in ScatterRowsParams
 
 #define SCATTER_DROPPED 0xFFFFFFFFu
 
@@ -119,7 +130,8 @@ extern "C" __global__ __launch_bounds__(256) void scatter_rows_rank(uint32_t* __
                                                                     const int32_t* __restrict__ idx, ScatterSortParams P) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= P.n_idx) return;
-    const int32_t r = idx[(uint64_t)i * P.idx_stride];
+    int32_t r = idx[(uint64_t)i * P.idx_stride];
+    if (P.clip) r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
     uint32_t k = SCATTER_DROPPED;
     if (r >= 0 && r < (int32_t)P.n_rows) k = atomicAdd(count + r, 1u);
     rank[i] = k;
@@ -188,7 +200,9 @@ extern "C" __global__ __launch_bounds__(256) void scatter_rows_order(uint32_t* _
     if (i >= P.n_idx) return;
     const uint32_t k = rank[i];
     if (k == SCATTER_DROPPED) return;
-    order[start[idx[(uint64_t)i * P.idx_stride]] + k] = i;
+    int32_t r = idx[(uint64_t)i * P.idx_stride];
+    if (P.clip) r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
+    order[start[r] + k] = i;
 }
 
 // ascending bitonic sort of one value per lane across the wave
@@ -298,6 +312,7 @@ struct ScatterGeneralParams {
     uint32_t window_sizes[IDX_MAX_RANK];              // per operand dim (1 where inserted)
     uint32_t sd2od[IDX_MAX_RANK];                     // indices component k -> operand dim
     uint32_t batch_dims[IDX_MAX_RANK];
+    uint32_t clip;                                    // windows that do not fit are moved inside instead of being dropped
 };
 
 extern "C" __global__ __launch_bounds__(256) void scatter_add_general(uint32_t* __restrict__ out, const int32_t* __restrict__ indices,
@@ -319,7 +334,11 @@ extern "C" __global__ __launch_bounds__(256) void scatter_add_general(uint32_t* 
     for (uint32_t k = 0; k < P.n_index; ++k) start[P.sd2od[k]] = indices[(uint64_t)batch * P.n_index + k];
     uint64_t off = 0;
     for (uint32_t d = 0, j = 0; d < P.op_rank; ++d) {
-        // the whole window must fit, otherwise the update is dropped
+        // the whole window must fit, otherwise the update is dropped (or, with clip, moved inside)
+        if (P.clip) {
+            const int32_t hi = (int32_t)P.op_dims[d] - (int32_t)P.window_sizes[d];
+            start[d] = start[d] < 0 ? 0 : (start[d] > hi ? hi : start[d]);
+        }
         if (start[d] < 0 || (uint32_t)start[d] + P.window_sizes[d] > P.op_dims[d]) return;
         uint32_t c = (uint32_t)start[d];
         if (!P.op_inserted[d]) c += wc[j++];

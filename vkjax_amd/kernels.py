@@ -1086,14 +1086,17 @@ def pad(out: Buffer, inp: Buffer, value: Buffer, padding_config) -> Launch:
 IDX_MAX_RANK = 6
 
 
-def gather_rows(out: Buffer, table: Buffer, idx: Buffer, n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1) -> Launch:
+def gather_rows(out: Buffer, table: Buffer, idx: Buffer, n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1,
+                fill: tp.Optional[int] = None) -> Launch:
+    '''`fill`: None clamps rows outside the table; a 32-bit pattern makes them read as that value instead.'''
     vec = 4 if row_len % 4 == 0 else 1
     total = n_idx * (row_len // vec)
     return Launch(f'gather_rows_v{vec}', (_cdiv(total, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (table, 0), (idx, 0)],
-                  _u32(n_idx, row_len, n_rows, idx_stride), bytes_moved=4 * (2 * n_idx * row_len + n_idx))
+                  _u32(n_idx, row_len, n_rows, idx_stride, int(fill is not None), fill or 0), bytes_moved=4 * (2 * n_idx * row_len + n_idx))
 
 
-def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, collapsed, start_index_map, slice_sizes) -> Launch:
+def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, collapsed, start_index_map, slice_sizes,
+                   fill: tp.Optional[int] = None) -> Launch:
     out_rank, op_rank = len(out.shape), len(operand.shape)
     if max(out_rank, op_rank, len(indices.shape)) > IDX_MAX_RANK:
         raise NotImplementedError('gather with rank > 6')
@@ -1102,27 +1105,30 @@ def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, c
                   *_pad(out.shape, IDX_MAX_RANK, 1), *_pad([int(d in offset_dims) for d in range(out_rank)], IDX_MAX_RANK),
                   *_pad(operand.shape, IDX_MAX_RANK, 1), *_pad(row_major_strides(operand.shape), IDX_MAX_RANK),
                   *_pad(slice_sizes, IDX_MAX_RANK, 1), *_pad([int(d in collapsed) for d in range(op_rank)], IDX_MAX_RANK),
-                  *_pad(start_index_map, IDX_MAX_RANK), *_pad(batch_dims, IDX_MAX_RANK, 1), len(batch_dims))
+                  *_pad(start_index_map, IDX_MAX_RANK), *_pad(batch_dims, IDX_MAX_RANK, 1), len(batch_dims),
+                  int(fill is not None), fill or 0)
     return Launch('gather_general', (_cdiv(out.size, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (operand, 0), (indices, 0)],
                   params, bytes_moved=4 * (2 * out.size + indices.size))
 
 
-def scatter_add_rows(out: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1) -> Launch:
+def scatter_add_rows(out: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1,
+                     clip: bool = False) -> Launch:
+    '''`clip`: rows outside the table go to its first / last row instead of being dropped.'''
     total = n_idx * row_len
     return Launch('scatter_add_rows', (_cdiv(total, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (idx, 0), (updates, 0)],
-                  _u32(n_idx, row_len, n_rows, idx_stride, int(out.dtype == np.float32)),
+                  _u32(n_idx, row_len, n_rows, idx_stride, int(out.dtype == np.float32), int(clip)),
                   bytes_moved=4 * (total + n_idx + out.size))
 
 
 def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, count: Buffer, start: Buffer, rank: Buffer,
                             order: Buffer, n_idx: int, row_len: int, n_rows: int, operand_is_scalar: bool = False,
-                            idx_stride: int = 1) -> tp.List[Launch]:
+                            idx_stride: int = 1, clip: bool = False) -> tp.List[Launch]:
     '''out = operand; out[idx[i], :] += updates[i, :] without atomics on the data: a counting sort of the indices
     (`count`: n_rows words that are zero before and after, `start`: n_rows + 1 words, `rank` and `order`: n_idx words
     each), then one wave per row sums its bucket. `operand` is the table, or one word when the table is a constant
     filled with a single value.'''
     assert count.size == n_rows and start.size == n_rows + 1 and rank.size == n_idx and order.size == n_idx
-    params = _u32(n_idx, row_len, n_rows, idx_stride, int(operand_is_scalar))
+    params = _u32(n_idx, row_len, n_rows, idx_stride, int(operand_is_scalar), int(clip))
     vec    = 4 if row_len % 4 == 0 else 1
     kind   = 'f' if out.dtype == np.float32 else 'i'
     #bucket starts: at most 256 workgroups, each scanning a segment of whole 1024-word tiles
@@ -1141,7 +1147,7 @@ def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: 
 
 
 def scatter_add_general(out: Buffer, indices: Buffer, updates: Buffer, update_window_dims, inserted_window_dims,
-                        scatter_dims_to_operand_dims) -> Launch:
+                        scatter_dims_to_operand_dims, clip: bool = False) -> Launch:
     upd_rank, op_rank = len(updates.shape), len(out.shape)
     if max(upd_rank, op_rank, len(indices.shape)) > IDX_MAX_RANK:
         raise NotImplementedError('scatter-add with rank > 6')
@@ -1154,7 +1160,7 @@ def scatter_add_general(out: Buffer, indices: Buffer, updates: Buffer, update_wi
                   *_pad(out.shape, IDX_MAX_RANK, 1), *_pad(row_major_strides(out.shape), IDX_MAX_RANK),
                   *_pad([int(d in inserted_window_dims) for d in range(op_rank)], IDX_MAX_RANK),
                   *_pad(window_sizes, IDX_MAX_RANK, 1), *_pad(scatter_dims_to_operand_dims, IDX_MAX_RANK),
-                  *_pad(batch_dims, IDX_MAX_RANK, 1))
+                  *_pad(batch_dims, IDX_MAX_RANK, 1), int(clip))
     return Launch('scatter_add_general', (_cdiv(max(updates.size, 1), BLOCK), 1, 1), (BLOCK, 1, 1),
                   [(out, 0), (indices, 0), (updates, 0)], params, bytes_moved=4 * (updates.size + indices.size + out.size))
 

@@ -496,7 +496,7 @@ def gather(operand, start_indices, dimension_numbers: GatherDimensionNumbers, sl
 
 
 def scatter_add(operand, scatter_indices, updates, dimension_numbers: ScatterDimensionNumbers,
-                indices_are_sorted=False, unique_indices=False):
+                indices_are_sorted=False, unique_indices=False, mode=None):
     dn = ScatterDimensionNumbers(*(tuple(int(i) for i in t) for t in dimension_numbers))
     dtype = result_dtype(operand, updates)
     operand, updates = _as_dtype(operand, dtype), _as_dtype(updates, dtype)
@@ -504,7 +504,7 @@ def scatter_add(operand, scatter_indices, updates, dimension_numbers: ScatterDim
         raise TypeError('scatter indices must be integers')
     return emit('scatter-add', [operand, scatter_indices, updates], [_aval(_shape(operand), dtype)],
                 dict(dimension_numbers=dn, indices_are_sorted=indices_are_sorted, unique_indices=unique_indices,
-                     update_jaxpr=None, update_consts=()))
+                     update_jaxpr=None, update_consts=(), **({} if mode is None else dict(mode=mode))))
 
 
 # ---------------------------------------------------------------- rng

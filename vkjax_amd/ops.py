@@ -866,14 +866,16 @@ def _index_mode(params) -> str:
     mode = params.get('mode')
     if mode is None:
         return ''
-    return str(getattr(mode, 'name', mode)).upper().rsplit('.', 1)[-1]
+    name = str(getattr(mode, 'name', mode)).upper().rsplit('.', 1)[-1]
+    return {'FILL': 'FILL_OR_DROP', 'DROP': 'FILL_OR_DROP'}.get(name, name)      #the strings jax accepts for the enum
 
 
 def gather(bufferpool, equation):
     params = equation.params
     #start indices are clamped so that the slice stays inside the operand: that is XLA's gather, CLIP, and what
-    #XLA makes of PROMISE_IN_BOUNDS; FILL_OR_DROP would have to return fill_value for such slices instead
-    if _index_mode(params) not in ('', 'CLIP', 'PROMISE_IN_BOUNDS'):
+    #XLA makes of PROMISE_IN_BOUNDS; under FILL_OR_DROP a slice that does not fit reads as fill_value instead
+    mode = _index_mode(params)
+    if mode not in ('', 'CLIP', 'PROMISE_IN_BOUNDS', 'FILL_OR_DROP'):
         raise NotImplementedError(f'gather with mode={params["mode"]}: {equation}')
     dn     = params['dimension_numbers']
     offset_dims, collapsed, start_index_map = (tuple(dn.offset_dims), tuple(dn.collapsed_slice_dims), tuple(dn.start_index_map))
@@ -884,6 +886,7 @@ def gather(bufferpool, equation):
         return []
     if _kind(indices.dtype) not in (_I, _U):
         raise NotImplementedError(equation)
+    fill = _gather_fill_word(operand.dtype, params.get('fill_value')) if mode == 'FILL_OR_DROP' else None
     op_rank, out_rank = len(operand.shape), len(outbuf.shape)
     n_batch = len(indices.shape) - 1
     #whole trailing slices addressed by one index on the leading axis: a row gather
@@ -894,23 +897,36 @@ def gather(bufferpool, equation):
         row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
         n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
         known   = getattr(indices, 'constant_value', None)
-        if n_idx == 1 and known is not None and operand.shape[0] > 0:
+        if n_idx == 1 and known is not None and operand.shape[0] > 0 and (fill is None or 0 <= int(np.asarray(known).reshape(-1)[0]) < operand.shape[0]):
             #one row whose number is known when the program is built (`keys[1]` of a split key, a static `x[3]`, which
             #old jax versions trace as a gather with a constant index): a copy of that row, which the consumer's
             #fusion can read in place. Clamped like any gather.
             row = builtins_min(builtins_max(int(np.asarray(known).reshape(-1)[0]), 0), operand.shape[0] - 1)
             return [_copy_op(equation, outbuf, EwOperand(operand, row * row_len, K.row_major_strides(outbuf.shape)))]
-        return [Op(equation, launch=K.gather_rows(outbuf, operand, indices, n_idx, row_len, operand.shape[0]))]
-    return [Op(equation, launch=K.gather_general(outbuf, operand, indices, offset_dims, collapsed, start_index_map, slice_sizes))]
+        return [Op(equation, launch=K.gather_rows(outbuf, operand, indices, n_idx, row_len, operand.shape[0], fill=fill))]
+    return [Op(equation, launch=K.gather_general(outbuf, operand, indices, offset_dims, collapsed, start_index_map, slice_sizes, fill=fill))]
+
+
+def _gather_fill_word(dtype, fill_value) -> int:
+    '''The 32-bit pattern a FILL_OR_DROP gather returns for slices outside the operand: the equation's fill_value,
+    or jax's default (NaN, the most negative signed integer, the largest unsigned one, True).'''
+    dtype = np.dtype(dtype)
+    if fill_value is None:
+        fill_value = (np.nan if dtype.kind == 'f' else np.iinfo(dtype).min if dtype.kind == 'i'
+                      else np.iinfo(dtype).max if dtype.kind == 'u' else True)
+    if dtype.kind == 'b':
+        return int(bool(fill_value))
+    return int(np.asarray(fill_value, dtype).reshape(1).view(np.uint32)[0])
 
 
 def scatter_add(bufferpool, equation):
     '''General XLA scatter-add (the reference implements two fixed patterns, vkjax/ops.py:404-433).
     The operand is copied to the output first, then updates are added with HBM atomics.'''
     #updates whose window does not fit into the operand are dropped: XLA's scatter, FILL_OR_DROP, and what holds
-    #trivially under PROMISE_IN_BOUNDS; CLIP would have to move such windows inside instead
-    if _index_mode(equation.params) not in ('', 'FILL_OR_DROP', 'PROMISE_IN_BOUNDS'):
+    #trivially under PROMISE_IN_BOUNDS; CLIP moves such windows inside instead
+    if _index_mode(equation.params) not in ('', 'FILL_OR_DROP', 'PROMISE_IN_BOUNDS', 'CLIP'):
         raise NotImplementedError(f'scatter-add with mode={equation.params["mode"]}: {equation}')
+    clip = _index_mode(equation.params) == 'CLIP'
     dn = equation.params['dimension_numbers']
     uwd, iwd, sd2od = tuple(dn.update_window_dims), tuple(dn.inserted_window_dims), tuple(dn.scatter_dims_to_operand_dims)
     operand, indices, updates = [bufferpool.get_buffer(v) for v in equation.invars]
@@ -951,11 +967,11 @@ def scatter_add(bufferpool, equation):
                 source = operand
             bufferpool.op_counter = counter_before + 1
             launches = K.scatter_add_rows_sorted(outbuf, source, indices, updates, count, start, rank, order, n_idx, row_len, n_rows,
-                                                 operand_is_scalar=uniform is not None)
+                                                 operand_is_scalar=uniform is not None, clip=clip)
             return [Op(equation, launch=l) for l in launches]
-        ops = [copy, Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, n_rows))]
+        ops = [copy, Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, n_rows, clip=clip))]
         return ops
-    return [copy, Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od))]
+    return [copy, Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od, clip=clip))]
 
 
 #scatter-add of rows: from this many update elements on, the sorted (atomic-free) kernels are used
