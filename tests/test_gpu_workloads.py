@@ -371,6 +371,24 @@ def test_affine_chains_in_straight_line_code():
     assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['ew_chain_v4_s4']
 
 
+def test_transposes_of_several_inputs_share_a_launch():
+    '''Copies that swap the two fastest dimensions of program inputs (a network's kernels, transposed for its backward
+    pass) are hoisted to the front and run as one launch per kernel variant: 64 x 64 and 128 x 128 tiles, leading
+    dimensions (3 x 3 kernels), extents that are no multiple of the tile, bit for bit.'''
+    lax = mj.lax
+    rng = np.random.default_rng(21)
+    shapes = [(3, 3, 64, 128), (1, 1, 256, 512), (3, 3, 128, 256), (1, 1, 72, 200), (200, 136), (1, 1, 512, 128), (2, 3, 20, 36), (640, 384)]
+    arrays = [rng.standard_normal(sh).astype(np.float32) for sh in shapes]
+    def f(*xs):
+        swapped = [lax.transpose(x, tuple(range(x.ndim - 2)) + (x.ndim - 1, x.ndim - 2)) for x in xs]
+        return [lax.mul(t, np.float32(2.0)) for t in swapped[:2]] + swapped[2:]
+    _, _, fn = check_against_oracle(f, arrays, exact=True)
+    kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+    assert kernels.count('transpose_tiled_batch_v4') == 1 and kernels.count('transpose_tiled_batch_v4_t128') == 1, kernels
+    assert not any(k in ('transpose_tiled_v4', 'transpose_tiled_v4_t128') for k in kernels), kernels
+    check_against_oracle(f, arrays, exact=True, fuse=False)
+
+
 def test_gather_fill_and_scatter_clip_modes():
     '''jax's indexing modes on the GPU against the oracle, bit for bit: FILL_OR_DROP gathers (rows of 5 and of 8
     words, a default and a given fill value, floats and integers, windows, a build-time index outside the table) and

@@ -502,13 +502,14 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled(uint32_t* __re
 // The same with 16-byte global accesses on both sides: needs I, J, sj, sb and the source offset to be
 // multiples of 4. A thread reads four consecutive i of one j and, after the exchange through LDS,
 // writes four consecutive j of one i.
-extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
-                                                                     TransposeParams P) {
+// (bx, by, bz): the workgroup's place in the copy's own grid of (gx, gy, B) workgroups
+__device__ __forceinline__ void transpose_v4_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const TransposeParams& P,
+                                                  const uint32_t bx, const uint32_t by, const uint32_t bz, const uint32_t gy) {
     __shared__ uint32_t tile[64][65];
     const uint32_t t16 = threadIdx.x & 15u, tr = threadIdx.x >> 4;        // 16 vectors per tile row, 16 rows per pass
     // Tiles are taken along diagonals: with a row pitch that is a large power of two, the tiles of one row or one
     // column of tiles all start in the same memory channel, and workgroups that run together would queue there.
-    const uint32_t j0 = blockIdx.x * 64u, i0 = ((blockIdx.y + blockIdx.x) % gridDim.y) * 64u, b = blockIdx.z;
+    const uint32_t j0 = bx * 64u, i0 = ((by + bx) % gy) * 64u, b = bz;
     const uint32_t* src = in + (int64_t)b * P.sb;
     uint32_t* dst = out + (uint64_t)b * P.I * P.J;
 #pragma unroll
@@ -532,14 +533,18 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4(uint32_t* _
         }
     }
 }
+extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                                     TransposeParams P) {
+    transpose_v4_body(out, in, P, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y);
+}
 
 // 128 x 128 tiles for large arrays: runs of 512 contiguous bytes on both sides, sixteen 16-byte loads
 // in flight per thread. Same conditions as transpose_tiled_v4.
-extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4_t128(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
-                                                                          TransposeParams P) {
+__device__ __forceinline__ void transpose_v4_t128_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const TransposeParams& P,
+                                                       const uint32_t bx, const uint32_t by, const uint32_t bz, const uint32_t gy) {
     __shared__ uint32_t tile[128][129];
     const uint32_t t32 = threadIdx.x & 31u, tr = threadIdx.x >> 5;        // 32 vectors per tile row, 8 rows per pass
-    const uint32_t j0 = blockIdx.x * 128u, i0 = ((blockIdx.y + blockIdx.x) % gridDim.y) * 128u, b = blockIdx.z;
+    const uint32_t j0 = bx * 128u, i0 = ((by + bx) % gy) * 128u, b = bz;
     const uint32_t* src = in + (int64_t)b * P.sb;
     uint32_t* dst = out + (uint64_t)b * P.I * P.J;
     u32x4 v[16];
@@ -565,4 +570,42 @@ extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4_t128(uint32
             *reinterpret_cast<u32x4*>(dst + (uint64_t)i * P.J + j) = w;
         }
     }
+}
+extern "C" __global__ __launch_bounds__(256) void transpose_tiled_v4_t128(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                                          TransposeParams P) {
+    transpose_v4_t128_body(out, in, P, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y);
+}
+
+// Several independent copies of this kind in ONE launch (the kernels of a network's convolutions, transposed for
+// the backward pass: dozens of launches of a few microseconds each). As for the batched chains above, the host
+// writes one entry per copy into a table in device memory and workgroup b belongs to the last entry whose
+// first_block is <= b; its place in that copy's own (grid_x, grid_y, B) grid follows from b - first_block.
+struct TransposeBatchEntry {
+    uint32_t        first_block, grid_x;
+    uint32_t*       out;
+    const uint32_t* in;
+    TransposeParams P;
+    uint32_t        grid_y;
+};
+static_assert(sizeof(TransposeBatchEntry) == 48, "the host lays the table out with 48-byte entries");
+
+template <bool BIG>
+__device__ __forceinline__ void transpose_batch_body(const TransposeBatchEntry* __restrict__ table, uint32_t entries) {
+    uint32_t lo = 0, hi = entries;
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (table[mid].first_block <= blockIdx.x) lo = mid; else hi = mid;
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    const TransposeBatchEntry& e = table[lo];
+    const uint32_t local = blockIdx.x - e.first_block, bx = local % e.grid_x, rest = local / e.grid_x;
+    const uint32_t by = rest % e.grid_y, bz = rest / e.grid_y;
+    if constexpr (BIG) transpose_v4_t128_body(e.out, e.in, e.P, bx, by, bz, e.grid_y);
+    else transpose_v4_body(e.out, e.in, e.P, bx, by, bz, e.grid_y);
+}
+extern "C" __global__ __launch_bounds__(256) void transpose_tiled_batch_v4(const TransposeBatchEntry* __restrict__ table, uint32_t entries) {
+    transpose_batch_body<false>(table, entries);
+}
+extern "C" __global__ __launch_bounds__(256) void transpose_tiled_batch_v4_t128(const TransposeBatchEntry* __restrict__ table, uint32_t entries) {
+    transpose_batch_body<true>(table, entries);
 }

@@ -865,6 +865,10 @@ def _is_small(op) -> bool:
     '''An element-wise chain or a plain float column sum of a few workgroups, of a kind that has a batch kernel.'''
     if op.chain is None and not (op.conv is None and op.launch.kernel in K.REDUCE_BATCH_KERNELS):
         return False
+    if op.launch.kernel in K.TRANSPOSE_BATCH_KERNELS:
+        #a tiled copy that swaps two dimensions (a network's kernels, transposed for its backward pass): batched up to a
+        #larger size, a launch of a few microseconds carries little more than its own latency
+        return op.launch.grid[0] * op.launch.grid[1] * op.launch.grid[2] <= K.TRANSPOSE_BATCH_MAX_BLOCKS
     return op.launch.kernel in K.BATCH_KERNELS and op.launch.grid[0] <= K.BATCH_MAX_BLOCKS
 
 

@@ -262,11 +262,19 @@ def _as_affine_chain(chain: EwChain, n: int, dims, strides) -> tp.Optional[Launc
 
 EW_BATCH_KERNELS     = ('ew_chain_v1_s2', 'ew_chain_v1_s4', 'ew_chain_v4_s2', 'ew_chain_v4_s4')
 REDUCE_BATCH_KERNELS = ('reduce_cols_fsum_v1', 'reduce_cols_fsum_v4')
+TRANSPOSE_BATCH_KERNELS = ('transpose_tiled_v4', 'transpose_tiled_v4_t128')
 BATCH_KERNELS        = {**{k: k.replace('ew_chain_', 'ew_chain_batch_') for k in EW_BATCH_KERNELS},
-                        **{k: k.replace('fsum_', 'fsum_batch_') for k in REDUCE_BATCH_KERNELS}}
-EW_BATCH_ENTRY_BYTES     = 432
-REDUCE_BATCH_ENTRY_BYTES = 56
+                        **{k: k.replace('fsum_', 'fsum_batch_') for k in REDUCE_BATCH_KERNELS},
+                        **{k: k.replace('tiled_', 'tiled_batch_') for k in TRANSPOSE_BATCH_KERNELS}}
+EW_BATCH_ENTRY_BYTES        = 432
+REDUCE_BATCH_ENTRY_BYTES    = 56
+TRANSPOSE_BATCH_ENTRY_BYTES = 48
 BATCH_MAX_BLOCKS         = 16          #launches of more workgroups than this keep a launch of their own
+TRANSPOSE_BATCH_MAX_BLOCKS = 1024      #... tiled transposes (the kernels of a network, for its backward pass) up to this many
+
+
+def _blocks(launch: Launch) -> int:
+    return launch.grid[0] * launch.grid[1] * launch.grid[2]
 
 
 def batch_launch(members: tp.Sequence[Launch]) -> Launch:
@@ -274,22 +282,27 @@ def batch_launch(members: tp.Sequence[Launch]) -> Launch:
     that do not depend on one another.'''
     kernel = members[0].kernel
     assert kernel in BATCH_KERNELS and all(m.kernel == kernel and not m.members for m in members), [m.kernel for m in members]
-    return Launch(BATCH_KERNELS[kernel], (sum(m.grid[0] for m in members), 1, 1), (BLOCK, 1, 1), [],
+    return Launch(BATCH_KERNELS[kernel], (sum(_blocks(m) for m in members), 1, 1), (BLOCK, 1, 1), [],
                   _u32(len(members)), bytes_moved=sum(m.bytes_moved for m in members), members=tuple(members))
 
 
 def batch_table(launch: Launch, device_address: tp.Callable[[Buffer], int]) -> np.ndarray:
-    '''The table of a batch launch as uint32 words, one entry per member: {first workgroup, 0, the addresses of the
-    member's arrays (0 = none), the member's parameter block}, padded to a multiple of 8 bytes.'''
-    is_chain = launch.members[0].kernel in EW_BATCH_KERNELS
-    entry_bytes, pointers = (EW_BATCH_ENTRY_BYTES, 1 + EW_MAX_STEPS) if is_chain else (REDUCE_BATCH_ENTRY_BYTES, 2)
+    '''The table of a batch launch as uint32 words, one entry per member: {first workgroup, 0 (tiled transposes: the
+    x extent of the member's grid), the addresses of the member's arrays (0 = none), the member's parameter block
+    (tiled transposes: then the y extent of its grid)}, padded to a multiple of 8 bytes.'''
+    kind = launch.members[0].kernel
+    is_chain, is_transpose = kind in EW_BATCH_KERNELS, kind in TRANSPOSE_BATCH_KERNELS
+    entry_bytes, pointers = ((EW_BATCH_ENTRY_BYTES, 1 + EW_MAX_STEPS) if is_chain else
+                             (TRANSPOSE_BATCH_ENTRY_BYTES, 2) if is_transpose else (REDUCE_BATCH_ENTRY_BYTES, 2))
     rows, first = [], 0
     for m in launch.members:
         assert len(m.buffers) == pointers, (m.kernel, len(m.buffers))
         addresses = [device_address(b) + off if b is not None else 0 for b, off in m.buffers]
-        row = _u32(first, 0) + np.asarray(addresses, dtype=np.uint64).tobytes() + m.params
+        #(a transpose has a three-dimensional grid of its own: its x extent follows first_block, its y extent the parameters)
+        row = (_u32(first, m.grid[0] if is_transpose else 0) + np.asarray(addresses, dtype=np.uint64).tobytes() + m.params
+               + (_u32(m.grid[1]) if is_transpose else b''))
         rows.append(row + bytes(entry_bytes - len(row)))
-        first += m.grid[0]
+        first += _blocks(m)
     table = b''.join(rows)
     assert len(table) == entry_bytes * len(launch.members)
     return np.frombuffer(table, dtype=np.uint32).copy()
