@@ -269,7 +269,8 @@ BATCH_KERNELS        = {**{k: k.replace('ew_chain_', 'ew_chain_batch_') for k in
 EW_BATCH_ENTRY_BYTES        = 432
 REDUCE_BATCH_ENTRY_BYTES    = 56
 TRANSPOSE_BATCH_ENTRY_BYTES = 48
-BATCH_MAX_BLOCKS         = 16          #launches of more workgroups than this keep a launch of their own
+BATCH_MAX_BLOCKS         = 4096        #launches of more workgroups than this keep a launch of their own
+REDUCE_NARROW_MAX_BLOCKS = 16          #column sums of at most this many workgroups trade block width for more blocks
 TRANSPOSE_BATCH_MAX_BLOCKS = 1024      #... tiled transposes (the kernels of a network, for its backward pass) up to this many
 
 
@@ -934,7 +935,7 @@ def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op:
     #few blocks with many rows each (the second stage of a split sum): narrower blocks, more of them, more thread rows
     #walking the rows side by side
     #(up to the number of blocks below which small sums are batched with their neighbours into one launch)
-    while TI > 8 and 2 * _cdiv(inner, TI * vec) * nsplit * outer <= BATCH_MAX_BLOCKS and _cdiv(R, nsplit) >= 128:
+    while TI > 8 and 2 * _cdiv(inner, TI * vec) * nsplit * outer <= REDUCE_NARROW_MAX_BLOCKS and _cdiv(R, nsplit) >= 128:
         TI //= 2
     params = _u32(outer, R, inner, RED[op], ty, r_chunk, nsplit, TI)
     blocks = _cdiv(inner, TI * vec) * nsplit * outer
