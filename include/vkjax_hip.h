@@ -135,8 +135,10 @@ int vkj_seq_eval_next(vkj_handle seq, void* const* host_ptrs, int nslots, uint32
  * on holds one copy until the process ends), are staged in the pinned buffers the sequence already
  * owns, and are moved on by a copy kernel. Slots are packed at multiples of 256 bytes; arguments
  * that do not fit are rejected with VKJ_EINVAL, sequences with timestamps, or with a graph that is
- * not built yet, with VKJ_ESTATE. All calls on one GPU share the array: calls that overlap in time
- * on one GPU race. Same arguments and results as vkj_seq_eval_next otherwise. */
+ * not built yet, with VKJ_ESTATE. All calls on one GPU share the array, which a call claims until it
+ * returns: a call that overlaps another one on the same GPU (another thread or context) is rejected
+ * with VKJ_ESTATE ("static landing array busy") and may be repeated. Same arguments and results as
+ * vkj_seq_eval_next otherwise. */
 #define VKJ_STATIC_LANDING_BYTES (64u << 20)
 int vkj_seq_eval_next_static(vkj_handle seq, void* const* host_ptrs, int nslots, uint32_t flags,
                              void* const* next_host_ptrs);

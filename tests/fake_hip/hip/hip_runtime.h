@@ -44,6 +44,8 @@ struct FakeHipState {
     std::set<void*> live;          // every allocation, stream, event and module that has not been released
     long calls_until_failure = -1; // >= 0: that many further fallible calls succeed, the next one fails
     long launches = 0;
+    long creations = 0;            // allocations (device and pinned), streams, events, modules, graphs ever made
+    void (*on_synchronize)() = nullptr;   // called from inside hipStreamSynchronize (the test re-enters the library there)
 };
 inline FakeHipState& fake_hip() { static FakeHipState s; return s; }
 inline bool fake_hip_should_fail() {
@@ -56,6 +58,7 @@ inline bool fake_hip_should_fail() {
 template <class T> inline hipError_t fake_hip_new(T** out) {
     if (fake_hip_should_fail()) return hipErrorOutOfMemory;
     *out = new T();
+    fake_hip().creations++;
     fake_hip().live.insert(*out);
     return hipSuccess;
 }
@@ -77,7 +80,10 @@ inline hipError_t hipGetDeviceProperties(hipDeviceProp_t* p, int) {
 }
 inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { return fake_hip_new(s); }
 inline hipError_t hipStreamDestroy(hipStream_t s) { return fake_hip_delete(s); }
-inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+inline hipError_t hipStreamSynchronize(hipStream_t) {
+    if (auto hook = fake_hip().on_synchronize) { fake_hip().on_synchronize = nullptr; hook(); }
+    return hipSuccess;
+}
 inline hipError_t hipStreamWaitEvent(hipStream_t, hipEvent_t, unsigned) { return hipSuccess; }
 inline hipError_t hipEventCreate(hipEvent_t* e) { return fake_hip_new(e); }
 inline hipError_t hipEventCreateWithFlags(hipEvent_t* e, unsigned) { return fake_hip_new(e); }
@@ -89,6 +95,7 @@ inline hipError_t fake_hip_alloc(void** p, size_t n) {
     if (fake_hip_should_fail()) return hipErrorOutOfMemory;
     *p = malloc(n ? n : 1);
     memset(*p, 0xCD, n ? n : 1);           // never hand out zeroed memory: stale-data bugs must show
+    fake_hip().creations++;
     fake_hip().live.insert(*p);
     return hipSuccess;
 }

@@ -69,6 +69,8 @@ def gather_fn0(x, i):
     return lax.gather(x, i, mj.core.GatherDimensionNumbers(offset_dims=(), collapsed_slice_dims=(0, 1), start_index_map=(0, 1)),
                       slice_sizes=(1, 1))
 def take_along_axis0(x, i): return jnp.take_along_axis(x, i, axis=-1)
+#gradient of take_along_axis: a scatter-add of single elements into zeros (the reference's point form)
+def take_along_axis0_g(x, i): return mj.grad(lambda *args: take_along_axis0(*args).ravel().mean())(x, i)
 def gather_fn1(x, i):
     return lax.gather(x, i, mj.core.GatherDimensionNumbers(offset_dims=(0,), collapsed_slice_dims=(1,), start_index_map=(1,)),
                       slice_sizes=(len(x), 1))
@@ -169,6 +171,7 @@ param_matrix = [
     (scatter_fn0, 'scatter_fn0',        [random([32, 10]), np.c_[randint(0, 32, size=[32]), randint(0, 10, size=[32])].reshape(32, 1, 2),
                                          random([32]).reshape(32, 1)]),
     (take_along_axis0, 'take_along0',   [random([32, 10]), randint(0, 10, size=32)[:, np.newaxis]]),
+    (take_along_axis0_g, 'take0_grad',  [random([32, 10]), randint(0, 10, size=32)[:, np.newaxis]]),
     (gather_fn1, 'gather_fn1',          [random([32, 10]), randint(0, 10, size=[1])]),
     (scatter_add_fn1, 'scatter_add1',   [random([32, 10]), randint(0, 10, size=[1]), random(32)]),
     (add_any0, 'add_any0',              [random([32, 32]), random([32, 32])]),
@@ -311,6 +314,36 @@ def test_tiled_transposes():
             assert len(kernels) == 1, kernels
         if k >= 14:
             assert kernels == ['transpose_tiled_v4_t128'], kernels
+
+
+def test_point_and_column_scatter_add_forms():
+    '''The two scatter-add forms of the reference (vkjax/ops.py:404-433): single elements `x[i0, i1] += u`
+    (shaders/scatter0.comp:10-31; what the gradient of take_along_axis emits, tests/test_basic_ops.py:96,266) and a
+    column `x[:, i0] += u` (shaders/scatter1.comp:10-23). Integer-valued operands make the sums exact whatever the
+    order of the additions, so fused and unfused programs are compared bit for bit with the oracle, with repeated
+    targets; random operands within the element-wise tolerance.'''
+    rng = np.random.RandomState(5)
+    ints = lambda *shape: rng.randint(-4, 5, size=shape).astype(np.float32)
+    for rows, cols, n in ((32, 10, 32), (7, 3, 200), (300, 129, 64), (1, 1, 5)):
+        points = np.c_[rng.randint(0, rows, size=[n]), rng.randint(0, cols, size=[n])].reshape(n, 1, 2)   #many targets repeat
+        column = rng.randint(0, cols, size=[1])
+        along  = rng.randint(0, cols, size=rows)[:, np.newaxis]
+        for fuse in (True, False):
+            print(f'case: scatter forms {rows}x{cols}, {n} points, fuse={fuse}', flush=True)
+            check_against_oracle(scatter_fn0, [ints(rows, cols), points, ints(n, 1)], exact=True, fuse=fuse)
+            check_against_oracle(scatter_add_fn1, [ints(rows, cols), column, ints(rows)], exact=True, fuse=fuse)
+            #the scatter behind an element-wise step and in front of one, so that the fusion passes see it
+            check_against_oracle(lambda x, i, u: scatter_fn0(x * 2.0, i, u + 1.0) - 3.0, [ints(rows, cols), points, ints(n, 1)], exact=True, fuse=fuse)
+            check_against_oracle(lambda x, i, u: scatter_add_fn1(x * 2.0, i, u + 1.0) - 3.0, [ints(rows, cols), column, ints(rows)], exact=True, fuse=fuse)
+            #the gradient of take_along_axis with a cotangent of small integers instead of 1 / n
+            g = lambda x, i: mj.grad(lambda x, i: (take_along_axis0(x, i) * 3.0).ravel().sum())(x, i)
+            y, _, fn = check_against_oracle(g, [ints(rows, cols), along], exact=True, fuse=fuse)
+            assert any(repr(op.equation).startswith('scatter-add') or 'scatter-add' in repr(op.equation)
+                       for op in list(fn._jaxpr_interpreters.values())[0].all_ops)
+            assert y.sum() == 3.0 * rows
+            check_against_oracle(take_along_axis0_g, [random([rows, cols]), along], rtol=1e-5, atol=1e-8, fuse=fuse)
+            check_against_oracle(scatter_fn0, [random([rows, cols]), points, random([n, 1])], rtol=1e-5, atol=1e-8, fuse=fuse)
+            check_against_oracle(scatter_add_fn1, [random([rows, cols]), column, random([rows])], rtol=1e-5, atol=1e-8, fuse=fuse)
 
 
 def test_nextafter_direction():

@@ -122,22 +122,17 @@ def test_every_tile_and_loader_variant(tile, bk):
     cases = {'ff': ([3, 20, 17, 16], [3, 3, 16, 24]), 'gg': ([2, 13, 11, 5], [3, 3, 5, 7]),
              'gf': ([2, 13, 11, 3], [3, 3, 3, 64]), 'fg': ([2, 13, 11, 8], [3, 3, 8, 10]),
              'ff2': ([2, 9, 11, 64], [3, 3, 64, 40]), 'ff3': ([2, 9, 11, 128], [1, 1, 128, 72])}
-    K.FORCE_CONV_TILE, K.FORCE_CONV_BK = tile, bk
-    try:
-        for variant, (xs, ks) in cases.items():
-            for general in (True, False):
-                K.FORCE_CONV_GENERAL = general
-                K.FORCE_CONV_B_GENERAL = variant[1] == 'g'           #(a dense kernel operand takes 16-byte loads whatever its width)
-                expected = variant[:2] if general or variant not in ('ff2', 'ff3') else 'lean'
-                print(f'tile {tile} bk {bk} loaders {variant} -> {expected}', flush=True)
-                x = rng.randint(-4, 5, size=xs).astype(np.float32)
-                k = rng.randint(-3, 4, size=ks).astype(np.float32)
+    for variant, (xs, ks) in cases.items():
+        for general in (True, False):
+            expected = variant[:2] if general or variant not in ('ff2', 'ff3') else 'lean'
+            print(f'tile {tile} bk {bk} loaders {variant} -> {expected}', flush=True)
+            x = rng.randint(-4, 5, size=xs).astype(np.float32)
+            k = rng.randint(-3, 4, size=ks).astype(np.float32)
+            #(a dense kernel operand takes 16-byte loads whatever its width)
+            with K.overrides(conv_tile=tile, conv_bk=bk, conv_general=general, conv_b_general=variant[1] == 'g'):
                 _, _, fn = check_against_oracle(conv2, [x, k], exact=True)
-                kernel = list(fn._jaxpr_interpreters.values())[0].launches[0].kernel
-                assert kernel == f'conv_gemm_{tile}x{bk}_{expected}', kernel
-    finally:
-        K.FORCE_CONV_TILE = K.FORCE_CONV_BK = None
-        K.FORCE_CONV_GENERAL = K.FORCE_CONV_B_GENERAL = False
+            kernel = list(fn._jaxpr_interpreters.values())[0].launches[0].kernel
+            assert kernel == f'conv_gemm_{tile}x{bk}_{expected}', kernel
 
 
 @pytest.mark.parametrize('tile,bk', TILES)
@@ -157,11 +152,8 @@ def test_lean_kernel_tile_chunks_with_epilogue(tile, bk):
     def bias_relu(x, k, bias):
         return nn.relu(lax.conv_general_dilated(x, k, (2, 2), 'VALID', dimension_numbers=dn) + bias)
 
-    K.FORCE_CONV_TILE, K.FORCE_CONV_BK = tile, bk
-    blocks_per_cu, min_tiles = K.CONV_BLOCKS_PER_CU, K.CONV_EVEN_SPLIT_MIN_TILES
-    try:
+    with K.overrides(conv_tile=tile, conv_bk=bk):
         for chunk in (1, 2, 3, 5):
-            K.FORCE_CONV_CHUNK = chunk
             for ksize, cin, cout in ((3, 64, 40), (1, 128, 72)):
                 print(f'tile {tile} bk {bk} chunk {chunk} kernel {ksize}x{ksize} {cin}->{cout}', flush=True)
                 x = rng.randint(-4, 5, size=[3, 13, 11, cin]).astype(np.float32)
@@ -170,30 +162,28 @@ def test_lean_kernel_tile_chunks_with_epilogue(tile, bk):
                 res = rng.randint(-50, 50, size=[3, 13, 11, cout]).astype(np.float32)
                 for f, args in ((bn_res_relu, [x, k, vec(-5, 5), vec(1, 4), vec(-9, 9), res]), (bias_relu, [x, k, vec(-9, 9)]),
                                 (conv2, [x, k])):
-                    _, _, fn = check_against_oracle(f, args, exact=True)
+                    with K.overrides(conv_chunk=chunk):
+                        _, _, fn = check_against_oracle(f, args, exact=True)
                     launches = list(fn._jaxpr_interpreters.values())[0].launches
                     assert [l.kernel for l in launches] == [f'conv_gemm_{tile}x{bk}_lean'], [l.kernel for l in launches]
         # a grid of a fixed number of blocks that share the M tiles of every N tile evenly (here 1, 2, 3 or 5 blocks
         # per N tile: runs of unequal length, blocks with a single tile, one block with all of them)
-        K.FORCE_CONV_CHUNK, K.CONV_EVEN_SPLIT_MIN_TILES = None, 0.0
         for per_n_tile in (1, 2, 3, 5):
             for ksize, cin, cout in ((3, 64, 40), (1, 128, 72)):
                 tiles_n = -(-cout // int(tile.split('x')[1]))
-                K.CONV_BLOCKS_PER_CU = (per_n_tile * tiles_n + 0.5) / 256
+                even = dict(conv_even_split_min_tiles=0.0, conv_blocks_per_cu=(per_n_tile * tiles_n + 0.5) / 256)
                 print(f'tile {tile} bk {bk} {per_n_tile} blocks per N tile, kernel {ksize}x{ksize} {cin}->{cout}', flush=True)
                 x = rng.randint(-4, 5, size=[3, 13, 11, cin]).astype(np.float32)
                 k = rng.randint(-3, 4, size=[ksize, ksize, cin, cout]).astype(np.float32)
                 vec = lambda lo, hi: rng.randint(lo, hi, size=[cout]).astype(np.float32)
                 res = rng.randint(-50, 50, size=[3, 13, 11, cout]).astype(np.float32)
                 for f, args in ((bn_res_relu, [x, k, vec(-5, 5), vec(1, 4), vec(-9, 9), res]), (bias_relu, [x, k, vec(-9, 9)])):
-                    _, _, fn = check_against_oracle(f, args, exact=True)
+                    with K.overrides(**even):
+                        _, _, fn = check_against_oracle(f, args, exact=True)
                     launches = list(fn._jaxpr_interpreters.values())[0].launches
                     assert [l.kernel for l in launches] == [f'conv_gemm_{tile}x{bk}_lean'], [l.kernel for l in launches]
                     tiles_m = -(-launches[0].buffers[0][0].size // cout // int(tile.split('x')[0]))
                     assert launches[0].grid[0] == min(per_n_tile, tiles_m) * tiles_n, (launches[0].grid, tiles_m, tiles_n)
-    finally:
-        K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = None
-        K.CONV_BLOCKS_PER_CU, K.CONV_EVEN_SPLIT_MIN_TILES = blocks_per_cu, min_tiles
 
 
 def test_four_waves_per_tile_kernel():
@@ -223,22 +213,17 @@ def test_four_waves_per_tile_kernel():
              #windows over 64 and 192 features: the 64-long k step
              (bn_res_relu, [ints(-4, 5, 1, 14, 9, 64), ints(-3, 4, 3, 3, 64, 64), ints(-5, 5, 64), ints(1, 4, 64), ints(-9, 9, 64), ints(-50, 50, 1, 14, 9, 64)]),
              (bn_res_relu, [ints(-4, 5, 2, 5, 6, 192), ints(-3, 4, 3, 3, 192, 33), ints(-5, 5, 33), ints(1, 4, 33), ints(-9, 9, 33), ints(-50, 50, 2, 5, 6, 33)])]
-    K.FORCE_CONV_KSPLIT, K.FORCE_CONV_K_SPLITS = True, 1
-    try:
-        for f, args in cases:
-            short = f is bn_res_relu and args[1].shape[0] == 3 and args[1].shape[2] % 128 != 0
-            for b_general in (False, True):
-                K.FORCE_CONV_B_GENERAL = b_general
-                print(f'four waves per tile: {f.__name__} {[a.shape for a in args]} element-wise kernel loads {b_general}', flush=True)
+    for f, args in cases:
+        short = f is bn_res_relu and args[1].shape[0] == 3 and args[1].shape[2] % 128 != 0
+        for b_general in (False, True):
+            print(f'four waves per tile: {f.__name__} {[a.shape for a in args]} element-wise kernel loads {b_general}', flush=True)
+            with K.overrides(conv_ksplit=True, conv_k_splits=1, conv_b_general=b_general):
                 _, _, fn = check_against_oracle(f, args, exact=True)
-                launches = list(fn._jaxpr_interpreters.values())[0].launches
-                if short:                                     #(this variant exists with 16-byte loads of the kernel operand only)
-                    assert ([l.kernel for l in launches] == ['conv_gemm_32x32x64_ks4']) == (not b_general), [l.kernel for l in launches]
-                else:
-                    assert [l.kernel for l in launches] == ['conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4'], [l.kernel for l in launches]
-    finally:
-        K.FORCE_CONV_KSPLIT = K.FORCE_CONV_K_SPLITS = None
-        K.FORCE_CONV_B_GENERAL = False
+            launches = list(fn._jaxpr_interpreters.values())[0].launches
+            if short:                                     #(this variant exists with 16-byte loads of the kernel operand only)
+                assert ([l.kernel for l in launches] == ['conv_gemm_32x32x64_ks4']) == (not b_general), [l.kernel for l in launches]
+            else:
+                assert [l.kernel for l in launches] == ['conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4'], [l.kernel for l in launches]
 
 
 def test_sliced_contractions():
@@ -266,20 +251,15 @@ def test_sliced_contractions():
              (bn_res_relu, [ints(-4, 5, 1, 7, 7, 512), ints(-3, 4, 1, 1, 512, 72), ints(-5, 5, 72), ints(1, 4, 72), ints(-9, 9, 72), ints(-50, 50, 1, 7, 7, 72)]),
              (bn_res_relu, [ints(-4, 5, 1, 7, 7, 128), ints(-3, 4, 3, 3, 128, 40), ints(-5, 5, 40), ints(1, 4, 40), ints(-9, 9, 40), ints(-50, 50, 1, 7, 7, 40)]),
              (bn_res_relu, [ints(-4, 5, 2, 5, 6, 256), ints(-3, 4, 3, 3, 256, 33), ints(-5, 5, 33), ints(1, 4, 33), ints(-9, 9, 33), ints(-50, 50, 2, 5, 6, 33)])]
-    K.FORCE_CONV_KSPLIT = True
-    try:
-        for f, args in cases:
-            for slices in (2, 3, 4, 7):
-                for b_general in (False, True):
-                    K.FORCE_CONV_K_SPLITS, K.FORCE_CONV_B_GENERAL = slices, b_general
-                    print(f'sliced contraction: {f.__name__} {[a.shape for a in args]} {slices} slices, element-wise kernel loads {b_general}', flush=True)
+    for f, args in cases:
+        for slices in (2, 3, 4, 7):
+            for b_general in (False, True):
+                print(f'sliced contraction: {f.__name__} {[a.shape for a in args]} {slices} slices, element-wise kernel loads {b_general}', flush=True)
+                with K.overrides(conv_ksplit=True, conv_k_splits=slices, conv_b_general=b_general):
                     _, _, fn = check_against_oracle(f, args, exact=True)
-                    launches = list(fn._jaxpr_interpreters.values())[0].launches
-                    assert launches[0].kernel == ('conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4')
-                    assert launches[0].buffers[0][0].shape[0] > 1 and all(l.kernel.startswith(('ew_chain', 'ew_affine')) for l in launches[1:]), [l.kernel for l in launches]
-    finally:
-        K.FORCE_CONV_KSPLIT = K.FORCE_CONV_K_SPLITS = None
-        K.FORCE_CONV_B_GENERAL = False
+                launches = list(fn._jaxpr_interpreters.values())[0].launches
+                assert launches[0].kernel == ('conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4')
+                assert launches[0].buffers[0][0].shape[0] > 1 and all(l.kernel.startswith(('ew_chain', 'ew_affine')) for l in launches[1:]), [l.kernel for l in launches]
     #by the heuristic: a 3x3 layer of a network's last stage on one image (32 tiles, 36 k steps), against float data
     x, k = rng.randn(1, 7, 7, 512).astype(np.float32), (rng.randn(3, 3, 512, 512) / 68).astype(np.float32)
     _, _, fn = check_against_oracle(lambda a, b: nn.relu(lax.conv_general_dilated(a, b, (1, 1), 'SAME', dimension_numbers=dn)), [x, k], rtol=1e-4, atol=1e-5)
@@ -313,23 +293,16 @@ def test_mixed_tiling():
     cases = [conv_case(3, 13, 11, 3, 64, 72), conv_case(2, 14, 14, 3, 128, 256), conv_case(5, 7, 7, 1, 256, 100),
              conv_case(3, 14, 14, 3, 64, 64, stride=2), (conv2, [ints(-4, 5, 2, 20, 17, 64), ints(-3, 4, 3, 3, 64, 40)]),
              (dense, [ints(-4, 5, 300, 328), ints(-3, 4, 328, 136), ints(-9, 9, 136)])]
-    try:
-        for f, args in cases:
-            for bk in (32, 64):
-                K.FORCE_CONV_TILE, K.FORCE_CONV_BK, K.FORCE_CONV_CHUNK, K.FORCE_CONV_KSPLIT = '64x64', bk, 1, False
-                try:
-                    for split in (1, 2, 5):
-                        K.FORCE_CONV_MIX = split
-                        print(f'mixed tiling: {f.__name__} {[a.shape for a in args]} bk {bk}, {split} M tiles of 64 rows', flush=True)
-                        _, _, fn = check_against_oracle(f, args, exact=True)
-                        launches = list(fn._jaxpr_interpreters.values())[0].launches
-                        m = launches[0].flops // (2 * int(np.prod(args[1].shape[:-1])) * args[1].shape[-1])
-                        expected = f'conv_gemm_64x64x{bk}_mix' if split * 64 < m else f'conv_gemm_64x64x{bk}_lean'
-                        assert [l.kernel for l in launches] == [expected], ([l.kernel for l in launches], m)
-                finally:
-                    K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = K.FORCE_CONV_KSPLIT = K.FORCE_CONV_MIX = None
-    finally:
-        K.FORCE_CONV_TILE = K.FORCE_CONV_BK = K.FORCE_CONV_CHUNK = K.FORCE_CONV_KSPLIT = K.FORCE_CONV_MIX = None
+    for f, args in cases:
+        for bk in (32, 64):
+            for split in (1, 2, 5):
+                print(f'mixed tiling: {f.__name__} {[a.shape for a in args]} bk {bk}, {split} M tiles of 64 rows', flush=True)
+                with K.overrides(conv_tile='64x64', conv_bk=bk, conv_chunk=1, conv_ksplit=False, conv_mix=split):
+                    _, _, fn = check_against_oracle(f, args, exact=True)
+                launches = list(fn._jaxpr_interpreters.values())[0].launches
+                m = launches[0].flops // (2 * int(np.prod(args[1].shape[:-1])) * args[1].shape[-1])
+                expected = f'conv_gemm_64x64x{bk}_mix' if split * 64 < m else f'conv_gemm_64x64x{bk}_lean'
+                assert [l.kernel for l in launches] == [expected], ([l.kernel for l in launches], m)
 
 
 def test_stem_kernel_for_few_input_features():

@@ -56,6 +56,28 @@ def test_argmax_argmin_ties_and_nans(shape, axis):
     check_against_oracle(lambda x: jnp.max(x, axis=axis), [x], exact=True)
 
 
+@pytest.mark.parametrize('width', [1000, 1003, 64, 257])
+def test_argmax_argmin_treat_signed_zeros_as_equal(width):
+    '''-0.0 and +0.0 compare equal, so the first of them wins whatever its sign, also when the two sit in different
+    lanes of the wave that reduces the row (numpy and XLA agree; widths divisible by 4 take the 16-byte kernel).'''
+    x = np.full((6, width), -5.0, np.float32)
+    x[0, 3], x[0, 200 % width] = -0.0, 0.0             #maximum: -0.0 first, +0.0 later in another lane
+    x[1, 5], x[1, width - 1] = 0.0, -0.0
+    x[2, 70 % width], x[2, 7] = -0.0, 0.0               #+0.0 first
+    y = -x                                              #minimum: rows of +5 with zeros of either sign
+    y[3:] = 0.0
+    y[3, 1::2] = -0.0                                   #a whole row of zeros of alternating sign: index 0
+    y[4, 0], y[5, :] = -0.0, -0.0
+    x[3:] = y[3:]
+    for a in (x, y):
+        check_against_oracle(lambda a: jnp.argmax(a, axis=1), [a], exact=True)
+        check_against_oracle(lambda a: jnp.argmin(a, axis=1), [a], exact=True)
+        check_against_oracle(lambda a: jnp.argmax(a, axis=0), [a], exact=True)     #the column kernel
+        check_against_oracle(lambda a: jnp.argmin(a, axis=0), [a], exact=True)
+    #the arg-max that a softmax launch returns with its probabilities (all of them positive: same labels as numpy)
+    check_against_oracle(lambda a: jnp.argmax(mj.nn.softmax(a, axis=-1), axis=-1), [x], exact=True)
+
+
 def test_float_sum_within_tolerance():
     x = rng.random_sample((3, 1 << 21)).astype(np.float32)
     check_against_oracle(lambda x: jnp.sum(x, axis=1), [x], rtol=1e-5, atol=0)

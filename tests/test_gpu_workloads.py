@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import vkjax_amd
-from vkjax_amd import minijax as mj, workloads as W
+from vkjax_amd import kernels as K, minijax as mj, workloads as W
 from tests.common import check_against_oracle, assert_tree_close, oracle_outputs
 
 pytestmark = pytest.mark.gpu
@@ -159,10 +159,8 @@ def test_scatter_add_rows_sorted_and_atomic_paths():
             return mj.numpy.index_add(mj.numpy.full((300, 64), fill, np.float32), idx, updates)
         return f
 
-    saved = ops.SCATTER_SORT_THRESHOLD
-    try:
-        for path, threshold in (('sum', 0), ('atomic', 1 << 60)):
-            ops.SCATTER_SORT_THRESHOLD = threshold
+    for path, threshold in (('sum', 0), ('atomic', 1 << 60)):
+        with K.overrides(scatter_sort_threshold=threshold):
             cases = [(50, 256, 400, np.float32), (9, 10, 37, np.float32), (300, 64, 200, np.int32), (4, 20, 500, np.float32),
                      (3000, 16, 9000, np.float32), (70, 520, 300, np.float32), (5, 8, 20000, np.int32), (1029, 4, 30000, np.float32),
                      (300000, 4, 5000, np.float32), (1025, 4, 3000, np.int32), (1024, 4, 3000, np.int32), (1023, 4, 3000, np.int32)]
@@ -194,8 +192,63 @@ def test_scatter_add_rows_sorted_and_atomic_paths():
                 if path == 'sum':
                     launch = [l for l in list(fn._jaxpr_interpreters.values())[0].launches if l.kernel.startswith('scatter_rows_sum')][0]
                     assert launch.buffers[1][0].size == 1, 'the constant table should have been replaced by its value'
-    finally:
-        ops.SCATTER_SORT_THRESHOLD = saved
+
+
+def test_binding_repeated_equations_to_one_buffer_changes_no_bit():
+    '''An equation that repeats an earlier one is bound to that one's buffer: programs in which that happens (the
+    index normalisation of a gather followed by a scatter-add, repeated views and element-wise steps) give the same
+    bits with the pass switched off, fused and unfused.'''
+    rng = np.random.default_rng(23)
+    def views_and_chains(x, y):
+        a = (x + 1.0) * (x + 1.0)
+        b = x.reshape(-1)[::2] + x.reshape(-1)[::2]
+        c = mj.numpy.exp(x.T) - mj.numpy.exp(x.T) * y.T
+        return a + y, b, c, (x + 1.0).sum(axis=0)
+    idx = rng.integers(-40, 40, size=(64, 3)).astype(np.int32)
+    programs = [(W.gather_scatter, [rng.random((40, 24), dtype=np.float32), idx, rng.random((64, 3, 24), dtype=np.float32)]),
+                (W.gather_scatter, W.gather_scatter_inputs(rows=512, cols=256, n0=256, n1=8)),
+                (views_and_chains, [rng.random((18, 32), dtype=np.float32), rng.random((18, 32), dtype=np.float32)])]
+    for f, args in programs:
+        for fuse in (True, False):
+            with K.overrides(reuse_equal_equations=True):
+                bound = vkjax_amd.wrap(f, frontend='minijax', fuse=fuse)
+                y = bound(*args)
+            with K.overrides(reuse_equal_equations=False):
+                plain = vkjax_amd.wrap(f, frontend='minijax', fuse=fuse)
+                ytrue = plain(*args)
+            count = lambda fn: len(list(fn._jaxpr_interpreters.values())[0].launches)
+            assert count(bound) < count(plain), (f.__name__, fuse, count(bound), count(plain))
+            assert_tree_close(y, ytrue, exact=True, what=f'{f.__name__} fuse={fuse}')
+
+
+def test_failed_evaluation_leaves_the_scatter_counters_zero():
+    '''The sorted scatter-add counts in an array that every evaluation leaves zero again - if it runs to the end.
+    After an evaluation that failed half way the interpreter writes the zeros again, so the next one is right.'''
+    from vkjax_amd import hip
+    rng = np.random.default_rng(17)
+    table   = rng.integers(-9, 9, size=(300, 64)).astype(np.float32)
+    idx     = rng.integers(0, 300, size=(2000,)).astype(np.int32)
+    updates = rng.integers(-5, 6, size=(2000, 64)).astype(np.float32)
+    expected = table.copy()
+    np.add.at(expected, idx, updates)
+    with K.overrides(scatter_sort_threshold=0):
+        fn = vkjax_amd.wrap(lambda t, i, u: mj.numpy.index_add(t, i, u), frontend='minijax')
+        assert np.array_equal(fn(table, idx, updates), expected)
+    interp = list(fn._jaxpr_interpreters.values())[0]
+    counters = [b for key, b in interp.bufferpool.buffers.items() if isinstance(key, tuple) and key[:1] == ('zeroed',)]
+    assert counters
+    real = interp.sequence.eval
+    def stopped_half_way(*args, **kwargs):
+        for b in counters:
+            b.tensor.upload(np.full(b.size, 7, np.uint32))     #what the counting launch leaves when the ordering launch never ran
+        raise hip.HipError('injected failure')
+    interp.sequence.eval = stopped_half_way
+    with pytest.raises(hip.HipError, match='injected'):
+        fn(table, idx, updates)
+    interp.sequence.eval = real
+    for b in counters:
+        assert not b.numpy().any()
+    assert np.array_equal(fn(table, idx, updates), expected)
 
 
 def test_fusion_does_not_change_a_single_bit():
@@ -334,13 +387,10 @@ def test_affine_chains_in_straight_line_code():
             args = [first, s1, s2, s3, vsub, vmul, vadd, full]
             results = []
             for forced in (True, False):
-                K.FORCE_EW_AFFINE = forced
-                try:
+                with K.overrides(ew_affine=forced):
                     fn = vkjax_amd.wrap(f, frontend='minijax')
                     results.append(fn(*args))
                     kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
-                finally:
-                    K.FORCE_EW_AFFINE = None
                 #(nine operands are two launches: a chain holds eight)
                 assert all((k == 'ew_affine_v4') == forced for k in kernels) and len(kernels) <= 2, (kernels, forced, shape, nsum, parts)
             assert_tree_close(results[0], results[1], exact=True, what=f'{shape} {nsum} {parts}')
@@ -354,13 +404,10 @@ def test_affine_chains_in_straight_line_code():
                     (lambda x, y, z, w, t: x + y + z + w + t, [big, res, big[::-1].copy(), res[::-1].copy(), t])):
         results = []
         for forced in (None, False):
-            K.FORCE_EW_AFFINE = forced
-            try:
+            with K.overrides(ew_affine=forced):
                 fn = vkjax_amd.wrap(f, frontend='minijax')
                 results.append(fn(*args))
                 kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
-            finally:
-                K.FORCE_EW_AFFINE = None
             assert kernels == (['ew_affine_big_v4'] if forced is None else [kernels[0]]) and (forced is None or kernels[0].startswith('ew_chain')), kernels
         assert_tree_close(results[0], results[1], exact=True, what='large affine chain')
     #by itself: chains of more than four operands on arrays that are not large
@@ -424,7 +471,7 @@ def test_gather_fill_and_scatter_clip_modes():
     check_against_oracle(lambda t, i, u: lax.scatter_add(t, i, u, S((1, 2), (), (0, 1)), mode='clip'), [table, starts, win], exact=True)
     #the sorted (atomic-free) kernels
     table = rng.integers(-50, 50, size=(500, 64)).astype(np.float32)
-    idx   = rng.integers(-100, 600, size=(ops.SCATTER_SORT_THRESHOLD // 64 + 7, 1)).astype(np.int32)
+    idx   = rng.integers(-100, 600, size=(K.CHOICES.scatter_sort_threshold // 64 + 7, 1)).astype(np.int32)
     upd   = rng.integers(-9, 9, size=(idx.shape[0], 64)).astype(np.float32)
     for mode in ('clip', None):
         _, _, fn = check_against_oracle(lambda t, i, u: lax.scatter_add(t, i, u, rows_sd, mode=mode), [table, idx, upd], exact=True)
@@ -526,6 +573,70 @@ def test_resident_arguments_are_uploaded_once():
     assert_tree_close(resident(params2, x2), plain(params2, x2), exact=True, what='one weight replaced')
     interp = list(resident._jaxpr_interpreters.values())[0]
     assert len(interp._resident_leaves) == len(leaves)
+
+
+def test_read_only_leaves_stay_in_hbm_without_being_asked():
+    '''Plain `wrap(f)(params, x)`: leaves that cannot change under the caller's feet (numpy arrays that are not
+    writeable) are uploaded once and again only when replaced; writeable ones are copied on every call, as the
+    reference does with every argument (vkjax/kompute_jaxpr_interpreter.py:72-75); a read-only view of a writeable
+    array counts as writeable. With resident_argnums a writeable leaf that is changed in place where the cheap
+    check looks (its first and last 64 bytes) is uploaded again.'''
+    from vkjax_amd.minijax import tree_util
+    params, x = W.mlp_inputs()
+    plain = vkjax_amd.wrap(W.mlp, frontend='minijax', resident_argnums=())
+    def frozen(a):
+        a = a.copy()
+        a.flags.writeable = False
+        return a
+    def counted(f, *args):
+        interp = f._get_or_create_jaxpr_interpreter(args)[0]
+        real, seen = interp.sequence.eval, []
+        def spy(host, *a, **kw):
+            seen.append(sum(host[s] is not None for s in interp._input_slots if s is not None))
+            return real(host, *a, **kw)
+        interp.sequence.eval = spy
+        try:
+            y = f(*args)
+        finally:
+            interp.sequence.eval = real
+        return y, seen[0]
+    n = len(tree_util.tree_leaves(params))
+    f = vkjax_amd.wrap(W.mlp, frontend='minijax')
+    ro = tree_util.tree_map(frozen, params)
+    for k, (xx, want) in enumerate([(x, n + 1), (x[::-1].copy(), 1), (x, 1)]):
+        y, uploads = counted(f, ro, xx)
+        assert uploads == want, (k, uploads)
+        assert_tree_close(y, plain(params, xx), exact=True, what=f'read-only weights, call {k}')
+    #a replaced leaf is picked up; the others stay
+    leaves, structure = tree_util.tree_flatten(ro)
+    ro2 = tree_util.tree_unflatten(structure, [frozen(leaves[0] * np.float32(0.5))] + list(leaves[1:]))
+    y, uploads = counted(f, ro2, x)
+    assert uploads == 2
+    assert_tree_close(y, plain(ro2, x), exact=True, what='one read-only weight replaced')
+    #writeable weights: every call copies everything, and sees changes made in place
+    g = vkjax_amd.wrap(W.mlp, frontend='minijax')
+    rw = tree_util.tree_map(np.copy, params)
+    for k in range(3):
+        tree_util.tree_leaves(rw)[0][5, 7] += np.float32(1.0)
+        y, uploads = counted(g, rw, x)
+        assert uploads == n + 1, (k, uploads)
+        assert_tree_close(y, plain(tree_util.tree_map(np.copy, rw), x), exact=True, what=f'writeable weights, call {k}')
+    #a read-only window into a writeable array can change: copied every call
+    views = tree_util.tree_map(lambda a: a.view(), rw)
+    for v in tree_util.tree_leaves(views):
+        v.flags.writeable = False
+    h = vkjax_amd.wrap(W.mlp, frontend='minijax')
+    assert counted(h, views, x)[1] == n + 1 and counted(h, views, x)[1] == n + 1
+    #resident_argnums with writeable leaves: kept, unless a change shows in the first or last 64 bytes
+    r = vkjax_amd.wrap(W.mlp, frontend='minijax', resident_argnums=(0,))
+    assert counted(r, rw, x)[1] == n + 1 and counted(r, rw, x)[1] == 1
+    first = tree_util.tree_leaves(rw)[0]
+    first.reshape(-1)[3] += np.float32(2.0)
+    y, uploads = counted(r, rw, x)
+    assert uploads == 2
+    assert_tree_close(y, plain(tree_util.tree_map(np.copy, rw), x), exact=True, what='changed in place near the start')
+    first.reshape(-1)[-1] -= np.float32(2.0)
+    assert counted(r, rw, x)[1] == 2
 
 
 def test_stream_matches_call_by_call():

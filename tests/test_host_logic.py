@@ -340,14 +340,11 @@ def test_batch_of_one_fuses_like_any_other():
     from vkjax_amd import workloads as W
     from vkjax_amd import kernels as K
     counts = []
-    K.FORCE_CONV_K_SPLITS = 1                  #(a sliced contraction would add a launch of its own)
-    try:
+    with K.overrides(conv_k_splits=1):         #(a sliced contraction would add a launch of its own)
         for batch in (1, 2):
             fn = vkjax_amd.wrap(W.resnet50, frontend='minijax', plan_only=True)
             interp, _ = fn._get_or_create_jaxpr_interpreter(tuple(W.resnet50_inputs(batch=batch, size=64, num_classes=40, width_scale=0.25)))
             counts.append(len(interp.launches))
-    finally:
-        K.FORCE_CONV_K_SPLITS = None
     assert counts[0] == counts[1] == 58, counts
 
 
@@ -374,12 +371,9 @@ def test_long_contractions_of_few_tiles_are_sliced():
     assert [l.kernel for l in plan(49, 640, 512).launches] == ['conv_gemm_32x32x128_ks4']        #5 k steps: too short to slice
     assert [l.kernel for l in plan(49, 1024, 512).launches][0] == 'conv_gemm_32x32x128_ks4' and plan(49, 1024, 512).launches[0].grid == (64, 1, 1)
     assert len(plan(2048, 4608, 512).launches) == 1                #1024 tiles
-    K.FORCE_CONV_K_SPLITS = 3
-    try:
+    with K.overrides(conv_k_splits=3):
         forced = plan(40, 1000, 24)                                #8 k steps in 3 slices of 3, 3 and 2
-        assert forced.launches[0].grid == (2 * 3, 1, 1) and forced.launches[0].buffers[0][0].shape == (3, 40 * 24)
-    finally:
-        K.FORCE_CONV_K_SPLITS = None
+    assert forced.launches[0].grid == (2 * 3, 1, 1) and forced.launches[0].buffers[0][0].shape == (3, 40 * 24)
 
 
 def test_size_limits_are_reported_when_the_program_is_built():
@@ -435,11 +429,13 @@ def test_repeated_equations_are_evaluated_once():
     closed = mj.make_jaxpr(fn)(*make())
     kernels = lambda **kw: [l.kernel for l in JaxprInterpreter(closed, plan_only=True, **kw).launches]
     assert len(kernels()) == 6 and len(kernels(fuse=False)) == 8          #(fused: x + n, x < 0 and the select in one pass)
-    ops.REUSE_EQUAL_EQUATIONS = False
-    try:
+    from vkjax_amd import kernels as K
+    with K.overrides(reuse_equal_equations=False):
         assert len(kernels()) == 7 and len(kernels(fuse=False)) == 11
-    finally:
-        ops.REUSE_EQUAL_EQUATIONS = True
+    with pytest.raises(TypeError, match='unknown choice'):
+        with K.overrides(no_such_choice=1):
+            pass
+    assert K.CHOICES.reuse_equal_equations is True
     def f(x):
         a = (x + 1.0) * (x + 1.0)          #x + 1 once
         b = (x + 2.0) * (x + np.float32(1.0))
@@ -531,3 +527,19 @@ def test_evenly_split_conv_grids():
     launch = K.conv_gemm(b(64, 28, 28, 512), b(64, 28, 28, 128), b(1, 1, 128, 512), geom)
     assert launch.kernel == 'conv_gemm_64x64x32_lean' and launch.grid[0] == 1280
     assert np.frombuffer(launch.params, np.int32)[-3 - 9:-9].tolist() == [160, 4, 144]   #blocks per N tile, tiles each, blocks with one more: the end of ConvParams, before the 9 of ConvDerived
+
+
+def test_which_argument_leaves_count_as_immutable():
+    '''Leaves that stay in HBM without being asked: only arrays nobody can write through.'''
+    from vkjax_amd.jaxpr_interpreter import _is_immutable, _may_change_in_place
+    a = np.arange(12, dtype=np.float32)
+    assert not _is_immutable(a) and _may_change_in_place(a)
+    view = a[2:8]
+    view.flags.writeable = False
+    assert not _is_immutable(view)                       #a window into a writeable array
+    b = a.copy()
+    b.flags.writeable = False
+    assert _is_immutable(b) and _is_immutable(b[1:5]) and not _may_change_in_place(b)
+    assert _is_immutable(np.frombuffer(b'\x00' * 16, np.float32))         #backed by a bytes object
+    assert not _is_immutable(np.frombuffer(bytearray(16), np.float32))
+    assert not _is_immutable(3.0) and not _is_immutable(np.float32(3.0)) and not _may_change_in_place(3.0)

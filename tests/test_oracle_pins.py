@@ -320,6 +320,9 @@ def test_reductions_and_argmax_rules():
     assert P.argmax(t, (1,)).tolist() == [1, 0, 0]       #first of ties; first NaN wins
     assert P.argmin(t, (1,)).tolist() == [0, 0, 0]
     assert np.isnan(P.reduce_max(t, (1,))[1])
+    z = np.array([[-1, -0.0, 0.0, -2], [-1, 0.0, -0.0, -2], [1, 0.0, -0.0, 2]], np.float32)
+    assert P.argmax(z, (1,)).tolist() == [1, 1, 3]       #the two zeros are equal: the first of them wins, whatever its sign
+    assert P.argmin(-z, (1,)).tolist() == [1, 1, 3]
 
 
 def test_integer_and_shift_semantics():

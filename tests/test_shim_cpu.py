@@ -26,12 +26,12 @@ def lib(tmp_path_factory):
                    check=True, capture_output=True, text=True)
     lib = C.CDLL(out)
     for name, (restype, argtypes) in hip._PROTOTYPES.items():
-        if name == 'vkj_seq_eval_next_static':
-            continue                                   #lives in static_landing.hip (device code), not in this build
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = restype, argtypes
     lib.fake_hip_live_objects.restype = C.c_long
     lib.fake_hip_launches.restype = C.c_long
+    lib.fake_hip_creations.restype = C.c_long
+    lib.fake_hip_on_synchronize.argtypes = [C.c_void_p]
     lib.fake_hip_fail_after.argtypes = [C.c_long]
     return lib
 
@@ -223,3 +223,89 @@ def test_objects_of_another_context_and_bad_ranges_are_rejected(lib):
         assert lib.vkj_buf_free(w.ctx, b) == 0
     assert lib.vkj_buf_free(w2.ctx, other) == 0
     w.close(); w2.close()
+
+
+def test_static_entry_point_allocates_nothing_and_equals_the_allocating_one(lib):
+    '''vkj_seq_eval_next_static (its host side; the stand-in build moves the landed bytes with a host copy): across
+    its calls the stand-in runtime sees no allocation, pinned allocation, stream, event or graph being made, for
+    small arguments and for ones that are staged in chunks by helper threads, and the results equal
+    vkj_seq_eval_next's.'''
+    w = World(lib)
+    rng = np.random.default_rng(11)
+    for n in (1000, 3 << 20):                                    #4 KB; 12 MB (three chunks)
+        seq, src, dst = w.add_one_sequence(n)
+        seq2, src2, dst2 = w.add_one_sequence(n)
+        xs = [rng.integers(0, 1 << 32, size=n, dtype=np.uint64).astype(np.uint32) for _ in range(4)]
+        want = [w.eval(seq2, xs[0], nxt=xs[1])] + [w.eval(seq2, None, nxt=x, flags=hip.EVAL_NULL_IS_RESIDENT, n=n) for x in xs[2:] + xs[:1]]
+        made = lib.fake_hip_creations()
+        got = []
+        for k in range(4):
+            y = np.zeros(n, np.uint32)
+            ptrs  = (C.c_void_p * 2)(xs[0].ctypes.data if k == 0 else None, y.ctypes.data)
+            nptrs = (C.c_void_p * 2)(xs[(k + 1) % 4].ctypes.data, None)
+            assert lib.vkj_seq_eval_next_static(seq, ptrs, 2, hip.EVAL_NULL_IS_RESIDENT, nptrs) == 0, lib.vkj_last_error()
+            got.append(y)
+        assert lib.fake_hip_creations() == made
+        for k, (a, b) in enumerate(zip(got, want)):
+            assert np.array_equal(a, b) and np.array_equal(a, xs[k] + 1), (n, k)
+        for q in (seq, seq2):
+            assert lib.vkj_seq_destroy(q) == 0
+        for b in (src, dst, src2, dst2):
+            assert lib.vkj_buf_free(w.ctx, b) == 0
+    w.close()
+
+
+def test_static_entry_point_refuses_a_call_that_overlaps_another(lib):
+    '''The static landing array is one per GPU: while a call is using it, a second call on that GPU (here: made from
+    inside the first one's final synchronisation, from another context) is refused, and the first is unharmed.'''
+    w, w2 = World(lib), World(lib)
+    seq, src, dst = w.add_one_sequence(256)
+    seq2, src2, dst2 = w2.add_one_sequence(256)
+    x = np.arange(256, dtype=np.uint32)
+    y, y2 = np.zeros(256, np.uint32), np.zeros(256, np.uint32)
+    ptrs,  nptrs  = (C.c_void_p * 2)(x.ctypes.data, y.ctypes.data),  (C.c_void_p * 2)(x.ctypes.data, None)
+    ptrs2, nptrs2 = (C.c_void_p * 2)(x.ctypes.data, y2.ctypes.data), (C.c_void_p * 2)(x.ctypes.data, None)
+    seen = []
+
+    @C.CFUNCTYPE(None)
+    def reenter():
+        seen.append(lib.vkj_seq_eval_next_static(seq2, ptrs2, 2, 0, nptrs2))
+        seen.append(lib.vkj_last_error())
+    lib.fake_hip_on_synchronize(C.cast(reenter, C.c_void_p))
+    assert lib.vkj_seq_eval_next_static(seq, ptrs, 2, 0, nptrs) == 0, lib.vkj_last_error()
+    assert seen[0] == ESTATE and b'busy' in seen[1], seen
+    assert np.array_equal(y, x + 1) and not y2.any()
+    assert lib.vkj_seq_eval_next_static(seq2, ptrs2, 2, 0, nptrs2) == 0      #free again once the first call has returned
+    assert np.array_equal(y2, x + 1)
+    for q in (seq, seq2):
+        assert lib.vkj_seq_destroy(q) == 0
+    for ww, bs in ((w, (src, dst)), (w2, (src2, dst2))):
+        for b in bs:
+            assert lib.vkj_buf_free(ww.ctx, b) == 0
+        ww.close()
+
+
+def test_static_entry_point_and_graphs(lib):
+    '''A sequence that replays as a graph is refused until the graph exists (building it allocates) - but a graph is
+    only ever built for more than one launch, so a single-launch sequence with graphs switched on is evaluated.'''
+    w = World(lib)
+    seq, src, dst = w.add_one_sequence(32)
+    assert lib.vkj_seq_use_graph(seq, 1) == 0
+    x = np.arange(32, dtype=np.uint32)
+    y = np.zeros(32, np.uint32)
+    ptrs = (C.c_void_p * 2)(x.ctypes.data, y.ctypes.data)
+    assert lib.vkj_seq_eval_next_static(seq, ptrs, 2, 0, None) == 0, lib.vkj_last_error()
+    assert np.array_equal(y, x + 1)
+    assert w.record_add_one(seq, src, dst, 32) == 0              #a second launch: src = dst + 1
+    assert lib.vkj_seq_eval_next_static(seq, ptrs, 2, 0, None) == ESTATE
+    assert b'graph' in lib.vkj_last_error()
+    assert lib.vkj_seq_eval(seq, ptrs, 2, 0) == 0                #builds it (the stand-in cannot: plain launches from now on)
+    assert lib.vkj_seq_eval_next_static(seq, ptrs, 2, 0, None) == 0, lib.vkj_last_error()
+    profiled = H()
+    assert lib.vkj_seq_create(w.ctx, 1, C.byref(profiled)) == 0
+    assert lib.vkj_seq_eval_next_static(profiled, None, 0, 0, None) == ESTATE
+    for q in (seq, profiled):
+        assert lib.vkj_seq_destroy(q) == 0
+    for b in (src, dst):
+        assert lib.vkj_buf_free(w.ctx, b) == 0
+    w.close()

@@ -323,6 +323,40 @@ def test_training_step_hip_matches_oracle(name, make_inputs):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize('name,make_inputs,atol', [('mlp_train', small_mlp_inputs, 1e-6), ('convnet_train', small_convnet_inputs, 5e-5)])
+def test_every_variable_of_a_training_step(name, make_inputs, atol):
+    '''The reference's deep inspection of a training step (tests/common.py:67-81, tests/test_elegy_mlp.py:120-129,
+    tests/test_elegy_conv.py:51-94): the program is built again without buffer reuse (and here without fusion, so
+    that every equation keeps a launch and a buffer of its own), run with return_all=True, and EVERY variable of
+    the jaxpr - not only the results - is compared with the evaluator's environment, at the reference's tolerances
+    (numpy's default rtol 1e-5 with atol 1e-6 for the MLP, 5e-5 for the conv net).'''
+    from vkjax_amd.minijax import tree_util
+    fn, _  = W.WORKLOADS[name]
+    args   = make_inputs()
+    closed = mj.make_jaxpr(fn)(*args)
+    interp = JaxprInterpreter(closed, reuse_buffers=False, fuse=False)
+    outs, envpred = interp.run(*args, return_all=True)
+    outs_true, envtrue = eval_closed_jaxpr(closed, *tree_util.tree_leaves(args), return_env=True)
+    assert len(envtrue) >= len(closed.jaxpr.eqns) and len(outs) == len(outs_true)
+    checked, worst = 0, (0.0, None)
+    for var, vtrue in envtrue.items():
+        if np.size(vtrue) == 0:
+            continue
+        vpred = envpred.get(var)
+        assert vpred is not None, f'{var}: no buffer'
+        assert np.shape(vpred) == np.shape(vtrue) and vpred.dtype == vtrue.dtype, (var, np.shape(vpred), np.shape(vtrue), vpred.dtype, vtrue.dtype)
+        if vtrue.dtype.kind in 'iub':
+            assert np.array_equal(vpred, vtrue), var
+        else:
+            err = float(np.max(np.abs(vpred.astype(np.float64) - vtrue) / (atol + 1e-5 * np.abs(vtrue))))
+            worst = max(worst, (err, str(var)))
+            assert err <= 1.0, f'{var} {np.shape(vtrue)}: |err| / (atol + rtol |y|) = {err:.3g}'
+        checked += 1
+    print(f'{name}: {checked} variables, worst |err| / (atol + rtol |y|) = {worst[0]:.3g} at {worst[1]}', flush=True)
+    assert checked >= len(closed.jaxpr.eqns)
+
+
+@pytest.mark.gpu
 def test_repeated_training_steps_reduce_the_loss():
     import vkjax_amd
     params, x, onehot = small_mlp_inputs()

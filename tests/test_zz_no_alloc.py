@@ -72,3 +72,22 @@ def test_static_landing_refuses_what_does_not_fit():
     prof._fresh_outputs(h)
     with pytest.raises(hip.HipError, match='timestamps'):
         prof.sequence.eval(h, next_host_arrays=[None] * len(h), static_landing=True)
+
+
+def test_static_landing_with_graphs_switched_on():
+    '''A program of one launch never becomes a graph, so it is evaluated although graphs are asked for; a program of
+    several launches is refused until an ordinary evaluation has built its graph, and equals it afterwards.'''
+    x = np.arange(4096, dtype=np.float32)
+    one = vkjax_amd.wrap(_program, frontend='minijax', graph=True)._get_or_create_jaxpr_interpreter((x,))[0]
+    assert len(one.launches) == 1
+    got = _streamed(one, [x, x + 1, x + 2], static_landing=True)
+    for k, g in enumerate(got):
+        assert np.array_equal(g, (x + k) * np.float32(3.0) + np.float32(1.0)), k
+    several = vkjax_amd.wrap(_program, frontend='minijax', graph=True, fuse=False)._get_or_create_jaxpr_interpreter((x,))[0]
+    assert len(several.launches) == 2
+    with pytest.raises(hip.HipError, match='graph has not been built'):
+        _streamed(several, [x, x + 1], static_landing=True)
+    expected = _streamed(several, [x, x + 1, x + 2], static_landing=False)
+    got = _streamed(several, [x, x + 1, x + 2], static_landing=True)
+    for g, e in zip(got, expected):
+        assert np.array_equal(g.view(np.uint32), e.view(np.uint32))

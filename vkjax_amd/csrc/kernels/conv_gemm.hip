@@ -109,14 +109,6 @@ struct ConvDerived {
     uint32_t left[CONV_MAX_DERIVED];        // the operand is the left argument
 };
 
-// Optional per-block phase time stamps (profiling builds only): slot s of block b lands in
-// ((uint64*)epi.p[CONV_MAX_EPI - 1])[16 * b + s].
-#ifdef CONV_PHASE_STAMPS
-#define CONV_STAMP(slot) stamps[slot] = wall_clock64();
-#else
-#define CONV_STAMP(slot)
-#endif
-
 // LEAN: the variant for the common case, with the rarely needed paths compiled out (they cost
 // registers, and with them resident waves, even when not taken): both operands on the 16-byte
 // path, k tiles that never straddle kernel taps, a row-major result, an epilogue that fits the
@@ -136,10 +128,6 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     float* const Bs = As + BM * LDA;                // [BK][LDB]
     float* const Es = Bs + BK * LDB;                // [CONV_MAX_EPI][BN]: per-column operands of the epilogue steps
     int*   const Rs = reinterpret_cast<int*>(Es + CONV_MAX_EPI * BN);   // [BM]: row offsets of outputs that are not row-major
-#ifdef CONV_PHASE_STAMPS
-    unsigned long long stamps[16] = {};
-#endif
-    CONV_STAMP(0)
 
     // Copy the hot part of the argument block into scalar registers once, at the very start. Left
     // to itself the compiler fetches each field right before its first use; under load every such
@@ -487,7 +475,6 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
 
     float full[PREFETCH_FULL ? TM : 1][PREFETCH_FULL ? TN : 1][16];
     setup_rows(region.m_base + tile_m0 * BM);
-    CONV_STAMP(1)
     load_tiles(kbase * BK);
     if constexpr (EPI_BEHIND_TILES) request_epilogue_operands();
     if (tid < BN) {
@@ -567,9 +554,6 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             for (int kt = 0; kt < ktiles; kt += 2) {
                 store_tiles(0);
                 if (kt == 0) __syncthreads(); else tile_barrier();
-#ifdef CONV_PHASE_STAMPS
-                if (kt == 0 && sub == 0) { CONV_STAMP(2) }
-#endif
                 if (kt + 2 < ktiles) load_tiles((kbase + kt + 2) * BK, 0);
                 compute();
                 tile_barrier();
@@ -585,31 +569,11 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
         } else {
             // all k steps but the last: the next step's loads are in flight during the MFMAs
             for (int kt = 1; kt < ktiles; ++kt) {
-#ifdef CONV_PHASE_STAMPS
-                const unsigned long long c0 = clock64();
-#endif
                 store_tiles();
-#ifdef CONV_PHASE_STAMPS
-                __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0): the LDS writes have landed
-                const unsigned long long c1 = clock64();
-#endif
                 tile_barrier();
-#ifdef CONV_PHASE_STAMPS
-                const unsigned long long c2 = clock64();
-#endif
                 load_tiles((kbase + kt) * BK);
-#ifdef CONV_PHASE_STAMPS
-                if (kt == 1 && sub == 0) { CONV_STAMP(2) }
-#endif
                 compute();
-#ifdef CONV_PHASE_STAMPS
-                const unsigned long long c3 = clock64();
-#endif
                 tile_barrier();
-#ifdef CONV_PHASE_STAMPS
-                const unsigned long long c4 = clock64();
-                stamps[8] += c1 - c0; stamps[9] += c2 - c1; stamps[10] += c3 - c2; stamps[11] += c4 - c3; stamps[12] += 1;
-#endif
             }
             // last k step: the loads in flight are those of the next M tile's first step and of
             // the residual operand
@@ -631,9 +595,6 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             compute();
             __syncthreads();
         }
-#ifdef CONV_PHASE_STAMPS
-        if (sub == 0) { CONV_STAMP(3) }
-#endif
 
         // ---------------- epilogue + store of the finished M tile ----------------
         // Outputs that are not a row-major [M, N] matrix need (batch, y, x) of every row: decoded
@@ -670,12 +631,6 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
 #pragma unroll
                 for (int v = 0; v < 16; ++v) c[0][0][v] += As[((s - 1) * WGM * WGN + wm * WGN + wn) * 16 * 64 + v * 64 + lane];
         }
-#ifdef CONV_PHASE_STAMPS
-        if (sub == 0) {
-            if (first_full >= 0) { float sink = full[0][0][0]; asm volatile("" :: "v"(sink)); }
-            CONV_STAMP(4)
-        }
-#endif
         const uint32_t slots = (P.flags >> 20) & 31u;
         if (LEAN || slots) {
             // The usual chains (bias, batch norm, residual add, ReLU in that order, each optional) run
@@ -785,29 +740,13 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
                     }
             }
         }
-#ifdef CONV_PHASE_STAMPS
-        if (sub == 0) {
-            { float sink = 0; for (int v = 0; v < 16; ++v) sink += c[0][0][v]; asm volatile("" :: "v"(sink)); }
-            CONV_STAMP(5)
-        }
-#endif
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 sub_tile(m0, i, j, [&](int v, uint32_t vo, uint32_t so) { buffer_store_x1(c[i][j][v], o_rsrc, vo, so); });
         if (!c_contig) __syncthreads();          // Rs is rewritten for the next M tile
-#ifdef CONV_PHASE_STAMPS
-        if (sub == 0) { CONV_STAMP(6) }
-#endif
     }
-#ifdef CONV_PHASE_STAMPS
-    CONV_STAMP(7)
-    if (epi.p[CONV_MAX_EPI - 1] != nullptr && tid == 0) {
-        unsigned long long* d = (unsigned long long*)epi.p[CONV_MAX_EPI - 1] + (size_t)blockIdx.x * 16;
-        for (int q = 0; q < 16; ++q) d[q] = stamps[q];
-    }
-#endif
 }
 
 #define CONV_KERNEL(name, WGM, WGN, TM, TN, BK, AF, BF, LEAN, ...)                                          \

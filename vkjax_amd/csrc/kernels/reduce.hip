@@ -162,7 +162,8 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
         // float argmax / argmin across the lanes as the maximum of one 64-bit key per lane: the value mapped to an
         // unsigned number that grows with its rank (a NaN above everything), then the complement of the index, so
         // that of two equal values the earlier one wins. Five operations per butterfly step instead of a dozen.
-        const uint32_t bits = best_v, flipped = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+        // -0.0 ranks with +0.0 (the two compare equal, so the earlier of them wins)
+        const uint32_t bits = best_v == 0x80000000u ? 0u : best_v, flipped = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
         const float    x    = u2f(bits);
         const uint32_t rank = x != x ? 0xFFFFFFFFu : (MODE == 3 ? flipped : ~flipped);
         uint64_t key = best_i == 0xFFFFFFFFu ? 0ull : ((uint64_t)rank << 32 | (uint32_t)~best_i);   // no rank of a value is 0
@@ -533,7 +534,8 @@ __device__ __forceinline__ void softmax_rows_body(float* __restrict__ out, const
     }
     if (arg_out == nullptr) return;
     // across the lanes as in reduce_rows: the maximum of (rank of the value, complement of the index)
-    const uint32_t flipped = best_v ^ ((best_v >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+    const uint32_t zb      = best_v == 0x80000000u ? 0u : best_v;      // -0.0 ranks with +0.0
+    const uint32_t flipped = zb ^ ((zb >> 31) ? 0xFFFFFFFFu : 0x80000000u);
     const float    bv      = u2f(best_v);
     uint64_t key = best_i == 0xFFFFFFFFu ? 0ull : ((uint64_t)(bv != bv ? 0xFFFFFFFFu : flipped) << 32 | (uint32_t)~best_i);
 #pragma unroll

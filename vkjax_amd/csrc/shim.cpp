@@ -391,6 +391,31 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
     return 0;
 }
 
+int vkj::seq_eval_static(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, void* const* next_host_ptrs,
+                         int (*move)(void* dst, const void* src, size_t nbytes, hipStream_t stream)) {
+    if (s->profiling)
+        return fail(VKJ_ESTATE, "vkj_seq_eval_next_static: a sequence with timestamps creates events when evaluated; use vkj_seq_eval_next");
+    // the same condition under which issue_all would build the graph (a single launch is never captured)
+    if (s->want_graph && !s->graph_failed && s->launches.size() > 1 && !s->graph_exec)
+        return fail(VKJ_ESTATE, "vkj_seq_eval_next_static: the sequence's graph has not been built yet (that allocates); "
+                                "evaluate it once with vkj_seq_eval first");
+    size_t needed = 0;
+    if (next_host_ptrs)
+        for (auto& t : s->uploads)
+            if (t.nbytes && t.slot < nslots && next_host_ptrs[t.slot]) needed += (t.nbytes + 255) & ~(size_t)255;
+    if (needed > (size_t)VKJ_STATIC_LANDING_BYTES)
+        return fail(VKJ_EINVAL, "vkj_seq_eval_next_static: the following evaluation's arguments take %zu bytes, the static landing "
+                                "array holds %zu; use vkj_seq_eval_next", needed, (size_t)VKJ_STATIC_LANDING_BYTES);
+    // one array per GPU, shared by every context and thread of the process: claimed for the whole call
+    static std::atomic<bool> busy[64];
+    std::atomic<bool>& mine = busy[(unsigned)s->ctx->device % 64u];
+    if (mine.exchange(true, std::memory_order_acquire))
+        return fail(VKJ_ESTATE, "vkj_seq_eval_next_static: static landing array busy (another call on device %d is using it)", s->ctx->device);
+    const LandingRegion region{(char*)s->ctx->static_landing, (size_t)VKJ_STATIC_LANDING_BYTES, move};
+    const int r = seq_eval(s, host_ptrs, nslots, flags, next_host_ptrs, &region);
+    mine.store(false, std::memory_order_release);
+    return r;
+}
 
 extern "C" {
 

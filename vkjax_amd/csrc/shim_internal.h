@@ -148,6 +148,12 @@ struct LandingRegion {
 int seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, void* const* next_host_ptrs,
              const LandingRegion* region);
 
+// vkj_seq_eval_next_static without its handle lookup: refuses what would make the evaluation allocate
+// (time stamps, a graph that is not built yet), arguments beyond the array's size and a call that overlaps
+// another one on the same GPU, then evaluates with the context's static landing array and `move`.
+int seq_eval_static(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, void* const* next_host_ptrs,
+                    int (*move)(void* dst, const void* src, size_t nbytes, hipStream_t stream));
+
 // static_landing.hip: resolves the device address of the static landing array for the current device
 int static_landing_init(Ctx* c);
 

@@ -11,8 +11,10 @@
 // Every GPU the library runs on holds its own copy of the array (VKJ_STATIC_LANDING_BYTES) from
 // the moment the library is loaded there until the process ends. All calls on one GPU share it,
 // and it keeps what the last call left: a call only reads back the bytes it has just written,
-// so nothing needs clearing, but two calls that overlap in time on one GPU (two threads, two
-// contexts) race on it.
+// so nothing needs clearing. Two calls that overlap in time on one GPU (two threads, two
+// contexts) would race on it: the array is claimed for the duration of a call and the second
+// caller is refused with VKJ_ESTATE (seq_eval_static in shim.cpp, which also holds the other
+// refusals, so that the host-only test build exercises them).
 #include "shim_internal.h"
 
 #include <cstring>
@@ -71,18 +73,5 @@ extern "C" int vkj_seq_eval_next_static(vkj_handle sh, void* const* host_ptrs, i
                                         void* const* next_host_ptrs) {
     Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
     if (!s) return fail(VKJ_EINVAL, "vkj_seq_eval_next_static: bad handle");
-    if (s->profiling)
-        return fail(VKJ_ESTATE, "vkj_seq_eval_next_static: a sequence with timestamps creates events when evaluated; use vkj_seq_eval_next");
-    if (s->want_graph && !s->graph_exec && !s->graph_failed)
-        return fail(VKJ_ESTATE, "vkj_seq_eval_next_static: the sequence's graph has not been built yet (that allocates); "
-                                "evaluate it once with vkj_seq_eval first");
-    size_t needed = 0;
-    if (next_host_ptrs)
-        for (auto& t : s->uploads)
-            if (t.nbytes && t.slot < nslots && next_host_ptrs[t.slot]) needed += (t.nbytes + 255) & ~(size_t)255;
-    if (needed > (size_t)VKJ_STATIC_LANDING_BYTES)
-        return fail(VKJ_EINVAL, "vkj_seq_eval_next_static: the following evaluation's arguments take %zu bytes, the static landing "
-                                "array holds %zu; use vkj_seq_eval_next", needed, (size_t)VKJ_STATIC_LANDING_BYTES);
-    const LandingRegion region{(char*)s->ctx->static_landing, (size_t)VKJ_STATIC_LANDING_BYTES, move_on};
-    return seq_eval(s, host_ptrs, nslots, flags, next_host_ptrs, &region);
+    return seq_eval_static(s, host_ptrs, nslots, flags, next_host_ptrs, move_on);
 }

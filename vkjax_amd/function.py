@@ -12,7 +12,6 @@ import typing as tp
 
 import numpy as np
 
-from . import hip
 from . import minijax
 from .jaxpr_interpreter import JaxprInterpreter
 from .minijax import core, tree_util
@@ -181,8 +180,7 @@ class Function:
                 overlap   = following is not None and following[0] is interpreter
                 next_host = interpreter._select_uploads(following[2]) if overlap else None
                 fresh     = interpreter._fresh_outputs(host)
-                interpreter.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT, next_host_arrays=next_host)
-                interpreter._evaluations += 1
+                interpreter.evaluate(host, next_host)
                 stamp, in_place = interpreter._evaluations, overlap
                 yield self._restore_shapes(interpreter._output_values(fresh), output_shapes)
                 current = following
@@ -217,4 +215,14 @@ class Function:
 
 
 def wrap(function: tp.Callable, *args, **kwargs) -> Function:
+    '''`vkjax.wrap` (reference: vkjax/function.py:46-47): `wrap(f, static_argnums=(), profiling=False)(*args)` traces
+    `f` for the arguments' signature and runs it on the device.
+
+    Arguments are copied to the device on every call, as the reference does, with two exceptions that save the
+    copy of weights and tables: leaves that cannot change while the caller holds them (numpy arrays with
+    `flags.writeable == False`, jax arrays) are uploaded once and again only when another object is passed in their
+    place; and `resident_argnums=(i, ...)` declares the same for every leaf of those arguments, writeable or not -
+    an in-place change of such a writeable array is noticed only if it moves the array or touches its first or last
+    64 bytes, so pass a new array for new values. Further keyword arguments: `frontend` ('jax', 'minijax', default:
+    jax where importable), `fuse`, `reuse_buffers`, `graph`.'''
     return Function(function, *args, **kwargs)

@@ -25,9 +25,15 @@ class JaxprInterpreter:
                  reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False, graph: bool = False,
                  resident_argnums: tp.Tuple[int, ...] = ()):
         self.jaxpr          = jaxpr
-        #Arguments named here (weights, tables) stay in HBM between calls: a leaf is uploaded when the
-        #object passed for it is not the one uploaded last. Changing such an array in place is not
-        #noticed (the reference copies every argument on every call, vkjax/kompute_jaxpr_interpreter.py:72-75).
+        #Which argument leaves stay in HBM between calls instead of being copied on every call, as the reference
+        #does (vkjax/kompute_jaxpr_interpreter.py:72-75):
+        # * leaves that cannot change under the caller's feet - numpy arrays that are not writeable (nor views of
+        #   writeable ones) and jax arrays - without being asked: such a leaf is uploaded when the object passed for
+        #   it is not the one uploaded last;
+        # * every leaf of the arguments named in resident_argnums (weights, tables), writeable or not. A writeable
+        #   one that is changed in place is noticed only when its address, shape, strides or its first or last
+        #   64 bytes change; pass a new array (or a read-only one) for a new value.
+        #All other leaves are copied on every call.
         self.resident_argnums = tuple(resident_argnums)
         self._resident_leaves = {}
         #graph=True replays the launches as one captured HIP graph (never with profiling)
@@ -117,7 +123,9 @@ class JaxprInterpreter:
                 continue
             these = [x] if type(x) is np.ndarray else tree_util.tree_leaves([x])
             leaves   += these
-            resident += [i in self.resident_argnums] * len(these)
+            named     = i in self.resident_argnums
+            resident += [RESIDENT_CHECKED if named and _may_change_in_place(leaf) else RESIDENT if named or _is_immutable(leaf) else 0
+                         for leaf in these]
         if len(self.input_buffers) != len(leaves):
             raise TypeError(f'Expected {len(self.input_buffers)} input arguments, received {len(leaves)}')
         return (leaves, resident) if with_residency else leaves
@@ -148,9 +156,11 @@ class JaxprInterpreter:
         host = [None] * self.sequence.n_slots
         for k, slot, x, words, is_resident in converted:
             if is_resident:
-                if self._resident_leaves.get(k) is x:
+                held = self._resident_leaves.get(k)
+                mark = _fingerprint(x, words) if is_resident == RESIDENT_CHECKED else None
+                if held is not None and held[0] is x and held[1] == mark:
                     continue                                    #already in HBM
-                self._resident_leaves[k] = x
+                self._resident_leaves[k] = (x, mark)
             host[slot] = words
         return host
 
@@ -169,12 +179,31 @@ class JaxprInterpreter:
         return tuple(None if b is None else view_or_convert_from_32bit(arr, b.dtype).reshape(b.shape)
                      for b, arr in zip(self.output_buffers, fresh))
 
+    def evaluate(self, host, next_host_arrays=None):
+        '''One evaluation of the recorded sequence: `host` holds the arrays to copy in and the fresh result arrays,
+        slots left None keep what their buffers hold. Launches that share zero-initialised scratch memory (the
+        counters of the sorted scatter-add) leave it zero again only when they run to the end: after an evaluation
+        that failed, the zeros are written again before the error is passed on, so that a later evaluation does not
+        start from whatever the failed one left.'''
+        try:
+            self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT, next_host_arrays=next_host_arrays)
+        except BaseException:
+            self._resident_leaves.clear()                       #nothing is known about what reached HBM
+            for key, b in self.bufferpool.buffers.items():
+                if isinstance(key, tuple) and key[:1] == ('zeroed',):
+                    try:
+                        b.tensor.upload(np.zeros(b.size, np.uint32))
+                    except Exception:                            #a device that is gone reports the first error
+                        pass
+            raise
+        finally:
+            self._evaluations += 1
+
     def run(self, *X, return_all=False):
         '''Executes a previously recorded sequence with actual data'''
         host  = self._host_inputs(X)
         fresh = self._fresh_outputs(host)
-        self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT if self.resident_argnums else 0)
-        self._evaluations += 1
+        self.evaluate(host)
         output_values = self._output_values(fresh)
         if not return_all:
             return output_values
@@ -200,8 +229,7 @@ class JaxprInterpreter:
             following = next(iterator, end)
             next_host = self._host_inputs(tuple(following)) if following is not end else None
             fresh     = self._fresh_outputs(host)
-            self.sequence.eval(host, flags=hip.EVAL_NULL_IS_RESIDENT, next_host_arrays=next_host)
-            self._evaluations += 1
+            self.evaluate(host, next_host)
             stamp, in_place = self._evaluations, following is not end
             yield self._output_values(fresh)
             if following is end:
@@ -228,6 +256,34 @@ class JaxprInterpreter:
         deltas     = np.diff(timestamps)
         labels     = ['data2device'] + [op.equation for op in self.all_ops] + ['data2host']
         return list(zip(labels, deltas))
+
+
+#kinds of resident leaves: identified by the object alone, or by the object and a fingerprint of its memory
+RESIDENT, RESIDENT_CHECKED = 1, 2
+
+
+def _is_immutable(leaf) -> bool:
+    '''True for an argument leaf whose values cannot change while the caller holds it: a numpy array that is not
+    writeable and does not look into a writeable one (or into anything but another array or a bytes object), or
+    an array of jax.'''
+    if type(leaf) is np.ndarray:
+        while type(leaf) is np.ndarray:
+            if leaf.flags.writeable:
+                return False
+            leaf = leaf.base
+        return leaf is None or type(leaf) is bytes
+    module = type(leaf).__module__
+    return module.startswith('jaxlib') or module.startswith('jax.')
+
+
+def _may_change_in_place(leaf) -> bool:
+    return isinstance(leaf, np.ndarray) and not _is_immutable(leaf)
+
+
+def _fingerprint(x: np.ndarray, words: np.ndarray):
+    '''What a cheap look at a writeable array can tell about a change in place: where it lives, its layout and its
+    first and last 64 bytes.'''
+    return (x.__array_interface__['data'][0], x.shape, x.strides, words[:16].tobytes(), words[-16:].tobytes())
 
 
 def _device_words_of_argument(x, aval) -> np.ndarray:

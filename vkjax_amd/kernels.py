@@ -6,6 +6,7 @@ time and take shapes and strides as kernel arguments. Each function below lays o
 block of one kernel (a struct of 32-bit fields that follows the pointer arguments, mirroring the
 `struct ...Params` in vkjax_amd/csrc/kernels/*.hip) and picks grid, block and kernel variant.
 '''
+import contextlib
 import os
 import re
 import typing as tp
@@ -26,6 +27,50 @@ EW = _read_opcodes()
 EW_MAX_STEPS = 8
 CONV_MAX_EPI = 6
 BLOCK = 256
+
+
+class _Choices:
+    '''Which kernel variant a lowering picks where several would do. Every field has the value the heuristics work
+    with; `overrides(...)` pins some of them for the duration of a `with` block, which is how tests reach every
+    variant whatever the heuristics would choose, and how measurements compare variants.'''
+    DEFAULTS = dict(
+        ew_affine=None,                  #the straight-line affine kernel: None = where it pays, True = wherever it applies, False = never
+        conv_tile=None,                  #name of the tile shape (CONV_TILES) instead of the estimate's choice
+        conv_bk=None,                    #k step
+        conv_chunk=None,                 #consecutive M tiles a lean block walks
+        conv_blocks_per_cu=5,            #blocks of the lean 64 x 64 kernels a CU holds at once (94 registers); 0 = no evenly split grids
+        conv_even_split_min_tiles=4.5,   #tiles per block from which an evenly split grid is used
+        conv_general=False,              #never pick the lean kernel variant
+        conv_b_general=False,            #element-wise loads of the kernel operand also where 16-byte loads would do
+        conv_ksplit=None,                #the four-waves-per-tile kernel: always (where it applies) / never
+        conv_dense_rows=None,            #the kernel for at most 16 output features: None = where it applies, False = never
+        conv_mix=None,                   #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
+        conv_stem=None,                  #the patch kernel for few input features: False = never; None / True: where it applies
+        conv_k_splits=None,              #slices a contraction is cut into where that applies (None: by the heuristic, 1: never)
+        scatter_sort_threshold=1 << 18,  #update elements from which a row scatter-add sorts its updates instead of using atomics
+        reuse_equal_equations=True,      #an equation that repeats an earlier one is bound to that one's buffer
+    )
+
+    def __init__(self):
+        self.__dict__.update(self.DEFAULTS)
+
+
+CHOICES = _Choices()
+
+
+@contextlib.contextmanager
+def overrides(**pinned):
+    '''`with overrides(conv_tile='64x64', conv_bk=32): ...` - programs built inside the block use the given
+    choices (fields of `_Choices.DEFAULTS`); the previous values return when the block is left.'''
+    unknown = set(pinned) - set(_Choices.DEFAULTS)
+    if unknown:
+        raise TypeError(f'overrides: unknown choice(s) {sorted(unknown)}; known: {sorted(_Choices.DEFAULTS)}')
+    saved = {name: getattr(CHOICES, name) for name in pinned}
+    CHOICES.__dict__.update(pinned)
+    try:
+        yield CHOICES
+    finally:
+        CHOICES.__dict__.update(saved)
 
 
 class Launch(tp.NamedTuple):
@@ -205,8 +250,6 @@ def lower_ew_chain(chain: EwChain) -> Launch:
                   [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
 
 
-#tests: None = where it applies, False = never
-FORCE_EW_AFFINE: tp.Optional[bool] = None
 EW_AFFINE_BIG_ELEMENTS = 1 << 22
 
 
@@ -218,8 +261,8 @@ def _as_affine_chain(chain: EwChain, n: int, dims, strides) -> tp.Optional[Launc
     51 M elements 4.5 TB/s, here 5.7). Shorter chains keep the general kernel, which is as fast for them and whose
     small launches are batched with their neighbours.'''
     operands = chain.operands()
-    if (FORCE_EW_AFFINE is False or not chain.steps or any(o is None for o in operands) or n % 4 or dims[-1] % 4 or n * 4 >= 2**32 - 2**16
-            or len(dims) > 2 or (FORCE_EW_AFFINE is None and len(operands) <= 4)
+    if (CHOICES.ew_affine is False or not chain.steps or any(o is None for o in operands) or n % 4 or dims[-1] % 4 or n * 4 >= 2**32 - 2**16
+            or len(dims) > 2 or (CHOICES.ew_affine is None and len(operands) <= 4)
             or any(np.dtype(b.dtype) != np.float32 for b in [chain.out] + [o.buffer for o in operands])):
         return None
     dense = row_major_strides(dims)
@@ -499,24 +542,13 @@ CONV_TILES = (('128x128', 128, 128, 256, 2, 0.92), ('128x64', 128, 64, 256, 2, 0
 #k steps each tile shape is built with
 CONV_TILE_BK = {'128x128': (32,), '128x64': (32,), '64x64': (32, 64), '32x32': (32, 64)}
 
-#tests set these to exercise every kernel variant irrespective of the heuristics
-FORCE_CONV_TILE: tp.Optional[str] = None
-FORCE_CONV_BK:   tp.Optional[int] = None
-FORCE_CONV_CHUNK: tp.Optional[int] = None
-CONV_BLOCKS_PER_CU = 5             #blocks of the lean 64 x 64 kernels a CU holds at once (94 registers); 0 = no evenly split grids
-CONV_EVEN_SPLIT_MIN_TILES = 4.5    #tiles per block from which an evenly split grid is used
-FORCE_CONV_GENERAL = False          #never pick the lean kernel variant
-FORCE_CONV_B_GENERAL = False        #element-wise loads of the kernel operand also where 16-byte loads would do
-FORCE_CONV_KSPLIT: tp.Optional[bool] = None    #the four-waves-per-tile kernel: always (where it applies) / never
-FORCE_CONV_DENSE_ROWS = None        #the kernel for at most 16 output features: None = where it applies, False = never
-FORCE_CONV_MIX = None               #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
 
 
 def choose_conv_tile(M: int, N: int, compute_units: int = 256):
     '''Smallest estimated time: tiles are dealt out over the CUs, a tile costs BM*BN / efficiency,
     and a block of one wave can drive only one of a CU's four MFMA units.'''
-    if FORCE_CONV_TILE is not None:
-        return next(t[:4] for t in CONV_TILES if t[0] == FORCE_CONV_TILE)
+    if CHOICES.conv_tile is not None:
+        return next(t[:4] for t in CONV_TILES if t[0] == CHOICES.conv_tile)
     best, best_time = None, None
     for tag, bm, bn, nt, occupancy, eff in CONV_TILES:
         tiles   = _cdiv(M, bm) * _cdiv(N, bn)
@@ -553,12 +585,12 @@ def choose_conv_chunk(tiles_m: int, tiles_n: int, compute_units: int = 256) -> i
 
 def choose_conv_m_blocks(tiles_m: int, tiles_n: int, compute_units: int = 256) -> int:
     '''0, or the number of blocks that share the M tiles of every N tile evenly: a grid of exactly as many blocks as
-    the GPU holds at once (CONV_BLOCKS_PER_CU per CU), each working through its tiles as one sequence of k steps, so
+    the GPU holds at once (CHOICES.conv_blocks_per_cu per CU), each working through its tiles as one sequence of k steps, so
     that only its first tile pays for the argument fetch and the first loads. Worth it from about five tiles per
     block: with fewer, one tile more or less per block leaves CUs idle at the end (measured on ResNet-50 layers at
     batch 64: -4 to -5 % at 4.9 tiles per block, +1 to +8 % at 2.45).'''
-    resident = int(CONV_BLOCKS_PER_CU * compute_units)
-    if resident < 1 or tiles_m * tiles_n < CONV_EVEN_SPLIT_MIN_TILES * resident:
+    resident = int(CHOICES.conv_blocks_per_cu * compute_units)
+    if resident < 1 or tiles_m * tiles_n < CHOICES.conv_even_split_min_tiles * resident:
         return 0
     return min(tiles_m, max(1, resident // tiles_n))
 
@@ -568,8 +600,8 @@ def choose_conv_bk(tag: str, g: 'ConvGeometry') -> int:
     for the 64x64 tile on long contractions, and only when whole k tiles stay inside one kernel
     tap (Cin % 64 == 0), which keeps the tap position in scalar registers.'''
     options = CONV_TILE_BK[tag]
-    if FORCE_CONV_BK is not None and FORCE_CONV_BK in options:
-        return FORCE_CONV_BK
+    if CHOICES.conv_bk is not None and CHOICES.conv_bk in options:
+        return CHOICES.conv_bk
     if tag == '64x64' and g.Cin % 64 == 0 and g.K >= 2048:
         return 64
     return 32
@@ -618,13 +650,12 @@ def _magic_division(d: int) -> tp.Tuple[int, int]:
 
 
 STEM_PATCH_FLOATS, STEM_PATCH_ROWS, STEM_VECTORS_PER_THREAD = 6272, 9, 6      #conv_gemm_stem_7x22's LDS patch
-FORCE_CONV_STEM: tp.Optional[bool] = None       #the patch kernel for few input features: never (False); None / True: where it applies
 
 
 def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_units, lhs_offset, rhs_offset, out_offset) -> tp.Optional[Launch]:
     '''conv_gemm_stem_7x22 where it applies: dense images with so few features that KW * Cin is 21 or 22 (7 x 7 x 3),
     seven kernel rows, a template epilogue; see the conditions listed at the kernel.'''
-    if FORCE_CONV_STEM is False or FORCE_CONV_TILE is not None or FORCE_CONV_GENERAL or lhs_offset or rhs_offset or out_offset:
+    if CHOICES.conv_stem is False or CHOICES.conv_tile is not None or CHOICES.conv_general or lhs_offset or rhs_offset or out_offset:
         return None
     M, N, K = g.M, g.N, g.K
     RL, WC = g.KW * g.Cin, g.W * g.Cin
@@ -664,8 +695,8 @@ DENSE_ROWS_MAX_N = 16
 def _dense_rows_shape(lhs: Buffer, g: 'ConvGeometry') -> bool:
     '''The operands of a product suit dense_rows_n16. `g` as the caller gave it: a matrix product, not a 1 x 1
     convolution over a feature map (those keep the kernels whose epilogue takes a residual operand).'''
-    if (FORCE_CONV_DENSE_ROWS is False or FORCE_CONV_TILE is not None or FORCE_CONV_BK is not None or FORCE_CONV_GENERAL
-            or FORCE_CONV_KSPLIT is not None):
+    if (CHOICES.conv_dense_rows is False or CHOICES.conv_tile is not None or CHOICES.conv_bk is not None or CHOICES.conv_general
+            or CHOICES.conv_ksplit is not None):
         return False
     M, N, K = g.M, g.N, g.K
     flat = (g.batch == 1 and g.Wo == 1 and g.KH == g.KW == 1 and g.SH == 1 and g.PH == g.PW == 0 and g.LH == 1 and g.H == g.Ho
@@ -740,7 +771,7 @@ def _conv_fast_paths(lhs: Buffer, rhs: Buffer, g: ConvGeometry, lhs_offset: int 
     #16-byte loads of the kernel operand need a dense [ky, kx, in, out] array, not an output width that is a multiple of 4:
     #a buffer load of four words only has to start at a word (verified on gfx950 with integer-exact products of odd
     #widths); the words a vector reads beyond its row belong to columns >= N, which are never stored
-    b_fast = (g.ws[3] == 1 and rhs_offset % 4 == 0 and not FORCE_CONV_B_GENERAL
+    b_fast = (g.ws[3] == 1 and rhs_offset % 4 == 0 and not CHOICES.conv_b_general
               and g.ws[2] == N and g.ws[1] == g.Cin * N and g.ws[0] == g.KW * g.Cin * N)
     c_contig = g.os == (g.Ho * g.Wo * N, g.Wo * N, N, 1)
     return needs_masks, x_bias, a_fast, b_fast, c_contig
@@ -749,13 +780,11 @@ def _conv_fast_paths(lhs: Buffer, rhs: Buffer, g: ConvGeometry, lhs_offset: int 
 def _four_waves_per_tile(g: ConvGeometry, a_fast: bool, c_contig: bool, compute_units: int) -> bool:
     '''A product with so few 32 x 32 tiles that one wave per tile leaves most MFMA units idle: four waves per tile,
     each taking a quarter of every (128-long) k step.'''
-    want = (FORCE_CONV_KSPLIT if FORCE_CONV_KSPLIT is not None else
-            (_cdiv(g.M, 32) * _cdiv(g.N, 32) <= 2 * compute_units and g.K >= 256 and FORCE_CONV_TILE is None and FORCE_CONV_BK is None))
-    return bool(want) and a_fast and c_contig and (g.Cin % 64 == 0 or g.KH * g.KW == 1) and not FORCE_CONV_GENERAL
+    want = (CHOICES.conv_ksplit if CHOICES.conv_ksplit is not None else
+            (_cdiv(g.M, 32) * _cdiv(g.N, 32) <= 2 * compute_units and g.K >= 256 and CHOICES.conv_tile is None and CHOICES.conv_bk is None))
+    return bool(want) and a_fast and c_contig and (g.Cin % 64 == 0 or g.KH * g.KW == 1) and not CHOICES.conv_general
 
 
-#tests: the number of slices a contraction is cut into where that applies (None: by the heuristic, 1: never)
-FORCE_CONV_K_SPLITS: tp.Optional[int] = None
 
 
 def conv_k_splits(lhs: Buffer, rhs: Buffer, g: ConvGeometry, compute_units: int = 256) -> int:
@@ -773,8 +802,8 @@ def conv_k_splits(lhs: Buffer, rhs: Buffer, g: ConvGeometry, compute_units: int 
     if not _four_waves_per_tile(g, a_fast, c_contig, compute_units) or (g.Cin % 128 != 0 and g.KH * g.KW != 1):
         return 1
     tiles, ksteps = _cdiv(g.M, 32) * _cdiv(g.N, 32), _cdiv(g.K, 128)
-    if FORCE_CONV_K_SPLITS is not None:
-        want = FORCE_CONV_K_SPLITS
+    if CHOICES.conv_k_splits is not None:
+        want = CHOICES.conv_k_splits
     else:
         want = min(4, compute_units // tiles, ksteps // 4)
     if want <= 1 or ksteps < 2:
@@ -820,7 +849,7 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     slots = _epilogue_template_slots(epilogue)
     #the lean kernel variant covers the common case only (see the kernel source)
     lean = (a_fast and b_fast and c_contig and (g.Cin % bk == 0 or g.KH * g.KW == 1)
-            and (not epilogue or slots != 0) and not FORCE_CONV_GENERAL)
+            and (not epilogue or slots != 0) and not CHOICES.conv_general)
     #the output row number is the input row number (a matrix product, or a one-column image walked without stride,
     #padding or taps outside the input): the kernel then skips the row decode and the validity masks
     flat_rows = g.batch == 1 and g.Wo == 1 and g.SH == 1 and g.PH == 0 and g.PW == 0 and not needs_masks
@@ -840,9 +869,9 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
         if (not ksplit or short_step or epilogue or taps or out_offset or out.size != g.k_splits * M * N
                 or _cdiv(_cdiv(K, 128), k_split_steps) != g.k_splits):
             raise ValueError('a sliced contraction needs the four-waves-per-tile kernel, no epilogue and one [M, N] matrix per non-empty slice')
-    chunk = (FORCE_CONV_CHUNK or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean and not ksplit else 1
+    chunk = (CHOICES.conv_chunk or choose_conv_chunk(tiles_m, tiles_n, compute_units)) if lean and not ksplit else 1
     m_blocks = 0
-    if lean and not ksplit and FORCE_CONV_CHUNK is None:
+    if lean and not ksplit and CHOICES.conv_chunk is None:
         m_blocks = choose_conv_m_blocks(tiles_m, tiles_n, compute_units)
         if m_blocks:
             chunk = 2                          #(a value other than 1 keeps the mixed tiling out; the kernel ignores it)
@@ -850,9 +879,9 @@ def conv_gemm(out: Buffer, lhs: Buffer, rhs: Buffer, g: ConvGeometry, epilogue: 
     #rows behind them are computed as 32 x 32 tiles with four waves per tile (a quarter of the work each)
     split_tiles_m = 0
     mixable = (lean and not ksplit and tag == '64x64' and chunk == 1 and b_fast and (g.Cin % 64 == 0 or g.KH * g.KW == 1) and K >= 256)
-    if mixable and FORCE_CONV_MIX is not None and FORCE_CONV_MIX is not False:
-        split_tiles_m = int(FORCE_CONV_MIX)                      #tests: whatever the other FORCE_ settings are
-    elif mixable and FORCE_CONV_MIX is None and FORCE_CONV_TILE is None and FORCE_CONV_BK is None and FORCE_CONV_CHUNK is None:
+    if mixable and CHOICES.conv_mix is not None and CHOICES.conv_mix is not False:
+        split_tiles_m = int(CHOICES.conv_mix)                      #tests: whatever the other pinned choices are
+    elif mixable and CHOICES.conv_mix is None and CHOICES.conv_tile is None and CHOICES.conv_bk is None and CHOICES.conv_chunk is None:
         split_tiles_m = choose_conv_split(tiles_m, tiles_n, compute_units)
     if split_tiles_m >= tiles_m:
         split_tiles_m = 0

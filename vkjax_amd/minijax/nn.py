@@ -26,6 +26,11 @@ def softmax(x, axis=-1):
     return unnormalized / mnp.sum(unnormalized, axis, keepdims=True)
 
 
+def log_softmax(x, axis=-1):
+    shifted = x - lax.stop_gradient(mnp.max(x, axis, keepdims=True))
+    return shifted - mnp.log(mnp.sum(mnp.exp(shifted), axis, keepdims=True))
+
+
 def batch_norm_inference(x, scale, shift, mean, var, eps=1e-5):
     '''Inference-mode batch norm over the trailing (channel) axis, written the way
     flax/haiku modules of the period lower it: the per-channel factor first, then three

@@ -95,10 +95,6 @@ def analyze_jaxpr(bufferpool: BufferPool, jaxpr) -> tp.List[Op]:
     return all_ops
 
 
-#Set to False to evaluate every equation, also one that repeats an earlier one.
-REUSE_EQUAL_EQUATIONS = True
-
-
 def _reuse_equal_equation(bufferpool: BufferPool, eq) -> bool:
     '''An element-wise or shape equation with the primitive, parameters and operands of an earlier one computes the same
     array: its result variable is bound to that equation's buffer and nothing is launched. (Tracing `x[i]` and
@@ -106,12 +102,12 @@ def _reuse_equal_equation(bufferpool: BufferPool, eq) -> bool:
     their own storage and equation.'''
     from .buffers import hashable
     name = eq.primitive.name
-    if not REUSE_EQUAL_EQUATIONS or len(eq.outvars) != 1 or not (name in _BINARY or name in _UNARY or name in _REUSABLE_OTHERS):
+    if not K.CHOICES.reuse_equal_equations or len(eq.outvars) != 1 or not (name in _BINARY or name in _UNARY or name in _REUSABLE_OTHERS):
         return False
     outvar = eq.outvars[0]
     if hashable(outvar) in bufferpool.buffers:
         return False                                       #a result of the program
-    operands = []
+    operands, cells = [], []
     for v in eq.invars:
         if core.is_literal(v):
             value = np.asarray(v.val)
@@ -121,14 +117,16 @@ def _reuse_equal_equation(bufferpool: BufferPool, eq) -> bool:
             if b is None:
                 return False
             operands.append((id(b._placeholder), str(b.dtype), b.shape))
+            cells.append(b._placeholder)
     params = _params_without_jax_bookkeeping(eq.params)
     key = (name, repr(sorted(params.items())), tuple(operands), str(outvar.aval.dtype), tuple(outvar.aval.shape))
     seen = bufferpool.__dict__.setdefault('_equal_equations', {})
+    #the entry keeps the operands' storage cells alive, so that the identities in the key cannot pass to other cells
     earlier = seen.get(key)
-    if earlier is None:
-        seen[key] = outvar
+    if earlier is None or len(earlier[1]) != len(cells) or any(a is not b for a, b in zip(earlier[1], cells)):
+        seen[key] = (outvar, cells)
         return False
-    bufferpool.set_buffer(outvar, bufferpool.get_buffer(earlier))
+    bufferpool.set_buffer(outvar, bufferpool.get_buffer(earlier[0]))
     return True
 
 
@@ -804,8 +802,8 @@ reduce_max = reduce_min = reduce_sum = reduce_prod = argmin = argmax = reduce_or
 def _reduce_window(bufferpool, equation, op_name):
     params = equation.params
     n = len(equation.outvars[0].aval.shape)
-    assert n <= 4, NotImplemented
-    assert tuple(params.get('base_dilation') or (1,) * n) == (1,) * n, NotImplemented
+    if n > 4 or tuple(params.get('base_dilation') or (1,) * n) != (1,) * n:
+        raise NotImplementedError(equation)
     inbuf  = bufferpool.get_buffer(equation.invars[0])
     outbuf = bufferpool.get_buffer(equation.outvars[0], increment_op_counter=True)
     if _kind(inbuf.dtype) == _B:
@@ -950,7 +948,7 @@ def scatter_add(bufferpool, equation):
         row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
         n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
         n_rows  = operand.shape[0]
-        if n_idx * row_len >= SCATTER_SORT_THRESHOLD and n_idx < 2**31 - 1 and n_rows < 2**31 - 1:
+        if n_idx * row_len >= K.CHOICES.scatter_sort_threshold and n_idx < 2**31 - 1 and n_rows < 2**31 - 1:
             #large: bucket the updates by row and sum each bucket (no atomics on the data, no copy of the operand)
             bufferpool.op_counter = counter_before
             count = bufferpool.zeroed_scratch(n_rows)          #every evaluation leaves it zero again
@@ -972,10 +970,6 @@ def scatter_add(bufferpool, equation):
         ops = [copy, Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, n_rows, clip=clip))]
         return ops
     return [copy, Op(equation, launch=K.scatter_add_general(outbuf, indices, updates, uwd, iwd, sd2od, clip=clip))]
-
-
-#scatter-add of rows: from this many update elements on, the sorted (atomic-free) kernels are used
-SCATTER_SORT_THRESHOLD = 1 << 18
 
 
 def _uniform_constant(b):
