@@ -335,6 +335,15 @@ def test_point_and_column_scatter_add_forms():
             #the scatter behind an element-wise step and in front of one, so that the fusion passes see it
             check_against_oracle(lambda x, i, u: scatter_fn0(x * 2.0, i, u + 1.0) - 3.0, [ints(rows, cols), points, ints(n, 1)], exact=True, fuse=fuse)
             check_against_oracle(lambda x, i, u: scatter_add_fn1(x * 2.0, i, u + 1.0) - 3.0, [ints(rows, cols), column, ints(rows)], exact=True, fuse=fuse)
+            #the scattered array read by what follows (the result of an in-place accumulation is not its copy launch's)
+            zeros = jnp.zeros((rows, cols), np.float32)
+            check_against_oracle(lambda x, i, u: (scatter_fn0(x, i, u) * 2.0, -scatter_fn0(zeros, i, u), scatter_fn0(x, i, u).T + 1.0),
+                                 [ints(rows, cols), points, ints(n, 1)], exact=True, fuse=fuse)
+            check_against_oracle(lambda x, i, u: (scatter_add_fn1(x, i, u) * 2.0, jnp.sum(-scatter_add_fn1(zeros, i, u), axis=1)),
+                                 [ints(rows, cols), column, ints(rows)], exact=True, fuse=fuse)
+            rows_idx = rng.randint(-rows, rows, size=(n,)).astype(np.int32)
+            check_against_oracle(lambda x, i, u: (jnp.index_add(x, i, u) * 2.0, -jnp.index_add(zeros, i, u)),
+                                 [ints(rows, cols), rows_idx, ints(n, cols)], exact=True, fuse=fuse)
             #the gradient of take_along_axis with a cotangent of small integers instead of 1 / n
             g = lambda x, i: mj.grad(lambda x, i: (take_along_axis0(x, i) * 3.0).ravel().sum())(x, i)
             y, _, fn = check_against_oracle(g, [ints(rows, cols), along], exact=True, fuse=fuse)

@@ -204,9 +204,11 @@ def test_binding_repeated_equations_to_one_buffer_changes_no_bit():
         b = x.reshape(-1)[::2] + x.reshape(-1)[::2]
         c = mj.numpy.exp(x.T) - mj.numpy.exp(x.T) * y.T
         return a + y, b, c, (x + 1.0).sum(axis=0)
+    #(integer-valued updates: the atomic additions of a small scatter-add come in any order)
     idx = rng.integers(-40, 40, size=(64, 3)).astype(np.int32)
-    programs = [(W.gather_scatter, [rng.random((40, 24), dtype=np.float32), idx, rng.random((64, 3, 24), dtype=np.float32)]),
-                (W.gather_scatter, W.gather_scatter_inputs(rows=512, cols=256, n0=256, n1=8)),
+    table, idx2, updates = W.gather_scatter_inputs(rows=512, cols=256, n0=256, n1=8)
+    programs = [(W.gather_scatter, [rng.random((40, 24), dtype=np.float32), idx, rng.integers(-9, 10, size=(64, 3, 24)).astype(np.float32)]),
+                (W.gather_scatter, [table, idx2, np.round(updates * 16)]),
                 (views_and_chains, [rng.random((18, 32), dtype=np.float32), rng.random((18, 32), dtype=np.float32)])]
     for f, args in programs:
         for fuse in (True, False):
@@ -617,7 +619,7 @@ def test_read_only_leaves_stay_in_hbm_without_being_asked():
     g = vkjax_amd.wrap(W.mlp, frontend='minijax')
     rw = tree_util.tree_map(np.copy, params)
     for k in range(3):
-        tree_util.tree_leaves(rw)[0][5, 7] += np.float32(1.0)
+        tree_util.tree_leaves(rw)[0].reshape(-1)[5] += np.float32(1.0)
         y, uploads = counted(g, rw, x)
         assert uploads == n + 1, (k, uploads)
         assert_tree_close(y, plain(tree_util.tree_map(np.copy, rw), x), exact=True, what=f'writeable weights, call {k}')

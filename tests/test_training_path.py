@@ -338,7 +338,7 @@ def test_every_variable_of_a_training_step(name, make_inputs, atol):
     outs, envpred = interp.run(*args, return_all=True)
     outs_true, envtrue = eval_closed_jaxpr(closed, *tree_util.tree_leaves(args), return_env=True)
     assert len(envtrue) >= len(closed.jaxpr.eqns) and len(outs) == len(outs_true)
-    checked, worst = 0, (0.0, None)
+    checked, worst = 0, (0.0, '')
     for var, vtrue in envtrue.items():
         if np.size(vtrue) == 0:
             continue
@@ -349,7 +349,7 @@ def test_every_variable_of_a_training_step(name, make_inputs, atol):
             assert np.array_equal(vpred, vtrue), var
         else:
             err = float(np.max(np.abs(vpred.astype(np.float64) - vtrue) / (atol + 1e-5 * np.abs(vtrue))))
-            worst = max(worst, (err, str(var)))
+            worst = (err, str(var)) if err > worst[0] else worst
             assert err <= 1.0, f'{var} {np.shape(vtrue)}: |err| / (atol + rtol |y|) = {err:.3g}'
         checked += 1
     print(f'{name}: {checked} variables, worst |err| / (atol + rtol |y|) = {worst[0]:.3g} at {worst[1]}', flush=True)

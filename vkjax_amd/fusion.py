@@ -276,6 +276,12 @@ def fuse_ops(all_ops, bufferpool, outvars):
         out = _out(new)
         if out is not None:
             producer[id(out._placeholder)] = len(result) - 1
+        else:
+            #a launch that is neither a chain nor a convolution may change its result buffer in place (scatter-add
+            #accumulates into a copy of its operand): whoever produced that buffer before no longer describes what
+            #it holds, so nothing behind this launch may be joined to that producer or read through it
+            for b in _writes(new):
+                producer.pop(id(b._placeholder), None)
     ops = fuse_random_streams([op for op in result if op is not None], bufferpool, outvars)
     ops = fuse_stream_chains(ops, bufferpool, outvars)
     ops = fuse_softmax(ops, bufferpool, outvars)
