@@ -47,6 +47,11 @@ BATCHED = ('resnet50', 'mlp', 'conv_block', 'mlp_train', 'convnet_train', 'resne
 OTHER_CONFIGS = ('affine', 'mlp', 'conv_block', 'rng_uniform', 'gather_scatter')
 
 
+#kernel families whose launches compute their results from their operands alone, so that replaying one changes nothing
+REPEATABLE = ('conv_gemm', 'dense_rows', 'softmax_rows', 'ew_chain', 'ew_affine', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows',
+              'reduce_cols', 'transpose_tiled', 'pad_nd')
+
+
 def kernel_family(name: str) -> str:
     for prefix in ('conv_gemm', 'wgrad_gemm', 'dense_rows', 'softmax_rows', 'ew_chain', 'ew_affine', 'threefry2x32', 'gather_rows', 'pool', 'reduce_rows', 'reduce_cols', 'scatter_rows',
                    'select_window', 'scatter_selected', 'pad_nd', 'scale_relu_backward', 'scale_backward', 'transpose_tiled'):
@@ -127,10 +132,26 @@ def measure(workload, steps, warmup, batch=None, fuse=True, graph=False, profile
             stamped += np.diff(stamps)[1:1 + len(prof.launches)]    #[uploads | launches ... | downloads]
         stamped /= max(profile_iters, 1)
         scale = device_ms_per_step / float(stamped.sum()) if stamped.sum() > 0 else 1.0
+        #Launches of less than 20 us: the event after every launch and the gaps between launches are a large part of
+        #the stamped figure. Such a launch is also replayed ALONE, 200 times back to back on the buffers as the step
+        #left them (`repeated_ms`: one launch without event and with one launch-to-launch gap; its operands may come
+        #from the last-level cache, as they mostly do behind the launch that produced them). Only kernels that read
+        #their inputs and write their outputs anew each time are repeated; the index passes of the sorted scatter-add
+        #count in place and are left out.
+        repeated = [None] * len(prof.launches)
+        for k, (launch, ms) in enumerate(zip(prof.launches, stamped * scale)):
+            if ms < 0.02 and kernel_family(launch.kernel) in REPEATABLE:
+                single = dev.sequence()
+                prof.record_launch(single, launch)
+                single.replay(20)
+                repeated[k] = single.replay(200) / 200
+                single.destroy()
         fam = {}
-        for launch, ms in zip(prof.launches, stamped):
-            f = fam.setdefault(kernel_family(launch.kernel), dict(launches=0, stamped_ms=0.0, flops=0, bytes=0))
+        for launch, ms, rep in zip(prof.launches, stamped, repeated):
+            f = fam.setdefault(kernel_family(launch.kernel), dict(launches=0, stamped_ms=0.0, flops=0, bytes=0, repeated_ms=0.0, repeated=0))
             f['launches'] += 1; f['stamped_ms'] += float(ms); f['flops'] += launch.flops; f['bytes'] += launch.bytes_moved
+            if rep is not None:
+                f['repeated'] += 1; f['repeated_ms'] += rep
         if dump_launches:
             with open(dump_launches, 'w') as fh:
                 for op, launch, ms in zip(prof.all_ops, prof.launches, stamped * scale):
@@ -148,6 +169,13 @@ def measure(workload, steps, warmup, batch=None, fuse=True, graph=False, profile
             entry['mbytes'] = round(f['bytes'] / 1e6, 3)
             entry['gbs'] = round(f['bytes'] / ms / 1e6, 1)
             entry['frac_hbm_peak'] = round(entry['gbs'] / PEAK_HBM_GBS, 4)
+            if f['repeated'] == f['launches'] and f['repeated_ms'] > 0:
+                #every launch of the family is a short one: the family's time without events and gaps
+                entry['repeated_ms'] = round(f['repeated_ms'], 5)
+                entry['repeated_gbs'] = round(f['bytes'] / f['repeated_ms'] / 1e6, 1)
+                entry['repeated_frac_hbm_peak'] = round(entry['repeated_gbs'] / PEAK_HBM_GBS, 4)
+                if f['flops']:
+                    entry['repeated_tflops'] = round(f['flops'] / f['repeated_ms'] / 1e9, 3)
             kernels[name] = entry
         dominant = max(fam, key=lambda k: fam[k]['stamped_ms'])
         d, ms = fam[dominant], fam[dominant]['stamped_ms'] * scale
@@ -179,21 +207,59 @@ def measure(workload, steps, warmup, batch=None, fuse=True, graph=False, profile
     return result, wrapped, inputs
 
 
+def measure_primitives(iters=30, warm=10, only=None):
+    '''Single primitives at sizes where HBM bandwidth is the bound (vkjax_amd.workloads.PRIMITIVES): each program is
+    built, its inputs are made resident, and its launches are replayed `iters` times back to back between two HIP
+    events on the launch stream (after `warm` untimed replays). `bytes` is the ALGORITHMIC traffic of one evaluation
+    - every operand read once, every result written once - so `gbs` is what the caller of the primitive sees;
+    gaps between the launches of a program (one to five launches) are inside the time.'''
+    import gc
+    import vkjax_amd
+    from vkjax_amd import hip, workloads as W
+    dev, rows = hip.Device.get(), []
+    for name, (fn, make_inputs, algorithmic_bytes) in W.PRIMITIVES.items():
+        if only and not any(o in name for o in only):
+            continue
+        inputs  = make_inputs()
+        wrapped = vkjax_amd.wrap(fn, frontend='minijax')
+        interp, _ = wrapped._get_or_create_jaxpr_interpreter(tuple(inputs))
+        interp.upload_inputs(*inputs)
+        interp.replay(warm)
+        ms = statistics.median(interp.replay(iters) for _ in range(3)) / iters
+        nbytes = int(algorithmic_bytes(inputs))
+        gbs = nbytes / ms / 1e6
+        rows.append(dict(primitive=name, kernels=[l.kernel for l in interp.launches], mbytes=round(nbytes / 1e6, 3), ms=round(ms, 5),
+                         gbs=round(gbs, 1), frac_hbm_peak=round(gbs / PEAK_HBM_GBS, 4)))
+        del interp, wrapped, inputs
+        gc.collect()
+        dev.sync()
+    return rows
+
+
 def time_whole_calls(fn, inputs, fuse):
     '''Whole calls through wrap(): host arrays in, host arrays out, uploads and Python included; once copying every
     argument per call (what the reference does, vkjax/kompute_jaxpr_interpreter.py:66-81), once with the weights
     resident, once streamed (each call's upload overlaps the call before it). Median of 5 / mean of 40 after 4.'''
     import vkjax_amd
+    from vkjax_amd.minijax import tree_util
     out = {}
-    for label, kw in (('all_arguments_copied_ms', {}), ('weights_resident_ms', dict(resident_argnums=(0,)))):
-        if label == 'weights_resident_ms' and not isinstance(inputs[0], dict):
+    def frozen(a):
+        a = a.copy()
+        a.flags.writeable = False
+        return a
+    #read_only_weights_ms: plain wrap(f)(params, x), nothing declared, with a parameter tree of read-only arrays, which
+    #stay in HBM by themselves; weights_resident_ms: writeable parameters declared resident (each looked at for changes)
+    for label, kw in (('all_arguments_copied_ms', {}), ('read_only_weights_ms', {}), ('weights_resident_ms', dict(resident_argnums=(0,)))):
+        if label != 'all_arguments_copied_ms' and not isinstance(inputs[0], dict):
             continue
         f = vkjax_amd.wrap(fn, frontend='minijax', fuse=fuse, **kw)
-        f(*inputs)
+        call_inputs = [tree_util.tree_map(frozen, inputs[0])] + list(inputs[1:]) if label == 'read_only_weights_ms' else inputs
+        f(*call_inputs)
+        f(*call_inputs)
         times = []
-        for _ in range(5):
+        for _ in range(9):
             t0 = time.perf_counter()
-            f(*inputs)
+            f(*call_inputs)
             times.append((time.perf_counter() - t0) * 1e3)
         out[label] = round(statistics.median(times), 3)
         if label == 'weights_resident_ms':
@@ -401,6 +467,9 @@ def main():
                     help='warm-up and timed replays only (no per-launch sequence, whole calls, other configurations or CPU baseline): '
                          'under a kernel trace every dispatch after the first warmup x launches_per_step then belongs to a timed step')
     ap.add_argument('--graph', action='store_true', help='replay the launches as one captured HIP graph')
+    ap.add_argument('--no-primitives', action='store_true', help='skip the single-primitive bandwidth measurements')
+    ap.add_argument('--primitives-only', nargs='*', default=None, metavar='NAME',
+                    help='measure only the single primitives (those whose name contains one of the given words; all if none is given)')
     ap.add_argument('--profile-iters', type=int, default=3)
     ap.add_argument('--dump-launches', default=None, help='write one line per launch (kernel, grid, FLOP, bytes, ms) to this file')
     ap.add_argument('--calibration-copy', action='store_true',
@@ -415,6 +484,10 @@ def main():
     from vkjax_amd import hip, workloads as W
     props = hip.Device.get().get_device_properties()
     lean  = args.replays_only
+    if args.primitives_only is not None:
+        print(json.dumps({'metric': 'per-primitive HBM GB/s', 'unit': 'GB/s', 'n_gpus': 1, 'dtype': 'f32', 'data': 'synthetic',
+                          'peak_hbm_gbs': PEAK_HBM_GBS, 'primitives': measure_primitives(only=args.primitives_only)}))
+        return
 
     head, wrapped, inputs = measure(args.workload, args.steps, args.warmup, batch=args.batch, fuse=not args.no_fuse, graph=args.graph,
                                     profile_iters=args.profile_iters, end_to_end=not (lean or args.no_end_to_end),
@@ -436,6 +509,10 @@ def main():
                               end_to_end=not args.no_end_to_end)
             configs.append(c)
 
+    primitives = None
+    if args.workload == 'resnet50' and args.batch in (None, 64) and not (args.no_configs or args.no_primitives or lean):
+        primitives = measure_primitives()
+
     out = {
         'metric': 'ResNet-50 bs64 fp32 images/sec' if args.workload == 'resnet50' else f'{args.workload} throughput',
         'value': head['value'], 'unit': head['unit'], 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -449,7 +526,7 @@ def main():
                    'hbm_bytes_allocated': head['hbm_bytes_allocated'], 'build_seconds': head['build_seconds'],
                    **({'end_to_end_call': head['end_to_end_call']} if 'end_to_end_call' in head else {})},
         'roofline': head.get('roofline'), 'kernels': head.get('kernels'), 'cpu_baseline': cpu_baseline, 'output_check': output_check,
-        'configs': configs,
+        'configs': configs, 'primitives': primitives,
     }
     print(json.dumps(out))
 

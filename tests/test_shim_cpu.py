@@ -175,13 +175,13 @@ def test_buffer_freed_under_a_live_sequence_outlives_it(lib):
 
 def test_context_creation_releases_everything_when_a_step_fails(lib):
     before = lib.fake_hip_live_objects()
-    for successes in range(6):                                   #two streams and four events are created
+    for successes in range(7):                                   #two streams and five events are created
         lib.fake_hip_fail_after(successes)
         ctx = H()
         assert lib.vkj_ctx_create(0, C.byref(ctx)) != 0
         assert b'injected' in lib.vkj_last_error()
         assert lib.fake_hip_live_objects() == before
-    lib.fake_hip_fail_after(6)                                   #nothing left to fail in creation
+    lib.fake_hip_fail_after(7)                                   #nothing left to fail in creation
     ctx = H()
     assert lib.vkj_ctx_create(0, C.byref(ctx)) == 0
     lib.fake_hip_fail_after(-1)

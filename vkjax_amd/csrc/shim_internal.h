@@ -37,6 +37,7 @@ struct Ctx {
     hipStream_t copy_stream = nullptr;   // uploads that overlap the launches of `stream`
     hipEvent_t  ev_landed = nullptr;     // the following evaluation's arguments have reached HBM
     hipEvent_t  ev_uploaded = nullptr;   // this evaluation's own uploads have left their staging buffers
+    hipEvent_t  ev_copied = nullptr;     // the share of this evaluation's uploads that went over the second stream has arrived
     void*       static_landing = nullptr;   // this device's copy of the static landing array (static_landing.hip)
 };
 

@@ -91,8 +91,18 @@ class Function:
         self._interpreter_args   = (args, kwargs)
 
     def __call__(self, *args: tp.Any, **kwargs: tp.Any) -> tp.Any:
-        jaxpr_interpreter, output_shapes = self._get_or_create_jaxpr_interpreter(args)
-        output = jaxpr_interpreter.run(*args, **kwargs)
+        if self._tree is tree_util and not kwargs:
+            #the arguments are flattened once, for the cache key and for the run
+            leaves, structure = tree_util.tree_flatten(args)
+            jaxpr_interpreter, output_shapes = self._get_or_create_jaxpr_interpreter(args, (leaves, structure))
+            per_argument, at = [], 0
+            for child in structure.children:
+                per_argument.append(leaves[at:at + child.num_leaves])
+                at += child.num_leaves
+            output = jaxpr_interpreter.run_leaves(per_argument)
+        else:
+            jaxpr_interpreter, output_shapes = self._get_or_create_jaxpr_interpreter(args)
+            output = jaxpr_interpreter.run(*args, **kwargs)
         output = self._restore_shapes(output, output_shapes)
         if not self._profiling:
             return output
@@ -187,15 +197,17 @@ class Function:
         finally:
             ahead.close()
 
-    def _signature(self, args: tp.Tuple[tp.Any, ...]):
-        leaves, structure = self._tree.tree_flatten(args)
-        args_shape        = tuple(np.shape(x) for x in leaves)
-        args_dtype        = tuple(np.asarray(x).dtype if not hasattr(x, 'dtype') else np.dtype(x.dtype) for x in leaves)
+    def _signature(self, args: tp.Tuple[tp.Any, ...], flattened=None):
+        leaves, structure = flattened or self._tree.tree_flatten(args)
+        array             = np.ndarray
+        args_shape        = tuple(x.shape if type(x) is array else np.shape(x) for x in leaves)
+        args_dtype        = tuple(x.dtype if type(x) is array else np.asarray(x).dtype if not hasattr(x, 'dtype') else np.dtype(x.dtype)
+                                  for x in leaves)
         static_values     = tuple(repr(args[i]) for i in self._static_argnums if i < len(args))
         return (args_shape, args_dtype, structure, static_values)
 
-    def _get_or_create_jaxpr_interpreter(self, args: tp.Tuple[tp.Any, ...]):
-        shape_structure = self._signature(args)
+    def _get_or_create_jaxpr_interpreter(self, args: tp.Tuple[tp.Any, ...], flattened=None):
+        shape_structure = self._signature(args, flattened)
         if shape_structure not in self._jaxpr_interpreters:
             #new input shapes or structure, need to re-trace
             jaxpr, output_shapes = self.jaxpr_function(*args)
@@ -222,7 +234,7 @@ def wrap(function: tp.Callable, *args, **kwargs) -> Function:
     copy of weights and tables: leaves that cannot change while the caller holds them (numpy arrays with
     `flags.writeable == False`, jax arrays) are uploaded once and again only when another object is passed in their
     place; and `resident_argnums=(i, ...)` declares the same for every leaf of those arguments, writeable or not -
-    an in-place change of such a writeable array is noticed only if it moves the array or touches its first or last
-    64 bytes, so pass a new array for new values. Further keyword arguments: `frontend` ('jax', 'minijax', default:
+    an in-place change of such a writeable array is noticed only if it touches its first or last 64 bytes, so pass a
+    new array for new values. Further keyword arguments: `frontend` ('jax', 'minijax', default:
     jax where importable), `fuse`, `reuse_buffers`, `graph`.'''
     return Function(function, *args, **kwargs)

@@ -31,8 +31,8 @@ class JaxprInterpreter:
         #   writeable ones) and jax arrays - without being asked: such a leaf is uploaded when the object passed for
         #   it is not the one uploaded last;
         # * every leaf of the arguments named in resident_argnums (weights, tables), writeable or not. A writeable
-        #   one that is changed in place is noticed only when its address, shape, strides or its first or last
-        #   64 bytes change; pass a new array (or a read-only one) for a new value.
+        #   one that is changed in place is noticed only when its first or last 64 bytes change; pass a new array
+        #   (or a read-only one) for a new value.
         #All other leaves are copied on every call.
         self.resident_argnums = tuple(resident_argnums)
         self._resident_leaves = {}
@@ -94,16 +94,7 @@ class JaxprInterpreter:
             self._input_slots.append(self.sequence.record_upload(b.tensor, b.nbytes()) if b is not None else None)
         self._batch_tables = []
         for op, launch in zip(self.all_ops, self.launches):
-            if launch.members:
-                #a batch of small launches reads its members' arguments from a table in HBM
-                table = self.mgr.tensor(K.batch_table(launch, lambda b: b.tensor.device_ptr()))
-                self._batch_tables.append(table)
-                self.sequence.record_launch(launch.kernel, launch.grid, launch.block, [(table, 0)], launch.params, launch.lds)
-                continue
-            bufs = [((b.tensor if b is not None else None), off) for b, off in launch.buffers]
-            for (b, _), (t, _) in zip(launch.buffers, bufs):
-                assert b is None or t is not None, f'{op}: buffer without storage'
-            self.sequence.record_launch(launch.kernel, launch.grid, launch.block, bufs, launch.params, launch.lds)
+            self.record_launch(self.sequence, launch, op)
         if self.graph:
             self.sequence.use_graph(True)
         self._output_slots = []
@@ -116,12 +107,27 @@ class JaxprInterpreter:
             self._output_slots.append(self.sequence.record_download(b.tensor, b.nbytes()))
             self._output_sizes.append(b.size)
 
-    def _flatten_args(self, X, with_residency: bool = False):
+    def record_launch(self, sequence, launch, op=None):
+        '''Records one of this program's launches into `sequence` (its own, or another sequence on the same buffers:
+        measurements replay single launches that way).'''
+        if launch.members:
+            #a batch of small launches reads its members' arguments from a table in HBM
+            table = self.mgr.tensor(K.batch_table(launch, lambda b: b.tensor.device_ptr()))
+            self._batch_tables.append(table)
+            sequence.record_launch(launch.kernel, launch.grid, launch.block, [(table, 0)], launch.params, launch.lds)
+            return
+        bufs = [((b.tensor if b is not None else None), off) for b, off in launch.buffers]
+        for (b, _), (t, _) in zip(launch.buffers, bufs):
+            assert b is None or t is not None, f'{op or launch.kernel}: buffer without storage'
+        sequence.record_launch(launch.kernel, launch.grid, launch.block, bufs, launch.params, launch.lds)
+
+    def _flatten_args(self, X, with_residency: bool = False, per_argument=None):
+        '''`per_argument`: the leaves of every argument (static ones included) where the caller has them already.'''
         leaves, resident = [], []
-        for i, x in enumerate(X):
+        for i, x in enumerate(X if per_argument is None else per_argument):
             if i in self.static_argnums:
                 continue
-            these = [x] if type(x) is np.ndarray else tree_util.tree_leaves([x])
+            these = x if per_argument is not None else [x] if type(x) is np.ndarray else tree_util.tree_leaves([x])
             leaves   += these
             named     = i in self.resident_argnums
             resident += [RESIDENT_CHECKED if named and _may_change_in_place(leaf) else RESIDENT if named or _is_immutable(leaf) else 0
@@ -130,24 +136,23 @@ class JaxprInterpreter:
             raise TypeError(f'Expected {len(self.input_buffers)} input arguments, received {len(leaves)}')
         return (leaves, resident) if with_residency else leaves
 
-    def _convert_inputs(self, X) -> tp.List[tp.Tuple]:
+    def _convert_inputs(self, X, per_argument=None) -> tp.List[tp.Tuple]:
         '''(leaf number, transfer slot, the leaf, its device words, whether it is a resident one) for every argument
-        leaf the program reads. Touches no state of the interpreter: it may run ahead of the evaluation it is for.'''
-        X, resident = self._flatten_args(X, with_residency=True)
+        leaf the program reads. The words of a leaf that is identified by its object alone are left out (None) and
+        made when the leaf turns out to need an upload. Touches no state of the interpreter: it may run ahead of the
+        evaluation it is for.'''
+        X, resident = self._flatten_args(X, with_residency=True, per_argument=per_argument)
         if self.sequence is None:
             raise RuntimeError('this interpreter was built with plan_only=True and has no device to run on')
-        converted = []
-        for k, (slot, x, var) in enumerate(zip(self._input_slots, X, self.jaxpr.jaxpr.invars)):
-            if slot is None:
-                continue
-            #the common case without the general conversion: an array that already is what the device holds
-            n, dtype = self._input_specs[k]
-            if type(x) is np.ndarray and x.dtype == dtype and x.size == n and x.flags.c_contiguous:
-                words = x.reshape(-1).view(np.uint32)
-            else:
-                words = _device_words_of_argument(x, var.aval)
-            converted.append((k, slot, x, words, resident[k]))
-        return converted
+        return [(k, slot, x, None if resident[k] == RESIDENT else self._device_words(k, x), resident[k])
+                for k, (slot, x) in enumerate(zip(self._input_slots, X)) if slot is not None]
+
+    def _device_words(self, k: int, x) -> np.ndarray:
+        #the common case without the general conversion: an array that already is what the device holds
+        n, dtype = self._input_specs[k]
+        if type(x) is np.ndarray and x.dtype == dtype and x.size == n and x.flags.c_contiguous:
+            return x.reshape(-1).view(np.uint32)
+        return _device_words_of_argument(x, self.jaxpr.jaxpr.invars[k].aval)
 
     def _select_uploads(self, converted) -> tp.List[tp.Optional[np.ndarray]]:
         '''One entry per transfer slot: the device words of every leaf that has to be copied. A resident leaf is
@@ -161,11 +166,11 @@ class JaxprInterpreter:
                 if held is not None and held[0] is x and held[1] == mark:
                     continue                                    #already in HBM
                 self._resident_leaves[k] = (x, mark)
-            host[slot] = words
+            host[slot] = words if words is not None else self._device_words(k, x)
         return host
 
-    def _host_inputs(self, X) -> tp.List[tp.Optional[np.ndarray]]:
-        return self._select_uploads(self._convert_inputs(X))
+    def _host_inputs(self, X, per_argument=None) -> tp.List[tp.Optional[np.ndarray]]:
+        return self._select_uploads(self._convert_inputs(X, per_argument))
 
     def _fresh_outputs(self, host) -> tp.List[tp.Optional[np.ndarray]]:
         #every call hands out fresh arrays: the runtime copies the results straight into them
@@ -198,6 +203,13 @@ class JaxprInterpreter:
             raise
         finally:
             self._evaluations += 1
+
+    def run_leaves(self, per_argument):
+        '''`run` for a caller that has flattened the arguments already: one list of leaves per argument.'''
+        host  = self._host_inputs(None, per_argument)
+        fresh = self._fresh_outputs(host)
+        self.evaluate(host)
+        return self._output_values(fresh)
 
     def run(self, *X, return_all=False):
         '''Executes a previously recorded sequence with actual data'''
@@ -281,9 +293,9 @@ def _may_change_in_place(leaf) -> bool:
 
 
 def _fingerprint(x: np.ndarray, words: np.ndarray):
-    '''What a cheap look at a writeable array can tell about a change in place: where it lives, its layout and its
-    first and last 64 bytes.'''
-    return (x.__array_interface__['data'][0], x.shape, x.strides, words[:16].tobytes(), words[-16:].tobytes())
+    '''What a cheap look at a writeable array can tell about a change in place: its first and last 64 bytes (the
+    object, and with it shape and element type, is compared by the caller).'''
+    return (words[:16].tobytes(), words[-16:].tobytes())
 
 
 def _device_words_of_argument(x, aval) -> np.ndarray:

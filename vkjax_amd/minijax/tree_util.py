@@ -4,6 +4,8 @@ tree_map / tree_multimap; reference: vkjax/function.py:26-43,
 vkjax/kompute_jaxpr_interpreter.py:69).'''
 import typing as tp
 
+import numpy as np
+
 
 class TreeDef:
     '''Hashable description of a container nest; leaves are `*`.'''
@@ -41,12 +43,19 @@ class TreeDef:
 _LEAF = TreeDef('leaf', None, ())
 
 
+_NONE = TreeDef('none', None, ())
+_ARRAY = np.ndarray
+
+
 def tree_flatten(tree) -> tp.Tuple[list, TreeDef]:
     leaves = []
 
     def rec(x):
+        if type(x) is _ARRAY:                       #by far the most frequent node: no further tests
+            leaves.append(x)
+            return _LEAF
         if x is None:
-            return TreeDef('none', None, ())
+            return _NONE
         if isinstance(x, tuple) and not hasattr(x, '_fields'):
             return TreeDef('tuple', None, [rec(c) for c in x])
         if isinstance(x, list):
@@ -62,7 +71,25 @@ def tree_flatten(tree) -> tp.Tuple[list, TreeDef]:
 
 
 def tree_leaves(tree) -> list:
-    return tree_flatten(tree)[0]
+    '''The leaves alone, in tree_flatten's order, without building the structure.'''
+    leaves = []
+
+    def rec(x):
+        if type(x) is _ARRAY:
+            leaves.append(x)
+        elif x is None:
+            pass
+        elif (isinstance(x, tuple) and not hasattr(x, '_fields')) or isinstance(x, list):
+            for c in x:
+                rec(c)
+        elif isinstance(x, dict):
+            for k in sorted(x.keys()):
+                rec(x[k])
+        else:
+            leaves.append(x)
+
+    rec(tree)
+    return leaves
 
 
 def tree_structure(tree) -> TreeDef:

@@ -281,6 +281,57 @@ def resnet50_train_inputs(seed=4, batch=64, size=224, num_classes=1000, width_sc
     return [params, x, onehot]
 
 
+# ------------------------------------------------------------------ single primitives at sizes where memory bandwidth is the bound
+
+def _uniform_words(n: int, seed: int) -> np.ndarray:
+    return np.random.default_rng(seed).random(n, dtype=np.float32)
+
+
+def _bn(c, seed=0):
+    rng = np.random.default_rng(seed)
+    return [(0.5 + rng.random(c, dtype=np.float32)).astype(np.float32), rng.standard_normal(c, dtype=np.float32),
+            rng.standard_normal(c, dtype=np.float32), (0.5 + rng.random(c, dtype=np.float32)).astype(np.float32)]
+
+
+_ACT  = (64, 56, 56, 256)          #a ResNet-50 activation of 51.4 M elements (205.5 MB)
+_WIDE = (64, 112, 112, 64)         #the input of ResNet-50's max-pool
+_N64M = 1 << 26
+
+#name -> (function, inputs, ALGORITHMIC bytes of one evaluation: every operand read once and every result written once)
+PRIMITIVES: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable, tp.Callable]] = {
+    'reduce_sum rows 65536x1000':   (lambda x: jnp.sum(x, axis=1), lambda: [_uniform_words(65536000, 1).reshape(65536, 1000)], lambda a: a[0].nbytes + 4 * 65536),
+    'reduce_sum rows 4096x16384':   (lambda x: jnp.sum(x, axis=1), lambda: [_uniform_words(_N64M, 2).reshape(4096, 16384)], lambda a: a[0].nbytes + 4 * 4096),
+    'reduce_sum columns 262144x256': (lambda x: jnp.sum(x, axis=0), lambda: [_uniform_words(_N64M, 3).reshape(262144, 256)], lambda a: a[0].nbytes + 4 * 256),
+    'reduce_sum all 64M':           (lambda x: jnp.sum(x), lambda: [_uniform_words(_N64M, 4)], lambda a: a[0].nbytes + 4),
+    'reduce_max rows 65536x1000':   (lambda x: jnp.max(x, axis=1), lambda: [_uniform_words(65536000, 5).reshape(65536, 1000)], lambda a: a[0].nbytes + 4 * 65536),
+    'argmax rows 65536x1000':       (lambda x: jnp.argmax(x, axis=1), lambda: [_uniform_words(65536000, 6).reshape(65536, 1000)], lambda a: a[0].nbytes + 4 * 65536),
+    'global average 64x7x7x2048':   (lambda x: jnp.mean(x, axis=(1, 2)), lambda: [_uniform_words(64 * 49 * 2048, 7).reshape(64, 7, 7, 2048)], lambda a: a[0].nbytes + 4 * 64 * 2048),
+    'add 64M':                      (lambda x, y: x + y, lambda: [_uniform_words(_N64M, 8), _uniform_words(_N64M, 9)], lambda a: 3 * a[0].nbytes),
+    'relu 64M':                     (lambda x: nn.relu(x - 0.5), lambda: [_uniform_words(_N64M, 10)], lambda a: 2 * a[0].nbytes),
+    'exp 64M':                      (lambda x: jnp.exp(x), lambda: [_uniform_words(_N64M, 11)], lambda a: 2 * a[0].nbytes),
+    'batch norm + relu 64x56x56x256': (lambda x, s, b, m, v: nn.relu(nn.batch_norm_inference(x, s, b, m, v)),
+                                     lambda: [_uniform_words(int(np.prod(_ACT)), 12).reshape(_ACT)] + _bn(256), lambda a: 2 * a[0].nbytes + 4 * 4 * 256),
+    'batch norm + residual + relu 64x56x56x256': (lambda x, r, s, b, m, v: nn.relu(nn.batch_norm_inference(x, s, b, m, v) + r),
+                                     lambda: [_uniform_words(int(np.prod(_ACT)), 13).reshape(_ACT), _uniform_words(int(np.prod(_ACT)), 14).reshape(_ACT)] + _bn(256),
+                                     lambda a: 3 * a[0].nbytes + 4 * 4 * 256),
+    'max pool 3x3 s2 64x112x112x64': (lambda x: lax.reduce_window(x, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (0, 1), (0, 1), (0, 0))),
+                                     lambda: [_uniform_words(int(np.prod(_WIDE)), 15).reshape(_WIDE)], lambda a: a[0].nbytes + a[0].nbytes // 4),
+    'sum pool 2x2 s2 64x112x112x64': (lambda x: lax.reduce_window(x, 0.0, lax.add, (1, 2, 2, 1), (1, 2, 2, 1), 'VALID'),
+                                     lambda: [_uniform_words(int(np.prod(_WIDE)), 16).reshape(_WIDE)], lambda a: a[0].nbytes + a[0].nbytes // 4),
+    'threefry2x32 8388608 lanes':   (lambda k0, k1, x0, x1: lax.threefry2x32(k0, k1, x0, x1),
+                                     lambda: [np.uint32(0x13198a2e), np.uint32(0x03707344), np.arange(1 << 23, dtype=np.uint32), np.arange(1 << 23, 1 << 24, dtype=np.uint32)],
+                                     lambda a: 4 * a[2].nbytes),
+    'transpose 8192x8192':          (lambda x: lax.transpose(x, (1, 0)), lambda: [_uniform_words(_N64M, 17).reshape(8192, 8192)], lambda a: 2 * a[0].nbytes),
+    'transpose NHWC to NCHW 64x56x56x256': (lambda x: lax.transpose(x, (0, 3, 1, 2)), lambda: [_uniform_words(int(np.prod(_ACT)), 18).reshape(_ACT)], lambda a: 2 * a[0].nbytes),
+    'pad height and width 64x56x56x256': (lambda x: lax.pad(x, 0.0, ((0, 0, 0), (1, 1, 0), (1, 1, 0), (0, 0, 0))),
+                                     lambda: [_uniform_words(int(np.prod(_ACT)), 19).reshape(_ACT)], lambda a: a[0].nbytes + 64 * 58 * 58 * 256 * 4),
+    'gather rows 262144x1KB of 65536': (lambda t, i: t[i], lambda: gather_scatter_inputs()[:2], lambda a: 2 * a[1].size * a[0].shape[1] * 4 + a[1].nbytes),
+    'scatter-add rows 262144x1KB into 65536': (lambda i, u: jnp.index_add(jnp.zeros((65536, 256), np.float32), i, u), lambda: gather_scatter_inputs()[1:],
+                                     lambda a: a[1].nbytes + a[0].nbytes + 65536 * 256 * 4),
+    'uniform 4096x4096 from a key': (rng_uniform, rng_inputs, lambda a: 4096 * 4096 * 4),
+}
+
+
 WORKLOADS: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable]] = {
     'affine':         (affine, affine_inputs),
     'mlp':            (mlp, mlp_inputs),
