@@ -114,6 +114,17 @@ int vkj_seq_record_download(vkj_handle seq, vkj_handle buf, size_t offset, int s
  * nodes inside a captured graph have given wrong results on replays after the first, and
  * vkj_seq_use_graph captures the launches of a sequence. vkj_buf_memset clears a buffer outside
  * sequences. */
+/* Puts recorded launch number `launch` (0-based, in recording order) on lane 0 (the context's stream, the
+ * default) or lane 1 (a second stream of the same priority), and says whether its lane has to wait, before
+ * the launch is issued, for everything recorded before it on the OTHER lane. Launches keep their recorded
+ * order within a lane; lane 1 starts behind the uploads and is joined before the downloads. The caller
+ * is responsible for the waits its data dependencies need (read after write, write after read and write
+ * after write, on the memory the launches touch). Events are created here, none when evaluating. A
+ * sequence replayed as a graph or created with timestamps issues all launches on lane 0 in recorded
+ * order. The reference records every dispatch into one in-order sequence
+ * (vkjax/kompute_jaxpr_interpreter.py:55-60); this lets launches that do not depend on each other share
+ * the GPU (the index passes of a scatter-add beside a gather, a projection beside the branch it joins). */
+int vkj_seq_set_launch_lane(vkj_handle seq, int launch, int lane, int wait_for_other_lane);
 int vkj_seq_num_steps(vkj_handle seq, int* uploads, int* launches, int* downloads);
 /* sequence.eval()                     reference: vkjax/kompute_jaxpr_interpreter.py:77
  * All uploads, then all launches, then all downloads, then one stream synchronisation.

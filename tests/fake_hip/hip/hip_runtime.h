@@ -17,7 +17,7 @@
 
 typedef int hipError_t;
 enum { hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2, hipErrorNotFound = 500, hipErrorUnknown = 999 };
-enum { hipStreamNonBlocking = 1, hipEventDisableTiming = 2, hipHostMallocDefault = 0, hipStreamCaptureModeThreadLocal = 1 };
+enum { hipStreamNonBlocking = 1, hipEventDisableTiming = 2, hipEventReleaseToDevice = 0x40000000, hipHostMallocDefault = 0, hipStreamCaptureModeThreadLocal = 1 };
 enum hipMemcpyKind { hipMemcpyHostToDevice = 1, hipMemcpyDeviceToHost = 2, hipMemcpyDeviceToDevice = 3 };
 #define HIP_LAUNCH_PARAM_BUFFER_POINTER ((void*)1)
 #define HIP_LAUNCH_PARAM_BUFFER_SIZE    ((void*)2)

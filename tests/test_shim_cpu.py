@@ -175,13 +175,13 @@ def test_buffer_freed_under_a_live_sequence_outlives_it(lib):
 
 def test_context_creation_releases_everything_when_a_step_fails(lib):
     before = lib.fake_hip_live_objects()
-    for successes in range(7):                                   #two streams and five events are created
+    for successes in range(8):                                   #three streams and five events are created
         lib.fake_hip_fail_after(successes)
         ctx = H()
         assert lib.vkj_ctx_create(0, C.byref(ctx)) != 0
         assert b'injected' in lib.vkj_last_error()
         assert lib.fake_hip_live_objects() == before
-    lib.fake_hip_fail_after(7)                                   #nothing left to fail in creation
+    lib.fake_hip_fail_after(8)                                   #nothing left to fail in creation
     ctx = H()
     assert lib.vkj_ctx_create(0, C.byref(ctx)) == 0
     lib.fake_hip_fail_after(-1)
@@ -309,3 +309,35 @@ def test_static_entry_point_and_graphs(lib):
     for b in (src, dst):
         assert lib.vkj_buf_free(w.ctx, b) == 0
     w.close()
+
+
+def test_launches_on_two_lanes(lib):
+    '''vkj_seq_set_launch_lane: launches of lane 1 go to the side stream, waits make events at record time (none when
+    evaluating), bad arguments are refused, and everything is released with the sequence.'''
+    before = lib.fake_hip_live_objects()
+    w = World(lib)
+    n = 100
+    a, b, c, seq = w.buf(4 * n), w.buf(4 * n), w.buf(4 * n), H()
+    assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq)) == 0
+    assert lib.vkj_seq_record_upload(seq, a, 0, 0, 4 * n) == 0
+    assert w.record_add_one(seq, b, a, n) == 0                   #b = a + 1
+    assert w.record_add_one(seq, c, a, n) == 0                   #c = a + 1   (independent of the first: lane 1)
+    assert w.record_add_one(seq, a, c, n) == 0                   #a = c + 1   (waits for lane 1, and for the first launch's read of a)
+    assert lib.vkj_seq_record_download(seq, a, 0, 1, 4 * n) == 0
+    assert lib.vkj_seq_set_launch_lane(seq, 1, 1, 0) == 0
+    assert lib.vkj_seq_set_launch_lane(seq, 2, 0, 1) == 0
+    assert lib.vkj_seq_set_launch_lane(seq, 3, 0, 0) == EINVAL    #no such launch
+    assert lib.vkj_seq_set_launch_lane(seq, 0, 2, 0) == EINVAL    #no such lane
+    made = lib.fake_hip_creations()
+    x = np.arange(n, dtype=np.uint32)
+    for _ in range(3):
+        assert np.array_equal(w.eval(seq, x), x + 2)
+    assert lib.fake_hip_creations() == made                      #fork, join and wait events exist since they were asked for
+    assert lib.vkj_seq_set_launch_lane(seq, 2, 0, 0) == 0         #a wait that is taken back gives its event back
+    assert lib.vkj_seq_set_launch_lane(seq, 1, 0, 0) == 0         #back on one lane
+    assert np.array_equal(w.eval(seq, x), x + 2)
+    assert lib.vkj_seq_destroy(seq) == 0
+    for buf in (a, b, c):
+        assert lib.vkj_buf_free(w.ctx, buf) == 0
+    w.close()
+    assert lib.fake_hip_live_objects() == before

@@ -181,8 +181,9 @@ void destroy_ctx_objects(Ctx* c) {
     if (c->ev_copied)   hipEventDestroy(c->ev_copied);
     if (c->stream)      hipStreamDestroy(c->stream);
     if (c->copy_stream) hipStreamDestroy(c->copy_stream);
+    if (c->side_stream) hipStreamDestroy(c->side_stream);
     c->ev_begin = c->ev_end = c->ev_landed = c->ev_uploaded = c->ev_copied = nullptr;
-    c->stream = c->copy_stream = nullptr;
+    c->stream = c->copy_stream = c->side_stream = nullptr;
 }
 
 // A sequence lets go of a buffer it recorded; the memory of a buffer that vkj_buf_free has
@@ -194,12 +195,12 @@ void unref_buf(Buf* b) {
     }
 }
 
-int issue_launch(Ctx* c, Launch& l) {
+int issue_launch(Ctx* c, Launch& l, hipStream_t stream = nullptr) {
     size_t size = l.kernarg.size();
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, l.kernarg.data(),
                      HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
     hipError_t e = hipModuleLaunchKernel(l.fn->fn, l.grid[0], l.grid[1], l.grid[2],
-                                         l.block[0], l.block[1], l.block[2], l.lds, c->stream, nullptr, extra);
+                                         l.block[0], l.block[1], l.block[2], l.lds, stream ? stream : c->stream, nullptr, extra);
     if (e != hipSuccess) {
         g_last_error = "launch of " + l.fn->name + ": " + hipGetErrorString(e);
         return (int)e;
@@ -237,8 +238,28 @@ int issue_all(Ctx* c, Seq* s) {
             return 0;
         }
     }
-    for (auto& l : s->launches)
-        if (int r = issue_launch(c, l)) return r;
+    if (!s->uses_side) {
+        for (auto& l : s->launches)
+            if (int r = issue_launch(c, l)) return r;
+        return 0;
+    }
+    // Two lanes: launches keep their recorded order on each lane's stream; where a launch was told to wait for the
+    // other lane, an event recorded there (behind everything issued on it so far) is waited for on its own lane
+    // first. Lane 1 starts behind what the stream holds already (the uploads) and is joined at the end, so that
+    // whatever follows on the stream - downloads, the final wait - follows both. (A captured graph and a sequence
+    // with time stamps issue every launch on the stream, in recorded order, which satisfies the same dependencies.)
+    HIP_TRY(hipEventRecord(s->ev_fork, c->stream));
+    HIP_TRY(hipStreamWaitEvent(c->side_stream, s->ev_fork, 0));
+    for (auto& l : s->launches) {
+        hipStream_t mine = l.lane ? c->side_stream : c->stream, other = l.lane ? c->stream : c->side_stream;
+        if (l.wait_event) {
+            HIP_TRY(hipEventRecord(l.wait_event, other));
+            HIP_TRY(hipStreamWaitEvent(mine, l.wait_event, 0));
+        }
+        if (int r = issue_launch(c, l, mine)) return r;
+    }
+    HIP_TRY(hipEventRecord(s->ev_join, c->side_stream));
+    HIP_TRY(hipStreamWaitEvent(c->stream, s->ev_join, 0));
     return 0;
 }
 
@@ -460,6 +481,7 @@ int vkj_ctx_create(int device, vkj_handle* out) {
         HIP_TRY(hipSetDevice(device));
         HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
         HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
+        HIP_TRY(hipStreamCreateWithFlags(&c->side_stream, hipStreamNonBlocking));
         HIP_TRY(hipEventCreate(&c->ev_begin));
         HIP_TRY(hipEventCreate(&c->ev_end));
         HIP_TRY(hipEventCreateWithFlags(&c->ev_landed, hipEventDisableTiming));
@@ -482,6 +504,7 @@ int vkj_ctx_destroy(vkj_handle h) {
     if (int r = use(c)) return r;
     hipStreamSynchronize(c->stream);
     hipStreamSynchronize(c->copy_stream);
+    hipStreamSynchronize(c->side_stream);
     destroy_ctx_objects(c);
     retire(c);
     delete c;
@@ -685,10 +708,14 @@ int vkj_seq_destroy(vkj_handle sh) {
         if (t.staging) hipHostFree(t.staging);
         unref_buf(t.buf);
     }
+    hipStreamSynchronize(s->ctx->side_stream);
     for (auto& l : s->launches) {
         l.fn->mod->seq_refs--;
         for (Buf* b : l.bufs) unref_buf(b);
+        if (l.wait_event) hipEventDestroy(l.wait_event);
     }
+    if (s->ev_fork) hipEventDestroy(s->ev_fork);
+    if (s->ev_join) hipEventDestroy(s->ev_join);
     for (auto e : s->stamps) hipEventDestroy(e);
     for (auto e : s->chunk_events) hipEventDestroy(e);
     drop_graph(s);
@@ -767,6 +794,28 @@ int vkj_seq_record_launch(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], 
     f->mod->seq_refs++;
     s->launches.push_back(std::move(l));
     drop_graph(s);                                  // a captured graph no longer matches the sequence
+    return 0;
+}
+
+int vkj_seq_set_launch_lane(vkj_handle sh, int launch, int lane, int wait_for_other_lane) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_set_launch_lane: bad handle");
+    if (launch < 0 || (size_t)launch >= s->launches.size() || lane < 0 || lane > 1)
+        return fail(VKJ_EINVAL, "vkj_seq_set_launch_lane: launch %d of %zu, lane %d (0 or 1)", launch, s->launches.size(), lane);
+    if (int r = use(s->ctx)) return r;
+    Launch& l = s->launches[launch];
+    // everything an evaluation needs is made here, so that evaluating creates nothing
+    if (lane == 1 && !s->ev_fork) {
+        HIP_TRY(hipEventCreateWithFlags(&s->ev_fork, hipEventDisableTiming | hipEventReleaseToDevice));
+        hipError_t e = hipEventCreateWithFlags(&s->ev_join, hipEventDisableTiming | hipEventReleaseToDevice);
+        if (e != hipSuccess) { hipEventDestroy(s->ev_fork); s->ev_fork = nullptr; return hip_fail(e, "hipEventCreateWithFlags"); }
+    }
+    if (wait_for_other_lane && !l.wait_event) HIP_TRY(hipEventCreateWithFlags(&l.wait_event, hipEventDisableTiming | hipEventReleaseToDevice));
+    if (!wait_for_other_lane && l.wait_event) { hipEventDestroy(l.wait_event); l.wait_event = nullptr; }
+    l.lane = lane;
+    s->uses_side = false;
+    for (auto& other : s->launches) if (other.lane) s->uses_side = true;
+    drop_graph(s);
     return 0;
 }
 

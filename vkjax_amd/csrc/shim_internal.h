@@ -35,6 +35,7 @@ struct Ctx {
     hipStream_t stream = nullptr;
     hipEvent_t  ev_begin = nullptr, ev_end = nullptr;
     hipStream_t copy_stream = nullptr;   // uploads that overlap the launches of `stream`
+    hipStream_t side_stream = nullptr;   // launches of lane 1: work that does not depend on what `stream` is running
     hipEvent_t  ev_landed = nullptr;     // the following evaluation's arguments have reached HBM
     hipEvent_t  ev_uploaded = nullptr;   // this evaluation's own uploads have left their staging buffers
     hipEvent_t  ev_copied = nullptr;     // the share of this evaluation's uploads that went over the second stream has arrived
@@ -85,6 +86,9 @@ struct Launch {
     uint32_t             grid[3], block[3], lds;
     std::vector<uint8_t> kernarg;
     std::vector<Buf*>    bufs;       // the buffers whose addresses the argument block holds
+    int                  lane = 0;   // 0: the context's stream, 1: its side stream
+    hipEvent_t           wait_event = nullptr;   // made when the launch is told to wait for the other lane: recorded there
+                                                 // and waited for on this launch's lane before the launch is issued
 };
 
 struct Seq {
@@ -97,6 +101,9 @@ struct Seq {
     std::vector<hipEvent_t> chunk_events;   // one behind every chunk of a large download
     std::vector<hipEvent_t> stamps;         // profiling: 1 + number of steps
     int                     stamps_valid = 0;
+    bool                    uses_side = false;      // some launch is on lane 1
+    hipEvent_t              ev_fork = nullptr;      // lane 1 starts behind everything queued on the stream so far (uploads)
+    hipEvent_t              ev_join = nullptr;      // the stream continues (downloads, the final wait) behind lane 1
     bool                    want_graph = false;     // issue the launches as one captured graph
     bool                    graph_failed = false;   // capture did not work once: keep to plain launches
     hipGraphExec_t          graph_exec = nullptr;

@@ -55,6 +55,7 @@ _PROTOTYPES = {
     'vkj_seq_create':          (C.c_int, [_H, C.c_int, C.POINTER(_H)]),
     'vkj_seq_destroy':         (C.c_int, [_H]),
     'vkj_seq_record_upload':   (C.c_int, [_H, _H, C.c_size_t, C.c_int, C.c_size_t]),
+    'vkj_seq_set_launch_lane': (C.c_int, [_H, C.c_int, C.c_int, C.c_int]),
     'vkj_seq_record_launch':   (C.c_int, [_H, _H, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_uint32,
                                           C.c_void_p, C.c_size_t, C.POINTER(_H), C.POINTER(C.c_uint32),
                                           C.POINTER(C.c_uint64), C.c_int]),
@@ -278,6 +279,11 @@ class Sequence:
         _check(self.device.lib.vkj_seq_record_launch(self.handle, fn, g, b, lds_bytes, kernarg, len(kernarg),
                                                       handles, argoffs, byteoff, n), f'vkj_seq_record_launch({kernel_name})')
         self.n_launches += 1
+
+    def set_launch_lane(self, launch: int, lane: int, wait_for_other_lane: bool):
+        '''Launch number `launch` goes to lane 0 (the stream) or 1 (the side stream); with `wait_for_other_lane` its
+        lane first waits for everything recorded before it on the other one.'''
+        _check(self.device.lib.vkj_seq_set_launch_lane(self.handle, launch, lane, int(bool(wait_for_other_lane))), 'vkj_seq_set_launch_lane')
 
     def eval(self, host_arrays: tp.Sequence[tp.Optional[np.ndarray]], flags: int = 0,
              next_host_arrays: tp.Optional[tp.Sequence[tp.Optional[np.ndarray]]] = None, static_landing: bool = False):

@@ -15,6 +15,7 @@ import numpy as np
 from . import fusion
 from . import hip
 from . import kernels as K
+from . import lanes
 from . import ops
 from .buffers import BufferPool, PlanOnlyDevice, to_device_words, view_or_convert_from_32bit
 from .minijax import core, tree_util
@@ -23,7 +24,7 @@ from .minijax import core, tree_util
 class JaxprInterpreter:
     def __init__(self, jaxpr, static_argnums: tp.Tuple[int, ...] = (), profiling: bool = False,
                  reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False, graph: bool = False,
-                 resident_argnums: tp.Tuple[int, ...] = ()):
+                 resident_argnums: tp.Tuple[int, ...] = (), two_lanes: bool = False):
         self.jaxpr          = jaxpr
         #Which argument leaves stay in HBM between calls instead of being copied on every call, as the reference
         #does (vkjax/kompute_jaxpr_interpreter.py:72-75):
@@ -36,6 +37,10 @@ class JaxprInterpreter:
         #All other leaves are copied on every call.
         self.resident_argnums = tuple(resident_argnums)
         self._resident_leaves = {}
+        #two_lanes: launches that do not depend on the ones before them run beside them on a second stream
+        #(vkjax_amd/lanes.py). Off by default: on this GPU a dependency between two streams costs about 12 us, more
+        #than the launches it would let overlap (see the measurements quoted in lanes.py)
+        self.two_lanes      = two_lanes
         #graph=True replays the launches as one captured HIP graph (never with profiling)
         self.graph          = graph and not profiling
         self.static_argnums = tuple(static_argnums)
@@ -80,6 +85,7 @@ class JaxprInterpreter:
         self.bufferpool.create_tensors()
         #lower every op now so that unsupported layouts fail at build time, not at run time
         self.launches = [op.launch for op in self.all_ops]
+        self.lane_plan = lanes.plan(self.all_ops, self.launches) if self.two_lanes else None
 
         if isinstance(self.mgr, PlanOnlyDevice):
             return
@@ -95,6 +101,10 @@ class JaxprInterpreter:
         self._batch_tables = []
         for op, launch in zip(self.all_ops, self.launches):
             self.record_launch(self.sequence, launch, op)
+        if self.lane_plan is not None and any(self.lane_plan.lane):
+            for k, (lane, wait) in enumerate(zip(self.lane_plan.lane, self.lane_plan.wait)):
+                if lane or wait:
+                    self.sequence.set_launch_lane(k, lane, wait)
         if self.graph:
             self.sequence.use_graph(True)
         self._output_slots = []

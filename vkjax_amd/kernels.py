@@ -86,6 +86,8 @@ class Launch(tp.NamedTuple):
     #a batch launch: the launches it evaluates, described to the kernel by a table in device memory
     #that is written when the launch is recorded (it holds device addresses)
     members: tp.Tuple['Launch', ...] = ()
+    #which of `buffers` the kernel writes (positions); everything else it only reads
+    written: tp.Tuple[int, ...] = (0,)
 
 
 def _u32(*values) -> bytes:
@@ -1011,7 +1013,7 @@ def scale_relu_backward(column_sum: Launch, dx: Buffer, sum_m: Buffer, sum_mx: B
     name = 'scale_relu_backward_' if select is not None else 'scale_backward_'
     return Launch(name + column_sum.kernel[-2:], column_sum.grid, column_sum.block,
                   [(dx, 0), (sum_m, 0), (sum_mx, 0), (ans, 0), (threshold, 0), (cotangent, 0), (otherwise, 0), (x, 0), (scale, 0)],
-                  column_sum.params, bytes_moved=4 * ((4 if select is not None else 3) * n + 2 * scale.size))
+                  column_sum.params, bytes_moved=4 * ((4 if select is not None else 3) * n + 2 * scale.size), written=(0, 1, 2))
 
 
 SOFTMAX_MAX_ROW = 4096      #rows this short run unsplit in reduce_rows, whose summation order softmax_rows repeats
@@ -1023,7 +1025,7 @@ def softmax_rows(out: Buffer, inp: Buffer, outer: int, R: int, arg_out: tp.Optio
     assert 0 < R < SOFTMAX_MAX_ROW and inp.size == out.size == outer * R and (arg_out is None or arg_out.size == outer)
     vec = 4 if R % 4 == 0 else 1
     return Launch(f'softmax_rows_v{vec}', (_cdiv(outer, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0), (arg_out, 0)], _u32(outer, R),
-                  bytes_moved=8 * outer * R + (4 * outer if arg_out is not None else 0))
+                  bytes_moved=8 * outer * R + (4 * outer if arg_out is not None else 0), written=(0, 2))
 
 
 def reduce_general(out: Buffer, inp: Buffer, kept, reduced, op: str) -> Launch:
@@ -1178,11 +1180,12 @@ def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: 
     seg    = 1024 * _cdiv(_cdiv(n_rows + 1, 1024), 256)
     table_passes = 1 if operand_is_scalar else 2
     return [
-        Launch('scatter_rows_rank', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(count, 0), (rank, 0), (idx, 0)], params, bytes_moved=12 * n_idx),
+        Launch('scatter_rows_rank', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(count, 0), (rank, 0), (idx, 0)], params, bytes_moved=12 * n_idx,
+               written=(0, 1)),
         Launch('scatter_rows_starts', (_cdiv(n_rows + 1, seg), 1, 1), (1024, 1, 1), [(start, 0), (count, 0)], _u32(n_rows, seg),
                bytes_moved=8 * (n_rows + 1)),
         Launch('scatter_rows_order', (_cdiv(max(n_idx, n_rows), BLOCK), 1, 1), (BLOCK, 1, 1),
-               [(order, 0), (count, 0), (start, 0), (rank, 0), (idx, 0)], params, bytes_moved=16 * n_idx + 4 * n_rows),
+               [(order, 0), (count, 0), (start, 0), (rank, 0), (idx, 0)], params, bytes_moved=16 * n_idx + 4 * n_rows, written=(0, 1)),
         Launch(f'scatter_rows_sum_{kind}_v{vec}', (_cdiv(n_rows, 4), 1, 1), (BLOCK, 1, 1),      #one wave per row
                [(out, 0), (operand, 0), (updates, 0), (start, 0), (order, 0)], params,
                bytes_moved=4 * (n_idx * row_len + n_idx + table_passes * n_rows * row_len)),
@@ -1213,4 +1216,4 @@ def threefry2x32(out0: Buffer, out1: Buffer, key0: Buffer, key1: Buffer, x0: Buf
     vec = 4 if n % 4 == 0 else 1
     return Launch(f'threefry2x32_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                   [(out0, 0), (out1, 0), (key0, 0), (key1, 0), (x0, 0), (x1, 0)], _u32(n, int(key_is_scalar)),
-                  bytes_moved=16 * n)
+                  bytes_moved=16 * n, written=(0, 1))
