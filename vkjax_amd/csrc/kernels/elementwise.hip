@@ -124,14 +124,19 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
         };
 #pragma unroll
         for (int k = 0; k < NS; ++k) {
-            const uint32_t idx = operand_index(k);
+            uint32_t byte = operand_index(k) * 4u;
+            // a single value is fetched by the first lane of the wave alone and handed to the others further down: 64
+            // lanes asking for the same 16 bytes are served one after the other (x * 2 + 1 on 64 M elements ran at
+            // 4.9 TB/s with two such operands, x * s + b with per-column vectors at 5.9). The other lanes' offsets lie
+            // beyond the descriptor's range, which returns zeros without touching memory.
+            if (((flags[k] >> 4) & 3u) == 3u && (threadIdx.x & 63u) != 0u) byte = 0x80000000u;
             // a single value, or a vector over the fastest dimension whose length divides the distance between a thread's
             // vectors: what the thread's first vector loads serves the others too. Their loads go through a descriptor
             // of size 0, which returns zeros without touching memory, so that every vector issues the same instructions.
             const int readable = (u > 0 && (flags[k] & 64u)) ? 0 : (int)nbytes[k];
             const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in[k]), 0, readable, 0x00020000);
-            if constexpr (VEC == 4) raw[k][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 4u, 0, 0);
-            else                    raw[k][u].x = __builtin_amdgcn_raw_buffer_load_b32(rsrc, idx * 4u, 0, 0);
+            if constexpr (VEC == 4) raw[k][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte, 0, 0);
+            else                    raw[k][u].x = __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte, 0, 0);
         }
     }
 
@@ -144,6 +149,8 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     for (int k = 0; k < NS; ++k) {
         const bool is_vec = (flags[k] & 4u) != 0;          // else one value per vector: its first word
         const bool shared = (flags[k] & 64u) != 0;
+        const bool single = ((flags[k] >> 4) & 3u) == 3u;   // what the wave's first lane has loaded is everybody's value
+        const uint32_t from_first_lane = __builtin_amdgcn_readfirstlane(raw[k][0].x);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             u32x4 t = raw[k][u];
@@ -151,6 +158,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
                 t.x = shared ? raw[k][0].x : t.x; t.y = shared ? raw[k][0].y : t.y;
                 t.z = shared ? raw[k][0].z : t.z; t.w = shared ? raw[k][0].w : t.w;
             }
+            t.x = single ? from_first_lane : t.x;
             if constexpr (VEC == 4) {
                 vals[k][u * 4 + 0] = t.x;
                 vals[k][u * 4 + 1] = is_vec ? t.y : t.x;
@@ -246,7 +254,9 @@ __device__ __forceinline__ void ew_affine_body(float* __restrict__ out, const fl
         if (!SKIP || (fl & 2u)) vm[u] = buffer_load_x4(r_mul, c);
         if (!SKIP || (fl & 4u)) va[u] = buffer_load_x4(r_add, c);
     }
-    if (!SKIP || (fl & 16u)) lo = buffer_load_x1(r_floor, 0u);
+    // (the floor is one value: the wave's first lane fetches it for all, see ew_chain_body)
+    if (!SKIP || (fl & 16u)) lo = buffer_load_x1(r_floor, (threadIdx.x & 63u) ? 0x80000000u : 0u);
+    lo = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, lo)));
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         f32x4 y = a[u];

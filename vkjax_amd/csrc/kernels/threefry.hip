@@ -27,7 +27,10 @@ __device__ __forceinline__ void threefry_block(uint32_t k0, uint32_t k1, uint32_
     }
 }
 
-template <int VEC>
+// SCALAR_KEY: one key for all elements (what jax.random passes), fetched through the scalar cache; else a key per
+// element. Two kernels rather than a run-time switch: with both paths in one body the compiler keeps the per-element
+// keys in vector registers and the scalar-key case, the usual one, ran at 4.8-5.2 TB/s instead of 5.7.
+template <int VEC, bool SCALAR_KEY>
 __device__ __forceinline__ void threefry_body(uint32_t* __restrict__ out0, uint32_t* __restrict__ out1,
                                               const uint32_t* __restrict__ key0, const uint32_t* __restrict__ key1,
                                               const uint32_t* __restrict__ in0, const uint32_t* __restrict__ in1,
@@ -44,7 +47,7 @@ __device__ __forceinline__ void threefry_body(uint32_t* __restrict__ out0, uint3
     } else {
         a[0] = in0[e]; b[0] = in1[e];
     }
-    if (P.key_is_scalar) {
+    if constexpr (SCALAR_KEY) {
         const uint32_t s0 = key0[0], s1 = key1[0];
 #pragma unroll
         for (int j = 0; j < VEC; ++j) { ka[j] = s0; kb[j] = s1; }
@@ -65,15 +68,16 @@ __device__ __forceinline__ void threefry_body(uint32_t* __restrict__ out0, uint3
     }
 }
 
-extern "C" __global__ __launch_bounds__(256) void threefry2x32_v1(uint32_t* out0, uint32_t* out1, const uint32_t* key0, const uint32_t* key1,
-                                                                  const uint32_t* in0, const uint32_t* in1, ThreefryParams P) {
-    threefry_body<1>(out0, out1, key0, key1, in0, in1, P);
-}
-// requires n % 4 == 0 and 16-byte aligned data pointers
-extern "C" __global__ __launch_bounds__(256) void threefry2x32_v4(uint32_t* out0, uint32_t* out1, const uint32_t* key0, const uint32_t* key1,
-                                                                  const uint32_t* in0, const uint32_t* in1, ThreefryParams P) {
-    threefry_body<4>(out0, out1, key0, key1, in0, in1, P);
-}
+#define THREEFRY_KERNEL(name, VEC, SCALAR_KEY)                                                                                   \
+    extern "C" __global__ __launch_bounds__(256) void name(uint32_t* out0, uint32_t* out1, const uint32_t* key0, const uint32_t* key1, \
+                                                           const uint32_t* in0, const uint32_t* in1, ThreefryParams P) {          \
+        threefry_body<VEC, SCALAR_KEY>(out0, out1, key0, key1, in0, in1, P);                                                       \
+    }
+THREEFRY_KERNEL(threefry2x32_v1, 1, false)
+THREEFRY_KERNEL(threefry2x32_k_v1, 1, true)
+// the _v4 kernels require n % 4 == 0 and 16-byte aligned data pointers
+THREEFRY_KERNEL(threefry2x32_v4, 4, false)
+THREEFRY_KERNEL(threefry2x32_k_v4, 4, true)
 
 // ---------------------------------------------------------------------------------------------
 // The whole random-bits pipeline in one pass. JAX (legacy counter layout) draws 2h words as
@@ -226,3 +230,4 @@ TF_STREAM_KERNEL(threefry2x32_stream_pairs_v1, 1, TF_PAIRS)
 // the steps are exactly jax.random.uniform's chain, every step with an operand (see threefry_uniform_steps)
 TF_STREAM_KERNEL(threefry2x32_stream_uniform_v4, 4, TF_HALVES, true)
 TF_STREAM_KERNEL(threefry2x32_stream_xor_uniform_v4, 4, TF_XOR, true)
+

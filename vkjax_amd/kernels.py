@@ -1214,6 +1214,6 @@ def scatter_add_general(out: Buffer, indices: Buffer, updates: Buffer, update_wi
 def threefry2x32(out0: Buffer, out1: Buffer, key0: Buffer, key1: Buffer, x0: Buffer, x1: Buffer, key_is_scalar: bool) -> Launch:
     n   = x0.size
     vec = 4 if n % 4 == 0 else 1
-    return Launch(f'threefry2x32_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+    return Launch(f'threefry2x32{"_k" if key_is_scalar else ""}_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                   [(out0, 0), (out1, 0), (key0, 0), (key1, 0), (x0, 0), (x1, 0)], _u32(n, int(key_is_scalar)),
                   bytes_moved=16 * n, written=(0, 1))
