@@ -226,6 +226,25 @@ def test_four_waves_per_tile_kernel():
                 assert [l.kernel for l in launches] == ['conv_gemm_32x32x128_ks4g' if b_general else 'conv_gemm_32x32x128_ks4'], [l.kernel for l in launches]
 
 
+def test_xcd_layouts_of_the_four_waves_per_tile_kernel():
+    '''The tile -> workgroup map of the four-waves-per-tile kernels with the XCDs laid over the tile grid as 8 x 1,
+    4 x 2, 2 x 4 and 1 x 8 rectangles and as row-major ranges, plain and with a sliced contraction: every layout is
+    a permutation of the tiles, so integer-valued products are exact under all of them.'''
+    from vkjax_amd import kernels as K
+    from vkjax_amd import minijax as mj
+    nn, jnp = mj.nn, mj.numpy
+    ints = lambda lo, hi, *shape: rng.randint(lo, hi, size=shape).astype(np.float32)
+    def dense(x, w, b): return nn.relu(jnp.dot(x, w) + b)
+    for m, k, n in ((256, 784, 512), (64, 1024, 256), (128, 300, 96), (32, 512, 256)):
+        args = [ints(-4, 5, m, k), ints(-3, 4, k, n), ints(-9, 9, n)]
+        for xn in (None, 0, 1, 2, 4, 8):
+            for slices in (1, 2):
+                print(f'xcd layout: {m}x{k}x{n}, {xn} columns, {slices} slice(s)', flush=True)
+                with K.overrides(conv_ksplit=True, conv_k_splits=slices, conv_xcd_columns=xn):
+                    _, _, fn = check_against_oracle(dense, args, exact=True)
+                assert list(fn._jaxpr_interpreters.values())[0].launches[0].kernel == 'conv_gemm_32x32x128_ks4'
+
+
 def test_sliced_contractions():
     '''Products with few tiles and a long contraction: blocks of their own sum slices of the contraction (2, 3, 4 and
     7 slices, also slices of unequal length and a last k step that is not full) into one matrix per slice, and an

@@ -63,7 +63,8 @@ struct ConvParams {
                                     // bits 20-24: the steps are, in this order, a subset of
                                     // (acc - vector, * vector, + vector, + full tensor, max(acc, scalar)):
                                     // bit 20+k set = template step k is present;
-                                    // bits 25-28: M tiles per block (at least 1)
+                                    // bits 25-28: M tiles per block (at least 1);
+                                    // bits 29-31: four-waves-per-tile kernels: 0, or 1 + log2 of the number of XCD columns
     uint32_t epi_desc[2];           // 10 bits per step, steps 0-2 in [0], 3-5 in [1]: bits 0-7 opcode * 2 +
                                     // (operand is the left argument), bits 8-9 kind: 1 scalar,
                                     // 2 per-feature vector [N], 3 full tensor laid out like out
@@ -195,11 +196,26 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
             out += (size_t)slice * (size_t)P.M * (size_t)P.N;
         }
     }
-    {
+    // Four-waves-per-tile kernels (products with few tiles, often with the kernel operand as the large one): the host may
+    // ask for the XCDs to be laid over the tile grid as 8 / xn rows of xn columns (flags bits 29-31 hold 1 + log2 xn),
+    // each XCD owning a rectangle of tiles_m / (8 / xn) x tiles_n / xn tiles (both divisible; the host checks). An XCD's
+    // L2 then fetches 1 / (8 / xn) of the rows of A and 1 / xn of the columns of B, instead of a few rows of A and
+    // all of B.
+    const int xcd_code = KSW > 1 ? (int)(P.flags >> 29) : 0;
+    int chunk_m, tile_n;
+    if (xcd_code > 0) {
+        const int xn = 1 << (xcd_code - 1), sub_n = div_small(region.tiles_n, xn);
+        const int x = work & 7, l = work >> 3, xi = x >> (xcd_code - 1), xj = x & (xn - 1);
+        const int sub_m = region.tiles_m >> (4 - xcd_code);                     // tiles_m / (8 / xn)
+        const int lm = div_small(l, sub_n);
+        chunk_m = xi * sub_m + lm;
+        tile_n  = xj * sub_n + (l - lm * sub_n);
+    } else {
         const int total = chunks_m * region.tiles_n, per = total / 8;
         if (per > 0 && work < per * 8) work = (work & 7) * per + (work >> 3);
+        chunk_m = div_small(work, region.tiles_n);
+        tile_n  = work - chunk_m * region.tiles_n;
     }
-    const int chunk_m = div_small(work, region.tiles_n), tile_n = work - chunk_m * region.tiles_n;
     int tile_m0 = chunk_m * chunk, nsub = LEAN ? min(chunk, region.tiles_m - tile_m0) : 1;
     if (m_blocks > 0) {
         tile_m0 = chunk_m * P.m_each + min(chunk_m, P.m_extra);
