@@ -43,8 +43,8 @@ param_matrix = [
     (conv6a, 'conv6a 3x3 window strides=1 + lhs_dilate=2',  [random([15, 67, 42, 11]), random([3, 3, 11, 7])]),
     (conv6b, 'conv6b 3x3 window strides=2 + lhs_dilate=2',  [random([15, 67, 42, 11]), random([3, 3, 11, 7])]),
     #shapes that take the 16-byte-load paths and every tile size
-    (conv2,  'fast 3x3 C64->64 (128x64 tile)',              [random([8, 56, 56, 64]), random([3, 3, 64, 64])]),
-    (conv1,  'fast 1x1 C64->256 (128x128 tile)',            [random([16, 56, 56, 64]), random([1, 1, 64, 256])]),
+    (conv2,  'fast 3x3 C64->64',              [random([8, 56, 56, 64]), random([3, 3, 64, 64])]),
+    (conv1,  'fast 1x1 C64->256',            [random([16, 56, 56, 64]), random([1, 1, 64, 256])]),
     (conv4,  'fast 3x3 s2 C32->64',                         [random([4, 28, 28, 32]), random([3, 3, 32, 64])]),
     (conv4,  'fast 1x1 s2 C128->96 (N not tile multiple)',  [random([3, 14, 14, 128]), random([1, 1, 128, 96])]),
     (conv2,  'generic lhs, fast rhs 7x7 C3->64',            [random([2, 64, 64, 3]), random([7, 7, 3, 64])]),
@@ -109,12 +109,12 @@ def test_reduce_window_matrix(f, desc, args, exact):
     check_against_oracle(f, args, exact=exact, rtol=1e-5, atol=1e-6)
 
 
-TILES = [('128x128', 32), ('128x64', 32), ('64x64', 32), ('64x64', 64), ('32x32', 32), ('32x32', 64)]
+TILES = [('64x64', 32), ('64x64', 64), ('32x32', 32), ('32x32', 64)]
 
 
 @pytest.mark.parametrize('tile,bk', TILES)
 def test_every_tile_and_loader_variant(tile, bk):
-    '''All 30 kernel instantiations: each tile shape and k step with 16-byte (f) or strided (g) loads on
+    '''All 20 kernel instantiations: each tile shape and k step with 16-byte (f) or strided (g) loads on
     either operand, and the lean variant. The ff2 / ff3 cases have Cin % 64 == 0 (tap position kept in
     scalar registers) and a 1x1 unpadded kernel (rows addressed as a flat matrix): they qualify for the
     lean variant and run through both it and the general ff kernel.'''

@@ -223,6 +223,40 @@ def test_binding_repeated_equations_to_one_buffer_changes_no_bit():
             assert_tree_close(y, ytrue, exact=True, what=f'{f.__name__} fuse={fuse}')
 
 
+def test_sorted_scatter_add_adds_in_update_order():
+    '''Rows that receive up to 4096 updates are summed as operand + u(i0) + u(i1) + ... in ascending update number,
+    whatever order the threads ran in: with random float data the result equals numpy's sequential float32
+    accumulation (np.add.at) bit for bit, and a second evaluation gives the same bits. Buckets of 1, 64, 65, 200,
+    1000 and 4096 entries, and one of 6000, which is summed in blocks whose membership may vary: that row is
+    compared within the tolerance of a float32 sum.'''
+    rng = np.random.default_rng(31)
+    rows, cols = 600, 64
+    sizes = {3: 1, 10: 64, 11: 65, 20: 200, 21: 1000, 30: 4096, 40: 6000}
+    idx = np.concatenate([np.full(n, r, np.int32) for r, n in sizes.items()] + [rng.integers(100, rows, size=3000).astype(np.int32)])
+    rng.shuffle(idx)
+    table   = rng.standard_normal((rows, cols)).astype(np.float32)
+    updates = rng.standard_normal((idx.size, cols)).astype(np.float32)
+    expected = table.copy()
+    np.add.at(expected, idx, updates)                          #sequential, in update order, in float32
+    with K.overrides(scatter_sort_threshold=0):
+        fn = vkjax_amd.wrap(lambda t, i, u: mj.numpy.index_add(t, i, u), frontend='minijax')
+        first  = fn(table, idx, updates)
+        second = fn(table, idx, updates)
+    kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+    assert any(k.startswith('scatter_rows_sum') for k in kernels), kernels
+    crowded = 40
+    others = np.arange(rows) != crowded
+    assert np.array_equal(first[others], expected[others])
+    assert np.array_equal(first[others], second[others])
+    assert np.allclose(first[crowded], expected[crowded], rtol=1e-4, atol=1e-3)
+    #integer data: exact everywhere, the crowded row included
+    itable, iupdates = np.round(table * 4).astype(np.int32), np.round(updates * 4).astype(np.int32)
+    iexpected = itable.copy()
+    np.add.at(iexpected, idx, iupdates)
+    with K.overrides(scatter_sort_threshold=0):
+        assert np.array_equal(vkjax_amd.wrap(lambda t, i, u: mj.numpy.index_add(t, i, u), frontend='minijax')(itable, idx, iupdates), iexpected)
+
+
 def test_failed_evaluation_leaves_the_scatter_counters_zero():
     '''The sorted scatter-add counts in an array that every evaluation leaves zero again - if it runs to the end.
     After an evaluation that failed half way the interpreter writes the zeros again, so the next one is right.'''

@@ -783,8 +783,6 @@ __device__ __forceinline__ void conv_gemm_body(float* __restrict__ pool, const C
     CONV_KERNEL(conv_gemm_##tag##_gf, WGM, WGN, TM, TN, BK, false, true, false)   \
     CONV_KERNEL(conv_gemm_##tag##_gg, WGM, WGN, TM, TN, BK, false, false, false)
 
-CONV_TILE(128x128x32, 2, 2, 2, 2, 32)
-CONV_TILE(128x64x32, 2, 2, 2, 1, 32)
 CONV_TILE(64x64x32, 2, 2, 1, 1, 32)
 CONV_TILE(64x64x64, 2, 2, 1, 1, 64)
 CONV_TILE(32x32x32, 1, 1, 1, 1, 32)

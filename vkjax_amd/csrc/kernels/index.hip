@@ -115,11 +115,16 @@ extern "C" __global__ __launch_bounds__(256) void scatter_add_rows(uint32_t* __r
 // wave per table row adds up its updates, in ascending update order, on top of the operand row
 // (or of one value, when the operand is a constant filled with it) and writes the result once.
 // Every update row is read exactly once, the table is written once, and for rows that receive at
-// most 64 updates the sum does not depend on the order in which threads happen to run (rows with
-// more are summed in blocks of 64, each block in ascending order; which updates share a block
-// depends on the order of arrival).
+// most SCATTER_SORTED_MAX updates the sum does not depend on the order in which threads happen to
+// run: it is operand + u(i0) + u(i1) + ... with i0 < i1 < ..., what a sequential loop over the
+// updates computes. (A bucket of at most 64 entries is sorted across the lanes; a larger one is first
+// sorted into the rank array, which nothing needs any more by then, by counting for every entry the
+// entries below it - quadratic, so only up to SCATTER_SORTED_MAX. Rows with more updates are summed
+// in blocks of 64, each block in ascending order; which updates share a block depends on the order
+// of arrival there.)
 // Scratch: count (n_rows words, all zero before and after), start (n_rows + 1), rank and order
 // (n_idx each).
+#define SCATTER_SORTED_MAX 4096u
 struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride, operand_is_scalar, clip; };   // clip: as in ScatterRowsParams
 
 #define SCATTER_DROPPED 0xFFFFFFFFu
@@ -230,6 +235,25 @@ __device__ __forceinline__ uint32_t wave_sort_first(uint32_t e, uint32_t n, uint
     return (uint32_t)__builtin_amdgcn_ds_permute((int)(below << 2), (int)e);
 }
 
+// sorted[s .. e) = order[s .. e) in ascending order, by one wave. Entry x goes to the place given by the number of
+// entries below it (they are distinct); the wave compares 64 of its entries at a time with all of them. The wave
+// reads back what it has written itself: both through the L2 (relaxed device-scope accesses). Kept out of line: it
+// runs for crowded rows only and must not cost the usual path registers.
+__device__ __attribute__((noinline)) void sort_bucket(uint32_t* sorted, const uint32_t* __restrict__ order, uint32_t s, uint32_t e, uint32_t lane) {
+    for (uint32_t p0 = s; p0 < e; p0 += 64u) {
+        const uint32_t own = p0 + lane < e ? order[p0 + lane] : SCATTER_DROPPED;
+        uint32_t below = 0;
+        for (uint32_t c0 = s; c0 < e; c0 += 64u) {
+            const uint32_t other = c0 + lane < e ? order[c0 + lane] : SCATTER_DROPPED;      // (nothing is below a dropped slot's own value)
+#pragma unroll
+            for (uint32_t j = 0; j < 64u; ++j) below += __builtin_amdgcn_readlane(other, j) < own ? 1u : 0u;
+        }
+        if (p0 + lane < e) __hip_atomic_store(sorted + s + below, own, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0);
+}
+
 // out[r, :] = operand[r, :] + sum over the updates i in row r's bucket of updates[i, :]; one wave per row.
 // Measured on 262144 updates of 1 KB into 65536 rows: the launch moves its bytes at the same rate whether a
 // wave takes one row or several with all their loads in flight together, i.e. it is not bound by the chain
@@ -238,7 +262,7 @@ __device__ __forceinline__ uint32_t wave_sort_first(uint32_t e, uint32_t n, uint
 template <int VEC, bool IS_FLOAT>
 __device__ __forceinline__ void scatter_rows_sum_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ operand,
                                                       const uint32_t* __restrict__ updates, const uint32_t* __restrict__ start,
-                                                      const uint32_t* __restrict__ order, const ScatterSortParams& P) {
+                                                      const uint32_t* __restrict__ order, uint32_t* sorted, const ScatterSortParams& P) {
     constexpr uint32_t INFLIGHT = 4;
     typedef uint32_t vec_t __attribute__((ext_vector_type(VEC)));
     const uint32_t lane = threadIdx.x & 63u;
@@ -271,6 +295,9 @@ __device__ __forceinline__ void scatter_rows_sum_body(uint32_t* __restrict__ out
         if (lane < e - s) ent = order[s + lane];
         ent = wave_sort_first(ent, e - s, lane);
     }
+    // A crowded row: the bucket in ascending order, written to sorted[s .. e).
+    const bool presorted = !one_block && e - s <= SCATTER_SORTED_MAX;
+    if (presorted) sort_bucket(sorted, order, s, e, lane);
     for (uint32_t c0 = 0; c0 < P.row_len; c0 += 64u * VEC) {
         const bool live = c0 + lane * VEC < P.row_len;                     // row_len is a multiple of VEC
         const uint32_t c = live ? c0 + lane * VEC : 0u;
@@ -282,8 +309,13 @@ __device__ __forceinline__ void scatter_rows_sum_body(uint32_t* __restrict__ out
         } else {
             for (uint32_t b0 = s; b0 < e; b0 += 64u) {
                 const uint32_t n = min(64u, e - b0);
-                uint32_t block = lane < n ? order[b0 + lane] : SCATTER_DROPPED;
-                block = wave_sort_first(block, n, lane);
+                uint32_t block = SCATTER_DROPPED;
+                if (presorted) {
+                    if (lane < n) block = __hip_atomic_load(sorted + b0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else {
+                    if (lane < n) block = order[b0 + lane];
+                    block = wave_sort_first(block, n, lane);
+                }
                 accumulate(block, n, c, acc);
             }
         }
@@ -293,8 +325,9 @@ __device__ __forceinline__ void scatter_rows_sum_body(uint32_t* __restrict__ out
 
 #define SCATTER_SUM_KERNEL(name, VEC, IS_FLOAT)                                                                   \
     extern "C" __global__ __launch_bounds__(256) void name(uint32_t* out, const uint32_t* operand, const uint32_t* updates, \
-                                                           const uint32_t* start, const uint32_t* order, ScatterSortParams P) { \
-        scatter_rows_sum_body<VEC, IS_FLOAT>(out, operand, updates, start, order, P);                              \
+                                                           const uint32_t* start, const uint32_t* order, uint32_t* sorted,       \
+                                                           ScatterSortParams P) {                                                 \
+        scatter_rows_sum_body<VEC, IS_FLOAT>(out, operand, updates, start, order, sorted, P);                      \
     }
 // the _v4 variants require row_len % 4 == 0 and 16-byte aligned data pointers
 SCATTER_SUM_KERNEL(scatter_rows_sum_f_v1, 1, true)

@@ -540,10 +540,11 @@ CONV_DERIVED_OPS = ('ADD_F', 'SUB_F', 'MUL_F', 'DIV_F', 'MAX_F', 'MIN_F', 'NEG_F
 
 #(tag, BM, BN, threads, resident blocks per CU, relative MFMA efficiency of the tile shape)
 #(efficiencies are measured: TFLOP/s of each tile on large ResNet-50 layers relative to the best)
-CONV_TILES = (('128x128', 128, 128, 256, 2, 0.92), ('128x64', 128, 64, 256, 2, 0.88),
-              ('64x64', 64, 64, 256, 4, 1.00), ('32x32', 32, 32, 64, 16, 0.80))
+#(128 x 128 and 128 x 64 tiles of 2 x 2 waves reached 0.92 and 0.88 of the 64 x 64 tile's rate on large layers and were
+#never the estimate's choice for any shape; they are no longer built)
+CONV_TILES = (('64x64', 64, 64, 256, 4, 1.00), ('32x32', 32, 32, 64, 16, 0.80))
 #k steps each tile shape is built with
-CONV_TILE_BK = {'128x128': (32,), '128x64': (32,), '64x64': (32, 64), '32x32': (32, 64)}
+CONV_TILE_BK = {'64x64': (32, 64), '32x32': (32, 64)}
 
 
 
@@ -1215,8 +1216,8 @@ def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: 
         Launch('scatter_rows_order', (_cdiv(max(n_idx, n_rows), BLOCK), 1, 1), (BLOCK, 1, 1),
                [(order, 0), (count, 0), (start, 0), (rank, 0), (idx, 0)], params, bytes_moved=16 * n_idx + 4 * n_rows, written=(0, 1)),
         Launch(f'scatter_rows_sum_{kind}_v{vec}', (_cdiv(n_rows, 4), 1, 1), (BLOCK, 1, 1),      #one wave per row
-               [(out, 0), (operand, 0), (updates, 0), (start, 0), (order, 0)], params,
-               bytes_moved=4 * (n_idx * row_len + n_idx + table_passes * n_rows * row_len)),
+               [(out, 0), (operand, 0), (updates, 0), (start, 0), (order, 0), (rank, 0)], params,       #(rank: room to sort crowded buckets in)
+               bytes_moved=4 * (n_idx * row_len + n_idx + table_passes * n_rows * row_len), written=(0, 5)),
     ]
 
 
