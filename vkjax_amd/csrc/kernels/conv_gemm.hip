@@ -931,22 +931,32 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
         ho0 = magic_div(m0 - b * HoWo, P.wo_magic, P.wo_shift);
         hi0 = ho0 * P.SH - P.PH;
     };
+    // Which image row and which 16 bytes of it a thread fetches, and where they go in the patch, is the same for every
+    // tile: worked out once, outside the tile loop.
+    int      p_row[NVEC];            // patch row of the thread's q-th vector; PR and above: nothing to fetch
+    uint32_t p_from[NVEC];           // byte offset of the vector behind the patch's first image row
+    int      p_to[NVEC];             // where it goes in the patch (floats)
+#pragma unroll
+    for (int q = 0; q < NVEC; ++q) {
+        const int v = tid + q * 256, r = v / vecs_per_row, c4 = v - r * vecs_per_row;
+        p_row[q]  = r;
+        p_from[q] = (uint32_t)(r * WC + c4 * 4) * 4u;
+        p_to[q]   = r * P.pitch + P.left + c4 * 4;
+    }
     auto request_patch = [&](int t) {
         int b, ho0, hi0;
         patch_geometry(t, b, ho0, hi0);
+        const uint32_t first_row = (uint32_t)((b * P.H + hi0) * WC) * 4u;       // (wraps for rows above the image, which are not fetched)
 #pragma unroll
         for (int q = 0; q < NVEC; ++q) {
-            const int v = tid + q * 256, r = v / vecs_per_row, c4 = v - r * vecs_per_row, hi = hi0 + r;
-            const bool ok = r < PR && (uint32_t)hi < (uint32_t)P.H;
-            pv[q] = buffer_load_x4(x_rsrc, ok ? (uint32_t)(((b * P.H + hi) * P.W) * P.Cin + c4 * 4) * 4u : CONV_OOB);   // zeros outside the image
+            const bool ok = p_row[q] < PR && (uint32_t)(hi0 + p_row[q]) < (uint32_t)P.H;
+            pv[q] = buffer_load_x4(x_rsrc, ok ? first_row + p_from[q] : CONV_OOB);   // zeros outside the image
         }
     };
     auto park_patch = [&]() {
 #pragma unroll
-        for (int q = 0; q < NVEC; ++q) {
-            const int v = tid + q * 256, r = v / vecs_per_row, c4 = v - r * vecs_per_row;
-            if (r < PR) *reinterpret_cast<f32x4*>(&Ps[r * P.pitch + P.left + c4 * 4]) = pv[q];
-        }
+        for (int q = 0; q < NVEC; ++q)
+            if (p_row[q] < PR) *reinterpret_cast<f32x4*>(&Ps[p_to[q]]) = pv[q];
     };
 
     int t = blockIdx.x;
