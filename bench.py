@@ -485,8 +485,16 @@ def main():
     props = hip.Device.get().get_device_properties()
     lean  = args.replays_only
     if args.primitives_only is not None:
+        if args.calibration_copy:
+            import vkjax_amd
+            copy = vkjax_amd.wrap(lambda x: x + 0.0, frontend='minijax')
+            ci, _ = copy._get_or_create_jaxpr_interpreter((np.zeros(64 * 1024 * 1024, np.float32),))
+            ci.replay(1)                                   #the first dispatch of the run: 256 MiB read, 256 MiB written
+            hip.Device.get().sync()
+            del ci, copy
         print(json.dumps({'metric': 'per-primitive HBM GB/s', 'unit': 'GB/s', 'n_gpus': 1, 'dtype': 'f32', 'data': 'synthetic',
-                          'peak_hbm_gbs': PEAK_HBM_GBS, 'primitives': measure_primitives(only=args.primitives_only)}))
+                          'peak_hbm_gbs': PEAK_HBM_GBS, 'replays_per_primitive': {'warm': 10, 'timed': 90},
+                          'primitives': measure_primitives(only=args.primitives_only)}))
         return
 
     head, wrapped, inputs = measure(args.workload, args.steps, args.warmup, batch=args.batch, fuse=not args.no_fuse, graph=args.graph,

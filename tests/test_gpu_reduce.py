@@ -118,3 +118,34 @@ def test_fused_softmax_equals_the_separate_launches(shape):
     unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)(x)
     assert np.array_equal(y, unfused)
     assert np.allclose(y.sum(axis=-1), 1.0, atol=1e-5)
+
+
+def test_means_store_the_quotient_from_the_summing_launch():
+    '''sum / c and sum * c with a single value c behind an unsplit float sum (a mean over rows, over columns, over
+    the spatial positions of an activation) are one launch, reduce_{rows,cols}_fsum_{div,times}; the values are those
+    of the two launches, bit for bit, and of the oracle within the tolerance of a float sum.'''
+    import vkjax_amd
+    x3 = rng.random_sample((6, 7, 7, 64)).astype(np.float32)
+    x2 = rng.random_sample((300, 1000)).astype(np.float32)
+    cases = [('global average', lambda x: jnp.mean(x, axis=(1, 2)), [x3], 'reduce_cols_fsum_div_v4'),
+             ('mean over rows', lambda x: jnp.mean(x, axis=1), [x2], 'reduce_rows_fsum_div_v4'),
+             ('mean over columns', lambda x: jnp.mean(x, axis=0), [x2[:64, :96]], 'reduce_cols_fsum_div_v4'),
+             ('odd width', lambda x: jnp.mean(x, axis=1), [x2[:, :999].copy()], 'reduce_rows_fsum_div_v1'),
+             ('sum times a value', lambda x, c: jnp.sum(x, axis=0) * c, [x2[:64, :96], np.float32(0.125)], 'reduce_cols_fsum_times_v4'),
+             ('a value times the sum', lambda x, c: c * jnp.sum(x, axis=1), [x2, np.float32(3.0)], 'reduce_rows_fsum_times_v4'),
+             ('sum divided by an argument', lambda x, c: jnp.sum(x, axis=1) / c, [x2, np.float32(7.0)], 'reduce_rows_fsum_div_v4')]
+    for name, f, args, kernel in cases:
+        print(f'case: {name}', flush=True)
+        y, _, fn = check_against_oracle(f, args, rtol=1e-5, atol=0)
+        kernels = [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
+        assert kernels == [kernel], kernels
+        unfused = vkjax_amd.wrap(f, frontend='minijax', fuse=False)
+        assert np.array_equal(y, unfused(*args))
+        assert len(list(unfused._jaxpr_interpreters.values())[0].launches) == 2
+    #not taken over: a value divided by the sum, a sum that something else reads as well, a sum split into ranges
+    for name, f, args, launches in [('c / sum', lambda x, c: c / jnp.sum(x, axis=1), [x2, np.float32(7.0)], 2),
+                                    ('two readers', lambda x: (jnp.sum(x, axis=1) / 3.0, jnp.sum(x, axis=1) + 1.0), [x2], 3),
+                                    ('split sum', lambda x: jnp.mean(x, axis=1), [rng.random_sample((2, 1 << 18)).astype(np.float32)], 3)]:
+        print(f'case: {name}', flush=True)
+        _, _, fn = check_against_oracle(f, args, rtol=1e-5, atol=0)
+        assert len(list(fn._jaxpr_interpreters.values())[0].launches) == launches

@@ -76,8 +76,18 @@ __device__ __forceinline__ uint32_t red_step(uint32_t op, uint32_t ty, uint32_t 
     else return red_combine(op, ty, a, b);
 }
 
-template <int VEC, int MODE>
-__device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P) {
+// POST (float sums only): the finished sum is divided (1) or multiplied (2) by the single value at `post` before it is
+// stored - the step behind a mean, with the rounding of the element-wise kernel's own division / multiplication.
+template <int POST>
+__device__ __forceinline__ uint32_t reduce_post(uint32_t sum, const uint32_t* __restrict__ post) {
+    if constexpr (POST == 1) return f2u(u2f(sum) / u2f(post[0]));
+    else if constexpr (POST == 2) return f2u(u2f(sum) * u2f(post[0]));
+    else return sum;
+}
+
+template <int VEC, int MODE, int POST = 0>
+__device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P,
+                                                 const uint32_t* __restrict__ post = nullptr) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint64_t unit = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
     if (unit >= (uint64_t)P.outer * P.nsplit) return;                 // whole wave leaves together
@@ -184,7 +194,7 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
             a = red_step<MODE>(P.op, P.type, a, __shfl_xor(a, s, 64));
         }
     }
-    if (lane == 0) out[unit] = is_arg ? (best_i == 0xFFFFFFFFu ? 0u : best_i) : a;
+    if (lane == 0) out[unit] = is_arg ? (best_i == 0xFFFFFFFFu ? 0u : best_i) : reduce_post<POST>(a, post);
 }
 
 // PRO: what is reduced. 0 the operand itself; 1 its product with a second array of the same shape;
@@ -194,9 +204,10 @@ __device__ __forceinline__ void reduce_rows_body(uint32_t* __restrict__ out, con
 enum { PRO_NONE = 0, PRO_MUL = 1, PRO_MULV = 2, PRO_NEG = 3 };
 
 // `block`: index of this workgroup in the reduction's own grid
-template <int VEC, int MODE, int PRO = PRO_NONE>
+template <int VEC, int MODE, int PRO = PRO_NONE, int POST = 0>
 __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ReduceParams& P,
-                                                 const uint32_t* __restrict__ in2 = nullptr, const uint32_t block = blockIdx.x) {
+                                                 const uint32_t* __restrict__ in2 = nullptr, const uint32_t block = blockIdx.x,
+                                                 const uint32_t* __restrict__ post = nullptr) {
     __shared__ uint32_t s_val[256 * VEC];
     __shared__ uint32_t s_idx[256 * VEC];
     const uint32_t TI = P.TI, TR = 256u / TI;
@@ -295,7 +306,8 @@ __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, con
     if (tr == 0 && i < P.inner) {
         uint32_t* dst = out + ((uint64_t)o * P.nsplit + sp) * P.inner + i;
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) dst[j] = is_arg ? (s_idx[tid * VEC + j] == 0xFFFFFFFFu ? 0u : s_idx[tid * VEC + j]) : s_val[tid * VEC + j];
+        for (int j = 0; j < VEC; ++j)
+            dst[j] = is_arg ? (s_idx[tid * VEC + j] == 0xFFFFFFFFu ? 0u : s_idx[tid * VEC + j]) : reduce_post<POST>(s_val[tid * VEC + j], post);
     }
 }
 
@@ -307,6 +319,12 @@ __device__ __forceinline__ void reduce_cols_body(uint32_t* __restrict__ out, con
 #define REDUCE_COLS_PROLOGUE_KERNELS(tag, PRO)                                                                                 \
     extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v1(uint32_t* out, const uint32_t* in, const uint32_t* in2, ReduceParams P) { reduce_cols_body<1, 0, PRO>(out, in, P, in2); } \
     extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v4(uint32_t* out, const uint32_t* in, const uint32_t* in2, ReduceParams P) { reduce_cols_body<4, 0, PRO>(out, in, P, in2); }
+// float sums followed by a division or a multiplication by one value (a mean): unsplit reductions only
+#define REDUCE_POST_KERNELS(tag, POST)                                                                                         \
+    extern "C" __global__ __launch_bounds__(256) void reduce_rows_fsum_##tag##_v1(uint32_t* out, const uint32_t* in, const uint32_t* post, ReduceParams P) { reduce_rows_body<1, 0, POST>(out, in, P, post); } \
+    extern "C" __global__ __launch_bounds__(256) void reduce_rows_fsum_##tag##_v4(uint32_t* out, const uint32_t* in, const uint32_t* post, ReduceParams P) { reduce_rows_body<4, 0, POST>(out, in, P, post); } \
+    extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v1(uint32_t* out, const uint32_t* in, const uint32_t* post, ReduceParams P) { reduce_cols_body<1, 0, PRO_NONE, POST>(out, in, P, nullptr, blockIdx.x, post); } \
+    extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_##tag##_v4(uint32_t* out, const uint32_t* in, const uint32_t* post, ReduceParams P) { reduce_cols_body<4, 0, PRO_NONE, POST>(out, in, P, nullptr, blockIdx.x, post); }
 // Several small, mutually independent float column sums in ONE launch (the second stages of split sums, the
 // per-channel sums of small layers): one table entry per sum, workgroup b belongs to the last entry whose
 // first_block is <= b, as in ew_chain_batch.
@@ -340,6 +358,8 @@ extern "C" __global__ __launch_bounds__(256) void reduce_cols_fsum_batch_v4(cons
 REDUCE_COLS_PROLOGUE_KERNELS(mul, PRO_MUL)
 REDUCE_COLS_PROLOGUE_KERNELS(mulv, PRO_MULV)
 REDUCE_COLS_PROLOGUE_KERNELS(neg, PRO_NEG)
+REDUCE_POST_KERNELS(div, 1)
+REDUCE_POST_KERNELS(times, 2)
 REDUCE_KERNELS(fsum, 0)
 REDUCE_KERNELS(fmax, 1)
 // Any other combination of operation and element type. The combine is selected once per launch: every case calls the

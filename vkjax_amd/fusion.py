@@ -287,6 +287,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
     ops = fuse_softmax(ops, bufferpool, outvars)
     ops = fuse_scale_relu_backward(ops, bufferpool, outvars)
     ops = fuse_reduce_prologues(ops, bufferpool, outvars)
+    ops = fuse_reduce_scales(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
     ops = fuse_index_wrap(ops, bufferpool, outvars)
     ops = fuse_dense_softmax(ops, bufferpool, outvars)
@@ -470,6 +471,51 @@ def fuse_reduce_prologues(ops, bufferpool, outvars):
         ch.out._placeholder.elided = True
         removed.add(w)
         replacement[i] = fused
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
+
+
+def fuse_reduce_scales(ops, bufferpool, outvars):
+    '''A float sum (one launch: not split into ranges) whose result is read once, by `sum / c` or `sum * c` with a
+    single value c - a mean - stores the quotient / product itself: the element-wise launch behind it goes away. The
+    division is the one the element-wise kernel would have made (same operands, same rounding).'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    removed, replacement = set(), {}
+    for i, R in enumerate(ops):
+        if R.meta is None or R.meta[0] != 'reduce' or i + 1 >= len(ops):
+            continue
+        _, out, inp, outer, rows, inner, name, partial, nsplit = R.meta
+        if name != 'reduce_sum' or nsplit != 1 or inp.dtype != 'float32' or uses[pid(out)] != 1:
+            continue
+        #the reader: the next launch that reads the sum (nothing in between touches it, it has one use)
+        C = next((j for j in range(i + 1, len(ops)) if any(b._placeholder is out._placeholder for b in _reads(ops[j]))), None)
+        if C is None or ops[C].chain is None:
+            continue
+        #the sum is taken where its reader stood: its operand must still hold the same values there
+        if any(w._placeholder is inp._placeholder for j in range(i + 1, C) for w in _may_write(ops[j])):
+            continue
+        ch = ops[C].chain
+        if len(ch.steps) != 1 or ch.steps[0].operand is None:
+            continue
+        step = ch.steps[0]
+        total, o = ch.first, step.operand
+        if step.op == EW['MUL_F'] and o.buffer._placeholder is out._placeholder:
+            total, o = o, ch.first                              #c * sum: the product is the same number
+        elif step.op == EW['DIV_F'] and step.operand_left:
+            continue                                            #c / sum
+        kind = 'div' if step.op == EW['DIV_F'] else 'times' if step.op == EW['MUL_F'] else None
+        if (kind is None or total.buffer._placeholder is not out._placeholder or not _is_full_contiguous_any_shape(total, ch.shape)
+                or o.buffer.size != 1 or o.offset != 0 or ch.out.size != out.size):
+            continue
+        launch = K.reduce(ch.out, inp, outer, rows, inner, name, None, 1, post=(kind, o.buffer))[0]
+        fused  = Op(_label(R, ops[C]), launch=launch, meta=None)
+        fused.index = ops[C].index
+        for b in (inp, o.buffer):
+            b.accesses.append(ops[C].index)
+        out._placeholder.elided = True
+        removed.add(i)
+        replacement[C] = fused
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
 
 

@@ -980,14 +980,21 @@ def plan_reduce_splits(outer: int, R: int, inner: int, op: str, compute_units: i
 
 
 def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str, nsplit: int, in_offset_ok=True,
-                   prologue: tp.Optional[tp.Tuple[str, tp.Optional[Buffer]]] = None) -> Launch:
+                   prologue: tp.Optional[tp.Tuple[str, tp.Optional[Buffer]]] = None,
+                   post: tp.Optional[tp.Tuple[str, Buffer]] = None) -> Launch:
     ty   = _RTYPE[inp.dtype]
     mode = {('reduce_sum', 0): 'fsum', ('reduce_max', 0): 'fmax', ('argmax', 0): 'fargmax', ('argmin', 0): 'fargmin'}.get((op, ty), 'any')
     r_chunk = _cdiv(_cdiv(R, nsplit), 4) * 4
     nsplit  = _cdiv(R, r_chunk)
+    if post is not None:
+        #('div' | 'times', one value): applied to every finished float sum of an unsplit reduction
+        assert mode == 'fsum' and nsplit == 1 and prologue is None and post[0] in ('div', 'times') and post[1].size == 1
     if inner == 1:
         vec = 4 if R % 4 == 0 else 1
         params = _u32(outer, R, 1, RED[op], ty, r_chunk, nsplit, 0)
+        if post is not None:
+            return Launch(f'reduce_rows_fsum_{post[0]}_v{vec}', (_cdiv(outer * nsplit, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0), (post[1], 0)],
+                          params, bytes_moved=4 * (outer * R + outer * nsplit)), nsplit
         return Launch(f'reduce_rows_{mode}_v{vec}', (_cdiv(outer * nsplit, 4), 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
                       bytes_moved=4 * (outer * R + outer * nsplit)), nsplit
     vec = 4 if inner % 4 == 0 else 1
@@ -1010,16 +1017,20 @@ def _reduce_launch(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op:
         extra = 0 if second is None else second.size
         return Launch(f'reduce_cols_fsum_{kind}_v{vec}', (blocks, 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0), (second, 0)], params,
                       bytes_moved=4 * (outer * R * inner + outer * nsplit * inner + extra)), nsplit
+    if post is not None:
+        return Launch(f'reduce_cols_fsum_{post[0]}_v{vec}', (blocks, 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0), (post[1], 0)], params,
+                      bytes_moved=4 * (outer * R * inner + outer * nsplit * inner)), nsplit
     return Launch(f'reduce_cols_{mode}_v{vec}', (blocks, 1, 1), (BLOCK, 1, 1), [(out, 0), (inp, 0)], params,
                   bytes_moved=4 * (outer * R * inner + outer * nsplit * inner)), nsplit
 
 
 def reduce(out: Buffer, inp: Buffer, outer: int, R: int, inner: int, op: str,
-           partial: tp.Optional[Buffer] = None, nsplit: int = 1, prologue=None) -> tp.List[Launch]:
+           partial: tp.Optional[Buffer] = None, nsplit: int = 1, prologue=None, post=None) -> tp.List[Launch]:
     '''[outer, R, inner] -> [outer, inner]. With nsplit > 1, `partial` (outer * nsplit * inner words) receives
-    the per-range results of a first launch and a second launch reduces them. `prologue`: see _reduce_launch.'''
+    the per-range results of a first launch and a second launch reduces them. `prologue`, `post`: see _reduce_launch.'''
     if nsplit <= 1:
-        return [_reduce_launch(out, inp, outer, R, inner, op, 1, prologue=prologue)[0]]
+        return [_reduce_launch(out, inp, outer, R, inner, op, 1, prologue=prologue, post=post)[0]]
+    assert post is None
     first, nsplit = _reduce_launch(partial, inp, outer, R, inner, op, nsplit, prologue=prologue)
     if nsplit == 1:
         return [_reduce_launch(out, inp, outer, R, inner, op, 1, prologue=prologue)[0]]
