@@ -428,10 +428,10 @@ def test_repeated_equations_are_evaluated_once():
     fn, make = W.WORKLOADS['gather_scatter']
     closed = mj.make_jaxpr(fn)(*make())
     kernels = lambda **kw: [l.kernel for l in JaxprInterpreter(closed, plan_only=True, **kw).launches]
-    assert len(kernels()) == 6 and len(kernels(fuse=False)) == 8          #(fused: x + n, x < 0 and the select in one pass)
+    assert len(kernels()) == 5 and len(kernels(fuse=False)) == 8          #(fused: the gather and the scatter-add read the indices as they are and add n to the negative ones)
     from vkjax_amd import kernels as K
     with K.overrides(reuse_equal_equations=False):
-        assert len(kernels()) == 7 and len(kernels(fuse=False)) == 11
+        assert len(kernels()) == 5 and len(kernels(fuse=False)) == 11
     with pytest.raises(TypeError, match='unknown choice'):
         with K.overrides(no_such_choice=1):
             pass
@@ -499,9 +499,9 @@ def test_index_modes():
     for mode, fill in (('clip', None), ('promise_in_bounds', None), (None, None), ('fill', 0x7FC00000), ('FILL_OR_DROP', 0x7FC00000)):
         closed = mj.make_jaxpr(lambda x, i: lax.gather(x, i, dn, (1, 4), mode=mode))(x, idx)
         (launch,) = JaxprInterpreter(closed, plan_only=True).launches
-        assert np.frombuffer(launch.params, np.uint32)[-2:].tolist() == [int(fill is not None), fill or 0], mode
+        assert np.frombuffer(launch.params, np.uint32)[-3:].tolist() == [int(fill is not None), fill or 0, 0], mode       #(fill flag, fill word, wrap)
     closed = mj.make_jaxpr(lambda x, i: lax.gather(x.astype(np.int32), i, dn, (1, 4), mode='fill', fill_value=-7))(x, idx)
-    assert np.frombuffer(JaxprInterpreter(closed, plan_only=True).launches[-1].params, np.int32)[-2:].tolist() == [1, -7]
+    assert np.frombuffer(JaxprInterpreter(closed, plan_only=True).launches[-1].params, np.int32)[-3:].tolist() == [1, -7, 0]
     sd = lax.ScatterDimensionNumbers(update_window_dims=(1,), inserted_window_dims=(0,), scatter_dims_to_operand_dims=(0,))
     for mode, clip in (('clip', 1), ('drop', 0), (None, 0), ('promise_in_bounds', 0)):
         closed = mj.make_jaxpr(lambda x, i, u: lax.scatter_add(x, i, u, sd, mode=mode))(x, idx, upd)

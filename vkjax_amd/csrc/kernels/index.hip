@@ -12,7 +12,9 @@
 
 #define IDX_MAX_RANK 6
 
-struct GatherRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride, fill_mode, fill_bits; };
+// wrap: added to negative indices first (0: nothing) - the normalisation `select(i < 0, i + n, i)` that tracing puts in
+// front of an indexing operation, taken over from an element-wise launch of its own
+struct GatherRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride, fill_mode, fill_bits, wrap; };
 
 // out[i, :] = table[clamp(idx[i*idx_stride]), :]; with fill_mode, rows outside the table read as fill_bits instead
 // (jax's GatherScatterMode.FILL_OR_DROP)
@@ -24,6 +26,7 @@ __device__ __forceinline__ void gather_rows_body(uint32_t* __restrict__ out, con
     if (q >= (uint64_t)P.n_idx * vpr) return;
     const uint32_t i = (uint32_t)(q / vpr), c = (uint32_t)(q - (uint64_t)i * vpr) * VEC;
     int32_t r = idx[(uint64_t)i * P.idx_stride];
+    r = r < 0 ? (int32_t)((uint32_t)r + P.wrap) : r;
     uint32_t* dst = out + (uint64_t)i * P.row_len + c;
     if (P.fill_mode && (r < 0 || r >= (int32_t)P.n_rows)) {
         if constexpr (VEC == 4) *reinterpret_cast<u32x4*>(dst) = u32x4{P.fill_bits, P.fill_bits, P.fill_bits, P.fill_bits};
@@ -125,7 +128,7 @@ extern "C" __global__ __launch_bounds__(256) void scatter_add_rows(uint32_t* __r
 // Scratch: count (n_rows words, all zero before and after), start (n_rows + 1), rank and order
 // (n_idx each).
 #define SCATTER_SORTED_MAX 4096u
-struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride, operand_is_scalar, clip; };   // clip: as in ScatterRowsParams
+struct ScatterSortParams { uint32_t n_idx, row_len, n_rows, idx_stride, operand_is_scalar, clip, wrap; };   // clip: as in ScatterRowsParams; wrap: as in GatherRowsParams
 
 #define SCATTER_DROPPED 0xFFFFFFFFu
 
@@ -136,6 +139,7 @@ extern "C" __global__ __launch_bounds__(256) void scatter_rows_rank(uint32_t* __
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= P.n_idx) return;
     int32_t r = idx[(uint64_t)i * P.idx_stride];
+    r = r < 0 ? (int32_t)((uint32_t)r + P.wrap) : r;
     if (P.clip) r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
     uint32_t k = SCATTER_DROPPED;
     if (r >= 0 && r < (int32_t)P.n_rows) k = atomicAdd(count + r, 1u);
@@ -206,6 +210,7 @@ extern "C" __global__ __launch_bounds__(256) void scatter_rows_order(uint32_t* _
     const uint32_t k = rank[i];
     if (k == SCATTER_DROPPED) return;
     int32_t r = idx[(uint64_t)i * P.idx_stride];
+    r = r < 0 ? (int32_t)((uint32_t)r + P.wrap) : r;
     if (P.clip) r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
     order[start[r] + k] = i;
 }

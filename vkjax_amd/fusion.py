@@ -290,6 +290,7 @@ def fuse_ops(all_ops, bufferpool, outvars):
     ops = fuse_reduce_scales(ops, bufferpool, outvars)
     ops = fuse_derived_epilogue_operands(ops, bufferpool, outvars)
     ops = fuse_index_wrap(ops, bufferpool, outvars)
+    ops = fold_index_wrap(ops, bufferpool, outvars)
     ops = fuse_dense_softmax(ops, bufferpool, outvars)
     ops = remove_dead_ops(ops, bufferpool, outvars)
     return batch_small_chains(ops)
@@ -386,6 +387,48 @@ def fuse_index_wrap(ops, bufferpool, outvars):
         pick.operand.buffer._placeholder.elided = True
         removed.add(a)
         replacement[i] = fused
+    return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
+
+
+def fold_index_wrap(ops, bufferpool, outvars):
+    '''The normalised copy of an index array, `select(i < 0, i + n, i)` (one launch after fuse_index_wrap), is not made
+    when everything that reads it is a row gather or a sorted row scatter-add: those kernels read the indices as they
+    are and add n to the negative ones themselves.'''
+    from .ops import Op
+    uses = _use_counts(ops, bufferpool, outvars)
+    pid  = lambda b: id(b._placeholder)
+    removed, replacement = set(), {}
+    for i, op in enumerate(ops):
+        ch = op.chain
+        if ch is None or len(ch.steps) != 1 or ch.steps[0].op != EW['WRAP_I'] or ch.steps[0].operand_left:
+            continue
+        o = ch.steps[0].operand
+        amount = getattr(o.buffer, 'constant_value', None) if o is not None and all(st == 0 for st in o.strides) else None
+        if (amount is None or np_prod(amount.shape) != 1 or not _is_full_contiguous_any_shape(ch.first, ch.shape)
+                or str(ch.first.buffer.dtype) != 'int32' or str(ch.out.dtype) != 'int32'):
+            continue
+        readers = [j for j in range(len(ops)) if j != i and any(b._placeholder is ch.out._placeholder for b in _reads(ops[j]))]
+        if not readers or len(readers) != uses[pid(ch.out)] or min(readers) < i:
+            continue                                           #(also a result of the program: its uses count two more)
+        ok = True
+        for j in readers:
+            r = replacement.get(j, ops[j])
+            where = K.INDEX_WRAP_KERNELS.get(r.launch.kernel) if r.chain is None and r.conv is None else None
+            places = [k for k, (b, _) in enumerate(r.launch.buffers) if b is not None and b._placeholder is ch.out._placeholder] if where else []
+            ok = ok and where is not None and places == [where[0]]
+        #the raw indices must still be what they were where the readers run
+        last = max(readers)
+        if not ok or any(w._placeholder is ch.first.buffer._placeholder for j in range(i + 1, last + 1) for w in _may_write(ops[j])):
+            continue
+        for j in readers:
+            r = replacement.get(j, ops[j])
+            launch = K.with_wrapped_index(r.launch, ch.first.buffer, ch.first.offset * 4, int(amount.reshape(-1)[0]))
+            new = Op(_label(op, r), launch=launch, meta=r.meta)
+            new.index = r.index
+            ch.first.buffer.accesses.append(r.index)
+            replacement[j] = new
+        ch.out._placeholder.elided = True
+        removed.add(i)
     return [replacement.get(i, op) for i, op in enumerate(ops) if i not in removed]
 
 

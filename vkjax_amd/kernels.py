@@ -1177,7 +1177,7 @@ def gather_rows(out: Buffer, table: Buffer, idx: Buffer, n_idx: int, row_len: in
     vec = 4 if row_len % 4 == 0 else 1
     total = n_idx * (row_len // vec)
     return Launch(f'gather_rows_v{vec}', (_cdiv(total, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (table, 0), (idx, 0)],
-                  _u32(n_idx, row_len, n_rows, idx_stride, int(fill is not None), fill or 0), bytes_moved=4 * (2 * n_idx * row_len + n_idx))
+                  _u32(n_idx, row_len, n_rows, idx_stride, int(fill is not None), fill or 0, 0), bytes_moved=4 * (2 * n_idx * row_len + n_idx))
 
 
 def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, collapsed, start_index_map, slice_sizes,
@@ -1194,6 +1194,20 @@ def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, c
                   int(fill is not None), fill or 0)
     return Launch('gather_general', (_cdiv(out.size, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (operand, 0), (indices, 0)],
                   params, bytes_moved=4 * (2 * out.size + indices.size))
+
+
+#kernels that can add a value to negative indices themselves: position of the index array among their arguments, and the
+#byte offset of the `wrap` field in their parameter block
+INDEX_WRAP_KERNELS = {'gather_rows_v1': (2, 24), 'gather_rows_v4': (2, 24), 'scatter_rows_rank': (2, 24), 'scatter_rows_order': (4, 24)}
+
+
+def with_wrapped_index(launch: Launch, raw: Buffer, raw_byte_offset: int, amount: int) -> Launch:
+    '''`launch` reading the raw index array `raw` instead of its normalised copy, adding `amount` to negative indices itself.'''
+    position, field = INDEX_WRAP_KERNELS[launch.kernel]
+    assert launch.params[field:field + 4] == _u32(0)
+    buffers = list(launch.buffers)
+    buffers[position] = (raw, buffers[position][1] + raw_byte_offset)
+    return launch._replace(buffers=buffers, params=launch.params[:field] + _u32(amount) + launch.params[field + 4:])
 
 
 def scatter_add_rows(out: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_len: int, n_rows: int, idx_stride: int = 1,
@@ -1213,7 +1227,7 @@ def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: 
     each), then one wave per row sums its bucket. `operand` is the table, or one word when the table is a constant
     filled with a single value.'''
     assert count.size == n_rows and start.size == n_rows + 1 and rank.size == n_idx and order.size == n_idx
-    params = _u32(n_idx, row_len, n_rows, idx_stride, int(operand_is_scalar), int(clip))
+    params = _u32(n_idx, row_len, n_rows, idx_stride, int(operand_is_scalar), int(clip), 0)
     vec    = 4 if row_len % 4 == 0 else 1
     kind   = 'f' if out.dtype == np.float32 else 'i'
     #bucket starts: at most 256 workgroups, each scanning a segment of whole 1024-word tiles
