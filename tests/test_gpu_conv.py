@@ -325,8 +325,8 @@ def test_mixed_tiling():
 
 
 def test_stem_kernel_for_few_input_features():
-    '''conv_gemm_stem_7x22: seven kernel rows whose KW * Cin values (21 or 22) are read from a patch of image rows
-    in LDS. 7 x 7 on 3 features with stride 2 and padding 3 (the ResNet stem), stride 1, a 7 x 11 kernel on 2
+    '''conv_gemm_stem_7x22 and its 512-thread form _m128: seven kernel rows whose KW * Cin values (21 or 22) are read from a
+    patch of image rows in LDS. 7 x 7 on 3 features with stride 2 and padding 3 (the ResNet stem), stride 1, a 7 x 11 kernel on 2
     features, fewer than 64 output features, images that are not square, several tiles per block (more tiles than
     the grid has blocks), with a batch-norm + ReLU epilogue, bias + ReLU and none; integer-valued data, so every
     result is exact.'''
@@ -363,15 +363,21 @@ def test_stem_kernel_for_few_input_features():
              (conv(2, ((3, 3), (5, 5))), [ints(-4, 5, 2, 16, 128, 2), ints(-3, 4, 7, 11, 2, 24)]),
              (conv(2, ((0, 2), (3, 4))), [ints(-4, 5, 1, 132, 128, 3), ints(-3, 4, 7, 7, 3, 64)]),
              (bn_relu(2, p3), [ints(-4, 5, 18, 128, 128, 3), ints(-3, 4, 7, 7, 3, 64), vec(-5, 5, 64), np.ones(64, np.float32), vec(1, 4, 64) * 2, vec(-9, 9, 64)])]
+    seen = set()
     for f, args in cases:
         print(f'stem kernel: {[a.shape for a in args]}', flush=True)
         for fuse in (True, False):
-            _, _, fn = check_against_oracle(f, args, exact=True, fuse=fuse)
-            launches = list(fn._jaxpr_interpreters.values())[0].launches
-            kernels = [l.kernel for l in launches if l.kernel.startswith('conv_gemm')]
-            assert kernels == ['conv_gemm_stem_7x22'], kernels
-            if fuse and 'and_activated' in f.__name__:
-                assert len(launches) == 1, [l.kernel for l in launches]       #both results from the one launch
+            #tiles of 128 output positions (512 threads) where the sizes allow them, and the 64-position tiles everywhere
+            for tile in (None, 64):
+                with K.overrides(conv_stem=tile):
+                    _, _, fn = check_against_oracle(f, args, exact=True, fuse=fuse)
+                launches = list(fn._jaxpr_interpreters.values())[0].launches
+                kernels = [l.kernel for l in launches if l.kernel.startswith('conv_gemm')]
+                assert kernels in (['conv_gemm_stem_7x22'], ['conv_gemm_stem_7x22_m128']) and (tile is None or kernels == ['conv_gemm_stem_7x22']), kernels
+                seen.add(kernels[0])
+                if fuse and 'and_activated' in f.__name__:
+                    assert len(launches) == 1, [l.kernel for l in launches]       #both results from the one launch
+    assert seen == {'conv_gemm_stem_7x22', 'conv_gemm_stem_7x22_m128'}
     #a shape it does not take falls back to the general kernel
     _, _, fn = check_against_oracle(conv(2, p3), [ints(-4, 5, 2, 30, 26, 3), ints(-3, 4, 7, 7, 3, 64)], exact=True)
     assert [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches] == ['conv_gemm_64x64x32_gf']

@@ -112,7 +112,7 @@ def test_kernel_argument_layouts_match_the_structs():
     sizes['ConvParams'] += sizes['ConvDerived']
     sizes['ConvStemParams'] += sizes['ConvDerived']
     assert launches['EwAffineParams'].kernel == 'ew_affine_v4' and len(launches['EwAffineParams'].buffers) == 10
-    assert launches['ConvStemParams'].kernel == 'conv_gemm_stem_7x22' and launches['DenseRowsParams'].kernel == 'dense_rows_n16'
+    assert launches['ConvStemParams'].kernel in ('conv_gemm_stem_7x22', 'conv_gemm_stem_7x22_m128') and launches['DenseRowsParams'].kernel == 'dense_rows_n16'
     assert len(launches['DenseRowsParams'].buffers) == 3 + K.CONV_MAX_EPI
     for struct, launch in launches.items():
         assert len(launch.params) == sizes[struct], (struct, len(launch.params), sizes[struct])

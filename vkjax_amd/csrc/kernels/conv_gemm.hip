@@ -843,18 +843,20 @@ struct ConvStemParams {
     uint32_t howo_magic, howo_shift, wo_magic, wo_shift;
 };
 
-template <int KH, int RLP, int PR, int NVEC>
+// NWM: 32-row sub-tiles of a block's tile (2: 64 output positions, 256 threads; 4: 128 positions, 512 threads - the
+// kernel and the patch take the same room in LDS either way, so the larger block brings twice the waves per CU).
+template <int KH, int RLP, int PR, int NVEC, int NWM = 2>
 __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
                                                const ConvEpiPtrs& epi, const ConvDerivedPtrs& Dp, const ConvStemParams& P,
                                                const ConvDerived& Dk, float* __restrict__ Ws, float* __restrict__ Ps, float* __restrict__ Es) {
-    constexpr int BN = 64, LDB = BN + 4, G = RLP / 2;
+    constexpr int BN = 64, LDB = BN + 4, G = RLP / 2, BM = 32 * NWM, NT = 128 * NWM;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, half = lane >> 5;
     const int RL = P.KW * P.Cin, WC = P.W * P.Cin, vecs_per_row = WC >> 2, HoWo = P.Ho * P.Wo;
     const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, P.x_bytes), w_rsrc = make_rsrc(w, P.w_bytes), o_rsrc = make_rsrc(out, P.out_bytes);
 
     // the kernel: Ws[ky * RLP + j][n] = w[ky, j, n] for j < KW * Cin, zero behind
-    for (int e = tid; e < KH * RLP * (BN / 4); e += 256) {
+    for (int e = tid; e < KH * RLP * (BN / 4); e += NT) {
         const int row = e / (BN / 4), n4 = (e - row * (BN / 4)) * 4, ky = row / RLP, j = row - ky * RLP;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
         if (j < RL) {
@@ -868,7 +870,7 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
         *reinterpret_cast<f32x4*>(&Ws[row * LDB + n4]) = v;
     }
     // the borders of the patch rows stay zero
-    for (int e = tid; e < PR * P.pitch; e += 256) {
+    for (int e = tid; e < PR * P.pitch; e += NT) {
         const int c = e % P.pitch;
         if (c < P.left || c >= P.left + WC) Ps[e] = 0.f;
     }
@@ -922,11 +924,11 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
             if (e < nepi) Es[e * BN + tid] = e_reg[e];
     }
 
-    const int tiles = P.M / 64;
+    const int tiles = P.M / BM;
     // the image rows of the patch of tile t: requested into registers, written to LDS later
     f32x4 pv[NVEC];
     auto patch_geometry = [&](int t, int& b, int& ho0, int& hi0) {
-        const int m0 = t * 64;
+        const int m0 = t * BM;
         b = magic_div(m0, P.howo_magic, P.howo_shift);
         ho0 = magic_div(m0 - b * HoWo, P.wo_magic, P.wo_shift);
         hi0 = ho0 * P.SH - P.PH;
@@ -938,7 +940,7 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
     int      p_to[NVEC];             // where it goes in the patch (floats)
 #pragma unroll
     for (int q = 0; q < NVEC; ++q) {
-        const int v = tid + q * 256, r = v / vecs_per_row, c4 = v - r * vecs_per_row;
+        const int v = tid + q * NT, r = v / vecs_per_row, c4 = v - r * vecs_per_row;
         p_row[q]  = r;
         p_from[q] = (uint32_t)(r * WC + c4 * 4) * 4u;
         p_to[q]   = r * P.pitch + P.left + c4 * 4;
@@ -969,7 +971,7 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
         int b, ho0, hi0;
         patch_geometry(t, b, ho0, hi0);
         // this lane's output position and where its kernel row 0 starts in the patch
-        const int m  = t * 64 + wm * 32 + l32;
+        const int m  = t * BM + wm * 32 + l32;
         const int r2 = m - b * HoWo, ho = magic_div(r2, P.wo_magic, P.wo_shift), wo = r2 - ho * P.Wo;
         const float* a_base = Ps + (ho - ho0) * P.SH * P.pitch + P.left + (wo * P.SW - P.PW) * P.Cin + half;
         const float* b_base = Ws + half * LDB + wn * 32 + l32;
@@ -992,7 +994,7 @@ __device__ __forceinline__ void conv_stem_body(float* __restrict__ out, const fl
         const uint32_t slots = (P.flags >> 20) & 31u;
         const int col = wn * 32 + l32;
         const int e_mul = __builtin_popcount(slots & 1u), e_add = __builtin_popcount(slots & 3u), e_max = __builtin_popcount(slots & 15u);
-        const uint32_t base = col < P.N ? (uint32_t)((t * 64 + wm * 32 + 4 * half) * P.N + col) * 4u : CONV_OOB;
+        const uint32_t base = col < P.N ? (uint32_t)((t * BM + wm * 32 + 4 * half) * P.N + col) * 4u : CONV_OOB;
         const uint32_t rowb = (uint32_t)P.N * 4u;
         // a second result (bits 12-15 of the flags, as in conv_gemm_body): the value as it stands before (1) or after (2) the first step
         const int tap = (int)((P.flags >> 12) & 15u) - 1;
@@ -1036,6 +1038,16 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     __shared__ __attribute__((aligned(16))) float Ps[CONV_STEM_PATCH_FLOATS];
     __shared__ float Es[CONV_MAX_EPI * 64];
     conv_stem_body<7, 22, 9, 6>(out, x, w, epi, dp, P, D, Ws, Ps, Es);
+}
+// 128 output positions per tile (they reach into three output rows at most: 11 image rows), 8 waves per block
+#define CONV_STEM_PATCH_FLOATS_M128 7680
+extern "C" __global__ __launch_bounds__(512) void conv_gemm_stem_7x22_m128(
+        float* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+        ConvEpiPtrs epi, ConvDerivedPtrs dp, ConvStemParams P, ConvDerived D) {
+    __shared__ __attribute__((aligned(16))) float Ws[7 * 22 * 68];
+    __shared__ __attribute__((aligned(16))) float Ps[CONV_STEM_PATCH_FLOATS_M128];
+    __shared__ float Es[CONV_MAX_EPI * 64];
+    conv_stem_body<7, 22, 11, 4, 4>(out, x, w, epi, dp, P, D, Ws, Ps, Es);
 }
 
 // ---------------------------------------------------------------------------------------------

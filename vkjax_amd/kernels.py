@@ -45,7 +45,7 @@ class _Choices:
         conv_ksplit=None,                #the four-waves-per-tile kernel: always (where it applies) / never
         conv_dense_rows=None,            #the kernel for at most 16 output features: None = where it applies, False = never
         conv_mix=None,                   #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
-        conv_stem=None,                  #the patch kernel for few input features: False = never; None / True: where it applies
+        conv_stem=None,                  #the patch kernel for few input features: False = never; None / True: where it applies; 64: its 64-position tiles only
         conv_k_splits=None,              #slices a contraction is cut into where that applies (None: by the heuristic, 1: never)
         conv_xcd_columns=0,              #four-waves-per-tile kernels: XCD columns over the tile grid (0: row-major ranges, None: least traffic)
         scatter_sort_threshold=1 << 18,  #update elements from which a row scatter-add sorts its updates instead of using atomics
@@ -679,6 +679,8 @@ def _magic_division(d: int) -> tp.Tuple[int, int]:
 
 
 STEM_PATCH_FLOATS, STEM_PATCH_ROWS, STEM_VECTORS_PER_THREAD = 6272, 9, 6      #conv_gemm_stem_7x22's LDS patch
+#conv_gemm_stem_7x22_m128: tiles of 128 output positions (up to three output rows), 512 threads
+STEM128_PATCH_FLOATS, STEM128_PATCH_ROWS, STEM128_VECTORS_PER_THREAD = 7680, 11, 4
 
 
 def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_units, lhs_offset, rhs_offset, out_offset) -> tp.Optional[Launch]:
@@ -714,6 +716,12 @@ def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_
     buffers = [(out, 0), (lhs, 0), (rhs, 0)] + operand_slots + derived_ptrs
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
     nbytes += 4 * taps[0][1].size if taps else 0
+    #twice the tile and twice the waves per block where the sizes allow it: the kernel and the patch take the same LDS,
+    #so a CU holds 16 waves instead of 8
+    if (CHOICES.conv_stem != 64 and M % 128 == 0 and (g.Ho * g.Wo) % 128 == 0 and g.KH + 2 * g.SH <= STEM128_PATCH_ROWS
+            and STEM128_PATCH_ROWS * pitch <= STEM128_PATCH_FLOATS and STEM128_PATCH_ROWS * (WC // 4) <= 512 * STEM128_VECTORS_PER_THREAD):
+        return Launch('conv_gemm_stem_7x22_m128', (min(M // 128, 2 * compute_units), 1, 1), (512, 1, 1), buffers, params,
+                      bytes_moved=nbytes, flops=2 * M * N * K)
     return Launch('conv_gemm_stem_7x22', (min(M // 64, 2 * compute_units), 1, 1), (256, 1, 1), buffers, params,
                   bytes_moved=nbytes, flops=2 * M * N * K)
 
