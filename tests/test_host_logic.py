@@ -446,6 +446,30 @@ def test_repeated_equations_are_evaluated_once():
     assert names.count('add') == 4 and names.count('mul') == 2, names          #x+1, x+2, a+b, the result x+1
 
 
+def test_equal_equations_are_told_by_their_operands_storage_not_by_a_number():
+    '''The table of earlier equations is keyed by the id() of the operands' storage cells. An id can pass to another
+    object once its owner is gone, so an entry holds the cells themselves and a later equation is bound to the
+    earlier one's result only if its operands' cells ARE those objects: an entry whose key matches but whose cells
+    are other objects is replaced, not used.'''
+    from vkjax_amd import minijax as mj, ops
+    closed = mj.make_jaxpr(lambda x: ((x + 1.0) * (x + 1.0) * (x + 1.0)).sum())(np.zeros((8, 4), np.float32))
+    jaxpr = closed.jaxpr
+    adds = [eq for eq in jaxpr.eqns if eq.primitive.name == 'add']
+    assert len(adds) == 3
+    pool = BufferPool(PlanOnlyDevice())
+    pool.get_buffer(jaxpr.invars[0])                                       #the argument has storage, as in a build
+    assert ops._reuse_equal_equation(pool, adds[0]) is False               #noted
+    (key, (outvar, cells)), = pool._equal_equations.items()
+    assert len(cells) == 1 and key[2][0][0] == id(cells[0])
+    assert ops._reuse_equal_equation(pool, adds[1]) is True                #same operand cell: bound to the first
+    #the same key with a stranger in the cell's place, as after a recycled id
+    class Cell:
+        pass
+    pool._equal_equations[key] = (outvar, [Cell()])
+    assert ops._reuse_equal_equation(pool, adds[2]) is False
+    assert pool._equal_equations[key][1][0] is cells[0]                    #the entry now describes the live operand
+
+
 # ------------------------------------------------------------------ boundary details
 
 def test_reference_module_path_resolves():
