@@ -147,7 +147,9 @@ def test_scatter_add_rows_sorted_and_atomic_paths():
     than 16 and more than 64, indices outside the table (dropped), row lengths that are not a multiple of 4 or
     longer than one pass of a wave, integer data, operands that are not zero, more than 256 x 1024 table rows
     (bucket starts in segments of several tiles), a constant table filled with one value (not read at all), and
-    evaluating twice (the counters go back to zero).'''
+    evaluating twice (the counters go back to zero). The sorted path runs with the table of fixed-capacity buckets
+    as the host would size it, without it (every update goes through the overflow table), and with 4 and 64 slots per
+    row: rows within their slots, rows beyond them and both in one program.'''
     from vkjax_amd import ops
     rng = np.random.default_rng(7)
 
@@ -159,8 +161,9 @@ def test_scatter_add_rows_sorted_and_atomic_paths():
             return mj.numpy.index_add(mj.numpy.full((300, 64), fill, np.float32), idx, updates)
         return f
 
-    for path, threshold in (('sum', 0), ('atomic', 1 << 60)):
-        with K.overrides(scatter_sort_threshold=threshold):
+    for path, threshold, cap in (('sum', 0, None), ('sum', 0, 0), ('sum', 0, 4), ('sum', 0, 64), ('atomic', 1 << 60, None)):
+        print(f'case: row scatter-add, {path} path, {cap} slots per row', flush=True)
+        with K.overrides(scatter_sort_threshold=threshold, scatter_bucket_cap=cap):
             cases = [(50, 256, 400, np.float32), (9, 10, 37, np.float32), (300, 64, 200, np.int32), (4, 20, 500, np.float32),
                      (3000, 16, 9000, np.float32), (70, 520, 300, np.float32), (5, 8, 20000, np.int32), (1029, 4, 30000, np.float32),
                      (300000, 4, 5000, np.float32), (1025, 4, 3000, np.int32), (1024, 4, 3000, np.int32), (1023, 4, 3000, np.int32)]
@@ -179,6 +182,16 @@ def test_scatter_add_rows_sorted_and_atomic_paths():
                 expected = table.copy()
                 np.add.at(expected, idx2, updates2)
                 assert np.array_equal(fn(table, idx2, updates2), expected), (path, rows, cols, n)
+                interp = list(fn._jaxpr_interpreters.values())[0]
+                for key, b in interp.bufferpool.buffers.items():
+                    if isinstance(key, tuple) and key[:1] == ('zeroed',):
+                        words = b.numpy().reshape(-1)
+                        #(the word behind the counters is the cursor that the bucketing launch resets itself)
+                        assert not (words[:-1] if key[2] == 'counters' else words).any(), 'counters and overflow table are zero after an evaluation'
+                if path == 'sum' and cap is not None:
+                    rank_launch = [l for l in interp.launches if l.kernel == 'scatter_rows_rank'][0]
+                    assert np.frombuffer(rank_launch.params, np.uint32)[7] == cap
+                    assert rank_launch.buffers[1][0].size == (rows * cap if cap else n)
             #indices beyond the table (jnp's normalisation only wraps negative ones)
             table   = np.zeros((16, 8), np.float32)
             idx     = np.array([3, 99, 16, 15, -1, 3], np.int32)
@@ -270,7 +283,7 @@ def test_index_normalisation_is_done_by_the_indexing_kernels():
     names = lambda fn: [l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches]
     with K.overrides(scatter_sort_threshold=0):
         _, _, fn = check_against_oracle(W.gather_scatter, [table, idx, updates], exact=True)
-        assert names(fn) == ['gather_rows_v4', 'scatter_rows_rank', 'scatter_rows_starts', 'scatter_rows_order', 'scatter_rows_sum_f_v4'], names(fn)
+        assert names(fn) == ['gather_rows_v4', 'scatter_rows_rank', 'scatter_rows_sum_f_v4'], names(fn)
         _, _, fn = check_against_oracle(lambda t, i: t[i], [table, idx], exact=True)
         assert names(fn) == ['gather_rows_v4']
         _, _, fn = check_against_oracle(lambda t, i, u: mj.numpy.index_add(t, i, u), [table, idx, updates], exact=True)

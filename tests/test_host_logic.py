@@ -101,7 +101,7 @@ def test_kernel_argument_layouts_match_the_structs():
         'GatherRowsParams': K.gather_rows(b(3, 8), b(4, 8), i(3, 1), 3, 8, 4),
         'GatherGeneralParams': K.gather_general(b(3, 8), b(4, 8), i(3, 1), (1,), (0,), (0,), (1, 8)),
         'ScatterRowsParams': K.scatter_add_rows(b(4, 8), i(3, 1), b(3, 8), 3, 8, 4),
-        'ScatterSortParams': K.scatter_add_rows_sorted(b(4, 8), b(4, 8), i(3, 1), b(3, 8), *[Buffer(None, np.dtype('uint32'), (n,)) for n in (4, 5, 3, 3)],
+        'ScatterSortParams': K.scatter_add_rows_sorted(b(4, 8), b(4, 8), i(3, 1), b(3, 8), *[Buffer(None, np.dtype('uint32'), (n,)) for n in (5, 128, 3, 3)],
                                                        3, 8, 4)[0],
         'ScatterGeneralParams': K.scatter_add_general(b(4, 8), i(3, 1), b(3, 8), (1,), (0,), (0,)),
         'ThreefryParams': K.threefry2x32(*[Buffer(None, np.dtype('uint32'), (8,)) for _ in range(6)], key_is_scalar=False),
@@ -428,10 +428,10 @@ def test_repeated_equations_are_evaluated_once():
     fn, make = W.WORKLOADS['gather_scatter']
     closed = mj.make_jaxpr(fn)(*make())
     kernels = lambda **kw: [l.kernel for l in JaxprInterpreter(closed, plan_only=True, **kw).launches]
-    assert len(kernels()) == 5 and len(kernels(fuse=False)) == 8          #(fused: the gather and the scatter-add read the indices as they are and add n to the negative ones)
+    assert len(kernels()) == 3 and len(kernels(fuse=False)) == 6          #(fused: the gather and the scatter-add read the indices as they are and add n to the negative ones)
     from vkjax_amd import kernels as K
     with K.overrides(reuse_equal_equations=False):
-        assert len(kernels()) == 5 and len(kernels(fuse=False)) == 11
+        assert len(kernels()) == 3 and len(kernels(fuse=False)) == 9
     with pytest.raises(TypeError, match='unknown choice'):
         with K.overrides(no_such_choice=1):
             pass

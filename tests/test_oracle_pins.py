@@ -344,6 +344,7 @@ def test_integer_and_shift_semantics():
 
 
 def test_whole_program_identities():
+    rng = np.random.RandomState(77)          #(a generator of its own: the values do not depend on which tests ran before)
     x = rng.rand(6, 10).astype(np.float32) * 4
     closed = mj.make_jaxpr(lambda v: mj.nn.softmax(v))(x)
     (p,) = eval_closed_jaxpr(closed, x)
@@ -354,7 +355,7 @@ def test_whole_program_identities():
     closed = mj.make_jaxpr(lambda v, s, b, m, var: mj.nn.batch_norm_inference(v, s, b, m, var))(*args)
     (y,) = eval_closed_jaxpr(closed, *args)
     v, s, b, m, var = [a.astype(np.float64) for a in args]
-    assert np.allclose(y, (v - m) / np.sqrt(var + 1e-5) * s + b, rtol=1e-5)
+    assert np.allclose(y, (v - m) / np.sqrt(var + 1e-5) * s + b, rtol=1e-5, atol=1e-6)          #(float32 result; sums of terms of opposite sign come close to 0)
     closed = mj.make_jaxpr(lambda a, i: jnp.take_along_axis(a, i, axis=-1))(x, np.zeros((6, 1), np.int32))
     idx = rng.randint(0, 10, size=(6, 1)).astype(np.int32)
     (t,) = eval_closed_jaxpr(closed, x, idx)

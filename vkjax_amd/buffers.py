@@ -205,10 +205,10 @@ class BufferPool:
             self.buffers[key] = b
         return self.buffers[key]
 
-    def zeroed_scratch(self, n_words: int) -> Buffer:
+    def zeroed_scratch(self, n_words: int, use: str = '') -> Buffer:
         '''n_words of uint32 that hold zeros when the program is built and are never handed to anything else.
-        Launches that use them leave them zero again, so launches of one size share one array.'''
-        key = ('zeroed', int(n_words))
+        Launches that use them leave them zero again, so launches of one size and use share one array.'''
+        key = ('zeroed', int(n_words), use)
         if key not in self.buffers:
             b = Buffer(self.device.tensor(np.zeros(n_words, np.uint32)), np.dtype('uint32'), (n_words,))
             b.accesses += [0, np.inf]

@@ -43,6 +43,7 @@ class _Choices:
         conv_general=False,              #never pick the lean kernel variant
         conv_b_general=False,            #element-wise loads of the kernel operand also where 16-byte loads would do
         conv_ksplit=None,                #the four-waves-per-tile kernel: always (where it applies) / never
+        scatter_bucket_cap=None,         #slots per row in the sorted scatter-add's table of fixed-capacity buckets (0: no table)
         conv_dense_rows=None,            #the kernel for at most 16 output features: None = where it applies, False = never
         conv_mix=None,                   #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
         conv_stem=None,                  #the patch kernel for few input features: False = never; None / True: where it applies; 64: its 64-position tiles only
@@ -1206,7 +1207,7 @@ def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, c
 
 #kernels that can add a value to negative indices themselves: position of the index array among their arguments, and the
 #byte offset of the `wrap` field in their parameter block
-INDEX_WRAP_KERNELS = {'gather_rows_v1': (2, 24), 'gather_rows_v4': (2, 24), 'scatter_rows_rank': (2, 24), 'scatter_rows_order': (4, 24)}
+INDEX_WRAP_KERNELS = {'gather_rows_v1': (2, 24), 'gather_rows_v4': (2, 24), 'scatter_rows_rank': (3, 24)}
 
 
 def with_wrapped_index(launch: Launch, raw: Buffer, raw_byte_offset: int, amount: int) -> Launch:
@@ -1227,30 +1228,55 @@ def scatter_add_rows(out: Buffer, idx: Buffer, updates: Buffer, n_idx: int, row_
                   bytes_moved=4 * (total + n_idx + out.size))
 
 
-def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, count: Buffer, start: Buffer, rank: Buffer,
-                            order: Buffer, n_idx: int, row_len: int, n_rows: int, operand_is_scalar: bool = False,
-                            idx_stride: int = 1, clip: bool = False) -> tp.List[Launch]:
-    '''out = operand; out[idx[i], :] += updates[i, :] without atomics on the data: a counting sort of the indices
-    (`count`: n_rows words that are zero before and after, `start`: n_rows + 1 words, `rank` and `order`: n_idx words
-    each), then one wave per row sums its bucket. `operand` is the table, or one word when the table is a constant
-    filled with a single value.'''
-    assert count.size == n_rows and start.size == n_rows + 1 and rank.size == n_idx and order.size == n_idx
-    params = _u32(n_idx, row_len, n_rows, idx_stride, int(operand_is_scalar), int(clip), 0)
+def choose_scatter_bucket_cap(n_idx: int, n_rows: int, row_len: int) -> int:
+    '''How many slots every table row gets in the sorted scatter-add's table of fixed-capacity buckets (0: none, every
+    update goes through the overflow table): four times the average number of updates per row, as a power of two
+    between 4 and 64 - with indices spread evenly a row with more than that is a rarity - as long as the slots take at
+    most an eighth of the table's own size and eight words per update.'''
+    if CHOICES.scatter_bucket_cap is not None:
+        cap = int(CHOICES.scatter_bucket_cap)
+        assert 0 <= cap <= 64
+        return cap
+    if n_rows == 0 or n_idx == 0:
+        return 0
+    cap = 4
+    while cap < 64 and cap * n_rows < 4 * n_idx:
+        cap *= 2
+    while cap >= 4 and (cap * 8 > row_len or cap * n_rows > 8 * n_idx):
+        cap //= 2
+    return cap if cap >= 4 else 0
+
+
+def scatter_table_slots(n_idx: int) -> int:
+    '''Slots of the overflow table of a sorted scatter-add of n_idx updates: a power of two, at least 64 and at least
+    twice the number of updates.'''
+    return max(64, _pow2_at_least(2 * n_idx))
+
+
+def scatter_add_rows_sorted(out: Buffer, operand: Buffer, idx: Buffer, updates: Buffer, count: Buffer, table: Buffer, gathered: Buffer,
+                            sorted_: Buffer, n_idx: int, row_len: int, n_rows: int, operand_is_scalar: bool = False,
+                            idx_stride: int = 1, clip: bool = False, fixed: tp.Optional[Buffer] = None, cap: int = 0) -> tp.List[Launch]:
+    '''out = operand; out[idx[i], :] += updates[i, :] without atomics on the data: the first launch buckets the updates by
+    row, then one wave per row sums its bucket. `count`: n_rows + 1 words, `table`: two words per slot of the overflow
+    table (scatter_table_slots), both zero before and after; `fixed`: n_rows * cap words, the first `cap` updates of
+    every row (cap = 0: no such table); `gathered`, `sorted_`: n_idx words each, room for the buckets of rows with
+    more than cap updates. `operand` is the table, or one word when the table is a constant filled with a single
+    value.'''
+    slots = scatter_table_slots(n_idx)
+    assert count.size == n_rows + 1 and table.size == 2 * slots and gathered.size == n_idx and sorted_.size == n_idx
+    assert 0 <= cap <= 64 and (cap == 0 or (fixed is not None and fixed.size == n_rows * cap))
+    if fixed is None:
+        fixed = gathered                 #(never touched: no update's number within its row is below 0)
+    params = _u32(n_idx, row_len, n_rows, idx_stride, int(operand_is_scalar), int(clip), 0, cap, slots - 1)
     vec    = 4 if row_len % 4 == 0 else 1
     kind   = 'f' if out.dtype == np.float32 else 'i'
-    #bucket starts: at most 256 workgroups, each scanning a segment of whole 1024-word tiles
-    seg    = 1024 * _cdiv(_cdiv(n_rows + 1, 1024), 256)
     table_passes = 1 if operand_is_scalar else 2
     return [
-        Launch('scatter_rows_rank', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(count, 0), (rank, 0), (idx, 0)], params, bytes_moved=12 * n_idx,
-               written=(0, 1)),
-        Launch('scatter_rows_starts', (_cdiv(n_rows + 1, seg), 1, 1), (1024, 1, 1), [(start, 0), (count, 0)], _u32(n_rows, seg),
-               bytes_moved=8 * (n_rows + 1)),
-        Launch('scatter_rows_order', (_cdiv(max(n_idx, n_rows), BLOCK), 1, 1), (BLOCK, 1, 1),
-               [(order, 0), (count, 0), (start, 0), (rank, 0), (idx, 0)], params, bytes_moved=16 * n_idx + 4 * n_rows, written=(0, 1)),
+        Launch('scatter_rows_rank', (_cdiv(n_idx, BLOCK), 1, 1), (BLOCK, 1, 1), [(count, 0), (fixed, 0), (table, 0), (idx, 0)], params,
+               bytes_moved=8 * n_idx, written=(0, 1, 2)),
         Launch(f'scatter_rows_sum_{kind}_v{vec}', (_cdiv(n_rows, 4), 1, 1), (BLOCK, 1, 1),      #one wave per row
-               [(out, 0), (operand, 0), (updates, 0), (start, 0), (order, 0), (rank, 0)], params,       #(rank: room to sort crowded buckets in)
-               bytes_moved=4 * (n_idx * row_len + n_idx + table_passes * n_rows * row_len), written=(0, 5)),
+               [(out, 0), (operand, 0), (updates, 0), (count, 0), (fixed, 0), (table, 0), (gathered, 0), (sorted_, 0)], params,
+               bytes_moved=4 * (n_idx * row_len + n_idx + n_rows + table_passes * n_rows * row_len), written=(0, 3, 5, 6, 7)),
     ]
 
 

@@ -20,9 +20,9 @@ Measured on MI355X (device time of a replayed step, HIP events): 64 small launch
 same with one of them on the second lane (one fork, one join) 165 us; alternating lanes with a wait before
 every launch 869 us, i.e. about 12 us per dependency between the streams, with events that release to device
 scope only (hipEventReleaseToDevice; 56 us for fork and join with default events). With the plans below,
-gather + scatter-add went from 164 to 190 us (three stream dependencies; the gather and the data pass of the
-scatter-add are both bound by HBM and gain nothing from running side by side, only the 23 us of index passes
-could hide), ResNet-50 at batch 64 from 4.96 to 5.06 ms (the first block of every stage: conv1 beside the
+gather + scatter-add went from 164 to 190 us (measured while the scatter-add had three index launches in front of
+its data pass: three stream dependencies; the gather and the data pass are both bound by HBM and gain nothing from
+running side by side, only the 23 us of index passes could hide), ResNet-50 at batch 64 from 4.96 to 5.06 ms (the first block of every stage: conv1 beside the
 projection; storage reuse makes conv2 wait for the projection's reads), the MLP training step from 147 to
 212 us. JaxprInterpreter(two_lanes=True) therefore has to be asked for; the default is one in-order stream.
 '''

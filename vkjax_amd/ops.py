@@ -948,14 +948,18 @@ def scatter_add(bufferpool, equation):
         row_len = int(np.prod(operand.shape[1:], dtype=np.int64))
         n_idx   = int(np.prod(indices.shape[:-1], dtype=np.int64))
         n_rows  = operand.shape[0]
-        if n_idx * row_len >= K.CHOICES.scatter_sort_threshold and n_idx < 2**31 - 1 and n_rows < 2**31 - 1:
+        #(up to 2**27 updates: the overflow table of the sorted form has at least two slots of eight bytes per update)
+        if n_idx * row_len >= K.CHOICES.scatter_sort_threshold and n_idx <= 2**27 and n_rows < 2**31 - 1:
             #large: bucket the updates by row and sum each bucket (no atomics on the data, no copy of the operand)
             bufferpool.op_counter = counter_before
-            count = bufferpool.zeroed_scratch(n_rows)          #every evaluation leaves it zero again
+            count = bufferpool.zeroed_scratch(n_rows + 1, 'counters')      #every evaluation leaves the counters zero again
             count.accesses.append(counter_before)
-            start = bufferpool.new_temporary(np.dtype('uint32'), (n_rows + 1,))
-            rank  = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
-            order = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
+            table = bufferpool.zeroed_scratch(2 * K.scatter_table_slots(n_idx), 'overflow')      #the overflow table: likewise
+            table.accesses.append(counter_before)
+            gathered = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
+            sorted_  = bufferpool.new_temporary(np.dtype('uint32'), (n_idx,))
+            cap   = K.choose_scatter_bucket_cap(n_idx, n_rows, row_len)
+            fixed = bufferpool.new_temporary(np.dtype('uint32'), (n_rows * cap,)) if cap else None
             uniform = _uniform_constant(operand)
             if uniform is not None:
                 #a table that is a constant filled with one value (zeros, usually) is not read at all
@@ -964,8 +968,8 @@ def scatter_add(bufferpool, equation):
             else:
                 source = operand
             bufferpool.op_counter = counter_before + 1
-            launches = K.scatter_add_rows_sorted(outbuf, source, indices, updates, count, start, rank, order, n_idx, row_len, n_rows,
-                                                 operand_is_scalar=uniform is not None, clip=clip)
+            launches = K.scatter_add_rows_sorted(outbuf, source, indices, updates, count, table, gathered, sorted_, n_idx, row_len, n_rows,
+                                                 operand_is_scalar=uniform is not None, clip=clip, fixed=fixed, cap=cap)
             return [Op(equation, launch=l) for l in launches]
         ops = [copy, Op(equation, launch=K.scatter_add_rows(outbuf, indices, updates, n_idx, row_len, n_rows, clip=clip))]
         return ops
