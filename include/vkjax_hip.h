@@ -125,6 +125,20 @@ int vkj_seq_record_download(vkj_handle seq, vkj_handle buf, size_t offset, int s
  * (vkjax/kompute_jaxpr_interpreter.py:55-60); this lets launches that do not depend on each other share
  * the GPU (the index passes of a scatter-add beside a gather, a projection beside the branch it joins). */
 int vkj_seq_set_launch_lane(vkj_handle seq, int launch, int lane, int wait_for_other_lane);
+/* An alternative form of the FIRST recorded launch, for evaluations that upload the argument in `upload_slot`: the
+ * launch cut into parts (recorded with one call each, in order; arguments as for vkj_seq_record_launch) that
+ * together compute exactly what it computes, part k reading no more than the first `bytes_needed` bytes of that
+ * argument (ascending over the parts). When an evaluation sends that argument as the last one of its chunked
+ * uploads (VKJ uploads of 8 MB and more travel in chunks), each part is issued, on a stream of its own, as soon as
+ * the chunks it reads have been handed to the copy engines, so the device computes while the rest of the argument
+ * is still on its way; the first launch itself is then skipped and the others follow the last part. In every other
+ * evaluation (the argument resident or small, time stamps, a captured graph, launches on two lanes) the first launch
+ * runs as recorded. Events are created here, none when evaluating. The reference uploads every argument, then
+ * evaluates (vkjax/kompute_jaxpr_interpreter.py:72-77). */
+int vkj_seq_record_early_part(vkj_handle seq, vkj_handle fn, const uint32_t grid[3], const uint32_t block[3],
+                              uint32_t lds_bytes, const void* kernarg, size_t kernarg_bytes,
+                              const vkj_handle* bufs, const uint32_t* buf_arg_offsets,
+                              const uint64_t* buf_byte_offsets, int nbufs, int upload_slot, size_t bytes_needed);
 int vkj_seq_num_steps(vkj_handle seq, int* uploads, int* launches, int* downloads);
 /* sequence.eval()                     reference: vkjax/kompute_jaxpr_interpreter.py:77
  * All uploads, then all launches, then all downloads, then one stream synchronisation.

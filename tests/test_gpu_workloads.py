@@ -788,3 +788,42 @@ def test_stream_loader_may_refill_its_batch_array():
         assert len(got) == len(values)
         for k, (g, v) in enumerate(zip(got, values)):
             assert_tree_close(g, plain(v, w), exact=True, what=f'{shape} batch {k}')
+
+
+def test_first_launch_starts_while_its_argument_arrives():
+    '''A convolution over a large argument as the program's first launch is recorded a second time, cut along the batch
+    into parts that the runtime issues while the rest of the argument is still being uploaded. Whole calls (parts) give
+    the bits of the same program replayed on resident inputs (the launch as recorded), call after call with new
+    images; the oracle agrees on a slice of the batch; programs whose first launch does not qualify record no parts.'''
+    rng = np.random.default_rng(41)
+    lax, nn = mj.lax, mj.nn
+    def stem(params, x):
+        y = lax.conv_general_dilated(x, params['w'], (2, 2), ((3, 3), (3, 3)), dimension_numbers=W.NHWC)
+        y = nn.relu(nn.batch_norm_inference(y, params['g'], params['b'], params['m'], params['v']))
+        return y.reshape(x.shape[0], -1, 16).mean(axis=1), y[:, ::37, ::41, :]
+    def frozen(a):
+        a.flags.writeable = False
+        return a
+    params = dict(w=frozen((rng.standard_normal((7, 7, 3, 16)) / 12).astype(np.float32)), g=frozen(rng.random(16, dtype=np.float32) + 0.5),
+                  b=frozen(rng.standard_normal(16).astype(np.float32)), m=frozen(rng.standard_normal(16).astype(np.float32)),
+                  v=frozen(rng.random(16, dtype=np.float32) + 0.5))
+    fn = vkjax_amd.wrap(stem, frontend='minijax')
+    images = [rng.standard_normal((32, 224, 224, 3)).astype(np.float32) for _ in range(3)]
+    results = [fn(params, x) for x in images]                       #(the first call uploads the parameters too, in front of x)
+    interp = list(fn._jaxpr_interpreters.values())[0]
+    assert len(interp.early_parts) == 4 and all(p.kernel == interp.launches[0].kernel for p, _, _ in interp.early_parts)
+    assert [needed for _, _, needed in interp.early_parts] == [(k + 1) * images[0].nbytes // 4 for k in range(4)]
+    for x, got in zip(images, results):
+        interp.upload_inputs(params, x)
+        interp.replay(1)
+        mean, samples = interp.read_outputs()
+        assert np.array_equal(np.asarray(got[0]).reshape(-1), mean.reshape(-1)) and np.array_equal(np.asarray(got[1]).reshape(-1), samples.reshape(-1))
+    expected, _ = oracle_outputs(stem, [params, images[2][:2]])
+    assert np.allclose(results[2][0][:2], expected[0], rtol=1e-4, atol=1e-5) and np.allclose(results[2][1][:2], expected[1], rtol=1e-4, atol=1e-5)
+    #a first launch that is no convolution over a large argument, or one in the mixed tiling: no parts
+    small = vkjax_amd.wrap(stem, frontend='minijax')
+    small(params, images[0][:4])
+    assert list(small._jaxpr_interpreters.values())[0].early_parts == []
+    fn2 = vkjax_amd.wrap(lambda x: nn.relu(x) * 2.0, frontend='minijax')
+    big = rng.standard_normal((1 << 23,)).astype(np.float32)
+    assert np.array_equal(fn2(big), np.maximum(big, 0) * 2.0) and list(fn2._jaxpr_interpreters.values())[0].early_parts == []

@@ -341,3 +341,65 @@ def test_launches_on_two_lanes(lib):
         assert lib.vkj_buf_free(w.ctx, buf) == 0
     w.close()
     assert lib.fake_hip_live_objects() == before
+
+
+def test_first_launch_in_parts_beside_the_upload(lib):
+    '''vkj_seq_record_early_part: when an evaluation uploads the argument the parts read (in chunks, as the last of its
+    uploads), each part is issued as soon as the chunks it needs have been handed over - the stand-in runs copies and
+    kernels at once, so a part issued too early would compute on bytes that are not there yet - and the first launch
+    itself is skipped; with the argument resident, or followed by another upload, the launch runs as recorded.
+    Nothing is created while evaluating; bad arguments are refused; everything goes with the sequence.'''
+    before = lib.fake_hip_live_objects()
+    w = World(lib)
+    n, nparts = 4 << 20, 4                                        #16 MB: uploads of 8 MB and more travel in chunks
+    src, mid, dst, other, seq = w.buf(4 * n), w.buf(4 * n), w.buf(4 * n), w.buf(64), H()
+    assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq)) == 0
+    grid = (C.c_uint32 * 3)(1, 1, 1)
+    def part_args(p):
+        kernarg = bytes(16) + np.uint32(n // nparts).tobytes() + bytes(4)
+        bufs = (C.c_uint64 * 2)(mid.value, src.value)
+        offs = (C.c_uint32 * 2)(0, 8)
+        byte = (C.c_uint64 * 2)(p * 4 * n // nparts, p * 4 * n // nparts)
+        return (seq, w.fn, grid, grid, 0, kernarg, len(kernarg), bufs, offs, byte, 2)
+    assert lib.vkj_seq_record_upload(seq, src, 0, 0, 4 * n) == 0
+    assert lib.vkj_seq_record_early_part(*part_args(0), 0, 4 * n // nparts) == ESTATE       #no launch to stand for yet
+    assert w.record_add_one(seq, mid, src, n) == 0               #mid = src + 1: the launch the parts stand for
+    assert w.record_add_one(seq, dst, mid, n) == 0               #dst = mid + 1
+    assert lib.vkj_seq_record_download(seq, dst, 0, 1, 4 * n) == 0
+    assert lib.vkj_seq_record_early_part(*part_args(0), 3, 4 * n // nparts) == EINVAL       #no upload in that slot
+    assert lib.vkj_seq_record_early_part(*part_args(0), 0, 4 * n + 4) == EINVAL             #more than the argument has
+    for p in range(nparts):
+        assert lib.vkj_seq_record_early_part(*part_args(p), 0, (p + 1) * 4 * n // nparts) == 0, lib.vkj_last_error()
+    assert lib.vkj_seq_record_early_part(*part_args(0), 0, 4 * n // nparts) == EINVAL       #parts come in ascending order
+    made = lib.fake_hip_creations()
+    rng = np.random.default_rng(3)
+    for _ in range(2):
+        x = rng.integers(0, 1 << 30, size=n, dtype=np.uint32)
+        launches = lib.fake_hip_launches()
+        assert np.array_equal(w.eval(seq, x), x + 2)
+        assert lib.fake_hip_launches() - launches == nparts + 1   #the parts, then the second launch
+    #the argument stays where it is: the launch as recorded
+    launches = lib.fake_hip_launches()
+    assert np.array_equal(w.eval(seq, None, flags=1, n=n), x + 2)            #VKJ_EVAL_NULL_IS_RESIDENT
+    assert lib.fake_hip_launches() - launches == 2
+    assert lib.fake_hip_creations() == made
+    assert lib.vkj_seq_destroy(seq) == 0
+    #another upload behind the argument: what the first launch reads besides it may not have arrived, so no parts
+    seq = H()
+    assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq)) == 0
+    assert lib.vkj_seq_record_upload(seq, src, 0, 0, 4 * n) == 0
+    assert lib.vkj_seq_record_upload(seq, other, 0, 2, 64) == 0
+    assert w.record_add_one(seq, mid, src, n) == 0
+    assert lib.vkj_seq_record_download(seq, mid, 0, 1, 4 * n) == 0
+    for p in range(nparts):
+        assert lib.vkj_seq_record_early_part(*part_args(p), 0, (p + 1) * 4 * n // nparts) == 0
+    y, small = np.zeros(n, np.uint32), np.zeros(16, np.uint32)
+    ptrs = (C.c_void_p * 3)(x.ctypes.data, y.ctypes.data, small.ctypes.data)
+    launches = lib.fake_hip_launches()
+    assert lib.vkj_seq_eval(seq, ptrs, 3, 0) == 0, lib.vkj_last_error()
+    assert np.array_equal(y, x + 1) and lib.fake_hip_launches() - launches == 1
+    assert lib.vkj_seq_destroy(seq) == 0
+    for b in (src, mid, dst, other):
+        assert lib.vkj_buf_free(w.ctx, b) == 0
+    w.close()
+    assert lib.fake_hip_live_objects() == before

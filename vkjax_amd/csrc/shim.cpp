@@ -131,7 +131,7 @@ int staged_upload_pieces(const std::vector<UploadPiece>& pieces, Issue&& issue) 
     for (size_t k = 0; k < nchunks; k++) {
         while (!done[k].load(std::memory_order_acquire)) std::this_thread::yield();
         const Chunk& ch = chunks[k];
-        if (status == 0) status = issue(k, pieces[ch.piece].device + ch.off, pieces[ch.piece].staging + ch.off, ch.len);
+        if (status == 0) status = issue(k, ch.piece, ch.off, ch.len);
     }
     for (auto& t : threads) t.join();
     return status;
@@ -213,8 +213,14 @@ void drop_graph(Seq* s) {
     s->graph_failed = false;
 }
 
-// All launches of a sequence, once: as its captured graph when that is asked for, else one by one.
-int issue_all(Ctx* c, Seq* s) {
+// All launches of a sequence, once: as its captured graph when that is asked for, else one by one. `first`: the
+// launches before it have been issued already (the first launch, in parts, beside the uploads).
+int issue_all(Ctx* c, Seq* s, size_t first = 0) {
+    if (first) {
+        for (size_t i = first; i < s->launches.size(); i++)
+            if (int r = issue_launch(c, s->launches[i])) return r;
+        return 0;
+    }
     if (s->want_graph && !s->profiling && !s->graph_failed && s->launches.size() > 1) {
         if (!s->graph_exec) {
             hipGraph_t graph = nullptr;
@@ -276,7 +282,7 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
         return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for upload slot %d", t.slot);
     if (down) for (auto& t : s->downloads) if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for download slot %d", t.slot);
 
-    size_t nstamps = 0;
+    size_t nstamps = 0, first_launch = 0;        // first_launch: 1 when the first launch has been issued in parts beside the uploads
     if (s->profiling) {
         nstamps = 3 + s->launches.size();       // begin, after uploads, after each launch, after downloads
         while (s->stamps.size() < nstamps) {
@@ -299,14 +305,46 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
                     pieces.push_back({(char*)t.staging, (const char*)host_ptrs[t.slot], (char*)t.buf->dptr + t.offset, t.nbytes});
             // the chunks alternate between the two streams (two copy engines work on them); the launches wait for both.
             // Both streams are idle here: every evaluation ends with everything it queued on them complete.
+            // The first launch in parts: a part goes to the side stream as soon as the chunks it reads have been
+            // handed to the copy engines (both streams are in order: an event behind a chunk covers every chunk
+            // before it), so the device computes while the rest of the argument is still on its way.
+            size_t early_piece = pieces.size(), next_part = 0;
+            if (!s->early.empty() && !s->profiling && !s->want_graph && !s->uses_side) {
+                size_t p = 0;
+                for (auto& t : s->uploads) {
+                    if (!(t.nbytes && host_ptrs[t.slot])) continue;
+                    if (t.slot == s->early_slot && t.nbytes >= s->early.back().bytes_needed) early_piece = p;
+                    p++;
+                }
+                // only as the last argument on its way: whatever else the launch reads has then been sent before it
+                if (early_piece + 1 != pieces.size()) early_piece = pieces.size();
+            }
             hipError_t err = hipSuccess;
-            const int r = staged_upload_pieces(pieces, [&](size_t k, char* device, const char* staging, size_t len) {
-                err = hipMemcpyAsync(device, staging, len, hipMemcpyHostToDevice, (k & 1) ? c->copy_stream : c->stream);
-                return err == hipSuccess ? 0 : 1;
+            int launch_status = 0;
+            const int r = staged_upload_pieces(pieces, [&](size_t k, size_t piece, size_t off, size_t len) {
+                err = hipMemcpyAsync(pieces[piece].device + off, pieces[piece].staging + off, len, hipMemcpyHostToDevice,
+                                     (k & 1) ? c->copy_stream : c->stream);
+                if (err != hipSuccess) return 1;
+                while (piece == early_piece && next_part < s->early.size() && s->early[next_part].bytes_needed <= off + len) {
+                    EarlyPart& part = s->early[next_part++];
+                    if ((err = hipEventRecord(part.ev_a, c->stream)) != hipSuccess) return 1;
+                    if ((err = hipEventRecord(part.ev_b, c->copy_stream)) != hipSuccess) return 1;
+                    if ((err = hipStreamWaitEvent(c->side_stream, part.ev_a, 0)) != hipSuccess) return 1;
+                    if ((err = hipStreamWaitEvent(c->side_stream, part.ev_b, 0)) != hipSuccess) return 1;
+                    if ((launch_status = issue_launch(c, part.launch, c->side_stream))) return 1;
+                }
+                return 0;
             });
+            if (launch_status) return launch_status;
             if (r) return hip_fail(err, "hipMemcpyAsync (staged upload)");
             HIP_TRY(hipEventRecord(c->ev_copied, c->copy_stream));
             HIP_TRY(hipStreamWaitEvent(c->stream, c->ev_copied, 0));
+            if (early_piece < pieces.size()) {
+                // (every part has been issued: the last one needs no more than the whole argument)
+                HIP_TRY(hipEventRecord(s->ev_early_done, c->side_stream));
+                HIP_TRY(hipStreamWaitEvent(c->stream, s->ev_early_done, 0));
+                first_launch = 1;
+            }
         } else {
             for (auto& t : s->uploads) {
                 if (!t.nbytes || !host_ptrs[t.slot]) continue;
@@ -328,7 +366,7 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
             if (int r = issue_launch(c, s->launches[i])) return r;
             HIP_TRY(hipEventRecord(s->stamps[2 + i], c->stream));
         }
-    } else if (int r = issue_all(c, s)) {
+    } else if (int r = issue_all(c, s, first_launch)) {
         return r;
     }
     bool landed = false;
@@ -714,6 +752,13 @@ int vkj_seq_destroy(vkj_handle sh) {
         for (Buf* b : l.bufs) unref_buf(b);
         if (l.wait_event) hipEventDestroy(l.wait_event);
     }
+    for (auto& part : s->early) {
+        part.launch.fn->mod->seq_refs--;
+        for (Buf* b : part.launch.bufs) unref_buf(b);
+        if (part.ev_a) hipEventDestroy(part.ev_a);
+        if (part.ev_b) hipEventDestroy(part.ev_b);
+    }
+    if (s->ev_early_done) hipEventDestroy(s->ev_early_done);
     if (s->ev_fork) hipEventDestroy(s->ev_fork);
     if (s->ev_join) hipEventDestroy(s->ev_join);
     for (auto e : s->stamps) hipEventDestroy(e);
@@ -758,42 +803,83 @@ int vkj_seq_record_download(vkj_handle sh, vkj_handle bh, size_t offset, int slo
     return 0;
 }
 
-int vkj_seq_record_launch(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], const uint32_t block[3],
-                          uint32_t lds_bytes, const void* kernarg, size_t kernarg_bytes,
-                          const vkj_handle* bufs, const uint32_t* buf_arg_offsets,
-                          const uint64_t* buf_byte_offsets, int nbufs) {
-    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+// The checks and the argument block of a recorded launch (vkj_seq_record_launch, vkj_seq_record_early_part): on
+// success `l` holds the launch, with the buffers' addresses patched in; nothing is referenced or recorded yet.
+static int make_launch(const char* who, Seq* s, vkj_handle fh, const uint32_t grid[3], const uint32_t block[3],
+                       uint32_t lds_bytes, const void* kernarg, size_t kernarg_bytes,
+                       const vkj_handle* bufs, const uint32_t* buf_arg_offsets,
+                       const uint64_t* buf_byte_offsets, int nbufs, Launch& l) {
     Fn*  f = from_handle<Fn>(fh, MAGIC_FN);
     if (!s || !f || f->mod->ctx != s->ctx || !grid || !block || (!kernarg && kernarg_bytes) || nbufs < 0 ||
         (nbufs && (!bufs || !buf_arg_offsets)))
-        return fail(VKJ_EINVAL, "vkj_seq_record_launch: bad argument");
+        return fail(VKJ_EINVAL, "%s: bad argument", who);
     for (int i = 0; i < 3; i++)
         if (grid[i] == 0 || block[i] == 0)
-            return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): zero-sized grid or block", f->name.c_str());
+            return fail(VKJ_EINVAL, "%s(%s): zero-sized grid or block", who, f->name.c_str());
     if ((uint64_t)block[0] * block[1] * block[2] > 1024)
-        return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): more than 1024 threads per block", f->name.c_str());
+        return fail(VKJ_EINVAL, "%s(%s): more than 1024 threads per block", who, f->name.c_str());
     if ((uint64_t)grid[0] * block[0] > 0xFFFFFFFFull || grid[1] > 65535 || grid[2] > 65535)
-        return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): grid too large", f->name.c_str());
-    Launch l;
+        return fail(VKJ_EINVAL, "%s(%s): grid too large", who, f->name.c_str());
     l.fn = f;
     for (int i = 0; i < 3; i++) { l.grid[i] = grid[i]; l.block[i] = block[i]; }
     l.lds = lds_bytes;
     l.kernarg.assign((const uint8_t*)kernarg, (const uint8_t*)kernarg + kernarg_bytes);
     for (int i = 0; i < nbufs; i++) {
         Buf* b = from_handle<Buf>(bufs[i], MAGIC_BUF);
-        if (!b || b->ctx != s->ctx) return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): bad buffer handle #%d", f->name.c_str(), i);
+        if (!b || b->ctx != s->ctx) return fail(VKJ_EINVAL, "%s(%s): bad buffer handle #%d", who, f->name.c_str(), i);
         uint64_t off = buf_byte_offsets ? buf_byte_offsets[i] : 0;
-        if (off > b->nbytes) return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): offset of buffer #%d beyond its end", f->name.c_str(), i);
+        if (off > b->nbytes) return fail(VKJ_EINVAL, "%s(%s): offset of buffer #%d beyond its end", who, f->name.c_str(), i);
         if ((size_t)buf_arg_offsets[i] + 8 > kernarg_bytes || (buf_arg_offsets[i] & 7))
-            return fail(VKJ_EINVAL, "vkj_seq_record_launch(%s): pointer slot #%d outside the argument block or misaligned", f->name.c_str(), i);
+            return fail(VKJ_EINVAL, "%s(%s): pointer slot #%d outside the argument block or misaligned", who, f->name.c_str(), i);
         uint64_t addr = (uint64_t)(uintptr_t)b->dptr + off;
         memcpy(l.kernarg.data() + buf_arg_offsets[i], &addr, 8);
         l.bufs.push_back(b);
     }
+    return 0;
+}
+
+int vkj_seq_record_launch(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], const uint32_t block[3],
+                          uint32_t lds_bytes, const void* kernarg, size_t kernarg_bytes,
+                          const vkj_handle* bufs, const uint32_t* buf_arg_offsets,
+                          const uint64_t* buf_byte_offsets, int nbufs) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    Launch l;
+    if (int r = make_launch("vkj_seq_record_launch", s, fh, grid, block, lds_bytes, kernarg, kernarg_bytes, bufs, buf_arg_offsets,
+                            buf_byte_offsets, nbufs, l)) return r;
     for (Buf* b : l.bufs) b->seq_refs++;
-    f->mod->seq_refs++;
+    l.fn->mod->seq_refs++;
     s->launches.push_back(std::move(l));
     drop_graph(s);                                  // a captured graph no longer matches the sequence
+    return 0;
+}
+
+int vkj_seq_record_early_part(vkj_handle sh, vkj_handle fh, const uint32_t grid[3], const uint32_t block[3],
+                              uint32_t lds_bytes, const void* kernarg, size_t kernarg_bytes,
+                              const vkj_handle* bufs, const uint32_t* buf_arg_offsets,
+                              const uint64_t* buf_byte_offsets, int nbufs, int upload_slot, size_t bytes_needed) {
+    Seq* s = from_handle<Seq>(sh, MAGIC_SEQ);
+    if (!s) return fail(VKJ_EINVAL, "vkj_seq_record_early_part: bad handle");
+    if (s->launches.empty()) return fail(VKJ_ESTATE, "vkj_seq_record_early_part: the launch the parts stand for is recorded first");
+    const Transfer* upload = nullptr;
+    for (auto& t : s->uploads) if (t.slot == upload_slot) upload = &t;
+    if (!upload || bytes_needed == 0 || bytes_needed > upload->nbytes)
+        return fail(VKJ_EINVAL, "vkj_seq_record_early_part: no upload in slot %d, or it has fewer than %zu bytes", upload_slot, bytes_needed);
+    if (!s->early.empty() && (s->early_slot != upload_slot || bytes_needed < s->early.back().bytes_needed))
+        return fail(VKJ_EINVAL, "vkj_seq_record_early_part: parts read one upload slot, in ascending order of what they need");
+    if (int r = use(s->ctx)) return r;
+    EarlyPart part;
+    if (int r = make_launch("vkj_seq_record_early_part", s, fh, grid, block, lds_bytes, kernarg, kernarg_bytes, bufs, buf_arg_offsets,
+                            buf_byte_offsets, nbufs, part.launch)) return r;
+    part.bytes_needed = bytes_needed;
+    // everything an evaluation needs is made here, so that evaluating creates nothing
+    if (!s->ev_early_done) HIP_TRY(hipEventCreateWithFlags(&s->ev_early_done, hipEventDisableTiming));
+    HIP_TRY(hipEventCreateWithFlags(&part.ev_a, hipEventDisableTiming));
+    hipError_t e = hipEventCreateWithFlags(&part.ev_b, hipEventDisableTiming);
+    if (e != hipSuccess) { hipEventDestroy(part.ev_a); return hip_fail(e, "hipEventCreateWithFlags"); }
+    for (Buf* b : part.launch.bufs) b->seq_refs++;
+    part.launch.fn->mod->seq_refs++;
+    s->early_slot = upload_slot;
+    s->early.push_back(std::move(part));
     return 0;
 }
 

@@ -91,6 +91,14 @@ struct Launch {
                                                  // and waited for on this launch's lane before the launch is issued
 };
 
+// One part of the first launch's alternative form (vkj_seq_record_early_part): what it needs of the argument in
+// upload slot Seq::early_slot, and the two events that tell its stream that those bytes have arrived.
+struct EarlyPart {
+    Launch     launch;
+    size_t     bytes_needed = 0;
+    hipEvent_t ev_a = nullptr, ev_b = nullptr;
+};
+
 struct Seq {
     uint64_t                handle = 0;
     uint32_t                magic = MAGIC_SEQ;
@@ -107,6 +115,9 @@ struct Seq {
     bool                    want_graph = false;     // issue the launches as one captured graph
     bool                    graph_failed = false;   // capture did not work once: keep to plain launches
     hipGraphExec_t          graph_exec = nullptr;
+    std::vector<EarlyPart>  early;                  // the first launch in parts, each issued while the rest of an argument is still on its way
+    int                     early_slot = -1;
+    hipEvent_t              ev_early_done = nullptr;
 };
 
 // Handles are keys into a process-wide table, never raw addresses, so that a stale or made-up

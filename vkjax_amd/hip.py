@@ -56,6 +56,9 @@ _PROTOTYPES = {
     'vkj_seq_destroy':         (C.c_int, [_H]),
     'vkj_seq_record_upload':   (C.c_int, [_H, _H, C.c_size_t, C.c_int, C.c_size_t]),
     'vkj_seq_set_launch_lane': (C.c_int, [_H, C.c_int, C.c_int, C.c_int]),
+    'vkj_seq_record_early_part': (C.c_int, [_H, _H, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_uint32,
+                                            C.c_void_p, C.c_size_t, C.POINTER(_H), C.POINTER(C.c_uint32),
+                                            C.POINTER(C.c_uint64), C.c_int, C.c_int, C.c_size_t]),
     'vkj_seq_record_launch':   (C.c_int, [_H, _H, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_uint32,
                                           C.c_void_p, C.c_size_t, C.POINTER(_H), C.POINTER(C.c_uint32),
                                           C.POINTER(C.c_uint64), C.c_int]),
@@ -263,9 +266,11 @@ class Sequence:
         return slot
 
     def record_launch(self, kernel_name: str, grid, block, buffers: tp.Sequence[tp.Tuple[tp.Optional[DeviceBuffer], int]],
-                      params: bytes, lds_bytes: int = 0):
+                      params: bytes, lds_bytes: int = 0, early_part_of: tp.Optional[tp.Tuple[int, int]] = None):
         '''`buffers` are (DeviceBuffer or None, byte offset) in kernel-argument order; they occupy
-        the first 8*len(buffers) bytes of the argument block, `params` follows.'''
+        the first 8*len(buffers) bytes of the argument block, `params` follows. `early_part_of` = (upload slot, bytes
+        needed): the launch is not a step of the sequence but one part of the alternative form of its first launch
+        (vkj_seq_record_early_part), issued while the rest of that slot's argument is still being uploaded.'''
         fn      = self.device.function(kernel_name)
         nptr    = len(buffers)
         kernarg = bytes(8 * nptr) + params
@@ -276,6 +281,12 @@ class Sequence:
         byteoff = (C.c_uint64 * max(n, 1))(*[off for _, _, off in present])
         g = (C.c_uint32 * 3)(*[int(x) for x in grid])
         b = (C.c_uint32 * 3)(*[int(x) for x in block])
+        if early_part_of is not None:
+            slot, needed = early_part_of
+            _check(self.device.lib.vkj_seq_record_early_part(self.handle, fn, g, b, lds_bytes, kernarg, len(kernarg),
+                                                              handles, argoffs, byteoff, n, int(slot), int(needed)),
+                   f'vkj_seq_record_early_part({kernel_name})')
+            return
         _check(self.device.lib.vkj_seq_record_launch(self.handle, fn, g, b, lds_bytes, kernarg, len(kernarg),
                                                       handles, argoffs, byteoff, n), f'vkj_seq_record_launch({kernel_name})')
         self.n_launches += 1

@@ -105,6 +105,11 @@ class JaxprInterpreter:
             for k, (lane, wait) in enumerate(zip(self.lane_plan.lane, self.lane_plan.wait)):
                 if lane or wait:
                     self.sequence.set_launch_lane(k, lane, wait)
+        #the first launch in parts that start while the rest of its (large) argument is still being uploaded
+        self.early_parts = self._early_parts_of_first_launch()
+        for part, slot, needed in self.early_parts:
+            bufs = [((b.tensor if b is not None else None), off) for b, off in part.buffers]
+            self.sequence.record_launch(part.kernel, part.grid, part.block, bufs, part.params, part.lds, early_part_of=(slot, needed))
         if self.graph:
             self.sequence.use_graph(True)
         self._output_slots = []
@@ -116,6 +121,43 @@ class JaxprInterpreter:
                 continue
             self._output_slots.append(self.sequence.record_download(b.tensor, b.nbytes()))
             self._output_sizes.append(b.size)
+
+    #an argument from this size on is worth starting the first launch on while it is still arriving (the link moves
+    #about 50 MB per millisecond; a part more costs a few microseconds of device time)
+    EARLY_PARTS_MIN_BYTES = 16 << 20
+
+    def _early_parts_of_first_launch(self):
+        '''[(launch, upload slot, bytes of the argument the part needs)]: the program's first launch cut along the batch
+        into parts that together compute what it computes, when it is a convolution or matrix product over a large
+        argument whose images (rows) are computed independently by one kernel of the family in which a wave sums
+        its contraction in one fixed order whatever the tiling (so every part's values are the whole launch's, bit for
+        bit). The runtime issues a part as soon as the chunks of the argument it reads are on their way
+        (vkj_seq_record_early_part); evaluations that do not upload that argument run the launch as it is.'''
+        if (not self.all_ops or self.profiling or self.graph or (self.lane_plan is not None and any(self.lane_plan.lane))
+                or self.all_ops[0].conv is None):
+            return []
+        out, lhs, rhs, geom, epilogue = self.all_ops[0].conv
+        whole = self.launches[0]
+        k = next((i for i, b in enumerate(self.input_buffers) if b is lhs), None)
+        if k is None or self._input_slots[k] is None or lhs.nbytes() < self.EARLY_PARTS_MIN_BYTES:
+            return []
+        B = geom.batch
+        nparts = 4 if B % 4 == 0 else 2 if B % 2 == 0 else 0
+        plain = (whole.kernel.startswith('conv_gemm') and not any(tag in whole.kernel for tag in ('_mix', '_ks4')) and not whole.members)
+        if (not nparts or not plain or geom.k_splits > 1 or lhs.size % B or out.size % B or geom.xs[0] != lhs.size // B
+                or geom.os[0] != out.size // B or any(e.kind == 3 or e.op in (K.CONV_TAP, K.CONV_SOFTMAX) for e in epilogue)):
+            return []
+        parts = []
+        for p in range(nparts):
+            try:
+                part = K.conv_gemm(out, lhs, rhs, geom._replace(batch=B // nparts), epilogue,
+                                   lhs_offset=p * (lhs.size // nparts), out_offset=p * (out.size // nparts))
+            except (ValueError, NotImplementedError):
+                return []
+            if part.kernel != whole.kernel:
+                return []
+            parts.append((part, self._input_slots[k], (p + 1) * (lhs.nbytes() // nparts)))
+        return parts
 
     def record_launch(self, sequence, launch, op=None):
         '''Records one of this program's launches into `sequence` (its own, or another sequence on the same buffers:

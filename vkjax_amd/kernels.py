@@ -687,7 +687,9 @@ STEM128_PATCH_FLOATS, STEM128_PATCH_ROWS, STEM128_VECTORS_PER_THREAD = 7680, 11,
 def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_units, lhs_offset, rhs_offset, out_offset) -> tp.Optional[Launch]:
     '''conv_gemm_stem_7x22 where it applies: dense images with so few features that KW * Cin is 21 or 22 (7 x 7 x 3),
     seven kernel rows, a template epilogue; see the conditions listed at the kernel.'''
-    if CHOICES.conv_stem is False or CHOICES.conv_tile is not None or CHOICES.conv_general or lhs_offset or rhs_offset or out_offset:
+    #(offsets: whole images further on in both arrays - a launch over a part of the batch)
+    if (CHOICES.conv_stem is False or CHOICES.conv_tile is not None or CHOICES.conv_general or rhs_offset or lhs_offset % 4 or out_offset % 4
+            or (taps and (lhs_offset or out_offset))):
         return None
     M, N, K = g.M, g.N, g.K
     RL, WC = g.KW * g.Cin, g.W * g.Cin
@@ -707,14 +709,14 @@ def _conv_stem_launch(out, lhs, rhs, g: 'ConvGeometry', epilogue, taps, compute_
     #a second result (the value before or after the first epilogue step) goes to the last operand slot, as in conv_gemm_body
     flags  = slots << 20 | ((taps[0][0] + 1) << 12 if taps else 0)
     params = (_i32(M, N, K, g.Ho, g.Wo, g.H, g.W, g.Cin, g.KH, g.KW, g.SH, g.SW, g.PH, g.PW, pitch, left)
-              + _u32(flags, lhs.size * 4, rhs.size * 4, out.size * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo)))
+              + _u32(flags, (lhs.size - lhs_offset) * 4, rhs.size * 4, (out.size - out_offset) * 4, *_magic_division(g.Ho * g.Wo), *_magic_division(g.Wo)))
     derived_ptrs, derived_desc = _conv_derived(epilogue, N)
     params += derived_desc
     operand_slots = _pad([(e.operand, 0) for e in epilogue], CONV_MAX_EPI, (None, 0))
     if taps:
         assert operand_slots[-1] == (None, 0)
         operand_slots[-1] = (taps[0][1], 0)
-    buffers = [(out, 0), (lhs, 0), (rhs, 0)] + operand_slots + derived_ptrs
+    buffers = [(out, out_offset * 4), (lhs, lhs_offset * 4), (rhs, 0)] + operand_slots + derived_ptrs
     nbytes  = 4 * (lhs.size + rhs.size + out.size) + sum(4 * e.operand.size for e in epilogue if e.operand is not None)
     nbytes += 4 * taps[0][1].size if taps else 0
     #twice the tile and twice the waves per block where the sizes allow it: the kernel and the patch take the same LDS,
