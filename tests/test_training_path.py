@@ -194,7 +194,7 @@ def test_training_steps_plan_at_full_size(name):
     kernels = [l.kernel for l in interp.launches]
     assert any(k.startswith('conv_gemm') for k in kernels)
     if name == 'convnet_train':
-        assert 'select_window_v4' in kernels and 'scatter_selected_v4' in kernels and any(k.startswith('pad_nd') for k in kernels)
+        assert 'select_window2d_3x3_v4' in kernels and 'scatter_selected2d_3x3_n2x2_v4' in kernels and any(k.startswith('pad_nd') for k in kernels), kernels
 
 
 @pytest.mark.parametrize('f,args', pad_cases, ids=[c[0].__name__ for c in pad_cases])
@@ -226,9 +226,17 @@ def test_pad_hip(f, args):
 @pytest.mark.gpu
 @pytest.mark.parametrize('desc,window,strides,padding,x,select', pool_cases, ids=[c[0] for c in pool_cases])
 def test_select_and_scatter_add_hip(desc, window, strides, padding, x, select):
-    print(f'case: {desc}', flush=True)
+    from vkjax_amd import kernels as K
     g = random(_pooled(x.shape, window, strides, padding)) + 0.25
-    check_against_oracle(pool_grad(window, strides, padding, select), [g, x], exact=True)
+    kernels = []
+    for two_d in (None, False):                              #the kernels for [batch, y, x, channels] where they apply, and the general ones
+        print(f'case: {desc}, 2-D kernels {two_d}', flush=True)
+        with K.overrides(pool_gradient_2d=two_d):
+            _, _, fn = check_against_oracle(pool_grad(window, strides, padding, select), [g, x], exact=True)
+        kernels.append([l.kernel for l in list(fn._jaxpr_interpreters.values())[0].launches if 'select' in l.kernel])
+    assert all('2d' not in k for k in kernels[1])
+    applies = len(window) == 4 and (window[0], window[3]) == (1, 1) and window[1:3] in ((3, 3), (2, 2)) and x.shape[3] % 4 == 0
+    assert all('2d' in k for k in kernels[0]) == applies and bool(kernels[0]), (desc, kernels)
 
 
 @pytest.mark.gpu

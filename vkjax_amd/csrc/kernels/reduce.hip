@@ -860,6 +860,129 @@ __device__ __forceinline__ void scatter_selected_body(uint32_t* __restrict__ out
     }
 }
 
+// The usual pooling layout, [batch, y, x, channels] with a KH x KW window over y and x only and float data: the two
+// passes with everything a thread reads requested before the first value is looked at, 32-bit index arithmetic and
+// contiguous block ranges per XCD, like pool2d above (the general kernels walk their windows one load at a time:
+// 69 + 115 us for the gradient of a 3 x 3 / 2 max pool over 64 x 112 x 112 x 64, where the pool itself takes 34).
+// Same selections and the same sums in the same order as the general kernels. Needs channels % 4 == 0 and fewer than
+// 2^31 bytes on either side; the host checks.
+template <int KH, int KW>
+__device__ __forceinline__ void select_window2d_body(uint32_t* __restrict__ sel_out, const uint32_t* __restrict__ operand, const PoolParams& P) {
+    const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u;
+    if (e0 >= P.n_out) return;
+    const uint32_t C = P.out_dims[3], Wo = P.out_dims[2], Ho = P.out_dims[1];
+    uint32_t r = e0 / C;
+    const uint32_t c = e0 - r * C;
+    const uint32_t wo = r % Wo; r /= Wo;
+    const uint32_t ho = r % Ho, b = r / Ho;
+    const int32_t y0 = (int32_t)(ho * P.stride[1]) - P.pad_low[1], x0 = (int32_t)(wo * P.stride[2]) - P.pad_low[2];
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(operand), 0,
+        (int)(P.in_dims[0] * P.in_dims[1] * P.in_dims[2] * P.in_dims[3] * 4u), 0x00020000);
+    u32x4 v[KH][KW];
+    bool inside[KH][KW];
+#pragma unroll
+    for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx) {
+            const int32_t y = y0 + ky, x = x0 + kx;
+            inside[ky][kx] = (uint32_t)y < P.in_dims[1] && (uint32_t)x < P.in_dims[2];
+            const uint32_t off = ((b * P.in_dims[1] + (uint32_t)y) * P.in_dims[2] + (uint32_t)x) * C + c;
+            v[ky][kx] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, inside[ky][kx] ? off * 4u : 0x80000000u, 0, 0);
+        }
+    const bool want_max = P.op == RED_MAX;
+    float sel[4] = {0.f, 0.f, 0.f, 0.f};
+    uint32_t pick[4] = {0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu};
+    bool have = false;
+#pragma unroll
+    for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx) {
+            // positions outside the array are not candidates (selects, no branches: the loads stay in flight together)
+            const float q[4] = {u2f(v[ky][kx].x), u2f(v[ky][kx].y), u2f(v[ky][kx].z), u2f(v[ky][kx].w)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool keep = have && (want_max ? sel[j] >= q[j] : sel[j] <= q[j]);
+                const bool take = inside[ky][kx] && !keep;
+                sel[j]  = take ? q[j] : sel[j];
+                pick[j] = take ? (uint32_t)(ky * KW + kx) : pick[j];
+            }
+            have = have || inside[ky][kx];
+        }
+    *reinterpret_cast<u32x4*>(sel_out + e0) = u32x4{pick[0], pick[1], pick[2], pick[3]};
+}
+
+// NY x NX: the most windows an element can lie in, ceil(window / stride) per dimension (the host picks the variant):
+// loads for windows that do not exist read nothing, but nine pairs of them where four would do cost a third more time.
+template <int KH, int KW, int NY, int NX>
+__device__ __forceinline__ void scatter_selected2d_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                        const uint32_t* __restrict__ selected, const PoolParams& P) {
+    const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u;
+    if (e0 >= P.n_out) return;
+    const uint32_t C = P.in_dims[3], W = P.in_dims[2], H = P.in_dims[1];
+    uint32_t r = e0 / C;
+    const uint32_t c = e0 - r * C;
+    const uint32_t x = r % W; r /= W;
+    const uint32_t y = r % H, b = r / H;
+    // windows that contain the element: o * stride - pad <= coordinate < o * stride - pad + window; at most KH x KW of them
+    int32_t lo[2], hi[2];
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+        const int32_t s = (int32_t)P.stride[d + 1], a = (int32_t)(d ? x : y) + P.pad_low[d + 1];
+        const int32_t first = a - (d ? KW : KH) + 1;
+        lo[d] = first <= 0 ? 0 : (first + s - 1) / s;
+        hi[d] = a < 0 ? -1 : a / s;
+        if (hi[d] > (int32_t)P.out_dims[d + 1] - 1) hi[d] = (int32_t)P.out_dims[d + 1] - 1;
+    }
+    const uint32_t nwin_bytes = P.out_dims[0] * P.out_dims[1] * P.out_dims[2] * P.out_dims[3] * 4u;
+    const __amdgpu_buffer_rsrc_t r_sel = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(selected), 0, (int)nwin_bytes, 0x00020000),
+                                 r_src = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(source), 0, (int)nwin_bytes, 0x00020000);
+    u32x4 s[NY][NX], g[NY][NX];
+    uint32_t tap[NY][NX];
+#pragma unroll
+    for (int i = 0; i < NY; ++i)
+#pragma unroll
+        for (int j = 0; j < NX; ++j) {
+            const int32_t oy = lo[0] + i, ox = lo[1] + j;
+            const bool ok = oy <= hi[0] && ox <= hi[1];
+            // this element's tap number inside that window (no window: a number no selection holds)
+            tap[i][j] = ok ? (uint32_t)(((int32_t)y + P.pad_low[1] - oy * (int32_t)P.stride[1]) * KW + ((int32_t)x + P.pad_low[2] - ox * (int32_t)P.stride[2]))
+                           : 0xFFFFFFFEu;
+            const uint32_t off = ((b * P.out_dims[1] + (uint32_t)oy) * P.out_dims[2] + (uint32_t)ox) * C + c;
+            s[i][j] = __builtin_amdgcn_raw_buffer_load_b128(r_sel, ok ? off * 4u : 0x80000000u, 0, 0);
+            g[i][j] = __builtin_amdgcn_raw_buffer_load_b128(r_src, ok ? off * 4u : 0x80000000u, 0, 0);
+        }
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NY; ++i)
+#pragma unroll
+        for (int j = 0; j < NX; ++j) {
+            if (s[i][j].x == tap[i][j]) acc[0] += u2f(g[i][j].x);
+            if (s[i][j].y == tap[i][j]) acc[1] += u2f(g[i][j].y);
+            if (s[i][j].z == tap[i][j]) acc[2] += u2f(g[i][j].z);
+            if (s[i][j].w == tap[i][j]) acc[3] += u2f(g[i][j].w);
+        }
+    *reinterpret_cast<u32x4*>(out + e0) = u32x4{f2u(acc[0]), f2u(acc[1]), f2u(acc[2]), f2u(acc[3])};
+}
+
+#define SELECT_WINDOW_2D(KH, KW)                                                                                                    \
+    extern "C" __global__ __launch_bounds__(256) void select_window2d_##KH##x##KW##_v4(uint32_t* __restrict__ sel,                   \
+                                                                                      const uint32_t* __restrict__ operand, PoolParams P) { \
+        select_window2d_body<KH, KW>(sel, operand, P);                                                                              \
+    }
+#define SCATTER_SELECTED_2D(KH, KW, NY, NX)                                                                                         \
+    extern "C" __global__ __launch_bounds__(256) void scatter_selected2d_##KH##x##KW##_n##NY##x##NX##_v4(uint32_t* __restrict__ out, \
+            const uint32_t* __restrict__ source, const uint32_t* __restrict__ selected, PoolParams P) {                             \
+        scatter_selected2d_body<KH, KW, NY, NX>(out, source, selected, P);                                                          \
+    }
+SELECT_WINDOW_2D(3, 3)
+SELECT_WINDOW_2D(2, 2)
+// 3 x 3 windows with strides of 1 (3 x 3 windows per element), 2 (2 x 2) and more (1 x 1); 2 x 2 windows with strides of 1 and more
+SCATTER_SELECTED_2D(3, 3, 3, 3)
+SCATTER_SELECTED_2D(3, 3, 2, 2)
+SCATTER_SELECTED_2D(3, 3, 1, 1)
+SCATTER_SELECTED_2D(2, 2, 2, 2)
+SCATTER_SELECTED_2D(2, 2, 1, 1)
+
 extern "C" __global__ __launch_bounds__(256) void select_window_v1(uint32_t* __restrict__ sel, const uint32_t* __restrict__ operand, PoolParams P) {
     select_window_body<1>(sel, operand, P);
 }

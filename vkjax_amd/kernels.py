@@ -43,6 +43,7 @@ class _Choices:
         conv_general=False,              #never pick the lean kernel variant
         conv_b_general=False,            #element-wise loads of the kernel operand also where 16-byte loads would do
         conv_ksplit=None,                #the four-waves-per-tile kernel: always (where it applies) / never
+        pool_gradient_2d=None,           #the 2-D kernels of a pooling gradient: None = where they apply, False = never
         scatter_bucket_cap=None,         #slots per row in the sorted scatter-add's table of fixed-capacity buckets (0: no table)
         conv_dense_rows=None,            #the kernel for at most 16 output features: None = where it applies, False = never
         conv_mix=None,                   #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
@@ -1135,9 +1136,16 @@ def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, selected: B
     assert tuple(selected.shape) == tuple(source.shape) and selected.dtype == np.uint32
     tail = _u32(RED[op], _RTYPE[operand.dtype], *in_dims, *out_dims, *window, *strides, 1, 1, 1, 1) + _i32(*pad_low)
     n_win, n = source.size, operand.size
-    first  = Launch(f'select_window_v{vec}', (_cdiv(_cdiv(n_win, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+    select, scatter = f'select_window_v{vec}', f'scatter_selected_v{vec}'
+    #[batch, y, x, channels] floats with a 3x3 or 2x2 window over y and x: the kernels that request everything at once
+    if (vec == 4 and window[0] == 1 and strides[0] == 1 and pad_low[0] == 0 and in_dims[0] == out_dims[0] and CHOICES.pool_gradient_2d is not False
+            and (window[1], window[2]) in ((3, 3), (2, 2)) and operand.dtype == np.float32 and n * 4 < 2**31 and n_win * 4 < 2**31):
+        #(an element lies in at most ceil(window / stride) windows per dimension; the variants are square in that count)
+        most = max(_cdiv(window[1], strides[1]), _cdiv(window[2], strides[2]))
+        select, scatter = f'select_window2d_{window[1]}x{window[2]}_v4', f'scatter_selected2d_{window[1]}x{window[2]}_n{most}x{most}_v4'
+    first  = Launch(select, (_cdiv(_cdiv(n_win, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                     [(selected, 0), (operand, 0)], _u32(n_win) + tail, bytes_moved=4 * (operand.size + source.size))
-    second = Launch(f'scatter_selected_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
+    second = Launch(scatter, (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                     [(out, 0), (source, 0), (selected, 0)], _u32(n) + tail, bytes_moved=4 * (operand.size + 2 * source.size))
     return [first, second]
 

@@ -297,6 +297,13 @@ _ACT  = (64, 56, 56, 256)          #a ResNet-50 activation of 51.4 M elements (2
 _WIDE = (64, 112, 112, 64)         #the input of ResNet-50's max-pool
 _N64M = 1 << 26
 
+def _max_pool_gradient(x, g):
+    '''The gradient that a 3 x 3 / 2 max pool hands back to its input for the cotangent g (select_and_scatter_add).'''
+    import vkjax_amd.minijax as mj
+    pooled = lambda v: lax.reduce_window(v, -jnp.inf, lax.max, (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (0, 1), (0, 1), (0, 0)))
+    return mj.grad(lambda v, c: (pooled(v) * c).sum())(x, g)
+
+
 #name -> (function, inputs, ALGORITHMIC bytes of one evaluation: every operand read once and every result written once)
 PRIMITIVES: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable, tp.Callable]] = {
     'reduce_sum rows 65536x1000':   (lambda x: jnp.sum(x, axis=1), lambda: [_uniform_words(65536000, 1).reshape(65536, 1000)], lambda a: a[0].nbytes + 4 * 65536),
@@ -325,6 +332,12 @@ PRIMITIVES: tp.Dict[str, tp.Tuple[tp.Callable, tp.Callable, tp.Callable]] = {
     'transpose NHWC to NCHW 64x56x56x256': (lambda x: lax.transpose(x, (0, 3, 1, 2)), lambda: [_uniform_words(int(np.prod(_ACT)), 18).reshape(_ACT)], lambda a: 2 * a[0].nbytes),
     'pad height and width 64x56x56x256': (lambda x: lax.pad(x, 0.0, ((0, 0, 0), (1, 1, 0), (1, 1, 0), (0, 0, 0))),
                                      lambda: [_uniform_words(int(np.prod(_ACT)), 19).reshape(_ACT)], lambda a: a[0].nbytes + 64 * 58 * 58 * 256 * 4),
+    'iota 64M':                     (lambda x: lax.broadcasted_iota(np.float32, (1 << 13, 1 << 13), 1), lambda: [np.float32(0.0)], lambda a: 4 * _N64M),      #(the argument is not used: a program of one launch that only writes)
+    'concatenate 2 x 32M':          (lambda x, y: lax.concatenate([x, y], 0), lambda: [_uniform_words(_N64M // 2, 20), _uniform_words(_N64M // 2, 21)],
+                                     lambda a: 2 * (a[0].nbytes + a[1].nbytes)),
+    'max pool gradient 3x3 s2 64x112x112x64': (_max_pool_gradient, lambda: [_uniform_words(int(np.prod(_WIDE)), 22).reshape(_WIDE),
+                                                                            _uniform_words(int(np.prod(_WIDE)) // 4, 23).reshape(64, 56, 56, 64)],
+                                     lambda a: 2 * a[0].nbytes + a[1].nbytes),
     'gather rows 262144x1KB of 65536': (lambda t, i: t[i], lambda: gather_scatter_inputs()[:2], lambda a: 2 * a[1].size * a[0].shape[1] * 4 + a[1].nbytes),
     'scatter-add rows 262144x1KB into 65536': (lambda i, u: jnp.index_add(jnp.zeros((65536, 256), np.float32), i, u), lambda: gather_scatter_inputs()[1:],
                                      lambda a: a[1].nbytes + a[0].nbytes + 65536 * 256 * 4),
