@@ -820,6 +820,29 @@ def test_first_launch_starts_while_its_argument_arrives():
         assert np.array_equal(np.asarray(got[0]).reshape(-1), mean.reshape(-1)) and np.array_equal(np.asarray(got[1]).reshape(-1), samples.reshape(-1))
     expected, _ = oracle_outputs(stem, [params, images[2][:2]])
     assert np.allclose(results[2][0][:2], expected[0], rtol=1e-4, atol=1e-5) and np.allclose(results[2][1][:2], expected[1], rtol=1e-4, atol=1e-5)
+    #the general kernels: 1x1 and padded 3x3 convolutions whose parts run the whole launch's kernel (images are independent
+    #of each other, and a wave adds up its contraction in one order whatever tile it works on)
+    def conv_then_mean(w, b, x, padding):
+        z = nn.relu(lax.conv_general_dilated(x, w, (1, 1), padding, dimension_numbers=W.NHWC) + b)
+        return z.mean(axis=(1, 2)), z[:, ::29, ::31, :]
+    with_parts = 0
+    for shape, cout, k, padding in (((32, 64, 64, 64), 32, 1, 'VALID'), ((8, 128, 128, 64), 64, 1, 'VALID'), ((8, 128, 128, 64), 64, 3, 'SAME'),
+                                    ((16, 96, 96, 32), 64, 3, 'SAME')):
+        print(f'case: first launch in parts, {k}x{k} convolution over {shape} to {cout} features', flush=True)
+        w, b = frozen((rng.standard_normal((k, k, shape[3], cout)) / 8).astype(np.float32)), frozen(rng.standard_normal(cout).astype(np.float32))
+        g = vkjax_amd.wrap(lambda w, b, x: conv_then_mean(w, b, x, padding), frontend='minijax')
+        xs = [rng.standard_normal(shape).astype(np.float32) for _ in range(2)]
+        got = [g(w, b, x) for x in xs]
+        interp = list(g._jaxpr_interpreters.values())[0]
+        with_parts += bool(interp.early_parts)
+        for x, (mean, samples) in zip(xs, got):
+            interp.upload_inputs(w, b, x)
+            interp.replay(1)
+            whole = interp.read_outputs()
+            assert np.array_equal(np.asarray(mean).reshape(-1), whole[0].reshape(-1)) and np.array_equal(np.asarray(samples).reshape(-1), whole[1].reshape(-1))
+        expected, _ = oracle_outputs(lambda w, b, x: conv_then_mean(w, b, x, padding), [w, b, xs[1][:1]])
+        assert np.allclose(got[1][0][:1], expected[0], rtol=1e-4, atol=1e-5) and np.allclose(got[1][1][:1], expected[1], rtol=1e-4, atol=1e-5)
+    assert with_parts >= 2
     #a first launch that is no convolution over a large argument, or one in the mixed tiling: no parts
     small = vkjax_amd.wrap(stem, frontend='minijax')
     small(params, images[0][:4])
