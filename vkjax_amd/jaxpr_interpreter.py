@@ -86,6 +86,7 @@ class JaxprInterpreter:
         #lower every op now so that unsupported layouts fail at build time, not at run time
         self.launches = [op.launch for op in self.all_ops]
         self.lane_plan = lanes.plan(self.all_ops, self.launches) if self.two_lanes else None
+        self.early_parts = []
 
         if isinstance(self.mgr, PlanOnlyDevice):
             return
