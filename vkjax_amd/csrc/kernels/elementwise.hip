@@ -24,7 +24,9 @@ struct EwParams {
                                        // bits 4-5: how the operand is addressed: 0 through its strides, 1 like the
                                        // output (element = base + linear index), 2 by the fastest dimension only
                                        // (element = base + coordinate), 3 a single element (base);
-                                       // bit6: every vector of a thread reads the same elements of the operand
+                                       // bit6: every vector of a thread reads the same elements of the operand;
+                                       // flags[0] bit8: the result is stored past the caches (nontemporal): a large
+                                       // array that no launch will find there anyway (relu on 64 M elements 92 -> 76 us)
     uint32_t imm[EW_MAX_STEPS];        // immediate (integer_pow exponent)
     int32_t  stride[EW_MAX_STEPS][4];  // operand strides per collapsed dim, in elements
     uint32_t nbytes[EW_MAX_STEPS];     // bytes readable from each operand pointer (0 = no operand)
@@ -77,6 +79,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     constexpr int U = (NS == 4 || NS == 6) ? 2 : 1;
     constexpr int W = U * VEC;                                    // values per thread
     const uint32_t first = (block * U * 256u + threadIdx.x) * VEC;          // the host keeps n below 2^31
+    const bool stream_out = flags[0] & 256u;
     if (first >= n) return;
 
     // Every operand is read through a buffer descriptor with one branch-free load per slot: 16 bytes
@@ -198,7 +201,10 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
         if (i0 < n) {
             if constexpr (VEC == 4) {
                 u32x4 t; t.x = acc[u * 4]; t.y = acc[u * 4 + 1]; t.z = acc[u * 4 + 2]; t.w = acc[u * 4 + 3];
-                *reinterpret_cast<u32x4*>(out + i0) = t;
+                // (a buffer store: written as two stores through the same pointer, one of them nontemporal, the compiler
+                // merges them into one plain store)
+                if (stream_out) __builtin_amdgcn_raw_buffer_store_b128(t, make_rsrc(out, n * 4u), i0 * 4u, 0, 2);
+                else *reinterpret_cast<u32x4*>(out + i0) = t;
             } else {
                 out[i0] = acc[u];
             }
@@ -218,7 +224,8 @@ struct EwAffineParams {
     uint32_t n, cq;                 // elements; C / 4
     uint32_t cq_magic, cq_shift;    // v / cq = mulhi(v, magic) >> shift for v < 2^31 (magic 0: cq == 1)
     uint32_t nsum;                  // 0..3
-    uint32_t flags;                 // bit0 - vsub, bit1 * vmul, bit2 + vadd, bit3 + full, bit4 max(., floor)
+    uint32_t flags;                 // bit0 - vsub, bit1 * vmul, bit2 + vadd, bit3 + full, bit4 max(., floor);
+                                    // bit5: the result is stored past the caches (a large array, see EwParams)
 };
 
 // SKIP = false: every load is issued, through a descriptor of size 0 for an absent operand (such a load returns zeros
@@ -287,7 +294,8 @@ __device__ __forceinline__ void ew_affine_body(float* __restrict__ out, const fl
                 y[j] = v;
             }
         }
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 0);
+        if (fl & 32u) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 2);
+        else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 0);
     }
 }
 
@@ -421,9 +429,11 @@ __device__ __forceinline__ void concat_body(uint32_t* __restrict__ out, const ui
     const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * VEC;
     if (i >= P.n) return;
     const uint32_t r = i / P.part_inner, c = i - r * P.part_inner;
-    uint32_t* dst = out + (uint64_t)r * P.out_inner + P.out_offset + c;
-    if constexpr (VEC == 4) *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(in + i);
-    else *dst = in[i];
+    const uint64_t at = (uint64_t)r * P.out_inner + P.out_offset + c;
+    // (the rows of the result this part reaches into: n / part_inner of them)
+    const uint64_t reach = ((uint64_t)(P.n / P.part_inner) * P.out_inner + P.out_offset) * 4u;
+    if constexpr (VEC == 4) store_x4(out, at, *reinterpret_cast<const u32x4*>(in + i), streams_result((uint64_t)P.n * 4u) && reach < (1ull << 32), (uint32_t)reach);
+    else out[at] = in[i];
 }
 extern "C" __global__ __launch_bounds__(256) void concat_part_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, ConcatParams P) {
     concat_body<1>(out, in, P);
@@ -470,7 +480,7 @@ __device__ __forceinline__ void pad_body(uint32_t* __restrict__ out, const uint3
     if constexpr (VEC == 4) {
         u32x4 q = u32x4{v, v, v, v};
         if (inside) q = *reinterpret_cast<const u32x4*>(in + off);
-        *reinterpret_cast<u32x4*>(out + e0) = q;
+        store_x4(out, e0, q, streams_result((uint64_t)P.n * 4u), P.n * 4u);
     } else {
         out[e0] = inside ? in[off] : v;
     }
@@ -524,7 +534,8 @@ __device__ __forceinline__ void transpose_v4_body(uint32_t* __restrict__ out, co
     // column of tiles all start in the same memory channel, and workgroups that run together would queue there.
     const uint32_t j0 = bx * 64u, i0 = ((by + bx) % gy) * 64u, b = bz;
     const uint32_t* src = in + (int64_t)b * P.sb;
-    uint32_t* dst = out + (uint64_t)b * P.I * P.J;
+    const uint64_t total = (uint64_t)P.B * P.I * P.J * 4u;
+    const bool stream = streams_result(total);
 #pragma unroll
     for (uint32_t p = 0; p < 4; ++p) {
         const uint32_t j = j0 + tr + 16u * p, i = i0 + 4u * t16;
@@ -542,7 +553,7 @@ __device__ __forceinline__ void transpose_v4_body(uint32_t* __restrict__ out, co
             u32x4 v;
             v.x = tile[4u * t16][tr + 16u * p]; v.y = tile[4u * t16 + 1u][tr + 16u * p];
             v.z = tile[4u * t16 + 2u][tr + 16u * p]; v.w = tile[4u * t16 + 3u][tr + 16u * p];
-            *reinterpret_cast<u32x4*>(dst + (uint64_t)i * P.J + j) = v;
+            store_x4(out, (uint64_t)b * P.I * P.J + (uint64_t)i * P.J + j, v, stream, (uint32_t)total);
         }
     }
 }
@@ -559,7 +570,8 @@ __device__ __forceinline__ void transpose_v4_t128_body(uint32_t* __restrict__ ou
     const uint32_t t32 = threadIdx.x & 31u, tr = threadIdx.x >> 5;        // 32 vectors per tile row, 8 rows per pass
     const uint32_t j0 = bx * 128u, i0 = ((by + bx) % gy) * 128u, b = bz;
     const uint32_t* src = in + (int64_t)b * P.sb;
-    uint32_t* dst = out + (uint64_t)b * P.I * P.J;
+    const uint64_t total = (uint64_t)P.B * P.I * P.J * 4u;
+    const bool stream = streams_result(total);
     u32x4 v[16];
 #pragma unroll
     for (uint32_t p = 0; p < 16; ++p) {
@@ -580,7 +592,7 @@ __device__ __forceinline__ void transpose_v4_t128_body(uint32_t* __restrict__ ou
             u32x4 w;
             w.x = tile[4u * t32][tr + 8u * p]; w.y = tile[4u * t32 + 1u][tr + 8u * p];
             w.z = tile[4u * t32 + 2u][tr + 8u * p]; w.w = tile[4u * t32 + 3u][tr + 8u * p];
-            *reinterpret_cast<u32x4*>(dst + (uint64_t)i * P.J + j) = w;
+            store_x4(out, (uint64_t)b * P.I * P.J + (uint64_t)i * P.J + j, w, stream, (uint32_t)total);
         }
     }
 }

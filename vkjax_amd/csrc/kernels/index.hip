@@ -35,7 +35,8 @@ __device__ __forceinline__ void gather_rows_body(uint32_t* __restrict__ out, con
     }
     r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
     const uint32_t* src = table + (uint64_t)r * P.row_len + c;
-    if constexpr (VEC == 4) *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
+    const uint64_t total = (uint64_t)P.n_idx * P.row_len * 4u;
+    if constexpr (VEC == 4) store_x4(out, (uint64_t)i * P.row_len + c, *reinterpret_cast<const u32x4*>(src), streams_result(total), (uint32_t)total);
     else *dst = *src;
 }
 
