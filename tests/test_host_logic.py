@@ -567,3 +567,24 @@ def test_which_argument_leaves_count_as_immutable():
     assert _is_immutable(np.frombuffer(b'\x00' * 16, np.float32))         #backed by a bytes object
     assert not _is_immutable(np.frombuffer(bytearray(16), np.float32))
     assert not _is_immutable(3.0) and not _is_immutable(np.float32(3.0)) and not _may_change_in_place(3.0)
+
+
+def test_large_results_that_nothing_reads_again_are_stored_past_the_caches():
+    '''Kernels that can store their result with the nontemporal hint are told to (bit 31 of their first parameter word)
+    for results of 64 MB and more that no later launch of the program reads; a result that a later launch reads, a small
+    one, and a kernel without that ability are left alone; a later launch that only writes the array (the second part
+    of a concatenation) does not count as a reader.'''
+    from vkjax_amd import kernels as K
+    streamed = lambda interp: [(l.kernel, int(np.frombuffer(l.params[:4], np.uint32)[0]) >> 31) for l in interp.launches]
+    big, small = np.zeros(1 << 24, np.float32), np.zeros(1 << 20, np.float32)
+    plan = lambda f, *args: JaxprInterpreter(mj.make_jaxpr(f)(*args), plan_only=True)
+    assert streamed(plan(lambda x: jnp.exp(x), big)) == [('ew_chain_v4_s2', 1)]
+    assert streamed(plan(lambda x: jnp.exp(x), small)) == [('ew_chain_v4_s2', 0)]
+    #the exponential is read by the sum: only a launch whose result leaves the program streams it
+    assert streamed(plan(lambda x: jnp.sum(jnp.exp(x).reshape(4096, 4096), axis=0), big)) [0][1] == 0
+    both = streamed(plan(lambda x: (jnp.exp(x), jnp.exp(x).reshape(4096, 4096).T), big))
+    #(the result exp(x) keeps a launch of its own: streamed; the one the transposition reads is not; the transposed result is)
+    assert [flag for _, flag in both] == [1, 0, 1] and both[2][0].startswith('transpose_tiled')
+    assert streamed(plan(lambda x, y: lax.concatenate([x, y], 0), big, big)) == [('concat_part_v4', 1), ('concat_part_v4', 1)]
+    for launch in plan(lambda x: jnp.exp(x), big).launches:
+        assert launch.streamable and K.with_streamed_result(launch._replace(params=K._u32(launch.params and 5) + launch.params[4:])).params[:4] == K._u32(5 | 1 << 31)

@@ -39,13 +39,16 @@ __device__ __forceinline__ void buffer_store_x1(float v, __amdgpu_buffer_rsrc_t 
 __device__ __forceinline__ float buffer_load_x1_nt(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 2));
 }
-// Results of this size and more are stored with the nontemporal hint: an array that no later launch will find in
-// the caches anyway only pushes out what could be reused, and the stores of a launch that reads and writes run faster
-// past the L2 (relu on 64 M elements 92 -> 76 us). Arrays of 4 GiB and more keep plain stores (a buffer addresses 32 bits).
-#define STREAM_RESULT_MIN_BYTES (64ull << 20)
-__device__ __forceinline__ bool streams_result(uint64_t result_bytes) {
-    return result_bytes >= STREAM_RESULT_MIN_BYTES && result_bytes < (1ull << 32);
-}
+// Bit 31 of the first word of a kernel's parameters (an element count below 2^31 in every kernel that looks at it):
+// the result is stored with the nontemporal hint. The host sets it for large results that no later launch of the
+// program reads (they leave for the host, or stay where they are): such an array only pushes out of the caches what
+// could be reused, and the stores of a launch that reads and writes run faster past the L2 (relu on 64 M elements
+// 92 -> 76 us). Results that the next launch reads are left to the caches (256 MB behind the L2s: a training step
+// whose backward kernels streamed their results was 0.15 ms slower). Only for results below 4 GiB (a buffer
+// addresses 32 bits); the host checks.
+#define STREAM_RESULT_BIT 0x80000000u
+__device__ __forceinline__ bool streams_result(uint32_t first_word) { return (first_word & STREAM_RESULT_BIT) != 0u; }
+__device__ __forceinline__ uint32_t without_stream_bit(uint32_t first_word) { return first_word & ~STREAM_RESULT_BIT; }
 // base[element .. element + 4) = v; `stream`: past the caches. (Through a buffer: written as two stores through one
 // pointer, one of them nontemporal, the compiler merges them into one plain store.)
 __device__ __forceinline__ void store_x4(uint32_t* base, uint64_t element, u32x4 v, bool stream, uint32_t result_bytes) {

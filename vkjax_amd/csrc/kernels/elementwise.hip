@@ -14,7 +14,7 @@
 #define EW_MAX_STEPS 8
 
 struct EwParams {
-    uint32_t n;                        // output elements
+    uint32_t n;                        // output elements; bit 31: the result is stored past the caches (STREAM_RESULT_BIT)
     uint32_t ndim;                     // 1..4 collapsed output dims
     uint32_t dims[4];                  // row-major, dims[ndim-1] fastest; unused = 1
     uint32_t nsteps;                   // 1..8; step 0 is the initial load
@@ -24,9 +24,7 @@ struct EwParams {
                                        // bits 4-5: how the operand is addressed: 0 through its strides, 1 like the
                                        // output (element = base + linear index), 2 by the fastest dimension only
                                        // (element = base + coordinate), 3 a single element (base);
-                                       // bit6: every vector of a thread reads the same elements of the operand;
-                                       // flags[0] bit8: the result is stored past the caches (nontemporal): a large
-                                       // array that no launch will find there anyway (relu on 64 M elements 92 -> 76 us)
+                                       // bit6: every vector of a thread reads the same elements of the operand
     uint32_t imm[EW_MAX_STEPS];        // immediate (integer_pow exponent)
     int32_t  stride[EW_MAX_STEPS][4];  // operand strides per collapsed dim, in elements
     uint32_t nbytes[EW_MAX_STEPS];     // bytes readable from each operand pointer (0 = no operand)
@@ -47,7 +45,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
                                               const EwParams& P, const uint32_t block) {
     // All fields are read first and pinned afterwards: an inline-asm statement is a boundary for the instruction
     // scheduler, and loads issued behind the first pin would wait for a second round trip to the argument block.
-    uint32_t n = P.n, ndim = P.ndim, nsteps = P.nsteps;
+    uint32_t n = without_stream_bit(P.n), ndim = P.ndim, nsteps = P.nsteps;
     uint32_t dims[4], op[NS], flags[NS], imm[NS], nbytes[NS], base[NS];
     int32_t  stride[NS][4];
     uint32_t dim_magic[4], dim_shift[4];
@@ -79,7 +77,7 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
     constexpr int U = (NS == 4 || NS == 6) ? 2 : 1;
     constexpr int W = U * VEC;                                    // values per thread
     const uint32_t first = (block * U * 256u + threadIdx.x) * VEC;          // the host keeps n below 2^31
-    const bool stream_out = flags[0] & 256u;
+    const bool stream_out = streams_result(P.n);
     if (first >= n) return;
 
     // Every operand is read through a buffer descriptor with one branch-free load per slot: 16 bytes
@@ -221,11 +219,10 @@ __device__ __forceinline__ void ew_chain_body(uint32_t* __restrict__ out, const 
 // spends 750 instructions and 170 branches per wave on such a chain, which is most of a small launch's duration and
 // a quarter of the bandwidth of a large one. n and C are multiples of 4; two 16-byte vectors per thread.
 struct EwAffineParams {
-    uint32_t n, cq;                 // elements; C / 4
+    uint32_t n, cq;                 // elements (bit 31: STREAM_RESULT_BIT); C / 4
     uint32_t cq_magic, cq_shift;    // v / cq = mulhi(v, magic) >> shift for v < 2^31 (magic 0: cq == 1)
     uint32_t nsum;                  // 0..3
-    uint32_t flags;                 // bit0 - vsub, bit1 * vmul, bit2 + vadd, bit3 + full, bit4 max(., floor);
-                                    // bit5: the result is stored past the caches (a large array, see EwParams)
+    uint32_t flags;                 // bit0 - vsub, bit1 * vmul, bit2 + vadd, bit3 + full, bit4 max(., floor)
 };
 
 // SKIP = false: every load is issued, through a descriptor of size 0 for an absent operand (such a load returns zeros
@@ -237,7 +234,7 @@ __device__ __forceinline__ void ew_affine_body(float* __restrict__ out, const fl
                                                const float* vsub, const float* vmul, const float* vadd, const float* full, const float* floor_,
                                                const EwAffineParams& P) {
     constexpr int U = 2;
-    const uint32_t nb = P.n * 4u, cb = P.cq * 16u, fl = P.flags;
+    const uint32_t nb = without_stream_bit(P.n) * 4u, cb = P.cq * 16u, fl = P.flags;
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out, nb), r_first = make_rsrc(first, nb),
         r_s1 = make_rsrc(s1, P.nsum >= 1u ? nb : 0u), r_s2 = make_rsrc(s2, P.nsum >= 2u ? nb : 0u), r_s3 = make_rsrc(s3, P.nsum >= 3u ? nb : 0u),
         r_sub = make_rsrc(vsub, (fl & 1u) ? cb : 0u), r_mul = make_rsrc(vmul, (fl & 2u) ? cb : 0u), r_add = make_rsrc(vadd, (fl & 4u) ? cb : 0u),
@@ -294,7 +291,7 @@ __device__ __forceinline__ void ew_affine_body(float* __restrict__ out, const fl
                 y[j] = v;
             }
         }
-        if (fl & 32u) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 2);
+        if (streams_result(P.n)) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 2);
         else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), r_out, off[u], 0, 0);
     }
 }
@@ -426,13 +423,13 @@ struct ConcatParams { uint32_t n, part_inner, out_inner, out_offset; };
 // VEC = 4 needs part_inner, out_inner and out_offset to be multiples of 4.
 template <int VEC>
 __device__ __forceinline__ void concat_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const ConcatParams& P) {
-    const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * VEC;
-    if (i >= P.n) return;
+    const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * VEC, n = without_stream_bit(P.n);
+    if (i >= n) return;
     const uint32_t r = i / P.part_inner, c = i - r * P.part_inner;
     const uint64_t at = (uint64_t)r * P.out_inner + P.out_offset + c;
-    // (the rows of the result this part reaches into: n / part_inner of them)
-    const uint64_t reach = ((uint64_t)(P.n / P.part_inner) * P.out_inner + P.out_offset) * 4u;
-    if constexpr (VEC == 4) store_x4(out, at, *reinterpret_cast<const u32x4*>(in + i), streams_result((uint64_t)P.n * 4u) && reach < (1ull << 32), (uint32_t)reach);
+    // (the rows of the result this part reaches into: n / part_inner of them; below 4 GiB when the host asks for streaming)
+    const uint64_t reach = ((uint64_t)(n / P.part_inner) * P.out_inner + P.out_offset) * 4u;
+    if constexpr (VEC == 4) store_x4(out, at, *reinterpret_cast<const u32x4*>(in + i), streams_result(P.n), (uint32_t)reach);
     else out[at] = in[i];
 }
 extern "C" __global__ __launch_bounds__(256) void concat_part_v1(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, ConcatParams P) {
@@ -458,8 +455,8 @@ struct PadParams {
 template <int VEC>
 __device__ __forceinline__ void pad_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
                                          const uint32_t* __restrict__ value, const PadParams& P) {
-    const uint32_t e0 = (blockIdx.x * 256u + threadIdx.x) * VEC;
-    if (e0 >= P.n) return;
+    const uint32_t e0 = (blockIdx.x * 256u + threadIdx.x) * VEC, n = without_stream_bit(P.n);
+    if (e0 >= n) return;
     uint32_t r = e0, off = 0, mul = 1;
     bool inside = true;
 #pragma unroll
@@ -480,7 +477,7 @@ __device__ __forceinline__ void pad_body(uint32_t* __restrict__ out, const uint3
     if constexpr (VEC == 4) {
         u32x4 q = u32x4{v, v, v, v};
         if (inside) q = *reinterpret_cast<const u32x4*>(in + off);
-        store_x4(out, e0, q, streams_result((uint64_t)P.n * 4u), P.n * 4u);
+        store_x4(out, e0, q, streams_result(P.n), n * 4u);
     } else {
         out[e0] = inside ? in[off] : v;
     }
@@ -498,7 +495,7 @@ extern "C" __global__ __launch_bounds__(256) void pad_nd_v4(uint32_t* __restrict
 // [B, I, J]. The strided gather of the element-wise kernel touches a new cache line per element on
 // one side; here a 64 x 64 tile goes through LDS, read along i (contiguous in `in`) and written
 // along j (contiguous in `out`). Covers 2-D transposes and NHWC <-> NCHW style permutations.
-struct TransposeParams { uint32_t B, I, J; int32_t sb; uint32_t sj; };      // sb may be negative (a reversed leading dimension)
+struct TransposeParams { uint32_t B, I, J; int32_t sb; uint32_t sj; };      // sb may be negative (a reversed leading dimension); bit 31 of B: STREAM_RESULT_BIT
 
 extern "C" __global__ __launch_bounds__(256) void transpose_tiled(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
                                                                   TransposeParams P) {
@@ -534,8 +531,8 @@ __device__ __forceinline__ void transpose_v4_body(uint32_t* __restrict__ out, co
     // column of tiles all start in the same memory channel, and workgroups that run together would queue there.
     const uint32_t j0 = bx * 64u, i0 = ((by + bx) % gy) * 64u, b = bz;
     const uint32_t* src = in + (int64_t)b * P.sb;
-    const uint64_t total = (uint64_t)P.B * P.I * P.J * 4u;
-    const bool stream = streams_result(total);
+    const uint64_t total = (uint64_t)without_stream_bit(P.B) * P.I * P.J * 4u;      // (below 4 GiB when the host asks for streaming)
+    const bool stream = streams_result(P.B);
 #pragma unroll
     for (uint32_t p = 0; p < 4; ++p) {
         const uint32_t j = j0 + tr + 16u * p, i = i0 + 4u * t16;
@@ -570,8 +567,8 @@ __device__ __forceinline__ void transpose_v4_t128_body(uint32_t* __restrict__ ou
     const uint32_t t32 = threadIdx.x & 31u, tr = threadIdx.x >> 5;        // 32 vectors per tile row, 8 rows per pass
     const uint32_t j0 = bx * 128u, i0 = ((by + bx) % gy) * 128u, b = bz;
     const uint32_t* src = in + (int64_t)b * P.sb;
-    const uint64_t total = (uint64_t)P.B * P.I * P.J * 4u;
-    const bool stream = streams_result(total);
+    const uint64_t total = (uint64_t)without_stream_bit(P.B) * P.I * P.J * 4u;      // (below 4 GiB when the host asks for streaming)
+    const bool stream = streams_result(P.B);
     u32x4 v[16];
 #pragma unroll
     for (uint32_t p = 0; p < 16; ++p) {

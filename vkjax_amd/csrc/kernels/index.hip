@@ -14,16 +14,16 @@
 
 // wrap: added to negative indices first (0: nothing) - the normalisation `select(i < 0, i + n, i)` that tracing puts in
 // front of an indexing operation, taken over from an element-wise launch of its own
-struct GatherRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride, fill_mode, fill_bits, wrap; };
+struct GatherRowsParams { uint32_t n_idx, row_len, n_rows, idx_stride, fill_mode, fill_bits, wrap; };      // bit 31 of n_idx: STREAM_RESULT_BIT
 
 // out[i, :] = table[clamp(idx[i*idx_stride]), :]; with fill_mode, rows outside the table read as fill_bits instead
 // (jax's GatherScatterMode.FILL_OR_DROP)
 template <int VEC>
 __device__ __forceinline__ void gather_rows_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ table,
                                                  const int32_t* __restrict__ idx, const GatherRowsParams& P) {
-    const uint32_t vpr = P.row_len / VEC;
+    const uint32_t vpr = P.row_len / VEC, n_idx = without_stream_bit(P.n_idx);
     const uint64_t q = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-    if (q >= (uint64_t)P.n_idx * vpr) return;
+    if (q >= (uint64_t)n_idx * vpr) return;
     const uint32_t i = (uint32_t)(q / vpr), c = (uint32_t)(q - (uint64_t)i * vpr) * VEC;
     int32_t r = idx[(uint64_t)i * P.idx_stride];
     r = r < 0 ? (int32_t)((uint32_t)r + P.wrap) : r;
@@ -35,8 +35,7 @@ __device__ __forceinline__ void gather_rows_body(uint32_t* __restrict__ out, con
     }
     r = r < 0 ? 0 : (r > (int32_t)P.n_rows - 1 ? (int32_t)P.n_rows - 1 : r);
     const uint32_t* src = table + (uint64_t)r * P.row_len + c;
-    const uint64_t total = (uint64_t)P.n_idx * P.row_len * 4u;
-    if constexpr (VEC == 4) store_x4(out, (uint64_t)i * P.row_len + c, *reinterpret_cast<const u32x4*>(src), streams_result(total), (uint32_t)total);
+    if constexpr (VEC == 4) store_x4(out, (uint64_t)i * P.row_len + c, *reinterpret_cast<const u32x4*>(src), streams_result(P.n_idx), n_idx * P.row_len * 4u);
     else *dst = *src;
 }
 

@@ -623,7 +623,7 @@ extern "C" __global__ __launch_bounds__(256) void reduce_general(uint32_t* __res
 // per thread; it requires window = stride = dilation = 1 and no padding on that dimension and
 // a last dimension divisible by 4.
 struct PoolParams {
-    uint32_t n_out;                 // output elements (VEC units are derived in-kernel)
+    uint32_t n_out;                 // output elements (VEC units are derived in-kernel); scatter_selected: bit 31 is STREAM_RESULT_BIT
     uint32_t op, type;              // RED_MAX or RED_SUM
     uint32_t in_dims[4], out_dims[4];
     uint32_t window[4], stride[4], dilation[4];
@@ -807,7 +807,7 @@ template <int VEC>
 __device__ __forceinline__ void scatter_selected_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
                                                       const uint32_t* __restrict__ selected, const PoolParams& P) {
     const uint64_t e0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * VEC;
-    if (e0 >= P.n_out) return;
+    if (e0 >= without_stream_bit(P.n_out)) return;
     int32_t c[4];
     {
         uint64_t r = e0;
@@ -854,7 +854,7 @@ __device__ __forceinline__ void scatter_selected_body(uint32_t* __restrict__ out
     }
     if constexpr (VEC == 4) {
         u32x4 r; r.x = f2u(acc[0]); r.y = f2u(acc[1]); r.z = f2u(acc[2]); r.w = f2u(acc[3]);
-        *reinterpret_cast<u32x4*>(out + e0) = r;
+        store_x4(out, e0, r, streams_result(P.n_out), without_stream_bit(P.n_out) * 4u);
     } else {
         out[e0] = f2u(acc[0]);
     }
@@ -916,8 +916,8 @@ __device__ __forceinline__ void select_window2d_body(uint32_t* __restrict__ sel_
 template <int KH, int KW, int NY, int NX>
 __device__ __forceinline__ void scatter_selected2d_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
                                                         const uint32_t* __restrict__ selected, const PoolParams& P) {
-    const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u;
-    if (e0 >= P.n_out) return;
+    const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u, n_out = without_stream_bit(P.n_out);
+    if (e0 >= n_out) return;
     const uint32_t C = P.in_dims[3], W = P.in_dims[2], H = P.in_dims[1];
     uint32_t r = e0 / C;
     const uint32_t c = e0 - r * C;
@@ -961,7 +961,7 @@ __device__ __forceinline__ void scatter_selected2d_body(uint32_t* __restrict__ o
             if (s[i][j].z == tap[i][j]) acc[2] += u2f(g[i][j].z);
             if (s[i][j].w == tap[i][j]) acc[3] += u2f(g[i][j].w);
         }
-    *reinterpret_cast<u32x4*>(out + e0) = u32x4{f2u(acc[0]), f2u(acc[1]), f2u(acc[2]), f2u(acc[3])};
+    store_x4(out, e0, u32x4{f2u(acc[0]), f2u(acc[1]), f2u(acc[2]), f2u(acc[3])}, streams_result(P.n_out), n_out * 4u);
 }
 
 #define SELECT_WINDOW_2D(KH, KW)                                                                                                    \

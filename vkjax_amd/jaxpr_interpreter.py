@@ -84,7 +84,7 @@ class JaxprInterpreter:
                 b.accesses.append(np.inf)
         self.bufferpool.create_tensors()
         #lower every op now so that unsupported layouts fail at build time, not at run time
-        self.launches = [op.launch for op in self.all_ops]
+        self.launches = self._stream_unread_results([op.launch for op in self.all_ops])
         self.lane_plan = lanes.plan(self.all_ops, self.launches) if self.two_lanes else None
         self.early_parts = []
 
@@ -122,6 +122,29 @@ class JaxprInterpreter:
                 continue
             self._output_slots.append(self.sequence.record_download(b.tensor, b.nbytes()))
             self._output_sizes.append(b.size)
+
+    def _stream_unread_results(self, launches):
+        '''Large results that no later launch of the program reads (they leave for the host, or simply stay) are stored
+        past the caches by the kernels that can do that (kernels.with_streamed_result): they would only push out what the
+        following launches could find there. Results that a later launch reads stay with the caches: the next launch often
+        finds a good part of them in the 256 MB behind the L2s.'''
+        touched_later = set()
+        result = list(launches)
+        for k in range(len(launches) - 1, -1, -1):
+            launch = launches[k]
+            members = launch.members or (launch,)
+            if launch.streamable and not launch.members:
+                out = launch.buffers[0][0]
+                nbytes = out.size * 4 if out is not None else 0
+                if (out is not None and out.tensor is not None and id(out.tensor) not in touched_later
+                        and K.STREAM_RESULT_MIN_BYTES <= nbytes < 2**32):
+                    result[k] = K.with_streamed_result(launch)
+            for m in members:
+                #(an array a later launch only writes - the next part of a concatenation - is not read by it; kernels that
+                #add to what their result array holds do read it)
+                touched_later |= {id(b.tensor) for i, (b, _) in enumerate(m.buffers) if b is not None and b.tensor is not None
+                                  and (i not in m.written or m.kernel in K.ACCUMULATING_KERNELS)}
+        return result
 
     #an argument from this size on is worth starting the first launch on while it is still arriving (the link moves
     #about 50 MB per millisecond; a part more costs a few microseconds of device time)

@@ -89,6 +89,9 @@ class Launch(tp.NamedTuple):
     #a batch launch: the launches it evaluates, described to the kernel by a table in device memory
     #that is written when the launch is recorded (it holds device addresses)
     members: tp.Tuple['Launch', ...] = ()
+    #the kernel stores its result (its first array) past the caches when bit 31 of its first parameter word is set
+    #(see with_streamed_result)
+    streamable: bool = False
     #which of `buffers` the kernel writes (positions); everything else it only reads
     written: tp.Tuple[int, ...] = (0,)
 
@@ -242,8 +245,6 @@ def lower_ew_chain(chain: EwChain) -> Launch:
     while len(stride_rows) < EW_MAX_STEPS:
         stride_rows.append([0, 0, 0, 0])
         buffers.append((None, 0))
-    if STREAM_RESULT_MIN_BYTES <= 4 * n < 2**32:
-        flags[0] |= 256                      #the result goes past the caches
     params = (_u32(n, ndim, *_pad(dims, 4, 1), nsteps, *_pad(ops, EW_MAX_STEPS), *_pad(flags, EW_MAX_STEPS),
                    *_pad(imms, EW_MAX_STEPS))
               + _i32(*[s for row in stride_rows for s in row]) + _u32(*_pad(extents, EW_MAX_STEPS), *_pad(bases, EW_MAX_STEPS))
@@ -254,14 +255,26 @@ def lower_ew_chain(chain: EwChain) -> Launch:
     slots = 2 if nsteps <= 2 else 4 if nsteps <= 4 else 6 if nsteps <= 6 else 8
     per_thread = {2: 1, 4: 2, 6: 2, 8: 1}[slots]               #vectors a thread works on (the kernel's U)
     return Launch(f'ew_chain_v{vec}_s{slots}', (_cdiv(_cdiv(n, vec), BLOCK * per_thread), 1, 1), (BLOCK, 1, 1),
-                  [(chain.out, 0)] + buffers, params, bytes_moved=nbytes)
+                  [(chain.out, 0)] + buffers, params, bytes_moved=nbytes, streamable=vec == 4)
 
 
 EW_AFFINE_BIG_ELEMENTS = 1 << 22
-#Results from this size on are stored with the nontemporal hint: an array that no later launch will find in the caches
-#(32 MB of L2 in all, 256 MB behind it) only pushes out what could be reused, and the stores of a launch that reads and
-#writes run faster past the L2 (relu on 64 M elements 92 -> 76 us, exp 96 -> 81 us).
+#Results from this size on that no later launch of the program reads are stored with the nontemporal hint: such an array
+#only pushes out of the caches what could be reused, and the stores of a launch that reads and writes run faster past the
+#L2 (relu on 64 M elements 92 -> 76 us, exp 96 -> 81 us). Results that the next launch reads are left to the caches.
 STREAM_RESULT_MIN_BYTES = 64 << 20
+STREAM_RESULT_BIT = 1 << 31
+#kernels that add to what their result array already holds (their first array is read as well as written)
+ACCUMULATING_KERNELS = ('scatter_add_rows', 'scatter_add_general')
+
+
+def with_streamed_result(launch: Launch) -> Launch:
+    '''`launch` with the flag set that makes its kernel store the result past the caches (bit 31 of the first
+    parameter word, an element count below 2**31 in every kernel that is marked streamable).'''
+    assert launch.streamable and not launch.members
+    first = int(np.frombuffer(launch.params[:4], np.uint32)[0])
+    assert first < STREAM_RESULT_BIT
+    return launch._replace(params=_u32(first | STREAM_RESULT_BIT) + launch.params[4:])
 
 
 def _as_affine_chain(chain: EwChain, n: int, dims, strides) -> tp.Optional[Launch]:
@@ -307,11 +320,11 @@ def _as_affine_chain(chain: EwChain, n: int, dims, strides) -> tp.Optional[Launc
     at = lambda o: (o.buffer, o.offset * 4) if o is not None else (None, 0)
     buffers = ([(chain.out, 0), at(operands[0])] + [at(o) for o in _pad(sums, 3, None)]
                + [at(slot.get(b)) for b in range(5)])
-    params  = _u32(n, C // 4, magic, shift, len(sums), sum(1 << b for b in slot) | (32 if 4 * n >= STREAM_RESULT_MIN_BYTES else 0))
+    params  = _u32(n, C // 4, magic, shift, len(sums), sum(1 << b for b in slot))
     nbytes  = 4 * n + sum(4 * min(n, o.buffer.size) for o in operands)
     #(arrays of more than 16 MB: the variant that skips absent operands instead of loading through empty descriptors)
     kernel = 'ew_affine_big_v4' if n > EW_AFFINE_BIG_ELEMENTS else 'ew_affine_v4'
-    return Launch(kernel, (_cdiv(n // 4, 2 * BLOCK), 1, 1), (BLOCK, 1, 1), buffers, params, bytes_moved=nbytes)
+    return Launch(kernel, (_cdiv(n // 4, 2 * BLOCK), 1, 1), (BLOCK, 1, 1), buffers, params, bytes_moved=nbytes, streamable=True)
 
 
 EW_BATCH_KERNELS     = ('ew_chain_v1_s2', 'ew_chain_v1_s4', 'ew_chain_v4_s2', 'ew_chain_v4_s4')
@@ -383,9 +396,9 @@ def _as_tiled_transpose(chain: EwChain, dims, strides) -> tp.Optional[Launch]:
     vec = all(v % 4 == 0 for v in (I, J, st[-1], sb, src.offset))
     if vec and I >= 128 and J >= 128 and I * J >= 1 << 16 and TRANSPOSE_BIG_TILES:
         return Launch('transpose_tiled_v4_t128', (_cdiv(J, 128), _cdiv(I, 128), B), (BLOCK, 1, 1), [(chain.out, 0), (src.buffer, src.offset * 4)],
-                      _u32(B, I, J, sb, st[-1]), lds=0, bytes_moved=8 * n)
+                      _u32(B, I, J, sb, st[-1]), lds=0, bytes_moved=8 * n, streamable=True)
     return Launch('transpose_tiled_v4' if vec else 'transpose_tiled', (_cdiv(J, 64), _cdiv(I, 64), B), (BLOCK, 1, 1), [(chain.out, 0), (src.buffer, src.offset * 4)],
-                  _u32(B, I, J, sb, st[-1]), bytes_moved=8 * n)
+                  _u32(B, I, J, sb, st[-1]), bytes_moved=8 * n, streamable=bool(vec))
 
 
 def iota(out: Buffer, dimension: int) -> Launch:
@@ -409,7 +422,7 @@ def concat_part(out: Buffer, part: Buffer, dimension: int, offset_along_dim: int
     n   = part.size
     vec = 4 if (part_inner % 4 == 0 and out_inner % 4 == 0 and (offset_along_dim * inner) % 4 == 0) else 1
     return Launch(f'concat_part_v{vec}', (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (part, 0)],
-                  _u32(n, part_inner, out_inner, offset_along_dim * inner), bytes_moved=8 * n)
+                  _u32(n, part_inner, out_inner, offset_along_dim * inner), bytes_moved=8 * n, streamable=vec == 4 and n < 2**31)
 
 
 TF_MAX_STEPS = 8
@@ -1152,7 +1165,8 @@ def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, selected: B
     first  = Launch(select, (_cdiv(_cdiv(n_win, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                     [(selected, 0), (operand, 0)], _u32(n_win) + tail, bytes_moved=4 * (operand.size + source.size))
     second = Launch(scatter, (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
-                    [(out, 0), (source, 0), (selected, 0)], _u32(n) + tail, bytes_moved=4 * (operand.size + 2 * source.size))
+                    [(out, 0), (source, 0), (selected, 0)], _u32(n) + tail, bytes_moved=4 * (operand.size + 2 * source.size),
+                    streamable=vec == 4 and n < 2**31)
     return [first, second]
 
 
@@ -1188,7 +1202,7 @@ def pad(out: Buffer, inp: Buffer, value: Buffer, padding_config) -> Launch:
     vec = 4 if (step == 1 and low % 4 == 0 and o % 4 == 0 and i % 4 == 0) else 1
     params = _u32(out.size, *[d[0] for d in dims], *[d[1] for d in dims]) + _i32(*[d[2] for d in dims]) + _u32(*[d[3] for d in dims])
     return Launch(f'pad_nd_v{vec}', (_cdiv(_cdiv(out.size, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
-                  [(out, 0), (inp, 0), (value, 0)], params, bytes_moved=4 * (inp.size + out.size))
+                  [(out, 0), (inp, 0), (value, 0)], params, bytes_moved=4 * (inp.size + out.size), streamable=vec == 4 and out.size < 2**31)
 
 
 # --------------------------------------------------------------------------- gather / scatter / rng
@@ -1202,7 +1216,8 @@ def gather_rows(out: Buffer, table: Buffer, idx: Buffer, n_idx: int, row_len: in
     vec = 4 if row_len % 4 == 0 else 1
     total = n_idx * (row_len // vec)
     return Launch(f'gather_rows_v{vec}', (_cdiv(total, BLOCK), 1, 1), (BLOCK, 1, 1), [(out, 0), (table, 0), (idx, 0)],
-                  _u32(n_idx, row_len, n_rows, idx_stride, int(fill is not None), fill or 0, 0), bytes_moved=4 * (2 * n_idx * row_len + n_idx))
+                  _u32(n_idx, row_len, n_rows, idx_stride, int(fill is not None), fill or 0, 0), bytes_moved=4 * (2 * n_idx * row_len + n_idx),
+                  streamable=vec == 4 and n_idx < 2**31)
 
 
 def gather_general(out: Buffer, operand: Buffer, indices: Buffer, offset_dims, collapsed, start_index_map, slice_sizes,
