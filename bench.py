@@ -239,7 +239,8 @@ def measure_primitives(iters=30, warm=10, only=None):
 def time_whole_calls(fn, inputs, fuse):
     '''Whole calls through wrap(): host arrays in, host arrays out, uploads and Python included; once copying every
     argument per call (what the reference does, vkjax/kompute_jaxpr_interpreter.py:66-81), once with the weights
-    resident, once streamed (each call's upload overlaps the call before it). Median of 5 / mean of 40 after 4.'''
+    resident, once streamed (each call's upload overlaps the call before it), once streamed with two calls on the device at
+    a time. Median of 9 / mean of 40 (80) after 4 (8).'''
     import vkjax_amd
     from vkjax_amd.minijax import tree_util
     out = {}
@@ -271,6 +272,15 @@ def time_whole_calls(fn, inputs, fuse):
             for _ in results:
                 pass
             out['weights_resident_streamed_ms'] = round((time.perf_counter() - t0) * 1e3 / n, 3)
+            #the same with two batches on the device at a time, each on a context of its own (Function.stream(in_flight=2)).
+            #The lanes run up to eight tuples ahead of the consumer, so results that were finished before the clock
+            #starts must not count: the rate is taken between arrivals that the consumer had to wait for
+            ahead = 8
+            arrivals = []
+            for _ in f.stream([tuple(inputs)] * (2 * n + 2 * warm + ahead), in_flight=2):
+                arrivals.append(time.perf_counter())
+            first = 2 * warm + ahead - 1
+            out['weights_resident_streamed_two_in_flight_ms'] = round((arrivals[-1] - arrivals[first]) * 1e3 / (len(arrivals) - 1 - first), 3)
     return out
 
 

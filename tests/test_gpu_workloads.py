@@ -1,6 +1,8 @@
 '''The benchmark workloads end to end through vkjax_amd.wrap against the CPU oracle, at sizes
 the oracle finishes in seconds; tolerances are the north-star ones (bit-exact RNG / gather /
 argmax, 1e-5 element-wise and reductions, 1e-4 dot and conv, 1e-3 ResNet logits).'''
+import threading
+
 import numpy as np
 import pytest
 
@@ -788,6 +790,80 @@ def test_stream_loader_may_refill_its_batch_array():
         assert len(got) == len(values)
         for k, (g, v) in enumerate(zip(got, values)):
             assert_tree_close(g, plain(v, w), exact=True, what=f'{shape} batch {k}')
+
+
+def test_stream_with_several_tuples_in_flight():
+    '''Function.stream(..., in_flight=n) evaluates n tuples at a time, each on a device context of its own driven by
+    its own thread; the results are those of plain calls, in the order of the tuples: small and large arguments,
+    a change of signature in the middle, fewer tuples than lanes, none; resident weights with one replaced on the
+    way; a loader that refills one batch array; a stream abandoned half way; an error raised by the iterable.'''
+    rng = np.random.default_rng(6)
+    def scale_shift(x, w):
+        return mj.numpy.tanh(x * w + 1.0), mj.numpy.sum(x, axis=0)
+    plain = vkjax_amd.wrap(scale_shift, frontend='minijax')
+    fast  = vkjax_amd.wrap(scale_shift, frontend='minijax')
+    small = [(rng.standard_normal((33, 17)).astype(np.float32), rng.standard_normal((17,)).astype(np.float32)) for _ in range(7)]
+    large = [(rng.standard_normal((1200, 2048)).astype(np.float32), rng.standard_normal((2048,)).astype(np.float32)) for _ in range(5)]
+    for lanes in (2, 3):
+        for name, tuples in [('small', small), ('large', large), ('mixed signatures', small[:3] + large[:2] + small[3:] + large[2:]),
+                             ('single', small[:1]), ('empty', [])]:
+            expected = [plain(*t) for t in tuples]
+            got = list(fast.stream(iter(tuples), in_flight=lanes))
+            assert len(got) == len(expected), (lanes, name)
+            for k, (g, e) in enumerate(zip(got, expected)):
+                assert_tree_close(g, e, exact=True, what=f'{lanes} lanes, {name} [{k}]')
+    #the function itself is not one of the lanes: calls between results of a stream do not disturb it
+    it = fast.stream(iter(small), in_flight=2)
+    for k in range(len(small)):
+        assert_tree_close(next(it), plain(*small[k]), exact=True, what=f'suspended stream [{k}]')
+        assert_tree_close(fast(*large[k % len(large)]), plain(*large[k % len(large)]), exact=True, what=f'call between results {k}')
+    assert next(it, None) is None
+
+    params, x = W.mlp_inputs()
+    plain_mlp = vkjax_amd.wrap(W.mlp, frontend='minijax')
+    resident  = vkjax_amd.wrap(W.mlp, frontend='minijax', resident_argnums=(0,))
+    from vkjax_amd.minijax import tree_util
+    leaves, structure = tree_util.tree_flatten(params)
+    params2 = tree_util.tree_unflatten(structure, [leaves[0] * np.float32(0.5)] + list(leaves[1:]))
+    batches = [(params, x), (params, x[::-1].copy()), (params2, x), (params2, x * np.float32(2)), (params, x), (params2, x[::-1].copy())]
+    expected = [plain_mlp(*t) for t in batches]
+    for repeat in range(2):                                   #(the second time the lanes exist and hold weights already)
+        for k, (g, e) in enumerate(zip(resident.stream(batches, in_flight=2), expected)):
+            assert_tree_close(g, e, exact=True, what=f'resident weights [{k}], pass {repeat}')
+
+    #one preallocated batch array, refilled for every tuple: each lane has copied its tuple before the next is asked for
+    def affine(x, w):
+        return x * w + 1.0
+    plain_affine, streamed = vkjax_amd.wrap(affine, frontend='minijax'), vkjax_amd.wrap(affine, frontend='minijax')
+    for shape in ((33, 17), (1200, 2048)):
+        w      = rng.standard_normal(shape[1:]).astype(np.float32)
+        values = [rng.standard_normal(shape).astype(np.float32) for _ in range(11)]
+        batch  = np.empty(shape, np.float32)
+        def loader():
+            for v in values:
+                batch[...] = v
+                yield batch, w
+        got = [np.array(y) for y in streamed.stream(loader(), in_flight=2)]
+        assert len(got) == len(values)
+        for k, (g, v) in enumerate(zip(got, values)):
+            assert_tree_close(g, plain_affine(v, w), exact=True, what=f'{shape} refilled batch {k}')
+
+    #abandoned half way: the lanes' threads end, the function and a new stream work
+    it = fast.stream(iter(small), in_flight=2)
+    next(it)
+    it.close()
+    assert_tree_close(fast(*small[0]), plain(*small[0]), exact=True, what='call after an abandoned stream')
+    assert len(list(fast.stream(iter(small), in_flight=2))) == len(small)
+    assert not [t for t in threading.enumerate() if t.name.startswith('vkjax-stream-lane')]
+
+    #an error of the iterable reaches the consumer, after the results of the tuples before it or instead of them
+    def failing():
+        yield small[0]
+        yield small[1]
+        raise KeyError('no third batch')
+    with pytest.raises(KeyError, match='no third batch'):
+        list(fast.stream(failing(), in_flight=2))
+    assert not [t for t in threading.enumerate() if t.name.startswith('vkjax-stream-lane')]
 
 
 def test_first_launch_starts_while_its_argument_arrives():

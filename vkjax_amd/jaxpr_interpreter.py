@@ -24,7 +24,7 @@ from .minijax import core, tree_util
 class JaxprInterpreter:
     def __init__(self, jaxpr, static_argnums: tp.Tuple[int, ...] = (), profiling: bool = False,
                  reuse_buffers: bool = True, fuse: bool = True, plan_only: bool = False, graph: bool = False,
-                 resident_argnums: tp.Tuple[int, ...] = (), two_lanes: bool = False):
+                 resident_argnums: tp.Tuple[int, ...] = (), two_lanes: bool = False, device: tp.Optional['hip.Device'] = None):
         self.jaxpr          = jaxpr
         #Which argument leaves stay in HBM between calls instead of being copied on every call, as the reference
         #does (vkjax/kompute_jaxpr_interpreter.py:72-75):
@@ -48,7 +48,9 @@ class JaxprInterpreter:
         self.fuse           = fuse
         #plan_only builds ops, buffers and launch parameters without touching a GPU; such an
         #interpreter cannot run
-        self.mgr            = PlanOnlyDevice() if plan_only else hip.Device.get()
+        #(device: a context other than the shared one of hip.Device.get(); it has its own streams, so programs on
+        #different contexts, each driven by a thread of its own, run side by side on the GPU)
+        self.mgr            = PlanOnlyDevice() if plan_only else (device if device is not None else hip.Device.get())
         self.workgroup_size = get_maximum_workgroup_size(self.mgr)
         self.bufferpool     = BufferPool(self.mgr, self.workgroup_size, reuse_buffers)
         self.sequence       = None
