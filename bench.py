@@ -272,15 +272,18 @@ def time_whole_calls(fn, inputs, fuse):
             for _ in results:
                 pass
             out['weights_resident_streamed_ms'] = round((time.perf_counter() - t0) * 1e3 / n, 3)
-            #the same with two batches on the device at a time, each on a context of its own (Function.stream(in_flight=2)).
-            #The lanes run up to eight tuples ahead of the consumer, so results that were finished before the clock
-            #starts must not count: the rate is taken between arrivals that the consumer had to wait for
-            ahead = 8
-            arrivals = []
-            for _ in f.stream([tuple(inputs)] * (2 * n + 2 * warm + ahead), in_flight=2):
-                arrivals.append(time.perf_counter())
-            first = 2 * warm + ahead - 1
-            out['weights_resident_streamed_two_in_flight_ms'] = round((arrivals[-1] - arrivals[first]) * 1e3 / (len(arrivals) - 1 - first), 3)
+            #the same with two and with three batches on the device at a time, each on a context of its own
+            #(Function.stream(in_flight=...)). The lanes run up to four tuples each ahead of the consumer, so results that
+            #were finished before the clock starts must not count: the rate is taken between arrivals that the consumer
+            #had to wait for
+            for lanes, label_lanes in ((2, 'two'), (3, 'three')):
+                ahead = 4 * lanes
+                arrivals = []
+                for _ in f.stream([tuple(inputs)] * (2 * n + 2 * warm + ahead), in_flight=lanes):
+                    arrivals.append(time.perf_counter())
+                first = 2 * warm + ahead - 1
+                out[f'weights_resident_streamed_{label_lanes}_in_flight_ms'] = round(
+                    (arrivals[-1] - arrivals[first]) * 1e3 / (len(arrivals) - 1 - first), 3)
     return out
 
 
