@@ -101,7 +101,14 @@ int vkj_seq_record_upload(vkj_handle seq, vkj_handle buf, size_t offset, int slo
  * `kernarg` is the kernel's argument block laid out by the caller. For each i < nbufs the
  * 8 bytes at kernarg[buf_arg_offsets[i]] are overwritten with the device address of
  * bufs[i] plus buf_byte_offsets[i] (may be NULL for all-zero). Addresses are resolved
- * once, here. */
+ * once, here. A buffer with buf_arg_offsets[i] == VKJ_NO_POINTER_SLOT gets no address written: the
+ * kernel reaches it through addresses it finds elsewhere (a table in device memory); the sequence
+ * keeps it alive like the others. Every buffer the kernel reads must be listed in one of the two
+ * ways: an evaluation that uploads large arguments sends them in the order in which the launches
+ * first read them and issues each launch as soon as what it and the launches before it read has
+ * been handed to the copy engines, while later arguments are still on their way (the reference
+ * uploads everything, then evaluates: vkjax/kompute_jaxpr_interpreter.py:72-77). */
+#define VKJ_NO_POINTER_SLOT 0xFFFFFFFFu
 int vkj_seq_record_launch(vkj_handle seq, vkj_handle function,
                           const uint32_t grid[3], const uint32_t block[3], uint32_t lds_bytes,
                           const void* kernarg, size_t kernarg_bytes,

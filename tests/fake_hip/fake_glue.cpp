@@ -22,4 +22,6 @@ extern "C" long fake_hip_live_objects() { return (long)fake_hip().live.size(); }
 extern "C" long fake_hip_creations() { return fake_hip().creations; }
 extern "C" void fake_hip_on_synchronize(void (*hook)()) { fake_hip().on_synchronize = hook; }
 extern "C" long fake_hip_launches() { return fake_hip().launches; }
+extern "C" long fake_hip_copies() { return fake_hip().copies; }
+extern "C" long fake_hip_copies_at_launch(long k) { return k >= 0 && k < (long)fake_hip().copies_at_launch.size() ? fake_hip().copies_at_launch[k] : -1; }
 extern "C" void fake_hip_fail_after(long successful_calls) { fake_hip().calls_until_failure = successful_calls; }

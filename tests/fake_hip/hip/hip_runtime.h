@@ -44,6 +44,8 @@ struct FakeHipState {
     std::set<void*> live;          // every allocation, stream, event and module that has not been released
     long calls_until_failure = -1; // >= 0: that many further fallible calls succeed, the next one fails
     long launches = 0;
+    long copies = 0;               // hipMemcpyAsync calls so far
+    std::vector<long> copies_at_launch;   // per launch: how many copies had been issued before it
     long creations = 0;            // allocations (device and pinned), streams, events, modules, graphs ever made
     void (*on_synchronize)() = nullptr;   // called from inside hipStreamSynchronize (the test re-enters the library there)
 };
@@ -108,7 +110,7 @@ inline hipError_t hipMalloc(void** p, size_t n) { return fake_hip_alloc(p, n); }
 inline hipError_t hipFree(void* p) { return fake_hip_release(p); }
 inline hipError_t hipHostMalloc(void** p, size_t n, unsigned) { return fake_hip_alloc(p, n); }
 inline hipError_t hipHostFree(void* p) { return fake_hip_release(p); }
-inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, hipMemcpyKind, hipStream_t) { memmove(dst, src, n); return hipSuccess; }
+inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, hipMemcpyKind, hipStream_t) { fake_hip().copies++; memmove(dst, src, n); return hipSuccess; }
 inline hipError_t hipMemsetAsync(void* dst, int v, size_t n, hipStream_t) { memset(dst, v, n); return hipSuccess; }
 inline hipError_t hipModuleLoadData(hipModule_t* m, const void* image) {
     if (hipError_t e = fake_hip_new(m)) return e;
@@ -128,6 +130,7 @@ inline hipError_t hipModuleGetFunction(hipFunction_t* f, hipModule_t m, const ch
 inline hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned,
                                         unsigned, hipStream_t, void**, void** extra) {
     fake_hip().launches++;
+    fake_hip().copies_at_launch.push_back(fake_hip().copies);
     if (f->name != "fake_add_one") return hipSuccess;
     struct Args { uint32_t* dst; const uint32_t* src; uint32_t n; } a;
     memcpy(&a, extra[1], sizeof(a));

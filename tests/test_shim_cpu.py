@@ -31,6 +31,9 @@ def lib(tmp_path_factory):
     lib.fake_hip_live_objects.restype = C.c_long
     lib.fake_hip_launches.restype = C.c_long
     lib.fake_hip_creations.restype = C.c_long
+    lib.fake_hip_copies.restype = C.c_long
+    lib.fake_hip_copies_at_launch.restype = C.c_long
+    lib.fake_hip_copies_at_launch.argtypes = [C.c_long]
     lib.fake_hip_on_synchronize.argtypes = [C.c_void_p]
     lib.fake_hip_fail_after.argtypes = [C.c_long]
     return lib
@@ -175,17 +178,74 @@ def test_buffer_freed_under_a_live_sequence_outlives_it(lib):
 
 def test_context_creation_releases_everything_when_a_step_fails(lib):
     before = lib.fake_hip_live_objects()
-    for successes in range(8):                                   #three streams and five events are created
+    made = 4 + 5 + 16                                            #four streams, five events, sixteen checkpoint events are created
+    for successes in range(made):
         lib.fake_hip_fail_after(successes)
         ctx = H()
         assert lib.vkj_ctx_create(0, C.byref(ctx)) != 0
         assert b'injected' in lib.vkj_last_error()
         assert lib.fake_hip_live_objects() == before
-    lib.fake_hip_fail_after(8)                                   #nothing left to fail in creation
+    lib.fake_hip_fail_after(made)                                #nothing left to fail in creation
     ctx = H()
     assert lib.vkj_ctx_create(0, C.byref(ctx)) == 0
     lib.fake_hip_fail_after(-1)
     assert lib.vkj_ctx_destroy(ctx) == 0
+    assert lib.fake_hip_live_objects() == before
+
+
+def test_launches_follow_the_uploads(lib):
+    '''An evaluation that brings large arguments sends them in the order in which the launches first read them,
+    whatever the order they were recorded in, and issues each launch once everything it and the launches before it
+    read has been handed to the copy engines - not after the last byte. The stand-in runs copies and kernels at once,
+    so a launch issued too early would compute on bytes that are not there yet. Arguments that stay resident, small
+    ones, and launches that read no argument at all are handled; nothing is created while evaluating.'''
+    before = lib.fake_hip_live_objects()
+    w = World(lib)
+    n = 4 << 20                                                    #16 MB each: 16 chunks
+    a, b, c, small = w.buf(4 * n), w.buf(4 * n), w.buf(4 * n), w.buf(4 * 16)
+    ra, rb, rc, rs, free = w.buf(4 * n), w.buf(4 * n), w.buf(4 * n), w.buf(4 * 16), w.buf(4 * 16)
+    seq = H()
+    assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq)) == 0
+    #recorded in the reverse of the order of use
+    assert lib.vkj_seq_record_upload(seq, c, 0, 2, 4 * n) == 0
+    assert lib.vkj_seq_record_upload(seq, b, 0, 1, 4 * n) == 0
+    assert lib.vkj_seq_record_upload(seq, small, 0, 3, 4 * 16) == 0
+    assert lib.vkj_seq_record_upload(seq, a, 0, 0, 4 * n) == 0
+    assert w.record_add_one(seq, free, free, 16) == 0              #reads no argument
+    assert w.record_add_one(seq, ra, a, n) == 0
+    assert w.record_add_one(seq, rb, b, n) == 0
+    assert w.record_add_one(seq, rs, small, 16) == 0
+    assert w.record_add_one(seq, rc, c, n) == 0
+    for slot, buf, count in ((4, ra, n), (5, rb, n), (6, rc, n), (7, rs, 16)):
+        assert lib.vkj_seq_record_download(seq, buf, 0, slot, 4 * count) == 0
+    rng = np.random.default_rng(8)
+    made = lib.fake_hip_creations()
+    def run(resident=()):
+        xs = [rng.integers(0, 1 << 30, size=n, dtype=np.uint32) for _ in range(3)] + [rng.integers(0, 1 << 30, size=16, dtype=np.uint32)]
+        ys = [np.zeros(n, np.uint32) for _ in range(3)] + [np.zeros(16, np.uint32)]
+        ptrs = (C.c_void_p * 8)(*[None if k in resident else x.ctypes.data for k, x in enumerate(xs)], *[y.ctypes.data for y in ys])
+        copies, launches = lib.fake_hip_copies(), lib.fake_hip_launches()
+        assert lib.vkj_seq_eval(seq, ptrs, 8, hip.EVAL_NULL_IS_RESIDENT if resident else 0) == 0, lib.vkj_last_error()
+        assert lib.fake_hip_launches() - launches == 5
+        return xs, ys, [lib.fake_hip_copies_at_launch(launches + k) - copies for k in range(5)]
+    xs, ys, at = run()
+    for k in (0, 1, 3):
+        assert np.array_equal(ys[k], xs[k] + 1)
+    assert np.array_equal(ys[2], xs[2] + 1)
+    #a (16 chunks) first, then b, the small one, c. Launches go at checkpoints - behind what the first launch reads, then
+    #every 16 MB or more, and at the end - so the launch on the small argument waits for the last one
+    assert at == [0, 16, 32, 49, 49], at
+    held = xs
+    #b stays where it is: a, the small one, c
+    xs, ys, at = run(resident=(1,))
+    assert np.array_equal(ys[0], xs[0] + 1) and np.array_equal(ys[1], held[1] + 1) and np.array_equal(ys[2], xs[2] + 1)
+    assert np.array_equal(ys[3], xs[3] + 1)
+    assert at[0] == 0 and at[1] == 16 and at[4] == 33, at
+    assert lib.fake_hip_creations() == made
+    assert lib.vkj_seq_destroy(seq) == 0
+    for buf in (a, b, c, small, ra, rb, rc, rs, free):
+        assert lib.vkj_buf_free(w.ctx, buf) == 0
+    w.close()
     assert lib.fake_hip_live_objects() == before
 
 
@@ -384,7 +444,7 @@ def test_first_launch_in_parts_beside_the_upload(lib):
     assert lib.fake_hip_launches() - launches == 2
     assert lib.fake_hip_creations() == made
     assert lib.vkj_seq_destroy(seq) == 0
-    #another upload behind the argument: what the first launch reads besides it may not have arrived, so no parts
+    #another argument recorded behind it, which the launch does not read: sent behind it too, parts as before
     seq = H()
     assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq)) == 0
     assert lib.vkj_seq_record_upload(seq, src, 0, 0, 4 * n) == 0
@@ -397,7 +457,7 @@ def test_first_launch_in_parts_beside_the_upload(lib):
     ptrs = (C.c_void_p * 3)(x.ctypes.data, y.ctypes.data, small.ctypes.data)
     launches = lib.fake_hip_launches()
     assert lib.vkj_seq_eval(seq, ptrs, 3, 0) == 0, lib.vkj_last_error()
-    assert np.array_equal(y, x + 1) and lib.fake_hip_launches() - launches == 1
+    assert np.array_equal(y, x + 1) and lib.fake_hip_launches() - launches == nparts
     assert lib.vkj_seq_destroy(seq) == 0
     for b in (src, mid, dst, other):
         assert lib.vkj_buf_free(w.ctx, b) == 0

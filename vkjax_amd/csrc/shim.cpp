@@ -55,6 +55,7 @@ using namespace vkj;
 constexpr size_t STAGE_CHUNK     = 4u << 20;   // results on their way back
 constexpr size_t UPLOAD_CHUNK    = 1u << 20;   // arguments
 constexpr size_t STAGE_MIN       = 8u << 20;   // smaller transfers are copied inline
+constexpr size_t CHECKPOINT_BYTES = 16u << 20; // launches that follow the uploads: at least this much between two of their waits
 constexpr int    STAGE_THREADS   = 8;
 constexpr int    UPLOAD_THREADS  = 4;
 
@@ -181,9 +182,11 @@ void destroy_ctx_objects(Ctx* c) {
     if (c->ev_copied)   hipEventDestroy(c->ev_copied);
     if (c->stream)      hipStreamDestroy(c->stream);
     if (c->copy_stream) hipStreamDestroy(c->copy_stream);
+    if (c->copy_stream2) hipStreamDestroy(c->copy_stream2);
+    for (auto& e : c->ev_checkpoint) { if (e) hipEventDestroy(e); e = nullptr; }
     if (c->side_stream) hipStreamDestroy(c->side_stream);
     c->ev_begin = c->ev_end = c->ev_landed = c->ev_uploaded = c->ev_copied = nullptr;
-    c->stream = c->copy_stream = c->side_stream = nullptr;
+    c->stream = c->copy_stream = c->copy_stream2 = c->side_stream = nullptr;
 }
 
 // A sequence lets go of a buffer it recorded; the memory of a buffer that vkj_buf_free has
@@ -283,6 +286,7 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
     if (down) for (auto& t : s->downloads) if (!slot_ok(t)) return fail(VKJ_EINVAL, "vkj_seq_eval: no host pointer for download slot %d", t.slot);
 
     size_t nstamps = 0, first_launch = 0;        // first_launch: 1 when the first launch has been issued in parts beside the uploads
+    bool launches_issued = false;                // all of them, beside the uploads
     if (s->profiling) {
         nstamps = 3 + s->launches.size();       // begin, after uploads, after each launch, after downloads
         while (s->stamps.size() < nstamps) {
@@ -300,50 +304,130 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
             // all arguments as one stream of chunks: a few threads stage them, this one hands each chunk to the
             // DMA engine as soon as it is staged
             std::vector<UploadPiece> pieces;
+            std::vector<int> piece_slot;
             for (auto& t : s->uploads)
-                if (t.nbytes && host_ptrs[t.slot])
+                if (t.nbytes && host_ptrs[t.slot]) {
                     pieces.push_back({(char*)t.staging, (const char*)host_ptrs[t.slot], (char*)t.buf->dptr + t.offset, t.nbytes});
-            // the chunks alternate between the two streams (two copy engines work on them); the launches wait for both.
-            // Both streams are idle here: every evaluation ends with everything it queued on them complete.
+                    piece_slot.push_back(t.slot);
+                }
+            const size_t nl = s->launches.size();
+            // Launches that follow the uploads: a program that brings all its weights with every call need not wait for
+            // the last of them before its first layer starts. The arguments travel in the order in which the launches
+            // first read them (the arrays of one launch smallest first), over two streams that carry nothing else, and
+            // at a few checkpoints along the way the launch stream is told to wait for what has been handed over so
+            // far and is given the launches that read nothing beyond it. (Not with time stamps, a captured graph, a
+            // second lane or a fixed landing region, whose bookkeeping assumes the uploads are over before the launches.)
+            const bool follow = nl > 0 && !s->profiling && !s->want_graph && !s->uses_side && !region;
+            std::vector<long> need(nl, -1);              // the last piece (in sending order) a launch or any launch before it reads
+            std::vector<size_t> checkpoints;             // pieces behind which launches are issued, ascending; the last piece is one
+            if (follow) {
+                std::vector<size_t> first_use(pieces.size(), nl), order(pieces.size());
+                std::unordered_multimap<const void*, size_t> piece_of;          // device allocation -> pieces that land in it
+                {
+                    size_t p = 0;
+                    for (auto& t : s->uploads) if (t.nbytes && host_ptrs[t.slot]) piece_of.emplace(t.buf, p++);
+                }
+                for (size_t i = 0; i < nl; i++)
+                    for (Buf* b : s->launches[i].bufs) {
+                        auto range = piece_of.equal_range(b);
+                        for (auto it = range.first; it != range.second; ++it) first_use[it->second] = std::min(first_use[it->second], i);
+                    }
+                for (size_t p = 0; p < order.size(); p++) order[p] = p;
+                std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) {
+                    return first_use[a] != first_use[b] ? first_use[a] < first_use[b] : pieces[a].nbytes < pieces[b].nbytes;
+                });
+                std::vector<UploadPiece> sorted_pieces;
+                std::vector<int> sorted_slot;
+                std::vector<size_t> sorted_use;
+                for (size_t p : order) { sorted_pieces.push_back(pieces[p]); sorted_slot.push_back(piece_slot[p]); sorted_use.push_back(first_use[p]); }
+                pieces.swap(sorted_pieces);
+                piece_slot.swap(sorted_slot);
+                // (sorted by first use: the pieces a launch needs end where the pieces first read by a later launch begin)
+                size_t p = 0;
+                long reached = -1;
+                for (size_t i = 0; i < nl; i++) {
+                    while (p < pieces.size() && sorted_use[p] <= i) reached = (long)p++;
+                    need[i] = reached;
+                }
+                // the first checkpoint lets the first launch go; behind it one per CHECKPOINT_BYTES or more, a handful in all
+                size_t rest = 0;
+                for (size_t q = (size_t)(need[0] + 1); q < pieces.size(); q++) rest += pieces[q].nbytes;
+                const size_t step = std::max<size_t>(CHECKPOINT_BYTES, rest / (Ctx::MAX_CHECKPOINTS - 2) + 1);
+                if (need[0] >= 0 && (size_t)need[0] + 1 < pieces.size()) checkpoints.push_back((size_t)need[0]);
+                size_t since = 0;
+                for (size_t q = (size_t)(need[0] + 1); q + 1 < pieces.size(); q++) {
+                    since += pieces[q].nbytes;
+                    if (since >= step && (int)checkpoints.size() < Ctx::MAX_CHECKPOINTS - 1) { checkpoints.push_back(q); since = 0; }
+                }
+                checkpoints.push_back(pieces.size() - 1);
+            }
+            // Without that the chunks alternate between the launch stream and the copy stream (two copy engines work on
+            // them) and the launches wait for both. All streams are idle here: every evaluation ends with everything
+            // it queued on them complete.
+            hipStream_t copy_even = follow ? c->copy_stream2 : c->stream, copy_odd = c->copy_stream;
             // The first launch in parts: a part goes to the side stream as soon as the chunks it reads have been
             // handed to the copy engines (both streams are in order: an event behind a chunk covers every chunk
-            // before it), so the device computes while the rest of the argument is still on its way.
+            // before it), so the device computes while the rest of the argument is still on its way. Only with that
+            // argument as the last thing the first launch reads to be sent: whatever else it reads has then been sent.
             size_t early_piece = pieces.size(), next_part = 0;
             if (!s->early.empty() && !s->profiling && !s->want_graph && !s->uses_side) {
-                size_t p = 0;
-                for (auto& t : s->uploads) {
-                    if (!(t.nbytes && host_ptrs[t.slot])) continue;
-                    if (t.slot == s->early_slot && t.nbytes >= s->early.back().bytes_needed) early_piece = p;
-                    p++;
-                }
-                // only as the last argument on its way: whatever else the launch reads has then been sent before it
-                if (early_piece + 1 != pieces.size()) early_piece = pieces.size();
+                for (size_t p = 0; p < pieces.size(); p++)
+                    if (piece_slot[p] == s->early_slot && pieces[p].nbytes >= s->early.back().bytes_needed) early_piece = p;
+                const size_t must_be = follow ? (size_t)(need[0] < 0 ? pieces.size() : need[0]) : pieces.size() - 1;
+                if (early_piece != must_be) early_piece = pieces.size();
             }
             hipError_t err = hipSuccess;
             int launch_status = 0;
+            size_t next_launch = 0, next_checkpoint = 0;
+            // launches that read nothing of this evaluation's uploads, and nothing behind such launches, need not wait at all
+            while (follow && next_launch < nl && need[next_launch] < 0) {
+                if ((launch_status = issue_launch(c, s->launches[next_launch++]))) return launch_status;
+            }
             const int r = staged_upload_pieces(pieces, [&](size_t k, size_t piece, size_t off, size_t len) {
                 err = hipMemcpyAsync(pieces[piece].device + off, pieces[piece].staging + off, len, hipMemcpyHostToDevice,
-                                     (k & 1) ? c->copy_stream : c->stream);
+                                     (k & 1) ? copy_odd : copy_even);
                 if (err != hipSuccess) return 1;
                 while (piece == early_piece && next_part < s->early.size() && s->early[next_part].bytes_needed <= off + len) {
                     EarlyPart& part = s->early[next_part++];
-                    if ((err = hipEventRecord(part.ev_a, c->stream)) != hipSuccess) return 1;
-                    if ((err = hipEventRecord(part.ev_b, c->copy_stream)) != hipSuccess) return 1;
+                    if ((err = hipEventRecord(part.ev_a, copy_even)) != hipSuccess) return 1;
+                    if ((err = hipEventRecord(part.ev_b, copy_odd)) != hipSuccess) return 1;
                     if ((err = hipStreamWaitEvent(c->side_stream, part.ev_a, 0)) != hipSuccess) return 1;
                     if ((err = hipStreamWaitEvent(c->side_stream, part.ev_b, 0)) != hipSuccess) return 1;
                     if ((launch_status = issue_launch(c, part.launch, c->side_stream))) return 1;
+                }
+                if (follow && next_checkpoint < checkpoints.size() && piece == checkpoints[next_checkpoint] && off + len == pieces[piece].nbytes) {
+                    hipEvent_t ev_even = c->ev_checkpoint[2 * next_checkpoint], ev_odd = c->ev_checkpoint[2 * next_checkpoint + 1];
+                    next_checkpoint++;
+                    if ((err = hipEventRecord(ev_even, copy_even)) != hipSuccess) return 1;
+                    if ((err = hipEventRecord(ev_odd, copy_odd)) != hipSuccess) return 1;
+                    if ((err = hipStreamWaitEvent(c->stream, ev_even, 0)) != hipSuccess) return 1;
+                    if ((err = hipStreamWaitEvent(c->stream, ev_odd, 0)) != hipSuccess) return 1;
+                    if (piece == early_piece && next_launch == 0) {
+                        // (every part has been issued: the last one needs no more than the whole argument)
+                        if ((err = hipEventRecord(s->ev_early_done, c->side_stream)) != hipSuccess) return 1;
+                        if ((err = hipStreamWaitEvent(c->stream, s->ev_early_done, 0)) != hipSuccess) return 1;
+                        next_launch = 1;
+                    }
+                    while (next_launch < nl && need[next_launch] <= (long)piece)
+                        if ((launch_status = issue_launch(c, s->launches[next_launch++]))) return 1;
                 }
                 return 0;
             });
             if (launch_status) return launch_status;
             if (r) return hip_fail(err, "hipMemcpyAsync (staged upload)");
-            HIP_TRY(hipEventRecord(c->ev_copied, c->copy_stream));
-            HIP_TRY(hipStreamWaitEvent(c->stream, c->ev_copied, 0));
-            if (early_piece < pieces.size()) {
-                // (every part has been issued: the last one needs no more than the whole argument)
-                HIP_TRY(hipEventRecord(s->ev_early_done, c->side_stream));
-                HIP_TRY(hipStreamWaitEvent(c->stream, s->ev_early_done, 0));
-                first_launch = 1;
+            if (follow) {
+                first_launch = next_launch;          // all of them: the last checkpoint is the last piece
+                if (first_launch != nl) return fail(VKJ_ESTATE, "vkj_seq_eval: %zu of %zu launches issued beside the uploads", first_launch, nl);
+                launches_issued = true;
+            } else {
+                HIP_TRY(hipEventRecord(c->ev_copied, c->copy_stream));
+                HIP_TRY(hipStreamWaitEvent(c->stream, c->ev_copied, 0));
+                if (early_piece < pieces.size()) {
+                    // (every part has been issued: the last one needs no more than the whole argument)
+                    HIP_TRY(hipEventRecord(s->ev_early_done, c->side_stream));
+                    HIP_TRY(hipStreamWaitEvent(c->stream, s->ev_early_done, 0));
+                    first_launch = 1;
+                }
             }
         } else {
             for (auto& t : s->uploads) {
@@ -366,8 +450,8 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
             if (int r = issue_launch(c, s->launches[i])) return r;
             HIP_TRY(hipEventRecord(s->stamps[2 + i], c->stream));
         }
-    } else if (int r = issue_all(c, s, first_launch)) {
-        return r;
+    } else if (!launches_issued) {
+        if (int r = issue_all(c, s, first_launch)) return r;
     }
     bool landed = false;
     if (next_host_ptrs) {
@@ -520,6 +604,8 @@ int vkj_ctx_create(int device, vkj_handle* out) {
         HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
         HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
         HIP_TRY(hipStreamCreateWithFlags(&c->side_stream, hipStreamNonBlocking));
+        HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream2, hipStreamNonBlocking));
+        for (auto& e : c->ev_checkpoint) HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
         HIP_TRY(hipEventCreate(&c->ev_begin));
         HIP_TRY(hipEventCreate(&c->ev_end));
         HIP_TRY(hipEventCreateWithFlags(&c->ev_landed, hipEventDisableTiming));
@@ -542,6 +628,7 @@ int vkj_ctx_destroy(vkj_handle h) {
     if (int r = use(c)) return r;
     hipStreamSynchronize(c->stream);
     hipStreamSynchronize(c->copy_stream);
+    hipStreamSynchronize(c->copy_stream2);
     hipStreamSynchronize(c->side_stream);
     destroy_ctx_objects(c);
     retire(c);
@@ -829,10 +916,12 @@ static int make_launch(const char* who, Seq* s, vkj_handle fh, const uint32_t gr
         if (!b || b->ctx != s->ctx) return fail(VKJ_EINVAL, "%s(%s): bad buffer handle #%d", who, f->name.c_str(), i);
         uint64_t off = buf_byte_offsets ? buf_byte_offsets[i] : 0;
         if (off > b->nbytes) return fail(VKJ_EINVAL, "%s(%s): offset of buffer #%d beyond its end", who, f->name.c_str(), i);
-        if ((size_t)buf_arg_offsets[i] + 8 > kernarg_bytes || (buf_arg_offsets[i] & 7))
-            return fail(VKJ_EINVAL, "%s(%s): pointer slot #%d outside the argument block or misaligned", who, f->name.c_str(), i);
-        uint64_t addr = (uint64_t)(uintptr_t)b->dptr + off;
-        memcpy(l.kernarg.data() + buf_arg_offsets[i], &addr, 8);
+        if (buf_arg_offsets[i] != VKJ_NO_POINTER_SLOT) {
+            if ((size_t)buf_arg_offsets[i] + 8 > kernarg_bytes || (buf_arg_offsets[i] & 7))
+                return fail(VKJ_EINVAL, "%s(%s): pointer slot #%d outside the argument block or misaligned", who, f->name.c_str(), i);
+            uint64_t addr = (uint64_t)(uintptr_t)b->dptr + off;
+            memcpy(l.kernarg.data() + buf_arg_offsets[i], &addr, 8);
+        }
         l.bufs.push_back(b);
     }
     return 0;

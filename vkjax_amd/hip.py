@@ -23,6 +23,7 @@ EVAL_SKIP_UPLOADS   = 1
 EVAL_SKIP_DOWNLOADS = 2
 EVAL_NULL_IS_RESIDENT = 4
 STATIC_LANDING_BYTES  = 64 << 20       #VKJ_STATIC_LANDING_BYTES
+NO_POINTER_SLOT       = 0xFFFFFFFF     #VKJ_NO_POINTER_SLOT
 
 
 class Props(C.Structure):
@@ -266,18 +267,23 @@ class Sequence:
         return slot
 
     def record_launch(self, kernel_name: str, grid, block, buffers: tp.Sequence[tp.Tuple[tp.Optional[DeviceBuffer], int]],
-                      params: bytes, lds_bytes: int = 0, early_part_of: tp.Optional[tp.Tuple[int, int]] = None):
+                      params: bytes, lds_bytes: int = 0, early_part_of: tp.Optional[tp.Tuple[int, int]] = None,
+                      reached_through_tables: tp.Sequence[DeviceBuffer] = ()):
         '''`buffers` are (DeviceBuffer or None, byte offset) in kernel-argument order; they occupy
         the first 8*len(buffers) bytes of the argument block, `params` follows. `early_part_of` = (upload slot, bytes
         needed): the launch is not a step of the sequence but one part of the alternative form of its first launch
-        (vkj_seq_record_early_part), issued while the rest of that slot's argument is still being uploaded.'''
+        (vkj_seq_record_early_part), issued while the rest of that slot's argument is still being uploaded.
+        `reached_through_tables`: buffers the kernel reads or writes through addresses it finds in device memory (a batch
+        launch's table) instead of its argument block; the runtime has to know them, for the order in which it sends
+        arguments and issues launches and to keep them allocated.'''
         fn      = self.device.function(kernel_name)
         nptr    = len(buffers)
         kernarg = bytes(8 * nptr) + params
-        present = [(i, b, off) for i, (b, off) in enumerate(buffers) if b is not None]
+        present = [(8 * i, b, off) for i, (b, off) in enumerate(buffers) if b is not None]
+        present += [(NO_POINTER_SLOT, b, 0) for b in reached_through_tables]
         n       = len(present)
         handles = (_H * max(n, 1))(*[b.handle for _, b, _ in present])
-        argoffs = (C.c_uint32 * max(n, 1))(*[8 * i for i, _, _ in present])
+        argoffs = (C.c_uint32 * max(n, 1))(*[slot for slot, _, _ in present])
         byteoff = (C.c_uint64 * max(n, 1))(*[off for _, _, off in present])
         g = (C.c_uint32 * 3)(*[int(x) for x in grid])
         b = (C.c_uint32 * 3)(*[int(x) for x in block])

@@ -192,7 +192,9 @@ class JaxprInterpreter:
             #a batch of small launches reads its members' arguments from a table in HBM
             table = self.mgr.tensor(K.batch_table(launch, lambda b: b.tensor.device_ptr()))
             self._batch_tables.append(table)
-            sequence.record_launch(launch.kernel, launch.grid, launch.block, [(table, 0)], launch.params, launch.lds)
+            members = {id(b.tensor): b.tensor for m in launch.members for b, _ in m.buffers if b is not None}
+            sequence.record_launch(launch.kernel, launch.grid, launch.block, [(table, 0)], launch.params, launch.lds,
+                                   reached_through_tables=list(members.values()))
             return
         bufs = [((b.tensor if b is not None else None), off) for b, off in launch.buffers]
         for (b, _), (t, _) in zip(launch.buffers, bufs):
