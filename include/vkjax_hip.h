@@ -80,6 +80,13 @@ int vkj_module_get_function(vkj_handle ctx, vkj_handle module, const char* name,
 int vkj_buf_alloc(vkj_handle ctx, size_t nbytes, vkj_handle* buf);
 /* The handle is retired at once. The memory of a buffer that live sequences have recorded (they hold
  * its address) is released when the last of those sequences is destroyed. */
+/* The same for arrays that are uploaded together, call after call (the parameter vectors of a network: hundreds of
+ * arrays of a few KB): arrays of at most 64 KB are placed next to each other, 256 bytes apart at least, in slabs of
+ * 1 MB, and a sequence stages its uploads into them side by side as well, so that an evaluation sends a run of
+ * neighbours with one transfer instead of one each. Larger requests are served as by vkj_buf_alloc. A buffer is
+ * used and freed like any other; a slab's memory is returned when the last buffer in it is freed.
+ *                                     reference: mgr.tensor(...) per variable, vkjax/buffers.py:202 */
+int vkj_buf_alloc_packed(vkj_handle ctx, size_t nbytes, vkj_handle* buf);
 int vkj_buf_free(vkj_handle ctx, vkj_handle buf);
 int vkj_buf_size(vkj_handle ctx, vkj_handle buf, size_t* nbytes);
 int vkj_buf_device_ptr(vkj_handle ctx, vkj_handle buf, uint64_t* device_address);

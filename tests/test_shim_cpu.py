@@ -232,19 +232,83 @@ def test_launches_follow_the_uploads(lib):
     for k in (0, 1, 3):
         assert np.array_equal(ys[k], xs[k] + 1)
     assert np.array_equal(ys[2], xs[2] + 1)
-    #a (16 chunks) first, then b, the small one, c. Launches go at checkpoints - behind what the first launch reads, then
-    #every 16 MB or more, and at the end - so the launch on the small argument waits for the last one
-    assert at == [0, 16, 32, 49, 49], at
+    #the small one first (small arguments all go ahead, whoever reads them), then a (16 chunks), b, c. Launches go at
+    #checkpoints: behind what the first launch reads, then after 2 MB, 4 MB, ... more (here: every array), and at the end
+    assert at == [1, 17, 33, 33, 49], at
     held = xs
     #b stays where it is: a, the small one, c
     xs, ys, at = run(resident=(1,))
     assert np.array_equal(ys[0], xs[0] + 1) and np.array_equal(ys[1], held[1] + 1) and np.array_equal(ys[2], xs[2] + 1)
     assert np.array_equal(ys[3], xs[3] + 1)
-    assert at[0] == 0 and at[1] == 16 and at[4] == 33, at
+    assert at == [1, 17, 17, 17, 33], at
     assert lib.fake_hip_creations() == made
     assert lib.vkj_seq_destroy(seq) == 0
     for buf in (a, b, c, small, ra, rb, rc, rs, free):
         assert lib.vkj_buf_free(w.ctx, buf) == 0
+    w.close()
+    assert lib.fake_hip_live_objects() == before
+
+
+def test_packed_arrays_travel_in_one_transfer(lib):
+    '''vkj_buf_alloc_packed places small arrays side by side in a slab, a sequence stages their uploads side by side
+    too, and an evaluation that uploads neighbours sends them with one transfer; an array that stays resident splits
+    the run; larger requests get allocations of their own; the slab's memory goes with its last array, also when that
+    one was still recorded in a sequence when it was freed.'''
+    before = lib.fake_hip_live_objects()
+    w = World(lib)
+    sizes = [25, 256, 65, 1000, 7, 300]                            #words; 100 B ... 4000 B
+    n_big = 4 << 20
+    small, made = [], lib.fake_hip_live_objects()
+    for n in sizes:
+        b = H()
+        assert lib.vkj_buf_alloc_packed(w.ctx, 4 * n, C.byref(b)) == 0
+        small.append(b)
+    assert lib.fake_hip_live_objects() == made + 1                #ONE slab
+    addresses = []
+    for b in small:
+        addr = C.c_uint64()
+        assert lib.vkj_buf_device_ptr(w.ctx, b, C.byref(addr)) == 0
+        addresses.append(addr.value)
+    assert all((a - addresses[0]) % 256 == 0 for a in addresses)          #(the slab itself starts where hipMalloc puts it)
+    assert [b - a for a, b in zip(addresses, addresses[1:])] == [-(-4 * n // 256) * 256 for n in sizes[:-1]]
+    large = H()
+    assert lib.vkj_buf_alloc_packed(w.ctx, 4 * n_big, C.byref(large)) == 0          #too large for a slab: on its own
+    results = [w.buf(4 * n) for n in sizes] + [w.buf(4 * n_big)]
+    seq, without_sequence = H(), lib.fake_hip_live_objects()
+    assert lib.vkj_seq_create(w.ctx, 0, C.byref(seq)) == 0
+    for k, (b, n) in enumerate(zip(small + [large], sizes + [n_big])):
+        assert lib.vkj_seq_record_upload(seq, b, 0, k, 4 * n) == 0
+        assert w.record_add_one(seq, results[k], b, n) == 0
+    for k, n in enumerate(sizes + [n_big]):
+        assert lib.vkj_seq_record_download(seq, results[k], 0, 7 + k, 4 * n) == 0
+    rng = np.random.default_rng(12)
+    def run(resident=()):
+        xs = [rng.integers(0, 1 << 30, size=n, dtype=np.uint32) for n in sizes + [n_big]]
+        ys = [np.zeros(n, np.uint32) for n in sizes + [n_big]]
+        ptrs = (C.c_void_p * 14)(*[None if k in resident else x.ctypes.data for k, x in enumerate(xs)], *[y.ctypes.data for y in ys])
+        copies = lib.fake_hip_copies()
+        assert lib.vkj_seq_eval(seq, ptrs, 14, hip.EVAL_NULL_IS_RESIDENT if resident else 0) == 0, lib.vkj_last_error()
+        return xs, ys, lib.fake_hip_copies() - copies
+    xs, ys, copies = run()
+    assert all(np.array_equal(y, x + 1) for x, y in zip(xs, ys))
+    held = xs
+    _, ys, downloads = run(resident=range(7))                      #nothing goes up: what the results cost to bring back
+    assert all(np.array_equal(y, x + 1) for x, y in zip(held, ys))
+    assert copies - downloads == 1 + 16                            #one run for the six small arrays, the large one's chunks
+    xs, ys, copies = run(resident=(2,))
+    assert all(np.array_equal(y, (held[k] if k == 2 else x) + 1) for k, (x, y) in enumerate(zip(xs, ys)))
+    assert copies - downloads == 2 + 16                            #the arrays before and behind the one that stays
+    #freed while the sequence still holds them: the slab stays until the sequence goes
+    for b in small:
+        assert lib.vkj_buf_free(w.ctx, b) == 0
+    live = lib.fake_hip_live_objects()
+    xs, ys, copies = run()
+    assert all(np.array_equal(y, x + 1) for x, y in zip(xs, ys))
+    assert lib.fake_hip_live_objects() == live                     #nothing has gone yet
+    assert lib.vkj_seq_destroy(seq) == 0
+    assert lib.fake_hip_live_objects() == without_sequence - 1     #everything the sequence had made, and the slab
+    for b in [large] + results:
+        assert lib.vkj_buf_free(w.ctx, b) == 0
     w.close()
     assert lib.fake_hip_live_objects() == before
 

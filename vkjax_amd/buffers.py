@@ -49,7 +49,7 @@ class PlanOnlyDevice:
     def tensor(self, array: np.ndarray) -> PlannedTensor:
         return PlannedTensor(max(array.nbytes, 4), array)
 
-    def alloc(self, nbytes: int) -> PlannedTensor:
+    def alloc(self, nbytes: int, packed: bool = False) -> PlannedTensor:
         return PlannedTensor(nbytes)
 
     def sequence(self, profiling=False):
@@ -253,7 +253,9 @@ class BufferPool:
         if core.is_literal(var):
             initial_value = var.val
         if initial_value is None:
-            return self.device.alloc(max(int(np.prod(shape, dtype=np.int64)) * 4, 4))
+            #an argument or result of the program: the small ones among them lie side by side in HBM, so that a call
+            #sends a run of them with one transfer
+            return self.device.alloc(max(int(np.prod(shape, dtype=np.int64)) * 4, 4), packed=True)
         initial_value = np.asarray(initial_value)
         assert initial_value.size == int(np.prod(shape, dtype=np.int64)), (initial_value.shape, shape)
         return self.device.tensor(to_device_words(initial_value, dtype))

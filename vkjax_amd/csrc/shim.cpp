@@ -55,7 +55,7 @@ using namespace vkj;
 constexpr size_t STAGE_CHUNK     = 4u << 20;   // results on their way back
 constexpr size_t UPLOAD_CHUNK    = 1u << 20;   // arguments
 constexpr size_t STAGE_MIN       = 8u << 20;   // smaller transfers are copied inline
-constexpr size_t CHECKPOINT_BYTES = 16u << 20; // launches that follow the uploads: at least this much between two of their waits
+constexpr size_t CHECKPOINT_BYTES = 2u << 20;  // launches that follow the uploads: this much until their first wait behind the first launch, then twice as much each time
 constexpr int    STAGE_THREADS   = 8;
 constexpr int    UPLOAD_THREADS  = 4;
 
@@ -191,9 +191,22 @@ void destroy_ctx_objects(Ctx* c) {
 
 // A sequence lets go of a buffer it recorded; the memory of a buffer that vkj_buf_free has
 // already been called on is released with the last such reference.
+// The device memory of a buffer goes: its own allocation, or its share of a slab (the slab with its last array).
+hipError_t free_buf_memory(Buf* b) {
+    if (!b->slab) return hipFree(b->dptr);
+    Slab* slab = b->slab;
+    b->slab = nullptr;
+    if (--slab->live > 0) return hipSuccess;
+    auto& slabs = b->ctx->slabs;
+    slabs.erase(std::remove(slabs.begin(), slabs.end(), slab), slabs.end());
+    hipError_t e = hipFree(slab->base);
+    delete slab;
+    return e;
+}
+
 void unref_buf(Buf* b) {
     if (--b->seq_refs == 0 && b->released) {
-        hipFree(b->dptr);
+        free_buf_memory(b);
         delete b;
     }
 }
@@ -332,8 +345,16 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
                         auto range = piece_of.equal_range(b);
                         for (auto it = range.first; it != range.second; ++it) first_use[it->second] = std::min(first_use[it->second], i);
                     }
-                for (size_t p = 0; p < order.size(); p++) order[p] = p;
+                // (small arrays first, in the order they were recorded in: together they are a fraction of a megabyte, and
+                // neighbours in memory stay neighbours on the way, which lets one transfer carry a run of them)
+                for (size_t p = 0; p < order.size(); p++) {
+                    order[p] = p;
+                    if (pieces[p].nbytes <= PACKED_MAX_BYTES) first_use[p] = 0;
+                }
                 std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) {
+                    const bool small_a = pieces[a].nbytes <= PACKED_MAX_BYTES, small_b = pieces[b].nbytes <= PACKED_MAX_BYTES;
+                    if (small_a != small_b) return small_a;
+                    if (small_a) return false;
                     return first_use[a] != first_use[b] ? first_use[a] < first_use[b] : pieces[a].nbytes < pieces[b].nbytes;
                 });
                 std::vector<UploadPiece> sorted_pieces;
@@ -349,15 +370,13 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
                     while (p < pieces.size() && sorted_use[p] <= i) reached = (long)p++;
                     need[i] = reached;
                 }
-                // the first checkpoint lets the first launch go; behind it one per CHECKPOINT_BYTES or more, a handful in all
-                size_t rest = 0;
-                for (size_t q = (size_t)(need[0] + 1); q < pieces.size(); q++) rest += pieces[q].nbytes;
-                const size_t step = std::max<size_t>(CHECKPOINT_BYTES, rest / (Ctx::MAX_CHECKPOINTS - 2) + 1);
+                // the first checkpoint lets the first launch go; behind it a handful, the distance doubling from
+                // CHECKPOINT_BYTES on (the first layers of a network read little and should not wait for much)
                 if (need[0] >= 0 && (size_t)need[0] + 1 < pieces.size()) checkpoints.push_back((size_t)need[0]);
-                size_t since = 0;
+                size_t since = 0, step = CHECKPOINT_BYTES;
                 for (size_t q = (size_t)(need[0] + 1); q + 1 < pieces.size(); q++) {
                     since += pieces[q].nbytes;
-                    if (since >= step && (int)checkpoints.size() < Ctx::MAX_CHECKPOINTS - 1) { checkpoints.push_back(q); since = 0; }
+                    if (since >= step && (int)checkpoints.size() < Ctx::MAX_CHECKPOINTS - 1) { checkpoints.push_back(q); since = 0; step *= 2; }
                 }
                 checkpoints.push_back(pieces.size() - 1);
             }
@@ -383,10 +402,37 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
             while (follow && next_launch < nl && need[next_launch] < 0) {
                 if ((launch_status = issue_launch(c, s->launches[next_launch++]))) return launch_status;
             }
+            // Small arrays that lie next to each other in HBM and in their staging memory alike (vkj_buf_alloc_packed) are
+            // sent as one transfer: the run is extended while the next array starts within the alignment step behind it,
+            // by the same distance on both sides. Hundreds of transfers of a few KB each would cost more host time than
+            // the bytes take to travel.
+            struct { uintptr_t device = 0, staging = 0; size_t len = 0; hipStream_t stream = nullptr; } run;
+            auto flush_run = [&]() {
+                if (run.len) err = hipMemcpyAsync((void*)run.device, (const void*)run.staging, run.len, hipMemcpyHostToDevice, run.stream);
+                run.len = 0;
+                return err == hipSuccess;
+            };
             const int r = staged_upload_pieces(pieces, [&](size_t k, size_t piece, size_t off, size_t len) {
-                err = hipMemcpyAsync(pieces[piece].device + off, pieces[piece].staging + off, len, hipMemcpyHostToDevice,
-                                     (k & 1) ? copy_odd : copy_even);
-                if (err != hipSuccess) return 1;
+                const uintptr_t device = (uintptr_t)(pieces[piece].device + off), staging = (uintptr_t)(pieces[piece].staging + off);
+                hipStream_t to = (k & 1) ? copy_odd : copy_even;
+                if (pieces[piece].nbytes <= PACKED_MAX_BYTES) {
+                    const size_t step = device - run.device;
+                    if (run.len && device > run.device && step == staging - run.staging && step >= run.len && step < run.len + PACKED_ALIGN
+                            && step + len <= UPLOAD_CHUNK) {
+                        run.len = step + len;
+                    } else {
+                        if (!flush_run()) return 1;
+                        run.device = device; run.staging = staging; run.len = len; run.stream = to;
+                    }
+                } else {
+                    if (!flush_run()) return 1;
+                    err = hipMemcpyAsync((void*)device, (const void*)staging, len, hipMemcpyHostToDevice, to);
+                    if (err != hipSuccess) return 1;
+                }
+                const bool part_due = piece == early_piece && next_part < s->early.size() && s->early[next_part].bytes_needed <= off + len;
+                const bool checkpoint_due = follow && next_checkpoint < checkpoints.size() && piece == checkpoints[next_checkpoint]
+                                            && off + len == pieces[piece].nbytes;
+                if ((part_due || checkpoint_due) && !flush_run()) return 1;
                 while (piece == early_piece && next_part < s->early.size() && s->early[next_part].bytes_needed <= off + len) {
                     EarlyPart& part = s->early[next_part++];
                     if ((err = hipEventRecord(part.ev_a, copy_even)) != hipSuccess) return 1;
@@ -414,7 +460,7 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
                 return 0;
             });
             if (launch_status) return launch_status;
-            if (r) return hip_fail(err, "hipMemcpyAsync (staged upload)");
+            if (r || !flush_run()) return hip_fail(err, "hipMemcpyAsync (staged upload)");
             if (follow) {
                 first_launch = next_launch;          // all of them: the last checkpoint is the last piece
                 if (first_launch != nl) return fail(VKJ_ESTATE, "vkj_seq_eval: %zu of %zu launches issued beside the uploads", first_launch, nl);
@@ -728,6 +774,36 @@ int vkj_buf_alloc(vkj_handle h, size_t nbytes, vkj_handle* out) {
     return 0;
 }
 
+int vkj_buf_alloc_packed(vkj_handle h, size_t nbytes, vkj_handle* out) {
+    if (nbytes > PACKED_MAX_BYTES) return vkj_buf_alloc(h, nbytes, out);
+    Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
+    if (!c || !out) return fail(VKJ_EINVAL, "vkj_buf_alloc_packed: bad argument");
+    if (int r = use(c)) return r;
+    const size_t need = ((nbytes ? nbytes : 4) + PACKED_ALIGN - 1) & ~(PACKED_ALIGN - 1);
+    Slab* slab = c->slabs.empty() ? nullptr : c->slabs.back();
+    if (!slab || slab->used + need > slab->size) {
+        slab = new (std::nothrow) Slab();
+        if (!slab) return fail(VKJ_ENOMEM, "vkj_buf_alloc_packed: out of host memory");
+        hipError_t e = hipMalloc(&slab->base, SLAB_BYTES);
+        if (e != hipSuccess) { delete slab; return hip_fail(e, "hipMalloc (slab)"); }
+        slab->size = SLAB_BYTES;
+        c->slabs.push_back(slab);
+    }
+    Buf* b = new (std::nothrow) Buf();
+    if (!b) {
+        if (slab->live == 0) { c->slabs.pop_back(); hipFree(slab->base); delete slab; }
+        return fail(VKJ_ENOMEM, "vkj_buf_alloc_packed: out of host memory");
+    }
+    b->ctx = c;
+    b->nbytes = nbytes;
+    b->dptr = (char*)slab->base + slab->used;
+    b->slab = slab;
+    slab->used += need;
+    slab->live++;
+    *out = to_handle(b);
+    return 0;
+}
+
 int vkj_buf_free(vkj_handle h, vkj_handle bh) {
     Ctx* c = from_handle<Ctx>(h, MAGIC_CTX);
     Buf* b = from_handle<Buf>(bh, MAGIC_BUF);
@@ -742,7 +818,7 @@ int vkj_buf_free(vkj_handle h, vkj_handle bh) {
     }
     HIP_TRY(hipStreamSynchronize(c->stream));
     HIP_TRY(hipStreamSynchronize(c->copy_stream));
-    HIP_TRY(hipFree(b->dptr));
+    HIP_TRY(free_buf_memory(b));
     retire(b);
     delete b;
     return 0;
@@ -823,8 +899,9 @@ int vkj_seq_destroy(vkj_handle sh) {
     if (int r = use(s->ctx)) return r;
     hipStreamSynchronize(s->ctx->stream);
     hipStreamSynchronize(s->ctx->copy_stream);
+    for (auto& m : s->slab_mirrors) hipHostFree(m.second);
     for (auto& t : s->uploads) {
-        if (t.staging) hipHostFree(t.staging);
+        if (t.staging && !t.staging_mirrors_slab) hipHostFree(t.staging);
         if (t.next_staging) hipHostFree(t.next_staging);
         if (t.landing) hipFree(t.landing);
         unref_buf(t.buf);
@@ -863,7 +940,20 @@ static int record_transfer(const char* who, std::vector<Transfer>& list, Seq* s,
     if (int r = check_range(who, b, offset, nbytes)) return r;
     if (int r = use(s->ctx)) return r;
     Transfer t{b, offset, nbytes, slot, nullptr};
-    if (nbytes) HIP_TRY(hipHostMalloc(&t.staging, nbytes, hipHostMallocDefault));
+    if (nbytes && b->slab && &list == &s->uploads) {
+        // staged at the array's place in a pinned copy of its slab: arrays that are neighbours in HBM are neighbours
+        // there too, and one transfer can carry a run of them
+        void* mirror = nullptr;
+        for (auto& m : s->slab_mirrors) if (m.first == b->slab) mirror = m.second;
+        if (!mirror) {
+            HIP_TRY(hipHostMalloc(&mirror, b->slab->size, hipHostMallocDefault));
+            s->slab_mirrors.emplace_back(b->slab, mirror);
+        }
+        t.staging = (char*)mirror + ((char*)b->dptr - (char*)b->slab->base) + offset;
+        t.staging_mirrors_slab = true;
+    } else if (nbytes) {
+        HIP_TRY(hipHostMalloc(&t.staging, nbytes, hipHostMallocDefault));
+    }
     list.push_back(t);
     b->seq_refs++;
     return 0;

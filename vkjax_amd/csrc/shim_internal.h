@@ -28,6 +28,16 @@ int hip_fail(hipError_t e, const char* what);
 constexpr uint32_t MAGIC_CTX = 0x766b4a43, MAGIC_BUF = 0x766b4a42, MAGIC_MOD = 0x766b4a4d,
                    MAGIC_FN = 0x766b4a46, MAGIC_SEQ = 0x766b4a53;
 
+// Small arrays that travel together (a network's per-feature vectors) are carved out of slabs, one next to the other
+// at 256-byte steps (vkj_buf_alloc_packed), so that an evaluation can send a run of them with one transfer. A slab
+// goes when the last array carved from it has gone; space is not handed out twice.
+struct Slab {
+    void*  base = nullptr;
+    size_t size = 0, used = 0;
+    int    live = 0;
+};
+constexpr size_t SLAB_BYTES = 1u << 20, PACKED_MAX_BYTES = 64u << 10, PACKED_ALIGN = 256;
+
 struct Ctx {
     uint64_t    handle = 0;
     uint32_t    magic = MAGIC_CTX;
@@ -44,6 +54,7 @@ struct Ctx {
     // so far (one event per copy stream and checkpoint), before the launches that need no more than that are issued.
     static constexpr int MAX_CHECKPOINTS = 8;
     hipStream_t copy_stream2 = nullptr;
+    std::vector<Slab*> slabs;            // those with live arrays; the last one is the one being filled
     hipEvent_t  ev_checkpoint[2 * MAX_CHECKPOINTS] = {};
     void*       static_landing = nullptr;   // this device's copy of the static landing array (static_landing.hip)
 };
@@ -58,6 +69,7 @@ struct Buf {
     size_t   nbytes = 0;
     int      seq_refs = 0;       // recorded transfers and launch arguments of live sequences
     bool     released = false;   // vkj_buf_free was called; memory goes when seq_refs drops to 0
+    Slab*    slab = nullptr;     // the slab `dptr` points into (vkj_buf_alloc_packed), or null: an allocation of its own
 };
 
 struct Fn;
@@ -83,6 +95,7 @@ struct Transfer {
     size_t offset, nbytes;
     int    slot;
     void*  staging;                  // pinned host memory owned by the sequence
+    bool   staging_mirrors_slab = false;   // ... inside the sequence's pinned copy of the buffer's slab, at the buffer's place in it
     void*  next_staging = nullptr;   // pinned host memory and device memory for the arguments of the
     void*  landing = nullptr;        // following evaluation, allocated when one is first handed in
 };
@@ -121,6 +134,7 @@ struct Seq {
     bool                    want_graph = false;     // issue the launches as one captured graph
     bool                    graph_failed = false;   // capture did not work once: keep to plain launches
     hipGraphExec_t          graph_exec = nullptr;
+    std::vector<std::pair<Slab*, void*>> slab_mirrors;   // pinned memory laid out like a slab: the staging of the uploads into its arrays
     std::vector<EarlyPart>  early;                  // the first launch in parts, each issued while the rest of an argument is still on its way
     int                     early_slot = -1;
     hipEvent_t              ev_early_done = nullptr;

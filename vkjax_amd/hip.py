@@ -47,6 +47,7 @@ _PROTOTYPES = {
     'vkj_module_unload':       (C.c_int, [_H, _H]),
     'vkj_module_get_function': (C.c_int, [_H, _H, C.c_char_p, C.POINTER(_H)]),
     'vkj_buf_alloc':           (C.c_int, [_H, C.c_size_t, C.POINTER(_H)]),
+    'vkj_buf_alloc_packed':    (C.c_int, [_H, C.c_size_t, C.POINTER(_H)]),
     'vkj_buf_free':            (C.c_int, [_H, _H]),
     'vkj_buf_size':            (C.c_int, [_H, _H, C.POINTER(C.c_size_t)]),
     'vkj_buf_device_ptr':      (C.c_int, [_H, _H, C.POINTER(C.c_uint64)]),
@@ -114,11 +115,13 @@ def device_count() -> int:
 
 class DeviceBuffer:
     '''One HBM allocation (the counterpart of a kp.Tensor). Hashable by identity.'''
-    def __init__(self, device: 'Device', nbytes: int):
+    def __init__(self, device: 'Device', nbytes: int, packed: bool = False):
         self.device = device
         self.nbytes = int(nbytes)
         h = _H(0)
-        _check(device.lib.vkj_buf_alloc(device.ctx, self.nbytes, C.byref(h)), f'vkj_buf_alloc({nbytes})')
+        #(packed: a small array that is uploaded together with others, placed next to them: vkj_buf_alloc_packed)
+        name = 'vkj_buf_alloc_packed' if packed else 'vkj_buf_alloc'
+        _check(getattr(device.lib, name)(device.ctx, self.nbytes, C.byref(h)), f'{name}({nbytes})')
         self.handle = h.value
 
     def upload(self, array: np.ndarray, offset: int = 0):
@@ -223,8 +226,8 @@ class Device:
                 raise NotImplementedError(f'no kernel named {kernel_name} in the loaded code objects (status {last})')
         return self._functions[kernel_name]
 
-    def alloc(self, nbytes: int) -> DeviceBuffer:
-        return DeviceBuffer(self, nbytes)
+    def alloc(self, nbytes: int, packed: bool = False) -> DeviceBuffer:
+        return DeviceBuffer(self, nbytes, packed)
 
     def tensor(self, array: np.ndarray) -> DeviceBuffer:
         '''Allocate and upload (blocking), like mgr.tensor + OpTensorSyncDevice (reference: vkjax/buffers.py:202-203).'''
