@@ -178,7 +178,7 @@ def test_buffer_freed_under_a_live_sequence_outlives_it(lib):
 
 def test_context_creation_releases_everything_when_a_step_fails(lib):
     before = lib.fake_hip_live_objects()
-    made = 4 + 5 + 16                                            #four streams, five events, sixteen checkpoint events are created
+    made = 3 + 5 + 16                                            #three streams, five events, sixteen checkpoint events are created
     for successes in range(made):
         lib.fake_hip_fail_after(successes)
         ctx = H()

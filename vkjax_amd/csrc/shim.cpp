@@ -182,11 +182,10 @@ void destroy_ctx_objects(Ctx* c) {
     if (c->ev_copied)   hipEventDestroy(c->ev_copied);
     if (c->stream)      hipStreamDestroy(c->stream);
     if (c->copy_stream) hipStreamDestroy(c->copy_stream);
-    if (c->copy_stream2) hipStreamDestroy(c->copy_stream2);
     for (auto& e : c->ev_checkpoint) { if (e) hipEventDestroy(e); e = nullptr; }
     if (c->side_stream) hipStreamDestroy(c->side_stream);
     c->ev_begin = c->ev_end = c->ev_landed = c->ev_uploaded = c->ev_copied = nullptr;
-    c->stream = c->copy_stream = c->copy_stream2 = c->side_stream = nullptr;
+    c->stream = c->copy_stream = c->side_stream = nullptr;
 }
 
 // A sequence lets go of a buffer it recorded; the memory of a buffer that vkj_buf_free has
@@ -383,7 +382,10 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
             // Without that the chunks alternate between the launch stream and the copy stream (two copy engines work on
             // them) and the launches wait for both. All streams are idle here: every evaluation ends with everything
             // it queued on them complete.
-            hipStream_t copy_even = follow ? c->copy_stream2 : c->stream, copy_odd = c->copy_stream;
+            hipStream_t copy_even = follow ? c->side_stream : c->stream, copy_odd = c->copy_stream;
+            // (the parts of the first launch: on the side stream beside chunks on the launch stream, or - the side stream
+            // carrying chunks - on the launch stream itself, which has nothing else to do until the first checkpoint)
+            hipStream_t parts_stream = follow ? c->stream : c->side_stream;
             // The first launch in parts: a part goes to the side stream as soon as the chunks it reads have been
             // handed to the copy engines (both streams are in order: an event behind a chunk covers every chunk
             // before it), so the device computes while the rest of the argument is still on its way. Only with that
@@ -437,9 +439,9 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
                     EarlyPart& part = s->early[next_part++];
                     if ((err = hipEventRecord(part.ev_a, copy_even)) != hipSuccess) return 1;
                     if ((err = hipEventRecord(part.ev_b, copy_odd)) != hipSuccess) return 1;
-                    if ((err = hipStreamWaitEvent(c->side_stream, part.ev_a, 0)) != hipSuccess) return 1;
-                    if ((err = hipStreamWaitEvent(c->side_stream, part.ev_b, 0)) != hipSuccess) return 1;
-                    if ((launch_status = issue_launch(c, part.launch, c->side_stream))) return 1;
+                    if ((err = hipStreamWaitEvent(parts_stream, part.ev_a, 0)) != hipSuccess) return 1;
+                    if ((err = hipStreamWaitEvent(parts_stream, part.ev_b, 0)) != hipSuccess) return 1;
+                    if ((launch_status = issue_launch(c, part.launch, parts_stream))) return 1;
                 }
                 if (follow && next_checkpoint < checkpoints.size() && piece == checkpoints[next_checkpoint] && off + len == pieces[piece].nbytes) {
                     hipEvent_t ev_even = c->ev_checkpoint[2 * next_checkpoint], ev_odd = c->ev_checkpoint[2 * next_checkpoint + 1];
@@ -448,12 +450,8 @@ int vkj::seq_eval(Seq* s, void* const* host_ptrs, int nslots, uint32_t flags, vo
                     if ((err = hipEventRecord(ev_odd, copy_odd)) != hipSuccess) return 1;
                     if ((err = hipStreamWaitEvent(c->stream, ev_even, 0)) != hipSuccess) return 1;
                     if ((err = hipStreamWaitEvent(c->stream, ev_odd, 0)) != hipSuccess) return 1;
-                    if (piece == early_piece && next_launch == 0) {
-                        // (every part has been issued: the last one needs no more than the whole argument)
-                        if ((err = hipEventRecord(s->ev_early_done, c->side_stream)) != hipSuccess) return 1;
-                        if ((err = hipStreamWaitEvent(c->stream, s->ev_early_done, 0)) != hipSuccess) return 1;
-                        next_launch = 1;
-                    }
+                    // (every part of the first launch has been issued, on this stream: the last one needs no more than the whole argument)
+                    if (piece == early_piece && next_launch == 0) next_launch = 1;
                     while (next_launch < nl && need[next_launch] <= (long)piece)
                         if ((launch_status = issue_launch(c, s->launches[next_launch++]))) return 1;
                 }
@@ -650,7 +648,6 @@ int vkj_ctx_create(int device, vkj_handle* out) {
         HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
         HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
         HIP_TRY(hipStreamCreateWithFlags(&c->side_stream, hipStreamNonBlocking));
-        HIP_TRY(hipStreamCreateWithFlags(&c->copy_stream2, hipStreamNonBlocking));
         for (auto& e : c->ev_checkpoint) HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
         HIP_TRY(hipEventCreate(&c->ev_begin));
         HIP_TRY(hipEventCreate(&c->ev_end));
@@ -674,7 +671,6 @@ int vkj_ctx_destroy(vkj_handle h) {
     if (int r = use(c)) return r;
     hipStreamSynchronize(c->stream);
     hipStreamSynchronize(c->copy_stream);
-    hipStreamSynchronize(c->copy_stream2);
     hipStreamSynchronize(c->side_stream);
     destroy_ctx_objects(c);
     retire(c);

@@ -49,13 +49,15 @@ struct Ctx {
     hipEvent_t  ev_landed = nullptr;     // the following evaluation's arguments have reached HBM
     hipEvent_t  ev_uploaded = nullptr;   // this evaluation's own uploads have left their staging buffers
     hipEvent_t  ev_copied = nullptr;     // the share of this evaluation's uploads that went over the second stream has arrived
-    // Launches that follow the uploads (seq_eval): the chunks then alternate between copy_stream and copy_stream2, and
+    // Launches that follow the uploads (seq_eval): the chunks then alternate between copy_stream and side_stream, and
     // at each of a few checkpoints along the upload the launch stream is told to wait for what both have been handed
     // so far (one event per copy stream and checkpoint), before the launches that need no more than that are issued.
+    // (No further stream for this: a process has few hardware queues, streams are dealt out over them in turn, and
+    // with three streams per context the launch streams of up to four contexts end up on different queues - which is
+    // what lets the lanes of Function.stream(in_flight=...) run side by side. With four they all shared one.)
     static constexpr int MAX_CHECKPOINTS = 8;
-    hipStream_t copy_stream2 = nullptr;
-    std::vector<Slab*> slabs;            // those with live arrays; the last one is the one being filled
     hipEvent_t  ev_checkpoint[2 * MAX_CHECKPOINTS] = {};
+    std::vector<Slab*> slabs;            // those with live arrays; the last one is the one being filled
     void*       static_landing = nullptr;   // this device's copy of the static landing array (static_landing.hip)
 };
 
