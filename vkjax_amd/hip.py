@@ -194,6 +194,25 @@ class Device:
             self._images.append(buf)
         self._props = None
 
+    def close(self):
+        '''Unloads the code objects and destroys the context. Only for contexts made directly (the lanes of
+        Function.stream(in_flight=...)): everything allocated or recorded on the context holds a reference to this
+        object, so it is collected - and closed - after the last of them has gone. The shared contexts of get() live as
+        long as the process.'''
+        if getattr(self, 'ctx', 0):
+            for module in self._modules.values():
+                self.lib.vkj_module_unload(self.ctx, module)
+            self._modules.clear()
+            self._functions.clear()
+            self.lib.vkj_ctx_destroy(self.ctx)
+            self.ctx = 0
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
     @property
     def props(self) -> Props:
         if self._props is None:
