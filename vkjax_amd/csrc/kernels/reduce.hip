@@ -628,7 +628,14 @@ struct PoolParams {
     uint32_t in_dims[4], out_dims[4];
     uint32_t window[4], stride[4], dilation[4];
     int32_t  pad_low[4];
+    // the 2-D kernels (pool2d, select_window2d, scatter_selected2d): n / d = mulhi(n, magic) >> shift (magic 0: d = 1) for
+    // the three extents a thread decodes its element number with: channels, width, height of the array the launch writes
+    // (prepared on the host; three divisions by run-time values cost a thread some 120 instructions)
+    uint32_t div_magic[3], div_shift[3];
 };
+
+// n / s for n >= 0 and a window stride s: 1 or 2, the usual ones, without a division
+__device__ __forceinline__ int32_t div_stride(int32_t n, int32_t s) { return s == 1 ? n : s == 2 ? n >> 1 : n / s; }
 
 template <int VEC>
 __device__ __forceinline__ void pool_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ in, const PoolParams& P) {
@@ -691,10 +698,11 @@ __device__ __forceinline__ void pool2d_body(uint32_t* __restrict__ out, const ui
     const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u;
     if (e0 >= P.n_out) return;
     const uint32_t C = P.out_dims[3], Wo = P.out_dims[2], Ho = P.out_dims[1];
-    uint32_t r = e0 / C;
+    const uint32_t r = (uint32_t)magic_div((int)e0, P.div_magic[0], P.div_shift[0]);
     const uint32_t c = e0 - r * C;
-    const uint32_t wo = r % Wo; r /= Wo;
-    const uint32_t ho = r % Ho, b = r / Ho;
+    const uint32_t q = (uint32_t)magic_div((int)r, P.div_magic[1], P.div_shift[1]);
+    const uint32_t wo = r - q * Wo;
+    const uint32_t b = (uint32_t)magic_div((int)q, P.div_magic[2], P.div_shift[2]), ho = q - b * Ho;
     const int32_t y0 = (int32_t)(ho * P.stride[1]) - P.pad_low[1], x0 = (int32_t)(wo * P.stride[2]) - P.pad_low[2];
     const uint32_t ident = MODE == 0 ? 0u : MODE == 1 ? 0xFF800000u : red_identity(P.op, P.type);
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(in), 0,
@@ -821,8 +829,8 @@ __device__ __forceinline__ void scatter_selected_body(uint32_t* __restrict__ out
     for (int d = 0; d < 4; ++d) {
         const int32_t s = (int32_t)P.stride[d], a = c[d] + P.pad_low[d];
         const int32_t first = a - (int32_t)P.window[d] + 1;
-        lo[d] = first <= 0 ? 0 : (first + s - 1) / s;
-        hi[d] = a < 0 ? -1 : a / s;
+        lo[d] = first <= 0 ? 0 : div_stride(first + s - 1, s);
+        hi[d] = a < 0 ? -1 : div_stride(a, s);
         if (hi[d] > (int32_t)P.out_dims[d] - 1) hi[d] = (int32_t)P.out_dims[d] - 1;
     }
     if constexpr (VEC == 4) { lo[3] = hi[3] = 0; }           // the last dimension is not windowed: handled per lane element
@@ -871,10 +879,11 @@ __device__ __forceinline__ void select_window2d_body(uint32_t* __restrict__ sel_
     const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u;
     if (e0 >= P.n_out) return;
     const uint32_t C = P.out_dims[3], Wo = P.out_dims[2], Ho = P.out_dims[1];
-    uint32_t r = e0 / C;
+    const uint32_t r = (uint32_t)magic_div((int)e0, P.div_magic[0], P.div_shift[0]);
     const uint32_t c = e0 - r * C;
-    const uint32_t wo = r % Wo; r /= Wo;
-    const uint32_t ho = r % Ho, b = r / Ho;
+    const uint32_t q = (uint32_t)magic_div((int)r, P.div_magic[1], P.div_shift[1]);
+    const uint32_t wo = r - q * Wo;
+    const uint32_t b = (uint32_t)magic_div((int)q, P.div_magic[2], P.div_shift[2]), ho = q - b * Ho;
     const int32_t y0 = (int32_t)(ho * P.stride[1]) - P.pad_low[1], x0 = (int32_t)(wo * P.stride[2]) - P.pad_low[2];
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(operand), 0,
         (int)(P.in_dims[0] * P.in_dims[1] * P.in_dims[2] * P.in_dims[3] * 4u), 0x00020000);
@@ -908,7 +917,9 @@ __device__ __forceinline__ void select_window2d_body(uint32_t* __restrict__ sel_
             }
             have = have || inside[ky][kx];
         }
-    *reinterpret_cast<u32x4*>(sel_out + e0) = u32x4{pick[0], pick[1], pick[2], pick[3]};
+    // a thread's four selections share one word, a byte each (0xFF: an empty window), word number e0 / 4: a quarter of the
+    // bytes to write here and to read in the launch that follows
+    sel_out[e0 >> 2] = (pick[0] & 255u) | (pick[1] & 255u) << 8 | (pick[2] & 255u) << 16 | (pick[3] & 255u) << 24;
 }
 
 // NY x NX: the most windows an element can lie in, ceil(window / stride) per dimension (the host picks the variant):
@@ -919,24 +930,26 @@ __device__ __forceinline__ void scatter_selected2d_body(uint32_t* __restrict__ o
     const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u, n_out = without_stream_bit(P.n_out);
     if (e0 >= n_out) return;
     const uint32_t C = P.in_dims[3], W = P.in_dims[2], H = P.in_dims[1];
-    uint32_t r = e0 / C;
+    const uint32_t r = (uint32_t)magic_div((int)e0, P.div_magic[0], P.div_shift[0]);
     const uint32_t c = e0 - r * C;
-    const uint32_t x = r % W; r /= W;
-    const uint32_t y = r % H, b = r / H;
+    const uint32_t q = (uint32_t)magic_div((int)r, P.div_magic[1], P.div_shift[1]);
+    const uint32_t x = r - q * W;
+    const uint32_t b = (uint32_t)magic_div((int)q, P.div_magic[2], P.div_shift[2]), y = q - b * H;
     // windows that contain the element: o * stride - pad <= coordinate < o * stride - pad + window; at most KH x KW of them
     int32_t lo[2], hi[2];
 #pragma unroll
     for (int d = 0; d < 2; ++d) {
         const int32_t s = (int32_t)P.stride[d + 1], a = (int32_t)(d ? x : y) + P.pad_low[d + 1];
         const int32_t first = a - (d ? KW : KH) + 1;
-        lo[d] = first <= 0 ? 0 : (first + s - 1) / s;
-        hi[d] = a < 0 ? -1 : a / s;
+        lo[d] = first <= 0 ? 0 : div_stride(first + s - 1, s);
+        hi[d] = a < 0 ? -1 : div_stride(a, s);
         if (hi[d] > (int32_t)P.out_dims[d + 1] - 1) hi[d] = (int32_t)P.out_dims[d + 1] - 1;
     }
     const uint32_t nwin_bytes = P.out_dims[0] * P.out_dims[1] * P.out_dims[2] * P.out_dims[3] * 4u;
     const __amdgpu_buffer_rsrc_t r_sel = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(selected), 0, (int)nwin_bytes, 0x00020000),
                                  r_src = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(source), 0, (int)nwin_bytes, 0x00020000);
-    u32x4 s[NY][NX], g[NY][NX];
+    uint32_t s[NY][NX];                  // the selections of four channels, a byte each (select_window2d_body)
+    u32x4 g[NY][NX];
     uint32_t tap[NY][NX];
 #pragma unroll
     for (int i = 0; i < NY; ++i)
@@ -946,9 +959,9 @@ __device__ __forceinline__ void scatter_selected2d_body(uint32_t* __restrict__ o
             const bool ok = oy <= hi[0] && ox <= hi[1];
             // this element's tap number inside that window (no window: a number no selection holds)
             tap[i][j] = ok ? (uint32_t)(((int32_t)y + P.pad_low[1] - oy * (int32_t)P.stride[1]) * KW + ((int32_t)x + P.pad_low[2] - ox * (int32_t)P.stride[2]))
-                           : 0xFFFFFFFEu;
+                           : 0xFEu;
             const uint32_t off = ((b * P.out_dims[1] + (uint32_t)oy) * P.out_dims[2] + (uint32_t)ox) * C + c;
-            s[i][j] = __builtin_amdgcn_raw_buffer_load_b128(r_sel, ok ? off * 4u : 0x80000000u, 0, 0);
+            s[i][j] = __builtin_amdgcn_raw_buffer_load_b32(r_sel, ok ? off : 0x80000000u, 0, 0);       // word off / 4
             g[i][j] = __builtin_amdgcn_raw_buffer_load_b128(r_src, ok ? off * 4u : 0x80000000u, 0, 0);
         }
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -956,10 +969,10 @@ __device__ __forceinline__ void scatter_selected2d_body(uint32_t* __restrict__ o
     for (int i = 0; i < NY; ++i)
 #pragma unroll
         for (int j = 0; j < NX; ++j) {
-            if (s[i][j].x == tap[i][j]) acc[0] += u2f(g[i][j].x);
-            if (s[i][j].y == tap[i][j]) acc[1] += u2f(g[i][j].y);
-            if (s[i][j].z == tap[i][j]) acc[2] += u2f(g[i][j].z);
-            if (s[i][j].w == tap[i][j]) acc[3] += u2f(g[i][j].w);
+            if ((s[i][j] & 255u) == tap[i][j])         acc[0] += u2f(g[i][j].x);
+            if ((s[i][j] >> 8 & 255u) == tap[i][j])    acc[1] += u2f(g[i][j].y);
+            if ((s[i][j] >> 16 & 255u) == tap[i][j])   acc[2] += u2f(g[i][j].z);
+            if ((s[i][j] >> 24) == tap[i][j])          acc[3] += u2f(g[i][j].w);
         }
     store_x4(out, e0, u32x4{f2u(acc[0]), f2u(acc[1]), f2u(acc[2]), f2u(acc[3])}, streams_result(P.n_out), n_out * 4u);
 }

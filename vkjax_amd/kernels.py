@@ -1112,6 +1112,12 @@ def reduce_general(out: Buffer, inp: Buffer, kept, reduced, op: str) -> Launch:
                   bytes_moved=4 * (inp.size + out.size))
 
 
+def _pool_divisions(dims) -> bytes:
+    '''PoolParams.div_magic / div_shift for an array [batch, height, width, channels]: channels, width, height.'''
+    pairs = [_magic_division(d) for d in (dims[3], dims[2], dims[1])]
+    return _u32(*[m for m, _ in pairs], *[sh for _, sh in pairs])
+
+
 def pool(out: Buffer, inp: Buffer, op: str, window, strides, pad_low, dilation) -> Launch:
     rank = len(inp.shape)
     if rank > 4:
@@ -1126,7 +1132,8 @@ def pool(out: Buffer, inp: Buffer, op: str, window, strides, pad_low, dilation) 
     n   = out.size
     vec = 4 if (window[3] == 1 and strides[3] == 1 and pad_low[3] == 0 and in_dims[3] % 4 == 0
                 and in_dims[3] == out_dims[3]) else 1
-    params = _u32(n, RED[op], _RTYPE[inp.dtype], *in_dims, *out_dims, *window, *strides, *dilation) + _i32(*pad_low)
+    params = (_u32(n, RED[op], _RTYPE[inp.dtype], *in_dims, *out_dims, *window, *strides, *dilation) + _i32(*pad_low)
+              + _pool_divisions(out_dims))
     #[batch, y, x, channels] with a 3x3 or 2x2 window over y and x: the kernel that requests all taps at once
     if (vec == 4 and window[0] == 1 and strides[0] == 1 and pad_low[0] == 0 and in_dims[0] == out_dims[0]
             and (window[1], window[2]) in ((3, 3), (2, 2)) and inp.size * 4 < 2**31 and n * 4 < 2**32):
@@ -1163,9 +1170,9 @@ def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, selected: B
         most = max(_cdiv(window[1], strides[1]), _cdiv(window[2], strides[2]))
         select, scatter = f'select_window2d_{window[1]}x{window[2]}_v4', f'scatter_selected2d_{window[1]}x{window[2]}_n{most}x{most}_v4'
     first  = Launch(select, (_cdiv(_cdiv(n_win, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
-                    [(selected, 0), (operand, 0)], _u32(n_win) + tail, bytes_moved=4 * (operand.size + source.size))
+                    [(selected, 0), (operand, 0)], _u32(n_win) + tail + _pool_divisions(out_dims), bytes_moved=4 * (operand.size + source.size))
     second = Launch(scatter, (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
-                    [(out, 0), (source, 0), (selected, 0)], _u32(n) + tail, bytes_moved=4 * (operand.size + 2 * source.size),
+                    [(out, 0), (source, 0), (selected, 0)], _u32(n) + tail + _pool_divisions(in_dims), bytes_moved=4 * (operand.size + 2 * source.size),
                     streamable=vec == 4 and n < 2**31)
     return [first, second]
 
