@@ -194,7 +194,7 @@ def test_training_steps_plan_at_full_size(name):
     kernels = [l.kernel for l in interp.launches]
     assert any(k.startswith('conv_gemm') for k in kernels)
     if name == 'convnet_train':
-        assert 'select_window2d_3x3_v4' in kernels and 'scatter_selected2d_3x3_n2x2_v4' in kernels and any(k.startswith('pad_nd') for k in kernels), kernels
+        assert 'select_window2d_3x3_v4' in kernels and 'scatter_selected2d_3x3_s2_v4' in kernels and any(k.startswith('pad_nd') for k in kernels), kernels
 
 
 @pytest.mark.parametrize('f,args', pad_cases, ids=[c[0].__name__ for c in pad_cases])
@@ -229,7 +229,9 @@ def test_select_and_scatter_add_hip(desc, window, strides, padding, x, select):
     from vkjax_amd import kernels as K
     g = random(_pooled(x.shape, window, strides, padding)) + 0.25
     kernels = []
-    for two_d in (None, False):                              #the kernels for [batch, y, x, channels] where they apply, and the general ones
+    #the kernels for [batch, y, x, channels] where they apply (with the one for groups of 2 x 2 elements under 3 x 3 windows at a
+    #stride of 2, and without it), and the general ones
+    for two_d in (None, False, 'elements'):
         print(f'case: {desc}, 2-D kernels {two_d}', flush=True)
         with K.overrides(pool_gradient_2d=two_d):
             _, _, fn = check_against_oracle(pool_grad(window, strides, padding, select), [g, x], exact=True)
@@ -237,6 +239,8 @@ def test_select_and_scatter_add_hip(desc, window, strides, padding, x, select):
     assert all('2d' not in k for k in kernels[1])
     applies = len(window) == 4 and (window[0], window[3]) == (1, 1) and window[1:3] in ((3, 3), (2, 2)) and x.shape[3] % 4 == 0
     assert all('2d' in k for k in kernels[0]) == applies and bool(kernels[0]), (desc, kernels)
+    assert all('2d' in k for k in kernels[2]) == applies and not any(k.endswith('_s2_v4') for k in kernels[2]), (desc, kernels)
+    assert any(k.endswith('3x3_s2_v4') for k in kernels[0]) == (applies and window[1:3] == (3, 3) and strides[1:3] == (2, 2)), (desc, kernels)
 
 
 @pytest.mark.gpu

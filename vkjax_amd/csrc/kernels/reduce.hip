@@ -977,6 +977,71 @@ __device__ __forceinline__ void scatter_selected2d_body(uint32_t* __restrict__ o
     store_x4(out, e0, u32x4{f2u(acc[0]), f2u(acc[1]), f2u(acc[2]), f2u(acc[3])}, streams_result(P.n_out), n_out * 4u);
 }
 
+// 3 x 3 windows at a stride of 2 in both directions, the usual pooling of a network's stem: a thread owns the 2 x 2
+// elements (by four channels) whose padded coordinates are (2t, 2t + 1) x (2u, 2u + 1). Those four lie in the windows
+// (t - 1 .. t) x (u - 1 .. u) and in no other, each at a fixed tap: four (selection, source) pairs serve four results,
+// where one thread per element reads up to four pairs for one. Same sums in the same order (windows ascending).
+// P.n_out counts the elements of the array of such groups, [batch, T, U, channels]; P.div_magic divides by channels, U, T.
+__device__ __forceinline__ void scatter_selected2d_3x3_s2_body(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                               const uint32_t* __restrict__ selected, const PoolParams& P) {
+    const uint32_t e0 = (xcd_contiguous_block() * 256u + threadIdx.x) * 4u, n_groups = without_stream_bit(P.n_out);
+    if (e0 >= n_groups) return;
+    const uint32_t C = P.in_dims[3], W = P.in_dims[2], H = P.in_dims[1];
+    const int32_t py = P.pad_low[1], px = P.pad_low[2];
+    const uint32_t t0 = (uint32_t)py >> 1, u0 = (uint32_t)px >> 1;
+    const uint32_t T = ((H + (uint32_t)py - 1u) >> 1) - t0 + 1u, U = ((W + (uint32_t)px - 1u) >> 1) - u0 + 1u;
+    const uint32_t r = (uint32_t)magic_div((int)e0, P.div_magic[0], P.div_shift[0]);
+    const uint32_t c = e0 - r * C;
+    const uint32_t q = (uint32_t)magic_div((int)r, P.div_magic[1], P.div_shift[1]);
+    const uint32_t b = (uint32_t)magic_div((int)q, P.div_magic[2], P.div_shift[2]);
+    const int32_t t = (int32_t)(q - b * T + t0), u = (int32_t)(r - q * U + u0);
+    const uint32_t nwin_bytes = P.out_dims[0] * P.out_dims[1] * P.out_dims[2] * P.out_dims[3] * 4u;
+    const __amdgpu_buffer_rsrc_t r_sel = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(selected), 0, (int)nwin_bytes, 0x00020000),
+                                 r_src = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(source), 0, (int)nwin_bytes, 0x00020000);
+    uint32_t s[2][2];                    // the selections of four channels, a byte each; 0xFF.. where there is no such window
+    u32x4 g[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int32_t oy = t - 1 + i, ox = u - 1 + j;
+            const bool ok = (uint32_t)oy < P.out_dims[1] && (uint32_t)ox < P.out_dims[2];
+            const uint32_t off = ((b * P.out_dims[1] + (uint32_t)oy) * P.out_dims[2] + (uint32_t)ox) * C + c;
+            const uint32_t word = __builtin_amdgcn_raw_buffer_load_b32(r_sel, ok ? off : 0x80000000u, 0, 0);       // word off / 4
+            s[i][j] = ok ? word : 0xFFFFFFFFu;
+            g[i][j] = __builtin_amdgcn_raw_buffer_load_b128(r_src, ok ? off * 4u : 0x80000000u, 0, 0);
+        }
+    // element (dy, dx) of the group holds tap (dy + 2 - 2 i, dx + 2 - 2 j) of window (i, j), where that is a tap (< 3)
+    const uint32_t result_bytes = P.in_dims[0] * H * W * C * 4u;
+    const bool stream = streams_result(P.n_out);
+#pragma unroll
+    for (int dy = 0; dy < 2; ++dy)
+#pragma unroll
+        for (int dx = 0; dx < 2; ++dx) {
+            const int32_t y = 2 * t + dy - py, x = 2 * u + dx - px;
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int ky = dy + 2 - 2 * i, kx = dx + 2 - 2 * j;
+                    if (ky > 2 || kx > 2) continue;
+                    const uint32_t tap = (uint32_t)(ky * 3 + kx);
+                    if ((s[i][j] & 255u) == tap)       acc[0] += u2f(g[i][j].x);
+                    if ((s[i][j] >> 8 & 255u) == tap)  acc[1] += u2f(g[i][j].y);
+                    if ((s[i][j] >> 16 & 255u) == tap) acc[2] += u2f(g[i][j].z);
+                    if ((s[i][j] >> 24) == tap)        acc[3] += u2f(g[i][j].w);
+                }
+            if ((uint32_t)y < H && (uint32_t)x < W)
+                store_x4(out, ((uint64_t)(b * H + (uint32_t)y) * W + (uint32_t)x) * C + c,
+                         u32x4{f2u(acc[0]), f2u(acc[1]), f2u(acc[2]), f2u(acc[3])}, stream, result_bytes);
+        }
+}
+extern "C" __global__ __launch_bounds__(256) void scatter_selected2d_3x3_s2_v4(uint32_t* __restrict__ out, const uint32_t* __restrict__ source,
+                                                                              const uint32_t* __restrict__ selected, PoolParams P) {
+    scatter_selected2d_3x3_s2_body(out, source, selected, P);
+}
+
 #define SELECT_WINDOW_2D(KH, KW)                                                                                                    \
     extern "C" __global__ __launch_bounds__(256) void select_window2d_##KH##x##KW##_v4(uint32_t* __restrict__ sel,                   \
                                                                                       const uint32_t* __restrict__ operand, PoolParams P) { \

@@ -43,7 +43,7 @@ class _Choices:
         conv_general=False,              #never pick the lean kernel variant
         conv_b_general=False,            #element-wise loads of the kernel operand also where 16-byte loads would do
         conv_ksplit=None,                #the four-waves-per-tile kernel: always (where it applies) / never
-        pool_gradient_2d=None,           #the 2-D kernels of a pooling gradient: None = where they apply, False = never
+        pool_gradient_2d=None,           #the 2-D kernels of a pooling gradient: None = where they apply, False = never, 'elements' = never the one for groups of 2 x 2 elements
         scatter_bucket_cap=None,         #slots per row in the sorted scatter-add's table of fixed-capacity buckets (0: no table)
         conv_dense_rows=None,            #the kernel for at most 16 output features: None = where it applies, False = never
         conv_mix=None,                   #mixed 64 x 64 / 32 x 32 tiling: None = by the heuristic, False = never, an int = that many M tiles stay 64 x 64
@@ -1174,6 +1174,14 @@ def select_scatter_add(out: Buffer, source: Buffer, operand: Buffer, selected: B
     second = Launch(scatter, (_cdiv(_cdiv(n, vec), BLOCK), 1, 1), (BLOCK, 1, 1),
                     [(out, 0), (source, 0), (selected, 0)], _u32(n) + tail + _pool_divisions(in_dims), bytes_moved=4 * (operand.size + 2 * source.size),
                     streamable=vec == 4 and n < 2**31)
+    #3 x 3 windows at a stride of 2: a thread per group of 2 x 2 elements (by four channels), which shares its windows' loads
+    if ('2d_3x3' in scatter and (strides[1], strides[2]) == (2, 2) and 0 <= pad_low[1] < 3 and 0 <= pad_low[2] < 3
+            and CHOICES.pool_gradient_2d != 'elements'):
+        groups = [((extent + pad - 1) >> 1) - (pad >> 1) + 1 for extent, pad in ((in_dims[1], pad_low[1]), (in_dims[2], pad_low[2]))]
+        n_groups = in_dims[0] * groups[0] * groups[1] * in_dims[3]
+        second = second._replace(kernel='scatter_selected2d_3x3_s2_v4', grid=(_cdiv(_cdiv(n_groups, 4), BLOCK), 1, 1),
+                                 params=_u32(n_groups) + tail + _pool_divisions([in_dims[0], groups[0], groups[1], in_dims[3]]),
+                                 streamable=n_groups < 2**31)
     return [first, second]
 
 
