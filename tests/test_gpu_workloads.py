@@ -792,6 +792,40 @@ def test_stream_loader_may_refill_its_batch_array():
             assert_tree_close(g, plain(v, w), exact=True, what=f'{shape} batch {k}')
 
 
+def test_launches_follow_the_uploads_of_a_network():
+    '''A call that copies every argument (writeable parameter arrays: the reference's semantics) sends them in the
+    order of first use, the small ones side by side in one transfer, and issues the launches while later weights are
+    still on their way. The results are those of the same program replayed on inputs uploaded one by one beforehand,
+    bit for bit, call after call with changed weights and images; the program contains launches that reach their
+    operands through a table (batched small chains at this batch size), which the runtime has to know as well.'''
+    rng = np.random.default_rng(47)
+    from vkjax_amd.minijax import tree_util
+    params, x = W.resnet50_inputs(batch=2, size=64, num_classes=100, width_scale=0.5)
+    assert sum(a.nbytes for a in tree_util.tree_leaves(params)) > (16 << 20)          #the chunked path, several checkpoints
+    fn = vkjax_amd.wrap(W.resnet50, frontend='minijax')
+    reference = vkjax_amd.wrap(W.resnet50, frontend='minijax')
+    reference(params, x)
+    interp = list(reference._jaxpr_interpreters.values())[0]
+    previous = None
+    for call in range(3):
+        print(f'case: every argument copied, call {call}', flush=True)
+        #new values in the same arrays (in place), a few arrays replaced
+        for k, leaf in enumerate(tree_util.tree_leaves(params)):
+            if k % 7 == call:
+                leaf *= np.float32(1.0 + 0.01 * (call + 1))
+        x = rng.standard_normal(x.shape).astype(np.float32)
+        got = fn(params, x)
+        interp.upload_inputs(params, x)
+        interp.replay(1)
+        whole = interp.read_outputs()
+        for g, w in zip(tree_util.tree_leaves(got), whole):
+            assert np.array_equal(np.asarray(g).reshape(-1), np.asarray(w).reshape(-1)), call
+        flat = np.concatenate([np.asarray(g, np.float32).reshape(-1) for g in tree_util.tree_leaves(got)])
+        assert np.isfinite(flat).all() and (previous is None or not np.array_equal(flat, previous))
+        previous = flat
+    assert any(l.members for l in interp.launches) or any('batch' in l.kernel for l in interp.launches), [l.kernel for l in interp.launches]
+
+
 def test_stream_with_several_tuples_in_flight():
     '''Function.stream(..., in_flight=n) evaluates n tuples at a time, each on a device context of its own driven by
     its own thread; the results are those of plain calls, in the order of the tuples: small and large arguments,
