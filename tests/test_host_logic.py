@@ -588,3 +588,67 @@ def test_large_results_that_nothing_reads_again_are_stored_past_the_caches():
     assert streamed(plan(lambda x, y: lax.concatenate([x, y], 0), big, big)) == [('concat_part_v4', 1), ('concat_part_v4', 1)]
     for launch in plan(lambda x: jnp.exp(x), big).launches:
         assert launch.streamable and K.with_streamed_result(launch._replace(params=K._u32(launch.params and 5) + launch.params[4:])).params[:4] == K._u32(5 | 1 << 31)
+
+
+def test_stream_in_flight_hands_out_results_in_order_whatever_the_lanes_do():
+    '''Function.stream(in_flight=n) without a device: stand-in lanes that take their tuples at different speeds. Results
+    come back in the order of the tuples; the iterable is never asked for a tuple while a lane has not finished copying
+    the one before (the loader may refill its arrays); at most 4 n tuples are under way; an error raised by the
+    iterable or by a lane reaches the consumer; a consumer that stops early leaves no thread behind.'''
+    import threading, time
+    import vkjax_amd
+
+    class Lane:
+        def __init__(self, delay, fail_at=None):
+            self.delay, self.fail_at, self.taken_while_copying = delay, fail_at, 0
+        def _stream_one(self, tuples, taken=None):
+            for (value,) in tuples:
+                state['copying'] += 1
+                time.sleep(0.0005)                      #"copies" what the loader may refill
+                state['overlapping_copies'] += state['copying'] > 1
+                state['copying'] -= 1
+                taken()
+                if value == self.fail_at:
+                    raise ValueError(f'lane failed at {value}')
+                time.sleep(self.delay * (1 + value % 3))
+                state['under_way'] = max(state['under_way'], state['taken'] - state['yielded'])
+                yield value * 10
+
+    def source(n, fail_at=None):
+        for k in range(n):
+            assert state['copying'] == 0, 'the iterable was asked for a tuple while a lane was still copying the one before'
+            if k == fail_at:
+                raise KeyError('no such batch')
+            state['taken'] += 1
+            yield (k,)
+
+    def run(lanes, n, **kw):
+        f = vkjax_amd.wrap(lambda x: x, frontend='minijax')
+        f._in_flight_lanes = lanes
+        return f.stream(source(n, **kw), in_flight=len(lanes))
+
+    for delays in ((0.001, 0.004), (0.003, 0.0, 0.002)):
+        state = dict(copying=0, overlapping_copies=0, under_way=0, taken=0, yielded=0)
+        got = []
+        for y in run([Lane(d) for d in delays], 40):
+            got.append(y)
+            state['yielded'] += 1
+        assert got == [10 * k for k in range(40)]
+        assert state['overlapping_copies'] == 0 and state['under_way'] <= 4 * len(delays) + 1, state
+    lane_threads = lambda: [t for t in threading.enumerate() if t.name.startswith('vkjax-stream-lane')]
+    assert not lane_threads()
+    #errors: of the iterable, of a lane
+    state = dict(copying=0, overlapping_copies=0, under_way=0, taken=0, yielded=0)
+    with pytest.raises(KeyError, match='no such batch'):
+        list(run([Lane(0.001), Lane(0.002)], 20, fail_at=7))
+    assert not lane_threads()
+    state = dict(copying=0, overlapping_copies=0, under_way=0, taken=0, yielded=0)
+    with pytest.raises(ValueError, match='lane failed at 5'):
+        list(run([Lane(0.001, fail_at=5), Lane(0.001, fail_at=5)], 20))
+    assert not lane_threads()
+    #a consumer that stops early
+    state = dict(copying=0, overlapping_copies=0, under_way=0, taken=0, yielded=0)
+    it = run([Lane(0.001), Lane(0.001)], 1000)
+    assert [next(it) for _ in range(5)] == [0, 10, 20, 30, 40]
+    it.close()
+    assert not lane_threads() and state['taken'] < 40
